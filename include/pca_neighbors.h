@@ -1,0 +1,144 @@
+/*
+ * pca_neighbors.h -- C ABI of the MI355X (gfx950) neighbour-search library.
+ *
+ * Plain pointers and sizes only: every pointer is DEVICE memory of the GPU
+ * that is current on the calling thread unless a parameter says otherwise.
+ * All entry points are asynchronous on `stream` (a hipStream_t passed as
+ * void*; NULL = the default stream) and return a status code; they never
+ * allocate, free or synchronise.  The library keeps no state between calls.
+ *
+ * The reference (rusty1s/pytorch_cluster 1.6.3) has no C ABI: its boundary is
+ * the TorchScript operator registry.  Each entry point below names the
+ * reference interface it stands under, so that a binding of that interface
+ * (the C++ operator shim of this repository, or a maintainer's own) is a few
+ * lines of validation, allocation and one call.
+ *
+ * Conventions shared by all entry points
+ *   x          [n, d] row-major points that are searched
+ *   y          [m, d] row-major query points
+ *   ptr_x/y    [num_segments + 1] int64 CSR pointers (non-decreasing,
+ *              ptr[0] = 0, ptr_x[last] = n, ptr_y[last] = m); segment b of y
+ *              searches segment b of x only.  Both NULL = one segment
+ *              ([0, n] / [0, m]); then num_segments is ignored.
+ *   edges      int64 buffer of capacity 2 * m * slots (slots = k, or the
+ *              effective max_num_neighbors).  On completion it holds a
+ *              contiguous [2, E] matrix at its start: edges[0 .. E) are the
+ *              query (y) rows, edges[E .. 2E) the matching x rows, global row
+ *              numbers, grouped by ascending query row.
+ *   num_edges  one int64 on the device that receives E.
+ *   workspace  scratch of at least the size the matching *_workspace_bytes()
+ *              call returns, 256-byte aligned.
+ *   n, m < 2^31 - 1.
+ */
+#ifndef PCA_NEIGHBORS_H
+#define PCA_NEIGHBORS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PCA_ABI_VERSION 1
+
+enum pca_status {
+  PCA_OK = 0,
+  PCA_ERR_INVALID_ARGUMENT = -1, /* NULL pointer, negative size, d mismatch   */
+  PCA_ERR_K_TOO_LARGE = -2,      /* k > PCA_KNN_MAX_K                         */
+  PCA_ERR_WORKSPACE = -3,        /* workspace too small or misaligned         */
+  PCA_ERR_LAUNCH = -4,           /* the HIP runtime refused a launch          */
+  PCA_ERR_UNSUPPORTED = -5,      /* combination not built (see message)       */
+  PCA_ERR_NO_DEVICE = -6         /* no usable gfx950 device is current        */
+};
+
+/* Same limit as the reference GPU operator (csrc/cuda/knn_cuda.cu:98). */
+#define PCA_KNN_MAX_K 100
+
+/* Element types of x / y. */
+enum pca_dtype {
+  PCA_F32 = 0,
+  PCA_F64 = 1,
+  PCA_F16 = 2,
+  PCA_BF16 = 3
+};
+
+/* ABI version of the loaded library (== PCA_ABI_VERSION it was built with). */
+int pca_abi_version(void);
+
+/* Static, human-readable text for a status code. */
+const char *pca_status_string(int status);
+
+/* Text describing the last failure on the calling thread ("" if none). */
+const char *pca_last_error(void);
+
+/* ------------------------------------------------------------------ kNN -- */
+
+/*
+ * Workspace size of pca_knn for these sizes (bytes; 0 on invalid arguments).
+ */
+size_t pca_knn_workspace_bytes(int64_t n, int64_t m, int64_t d,
+                               int64_t num_segments, int64_t k, int dtype);
+
+/*
+ * For every row of y the k nearest rows of x of the same segment.
+ *
+ * Stands under the reference operator
+ *   torch_cluster::knn(x, y, ptr_x, ptr_y, k, cosine, num_workers)
+ *   csrc/knn.cpp:22-40 -> knn_cuda, csrc/cuda/knn_cuda.cu:86-135
+ * and reproduces knn_kernel (csrc/cuda/knn_cuda.cu:30-84): squared Euclidean
+ * distance accumulated over the dimensions in ascending order (or
+ * 1 - x.y / (|x| |y|) when cosine != 0), neighbours of a query ordered by
+ * ascending distance with ties by ascending x row, min(k, segment size)
+ * neighbours per query, candidates whose distance is >= 1e10 or NaN are never
+ * returned.  `dtype` selects the element type of x and y (enum pca_dtype).
+ *
+ * edges: capacity 2 * m * k.  Optional outputs (NULL to skip):
+ *   dist   [capacity m * k] element type of x: the distance of each returned
+ *          edge, in edge order (the reference discards these).
+ */
+int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
+            const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+            int64_t num_segments, int64_t k, int cosine, int dtype,
+            int64_t *edges, int64_t *num_edges, void *dist, void *workspace,
+            size_t workspace_bytes, void *stream);
+
+/* --------------------------------------------------------------- radius -- */
+
+/*
+ * Number of neighbour slots per query pca_radius uses for these sizes:
+ * min(max_num_neighbors, n).  `edges` must hold 2 * m * slots int64.
+ */
+int64_t pca_radius_slots(int64_t n, int64_t max_num_neighbors);
+
+size_t pca_radius_workspace_bytes(int64_t n, int64_t m, int64_t d,
+                                  int64_t num_segments,
+                                  int64_t max_num_neighbors, int dtype);
+
+/*
+ * For every row of y the rows of x of the same segment with squared distance
+ * strictly below r * r, at most max_num_neighbors of them: the first ones in
+ * ascending x row order.
+ *
+ * Stands under the reference operator
+ *   torch_cluster::radius(x, y, ptr_x, ptr_y, r, max_num_neighbors,
+ *                         num_workers, ignore_same_index)
+ *   csrc/radius.cpp:22-39 -> radius_cuda, csrc/cuda/radius_cuda.cu:44-96
+ * and reproduces radius_kernel (csrc/cuda/radius_cuda.cu:9-42); r * r is
+ * formed in double and narrowed to the element type as at
+ * csrc/cuda/radius_cuda.cu:90.  With ignore_same_index != 0 the x row whose
+ * global number equals the query's is skipped.  max_num_neighbors must be
+ * >= 1 (the reference is undefined for 0).
+ */
+int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
+               const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+               int64_t num_segments, double r, int64_t max_num_neighbors,
+               int ignore_same_index, int dtype, int64_t *edges,
+               int64_t *num_edges, void *workspace, size_t workspace_bytes,
+               void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* PCA_NEIGHBORS_H */

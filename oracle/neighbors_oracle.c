@@ -1,0 +1,223 @@
+/*
+ * TEST INFRASTRUCTURE ONLY -- the product never links, loads or calls this.
+ *
+ * CPU restatement of the reference's GPU semantics for the kNN / radius
+ * neighbour-search path, in plain C.  It is the checker for the HIP kernels
+ * (tests/, the smoke check and the cpu_baseline leg of the benchmark may use
+ * it; nothing else may).
+ *
+ * What is restated (reference file:line):
+ *   oracle_knn_dense_*     csrc/cuda/knn_cuda.cu:30-84   (knn_kernel) with the
+ *                          default ptr of the host wrapper (:100-112) and
+ *                          csrc/cuda/utils.cuh:11-19     (get_example_idx)
+ *   cosine distance        csrc/cuda/knn_cuda.cu:9-28,55-59
+ *   oracle_radius_dense_*  csrc/cuda/radius_cuda.cu:9-42 (radius_kernel); the
+ *                          caller passes r*r formed in double and narrowed to
+ *                          the element type as the host wrapper does (:90)
+ *   oracle_compact         csrc/cuda/knn_cuda.cu:133-134 and
+ *                          csrc/cuda/radius_cuda.cu:94-95 (mask on -1, two
+ *                          masked_selects, stack)
+ *
+ * Arithmetic: `fma_mode` = 1 evaluates every `acc += a * b` of the reference
+ * kernels as one fused multiply-add (what a GPU compiler emits for that
+ * source, and what the HIP kernels of this repository do explicitly), 0 rounds
+ * the product and the sum separately (what a CPU build without FMA
+ * contraction does).  The file is compiled with -ffp-contract=off so nothing
+ * else is fused.
+ *
+ * Parity pins (see tests/test_oracle_*.py): the reference's inline fixtures
+ * test/test_knn.py:16-52,57-75, test/test_radius.py:25-116, the ordered README
+ * outputs README.md:188-191,217-220, the reference's compiled CPU operators
+ * (oracle/_ref), scipy's cKDTree as in test/test_knn.py:84-88 and
+ * test/test_radius.py:129-133, and float64 brute force.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* csrc/cuda/utils.cuh:11-19 -- first i with ptr[i+1] > idx, else the last
+ * segment. */
+static int64_t example_idx(int64_t idx, const int64_t *ptr,
+                           int64_t num_examples) {
+  for (int64_t i = 0; i < num_examples; i++) {
+    if (ptr[i + 1] > idx)
+      return i;
+  }
+  return num_examples - 1;
+}
+
+#define DEFINE_ORACLE(SUFFIX, T, FMA, SQRT)                                    \
+                                                                               \
+  static T sqdist_##SUFFIX(const T *x, const T *y, int64_t n_x, int64_t n_y,   \
+                           int64_t dim, int fma_mode) {                        \
+    T acc = 0;                                                                 \
+    for (int64_t d = 0; d < dim; d++) {                                        \
+      T diff = x[n_x * dim + d] - y[n_y * dim + d];                            \
+      if (fma_mode)                                                            \
+        acc = FMA(diff, diff, acc);                                            \
+      else {                                                                   \
+        T sq = diff * diff;                                                    \
+        acc = acc + sq;                                                        \
+      }                                                                        \
+    }                                                                          \
+    return acc;                                                                \
+  }                                                                            \
+                                                                               \
+  static T dot_##SUFFIX(const T *a, const T *b, int64_t n_a, int64_t n_b,      \
+                        int64_t size, int fma_mode) {                          \
+    T result = 0;                                                              \
+    for (int64_t i = 0; i < size; i++) {                                       \
+      if (fma_mode)                                                            \
+        result = FMA(a[n_a * size + i], b[n_b * size + i], result);            \
+      else {                                                                   \
+        T p = a[n_a * size + i] * b[n_b * size + i];                           \
+        result = result + p;                                                   \
+      }                                                                        \
+    }                                                                          \
+    return result;                                                             \
+  }                                                                            \
+                                                                               \
+  static T norm_##SUFFIX(const T *a, int64_t n_a, int64_t size,                \
+                         int fma_mode) {                                       \
+    return SQRT(dot_##SUFFIX(a, a, n_a, n_a, size, fma_mode));                 \
+  }                                                                            \
+                                                                               \
+  /* One query of knn_kernel: sorted insertion list with the strict `>` test   \
+   * (an equal distance never displaces an earlier, lower-index entry), 1e10   \
+   * sentinel, -1 padded indices. */                                           \
+  static void knn_query_##SUFFIX(const T *x, const T *y, int64_t n_y,          \
+                                 int64_t x_begin, int64_t x_end, int64_t dim,  \
+                                 int64_t k, int cosine, int fma_mode,          \
+                                 T *best_dist, int64_t *best_idx) {            \
+    for (int64_t e = 0; e < k; e++) {                                          \
+      best_dist[e] = (T)1e10;                                                  \
+      best_idx[e] = -1;                                                        \
+    }                                                                          \
+    for (int64_t n_x = x_begin; n_x < x_end; n_x++) {                          \
+      T tmp_dist;                                                              \
+      if (cosine) {                                                            \
+        T den = norm_##SUFFIX(x, n_x, dim, fma_mode) *                         \
+                norm_##SUFFIX(y, n_y, dim, fma_mode);                          \
+        tmp_dist = dot_##SUFFIX(x, y, n_x, n_y, dim, fma_mode) / den;          \
+        /* `1. - tmp_dist`: the literal is a double in the reference */        \
+        tmp_dist = (T)(1. - (double)tmp_dist);                                 \
+      } else {                                                                 \
+        tmp_dist = sqdist_##SUFFIX(x, y, n_x, n_y, dim, fma_mode);             \
+      }                                                                        \
+      for (int64_t e1 = 0; e1 < k; e1++) {                                     \
+        if (best_dist[e1] > tmp_dist) {                                        \
+          for (int64_t e2 = k - 1; e2 > e1; e2--) {                            \
+            best_dist[e2] = best_dist[e2 - 1];                                 \
+            best_idx[e2] = best_idx[e2 - 1];                                   \
+          }                                                                    \
+          best_dist[e1] = tmp_dist;                                            \
+          best_idx[e1] = n_x;                                                  \
+          break;                                                               \
+        }                                                                      \
+      }                                                                        \
+    }                                                                          \
+  }                                                                            \
+                                                                               \
+  /* row/col: [m*k] as the kernel leaves them (col -1 where fewer than k       \
+   * candidates exist).  dist: optional [m*k] distances (1e10 where empty). */ \
+  int oracle_knn_dense_##SUFFIX(                                               \
+      const T *x, const T *y, const int64_t *ptr_x, const int64_t *ptr_y,      \
+      int64_t n, int64_t m, int64_t dim, int64_t num_examples, int64_t k,      \
+      int cosine, int fma_mode, int64_t *row, int64_t *col, T *dist) {         \
+    int64_t default_ptr_x[2] = {0, n}, default_ptr_y[2] = {0, m};              \
+    if (ptr_x == NULL || ptr_y == NULL) {                                      \
+      ptr_x = default_ptr_x;                                                   \
+      ptr_y = default_ptr_y;                                                   \
+      num_examples = 1;                                                        \
+    }                                                                          \
+    if (k <= 0)                                                                \
+      return 1;                                                                \
+    _Pragma("omp parallel") {                                                  \
+      T *best_dist = (T *)malloc(sizeof(T) * (size_t)k);                       \
+      int64_t *best_idx = (int64_t *)malloc(sizeof(int64_t) * (size_t)k);      \
+      _Pragma("omp for schedule(dynamic, 64)") for (int64_t n_y = 0; n_y < m;  \
+                                                    n_y++) {                   \
+        int64_t b = example_idx(n_y, ptr_y, num_examples);                     \
+        knn_query_##SUFFIX(x, y, n_y, ptr_x[b], ptr_x[b + 1], dim, k, cosine,  \
+                           fma_mode, best_dist, best_idx);                     \
+        for (int64_t e = 0; e < k; e++) {                                      \
+          row[n_y * k + e] = n_y;                                              \
+          col[n_y * k + e] = best_idx[e];                                      \
+          if (dist)                                                            \
+            dist[n_y * k + e] = best_dist[e];                                  \
+        }                                                                      \
+      }                                                                        \
+      free(best_dist);                                                         \
+      free(best_idx);                                                          \
+    }                                                                          \
+    return 0;                                                                  \
+  }                                                                            \
+                                                                               \
+  /* row/col: [m*max_num_neighbors], pre-filled with -1 like the host wrapper  \
+   * (radius_cuda.cu:75-78).  scanned: optional [m], the number of x rows the  \
+   * query visited before it stopped (for the required-pairs work count). */   \
+  int oracle_radius_dense_##SUFFIX(                                            \
+      const T *x, const T *y, const int64_t *ptr_x, const int64_t *ptr_y,      \
+      int64_t n, int64_t m, int64_t dim, int64_t num_examples, T r2,           \
+      int64_t max_num_neighbors, int ignore_same_index, int fma_mode,          \
+      int64_t *row, int64_t *col, int64_t *scanned) {                          \
+    int64_t default_ptr_x[2] = {0, n}, default_ptr_y[2] = {0, m};              \
+    if (ptr_x == NULL || ptr_y == NULL) {                                      \
+      ptr_x = default_ptr_x;                                                   \
+      ptr_y = default_ptr_y;                                                   \
+      num_examples = 1;                                                        \
+    }                                                                          \
+    if (max_num_neighbors <= 0)                                                \
+      return 1; /* the reference writes out of bounds here: undefined */       \
+    for (int64_t i = 0; i < m * max_num_neighbors; i++) {                      \
+      row[i] = -1;                                                             \
+      col[i] = -1;                                                             \
+    }                                                                          \
+    _Pragma("omp parallel for schedule(dynamic, 64)") for (int64_t n_y = 0;    \
+                                                           n_y < m; n_y++) {   \
+      int64_t count = 0;                                                       \
+      int64_t b = example_idx(n_y, ptr_y, num_examples);                       \
+      int64_t n_x = ptr_x[b];                                                  \
+      for (; n_x < ptr_x[b + 1]; n_x++) {                                      \
+        T d = sqdist_##SUFFIX(x, y, n_x, n_y, dim, fma_mode);                  \
+        if (d < r2 && !(ignore_same_index && n_y == n_x)) {                    \
+          row[n_y * max_num_neighbors + count] = n_y;                          \
+          col[n_y * max_num_neighbors + count] = n_x;                          \
+          count++;                                                             \
+        }                                                                      \
+        if (count >= max_num_neighbors) {                                      \
+          n_x++;                                                               \
+          break;                                                               \
+        }                                                                      \
+      }                                                                        \
+      if (scanned)                                                             \
+        scanned[n_y] = n_x - ptr_x[b];                                         \
+    }                                                                          \
+    return 0;                                                                  \
+  }
+
+DEFINE_ORACLE(f32, float, fmaf, sqrtf)
+DEFINE_ORACLE(f64, double, fma, sqrt)
+
+/* Host-wrapper epilogue: keep the slots whose `mask_src` entry is not -1, in
+ * slot order, and stack them as [2, E] (row-major, leading dimension E).
+ * Returns E; writes nothing when out is NULL. */
+int64_t oracle_compact(const int64_t *row, const int64_t *col,
+                       const int64_t *mask_src, int64_t slots, int64_t *out,
+                       int64_t capacity) {
+  int64_t e = 0;
+  for (int64_t i = 0; i < slots; i++)
+    e += mask_src[i] != -1;
+  if (out == NULL || e > capacity)
+    return e;
+  int64_t j = 0;
+  for (int64_t i = 0; i < slots; i++) {
+    if (mask_src[i] != -1) {
+      out[j] = row[i];
+      out[e + j] = col[i];
+      j++;
+    }
+  }
+  return e;
+}

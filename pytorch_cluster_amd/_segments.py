@@ -1,0 +1,63 @@
+"""Host-side prologue shared by ``knn`` and ``radius``.
+
+The reference repeats this block in both wrappers
+(``torch_cluster/knn.py:58-79``, ``torch_cluster/radius.py:62-84``): make the
+point matrices 2-D and contiguous, find the number of examples, and turn the
+sorted batch vectors into CSR pointers.  Everything here is
+``torch.jit.script``-able.
+"""
+from typing import Optional, Tuple
+
+import torch
+
+
+def as_points(t: torch.Tensor) -> torch.Tensor:
+    """``[N]`` -> ``[N, 1]``; returns a contiguous ``[N, F]`` matrix."""
+    if t.dim() == 1:
+        t = t.view(-1, 1)
+    return t.contiguous()
+
+
+def num_examples(x: torch.Tensor, y: torch.Tensor,
+                 batch_x: Optional[torch.Tensor],
+                 batch_y: Optional[torch.Tensor],
+                 batch_size: Optional[int]) -> int:
+    """Number of examples B; reads ``batch.max()`` from the device only when
+    the caller did not pass ``batch_size``."""
+    if batch_size is not None:
+        assert batch_size > 0
+        return batch_size
+    b = 1
+    if batch_x is not None:
+        assert x.size(0) == batch_x.numel()
+        b = int(batch_x.max()) + 1
+    if batch_y is not None:
+        assert y.size(0) == batch_y.numel()
+        b = max(b, int(batch_y.max()) + 1)
+    assert b > 0
+    return b
+
+
+def segment_pointers(
+    x: torch.Tensor, y: torch.Tensor, batch_x: Optional[torch.Tensor],
+    batch_y: Optional[torch.Tensor], batch_size: Optional[int]
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """CSR pointers ``[B + 1]`` of both sorted batch vectors, or
+    ``(None, None)`` for a single example: ``ptr[b]`` is the first row whose
+    example id is ``>= b`` (examples without rows get empty segments)."""
+    b = num_examples(x, y, batch_x, batch_y, batch_size)
+    if b <= 1:
+        return None, None
+    assert batch_x is not None
+    assert batch_y is not None
+    ids = torch.arange(b + 1, device=x.device)
+    return torch.bucketize(ids, batch_x), torch.bucketize(ids, batch_y)
+
+
+def orient(edge_index: torch.Tensor, flow: str) -> torch.Tensor:
+    """The search operators return (query, neighbour) pairs.  With
+    ``source_to_target`` messages flow from the neighbour to the query, so the
+    neighbour row comes first."""
+    if flow == 'source_to_target':
+        return edge_index.flip(0)
+    return edge_index

@@ -1,0 +1,104 @@
+"""Builds the native libraries of this package in-tree for gfx950.
+
+    python -m pytorch_cluster_amd.build [--jobs N] [--skip-torch-ops]
+
+Outputs (next to this file, git-ignored):
+  libpca_neighbors.so   HIP kernels + the C ABI of include/pca_neighbors.h
+  _torch_ops.so         TorchScript operator binding (links the above)
+"""
+import argparse
+import concurrent.futures
+import glob
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ_DIR = os.path.join(HERE, "_build")
+CAPI_LIB = os.path.join(HERE, "libpca_neighbors.so")
+TORCH_OPS_LIB = os.path.join(HERE, "_torch_ops.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ARCH = "gfx950"
+
+# Packed FP32 instructions are switched off for every device compile.
+HIP_FLAGS = [
+    "--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                          text=True)
+    # the host pass does not know the packed-fp32 feature; that is harmless
+    out = "\n".join(line for line in proc.stdout.splitlines()
+                    if "packed-fp32-ops" not in line)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def _compile_hip(src):
+    obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
+    _run([HIPCC] + HIP_FLAGS + ["-c", src, "-o", obj])
+    return obj
+
+
+def build_capi(jobs):
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        objects = list(pool.map(_compile_hip, sources))
+    _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", CAPI_LIB]
+         + objects)
+    return CAPI_LIB
+
+
+def build_torch_ops():
+    import torch
+    from torch.utils import cpp_extension
+
+    includes = []
+    for path in cpp_extension.include_paths():
+        includes += ["-I", path]
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    cmd = [
+        "g++", "-O2", "-std=c++17", "-fPIC", "-shared",
+        "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+        "-D_GLIBCXX_USE_CXX11_ABI=%d" % abi, "-Wno-deprecated-declarations",
+        "-I", "/opt/rocm/include",
+    ] + includes + [
+        os.path.join(CSRC, "torch_ops.cpp"), "-o", TORCH_OPS_LIB,
+        "-L", HERE, "-lpca_neighbors",
+        "-L", torch_lib, "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10",
+        "-lc10_hip", "-lamdhip64",
+        "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib,
+    ]
+    _run(cmd)
+    return TORCH_OPS_LIB
+
+
+def build_all(jobs=None, torch_ops=True):
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    build_capi(jobs)
+    if torch_ops:
+        build_torch_ops()
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--jobs", type=int, default=None)
+    ap.add_argument("--skip-torch-ops", action="store_true")
+    args = ap.parse_args(argv)
+    build_all(args.jobs, not args.skip_torch_ops)
+    print("built", CAPI_LIB)
+    if not args.skip_torch_ops:
+        print("built", TORCH_OPS_LIB)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,281 @@
+// C ABI of the neighbour-search library (declared in include/pca_neighbors.h).
+//
+// Validates sizes on the host, carves the caller's workspace and queues the
+// kernels on the caller's stream.  No allocation, no synchronisation, no
+// state: the operator-level behaviour of the reference's host wrappers
+// (csrc/cuda/knn_cuda.cu:86-135, csrc/cuda/radius_cuda.cu:44-96) minus tensor
+// handling, which belongs to the binding above this layer.
+#include "../../include/pca_neighbors.h"
+
+#include "device_utils.hpp"
+#include "launchers.hpp"
+
+#include <cstdarg>
+#include <cstdio>
+
+namespace {
+
+thread_local char g_last_error[256] = "";
+
+int fail(int status, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return status;
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct Carver {
+  char *base;
+  size_t offset = 0;
+  explicit Carver(void *p) : base(static_cast<char *>(p)) {}
+  template <typename T> T *take(size_t count) {
+    T *p = reinterpret_cast<T *>(base + offset);
+    offset += align256(sizeof(T) * count);
+    return p;
+  }
+};
+
+__global__ void set_i64_kernel(int64_t *p, int64_t v) { *p = v; }
+
+constexpr int64_t kMaxRows = 2147483646; // n, m < 2^31 - 1
+
+bool sizes_ok(int64_t n, int64_t m, int64_t d, int64_t num_segments) {
+  return n >= 0 && m >= 0 && n <= kMaxRows && m <= kMaxRows && d >= 1 &&
+         d <= (1 << 20) && num_segments >= 1 && num_segments <= kMaxRows;
+}
+
+size_t knn_workspace(int64_t m, int64_t num_segments, int64_t k) {
+  size_t bytes = 0;
+  bytes += align256(sizeof(int) * (size_t)(num_segments + 1)); // work_start
+  bytes += align256(sizeof(int) * (size_t)m * (size_t)k);      // idx
+  bytes += align256(sizeof(float) * (size_t)m * (size_t)k);    // dist
+  bytes += align256(sizeof(int) * (size_t)m);                  // count
+  bytes += pca::compact_workspace_bytes((int)m);
+  return bytes;
+}
+
+size_t radius_workspace(int64_t m, int64_t num_segments, int64_t slots) {
+  size_t bytes = 0;
+  bytes += align256(sizeof(int) * (size_t)(num_segments + 1));
+  bytes += align256(sizeof(int) * (size_t)m * (size_t)slots);
+  bytes += align256(sizeof(int) * (size_t)m);
+  bytes += pca::compact_workspace_bytes((int)m);
+  return bytes;
+}
+
+int check_launch(hipError_t err, const char *what) {
+  if (err != hipSuccess)
+    return fail(PCA_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(err));
+  return PCA_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int pca_abi_version(void) { return PCA_ABI_VERSION; }
+
+const char *pca_status_string(int status) {
+  switch (status) {
+  case PCA_OK:
+    return "ok";
+  case PCA_ERR_INVALID_ARGUMENT:
+    return "invalid argument";
+  case PCA_ERR_K_TOO_LARGE:
+    return "`k` needs to smaller than or equal to 100";
+  case PCA_ERR_WORKSPACE:
+    return "workspace too small or misaligned";
+  case PCA_ERR_LAUNCH:
+    return "HIP launch failed";
+  case PCA_ERR_UNSUPPORTED:
+    return "combination not supported";
+  case PCA_ERR_NO_DEVICE:
+    return "no usable device";
+  default:
+    return "unknown status";
+  }
+}
+
+const char *pca_last_error(void) { return g_last_error; }
+
+size_t pca_knn_workspace_bytes(int64_t n, int64_t m, int64_t d,
+                               int64_t num_segments, int64_t k, int dtype) {
+  (void)dtype;
+  if (num_segments < 1)
+    num_segments = 1;
+  if (!sizes_ok(n, m, d, num_segments) || k < 1 || k > PCA_KNN_MAX_K)
+    return 0;
+  return knn_workspace(m, num_segments, k);
+}
+
+int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
+            const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+            int64_t num_segments, int64_t k, int cosine, int dtype,
+            int64_t *edges, int64_t *num_edges, void *dist, void *workspace,
+            size_t workspace_bytes, void *stream_) {
+  g_last_error[0] = 0;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if ((ptr_x == nullptr) != (ptr_y == nullptr))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "ptr_x and ptr_y must both be given or both be NULL");
+  if (ptr_x == nullptr)
+    num_segments = 1;
+  if (!sizes_ok(n, m, d, num_segments))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "bad sizes n=%lld m=%lld d=%lld num_segments=%lld",
+                (long long)n, (long long)m, (long long)d,
+                (long long)num_segments);
+  if (k < 1)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "k must be >= 1, got %lld",
+                (long long)k);
+  if (k > PCA_KNN_MAX_K)
+    return fail(PCA_ERR_K_TOO_LARGE, "%s",
+                pca_status_string(PCA_ERR_K_TOO_LARGE));
+  if (num_edges == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "num_edges is NULL");
+  if (dtype != PCA_F32)
+    return fail(PCA_ERR_UNSUPPORTED, "element type %d is not built", dtype);
+
+  if (n == 0 || m == 0) {
+    hipLaunchKernelGGL(set_i64_kernel, dim3(1), dim3(1), 0, stream, num_edges,
+                       (int64_t)0);
+    return check_launch(hipGetLastError(), "set_i64_kernel");
+  }
+  if (x == nullptr || y == nullptr || edges == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "x, y or edges is NULL");
+  if (workspace == nullptr || ((uintptr_t)workspace & 255) != 0 ||
+      workspace_bytes < knn_workspace(m, num_segments, k))
+    return fail(PCA_ERR_WORKSPACE, "workspace needs %zu bytes, 256-aligned",
+                knn_workspace(m, num_segments, k));
+
+  if (!pca::knn_lowd_supported((int)d, (int)k, cosine != 0))
+    return fail(PCA_ERR_UNSUPPORTED, "kNN for d=%lld is not built",
+                (long long)d);
+
+  Carver ws(workspace);
+  int *work_start = ws.take<int>((size_t)num_segments + 1);
+  pca::DenseResult dense;
+  dense.idx = ws.take<int>((size_t)m * k);
+  dense.dist = ws.take<float>((size_t)m * k);
+  dense.count = ws.take<int>((size_t)m);
+  dense.slots = (int)k;
+  void *compact_ws = ws.take<char>(pca::compact_workspace_bytes((int)m));
+  if (dist == nullptr)
+    dense.dist = nullptr;
+
+  pca::SearchInput in{x,      y,      ptr_x,  ptr_y,
+                      (int)n, (int)m, (int)d, (int)num_segments};
+  const pca::KnnLowdConfig cfg = pca::knn_lowd_config((int)d, (int)k, (int)m);
+  int rc = check_launch(pca::launch_plan(ptr_y, (int)m, (int)num_segments,
+                                         cfg.tile_queries, work_start, stream),
+                        "plan_kernel");
+  if (rc != PCA_OK)
+    return rc;
+  const int bound =
+      pca::plan_upper_bound((int)m, (int)num_segments, cfg.tile_queries);
+  rc = check_launch(pca::launch_knn_lowd(in, (int)k, cosine != 0, cfg,
+                                         work_start, bound, dense, stream),
+                    "knn_lowd_kernel");
+  if (rc != PCA_OK)
+    return rc;
+  return check_launch(pca::launch_compact(dense, (int)m, edges, num_edges,
+                                          static_cast<float *>(dist),
+                                          compact_ws, stream),
+                      "compaction kernels");
+}
+
+int64_t pca_radius_slots(int64_t n, int64_t max_num_neighbors) {
+  if (n < 0 || max_num_neighbors < 0)
+    return 0;
+  return max_num_neighbors < n ? max_num_neighbors : n;
+}
+
+size_t pca_radius_workspace_bytes(int64_t n, int64_t m, int64_t d,
+                                  int64_t num_segments,
+                                  int64_t max_num_neighbors, int dtype) {
+  (void)dtype;
+  if (num_segments < 1)
+    num_segments = 1;
+  if (!sizes_ok(n, m, d, num_segments) || max_num_neighbors < 1)
+    return 0;
+  return radius_workspace(m, num_segments,
+                          pca_radius_slots(n, max_num_neighbors));
+}
+
+int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
+               const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+               int64_t num_segments, double r, int64_t max_num_neighbors,
+               int ignore_same_index, int dtype, int64_t *edges,
+               int64_t *num_edges, void *workspace, size_t workspace_bytes,
+               void *stream_) {
+  g_last_error[0] = 0;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if ((ptr_x == nullptr) != (ptr_y == nullptr))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "ptr_x and ptr_y must both be given or both be NULL");
+  if (ptr_x == nullptr)
+    num_segments = 1;
+  if (!sizes_ok(n, m, d, num_segments))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "bad sizes n=%lld m=%lld d=%lld num_segments=%lld",
+                (long long)n, (long long)m, (long long)d,
+                (long long)num_segments);
+  if (max_num_neighbors < 1)
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "max_num_neighbors must be >= 1, got %lld",
+                (long long)max_num_neighbors);
+  if (num_edges == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "num_edges is NULL");
+  if (dtype != PCA_F32)
+    return fail(PCA_ERR_UNSUPPORTED, "element type %d is not built", dtype);
+
+  if (n == 0 || m == 0) {
+    hipLaunchKernelGGL(set_i64_kernel, dim3(1), dim3(1), 0, stream, num_edges,
+                       (int64_t)0);
+    return check_launch(hipGetLastError(), "set_i64_kernel");
+  }
+  if (x == nullptr || y == nullptr || edges == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "x, y or edges is NULL");
+  const int64_t slots = pca_radius_slots(n, max_num_neighbors);
+  if (workspace == nullptr || ((uintptr_t)workspace & 255) != 0 ||
+      workspace_bytes < radius_workspace(m, num_segments, slots))
+    return fail(PCA_ERR_WORKSPACE, "workspace needs %zu bytes, 256-aligned",
+                radius_workspace(m, num_segments, slots));
+
+  Carver ws(workspace);
+  int *work_start = ws.take<int>((size_t)num_segments + 1);
+  pca::DenseResult dense;
+  dense.idx = ws.take<int>((size_t)m * slots);
+  dense.dist = nullptr;
+  dense.count = ws.take<int>((size_t)m);
+  dense.slots = (int)slots;
+  void *compact_ws = ws.take<char>(pca::compact_workspace_bytes((int)m));
+
+  // r * r in double, narrowed to the element type at the launch
+  // (csrc/cuda/radius_cuda.cu:90)
+  const float r2 = (float)(r * r);
+
+  pca::SearchInput in{x,      y,      ptr_x,  ptr_y,
+                      (int)n, (int)m, (int)d, (int)num_segments};
+  int rc = check_launch(pca::launch_plan(ptr_y, (int)m, (int)num_segments,
+                                         pca::kRadiusQueriesPerWave,
+                                         work_start, stream),
+                        "plan_kernel");
+  if (rc != PCA_OK)
+    return rc;
+  const int bound = pca::plan_upper_bound((int)m, (int)num_segments,
+                                          pca::kRadiusQueriesPerWave);
+  rc = check_launch(pca::launch_radius(in, r2, ignore_same_index != 0,
+                                       work_start, bound, dense, stream),
+                    "radius_kernel");
+  if (rc != PCA_OK)
+    return rc;
+  return check_launch(pca::launch_compact(dense, (int)m, edges, num_edges,
+                                          nullptr, compact_ws, stream),
+                      "compaction kernels");
+}
+
+} // extern "C"

@@ -1,0 +1,119 @@
+// Device-side helpers shared by the neighbour-search kernels (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pca {
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256; // 4 waves: one per SIMD of a CU
+
+// Distance every kNN slot starts from; a candidate must be strictly below it
+// to be returned (csrc/cuda/knn_cuda.cu:48,68 in the reference).
+constexpr float kKnnSentinel = 1e10f;
+
+// ---------------------------------------------------------------------------
+// 64-bit selection keys.
+//
+// A candidate is the pair (distance, x row).  The reference orders neighbours
+// by ascending distance and, among equal distances, by ascending row.  Packing
+// the float's bit pattern into the high word and the row into the low word of
+// one 64-bit value and reading that value as an IEEE double gives a single
+// number whose floating-point order is exactly that lexicographic order:
+//   * for d >= 0 the bit patterns of floats order like the floats, and
+//     positive doubles order like their bit patterns;
+//   * for d < 0 (only the cosine distance can be slightly negative) a larger
+//     magnitude is more negative in both formats; the low word then holds the
+//     complemented row so that ties still come out in ascending row order.
+// The high word is biased by one double-exponent step so that no key is a
+// denormal double, whatever the kernel's denormal mode is.  Keys are never
+// NaN: the high word stays below 0x7ff00000 because only distances below
+// kKnnSentinel are ever packed.
+//
+// With keys as doubles, one step of a sorted-insertion network is
+//   b[j] = min(b[j], max(b[j-1], key))
+// i.e. two full-rate f64 VALU instructions per slot and no index bookkeeping.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kKeyBias = 0x00100000u;
+
+__device__ __forceinline__ double make_key(float d, uint32_t row) {
+  uint32_t hi = __float_as_uint(d);
+  uint32_t lo = (hi & 0x80000000u) ? ~row : row;
+  hi += kKeyBias;
+  return __hiloint2double((int)hi, (int)lo);
+}
+
+__device__ __forceinline__ float key_dist(double key) {
+  return __uint_as_float((uint32_t)__double2hiint(key) - kKeyBias);
+}
+
+__device__ __forceinline__ int key_row(double key) {
+  uint32_t hi = (uint32_t)__double2hiint(key) - kKeyBias;
+  uint32_t lo = (uint32_t)__double2loint(key);
+  return (int)((hi & 0x80000000u) ? ~lo : lo);
+}
+
+// Key of an empty slot: distance = sentinel, row = -1.  Larger than every key
+// a real candidate can have.
+__device__ __forceinline__ double empty_key() {
+  return __hiloint2double((int)(0x501502F9u /* 1e10f */ + kKeyBias), -1);
+}
+
+// Key below every real key: fills the slots of a K-wide list that the caller
+// did not ask for (k < K), so that they never take part in the selection.
+__device__ __forceinline__ double lowest_key() {
+  return __hiloint2double((int)0xfff00000u, 0); // -inf
+}
+
+// v_min_f64 / v_max_f64 issued directly: the operands are never NaN, so the
+// canonicalisation a compiler adds around fmin()/fmax() is not needed.
+__device__ __forceinline__ double key_min(double a, double b) {
+  double r;
+  asm("v_min_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+__device__ __forceinline__ double key_max(double a, double b) {
+  double r;
+  asm("v_max_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+// Inserts `key` into the ascending list b[0..K) and drops the largest entry.
+template <int K>
+__device__ __forceinline__ void sorted_insert(double (&b)[K], double key) {
+#pragma unroll
+  for (int j = K - 1; j >= 1; --j)
+    b[j] = key_min(b[j], key_max(b[j - 1], key));
+  b[0] = key_min(b[0], key);
+}
+
+__device__ __forceinline__ float min3f(float a, float b, float c) {
+  return __builtin_fminf(__builtin_fminf(a, b), c);
+}
+
+// Largest b in [0, num_segments) with start[b] <= v; `start` has
+// num_segments + 1 non-decreasing entries and start[num_segments] > v.
+__device__ __forceinline__ int find_segment(const int *__restrict__ start,
+                                            int num_segments, int v) {
+  int lo = 0, hi = num_segments;
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (start[mid] <= v)
+      lo = mid;
+    else
+      hi = mid;
+  }
+  return lo;
+}
+
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  This
+// maps the hardware block id to a logical one such that blocks with
+// neighbouring logical ids (which scan the same segment of x) land on the same
+// XCD.  `grid` must be a multiple of 8.
+__device__ __forceinline__ int xcd_swizzle(int block, int grid) {
+  return (block & 7) * (grid >> 3) + (block >> 3);
+}
+
+} // namespace pca

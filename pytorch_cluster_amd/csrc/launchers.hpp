@@ -1,0 +1,74 @@
+// Host-side launch interface between the C ABI (capi.hip) and the kernel
+// translation units.  Everything here is asynchronous on `stream`.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace pca {
+
+// Per-query result slots every search kernel writes before compaction:
+//   idx   [m, slots] int32  x rows (global numbers), valid in [0, count[q])
+//   dist  [m, slots] fp32   their distances (kNN only; may be NULL)
+//   count [m]        int32  number of valid slots of each query
+struct DenseResult {
+  int *idx;
+  float *dist;
+  int *count;
+  int slots;
+};
+
+struct SearchInput {
+  const void *x;
+  const void *y;
+  const int64_t *ptr_x; // NULL = one segment
+  const int64_t *ptr_y;
+  int n, m, d;
+  int num_segments; // >= 1 (1 when ptr_* are NULL)
+};
+
+// --- segments.hip ----------------------------------------------------------
+
+// work_start[b] = sum over b' < b of ceil(m_b' / per_item): the first work item
+// (query tile / wave task) of each segment; work_start has num_segments + 1
+// entries.
+hipError_t launch_plan(const int64_t *ptr_y, int m, int num_segments,
+                       int per_item, int *work_start, hipStream_t stream);
+
+// Upper bound of work_start[num_segments] that needs no device data.
+inline int plan_upper_bound(int m, int num_segments, int per_item) {
+  return m / per_item + num_segments;
+}
+
+size_t compact_workspace_bytes(int m);
+
+// count -> exclusive offsets -> edges [2, E] (+ optional distances) and E.
+hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
+                          int64_t *num_edges, float *dist_out, void *workspace,
+                          hipStream_t stream);
+
+// --- knn_lowd_*.hip --------------------------------------------------------
+
+// Queries per work item of the low-dimensional kNN kernel for this problem.
+struct KnnLowdConfig {
+  int kbucket;          // compiled list width (>= k)
+  int queries_per_lane; // 1 or 2
+  int tile_queries;     // kBlock * queries_per_lane
+};
+bool knn_lowd_supported(int d, int k, bool cosine);
+KnnLowdConfig knn_lowd_config(int d, int k, int m);
+hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
+                           const KnnLowdConfig &cfg, const int *work_start,
+                           int grid_bound, const DenseResult &out,
+                           hipStream_t stream);
+
+// --- radius.hip ------------------------------------------------------------
+
+constexpr int kRadiusQueriesPerWave = 8;
+hipError_t launch_radius(const SearchInput &in, float r2,
+                         bool ignore_same_index, const int *work_start,
+                         int task_bound, const DenseResult &out,
+                         hipStream_t stream);
+
+} // namespace pca

@@ -1,0 +1,196 @@
+// Segment planning and output compaction kernels.
+//
+// Replaces, on the device and without host synchronisation:
+//   * get_example_idx (csrc/cuda/utils.cuh:11-19 in the reference): instead of
+//     every thread scanning ptr linearly, one tiny kernel turns ptr_y into a
+//     table "first work item of each segment" that workgroups binary-search;
+//   * the reference's post-kernel epilogue `mask = col != -1`,
+//     2x masked_select, stack (csrc/cuda/knn_cuda.cu:133-134,
+//     csrc/cuda/radius_cuda.cu:94-95): per-query counts -> exclusive scan ->
+//     scatter into a contiguous [2, E] matrix, E left in device memory.
+#include "device_utils.hpp"
+#include "launchers.hpp"
+
+namespace pca {
+
+namespace {
+
+constexpr int kPlanThreads = 1024;
+
+// Single workgroup: exclusive scan of ceil(m_b / per_item) over segments.
+__global__ __launch_bounds__(kPlanThreads) void plan_kernel(
+    const int64_t *__restrict__ ptr_y, int m, int num_segments, int per_item,
+    int *__restrict__ work_start) {
+  __shared__ int partial[kPlanThreads];
+  const int tid = threadIdx.x;
+  // contiguous chunk of segments per thread
+  const int per_thread = (num_segments + kPlanThreads - 1) / kPlanThreads;
+  const int b0 = min(tid * per_thread, num_segments);
+  const int b1 = min(b0 + per_thread, num_segments);
+
+  int sum = 0;
+  for (int b = b0; b < b1; ++b) {
+    int64_t lo = ptr_y ? ptr_y[b] : 0;
+    int64_t hi = ptr_y ? ptr_y[b + 1] : m;
+    int len = (int)max((int64_t)0, hi - lo);
+    sum += (len + per_item - 1) / per_item;
+  }
+  partial[tid] = sum;
+  __syncthreads();
+  // Hillis-Steele inclusive scan over the 1024 partial sums
+  for (int off = 1; off < kPlanThreads; off <<= 1) {
+    int v = tid >= off ? partial[tid - off] : 0;
+    __syncthreads();
+    partial[tid] += v;
+    __syncthreads();
+  }
+  int run = partial[tid] - sum; // exclusive prefix of this thread's chunk
+  for (int b = b0; b < b1; ++b) {
+    work_start[b] = run;
+    int64_t lo = ptr_y ? ptr_y[b] : 0;
+    int64_t hi = ptr_y ? ptr_y[b + 1] : m;
+    int len = (int)max((int64_t)0, hi - lo);
+    run += (len + per_item - 1) / per_item;
+  }
+  if (tid == kPlanThreads - 1)
+    work_start[num_segments] = partial[tid];
+}
+
+// ---- compaction -----------------------------------------------------------
+
+constexpr int kCompactQueries = kBlock; // queries per workgroup
+
+// Block-wide exclusive scan of one int per thread; returns the exclusive
+// prefix, *total receives the block sum.
+__device__ __forceinline__ int block_exclusive_scan(int v, int *lds,
+                                                    int *total) {
+  const int tid = threadIdx.x;
+  lds[tid] = v;
+  __syncthreads();
+  for (int off = 1; off < kBlock; off <<= 1) {
+    int t = tid >= off ? lds[tid - off] : 0;
+    __syncthreads();
+    lds[tid] += t;
+    __syncthreads();
+  }
+  *total = lds[kBlock - 1];
+  return lds[tid] - v;
+}
+
+__global__ __launch_bounds__(kBlock) void block_sum_kernel(
+    const int *__restrict__ count, int m, int64_t *__restrict__ block_sums) {
+  __shared__ int lds[kBlock];
+  const int q = blockIdx.x * kCompactQueries + threadIdx.x;
+  int total;
+  block_exclusive_scan(q < m ? count[q] : 0, lds, &total);
+  if (threadIdx.x == 0)
+    block_sums[blockIdx.x] = total;
+}
+
+// Single workgroup: in-place exclusive scan of the block sums, total -> E.
+__global__ __launch_bounds__(kPlanThreads) void scan_block_sums_kernel(
+    int64_t *__restrict__ block_sums, int num_blocks,
+    int64_t *__restrict__ num_edges) {
+  __shared__ int64_t partial[kPlanThreads];
+  const int tid = threadIdx.x;
+  const int per_thread = (num_blocks + kPlanThreads - 1) / kPlanThreads;
+  const int i0 = min(tid * per_thread, num_blocks);
+  const int i1 = min(i0 + per_thread, num_blocks);
+  int64_t sum = 0;
+  for (int i = i0; i < i1; ++i)
+    sum += block_sums[i];
+  partial[tid] = sum;
+  __syncthreads();
+  for (int off = 1; off < kPlanThreads; off <<= 1) {
+    int64_t v = tid >= off ? partial[tid - off] : 0;
+    __syncthreads();
+    partial[tid] += v;
+    __syncthreads();
+  }
+  int64_t run = partial[tid] - sum;
+  for (int i = i0; i < i1; ++i) {
+    int64_t v = block_sums[i];
+    block_sums[i] = run;
+    run += v;
+  }
+  if (tid == kPlanThreads - 1)
+    *num_edges = partial[tid];
+}
+
+__global__ __launch_bounds__(kBlock) void scatter_kernel(
+    const int *__restrict__ idx, const float *__restrict__ dist,
+    const int *__restrict__ count, int m, int slots, int group_shift,
+    const int64_t *__restrict__ block_offsets,
+    const int64_t *__restrict__ num_edges, int64_t *__restrict__ edges,
+    float *__restrict__ dist_out) {
+  __shared__ int lds[kBlock];
+  __shared__ int s_count[kCompactQueries];
+  __shared__ int s_offset[kCompactQueries];
+  const int tid = threadIdx.x;
+  const int q0 = blockIdx.x * kCompactQueries;
+  const int q = q0 + tid;
+  const int c = q < m ? count[q] : 0;
+  int total;
+  const int off = block_exclusive_scan(c, lds, &total);
+  s_count[tid] = c;
+  s_offset[tid] = off;
+  __syncthreads();
+  if (total == 0)
+    return;
+
+  const int64_t E = *num_edges;
+  const int64_t base = block_offsets[blockIdx.x];
+  const int nq = min(kCompactQueries, m - q0);
+  // 2^group_shift consecutive threads walk the slots of one query, so that
+  // reads of the slot rows and writes of the edge columns stay contiguous.
+  const int group = 1 << group_shift;
+  const int sub = tid & (group - 1);
+  const int rows_per_pass = kBlock >> group_shift;
+  for (int ql = tid >> group_shift; ql < nq; ql += rows_per_pass) {
+    const int cq = s_count[ql];
+    const int64_t row_base = (int64_t)(q0 + ql) * slots;
+    const int64_t e0 = base + s_offset[ql];
+    for (int s = sub; s < cq; s += group) {
+      edges[e0 + s] = q0 + ql;
+      edges[E + e0 + s] = idx[row_base + s];
+      if (dist_out)
+        dist_out[e0 + s] = dist[row_base + s];
+    }
+  }
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+} // namespace
+
+hipError_t launch_plan(const int64_t *ptr_y, int m, int num_segments,
+                       int per_item, int *work_start, hipStream_t stream) {
+  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(kPlanThreads), 0, stream, ptr_y,
+                     m, num_segments, per_item, work_start);
+  return hipGetLastError();
+}
+
+size_t compact_workspace_bytes(int m) {
+  const int blocks = (m + kCompactQueries - 1) / kCompactQueries;
+  return align256(sizeof(int64_t) * (size_t)(blocks + 1));
+}
+
+hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
+                          int64_t *num_edges, float *dist_out, void *workspace,
+                          hipStream_t stream) {
+  const int blocks = (m + kCompactQueries - 1) / kCompactQueries;
+  int64_t *block_sums = static_cast<int64_t *>(workspace);
+  int group_shift = 0;
+  while ((1 << group_shift) < dense.slots && group_shift < 8)
+    ++group_shift;
+  hipLaunchKernelGGL(block_sum_kernel, dim3(blocks), dim3(kBlock), 0, stream,
+                     dense.count, m, block_sums);
+  hipLaunchKernelGGL(scan_block_sums_kernel, dim3(1), dim3(kPlanThreads), 0,
+                     stream, block_sums, blocks, num_edges);
+  hipLaunchKernelGGL(scatter_kernel, dim3(blocks), dim3(kBlock), 0, stream,
+                     dense.idx, dense.dist, dense.count, m, dense.slots,
+                     group_shift, block_sums, num_edges, edges, dist_out);
+  return hipGetLastError();
+}
+
+} // namespace pca

@@ -1,0 +1,216 @@
+// TorchScript operator binding: registers `torch_cluster::knn` and
+// `torch_cluster::radius` with the reference's operator signatures
+// (csrc/knn.cpp:22-40, csrc/radius.cpp:22-39) on top of the C ABI in
+// include/pca_neighbors.h.  Tensor validation, allocation through PyTorch's
+// caching allocator, the current HIP stream and the single host read of the
+// edge count live here; the kernels never see a torch type.
+//
+// Validation and error texts follow the reference's GPU host wrappers
+// (csrc/cuda/knn_cuda.cu:91-114, csrc/cuda/radius_cuda.cu:49-73,
+// csrc/cuda/utils.cuh:5-9).  There is no CPU implementation behind these
+// operators: tensors that are not on an AMD GPU are rejected.
+#include <ATen/ATen.h>
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
+#include <hip/hip_version.h>
+#include <torch/library.h>
+
+#include <optional>
+
+#include "../../include/pca_neighbors.h"
+
+namespace {
+
+#define PCA_CHECK_GPU(x)                                                       \
+  TORCH_CHECK((x).device().is_cuda(), #x " must be CUDA tensor")
+#define PCA_CHECK_CONTIGUOUS(x)                                                \
+  TORCH_CHECK((x).is_contiguous(), #x " must be contiguous")
+#define PCA_CHECK_INPUT(cond) TORCH_CHECK(cond, "Input mismatch")
+
+int dtype_code(const at::Tensor &x) {
+  switch (x.scalar_type()) {
+  case at::kFloat:
+    return PCA_F32;
+  case at::kDouble:
+    return PCA_F64;
+  case at::kHalf:
+    return PCA_F16;
+  case at::kBFloat16:
+    return PCA_BF16;
+  default:
+    TORCH_CHECK(false, "unsupported element type ", x.scalar_type());
+  }
+}
+
+// Restores the previously current device when it goes out of scope
+// (the reference calls c10::cuda::MaybeSetDevice, knn_cuda.cu:116).
+struct DeviceScope {
+  int previous = -1;
+  explicit DeviceScope(int device) {
+    TORCH_CHECK(hipGetDevice(&previous) == hipSuccess, "hipGetDevice failed");
+    if (previous != device) {
+      TORCH_CHECK(hipSetDevice(device) == hipSuccess, "hipSetDevice failed");
+    } else {
+      previous = -1;
+    }
+  }
+  ~DeviceScope() {
+    if (previous >= 0)
+      (void)hipSetDevice(previous);
+  }
+};
+
+void check_status(int status) {
+  if (status == PCA_OK)
+    return;
+  const char *detail = pca_last_error();
+  TORCH_CHECK(false, (detail && detail[0]) ? detail
+                                           : pca_status_string(status));
+}
+
+struct Segments {
+  const int64_t *ptr_x = nullptr;
+  const int64_t *ptr_y = nullptr;
+  int64_t count = 1;
+  at::Tensor keep_x, keep_y;
+};
+
+// One missing pointer is replaced by [0, N] like the reference does
+// (knn_cuda.cu:100-112); both missing = one segment, no device array needed.
+Segments resolve_segments(const at::Tensor &x, const at::Tensor &y,
+                          std::optional<at::Tensor> ptr_x,
+                          std::optional<at::Tensor> ptr_y) {
+  Segments s;
+  if (ptr_x.has_value()) {
+    PCA_CHECK_GPU(ptr_x.value());
+    PCA_CHECK_INPUT(ptr_x.value().dim() == 1);
+  }
+  if (ptr_y.has_value()) {
+    PCA_CHECK_GPU(ptr_y.value());
+    PCA_CHECK_INPUT(ptr_y.value().dim() == 1);
+  }
+  if (!ptr_x.has_value() && !ptr_y.has_value())
+    return s;
+  if (!ptr_x.has_value())
+    ptr_x = at::arange(0, x.size(0) + 1, x.size(0),
+                       x.options().dtype(at::kLong));
+  if (!ptr_y.has_value())
+    ptr_y = at::arange(0, y.size(0) + 1, y.size(0),
+                       y.options().dtype(at::kLong));
+  PCA_CHECK_INPUT(ptr_x.value().numel() == ptr_y.value().numel());
+  PCA_CHECK_INPUT(ptr_x.value().numel() >= 2);
+  s.keep_x = ptr_x.value().to(at::kLong).contiguous();
+  s.keep_y = ptr_y.value().to(at::kLong).contiguous();
+  s.ptr_x = s.keep_x.data_ptr<int64_t>();
+  s.ptr_y = s.keep_y.data_ptr<int64_t>();
+  s.count = s.keep_x.numel() - 1;
+  return s;
+}
+
+at::Tensor finish(const at::Tensor &edges, const at::Tensor &num_edges) {
+  // the only host synchronisation of the operator: the edge count sizes the
+  // result (the reference synchronises in its masked_selects)
+  const int64_t E = num_edges.item<int64_t>();
+  return edges.narrow(0, 0, 2 * E).view({2, E});
+}
+
+at::Tensor knn(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
+               std::optional<at::Tensor> ptr_y, int64_t k, bool cosine,
+               int64_t num_workers) {
+  (void)num_workers; // unused by the reference as well (csrc/cpu/knn_cpu.cpp)
+  PCA_CHECK_GPU(x);
+  PCA_CHECK_CONTIGUOUS(x);
+  PCA_CHECK_INPUT(x.dim() == 2);
+  PCA_CHECK_GPU(y);
+  PCA_CHECK_CONTIGUOUS(y);
+  PCA_CHECK_INPUT(y.dim() == 2);
+  PCA_CHECK_INPUT(x.size(1) == y.size(1));
+  PCA_CHECK_INPUT(x.scalar_type() == y.scalar_type());
+  PCA_CHECK_INPUT(x.get_device() == y.get_device());
+  TORCH_CHECK(k <= PCA_KNN_MAX_K, "`k` needs to smaller than or equal to 100");
+  TORCH_CHECK(k >= 1, "`k` needs to be positive");
+
+  Segments seg = resolve_segments(x, y, ptr_x, ptr_y);
+  DeviceScope scope(x.get_device());
+  auto long_opts = x.options().dtype(at::kLong);
+  const int64_t n = x.size(0), m = y.size(0), d = x.size(1);
+  if (n == 0 || m == 0)
+    return at::empty({2, 0}, long_opts);
+
+  const int dtype = dtype_code(x);
+  const size_t ws_bytes = pca_knn_workspace_bytes(n, m, d, seg.count, k, dtype);
+  TORCH_CHECK(ws_bytes > 0, "problem size not supported");
+  auto workspace =
+      at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+  auto edges = at::empty({2 * m * k}, long_opts);
+  auto num_edges = at::empty({1}, long_opts);
+
+  hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
+  check_status(pca_knn(x.data_ptr(), y.data_ptr(), seg.ptr_x, seg.ptr_y, n, m,
+                       d, seg.count, k, cosine ? 1 : 0, dtype,
+                       edges.data_ptr<int64_t>(),
+                       num_edges.data_ptr<int64_t>(), nullptr,
+                       workspace.data_ptr(), ws_bytes, stream));
+  return finish(edges, num_edges);
+}
+
+at::Tensor radius(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
+                  std::optional<at::Tensor> ptr_y, double r,
+                  int64_t max_num_neighbors, int64_t num_workers,
+                  bool ignore_same_index) {
+  (void)num_workers;
+  PCA_CHECK_GPU(x);
+  PCA_CHECK_CONTIGUOUS(x);
+  PCA_CHECK_INPUT(x.dim() == 2);
+  PCA_CHECK_GPU(y);
+  PCA_CHECK_CONTIGUOUS(y);
+  PCA_CHECK_INPUT(y.dim() == 2);
+  PCA_CHECK_INPUT(x.size(1) == y.size(1));
+  PCA_CHECK_INPUT(x.scalar_type() == y.scalar_type());
+  PCA_CHECK_INPUT(x.get_device() == y.get_device());
+  TORCH_CHECK(max_num_neighbors >= 1,
+              "`max_num_neighbors` needs to be positive");
+
+  Segments seg = resolve_segments(x, y, ptr_x, ptr_y);
+  DeviceScope scope(x.get_device());
+  auto long_opts = x.options().dtype(at::kLong);
+  const int64_t n = x.size(0), m = y.size(0), d = x.size(1);
+  if (n == 0 || m == 0)
+    return at::empty({2, 0}, long_opts);
+
+  const int dtype = dtype_code(x);
+  const size_t ws_bytes = pca_radius_workspace_bytes(n, m, d, seg.count,
+                                                     max_num_neighbors, dtype);
+  TORCH_CHECK(ws_bytes > 0, "problem size not supported");
+  auto workspace =
+      at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+  const int64_t slots = pca_radius_slots(n, max_num_neighbors);
+  auto edges = at::empty({2 * m * slots}, long_opts);
+  auto num_edges = at::empty({1}, long_opts);
+
+  hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
+  check_status(pca_radius(x.data_ptr(), y.data_ptr(), seg.ptr_x, seg.ptr_y, n,
+                          m, d, seg.count, r, max_num_neighbors,
+                          ignore_same_index ? 1 : 0, dtype,
+                          edges.data_ptr<int64_t>(),
+                          num_edges.data_ptr<int64_t>(), workspace.data_ptr(),
+                          ws_bytes, stream));
+  return finish(edges, num_edges);
+}
+
+// The stock loader of the reference package calls this
+// (torch_cluster/__init__.py:23, csrc/version.cpp:26-41).
+int64_t cuda_version() { return HIP_VERSION; }
+
+} // namespace
+
+TORCH_LIBRARY(torch_cluster, m) {
+  m.def("knn(Tensor x, Tensor y, Tensor? ptr_x, Tensor? ptr_y, int k, "
+        "bool cosine, int num_workers) -> Tensor",
+        &knn);
+  m.def("radius(Tensor x, Tensor y, Tensor? ptr_x, Tensor? ptr_y, float r, "
+        "int max_num_neighbors, int num_workers, bool ignore_same_index) "
+        "-> Tensor",
+        &radius);
+  m.def("cuda_version() -> int", &cuda_version);
+}
