@@ -1,0 +1,116 @@
+"""ctypes binding of the C ABI (``include/pca_neighbors.h``) for torch tensors.
+
+The TorchScript operators go through the same entry points from C++; this
+module lets Python call them directly -- with the per-edge distances, on an
+explicit stream, or without the final host read of the edge count.
+"""
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from ._native import PCA_F32, capi
+
+
+class PcaError(RuntimeError):
+    def __init__(self, status: int):
+        detail = capi.pca_last_error().decode()
+        text = detail or capi.pca_status_string(status).decode()
+        super().__init__(text)
+        self.status = status
+
+
+def _check(status: int):
+    if status != 0:
+        raise PcaError(status)
+
+
+def _dev_ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream_handle(stream: Optional[torch.cuda.Stream], device):
+    s = stream if stream is not None else torch.cuda.current_stream(device)
+    return ctypes.c_void_p(s.cuda_stream)
+
+
+def _segments(ptr_x, ptr_y):
+    if ptr_x is None and ptr_y is None:
+        return None, None, 1
+    assert ptr_x is not None and ptr_y is not None
+    assert ptr_x.dtype == torch.long and ptr_y.dtype == torch.long
+    assert ptr_x.is_contiguous() and ptr_y.is_contiguous()
+    assert ptr_x.numel() == ptr_y.numel()
+    return ptr_x, ptr_y, ptr_x.numel() - 1
+
+
+def knn_launch(x, y, ptr_x, ptr_y, k: int, cosine: bool = False,
+               want_dist: bool = False, stream=None):
+    """Queues ``pca_knn``; returns (edges buffer [2*m*k], num_edges [1] on the
+    device, dist buffer or None, workspace).  Nothing is synchronised."""
+    assert x.is_cuda and y.is_cuda and x.is_contiguous() and y.is_contiguous()
+    assert x.dtype == torch.float32 and y.dtype == torch.float32
+    n, d = x.shape
+    m = y.shape[0]
+    ptr_x, ptr_y, nseg = _segments(ptr_x, ptr_y)
+    ws_bytes = capi.pca_knn_workspace_bytes(n, m, d, nseg, k, PCA_F32)
+    if ws_bytes == 0:
+        # let the entry point produce the precise error
+        ws_bytes = 256
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    edges = torch.empty(max(2 * m * max(k, 0), 1), dtype=torch.long,
+                        device=x.device)
+    num_edges = torch.empty(1, dtype=torch.long, device=x.device)
+    dist = (torch.empty(max(m * max(k, 0), 1), dtype=torch.float32,
+                        device=x.device) if want_dist else None)
+    _check(capi.pca_knn(_dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x),
+                        _dev_ptr(ptr_y), n, m, d, nseg, k, int(cosine),
+                        PCA_F32, _dev_ptr(edges), _dev_ptr(num_edges),
+                        _dev_ptr(dist), _dev_ptr(ws), ws_bytes,
+                        _stream_handle(stream, x.device)))
+    return edges, num_edges, dist, ws
+
+
+def knn_edges(x, y, ptr_x=None, ptr_y=None, k: int = 1, cosine: bool = False,
+              want_dist: bool = False,
+              stream=None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """``[2, E]`` edges (and the ``[E]`` distances when asked for)."""
+    edges, num_edges, dist, _ws = knn_launch(x, y, ptr_x, ptr_y, k, cosine,
+                                             want_dist, stream)
+    e = int(num_edges.item())
+    out = edges[:2 * e].view(2, e)
+    return out, (dist[:e] if dist is not None else None)
+
+
+def radius_launch(x, y, ptr_x, ptr_y, r: float, max_num_neighbors: int,
+                  ignore_same_index: bool = False, stream=None):
+    assert x.is_cuda and y.is_cuda and x.is_contiguous() and y.is_contiguous()
+    assert x.dtype == torch.float32 and y.dtype == torch.float32
+    n, d = x.shape
+    m = y.shape[0]
+    ptr_x, ptr_y, nseg = _segments(ptr_x, ptr_y)
+    ws_bytes = capi.pca_radius_workspace_bytes(n, m, d, nseg,
+                                               max_num_neighbors, PCA_F32)
+    if ws_bytes == 0:
+        ws_bytes = 256
+    slots = capi.pca_radius_slots(n, max_num_neighbors)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    edges = torch.empty(max(2 * m * slots, 1), dtype=torch.long,
+                        device=x.device)
+    num_edges = torch.empty(1, dtype=torch.long, device=x.device)
+    _check(capi.pca_radius(_dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x),
+                           _dev_ptr(ptr_y), n, m, d, nseg, float(r),
+                           max_num_neighbors, int(ignore_same_index), PCA_F32,
+                           _dev_ptr(edges), _dev_ptr(num_edges), _dev_ptr(ws),
+                           ws_bytes, _stream_handle(stream, x.device)))
+    return edges, num_edges, ws
+
+
+def radius_edges(x, y, ptr_x=None, ptr_y=None, r: float = 1.0,
+                 max_num_neighbors: int = 32, ignore_same_index: bool = False,
+                 stream=None) -> torch.Tensor:
+    edges, num_edges, _ws = radius_launch(x, y, ptr_x, ptr_y, r,
+                                          max_num_neighbors,
+                                          ignore_same_index, stream)
+    e = int(num_edges.item())
+    return edges[:2 * e].view(2, e)

@@ -1,0 +1,275 @@
+"""GPU parity of the kNN path against the CPU oracle, through the C ABI and
+through the registered operator / Python entry points.
+
+Bar: integer outputs (edge indices, counts, order) bit-exact against the
+oracle evaluated with fused multiply-adds (the arithmetic the kernels use);
+distances bit-exact as well.  Against float64 brute force the neighbour sets
+may differ only where distances tie within 1e-6 relative.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import pytorch_cluster_amd as pca  # noqa: E402
+from pytorch_cluster_amd import capi, testing  # noqa: E402
+from gpu_common import (DEV, dev, gpu_knn, oracle_knn_edges,  # noqa: E402
+                        ragged_ptrs)
+from helpers import (brute_force_knn_f64, check_knn_against_exact,  # noqa
+                     to_set)
+
+
+def tensor(v, dtype=torch.float32):
+    return torch.tensor(v, dtype=dtype, device=DEV)
+
+
+# ---- the reference's fixtures (test/test_knn.py:16-75, README.md:188-191) --
+
+def test_reference_fixtures():
+    x = tensor([[-1, -1], [-1, +1], [+1, +1], [+1, -1],
+                [-1, -1], [-1, +1], [+1, +1], [+1, -1]])
+    y = tensor([[1, 0], [-1, 0]])
+    batch_x = tensor([0, 0, 0, 0, 1, 1, 1, 1], torch.long)
+    batch_y = tensor([0, 1], torch.long)
+
+    e = pca.knn(x, y, 2)
+    assert to_set(e.cpu()) == {(0, 2), (0, 3), (1, 0), (1, 1)}
+    jit = torch.jit.script(pca.knn)
+    assert to_set(jit(x, y, 2).cpu()) == {(0, 2), (0, 3), (1, 0), (1, 1)}
+    e = pca.knn(x, y, 2, batch_x, batch_y)
+    assert to_set(e.cpu()) == {(0, 2), (0, 3), (1, 4), (1, 5)}
+    e = pca.knn(x, y, 2, batch_x, batch_y, cosine=True)
+    assert to_set(e.cpu()) == {(0, 2), (0, 3), (1, 4), (1, 5)}
+    batch_x = tensor([0, 0, 0, 0, 2, 2, 2, 2], torch.long)
+    batch_y = tensor([0, 2], torch.long)
+    e = pca.knn(x, y, 2, batch_x, batch_y)
+    assert to_set(e.cpu()) == {(0, 2), (0, 3), (1, 4), (1, 5)}
+    assert e.dtype == torch.long and e.is_cuda and e.is_contiguous()
+
+
+def test_reference_knn_graph_fixtures():
+    x = tensor([[-1, -1], [-1, +1], [+1, +1], [+1, -1]])
+    e = pca.knn_graph(x, k=2, flow='target_to_source')
+    assert to_set(e.cpu()) == {(0, 1), (0, 3), (1, 0), (1, 2), (2, 1), (2, 3),
+                               (3, 0), (3, 2)}
+    e = pca.knn_graph(x, k=2, flow='source_to_target')
+    assert to_set(e.cpu()) == {(1, 0), (3, 0), (0, 1), (2, 1), (1, 2), (3, 2),
+                               (0, 3), (2, 3)}
+    jit = torch.jit.script(pca.knn_graph)
+    e = jit(x, k=2, flow='source_to_target')
+    assert to_set(e.cpu()) == {(1, 0), (3, 0), (0, 1), (2, 1), (1, 2), (3, 2),
+                               (0, 3), (2, 3)}
+    x = tensor([[-1., -1.], [-1., 1.], [1., -1.], [1., 1.]])
+    batch = tensor([0, 0, 0, 0], torch.long)
+    e = pca.knn_graph(x, k=2, batch=batch, loop=False)
+    assert e.tolist() == [[1, 2, 0, 3, 0, 3, 1, 2], [0, 0, 1, 1, 2, 2, 3, 3]]
+
+
+def test_knn_graph_large_vs_ckdtree():
+    # test/test_knn.py:78-88
+    import scipy.spatial
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(1000, 3, generator=g)
+    e = pca.knn_graph(x.to(DEV), k=5, flow='target_to_source', loop=True)
+    _, col = scipy.spatial.cKDTree(x.numpy()).query(x.numpy(), k=5)
+    truth = {(i, j) for i, ns in enumerate(col) for j in ns}
+    assert to_set(e.cpu()) == truth
+
+
+# ---- bit-exact parity against the oracle -----------------------------------
+
+@pytest.mark.parametrize("d", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("k", [1, 7, 16, 17, 32, 33, 64, 100])
+def test_parity_single_segment(oracle, d, k):
+    rng = np.random.default_rng(100 * d + k)
+    n = int(rng.choice([1023, 1024, 1025, 2500]))
+    m = int(rng.choice([255, 256, 257, 700]))
+    x = rng.random((n, d), dtype=np.float32)
+    y = rng.random((m, d), dtype=np.float32)
+    got, gd = gpu_knn(x, y, None, None, k)
+    want, wd = oracle_knn_edges(oracle, x, y, None, None, k)
+    assert got.shape == want.shape
+    assert (got == want).all()
+    assert (gd == wd).all()
+
+
+@pytest.mark.parametrize("d,k,segments", [(3, 5, 2), (3, 21, 16), (2, 16, 7),
+                                          (4, 9, 33), (8, 24, 5), (3, 48, 3)])
+def test_parity_ragged_segments(oracle, d, k, segments):
+    rng = np.random.default_rng(d * 1000 + k * 10 + segments)
+    n, m = 6000, 1900
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    y = rng.standard_normal((m, d)).astype(np.float32)
+    ptr_x = ragged_ptrs(rng, n, segments)
+    ptr_y = ragged_ptrs(rng, m, segments)
+    got, gd = gpu_knn(x, y, ptr_x, ptr_y, k)
+    want, wd = oracle_knn_edges(oracle, x, y, ptr_x, ptr_y, k)
+    assert got.shape == want.shape
+    assert (got == want).all()
+    assert (gd == wd).all()
+
+
+def test_k_larger_than_segment_and_empty_segments(oracle):
+    rng = np.random.default_rng(5)
+    x = rng.random((40, 3), dtype=np.float32)
+    y = rng.random((600, 3), dtype=np.float32)
+    ptr_x = np.array([0, 3, 3, 40, 40])
+    ptr_y = np.array([0, 300, 310, 599, 600])
+    got, _ = gpu_knn(x, y, ptr_x, ptr_y, 5)
+    want, _ = oracle_knn_edges(oracle, x, y, ptr_x, ptr_y, 5)
+    assert (got == want).all()
+    counts = np.bincount(got[0], minlength=600)
+    assert (counts[:300] == 3).all() and (counts[300:310] == 0).all()
+    assert (counts[310:599] == 5).all() and counts[599] == 0
+
+
+def test_exact_ties_keep_lowest_rows(oracle):
+    # integer grid: many exactly equal distances; order must be by
+    # (distance, row) -- float64 stable brute force is the independent check
+    rng = np.random.default_rng(11)
+    x = rng.integers(0, 5, (3000, 3)).astype(np.float32)
+    y = rng.integers(0, 5, (500, 3)).astype(np.float32)
+    ptr_x = np.array([0, 1000, 3000])
+    ptr_y = np.array([0, 200, 500])
+    for k in (6, 30):
+        got, gd = gpu_knn(x, y, ptr_x, ptr_y, k)
+        rows, d2 = brute_force_knn_f64(x, y, ptr_x, ptr_y, k)
+        assert (got[1].reshape(500, k) == rows).all()
+        assert (gd.reshape(500, k) == d2).all()
+
+
+def test_duplicate_points(oracle):
+    x = np.zeros((700, 3), dtype=np.float32)
+    got, gd = gpu_knn(x, x[:300], None, None, 9)
+    assert (got[1].reshape(300, 9) == np.arange(9)).all()
+    assert (gd == 0).all()
+
+
+def test_sentinel_and_nan_candidates(oracle):
+    # distance >= 1e10 or NaN is never returned
+    # (csrc/cuda/knn_cuda.cu:48,68 in the reference)
+    x = np.array([[0.0, 0.0], [1.0, 0.0], [2e5, 0.0], [np.nan, 0.0],
+                  [3.0, 0.0], [np.inf, 0.0]], dtype=np.float32)
+    y = np.array([[0.0, 0.0], [np.nan, 1.0]], dtype=np.float32)
+    got, gd = gpu_knn(x, y, None, None, 5)
+    want, wd = oracle_knn_edges(oracle, x, y, None, None, 5)
+    assert got.tolist() == want.tolist() == [[0, 0, 0], [0, 1, 4]]
+    assert gd.tolist() == [0.0, 1.0, 9.0]
+
+
+@pytest.mark.parametrize("d,k", [(2, 4), (3, 16), (3, 40), (6, 10)])
+def test_cosine_parity(oracle, d, k):
+    rng = np.random.default_rng(d + k)
+    x = rng.standard_normal((2100, d)).astype(np.float32)
+    y = rng.standard_normal((333, d)).astype(np.float32)
+    ptr_x = np.array([0, 900, 2100])
+    ptr_y = np.array([0, 100, 333])
+    got, gd = gpu_knn(x, y, ptr_x, ptr_y, k, cosine=True)
+    want, wd = oracle_knn_edges(oracle, x, y, ptr_x, ptr_y, k, cosine=True)
+    assert got.shape == want.shape
+    assert (got == want).all()
+    assert (gd == wd).all()
+    # slightly negative cosine distances (x == y up to scale) stay ordered
+    got, gd = gpu_knn(x, 3.0 * x[:64], None, None, 3, cosine=True)
+    want, wd = oracle_knn_edges(oracle, x, 3.0 * x[:64], None, None, 3,
+                                cosine=True)
+    assert (got == want).all() and (gd == wd).all()
+
+
+def test_two_queries_per_lane_path(oracle, monkeypatch):
+    rng = np.random.default_rng(77)
+    x = rng.random((5000, 3), dtype=np.float32)
+    y = rng.random((1500, 3), dtype=np.float32)
+    ptr_x = np.array([0, 2000, 5000])
+    ptr_y = np.array([0, 515, 1500])
+    want, wd = oracle_knn_edges(oracle, x, y, ptr_x, ptr_y, 16)
+    for qpt in ("1", "2"):
+        monkeypatch.setenv("PCA_KNN_QUERIES_PER_LANE", qpt)
+        got, gd = gpu_knn(x, y, ptr_x, ptr_y, 16)
+        assert (got == want).all() and (gd == wd).all()
+
+
+def test_against_float64_within_tie_tolerance():
+    rng = np.random.default_rng(9)
+    x = rng.random((4000, 3), dtype=np.float32)
+    ptr = np.array([0, 1500, 4000])
+    got, _ = gpu_knn(x, x, ptr, ptr, 12, want_dist=False)
+    bad = check_knn_against_exact(got, x, x, ptr, ptr, 12)
+    assert bad <= 2  # queries whose k-th and (k+1)-th distances tie in fp32
+
+
+def test_operator_errors():
+    x = torch.rand(10, 3, device=DEV)
+    op = torch.ops.torch_cluster.knn
+    with pytest.raises(RuntimeError, match="smaller than or equal to 100"):
+        op(x, x, None, None, 101, False, 1)
+    with pytest.raises(RuntimeError, match="must be contiguous"):
+        op(torch.rand(3, 10, device=DEV).t(), x, None, None, 2, False, 1)
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        op(x, torch.rand(10, 2, device=DEV), None, None, 2, False, 1)
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        op(x, x, torch.tensor([0, 10], device=DEV),
+           torch.tensor([0, 5, 10], device=DEV), 2, False, 1)
+    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
+        op(x.cpu(), x, None, None, 2, False, 1)
+
+
+def test_runs_on_the_current_stream(oracle):
+    rng = np.random.default_rng(21)
+    x = rng.random((3000, 3), dtype=np.float32)
+    want, _ = oracle_knn_edges(oracle, x, x, None, None, 8)
+    xs = dev(x)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        e = pca.knn(xs, xs, 8)
+    side.synchronize()
+    assert (e.cpu().numpy() == want).all()
+
+
+# ---- BASELINE configurations -----------------------------------------------
+
+def test_config1_knn_graph_1024(oracle):
+    data = testing.uniform_cloud(0)
+    x = data["x"]
+    e = pca.knn_graph(x.to(DEV), k=16, loop=False, flow='source_to_target')
+    want = oracle.knn_graph(x.numpy(), 16, loop=False,
+                            flow='source_to_target')
+    assert e.shape == (2, 16384)
+    assert (e.cpu().numpy() == want).all()
+
+
+def test_config2_batched_knn_graph(oracle):
+    data = testing.uniform_batched(0)
+    x, batch = data["x"], data["batch"]
+    e = pca.knn_graph(x.to(DEV), k=20, batch=batch.to(DEV), loop=False)
+    want = oracle.knn_graph(x.numpy(), 20, batch.numpy(), loop=False)
+    assert e.shape == (2, 16 * 4096 * 20)
+    assert (e.cpu().numpy() == want).all()
+
+
+def test_config5_ragged_lidar_full_size(oracle):
+    data = testing.lidar_scans(0)
+    x, y = data["x"], data["y"]
+    bx, by, B = data["batch_x"], data["batch_y"], data["batch_size"]
+    e = pca.knn(x.to(DEV), y.to(DEV), 16, bx.to(DEV), by.to(DEV),
+                batch_size=B).cpu().numpy()
+    m = y.shape[0]
+    # size-independent properties at full size
+    assert e.shape == (2, 16 * m)
+    assert (e[0] == np.repeat(np.arange(m), 16)).all()
+    assert (bx.numpy()[e[1]] == by.numpy()[e[0]]).all()
+    d2 = ((x.numpy()[e[1]].astype(np.float64)
+           - y.numpy()[e[0]].astype(np.float64)) ** 2).sum(1).reshape(m, 16)
+    assert (np.diff(d2, axis=1) >= -1e-6 * d2[:, 1:] - 1e-12).all()
+    # every query is its own nearest neighbour candidate (y is a subset of x)
+    assert (d2[:, 0] == 0).all()
+    # exact parity on a strided sample of the queries
+    ptr_x = testing.pointers(bx, B).numpy()
+    sample = np.arange(0, m, 101)
+    ys = y.numpy()[sample]
+    ptr_ys = np.searchsorted(sample, testing.pointers(by, B).numpy())
+    want, _ = oracle_knn_edges(oracle, x.numpy(), ys, ptr_x, ptr_ys, 16)
+    got = e[1].reshape(m, 16)[sample]
+    assert (got == want[1].reshape(len(sample), 16)).all()

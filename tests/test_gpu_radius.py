@@ -1,0 +1,152 @@
+"""GPU parity of the radius path against the CPU oracle (bit-exact: edge
+sets, order and counts), through the C ABI and the Python entry points."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import pytorch_cluster_amd as pca  # noqa: E402
+from pytorch_cluster_amd import testing  # noqa: E402
+from gpu_common import DEV, dev, gpu_radius, ragged_ptrs  # noqa: E402
+from helpers import to_set  # noqa: E402
+
+
+def tensor(v, dtype=torch.float32):
+    return torch.tensor(v, dtype=dtype, device=DEV)
+
+
+def to_degree(e):
+    _, counts = torch.unique(e[1], return_counts=True)
+    return counts.tolist()
+
+
+# ---- the reference's fixtures (test/test_radius.py:25-116) -----------------
+
+def test_reference_fixtures():
+    x = tensor([[-1, -1], [-1, +1], [+1, +1], [+1, -1],
+                [-1, -1], [-1, +1], [+1, +1], [+1, -1]])
+    y = tensor([[0, 0], [0, 1]])
+    batch_x = tensor([0, 0, 0, 0, 1, 1, 1, 1], torch.long)
+    batch_y = tensor([0, 1], torch.long)
+    full = {(0, 0), (0, 1), (0, 2), (0, 3), (1, 1), (1, 2), (1, 5), (1, 6)}
+    assert to_set(pca.radius(x, y, 2, max_num_neighbors=4).cpu()) == full
+    jit = torch.jit.script(pca.radius)
+    assert to_set(jit(x, y, 2, max_num_neighbors=4).cpu()) == full
+    part = {(0, 0), (0, 1), (0, 2), (0, 3), (1, 5), (1, 6)}
+    e = pca.radius(x, y, 2, batch_x, batch_y, max_num_neighbors=4)
+    assert to_set(e.cpu()) == part
+    batch_x = tensor([0, 0, 0, 0, 2, 2, 2, 2], torch.long)
+    batch_y = tensor([0, 2], torch.long)
+    e = pca.radius(x, y, 2, batch_x, batch_y, max_num_neighbors=4)
+    assert to_set(e.cpu()) == part
+
+
+def test_reference_radius_graph_fixtures():
+    x = tensor([[-1, -1], [-1, +1], [+1, +1], [+1, -1]])
+    e = pca.radius_graph(x, r=2.5, flow='target_to_source')
+    assert to_set(e.cpu()) == {(0, 1), (0, 3), (1, 0), (1, 2), (2, 1), (2, 3),
+                               (3, 0), (3, 2)}
+    e = pca.radius_graph(x, r=2.5, flow='source_to_target')
+    assert to_set(e.cpu()) == {(1, 0), (3, 0), (0, 1), (2, 1), (1, 2), (3, 2),
+                               (0, 3), (2, 3)}
+    jit = torch.jit.script(pca.radius_graph)
+    e = jit(x, r=2.5, flow='source_to_target')
+    assert to_set(e.cpu()) == {(1, 0), (3, 0), (0, 1), (2, 1), (1, 2), (3, 2),
+                               (0, 3), (2, 3)}
+    e = pca.radius_graph(x, r=100, flow='source_to_target',
+                         max_num_neighbors=1)
+    assert set(to_degree(e)) == {1}
+    same = tensor([[-1, -1]] * 4)
+    e = pca.radius_graph(same, r=100, flow='source_to_target',
+                         max_num_neighbors=1)
+    assert set(to_degree(e)) == {1}
+    x8 = tensor([[-1, -1], [-1, +1], [+1, +1], [+1, -1],
+                 [-1, -1], [-1, +1], [+1, +1], [+1, -1]])
+    batch = tensor([0, 0, 0, 0, 1, 1, 1, 1], torch.long)
+    e = pca.radius_graph(x8, r=100, batch=batch, flow='source_to_target',
+                         max_num_neighbors=1)
+    assert set(to_degree(e)) == {1}
+    assert [int(i / 4) for i in e[0].tolist()] == batch.tolist()
+    # README.md:217-220, ordered
+    x = tensor([[-1., -1.], [-1., 1.], [1., -1.], [1., 1.]])
+    e = pca.radius_graph(x, r=2.5, batch=tensor([0] * 4, torch.long))
+    assert e.tolist() == [[1, 2, 0, 3, 0, 3, 1, 2], [0, 0, 1, 1, 2, 2, 3, 3]]
+
+
+def test_radius_graph_large_vs_ckdtree():
+    # test/test_radius.py:119-133
+    import scipy.spatial
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(1000, 3, generator=g)
+    e = pca.radius_graph(x.to(DEV), r=0.5, flow='target_to_source', loop=True,
+                         max_num_neighbors=2000)
+    col = scipy.spatial.cKDTree(x.numpy()).query_ball_point(x.numpy(), r=0.5)
+    truth = {(i, j) for i, ns in enumerate(col) for j in ns}
+    assert to_set(e.cpu()) == truth
+
+
+# ---- bit-exact parity against the oracle -----------------------------------
+
+@pytest.mark.parametrize("d", [1, 2, 3, 4, 7, 16])
+@pytest.mark.parametrize("cap,ignore", [(1, False), (5, True), (32, False),
+                                        (64, True), (5000, False)])
+def test_parity_ragged(oracle, d, cap, ignore):
+    rng = np.random.default_rng(31 * d + cap)
+    n = 3000
+    x = rng.random((n, d), dtype=np.float32)
+    segments = int(rng.choice([1, 2, 9]))
+    ptr = ragged_ptrs(rng, n, segments)
+    # radius chosen so the mean degree is a few dozen in any dimension
+    r = 0.5 * (40.0 / n) ** (1.0 / d)
+    got = gpu_radius(x, x, ptr, ptr, r, cap, ignore)
+    want = oracle.radius_op(x, x, ptr, ptr, r, cap, 1, ignore)
+    assert got.shape == want.shape
+    assert (got == want).all()
+
+
+def test_parity_bipartite_with_empty_segments(oracle):
+    rng = np.random.default_rng(8)
+    x = rng.random((5000, 3), dtype=np.float32)
+    y = rng.random((777, 3), dtype=np.float32)
+    ptr_x = np.array([0, 0, 2000, 2000, 5000])
+    ptr_y = np.array([0, 100, 400, 401, 777])
+    for cap in (3, 32):
+        got = gpu_radius(x, y, ptr_x, ptr_y, 0.11, cap)
+        want = oracle.radius_op(x, y, ptr_x, ptr_y, 0.11, cap)
+        assert (got == want).all()
+
+
+def test_strict_inequality_at_the_radius(oracle):
+    # points exactly at distance r are excluded (dist < r*r, strict)
+    x = np.array([[0, 0], [3, 4], [5, 0], [0, 4.9999995]], dtype=np.float32)
+    y = np.array([[0, 0]], dtype=np.float32)
+    got = gpu_radius(x, y, None, None, 5.0, 8)
+    want = oracle.radius_op(x, y, None, None, 5.0, 8)
+    assert got.tolist() == want.tolist() == [[0, 0], [0, 3]]
+
+
+def test_operator_errors():
+    x = torch.rand(10, 3, device=DEV)
+    op = torch.ops.torch_cluster.radius
+    with pytest.raises(RuntimeError, match="must be contiguous"):
+        op(torch.rand(3, 10, device=DEV).t(), x, None, None, 1.0, 4, 1, False)
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        op(x, torch.rand(10, 2, device=DEV), None, None, 1.0, 4, 1, False)
+    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
+        op(x, x.cpu(), None, None, 1.0, 4, 1, False)
+
+
+# ---- BASELINE configuration 3 ------------------------------------------------
+
+def test_config3_gaussian_mixture_radius_graph(oracle):
+    data = testing.gaussian_mixture_batched(0)
+    x, batch = data["x"], data["batch"]
+    e = pca.radius_graph(x.to(DEV), r=0.05, batch=batch.to(DEV),
+                         max_num_neighbors=32, loop=False,
+                         batch_size=data["batch_size"])
+    want = oracle.radius_graph(x.numpy(), 0.05, batch.numpy(), loop=False,
+                               max_num_neighbors=32)
+    assert e.shape == want.shape
+    assert (e.cpu().numpy() == want).all()
+    assert (batch.numpy()[want[0]] == batch.numpy()[want[1]]).all()
