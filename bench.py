@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""Benchmark of the kNN hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one `knn(x, y, k=16, batch_x, batch_y)` call over the ragged
+LiDAR-like workload (8 scans, ~1.03 M points, every 4th point a query), inputs
+resident in HBM.  Prints ONE JSON line with whole-job queries/s, the roofline
+of the dominant kernel (brute-force distance tiles, FP32 VALU bound) measured
+with HIP events around that kernel inside the timed region, and the
+reference's CPU path timed on this host beside it.
+"""
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+K = 16
+PEAK_FP32_TFLOPS = 157.3  # MI355X vector FP32 (includes packed FP32 issue)
+FLOP_PER_PAIR = 9         # 3-D: 3 subtractions + 3 multiply-adds
+
+
+class HipEvents:
+    """hipEvent_t pairs through the HIP runtime PyTorch has loaded."""
+
+    def __init__(self, torch):
+        lib_dir = os.path.join(os.path.dirname(torch.__file__), "lib")
+        self.hip = ctypes.CDLL(os.path.join(lib_dir, "libamdhip64.so"))
+
+    def create(self):
+        ev = ctypes.c_void_p()
+        rc = self.hip.hipEventCreate(ctypes.byref(ev))
+        assert rc == 0, "hipEventCreate failed: %d" % rc
+        return ev
+
+    def elapsed_ms(self, start, stop):
+        ms = ctypes.c_float()
+        rc = self.hip.hipEventElapsedTime(ctypes.byref(ms), start, stop)
+        assert rc == 0, "hipEventElapsedTime failed: %d" % rc
+        return ms.value
+
+    def destroy(self, ev):
+        self.hip.hipEventDestroy(ev)
+
+
+def cpu_baseline(data, ptr_x, ptr_y):
+    """The reference's CPU operator (nanoflann KD-tree; single-threaded by
+    construction, `num_workers` is never read) on the same inputs, or the
+    brute-force port on a sample of the queries when it is not available."""
+    import numpy as np
+    import oracle
+
+    x = data["x"].numpy()
+    y = data["y"].numpy()
+    px, py = ptr_x.numpy(), ptr_y.numpy()
+    m = y.shape[0]
+    if oracle.have_ref():
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            e = oracle.ref_knn(x, y, px, py, K)
+            times.append(time.perf_counter() - t0)
+        assert e.shape[1] == m * K
+        return {"value": m / statistics.median(times), "unit": "queries/s",
+                "cores": 1, "kind": "reference",
+                "sample": "full workload (%d queries over %d points), median "
+                          "of 3 runs; nanoflann KD-tree operator of the "
+                          "reference, single-threaded by construction"
+                          % (m, x.shape[0])}
+    stride = 64
+    sample = np.arange(0, m, stride)
+    ys = np.ascontiguousarray(y[sample])
+    pys = np.searchsorted(sample, py)
+    t0 = time.perf_counter()
+    oracle.knn_op(x, ys, px, pys, K)
+    dt = time.perf_counter() - t0
+    return {"value": len(sample) / dt, "unit": "queries/s",
+            "cores": os.cpu_count(), "kind": "port",
+            "sample": "every %dth query (%d queries), brute-force C port with "
+                      "OpenMP" % (stride, len(sample))}
+
+
+def measured_traffic():
+    """HBM bytes per launch of the dominant kernel from the committed rocprof
+    counter summary, if there is one."""
+    import re
+    path = os.path.join(ROOT, "profiles", "knn_lowd_lidar_traffic.md")
+    try:
+        with open(path) as f:
+            found = re.search(r"hbm_bytes_per_launch:\s*(\d+)", f.read())
+        return int(found.group(1)) if found else None
+    except OSError:
+        return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy three times, so "
+                         "that a counter profile of this command can scale "
+                         "FETCH_SIZE / WRITE_SIZE by a kernel of known traffic")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not "
+                 "supported (the path shards by segment without "
+                 "communication, see DESIGN.md)" % args.gpus)
+
+    import torch
+    import pytorch_cluster_amd as pca
+    from pytorch_cluster_amd import testing
+    from pytorch_cluster_amd._native import capi
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    data = testing.lidar_scans(0)
+    B = data["batch_size"]
+    ptr_x = testing.pointers(data["batch_x"], B)
+    ptr_y = testing.pointers(data["batch_y"], B)
+    x, y = data["x"].to(dev), data["y"].to(dev)
+    bx, by = data["batch_x"].to(dev), data["batch_y"].to(dev)
+    n, m = x.shape[0], y.shape[0]
+    pairs = int(((ptr_x[1:] - ptr_x[:-1]) * (ptr_y[1:] - ptr_y[:-1])).sum())
+
+    def step():
+        return pca.knn(x, y, K, bx, by, batch_size=B)
+
+    for _ in range(args.warmup):
+        out = step()
+    torch.cuda.synchronize()
+    assert out.shape == (2, m * K)
+
+    events = HipEvents(torch)
+    pairs_of_events = [(events.create(), events.create())
+                       for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for start, stop in pairs_of_events:
+        capi.pca_time_next_search(start, stop)
+        out = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    kernel_ms = [events.elapsed_ms(a, b) for a, b in pairs_of_events]
+    for a, b in pairs_of_events:
+        events.destroy(a)
+        events.destroy(b)
+    kernel_s = sum(kernel_ms) / len(kernel_ms) / 1e3
+    flops = FLOP_PER_PAIR * pairs
+    achieved = flops / kernel_s / 1e12
+
+    result = {
+        "metric": "kNN queries/sec (k=16, 3D, 1M pts)",
+        "value": m * args.steps / elapsed,
+        "unit": "queries/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[4]: ragged LiDAR-like knn(x, y, k=16, "
+                        "batch_x, batch_y), 8 scans of 60k-200k points, "
+                        "y = every 4th point",
+            "points": n, "queries": m, "k": K, "dim": 3, "segments": B,
+            "pairs": pairs, "seed": 0,
+        },
+        "edges_per_s": m * K * args.steps / elapsed,
+        "roofline": {
+            "bound": "fp32_valu",
+            "kernel": "knn_lowd_kernel<3,16,*>",
+            "achieved": achieved,
+            "peak": PEAK_FP32_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / PEAK_FP32_TFLOPS,
+            "kernel_ms": kernel_s * 1e3,
+            "flop_per_launch": flops,
+            "traffic": measured_traffic(),
+        },
+    }
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(data, ptr_x, ptr_y)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -5,7 +5,9 @@
  * that is current on the calling thread unless a parameter says otherwise.
  * All entry points are asynchronous on `stream` (a hipStream_t passed as
  * void*; NULL = the default stream) and return a status code; they never
- * allocate, free or synchronise.  The library keeps no state between calls.
+ * allocate, free or synchronise.  The library keeps no state between calls
+ * (pca_last_error's text and the one-shot pca_time_next_search request are
+ * per calling thread).
  *
  * The reference (rusty1s/pytorch_cluster 1.6.3) has no C ABI: its boundary is
  * the TorchScript operator registry.  Each entry point below names the
@@ -71,6 +73,16 @@ const char *pca_status_string(int status);
 
 /* Text describing the last failure on the calling thread ("" if none). */
 const char *pca_last_error(void);
+
+/*
+ * Measurement hook: the next pca_knn / pca_radius call of the calling thread
+ * records `start_event` immediately before and `stop_event` immediately after
+ * its search kernel (the dominant kernel; planning and compaction kernels stay
+ * outside) on that call's stream.  Both are hipEvent_t created by the caller
+ * with timing enabled.  The request is consumed by that one call; pass NULLs
+ * to cancel it.  No counterpart in the reference.
+ */
+int pca_time_next_search(void *start_event, void *stop_event);
 
 /* ------------------------------------------------------------------ kNN -- */
 

@@ -18,7 +18,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CAPI_PATH = os.path.join(_HERE, "libpca_neighbors.so")
 TORCH_OPS_PATH = os.path.join(_HERE, "_torch_ops.so")
 
-_BUILD_HINT = ("build it with `python -m pytorch_cluster_amd.build` "
+_BUILD_HINT = ("build it with `python pytorch_cluster_amd/build.py` "
                "(or `python -c 'import __graft_entry__ as g; g.build()'`)")
 
 PCA_F32, PCA_F64, PCA_F16, PCA_BF16 = 0, 1, 2, 3
@@ -31,6 +31,7 @@ C_ABI = {
     "pca_abi_version": (ctypes.c_int, []),
     "pca_status_string": (ctypes.c_char_p, [ctypes.c_int]),
     "pca_last_error": (ctypes.c_char_p, []),
+    "pca_time_next_search": (ctypes.c_int, [_vp, _vp]),
     "pca_knn_workspace_bytes": (ctypes.c_size_t,
                                 [_i64, _i64, _i64, _i64, _i64, ctypes.c_int]),
     "pca_knn": (ctypes.c_int,

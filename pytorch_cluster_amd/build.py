@@ -1,6 +1,8 @@
 """Builds the native libraries of this package in-tree for gfx950.
 
-    python -m pytorch_cluster_amd.build [--jobs N] [--skip-torch-ops]
+    python pytorch_cluster_amd/build.py [--jobs N] [--skip-torch-ops]
+
+(run as a script: importing the package needs the libraries built here)
 
 Outputs (next to this file, git-ignored):
   libpca_neighbors.so   HIP kernels + the C ABI of include/pca_neighbors.h

@@ -25,6 +25,29 @@ int fail(int status, const char *fmt, ...) {
   return status;
 }
 
+// one-shot request of pca_time_next_search
+thread_local hipEvent_t g_time_start = nullptr;
+thread_local hipEvent_t g_time_stop = nullptr;
+
+struct SearchTimer {
+  hipStream_t stream;
+  hipEvent_t start, stop;
+  explicit SearchTimer(hipStream_t s)
+      : stream(s), start(g_time_start), stop(g_time_stop) {
+    // consumed by this call whether or not it reaches its search kernel
+    g_time_start = g_time_stop = nullptr;
+  }
+  void begin() {
+    if (start)
+      (void)hipEventRecord(start, stream);
+  }
+  void done() {
+    if (stop)
+      (void)hipEventRecord(stop, stream);
+    stop = nullptr;
+  }
+};
+
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Carver {
@@ -101,6 +124,15 @@ const char *pca_status_string(int status) {
 
 const char *pca_last_error(void) { return g_last_error; }
 
+int pca_time_next_search(void *start_event, void *stop_event) {
+  if ((start_event == nullptr) != (stop_event == nullptr))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "start and stop events must both be given or both be NULL");
+  g_time_start = static_cast<hipEvent_t>(start_event);
+  g_time_stop = static_cast<hipEvent_t>(stop_event);
+  return PCA_OK;
+}
+
 size_t pca_knn_workspace_bytes(int64_t n, int64_t m, int64_t d,
                                int64_t num_segments, int64_t k, int dtype) {
   (void)dtype;
@@ -118,6 +150,7 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
             size_t workspace_bytes, void *stream_) {
   g_last_error[0] = 0;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  SearchTimer timer(stream);
   if ((ptr_x == nullptr) != (ptr_y == nullptr))
     return fail(PCA_ERR_INVALID_ARGUMENT,
                 "ptr_x and ptr_y must both be given or both be NULL");
@@ -176,9 +209,11 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
     return rc;
   const int bound =
       pca::plan_upper_bound((int)m, (int)num_segments, cfg.tile_queries);
+  timer.begin();
   rc = check_launch(pca::launch_knn_lowd(in, (int)k, cosine != 0, cfg,
                                          work_start, bound, dense, stream),
                     "knn_lowd_kernel");
+  timer.done();
   if (rc != PCA_OK)
     return rc;
   return check_launch(pca::launch_compact(dense, (int)m, edges, num_edges,
@@ -213,6 +248,7 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
                void *stream_) {
   g_last_error[0] = 0;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  SearchTimer timer(stream);
   if ((ptr_x == nullptr) != (ptr_y == nullptr))
     return fail(PCA_ERR_INVALID_ARGUMENT,
                 "ptr_x and ptr_y must both be given or both be NULL");
@@ -268,9 +304,11 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
     return rc;
   const int bound = pca::plan_upper_bound((int)m, (int)num_segments,
                                           pca::kRadiusQueriesPerWave);
+  timer.begin();
   rc = check_launch(pca::launch_radius(in, r2, ignore_same_index != 0,
                                        work_start, bound, dense, stream),
                     "radius_kernel");
+  timer.done();
   if (rc != PCA_OK)
     return rc;
   return check_launch(pca::launch_compact(dense, (int)m, edges, num_edges,
