@@ -70,8 +70,11 @@ bool sizes_ok(int64_t n, int64_t m, int64_t d, int64_t num_segments) {
          d <= (1 << 20) && num_segments >= 1 && num_segments <= kMaxRows;
 }
 
-size_t knn_workspace(int64_t m, int64_t num_segments, int64_t k) {
+size_t knn_workspace(int64_t n, int64_t m, int64_t d, int64_t num_segments,
+                     int64_t k) {
   size_t bytes = 0;
+  if (d > 8)
+    bytes += align256(sizeof(float) * (size_t)n); // |x| for the cosine distance
   bytes += align256(sizeof(int) * (size_t)(num_segments + 1)); // work_start
   bytes += align256(sizeof(int) * (size_t)m * (size_t)k);      // idx
   bytes += align256(sizeof(float) * (size_t)m * (size_t)k);    // dist
@@ -140,7 +143,7 @@ size_t pca_knn_workspace_bytes(int64_t n, int64_t m, int64_t d,
     num_segments = 1;
   if (!sizes_ok(n, m, d, num_segments) || k < 1 || k > PCA_KNN_MAX_K)
     return 0;
-  return knn_workspace(m, num_segments, k);
+  return knn_workspace(n, m, d, num_segments, k);
 }
 
 int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
@@ -180,15 +183,14 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
   if (x == nullptr || y == nullptr || edges == nullptr)
     return fail(PCA_ERR_INVALID_ARGUMENT, "x, y or edges is NULL");
   if (workspace == nullptr || ((uintptr_t)workspace & 255) != 0 ||
-      workspace_bytes < knn_workspace(m, num_segments, k))
+      workspace_bytes < knn_workspace(n, m, d, num_segments, k))
     return fail(PCA_ERR_WORKSPACE, "workspace needs %zu bytes, 256-aligned",
-                knn_workspace(m, num_segments, k));
+                knn_workspace(n, m, d, num_segments, k));
 
-  if (!pca::knn_lowd_supported((int)d, (int)k, cosine != 0))
-    return fail(PCA_ERR_UNSUPPORTED, "kNN for d=%lld is not built",
-                (long long)d);
+  const bool low_d = pca::knn_lowd_supported((int)d, (int)k, cosine != 0);
 
   Carver ws(workspace);
+  float *x_norm = d > 8 ? ws.take<float>((size_t)n) : nullptr;
   int *work_start = ws.take<int>((size_t)num_segments + 1);
   pca::DenseResult dense;
   dense.idx = ws.take<int>((size_t)m * k);
@@ -201,7 +203,9 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
 
   pca::SearchInput in{x,      y,      ptr_x,  ptr_y,
                       (int)n, (int)m, (int)d, (int)num_segments};
-  const pca::KnnLowdConfig cfg = pca::knn_lowd_config((int)d, (int)k, (int)m);
+  pca::KnnLowdConfig cfg = pca::knn_lowd_config((int)d, (int)k, (int)m);
+  if (!low_d)
+    cfg.tile_queries = pca::kBlock; // any-dimension kernel: one query per lane
   int rc = check_launch(pca::launch_plan(ptr_y, (int)m, (int)num_segments,
                                          cfg.tile_queries, work_start, stream),
                         "plan_kernel");
@@ -209,11 +213,27 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
     return rc;
   const int bound =
       pca::plan_upper_bound((int)m, (int)num_segments, cfg.tile_queries);
-  timer.begin();
-  rc = check_launch(pca::launch_knn_lowd(in, (int)k, cosine != 0, cfg,
-                                         work_start, bound, dense, stream),
-                    "knn_lowd_kernel");
-  timer.done();
+  if (low_d) {
+    timer.begin();
+    rc = check_launch(pca::launch_knn_lowd(in, (int)k, cosine != 0, cfg,
+                                           work_start, bound, dense, stream),
+                      "knn_lowd_kernel");
+    timer.done();
+  } else {
+    if (cosine) {
+      rc = check_launch(pca::launch_row_norms(static_cast<const float *>(x),
+                                              (int)n, (int)d, x_norm, stream),
+                        "row_norm_kernel");
+      if (rc != PCA_OK)
+        return rc;
+    }
+    timer.begin();
+    rc = check_launch(pca::launch_knn_generic(in, (int)k, cosine != 0, x_norm,
+                                              work_start, bound, dense,
+                                              stream),
+                      "knn_generic_kernel");
+    timer.done();
+  }
   if (rc != PCA_OK)
     return rc;
   return check_launch(pca::launch_compact(dense, (int)m, edges, num_edges,

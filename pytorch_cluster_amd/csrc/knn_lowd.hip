@@ -1,4 +1,5 @@
 // Dispatch of the low-dimensional kNN kernels (see knn_lowd_impl.hpp).
+#include "knn_generic_impl.hpp"
 #include "knn_lowd_impl.hpp"
 
 #include <cstdlib>
@@ -69,6 +70,19 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
   }
 #undef PCA_DIM_CASE
   return hipErrorInvalidValue;
+}
+
+hipError_t launch_knn_generic(const SearchInput &in, int k, bool cosine,
+                              const float *x_norm, const int *work_start,
+                              int grid_bound, const DenseResult &out,
+                              hipStream_t stream) {
+  const int kb = k_bucket(k);
+  return cosine ? launch_knn_generic_metric<true>(in, k, kb, x_norm,
+                                                  work_start, grid_bound, out,
+                                                  stream)
+                : launch_knn_generic_metric<false>(in, k, kb, x_norm,
+                                                   work_start, grid_bound, out,
+                                                   stream);
 }
 
 } // namespace pca

@@ -63,6 +63,18 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
                            int grid_bound, const DenseResult &out,
                            hipStream_t stream);
 
+// --- knn_generic_*.hip -----------------------------------------------------
+
+// |x_i| for the cosine distance of the any-dimension kernel.
+hipError_t launch_row_norms(const float *x, int n, int d, float *norm,
+                            hipStream_t stream);
+// x_norm: [n] row norms of x (cosine only, else NULL).  One query per lane:
+// work items are tiles of kBlock queries.
+hipError_t launch_knn_generic(const SearchInput &in, int k, bool cosine,
+                              const float *x_norm, const int *work_start,
+                              int grid_bound, const DenseResult &out,
+                              hipStream_t stream);
+
 // --- radius.hip ------------------------------------------------------------
 
 constexpr int kRadiusQueriesPerWave = 8;

@@ -177,6 +177,24 @@ def test_cosine_parity(oracle, d, k):
     assert (got == want).all() and (gd == wd).all()
 
 
+@pytest.mark.parametrize("d,k,cosine", [(9, 5, False), (16, 16, False),
+                                        (17, 33, True), (33, 8, False),
+                                        (128, 32, False), (128, 32, True),
+                                        (300, 7, False), (515, 3, True)])
+def test_parity_high_dimension(oracle, d, k, cosine):
+    rng = np.random.default_rng(d * 7 + k)
+    n, m = 1500, 300
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    y = rng.standard_normal((m, d)).astype(np.float32)
+    ptr_x = np.array([0, 40, 40, 1500])
+    ptr_y = np.array([0, 100, 130, 300])
+    got, gd = gpu_knn(x, y, ptr_x, ptr_y, k, cosine=cosine)
+    want, wd = oracle_knn_edges(oracle, x, y, ptr_x, ptr_y, k, cosine=cosine)
+    assert got.shape == want.shape
+    assert (got == want).all()
+    assert (gd == wd).all()
+
+
 def test_two_queries_per_lane_path(oracle, monkeypatch):
     rng = np.random.default_rng(77)
     x = rng.random((5000, 3), dtype=np.float32)
@@ -247,6 +265,17 @@ def test_config2_batched_knn_graph(oracle):
     want = oracle.knn_graph(x.numpy(), 20, batch.numpy(), loop=False)
     assert e.shape == (2, 16 * 4096 * 20)
     assert (e.cpu().numpy() == want).all()
+
+
+def test_config4_feature_space_reduced(oracle):
+    # the 200,000 x 128 / 50,000 x 128 workload at 1/25 of the rows, Euclidean
+    # and cosine, bit-exact against the oracle
+    data = testing.feature_space(0, n=8000, m=2000, d=128)
+    x, y = data["x"], data["y"]
+    for cosine in (False, True):
+        e = pca.knn(x.to(DEV), y.to(DEV), 32, cosine=cosine).cpu().numpy()
+        want = oracle.knn(x.numpy(), y.numpy(), 32, cosine=cosine)
+        assert (e == want).all()
 
 
 def test_config5_ragged_lidar_full_size(oracle):
