@@ -10,6 +10,7 @@
 #include "device_utils.hpp"
 #include "launchers.hpp"
 
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
 
@@ -70,17 +71,43 @@ bool sizes_ok(int64_t n, int64_t m, int64_t d, int64_t num_segments) {
          d <= (1 << 20) && num_segments >= 1 && num_segments <= kMaxRows;
 }
 
+// Sizes of the pieces pca_knn carves out of the workspace, in carving order.
+struct KnnLayout {
+  size_t x_norm = 0;  // |x| (any-dimension kernel, cosine)
+  size_t sliced = 0;  // shared bounds + partial key lists of sliced segments
+  size_t work_start, idx, dist, count, compact;
+  size_t total() const {
+    return x_norm + sliced + work_start + idx + dist + count + compact;
+  }
+};
+
+KnnLayout knn_layout(int64_t n, int64_t m, int64_t d, int64_t num_segments,
+                     int64_t k) {
+  KnnLayout w;
+  if (d > 8) {
+    w.x_norm = align256(sizeof(float) * (size_t)n);
+  } else {
+    // the larger of the two metrics' needs, so one size query serves both
+    for (int cosine = 0; cosine < 2; ++cosine) {
+      const pca::KnnLowdConfig cfg = pca::knn_lowd_config(
+          (int)d, (int)k, (int)n, (int)m, (int)num_segments, cosine != 0);
+      w.sliced = std::max(w.sliced,
+                          pca::knn_lowd_scratch_bytes(cfg, (int)m,
+                                                      (int)num_segments,
+                                                      (int)k));
+    }
+  }
+  w.work_start = align256(sizeof(int) * (size_t)(num_segments + 1));
+  w.idx = align256(sizeof(int) * (size_t)m * (size_t)k);
+  w.dist = align256(sizeof(float) * (size_t)m * (size_t)k);
+  w.count = align256(sizeof(int) * (size_t)m);
+  w.compact = pca::compact_workspace_bytes((int)m);
+  return w;
+}
+
 size_t knn_workspace(int64_t n, int64_t m, int64_t d, int64_t num_segments,
                      int64_t k) {
-  size_t bytes = 0;
-  if (d > 8)
-    bytes += align256(sizeof(float) * (size_t)n); // |x| for the cosine distance
-  bytes += align256(sizeof(int) * (size_t)(num_segments + 1)); // work_start
-  bytes += align256(sizeof(int) * (size_t)m * (size_t)k);      // idx
-  bytes += align256(sizeof(float) * (size_t)m * (size_t)k);    // dist
-  bytes += align256(sizeof(int) * (size_t)m);                  // count
-  bytes += pca::compact_workspace_bytes((int)m);
-  return bytes;
+  return knn_layout(n, m, d, num_segments, k).total();
 }
 
 size_t radius_workspace(int64_t m, int64_t num_segments, int64_t slots) {
@@ -189,21 +216,29 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
 
   const bool low_d = pca::knn_lowd_supported((int)d, (int)k, cosine != 0);
 
-  Carver ws(workspace);
-  float *x_norm = d > 8 ? ws.take<float>((size_t)n) : nullptr;
-  int *work_start = ws.take<int>((size_t)num_segments + 1);
+  const KnnLayout lay = knn_layout(n, m, d, num_segments, k);
+  char *cursor = static_cast<char *>(workspace);
+  auto take = [&cursor](size_t bytes) {
+    char *piece = cursor;
+    cursor += bytes;
+    return static_cast<void *>(piece);
+  };
+  float *x_norm = static_cast<float *>(take(lay.x_norm));
+  void *lowd_scratch = take(lay.sliced);
+  int *work_start = static_cast<int *>(take(lay.work_start));
   pca::DenseResult dense;
-  dense.idx = ws.take<int>((size_t)m * k);
-  dense.dist = ws.take<float>((size_t)m * k);
-  dense.count = ws.take<int>((size_t)m);
+  dense.idx = static_cast<int *>(take(lay.idx));
+  dense.dist = static_cast<float *>(take(lay.dist));
+  dense.count = static_cast<int *>(take(lay.count));
   dense.slots = (int)k;
-  void *compact_ws = ws.take<char>(pca::compact_workspace_bytes((int)m));
+  void *compact_ws = take(lay.compact);
   if (dist == nullptr)
     dense.dist = nullptr;
+  pca::KnnLowdConfig cfg = pca::knn_lowd_config(
+      (int)d, (int)k, (int)n, (int)m, (int)num_segments, cosine != 0);
 
   pca::SearchInput in{x,      y,      ptr_x,  ptr_y,
                       (int)n, (int)m, (int)d, (int)num_segments};
-  pca::KnnLowdConfig cfg = pca::knn_lowd_config((int)d, (int)k, (int)m);
   if (!low_d)
     cfg.tile_queries = pca::kBlock; // any-dimension kernel: one query per lane
   int rc = check_launch(pca::launch_plan(ptr_y, (int)m, (int)num_segments,
@@ -214,11 +249,13 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
   const int bound =
       pca::plan_upper_bound((int)m, (int)num_segments, cfg.tile_queries);
   if (low_d) {
-    timer.begin();
+    // the events bracket the search kernel itself, not the bound fill and
+    // the merge around it
     rc = check_launch(pca::launch_knn_lowd(in, (int)k, cosine != 0, cfg,
-                                           work_start, bound, dense, stream),
+                                           work_start, lowd_scratch, dense,
+                                           timer.start, timer.stop, stream),
                       "knn_lowd_kernel");
-    timer.done();
+    timer.stop = nullptr;
   } else {
     if (cosine) {
       rc = check_launch(pca::launch_row_norms(static_cast<const float *>(x),

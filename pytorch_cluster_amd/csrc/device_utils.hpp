@@ -117,3 +117,10 @@ __device__ __forceinline__ int xcd_swizzle(int block, int grid) {
 }
 
 } // namespace pca
+
+// experiment switch: -DPCA_NO_SWIZZLE maps workgroup ids to tiles directly
+#ifdef PCA_NO_SWIZZLE
+#define PCA_TILE_OF_BLOCK(b, g) (b)
+#else
+#define PCA_TILE_OF_BLOCK(b, g) pca::xcd_swizzle(b, g)
+#endif

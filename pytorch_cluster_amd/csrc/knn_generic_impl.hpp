@@ -47,7 +47,7 @@ __global__ __launch_bounds__(kBlock) void knn_generic_kernel(
   __shared__ double queue[QCAP][kBlock];
 
   const int tid = threadIdx.x;
-  const int tile = xcd_swizzle(blockIdx.x, grid);
+  const int tile = PCA_TILE_OF_BLOCK(blockIdx.x, grid);
   if (tile >= work_start[num_segments])
     return;
   const int seg = find_segment(work_start, num_segments, tile);

@@ -1,4 +1,5 @@
-// Dispatch of the low-dimensional kNN kernels (see knn_lowd_impl.hpp).
+// Dispatch of the low-dimensional kNN kernels (see knn_lowd_impl.hpp) and of
+// the any-dimension kernel (knn_generic_impl.hpp).
 #include "knn_generic_impl.hpp"
 #include "knn_lowd_impl.hpp"
 
@@ -26,42 +27,123 @@ int k_bucket(int k) {
   return 0;
 }
 
+int env_int(const char *name, int fallback) {
+  const char *v = std::getenv(name);
+  return v ? std::atoi(v) : fallback;
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+__global__ __launch_bounds__(kBlock) void fill_f32_kernel(float *p, int n,
+                                                          float v) {
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < n)
+    p[i] = v;
+}
+
+template <int KB>
+void launch_merge(const KnnLowdParams &p, int queries_per_lane,
+                  int tiles_bound, hipStream_t stream) {
+  if constexpr (KB <= 32) {
+    if (queries_per_lane == 2) {
+      hipLaunchKernelGGL((knn_lowd_merge_kernel<KB, 2>), dim3(tiles_bound),
+                         dim3(kBlock), 0, stream, p);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((knn_lowd_merge_kernel<KB, 1>), dim3(tiles_bound),
+                     dim3(kBlock), 0, stream, p);
+}
+
 } // namespace
 
 bool knn_lowd_supported(int d, int k, bool /*cosine*/) {
   return d >= 1 && d <= 8 && k >= 1 && k <= 100;
 }
 
-KnnLowdConfig knn_lowd_config(int /*d*/, int k, int m) {
+KnnLowdConfig knn_lowd_config(int /*d*/, int k, int n, int m,
+                              int num_segments, bool cosine) {
   KnnLowdConfig cfg;
   cfg.kbucket = k_bucket(k);
   // Two queries per lane halve the LDS reads per distance but need twice the
   // queries to fill the 256 CUs; worth it once there are enough query tiles.
-  int qpt = (cfg.kbucket <= 32 && m >= 2 * kBlock * 256) ? 2 : 1;
-  if (const char *env = std::getenv("PCA_KNN_QUERIES_PER_LANE")) {
-    const int v = std::atoi(env);
-    if ((v == 1 || v == 2) && (v == 1 || cfg.kbucket <= 32))
-      qpt = v;
-  }
+  int qpt = (!cosine && cfg.kbucket <= 32 && m >= 2 * kBlock * 256) ? 2 : 1;
+  const int forced_qpt = env_int("PCA_KNN_QUERIES_PER_LANE", 0);
+  if (forced_qpt == 1 || (forced_qpt == 2 && cfg.kbucket <= 32 && !cosine))
+    qpt = forced_qpt;
   cfg.queries_per_lane = qpt;
   cfg.tile_queries = kBlock * qpt;
+
+  // Slices of x per segment: enough work items (~16 per CU) to even out
+  // ragged segments, but slices of at least ~4 LDS tiles on average -- every
+  // slice pays the start-up phase of its candidate lists again.
+  const int tiles = plan_upper_bound(m, num_segments, cfg.tile_queries);
+  const int want = (4096 + tiles - 1) / tiles;
+  const int by_length = (n / num_segments) / (4 * kLowdTileX);
+  int chunks = std::max(1, std::min(std::min(want, 16), by_length));
+  const int forced_chunks = env_int("PCA_KNN_SLICES", 0);
+  if (forced_chunks >= 1 && forced_chunks <= 64)
+    chunks = forced_chunks;
+  cfg.num_chunks = chunks;
   return cfg;
+}
+
+size_t knn_lowd_scratch_bytes(const KnnLowdConfig &cfg, int m,
+                              int num_segments, int k) {
+  if (cfg.num_chunks <= 1)
+    return 0;
+  const size_t tiles = plan_upper_bound(m, num_segments, cfg.tile_queries);
+  return align256(sizeof(float) * (size_t)m) +
+         align256(sizeof(double) * tiles * cfg.num_chunks * (size_t)k *
+                  cfg.tile_queries);
 }
 
 hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
                            const KnnLowdConfig &cfg, const int *work_start,
-                           int grid_bound, const DenseResult &out,
+                           void *scratch, const DenseResult &out,
+                           hipEvent_t time_start, hipEvent_t time_stop,
                            hipStream_t stream) {
-  KnnLowdConfig c = cfg;
-  if (cosine) {
-    c.queries_per_lane = 1;
+  const int tiles_bound =
+      plan_upper_bound(in.m, in.num_segments, cfg.tile_queries);
+  KnnLowdParams p;
+  p.x = static_cast<const float *>(in.x);
+  p.y = static_cast<const float *>(in.y);
+  p.ptr_x = in.ptr_x;
+  p.ptr_y = in.ptr_y;
+  p.n = in.n;
+  p.m = in.m;
+  p.d_in = in.d;
+  p.num_segments = in.num_segments;
+  p.k = k;
+  p.work_start = work_start;
+  p.num_chunks = cfg.num_chunks;
+  p.tau = nullptr;
+  p.partial = nullptr;
+  p.out_idx = out.idx;
+  p.out_dist = out.dist;
+  p.out_count = out.count;
+  if (cfg.num_chunks > 1) {
+    char *base = static_cast<char *>(scratch);
+    float *tau = reinterpret_cast<float *>(base);
+    p.partial = reinterpret_cast<double *>(
+        base + align256(sizeof(float) * (size_t)in.m));
+    if (!cosine) {
+      // cosine distances can be negative: their bit patterns do not order
+      // like the values, so those slices keep their bounds to themselves
+      p.tau = tau;
+      hipLaunchKernelGGL(fill_f32_kernel, dim3((in.m + kBlock - 1) / kBlock),
+                         dim3(kBlock), 0, stream, tau, in.m, kKnnSentinel);
+    }
   }
+
+  if (time_start)
+    (void)hipEventRecord(time_start, stream);
+  hipError_t err = hipErrorInvalidValue;
 #define PCA_DIM_CASE(D)                                                        \
   case D:                                                                      \
-    return cosine ? launch_knn_lowd_dim<D, true>(in, k, c, work_start,         \
-                                                 grid_bound, out, stream)      \
-                  : launch_knn_lowd_dim<D, false>(in, k, c, work_start,        \
-                                                  grid_bound, out, stream);
+    err = cosine ? launch_knn_lowd_dim<D, true>(p, cfg, tiles_bound, stream)   \
+                 : launch_knn_lowd_dim<D, false>(p, cfg, tiles_bound, stream); \
+    break;
   switch (padded_dim(in.d)) {
     PCA_DIM_CASE(2)
     PCA_DIM_CASE(3)
@@ -69,7 +151,37 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
     PCA_DIM_CASE(8)
   }
 #undef PCA_DIM_CASE
-  return hipErrorInvalidValue;
+  if (time_stop)
+    (void)hipEventRecord(time_stop, stream);
+  if (err != hipSuccess || cfg.num_chunks <= 1)
+    return err;
+
+  switch (cfg.kbucket) {
+  case 8:
+    launch_merge<8>(p, cfg.queries_per_lane, tiles_bound, stream);
+    break;
+  case 16:
+    launch_merge<16>(p, cfg.queries_per_lane, tiles_bound, stream);
+    break;
+  case 24:
+    launch_merge<24>(p, cfg.queries_per_lane, tiles_bound, stream);
+    break;
+  case 32:
+    launch_merge<32>(p, cfg.queries_per_lane, tiles_bound, stream);
+    break;
+  case 48:
+    launch_merge<48>(p, cfg.queries_per_lane, tiles_bound, stream);
+    break;
+  case 64:
+    launch_merge<64>(p, cfg.queries_per_lane, tiles_bound, stream);
+    break;
+  case 100:
+    launch_merge<100>(p, cfg.queries_per_lane, tiles_bound, stream);
+    break;
+  default:
+    return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
 }
 
 hipError_t launch_knn_generic(const SearchInput &in, int k, bool cosine,

@@ -50,17 +50,24 @@ hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
 
 // --- knn_lowd_*.hip --------------------------------------------------------
 
-// Queries per work item of the low-dimensional kNN kernel for this problem.
+// Shape of a low-dimensional kNN launch for a problem.
 struct KnnLowdConfig {
   int kbucket;          // compiled list width (>= k)
   int queries_per_lane; // 1 or 2
   int tile_queries;     // kBlock * queries_per_lane
+  int num_chunks;       // slices of every segment's x rows (>= 1)
 };
 bool knn_lowd_supported(int d, int k, bool cosine);
-KnnLowdConfig knn_lowd_config(int d, int k, int m);
+KnnLowdConfig knn_lowd_config(int d, int k, int n, int m, int num_segments,
+                              bool cosine);
+// Scratch the launch needs beyond the dense result (shared bounds + partial
+// key lists; 0 when the segments are not sliced).
+size_t knn_lowd_scratch_bytes(const KnnLowdConfig &cfg, int m,
+                              int num_segments, int k);
 hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
                            const KnnLowdConfig &cfg, const int *work_start,
-                           int grid_bound, const DenseResult &out,
+                           void *scratch, const DenseResult &out,
+                           hipEvent_t time_start, hipEvent_t time_stop,
                            hipStream_t stream);
 
 // --- knn_generic_*.hip -----------------------------------------------------

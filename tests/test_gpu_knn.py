@@ -208,6 +208,36 @@ def test_two_queries_per_lane_path(oracle, monkeypatch):
         assert (got == want).all() and (gd == wd).all()
 
 
+@pytest.mark.parametrize("slices", [1, 2, 3, 5, 8, 16])
+@pytest.mark.parametrize("qpt", ["1", "2"])
+def test_sliced_segments_merge_exactly(oracle, monkeypatch, slices, qpt):
+    # every segment's x rows cut into `slices` parts that share pruning
+    # bounds and are merged by key: same bits as the unsliced scan, including
+    # exact distance ties across slices (integer grid) and slices shorter
+    # than k
+    monkeypatch.setenv("PCA_KNN_SLICES", str(slices))
+    monkeypatch.setenv("PCA_KNN_QUERIES_PER_LANE", qpt)
+    rng = np.random.default_rng(slices)
+    x = rng.integers(0, 7, (9000, 3)).astype(np.float32)
+    y = rng.integers(0, 7, (1100, 3)).astype(np.float32)
+    ptr_x = np.array([0, 5000, 5000, 5013, 9000])
+    ptr_y = np.array([0, 600, 650, 900, 1100])
+    for k in (16, 21):
+        got, gd = gpu_knn(x, y, ptr_x, ptr_y, k)
+        want, wd = oracle_knn_edges(oracle, x, y, ptr_x, ptr_y, k)
+        assert got.shape == want.shape
+        assert (got == want).all()
+        assert (gd == wd).all()
+    xr = rng.standard_normal((30000, 3)).astype(np.float32)
+    got, gd = gpu_knn(xr, xr[:700], None, None, 10)
+    want, wd = oracle_knn_edges(oracle, xr, xr[:700], None, None, 10)
+    assert (got == want).all() and (gd == wd).all()
+    got, gd = gpu_knn(xr[:6000], xr[:300], None, None, 5, cosine=True)
+    want, wd = oracle_knn_edges(oracle, xr[:6000], xr[:300], None, None, 5,
+                                cosine=True)
+    assert (got == want).all() and (gd == wd).all()
+
+
 def test_against_float64_within_tie_tolerance():
     rng = np.random.default_rng(9)
     x = rng.random((4000, 3), dtype=np.float32)
