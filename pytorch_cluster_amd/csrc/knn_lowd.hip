@@ -65,20 +65,22 @@ KnnLowdConfig knn_lowd_config(int /*d*/, int k, int n, int m,
                               int num_segments, bool cosine) {
   KnnLowdConfig cfg;
   cfg.kbucket = k_bucket(k);
-  // Two queries per lane halve the LDS reads per distance but need twice the
-  // queries to fill the 256 CUs; worth it once there are enough query tiles.
-  int qpt = (!cosine && cfg.kbucket <= 32 && m >= 2 * kBlock * 256) ? 2 : 1;
+  // One query per lane keeps four waves per SIMD resident and measures
+  // fastest; two per lane (half the LDS reads per distance, more registers)
+  // stay available for experiments.
+  int qpt = 1;
   const int forced_qpt = env_int("PCA_KNN_QUERIES_PER_LANE", 0);
   if (forced_qpt == 1 || (forced_qpt == 2 && cfg.kbucket <= 32 && !cosine))
     qpt = forced_qpt;
+  (void)m;
   cfg.queries_per_lane = qpt;
   cfg.tile_queries = kBlock * qpt;
 
-  // Slices of x per segment: enough work items (~16 per CU) to even out
+  // Slices of x per segment: enough work items (~32 per CU) to even out
   // ragged segments, but slices of at least ~4 LDS tiles on average -- every
   // slice pays the start-up phase of its candidate lists again.
   const int tiles = plan_upper_bound(m, num_segments, cfg.tile_queries);
-  const int want = (4096 + tiles - 1) / tiles;
+  const int want = (8192 + tiles - 1) / tiles;
   const int by_length = (n / num_segments) / (4 * kLowdTileX);
   int chunks = std::max(1, std::min(std::min(want, 16), by_length));
   const int forced_chunks = env_int("PCA_KNN_SLICES", 0);

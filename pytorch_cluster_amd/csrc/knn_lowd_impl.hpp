@@ -383,10 +383,9 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
         cx[c][2] = grp[c].z;
         cx[c][3] = grp[c].w;
       }
-      // score of every (query, candidate) pair of the group and, per pair,
-      // the set of lanes whose score is below their bound
+      // score of every (query, candidate) pair of the group; per query the
+      // smallest of them decides whether anything needs a closer look
       float score[QPT][U];
-      uint64_t hit[QPT][U];
       uint64_t any_hit = 0;
 #pragma unroll
       for (int qi = 0; qi < QPT; ++qi) {
@@ -410,21 +409,27 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
             acc = exact_sqdist<DIM>(cx, u, yq[qi]);
           }
           score[qi][u] = acc;
-          hit[qi][u] = __ballot(acc < bound[qi]);
-          any_hit |= hit[qi][u];
         }
+        const float lo = __builtin_fminf(
+            min3f(score[qi][0], score[qi][1], score[qi][2]), score[qi][3]);
+        any_hit |= __ballot(lo < bound[qi]);
       }
-      // One scalar branch on the hot path.  The lane sets live in scalar
-      // registers, so finding the pairs with work is scalar code too; only a
-      // pair some lane passed runs vector instructions, and those just park
-      // the candidate's position -- the exact distance is taken when the
-      // queue is drained, by all lanes together.
+      // One scalar branch on the hot path.  On the rare path the lanes that
+      // passed are collected per pair with a ballot into scalar registers, so
+      // finding the pairs with work is scalar code; only a pair some lane
+      // passed runs vector instructions, and those just park the candidate's
+      // position -- the exact distance is taken when the queue is drained, by
+      // all lanes together.
       if (any_hit != 0) {
 #pragma unroll
         for (int qi = 0; qi < QPT; ++qi) {
+          uint64_t hit[U];
+#pragma unroll
+          for (int u = 0; u < U; ++u)
+            hit[u] = __ballot(score[qi][u] < bound[qi]);
 #pragma unroll
           for (int u = 0; u < U; ++u) {
-            if (hit[qi][u] != 0 && score[qi][u] < bound[qi]) {
+            if (hit[u] != 0 && score[qi][u] < bound[qi]) {
               queue[qi][qcount[qi]][tid] = (uint16_t)(j + u);
               ++qcount[qi];
             }
