@@ -86,6 +86,9 @@ KnnLayout knn_layout(int64_t n, int64_t m, int64_t d, int64_t num_segments,
   KnnLayout w;
   if (d > 8) {
     w.x_norm = align256(sizeof(float) * (size_t)n);
+    if (pca::knn_mfma_supported((int)d, (int)k, false))
+      w.sliced = pca::knn_mfma_scratch_bytes((int)n, (int)m,
+                                             (int)num_segments, (int)k);
   } else {
     // the larger of the two metrics' needs, so one size query serves both
     for (int cosine = 0; cosine < 2; ++cosine) {
@@ -239,7 +242,11 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
 
   pca::SearchInput in{x,      y,      ptr_x,  ptr_y,
                       (int)n, (int)m, (int)d, (int)num_segments};
-  if (!low_d)
+  const bool mfma =
+      !low_d && pca::knn_mfma_supported((int)d, (int)k, cosine != 0);
+  if (mfma)
+    cfg.tile_queries = pca::kMfmaTileQueries;
+  else if (!low_d)
     cfg.tile_queries = pca::kBlock; // any-dimension kernel: one query per lane
   int rc = check_launch(pca::launch_plan(ptr_y, (int)m, (int)num_segments,
                                          cfg.tile_queries, work_start, stream),
@@ -255,6 +262,12 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
                                            work_start, lowd_scratch, dense,
                                            timer.start, timer.stop, stream),
                       "knn_lowd_kernel");
+    timer.stop = nullptr;
+  } else if (mfma) {
+    rc = check_launch(pca::launch_knn_mfma(in, (int)k, work_start,
+                                           lowd_scratch, dense, timer.start,
+                                           timer.stop, stream),
+                      "knn_mfma_kernel");
     timer.stop = nullptr;
   } else {
     if (cosine) {

@@ -46,12 +46,12 @@ void launch_merge(const KnnLowdParams &p, int queries_per_lane,
                   int tiles_bound, hipStream_t stream) {
   if constexpr (KB <= 32) {
     if (queries_per_lane == 2) {
-      hipLaunchKernelGGL((knn_lowd_merge_kernel<KB, 2>), dim3(tiles_bound),
+      hipLaunchKernelGGL((knn_merge_kernel<KB, 2 * kBlock>), dim3(tiles_bound),
                          dim3(kBlock), 0, stream, p);
       return;
     }
   }
-  hipLaunchKernelGGL((knn_lowd_merge_kernel<KB, 1>), dim3(tiles_bound),
+  hipLaunchKernelGGL((knn_merge_kernel<KB, kBlock>), dim3(tiles_bound),
                      dim3(kBlock), 0, stream, p);
 }
 

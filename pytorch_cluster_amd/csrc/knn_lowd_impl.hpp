@@ -487,12 +487,12 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
   }
 }
 
-// Merges the S sorted key lists of every query of a tile (one workgroup per
-// tile, same lane <-> query mapping as the search kernel).
-template <int K, int QPT>
-__global__ __launch_bounds__(kBlock) void knn_lowd_merge_kernel(
-    KnnLowdParams p) {
-  constexpr int TQ = kBlock * QPT;
+// Merges the sorted key lists of every query of a tile of TQ queries (one
+// workgroup per tile; list c of the tile's query at position `pos` starts at
+// partial[((c * tiles + tile) * k) * TQ + pos], consecutive slots TQ apart).
+// p.num_chunks is the number of lists per query.
+template <int K, int TQ>
+__global__ __launch_bounds__(kBlock) void knn_merge_kernel(KnnLowdParams p) {
   const int tid = threadIdx.x;
   const int total_tiles = p.work_start[p.num_segments];
   const int tile = blockIdx.x;
@@ -504,17 +504,16 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_merge_kernel(
   const int q_base = y_begin + (tile - p.work_start[seg]) * TQ;
   const int k = p.k;
 
-#pragma unroll
-  for (int qi = 0; qi < QPT; ++qi) {
-    const int q = q_base + qi * kBlock + tid;
+  // TQ is a multiple of the wave size, so a wave is either all in or all out
+  for (int pos = tid; pos < TQ; pos += kBlock) {
+    const int q = q_base + pos;
     double best[K];
 #pragma unroll
     for (int j = 0; j < K; ++j)
       best[j] = (j < K - k) ? lowest_key() : empty_key();
     for (int c = 0; c < p.num_chunks; ++c) {
       const double *src =
-          p.partial + (size_t)(c * total_tiles + tile) * k * TQ +
-          qi * kBlock + tid;
+          p.partial + (size_t)(c * total_tiles + tile) * k * TQ + pos;
       for (int e = 0; e < k; ++e) {
         const double key = src[(size_t)e * TQ];
         // lists are ascending: once no lane's entry beats its worst kept

@@ -1,0 +1,186 @@
+// Dispatch of the matrix-core kNN kernels (see knn_mfma_impl.hpp).
+#include "knn_mfma_impl.hpp"
+
+#include <algorithm>
+#include <cstdlib>
+
+namespace pca {
+
+template <int STEPS>
+hipError_t launch_knn_mfma_steps(const KnnMfmaParams &p, int kbucket,
+                                 int grid, hipStream_t stream);
+template <>
+hipError_t launch_knn_mfma_steps<8>(const KnnMfmaParams &, int, int,
+                                    hipStream_t);
+template <>
+hipError_t launch_knn_mfma_steps<16>(const KnnMfmaParams &, int, int,
+                                     hipStream_t);
+template <>
+hipError_t launch_knn_mfma_steps<32>(const KnnMfmaParams &, int, int,
+                                     hipStream_t);
+template <>
+hipError_t launch_knn_mfma_steps<64>(const KnnMfmaParams &, int, int,
+                                     hipStream_t);
+
+__global__ __launch_bounds__(kBlock) void row_sqnorm_kernel(
+    const float *__restrict__ x, int n, int d, float *__restrict__ out) {
+  const int row = blockIdx.x * kBlock + threadIdx.x;
+  if (row >= n)
+    return;
+  const float *p = x + (size_t)row * d;
+  float s = 0.0f;
+  for (int c = 0; c < d; ++c)
+    s = __builtin_fmaf(p[c], p[c], s);
+  out[row] = s;
+}
+
+namespace {
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+int k_bucket(int k) {
+  static const int buckets[] = {8, 16, 24, 32};
+  for (int b : buckets)
+    if (k <= b)
+      return b;
+  return 0;
+}
+
+__global__ __launch_bounds__(kBlock) void fill_tau_kernel(float *p, int n,
+                                                          float v) {
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < n)
+    p[i] = v;
+}
+
+template <int KB>
+void launch_mfma_merge(const KnnLowdParams &p, int tiles_bound,
+                       hipStream_t stream) {
+  hipLaunchKernelGGL((knn_merge_kernel<KB, kMfmaQueries>), dim3(tiles_bound),
+                     dim3(kBlock), 0, stream, p);
+}
+
+} // namespace
+
+bool knn_mfma_supported(int d, int k, bool cosine) {
+  if (const char *env = std::getenv("PCA_KNN_NO_MFMA"))
+    if (env[0] == '1')
+      return false;
+  return !cosine && d > 8 && d <= 128 && k >= 1 && k <= 32;
+}
+
+int knn_mfma_slices(int n, int m, int num_segments) {
+  const int tiles = plan_upper_bound(m, num_segments, kMfmaQueries);
+  const int want = (3072 + tiles - 1) / tiles;
+  const int by_length = (n / num_segments) / 4096;
+  int chunks = std::max(1, std::min(std::min(want, 16), by_length));
+  if (const char *env = std::getenv("PCA_KNN_SLICES")) {
+    const int v = std::atoi(env);
+    if (v >= 1 && v <= 64)
+      chunks = v;
+  }
+  return chunks;
+}
+
+size_t knn_mfma_scratch_bytes(int n, int m, int num_segments, int k) {
+  const size_t tiles = plan_upper_bound(m, num_segments, kMfmaQueries);
+  // the largest slice count a call may choose
+  const int chunks = std::max(knn_mfma_slices(n, m, num_segments), 1);
+  return align256(sizeof(float) * (size_t)n) +
+         align256(sizeof(float) * (size_t)m) +
+         align256(sizeof(double) * tiles * chunks * (size_t)k *
+                  kMfmaQueries);
+}
+
+hipError_t launch_knn_mfma(const SearchInput &in, int k,
+                           const int *work_start, void *scratch,
+                           const DenseResult &out, hipEvent_t time_start,
+                           hipEvent_t time_stop, hipStream_t stream) {
+  const int tiles_bound =
+      plan_upper_bound(in.m, in.num_segments, kMfmaQueries);
+  const int chunks = knn_mfma_slices(in.n, in.m, in.num_segments);
+  char *base = static_cast<char *>(scratch);
+  float *x_sq = reinterpret_cast<float *>(base);
+  base += align256(sizeof(float) * (size_t)in.n);
+  float *tau = reinterpret_cast<float *>(base);
+  base += align256(sizeof(float) * (size_t)in.m);
+  double *partial = reinterpret_cast<double *>(base);
+
+  hipLaunchKernelGGL(row_sqnorm_kernel, dim3((in.n + kBlock - 1) / kBlock),
+                     dim3(kBlock), 0, stream,
+                     static_cast<const float *>(in.x), in.n, in.d, x_sq);
+  hipLaunchKernelGGL(fill_tau_kernel, dim3((in.m + kBlock - 1) / kBlock),
+                     dim3(kBlock), 0, stream, tau, in.m, kKnnSentinel);
+
+  KnnMfmaParams p;
+  p.x = static_cast<const float *>(in.x);
+  p.y = static_cast<const float *>(in.y);
+  p.ptr_x = in.ptr_x;
+  p.ptr_y = in.ptr_y;
+  p.x_sq = x_sq;
+  p.n = in.n;
+  p.m = in.m;
+  p.d = in.d;
+  p.num_segments = in.num_segments;
+  p.k = k;
+  p.work_start = work_start;
+  p.num_chunks = chunks;
+  p.tau = tau;
+  p.partial = partial;
+
+  const int kb = k_bucket(k);
+  const int grid = tiles_bound * chunks;
+  if (time_start)
+    (void)hipEventRecord(time_start, stream);
+  hipError_t err;
+  if (in.d <= 16)
+    err = launch_knn_mfma_steps<8>(p, kb, grid, stream);
+  else if (in.d <= 32)
+    err = launch_knn_mfma_steps<16>(p, kb, grid, stream);
+  else if (in.d <= 64)
+    err = launch_knn_mfma_steps<32>(p, kb, grid, stream);
+  else
+    err = launch_knn_mfma_steps<64>(p, kb, grid, stream);
+  if (time_stop)
+    (void)hipEventRecord(time_stop, stream);
+  if (err != hipSuccess)
+    return err;
+
+  // one list per query and slice
+  KnnLowdParams mp;
+  mp.x = p.x;
+  mp.y = p.y;
+  mp.ptr_x = in.ptr_x;
+  mp.ptr_y = in.ptr_y;
+  mp.n = in.n;
+  mp.m = in.m;
+  mp.d_in = in.d;
+  mp.num_segments = in.num_segments;
+  mp.k = k;
+  mp.work_start = work_start;
+  mp.num_chunks = chunks;
+  mp.tau = nullptr;
+  mp.partial = partial;
+  mp.out_idx = out.idx;
+  mp.out_dist = out.dist;
+  mp.out_count = out.count;
+  switch (kb) {
+  case 8:
+    launch_mfma_merge<8>(mp, tiles_bound, stream);
+    break;
+  case 16:
+    launch_mfma_merge<16>(mp, tiles_bound, stream);
+    break;
+  case 24:
+    launch_mfma_merge<24>(mp, tiles_bound, stream);
+    break;
+  case 32:
+    launch_mfma_merge<32>(mp, tiles_bound, stream);
+    break;
+  default:
+    return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+} // namespace pca

@@ -195,6 +195,45 @@ def test_parity_high_dimension(oracle, d, k, cosine):
     assert (gd == wd).all()
 
 
+@pytest.mark.parametrize("d,k", [(3, 16), (2, 8), (8, 24), (24, 16),
+                                 (128, 32)])
+@pytest.mark.parametrize("case", ["offset", "huge", "tiny", "mixed_scale",
+                                  "clustered"])
+def test_prefilter_never_drops_a_neighbour(oracle, d, k, case):
+    # the expanded-form pre-filter must stay conservative where it is least
+    # accurate: tight clusters far from the origin, coordinates near the
+    # overflow / underflow ends of fp32, wildly mixed scales
+    rng = np.random.default_rng(hash((d, k, case)) % (2 ** 32))
+    n, m = 5000, 600
+    if case == "offset":
+        x = 1000.0 + 1e-2 * rng.standard_normal((n, d))
+        y = 1000.0 + 1e-2 * rng.standard_normal((m, d))
+    elif case == "huge":
+        x = 1e17 * rng.standard_normal((n, d))
+        y = 1e17 * rng.standard_normal((m, d))
+        y[:50] = x[:50]  # exact duplicates at distance 0
+    elif case == "tiny":
+        x = 1e-21 * rng.standard_normal((n, d))
+        y = 1e-21 * rng.standard_normal((m, d))
+    elif case == "mixed_scale":
+        scale = 10.0 ** rng.integers(-6, 7, (n, 1))
+        x = scale * rng.standard_normal((n, d))
+        y = (10.0 ** rng.integers(-6, 7, (m, 1))) * rng.standard_normal((m, d))
+    else:
+        centres = 50.0 * rng.standard_normal((20, d))
+        x = centres[rng.integers(0, 20, n)] + 1e-3 * rng.standard_normal((n, d))
+        y = centres[rng.integers(0, 20, m)] + 1e-3 * rng.standard_normal((m, d))
+    x = x.astype(np.float32)
+    y = y.astype(np.float32)
+    ptr_x = np.array([0, 2000, 5000])
+    ptr_y = np.array([0, 250, 600])
+    got, gd = gpu_knn(x, y, ptr_x, ptr_y, k)
+    want, wd = oracle_knn_edges(oracle, x, y, ptr_x, ptr_y, k)
+    assert got.shape == want.shape
+    assert (got == want).all()
+    assert (gd == wd).all()
+
+
 def test_two_queries_per_lane_path(oracle, monkeypatch):
     rng = np.random.default_rng(77)
     x = rng.random((5000, 3), dtype=np.float32)
