@@ -87,6 +87,47 @@ def cpu_baseline(data, ptr_x, ptr_y):
                       "OpenMP" % (stride, len(sample))}
 
 
+def other_configs(torch, pca, testing, dev):
+    """End-to-end times of the other BASELINE configurations (median of a few
+    calls, inputs resident in HBM); reported beside the headline number, they
+    are parity-test cases, not the benchmark."""
+    def median_ms(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            out = fn()
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+        return statistics.median(times), out
+
+    report = {}
+    c2 = testing.uniform_batched(0)
+    x, b = c2["x"].to(dev), c2["batch"].to(dev)
+    ms, out = median_ms(lambda: pca.knn_graph(x, 20, b, batch_size=16), 10)
+    report["configs[1] knn_graph 16x4096 k=20"] = {
+        "ms": ms, "queries_per_s": x.shape[0] / ms * 1e3,
+        "edges": int(out.shape[1])}
+    c3 = testing.gaussian_mixture_batched(0)
+    x, b = c3["x"].to(dev), c3["batch"].to(dev)
+    ms, out = median_ms(
+        lambda: pca.radius_graph(x, 0.05, b, max_num_neighbors=32,
+                                 batch_size=8), 10)
+    report["configs[2] radius_graph 8x16384 r=0.05 max 32"] = {
+        "ms": ms, "edges_per_s": out.shape[1] / ms * 1e3,
+        "edges": int(out.shape[1])}
+    c4 = testing.feature_space(0)
+    x, y = c4["x"].to(dev), c4["y"].to(dev)
+    for cosine in (False, True):
+        ms, out = median_ms(lambda: pca.knn(x, y, 32, cosine=cosine), 3)
+        report["configs[3] knn 200000x128 / 50000x128 k=32 cosine=%s"
+               % cosine] = {
+            "ms": ms, "queries_per_s": y.shape[0] / ms * 1e3,
+            "gemm_tflops": 2 * 128 * x.shape[0] * y.shape[0] / ms / 1e9}
+    return report
+
+
 def measured_traffic():
     """HBM bytes per launch of the dominant kernel from the committed rocprof
     counter summary, if there is one."""
@@ -106,6 +147,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the short timings of the other BASELINE "
+                         "configurations")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy three times, so "
                          "that a counter profile of this command can scale "
@@ -182,7 +226,7 @@ def main():
         "edges_per_s": m * K * args.steps / elapsed,
         "roofline": {
             "bound": "fp32_valu",
-            "kernel": "knn_lowd_kernel<3,16,*>",
+            "kernel": "knn_lowd_kernel<3,16,1,false>",
             "achieved": achieved,
             "peak": PEAK_FP32_TFLOPS,
             "unit": "TFLOP/s",
@@ -192,6 +236,8 @@ def main():
             "traffic": measured_traffic(),
         },
     }
+    if not args.no_extras:
+        result["other_configs"] = other_configs(torch, pca, testing, dev)
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
         dst = torch.empty_like(src)
