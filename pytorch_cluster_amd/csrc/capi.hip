@@ -264,7 +264,7 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
                       "knn_lowd_kernel");
     timer.stop = nullptr;
   } else if (mfma) {
-    rc = check_launch(pca::launch_knn_mfma(in, (int)k, work_start,
+    rc = check_launch(pca::launch_knn_mfma(in, (int)k, cosine != 0, work_start,
                                            lowd_scratch, dense, timer.start,
                                            timer.stop, stream),
                       "knn_mfma_kernel");

@@ -129,13 +129,9 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
     float *tau = reinterpret_cast<float *>(base);
     p.partial = reinterpret_cast<double *>(
         base + align256(sizeof(float) * (size_t)in.m));
-    if (!cosine) {
-      // cosine distances can be negative: their bit patterns do not order
-      // like the values, so those slices keep their bounds to themselves
-      p.tau = tau;
-      hipLaunchKernelGGL(fill_f32_kernel, dim3((in.m + kBlock - 1) / kBlock),
-                         dim3(kBlock), 0, stream, tau, in.m, kKnnSentinel);
-    }
+    p.tau = tau;
+    hipLaunchKernelGGL(fill_f32_kernel, dim3((in.m + kBlock - 1) / kBlock),
+                       dim3(kBlock), 0, stream, tau, in.m, kKnnSentinel);
   }
 
   if (time_start)

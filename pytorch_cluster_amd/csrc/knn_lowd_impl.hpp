@@ -65,7 +65,7 @@ struct KnnLowdParams {
   int n, m, d_in, num_segments, k;
   const int *work_start; // [num_segments + 1] first query tile of each segment
   int num_chunks;        // S: slices of every segment's x rows
-  float *tau;            // [m] shared pruning bounds (S > 1, Euclidean) or NULL
+  float *tau;            // [m] shared pruning bounds (S > 1) or NULL
   double *partial;       // [S * tiles][k][tile queries] keys (S > 1) or NULL
   int *out_idx;          // dense results (written here only when S == 1)
   float *out_dist;
@@ -334,11 +334,12 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
 #pragma unroll
     for (int qi = 0; qi < QPT; ++qi) {
       if (q[qi] < y_end) {
-        const float own = key_dist(best[qi][K - 1]);
+        // a (slightly) negative cosine distance is published as 0: still an
+        // upper bound, and non-negative floats order like their bit patterns
+        const float own = __builtin_fmaxf(key_dist(best[qi][K - 1]), 0.0f);
         const float seen = __hip_atomic_load(&p.tau[q[qi]], __ATOMIC_RELAXED,
                                              __HIP_MEMORY_SCOPE_AGENT);
         if (own < seen && own < posted[qi]) {
-          // non-negative floats order like their bit patterns
           __hip_atomic_fetch_min(reinterpret_cast<int *>(&p.tau[q[qi]]),
                                  (int)__float_as_uint(own), __ATOMIC_RELAXED,
                                  __HIP_MEMORY_SCOPE_AGENT);

@@ -8,19 +8,23 @@ namespace pca {
 
 template <int STEPS>
 hipError_t launch_knn_mfma_steps(const KnnMfmaParams &p, int kbucket,
-                                 int grid, hipStream_t stream);
+                                 bool cosine, int grid, hipStream_t stream);
 template <>
-hipError_t launch_knn_mfma_steps<8>(const KnnMfmaParams &, int, int,
+hipError_t launch_knn_mfma_steps<8>(const KnnMfmaParams &, int, bool, int,
                                     hipStream_t);
 template <>
-hipError_t launch_knn_mfma_steps<16>(const KnnMfmaParams &, int, int,
+hipError_t launch_knn_mfma_steps<16>(const KnnMfmaParams &, int, bool, int,
                                      hipStream_t);
 template <>
-hipError_t launch_knn_mfma_steps<32>(const KnnMfmaParams &, int, int,
+hipError_t launch_knn_mfma_steps<32>(const KnnMfmaParams &, int, bool, int,
                                      hipStream_t);
 template <>
-hipError_t launch_knn_mfma_steps<64>(const KnnMfmaParams &, int, int,
+hipError_t launch_knn_mfma_steps<64>(const KnnMfmaParams &, int, bool, int,
                                      hipStream_t);
+
+// csrc/knn_generic_cos.hip
+hipError_t launch_row_norms(const float *x, int n, int d, float *norm,
+                            hipStream_t stream);
 
 __global__ __launch_bounds__(kBlock) void row_sqnorm_kernel(
     const float *__restrict__ x, int n, int d, float *__restrict__ out) {
@@ -66,7 +70,8 @@ bool knn_mfma_supported(int d, int k, bool cosine) {
   if (const char *env = std::getenv("PCA_KNN_NO_MFMA"))
     if (env[0] == '1')
       return false;
-  return !cosine && d > 8 && d <= 128 && k >= 1 && k <= 32;
+  (void)cosine;
+  return d > 8 && d <= 128 && k >= 1 && k <= 32;
 }
 
 int knn_mfma_slices(int n, int m, int num_segments) {
@@ -92,7 +97,7 @@ size_t knn_mfma_scratch_bytes(int n, int m, int num_segments, int k) {
                   kMfmaQueries);
 }
 
-hipError_t launch_knn_mfma(const SearchInput &in, int k,
+hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
                            const int *work_start, void *scratch,
                            const DenseResult &out, hipEvent_t time_start,
                            hipEvent_t time_stop, hipStream_t stream) {
@@ -106,9 +111,13 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k,
   base += align256(sizeof(float) * (size_t)in.m);
   double *partial = reinterpret_cast<double *>(base);
 
-  hipLaunchKernelGGL(row_sqnorm_kernel, dim3((in.n + kBlock - 1) / kBlock),
-                     dim3(kBlock), 0, stream,
-                     static_cast<const float *>(in.x), in.n, in.d, x_sq);
+  if (cosine)
+    (void)launch_row_norms(static_cast<const float *>(in.x), in.n, in.d, x_sq,
+                           stream);
+  else
+    hipLaunchKernelGGL(row_sqnorm_kernel, dim3((in.n + kBlock - 1) / kBlock),
+                       dim3(kBlock), 0, stream,
+                       static_cast<const float *>(in.x), in.n, in.d, x_sq);
   hipLaunchKernelGGL(fill_tau_kernel, dim3((in.m + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, tau, in.m, kKnnSentinel);
 
@@ -134,13 +143,13 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k,
     (void)hipEventRecord(time_start, stream);
   hipError_t err;
   if (in.d <= 16)
-    err = launch_knn_mfma_steps<8>(p, kb, grid, stream);
+    err = launch_knn_mfma_steps<8>(p, kb, cosine, grid, stream);
   else if (in.d <= 32)
-    err = launch_knn_mfma_steps<16>(p, kb, grid, stream);
+    err = launch_knn_mfma_steps<16>(p, kb, cosine, grid, stream);
   else if (in.d <= 64)
-    err = launch_knn_mfma_steps<32>(p, kb, grid, stream);
+    err = launch_knn_mfma_steps<32>(p, kb, cosine, grid, stream);
   else
-    err = launch_knn_mfma_steps<64>(p, kb, grid, stream);
+    err = launch_knn_mfma_steps<64>(p, kb, cosine, grid, stream);
   if (time_stop)
     (void)hipEventRecord(time_stop, stream);
   if (err != hipSuccess)

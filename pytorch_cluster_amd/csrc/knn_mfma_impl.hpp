@@ -1,5 +1,5 @@
-// Feature-space kNN (8 < d <= 128, k <= 32, Euclidean) on the gfx950 matrix
-// cores, with results bit-identical to the reference's scalar loop
+// Feature-space kNN (8 < d <= 128, k <= 32, Euclidean or cosine) on the gfx950
+// matrix cores, with results bit-identical to the reference's scalar loop
 // (csrc/cuda/knn_cuda.cu:52-78).
 //
 // The distance of a (query, candidate) pair is |x|^2 + |y|^2 - 2 x.y.  The
@@ -25,6 +25,13 @@
 // its partner lane (v_permlane32_swap) -- and feed the usual (distance, row)
 // key lists.  No memory latency is involved, and the vector work of one wave
 // overlaps the matrix-core chain of the other wave on the same SIMD.
+//
+// The cosine distance 1 - x.y / (|x| |y|) uses the same matrix-core dot
+// product: the filter value is 1 - mfma_dot * (1/|x|) * (1/|y|), within
+// (3d + 40) u of the exactly evaluated distance, and is tested against
+// thresh + (4d + 64) u; the exact value divides the sequentially accumulated
+// dot product by the product of the two norms like the reference does
+// (csrc/cuda/knn_cuda.cu:9-28,55-59).
 //
 // Mapping: a workgroup owns 128 queries of one segment (4 waves x 32) and one
 // slice of the segment's x rows.  A = 32 candidates (rows i), B = 32 queries
@@ -60,7 +67,7 @@ struct KnnMfmaParams {
   const float *y;
   const int64_t *ptr_x;
   const int64_t *ptr_y;
-  const float *x_sq; // [n] squared norms of the x rows
+  const float *x_sq; // [n] squared norms of the x rows (cosine: norms)
   int n, m, d, num_segments, k;
   const int *work_start; // [num_segments + 1] first 128-query tile per segment
   int num_chunks;        // slices of every segment's x rows
@@ -86,7 +93,7 @@ __device__ __forceinline__ float mfma_filter_cut(float thresh, float ysq,
 }
 
 // STEPS = padded d / 2: matrix-core steps per tile.
-template <int STEPS, int K>
+template <int STEPS, int K, bool COSINE>
 __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   constexpr int DP = 2 * STEPS;  // padded number of components
   constexpr int RS = DP + 4;     // LDS row stride (floats), keeps b128 reads
@@ -96,7 +103,10 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   constexpr int PER_THREAD = TR * DP / kBlock; // floats staged per thread
 
   __shared__ __attribute__((aligned(16))) float xs[2][TR][RS];
+  // per row: damped squared norm (Euclidean) or 1 / norm (cosine) ...
   __shared__ __attribute__((aligned(16))) float wn[2][TR];
+  // ... and, for the cosine distance, the norm itself
+  __shared__ float xnorm[2][COSINE ? TR : 1];
   __shared__ uint8_t queue[16][kBlock]; // parked rows of the current tile
 
   const int tid = threadIdx.x;
@@ -143,19 +153,23 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   float ysq = 0.0f;
   for (int c = 0; c < d; ++c)
     ysq = __builtin_fmaf(yrow[c], yrow[c], ysq);
+  const float ynorm = __builtin_sqrtf(ysq);
+  const float yrinv = 1.0f / ynorm;
+  const float cos_margin = (float)(4 * d + 64) * 5.9604644775390625e-08f;
 
   double best[K];
 #pragma unroll
   for (int j = 0; j < K; ++j)
     best[j] = (j < K - k) ? lowest_key() : empty_key();
   float thresh = kKnnSentinel;
-  float bound = mfma_filter_cut(thresh, ysq, eps);
+  float bound =
+      COSINE ? thresh + cos_margin : mfma_filter_cut(thresh, ysq, eps);
   float shared = kKnnSentinel;
   float posted = kKnnSentinel;
 
   auto set_thresh = [&](float v) {
     thresh = v;
-    bound = mfma_filter_cut(v, ysq, eps);
+    bound = COSINE ? v + cos_margin : mfma_filter_cut(v, ysq, eps);
   };
 
   // ---- tile staging -------------------------------------------------------
@@ -164,6 +178,7 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   const int st_c0 = (tid & 7) * (DP / 8);
   float stage[PER_THREAD];
   float stage_w = 0.0f;
+  float stage_norm = 0.0f;
 
   auto load_tile = [&](int t) {
     const int g = c_begin + t * TR + st_row;
@@ -177,7 +192,18 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
     if (tid < TR) {
       const int gr = c_begin + t * TR + tid;
       float w = __builtin_inff();
-      if (gr < c_end) {
+      if (COSINE) {
+        // filter value = 1 - dot * w * (1 / |y|); padding rows: w = 0 and
+        // |x| = NaN, so that neither the filter (bound < 1 once a list is
+        // full) nor the exact distance (NaN) can accept them
+        float nx = __builtin_nanf("");
+        w = 0.0f;
+        if (gr < c_end) {
+          nx = p.x_sq[gr];
+          w = 1.0f / nx;
+        }
+        stage_norm = nx;
+      } else if (gr < c_end) {
         const float s = p.x_sq[gr];
         // norms that are not moderate finite numbers always pass the filter
         w = (s <= kFilterNormLimit) ? s * damp : -__builtin_inff();
@@ -191,19 +217,23 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
       const int c = st_c0 + e;
       xs[buf][st_row][(c & 1) * STEPS + (c >> 1)] = stage[e];
     }
-    if (tid < TR)
+    if (tid < TR) {
       wn[buf][tid] = stage_w;
+      if (COSINE)
+        xnorm[buf][tid] = stage_norm;
+    }
   };
 
   // Exchange of pruning bounds between the slices of a query: the k-th best
   // distance any slice has reached bounds the final k-th distance from above.
   auto sync_bounds = [&]() {
     if (valid) {
-      const float own = key_dist(best[K - 1]);
+      // a (slightly) negative cosine distance is published as 0: still an
+      // upper bound, and non-negative floats order like their bit patterns
+      const float own = __builtin_fmaxf(key_dist(best[K - 1]), 0.0f);
       const float seen = __hip_atomic_load(&p.tau[q], __ATOMIC_RELAXED,
                                            __HIP_MEMORY_SCOPE_AGENT);
       if (own < seen && own < posted) {
-        // non-negative floats order like their bit patterns
         __hip_atomic_fetch_min(reinterpret_cast<int *>(&p.tau[q]),
                                (int)__float_as_uint(own), __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
@@ -242,11 +272,20 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
           const auto both = __builtin_amdgcn_permlane32_swap(
               __float_as_uint(yb[4 * s4 + e]), __float_as_uint(yb[4 * s4 + e]),
               false, false);
-          const float d0 = xev[e] - __uint_as_float(both[0]);
-          dist = __builtin_fmaf(d0, d0, dist);
-          const float d1 = xov[e] - __uint_as_float(both[1]);
-          dist = __builtin_fmaf(d1, d1, dist);
+          if (COSINE) {
+            dist = __builtin_fmaf(xev[e], __uint_as_float(both[0]), dist);
+            dist = __builtin_fmaf(xov[e], __uint_as_float(both[1]), dist);
+          } else {
+            const float d0 = xev[e] - __uint_as_float(both[0]);
+            dist = __builtin_fmaf(d0, d0, dist);
+            const float d1 = xov[e] - __uint_as_float(both[1]);
+            dist = __builtin_fmaf(d1, d1, dist);
+          }
         }
+      }
+      if (COSINE) {
+        dist = dist / (xnorm[buf][row] * ynorm);
+        dist = 1.0f - dist;
       }
       // The two lanes that share a query keep ONE list between them: each
       // hands its key to the other, both insert both, so the lists stay
@@ -314,10 +353,17 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
     for (int v4 = 0; v4 < 4; ++v4) {
       const float4 w =
           *reinterpret_cast<const float4 *>(&wn[buf][8 * v4 + 4 * half]);
-      score[4 * v4 + 0] = __builtin_fmaf(-2.0f, acc[4 * v4 + 0], w.x);
-      score[4 * v4 + 1] = __builtin_fmaf(-2.0f, acc[4 * v4 + 1], w.y);
-      score[4 * v4 + 2] = __builtin_fmaf(-2.0f, acc[4 * v4 + 2], w.z);
-      score[4 * v4 + 3] = __builtin_fmaf(-2.0f, acc[4 * v4 + 3], w.w);
+      if (COSINE) {
+        score[4 * v4 + 0] = __builtin_fmaf(-acc[4 * v4 + 0], w.x * yrinv, 1.0f);
+        score[4 * v4 + 1] = __builtin_fmaf(-acc[4 * v4 + 1], w.y * yrinv, 1.0f);
+        score[4 * v4 + 2] = __builtin_fmaf(-acc[4 * v4 + 2], w.z * yrinv, 1.0f);
+        score[4 * v4 + 3] = __builtin_fmaf(-acc[4 * v4 + 3], w.w * yrinv, 1.0f);
+      } else {
+        score[4 * v4 + 0] = __builtin_fmaf(-2.0f, acc[4 * v4 + 0], w.x);
+        score[4 * v4 + 1] = __builtin_fmaf(-2.0f, acc[4 * v4 + 1], w.y);
+        score[4 * v4 + 2] = __builtin_fmaf(-2.0f, acc[4 * v4 + 2], w.z);
+        score[4 * v4 + 3] = __builtin_fmaf(-2.0f, acc[4 * v4 + 3], w.w);
+      }
       lo = __builtin_fminf(
           lo, __builtin_fminf(min3f(score[4 * v4], score[4 * v4 + 1],
                                     score[4 * v4 + 2]),

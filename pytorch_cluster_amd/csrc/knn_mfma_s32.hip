@@ -5,27 +5,35 @@ namespace pca {
 
 template <int STEPS>
 hipError_t launch_knn_mfma_steps(const KnnMfmaParams &p, int kbucket,
-                                 int grid, hipStream_t stream);
+                                 bool cosine, int grid, hipStream_t stream);
+
+template <int STEPS, int KB>
+void launch_one(const KnnMfmaParams &p, bool cosine, int grid,
+                hipStream_t stream) {
+  if (cosine)
+    hipLaunchKernelGGL((knn_mfma_kernel<STEPS, KB, true>), dim3(grid),
+                       dim3(kBlock), 0, stream, p);
+  else
+    hipLaunchKernelGGL((knn_mfma_kernel<STEPS, KB, false>), dim3(grid),
+                       dim3(kBlock), 0, stream, p);
+}
 
 template <>
 hipError_t launch_knn_mfma_steps<32>(const KnnMfmaParams &p, int kbucket,
-                                     int grid, hipStream_t stream) {
+                                     bool cosine, int grid,
+                                     hipStream_t stream) {
   switch (kbucket) {
   case 8:
-    hipLaunchKernelGGL((knn_mfma_kernel<32, 8>), dim3(grid), dim3(kBlock), 0,
-                       stream, p);
+    launch_one<32, 8>(p, cosine, grid, stream);
     break;
   case 16:
-    hipLaunchKernelGGL((knn_mfma_kernel<32, 16>), dim3(grid), dim3(kBlock), 0,
-                       stream, p);
+    launch_one<32, 16>(p, cosine, grid, stream);
     break;
   case 24:
-    hipLaunchKernelGGL((knn_mfma_kernel<32, 24>), dim3(grid), dim3(kBlock), 0,
-                       stream, p);
+    launch_one<32, 24>(p, cosine, grid, stream);
     break;
   case 32:
-    hipLaunchKernelGGL((knn_mfma_kernel<32, 32>), dim3(grid), dim3(kBlock), 0,
-                       stream, p);
+    launch_one<32, 32>(p, cosine, grid, stream);
     break;
   default:
     return hipErrorInvalidValue;

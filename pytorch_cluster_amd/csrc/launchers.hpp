@@ -76,7 +76,7 @@ constexpr int kMfmaTileQueries = 128;
 bool knn_mfma_supported(int d, int k, bool cosine);
 size_t knn_mfma_scratch_bytes(int n, int m, int num_segments, int k);
 // work_start: tiles of kMfmaTileQueries queries.
-hipError_t launch_knn_mfma(const SearchInput &in, int k,
+hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
                            const int *work_start, void *scratch,
                            const DenseResult &out, hipEvent_t time_start,
                            hipEvent_t time_stop, hipStream_t stream);

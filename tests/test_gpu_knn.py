@@ -234,6 +234,40 @@ def test_prefilter_never_drops_a_neighbour(oracle, d, k, case):
     assert (gd == wd).all()
 
 
+@pytest.mark.parametrize("d,k", [(3, 16), (24, 16), (128, 32), (100, 7)])
+@pytest.mark.parametrize("case", ["parallel", "random", "scaled_copies",
+                                  "zero_rows"])
+def test_cosine_prefilter_never_drops_a_neighbour(oracle, d, k, case):
+    rng = np.random.default_rng(hash((d, k, case, "cos")) % (2 ** 32))
+    n, m = 4000, 500
+    if case == "parallel":
+        # all rows within a narrow cone: cosine distances ~1e-6, many
+        # near-ties and slightly negative values
+        axis = rng.standard_normal((1, d))
+        x = axis * rng.uniform(0.5, 2.0, (n, 1)) + 1e-3 * rng.standard_normal((n, d))
+        y = axis * rng.uniform(0.5, 2.0, (m, 1)) + 1e-3 * rng.standard_normal((m, d))
+    elif case == "random":
+        x = rng.standard_normal((n, d))
+        y = rng.standard_normal((m, d))
+    elif case == "scaled_copies":
+        x = rng.standard_normal((n, d))
+        y = x[rng.integers(0, n, m)] * rng.uniform(1e-3, 1e3, (m, 1))
+    else:
+        x = rng.standard_normal((n, d))
+        y = rng.standard_normal((m, d))
+        x[::97] = 0.0
+        y[::31] = 0.0
+    x = x.astype(np.float32)
+    y = y.astype(np.float32)
+    ptr_x = np.array([0, 1500, 4000])
+    ptr_y = np.array([0, 200, 500])
+    got, gd = gpu_knn(x, y, ptr_x, ptr_y, k, cosine=True)
+    want, wd = oracle_knn_edges(oracle, x, y, ptr_x, ptr_y, k, cosine=True)
+    assert got.shape == want.shape
+    assert (got == want).all()
+    assert (gd == wd).all()
+
+
 def test_two_queries_per_lane_path(oracle, monkeypatch):
     rng = np.random.default_rng(77)
     x = rng.random((5000, 3), dtype=np.float32)
