@@ -183,6 +183,72 @@ def radius_op(x, y, ptr_x, ptr_y, r, max_num_neighbors, num_workers=1,
 
 
 # --------------------------------------------------------------------------
+# 16-bit element types (bit patterns as uint16; kind 0 = fp16, 1 = bf16)
+# --------------------------------------------------------------------------
+
+def _as_bits(a):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.float16:
+        a = a.view(np.uint16)
+    if a.dtype != np.uint16 or a.ndim != 2:
+        raise TypeError("expected a 2-D uint16 / float16 array")
+    return a
+
+
+def round16(v, kind):
+    lib = _load()
+    lib.oracle_round16.restype = ctypes.c_float
+    return float(lib.oracle_round16(ctypes.c_float(float(v)),
+                                    ctypes.c_int(kind)))
+
+
+def knn_op16(x_bits, y_bits, ptr_x, ptr_y, k, cosine=False, kind=0):
+    """``torch_cluster::knn`` for fp16 / bf16 points as the GPU build computes
+    it (c10::Half / c10::BFloat16 arithmetic); returns ([2, E], dist [E])."""
+    lib = _load()
+    if k > 100:
+        raise RuntimeError("`k` needs to smaller than or equal to 100")
+    x, y = _as_bits(x_bits), _as_bits(y_bits)
+    ptr_x, ptr_y = _as_ptr(ptr_x), _as_ptr(ptr_y)
+    nseg = 1 if ptr_x is None else ptr_x.size - 1
+    m = y.shape[0]
+    row = np.empty(m * k, dtype=np.int64)
+    col = np.empty(m * k, dtype=np.int64)
+    dist = np.empty(m * k, dtype=np.float32)
+    rc = lib.oracle_knn_dense_16(
+        _ptr(x), _ptr(y), _ptr(ptr_x), _ptr(ptr_y), ctypes.c_int64(x.shape[0]),
+        ctypes.c_int64(m), ctypes.c_int64(x.shape[1]), ctypes.c_int64(nseg),
+        ctypes.c_int64(k), ctypes.c_int(int(cosine)), ctypes.c_int(kind),
+        _ptr(row), _ptr(col), _ptr(dist))
+    if rc != 0:
+        raise RuntimeError("oracle_knn_dense_16 failed")
+    return _compact(row, col, col), dist[col != -1]
+
+
+def radius_op16(x_bits, y_bits, ptr_x, ptr_y, r, max_num_neighbors,
+                ignore_same_index=False, kind=0):
+    """``torch_cluster::radius`` for fp16 / bf16 points."""
+    lib = _load()
+    x, y = _as_bits(x_bits), _as_bits(y_bits)
+    ptr_x, ptr_y = _as_ptr(ptr_x), _as_ptr(ptr_y)
+    nseg = 1 if ptr_x is None else ptr_x.size - 1
+    m = y.shape[0]
+    row = np.empty(m * max_num_neighbors, dtype=np.int64)
+    col = np.empty(m * max_num_neighbors, dtype=np.int64)
+    # (scalar_t)(r * r): double -> float -> 16 bits
+    r2 = round16(np.float32(float(r) * float(r)), kind)
+    rc = lib.oracle_radius_dense_16(
+        _ptr(x), _ptr(y), _ptr(ptr_x), _ptr(ptr_y), ctypes.c_int64(x.shape[0]),
+        ctypes.c_int64(m), ctypes.c_int64(x.shape[1]), ctypes.c_int64(nseg),
+        ctypes.c_float(r2), ctypes.c_int64(max_num_neighbors),
+        ctypes.c_int(int(ignore_same_index)), ctypes.c_int(kind), _ptr(row),
+        _ptr(col))
+    if rc != 0:
+        raise RuntimeError("oracle_radius_dense_16 failed")
+    return _compact(row, col, row)
+
+
+# --------------------------------------------------------------------------
 # Python entry points (torch_cluster/knn.py, torch_cluster/radius.py)
 # --------------------------------------------------------------------------
 

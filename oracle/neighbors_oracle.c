@@ -200,6 +200,246 @@ static int64_t example_idx(int64_t idx, const int64_t *ptr,
 DEFINE_ORACLE(f32, float, fmaf, sqrtf)
 DEFINE_ORACLE(f64, double, fma, sqrt)
 
+/* ------------------------------------------------------------------------
+ * 16-bit element types (IEEE half, bfloat16).
+ *
+ * In the reference's kernels `scalar_t` is c10::Half / c10::BFloat16, whose
+ * arithmetic operators convert to float, operate, and round the result back
+ * to 16 bits (torch/headeronly/util/Half.h:501-560, BFloat16.h): every
+ * `x - y`, every product and every `+=` of knn_kernel / radius_kernel rounds
+ * once, and nothing is fused.  The functions below restate exactly that:
+ * values are carried as floats that are representable in the 16-bit type.
+ * kind: 0 = IEEE half, 1 = bfloat16.
+ * ------------------------------------------------------------------------ */
+
+static float half_bits_to_float(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1fu;
+  uint32_t man = h & 0x3ffu;
+  uint32_t bits;
+  if (exp == 0) {
+    if (man == 0) {
+      bits = sign;
+    } else { /* subnormal: normalise */
+      int shift = 0;
+      while (!(man & 0x400u)) {
+        man <<= 1;
+        shift++;
+      }
+      man &= 0x3ffu;
+      bits = sign | ((uint32_t)(127 - 15 - shift + 1) << 23) | (man << 13);
+    }
+  } else if (exp == 31) {
+    bits = sign | 0x7f800000u | (man << 13);
+  } else {
+    bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+  }
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+
+/* float -> nearest half (ties to even) -> float */
+static float round_to_half(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  uint32_t sign = x & 0x80000000u;
+  uint32_t ax = x & 0x7fffffffu;
+  uint16_t h;
+  if (ax > 0x7f800000u) { /* NaN */
+    h = 0x7e00u;
+  } else if (ax >= 0x477ff000u) { /* rounds to >= 65520 -> inf */
+    h = 0x7c00u;
+  } else if (ax < 0x33000001u) { /* below half of the smallest subnormal */
+    h = 0;
+  } else if (ax < 0x38800000u) { /* subnormal half */
+    int e = (int)(ax >> 23);          /* biased float exponent */
+    uint32_t man = (ax & 0x7fffffu) | 0x800000u;
+    int shift = 126 - e;              /* bits dropped below 2^-24 */
+    uint32_t kept = man >> shift;
+    uint32_t rem = man & ((1u << shift) - 1u);
+    uint32_t halfway = 1u << (shift - 1);
+    if (rem > halfway || (rem == halfway && (kept & 1u)))
+      kept++;
+    h = (uint16_t)kept;
+  } else {
+    uint32_t man = ax & 0x7fffffu;
+    uint32_t e = (ax >> 23) - 127 + 15;
+    uint32_t kept = (e << 10) | (man >> 13);
+    uint32_t rem = man & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (kept & 1u)))
+      kept++;
+    h = (uint16_t)kept;
+  }
+  float r = half_bits_to_float(h);
+  uint32_t rb;
+  memcpy(&rb, &r, 4);
+  rb |= sign;
+  memcpy(&r, &rb, 4);
+  return r;
+}
+
+static float bf16_bits_to_float(uint16_t b) {
+  uint32_t bits = (uint32_t)b << 16;
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+
+/* float -> nearest bfloat16 (ties to even) -> float */
+static float round_to_bf16(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  if ((x & 0x7fffffffu) > 0x7f800000u) {
+    x = 0x7fc00000u;
+  } else {
+    x += 0x7fffu + ((x >> 16) & 1u);
+    x &= 0xffff0000u;
+  }
+  memcpy(&f, &x, 4);
+  return f;
+}
+
+static float load16(const uint16_t *p, int64_t i, int kind) {
+  return kind ? bf16_bits_to_float(p[i]) : half_bits_to_float(p[i]);
+}
+
+static float round16(float v, int kind) {
+  return kind ? round_to_bf16(v) : round_to_half(v);
+}
+
+float oracle_round16(float v, int kind) { return round16(v, kind); }
+
+static float sqdist16(const uint16_t *x, const uint16_t *y, int64_t n_x,
+                      int64_t n_y, int64_t dim, int kind) {
+  float acc = 0;
+  for (int64_t d = 0; d < dim; d++) {
+    float diff = round16(
+        load16(x, n_x * dim + d, kind) - load16(y, n_y * dim + d, kind), kind);
+    float prod = round16(diff * diff, kind);
+    acc = round16(acc + prod, kind);
+  }
+  return acc;
+}
+
+static float dot16(const uint16_t *a, const uint16_t *b, int64_t n_a,
+                   int64_t n_b, int64_t size, int kind) {
+  float result = 0;
+  for (int64_t i = 0; i < size; i++) {
+    float prod = round16(
+        load16(a, n_a * size + i, kind) * load16(b, n_b * size + i, kind),
+        kind);
+    result = round16(result + prod, kind);
+  }
+  return result;
+}
+
+static float norm16(const uint16_t *a, int64_t n_a, int64_t size, int kind) {
+  return round16(sqrtf(dot16(a, a, n_a, n_a, size, kind)), kind);
+}
+
+/* knn_kernel with a 16-bit scalar_t; dist (optional) receives the distances
+ * as floats holding 16-bit-representable values. */
+int oracle_knn_dense_16(const uint16_t *x, const uint16_t *y,
+                        const int64_t *ptr_x, const int64_t *ptr_y, int64_t n,
+                        int64_t m, int64_t dim, int64_t num_examples,
+                        int64_t k, int cosine, int kind, int64_t *row,
+                        int64_t *col, float *dist) {
+  int64_t default_ptr_x[2] = {0, n}, default_ptr_y[2] = {0, m};
+  if (ptr_x == NULL || ptr_y == NULL) {
+    ptr_x = default_ptr_x;
+    ptr_y = default_ptr_y;
+    num_examples = 1;
+  }
+  if (k <= 0)
+    return 1;
+  const float sentinel = round16(1e10f, kind); /* half: +inf */
+#pragma omp parallel
+  {
+    float *best_dist = (float *)malloc(sizeof(float) * (size_t)k);
+    int64_t *best_idx = (int64_t *)malloc(sizeof(int64_t) * (size_t)k);
+#pragma omp for schedule(dynamic, 64)
+    for (int64_t n_y = 0; n_y < m; n_y++) {
+      int64_t b = example_idx(n_y, ptr_y, num_examples);
+      for (int64_t e = 0; e < k; e++) {
+        best_dist[e] = sentinel;
+        best_idx[e] = -1;
+      }
+      for (int64_t n_x = ptr_x[b]; n_x < ptr_x[b + 1]; n_x++) {
+        float tmp_dist;
+        if (cosine) {
+          float den = round16(norm16(x, n_x, dim, kind) *
+                                  norm16(y, n_y, dim, kind),
+                              kind);
+          tmp_dist =
+              round16(dot16(x, y, n_x, n_y, dim, kind) / den, kind);
+          /* `1. - tmp_dist`: double arithmetic, narrowed through float */
+          tmp_dist = round16((float)(1. - (double)tmp_dist), kind);
+        } else {
+          tmp_dist = sqdist16(x, y, n_x, n_y, dim, kind);
+        }
+        for (int64_t e1 = 0; e1 < k; e1++) {
+          if (best_dist[e1] > tmp_dist) {
+            for (int64_t e2 = k - 1; e2 > e1; e2--) {
+              best_dist[e2] = best_dist[e2 - 1];
+              best_idx[e2] = best_idx[e2 - 1];
+            }
+            best_dist[e1] = tmp_dist;
+            best_idx[e1] = n_x;
+            break;
+          }
+        }
+      }
+      for (int64_t e = 0; e < k; e++) {
+        row[n_y * k + e] = n_y;
+        col[n_y * k + e] = best_idx[e];
+        if (dist)
+          dist[n_y * k + e] = best_dist[e];
+      }
+    }
+    free(best_dist);
+    free(best_idx);
+  }
+  return 0;
+}
+
+/* radius_kernel with a 16-bit scalar_t; r2 = (scalar_t)(r * r) as a float. */
+int oracle_radius_dense_16(const uint16_t *x, const uint16_t *y,
+                           const int64_t *ptr_x, const int64_t *ptr_y,
+                           int64_t n, int64_t m, int64_t dim,
+                           int64_t num_examples, float r2,
+                           int64_t max_num_neighbors, int ignore_same_index,
+                           int kind, int64_t *row, int64_t *col) {
+  int64_t default_ptr_x[2] = {0, n}, default_ptr_y[2] = {0, m};
+  if (ptr_x == NULL || ptr_y == NULL) {
+    ptr_x = default_ptr_x;
+    ptr_y = default_ptr_y;
+    num_examples = 1;
+  }
+  if (max_num_neighbors <= 0)
+    return 1;
+  for (int64_t i = 0; i < m * max_num_neighbors; i++) {
+    row[i] = -1;
+    col[i] = -1;
+  }
+#pragma omp parallel for schedule(dynamic, 64)
+  for (int64_t n_y = 0; n_y < m; n_y++) {
+    int64_t count = 0;
+    int64_t b = example_idx(n_y, ptr_y, num_examples);
+    for (int64_t n_x = ptr_x[b]; n_x < ptr_x[b + 1]; n_x++) {
+      float d = sqdist16(x, y, n_x, n_y, dim, kind);
+      if (d < r2 && !(ignore_same_index && n_y == n_x)) {
+        row[n_y * max_num_neighbors + count] = n_y;
+        col[n_y * max_num_neighbors + count] = n_x;
+        count++;
+      }
+      if (count >= max_num_neighbors)
+        break;
+    }
+  }
+  return 0;
+}
+
 /* Host-wrapper epilogue: keep the slots whose `mask_src` entry is not -1, in
  * slot order, and stack them as [2, E] (row-major, leading dimension E).
  * Returns E; writes nothing when out is NULL. */

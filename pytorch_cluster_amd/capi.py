@@ -9,7 +9,10 @@ from typing import Optional, Tuple
 
 import torch
 
-from ._native import PCA_F32, capi
+from ._native import PCA_BF16, PCA_F16, PCA_F32, PCA_F64, capi
+
+_DTYPE_CODE = {torch.float32: PCA_F32, torch.float64: PCA_F64,
+               torch.float16: PCA_F16, torch.bfloat16: PCA_BF16}
 
 
 class PcaError(RuntimeError):
@@ -49,11 +52,12 @@ def knn_launch(x, y, ptr_x, ptr_y, k: int, cosine: bool = False,
     """Queues ``pca_knn``; returns (edges buffer [2*m*k], num_edges [1] on the
     device, dist buffer or None, workspace).  Nothing is synchronised."""
     assert x.is_cuda and y.is_cuda and x.is_contiguous() and y.is_contiguous()
-    assert x.dtype == torch.float32 and y.dtype == torch.float32
+    assert x.dtype == y.dtype and x.dtype in _DTYPE_CODE
+    dtype = _DTYPE_CODE[x.dtype]
     n, d = x.shape
     m = y.shape[0]
     ptr_x, ptr_y, nseg = _segments(ptr_x, ptr_y)
-    ws_bytes = capi.pca_knn_workspace_bytes(n, m, d, nseg, k, PCA_F32)
+    ws_bytes = capi.pca_knn_workspace_bytes(n, m, d, nseg, k, dtype)
     if ws_bytes == 0:
         # let the entry point produce the precise error
         ws_bytes = 256
@@ -65,7 +69,7 @@ def knn_launch(x, y, ptr_x, ptr_y, k: int, cosine: bool = False,
                         device=x.device) if want_dist else None)
     _check(capi.pca_knn(_dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x),
                         _dev_ptr(ptr_y), n, m, d, nseg, k, int(cosine),
-                        PCA_F32, _dev_ptr(edges), _dev_ptr(num_edges),
+                        dtype, _dev_ptr(edges), _dev_ptr(num_edges),
                         _dev_ptr(dist), _dev_ptr(ws), ws_bytes,
                         _stream_handle(stream, x.device)))
     return edges, num_edges, dist, ws
@@ -85,12 +89,13 @@ def knn_edges(x, y, ptr_x=None, ptr_y=None, k: int = 1, cosine: bool = False,
 def radius_launch(x, y, ptr_x, ptr_y, r: float, max_num_neighbors: int,
                   ignore_same_index: bool = False, stream=None):
     assert x.is_cuda and y.is_cuda and x.is_contiguous() and y.is_contiguous()
-    assert x.dtype == torch.float32 and y.dtype == torch.float32
+    assert x.dtype == y.dtype and x.dtype in _DTYPE_CODE
+    dtype = _DTYPE_CODE[x.dtype]
     n, d = x.shape
     m = y.shape[0]
     ptr_x, ptr_y, nseg = _segments(ptr_x, ptr_y)
     ws_bytes = capi.pca_radius_workspace_bytes(n, m, d, nseg,
-                                               max_num_neighbors, PCA_F32)
+                                               max_num_neighbors, dtype)
     if ws_bytes == 0:
         ws_bytes = 256
     slots = capi.pca_radius_slots(n, max_num_neighbors)
@@ -100,7 +105,7 @@ def radius_launch(x, y, ptr_x, ptr_y, r: float, max_num_neighbors: int,
     num_edges = torch.empty(1, dtype=torch.long, device=x.device)
     _check(capi.pca_radius(_dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x),
                            _dev_ptr(ptr_y), n, m, d, nseg, float(r),
-                           max_num_neighbors, int(ignore_same_index), PCA_F32,
+                           max_num_neighbors, int(ignore_same_index), dtype,
                            _dev_ptr(edges), _dev_ptr(num_edges), _dev_ptr(ws),
                            ws_bytes, _stream_handle(stream, x.device)))
     return edges, num_edges, ws

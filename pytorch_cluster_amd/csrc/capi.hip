@@ -82,9 +82,11 @@ struct KnnLayout {
 };
 
 KnnLayout knn_layout(int64_t n, int64_t m, int64_t d, int64_t num_segments,
-                     int64_t k) {
+                     int64_t k, int dtype) {
   KnnLayout w;
-  if (d > 8) {
+  if (dtype != PCA_F32) {
+    w.x_norm = align256(pca::anytype_norm_bytes((int)n));
+  } else if (d > 8) {
     w.x_norm = align256(sizeof(float) * (size_t)n);
     if (pca::knn_mfma_supported((int)d, (int)k, false))
       w.sliced = pca::knn_mfma_scratch_bytes((int)n, (int)m,
@@ -109,8 +111,13 @@ KnnLayout knn_layout(int64_t n, int64_t m, int64_t d, int64_t num_segments,
 }
 
 size_t knn_workspace(int64_t n, int64_t m, int64_t d, int64_t num_segments,
-                     int64_t k) {
-  return knn_layout(n, m, d, num_segments, k).total();
+                     int64_t k, int dtype) {
+  return knn_layout(n, m, d, num_segments, k, dtype).total();
+}
+
+bool dtype_ok(int dtype) {
+  return dtype == PCA_F32 || dtype == PCA_F64 || dtype == PCA_F16 ||
+         dtype == PCA_BF16;
 }
 
 size_t radius_workspace(int64_t m, int64_t num_segments, int64_t slots) {
@@ -168,12 +175,12 @@ int pca_time_next_search(void *start_event, void *stop_event) {
 
 size_t pca_knn_workspace_bytes(int64_t n, int64_t m, int64_t d,
                                int64_t num_segments, int64_t k, int dtype) {
-  (void)dtype;
   if (num_segments < 1)
     num_segments = 1;
-  if (!sizes_ok(n, m, d, num_segments) || k < 1 || k > PCA_KNN_MAX_K)
+  if (!sizes_ok(n, m, d, num_segments) || k < 1 || k > PCA_KNN_MAX_K ||
+      !dtype_ok(dtype))
     return 0;
-  return knn_workspace(n, m, d, num_segments, k);
+  return knn_workspace(n, m, d, num_segments, k, dtype);
 }
 
 int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
@@ -202,8 +209,11 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
                 pca_status_string(PCA_ERR_K_TOO_LARGE));
   if (num_edges == nullptr)
     return fail(PCA_ERR_INVALID_ARGUMENT, "num_edges is NULL");
-  if (dtype != PCA_F32)
+  if (!dtype_ok(dtype))
     return fail(PCA_ERR_UNSUPPORTED, "element type %d is not built", dtype);
+  if (dtype != PCA_F32 && dist != nullptr)
+    return fail(PCA_ERR_UNSUPPORTED,
+                "per-edge distances are returned for fp32 points only");
 
   if (n == 0 || m == 0) {
     hipLaunchKernelGGL(set_i64_kernel, dim3(1), dim3(1), 0, stream, num_edges,
@@ -213,13 +223,15 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
   if (x == nullptr || y == nullptr || edges == nullptr)
     return fail(PCA_ERR_INVALID_ARGUMENT, "x, y or edges is NULL");
   if (workspace == nullptr || ((uintptr_t)workspace & 255) != 0 ||
-      workspace_bytes < knn_workspace(n, m, d, num_segments, k))
+      workspace_bytes < knn_workspace(n, m, d, num_segments, k, dtype))
     return fail(PCA_ERR_WORKSPACE, "workspace needs %zu bytes, 256-aligned",
-                knn_workspace(n, m, d, num_segments, k));
+                knn_workspace(n, m, d, num_segments, k, dtype));
 
-  const bool low_d = pca::knn_lowd_supported((int)d, (int)k, cosine != 0);
+  const bool f32 = dtype == PCA_F32;
+  const bool low_d =
+      f32 && pca::knn_lowd_supported((int)d, (int)k, cosine != 0);
 
-  const KnnLayout lay = knn_layout(n, m, d, num_segments, k);
+  const KnnLayout lay = knn_layout(n, m, d, num_segments, k, dtype);
   char *cursor = static_cast<char *>(workspace);
   auto take = [&cursor](size_t bytes) {
     char *piece = cursor;
@@ -243,7 +255,7 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
   pca::SearchInput in{x,      y,      ptr_x,  ptr_y,
                       (int)n, (int)m, (int)d, (int)num_segments};
   const bool mfma =
-      !low_d && pca::knn_mfma_supported((int)d, (int)k, cosine != 0);
+      f32 && !low_d && pca::knn_mfma_supported((int)d, (int)k, cosine != 0);
   if (mfma)
     cfg.tile_queries = pca::kMfmaTileQueries;
   else if (!low_d)
@@ -269,6 +281,13 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
                                            timer.stop, stream),
                       "knn_mfma_kernel");
     timer.stop = nullptr;
+  } else if (!f32) {
+    timer.begin();
+    rc = check_launch(pca::launch_knn_anytype(dtype, in, (int)k, cosine != 0,
+                                              x_norm, work_start, bound,
+                                              dense, stream),
+                      "knn_any_kernel");
+    timer.done();
   } else {
     if (cosine) {
       rc = check_launch(pca::launch_row_norms(static_cast<const float *>(x),
@@ -301,10 +320,10 @@ int64_t pca_radius_slots(int64_t n, int64_t max_num_neighbors) {
 size_t pca_radius_workspace_bytes(int64_t n, int64_t m, int64_t d,
                                   int64_t num_segments,
                                   int64_t max_num_neighbors, int dtype) {
-  (void)dtype;
   if (num_segments < 1)
     num_segments = 1;
-  if (!sizes_ok(n, m, d, num_segments) || max_num_neighbors < 1)
+  if (!sizes_ok(n, m, d, num_segments) || max_num_neighbors < 1 ||
+      !dtype_ok(dtype))
     return 0;
   return radius_workspace(m, num_segments,
                           pca_radius_slots(n, max_num_neighbors));
@@ -335,7 +354,7 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
                 (long long)max_num_neighbors);
   if (num_edges == nullptr)
     return fail(PCA_ERR_INVALID_ARGUMENT, "num_edges is NULL");
-  if (dtype != PCA_F32)
+  if (!dtype_ok(dtype))
     return fail(PCA_ERR_UNSUPPORTED, "element type %d is not built", dtype);
 
   if (n == 0 || m == 0) {
@@ -375,9 +394,16 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
   const int bound = pca::plan_upper_bound((int)m, (int)num_segments,
                                           pca::kRadiusQueriesPerWave);
   timer.begin();
-  rc = check_launch(pca::launch_radius(in, r2, ignore_same_index != 0,
-                                       work_start, bound, dense, stream),
-                    "radius_kernel");
+  if (dtype == PCA_F32)
+    rc = check_launch(pca::launch_radius(in, r2, ignore_same_index != 0,
+                                         work_start, bound, dense, stream),
+                      "radius_kernel");
+  else
+    rc = check_launch(pca::launch_radius_anytype(dtype, in, r,
+                                                 ignore_same_index != 0,
+                                                 work_start, bound, dense,
+                                                 stream),
+                      "radius_any_kernel");
   timer.done();
   if (rc != PCA_OK)
     return rc;

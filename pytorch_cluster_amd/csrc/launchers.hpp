@@ -93,6 +93,20 @@ hipError_t launch_knn_generic(const SearchInput &in, int k, bool cosine,
                               int grid_bound, const DenseResult &out,
                               hipStream_t stream);
 
+// --- anytype.hip (fp64 / fp16 / bf16; dtype codes of enum pca_dtype) -------
+
+size_t anytype_norm_bytes(int n);
+// work_start: tiles of kBlock queries (kNN), wave tasks of
+// kRadiusQueriesPerWave queries (radius).
+hipError_t launch_knn_anytype(int dtype, const SearchInput &in, int k,
+                              bool cosine, void *x_norm,
+                              const int *work_start, int grid_bound,
+                              const DenseResult &out, hipStream_t stream);
+hipError_t launch_radius_anytype(int dtype, const SearchInput &in, double r,
+                                 bool ignore_same_index,
+                                 const int *work_start, int task_bound,
+                                 const DenseResult &out, hipStream_t stream);
+
 // --- radius.hip ------------------------------------------------------------
 
 constexpr int kRadiusQueriesPerWave = 8;

@@ -43,9 +43,12 @@ def test_capi_validation_needs_no_gpu():
     rc = capi.pca_knn(one, one, None, None, 10, 10, 3, 1, 4, 0, 0, one, one,
                       None, one, 16, None)
     assert rc == -3  # workspace too small
-    rc = capi.pca_knn(one, one, None, None, 10, 10, 3, 1, 4, 0, 1, one, one,
+    rc = capi.pca_knn(one, one, None, None, 10, 10, 3, 1, 4, 0, 7, one, one,
                       None, one, 1 << 20, None)
-    assert rc == -5  # float64 not built
+    assert rc == -5  # no such element type
+    rc = capi.pca_knn(one, one, None, None, 10, 10, 3, 1, 4, 0, 1, one, one,
+                      one, one, 1 << 20, None)
+    assert rc == -5  # distances are written for fp32 points only
     rc = capi.pca_radius(one, one, None, None, 10, 10, 3, 1, 0.5, 0, 0, 0,
                          one, one, one, 1 << 20, None)
     assert rc == -1  # max_num_neighbors must be >= 1

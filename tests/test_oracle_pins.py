@@ -256,3 +256,46 @@ def test_ref_radius_truncated_counts_and_subset(ref):
     assert (np.bincount(ours[0], minlength=2000) ==
             np.bincount(theirs[0], minlength=2000)).all()
     assert to_set(ours) <= full and to_set(theirs) <= full
+
+
+# ---- 16-bit element types ---------------------------------------------------
+
+def _bits(t):
+    import torch
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("kind", [0, 1])
+def test_16bit_rounding_matches_torch(oracle, kind):
+    import torch
+    dt = torch.float16 if kind == 0 else torch.bfloat16
+    rng = np.random.default_rng(kind)
+    vals = np.concatenate(
+        [rng.standard_normal(3000).astype(np.float32) * s
+         for s in (1e-8, 1e-5, 1e-3, 1, 100, 6e4, 1e5)] +
+        [np.array([0, -0.0, np.inf, -np.inf, 65504, 65519.99, 65520, 6.1e-5,
+                   5.96e-8, 2.98e-8, 2.9802325e-8, 8.9e-8], dtype=np.float32)])
+    want = torch.from_numpy(vals).to(dt).to(torch.float32).numpy()
+    got = np.array([oracle.round16(v, kind) for v in vals], dtype=np.float32)
+    assert (got.view(np.uint32) == want.view(np.uint32)).all()
+
+
+@pytest.mark.parametrize("kind", [0, 1])
+def test_16bit_knn_matches_torch_scalar_semantics(oracle, kind):
+    # independent restatement with torch CPU tensors of the 16-bit type: every
+    # elementwise operator rounds once, like c10::Half / c10::BFloat16
+    import torch
+    dt = torch.float16 if kind == 0 else torch.bfloat16
+    g = torch.Generator().manual_seed(kind)
+    x = torch.randn(60, 3, generator=g).to(dt)
+    y = torch.randn(9, 3, generator=g).to(dt)
+    k = 5
+    got, dist = oracle.knn_op16(_bits(x), _bits(y), None, None, k, False, kind)
+    acc = torch.zeros(9, 60, dtype=dt)
+    for c in range(3):
+        diff = y[:, None, c] - x[None, :, c]
+        acc = acc + diff * diff
+    d = acc.to(torch.float32).numpy()
+    order = np.argsort(d, axis=1, kind="stable")[:, :k]
+    assert (got[1].reshape(9, k) == order).all()
+    assert (dist.reshape(9, k) == np.take_along_axis(d, order, 1)).all()
