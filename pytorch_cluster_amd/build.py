@@ -24,10 +24,13 @@ TORCH_OPS_LIB = os.path.join(HERE, "_torch_ops.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 
-# Packed FP32 instructions are switched off for every device compile.
+# Packed FP32 instructions are switched off for every device compile.  Matrix
+# core results are compared by the vector ALU right away, so they are kept in
+# ordinary vector registers (no accumulator-register copies).
 HIP_FLAGS = [
     "--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument",
 ]
 

@@ -97,7 +97,8 @@ KnnLayout knn_layout(int64_t n, int64_t m, int64_t d, int64_t num_segments,
       const pca::KnnLowdConfig cfg = pca::knn_lowd_config(
           (int)d, (int)k, (int)n, (int)m, (int)num_segments, cosine != 0);
       w.sliced = std::max(w.sliced,
-                          pca::knn_lowd_scratch_bytes(cfg, (int)m,
+                          pca::knn_lowd_scratch_bytes(cfg, (int)n, (int)m,
+                                                      (int)d,
                                                       (int)num_segments,
                                                       (int)k));
     }

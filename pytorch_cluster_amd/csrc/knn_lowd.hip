@@ -2,6 +2,7 @@
 // the any-dimension kernel (knn_generic_impl.hpp).
 #include "knn_generic_impl.hpp"
 #include "knn_lowd_impl.hpp"
+#include "knn_lowd_mc_impl.hpp"
 
 #include <cstdlib>
 
@@ -42,10 +43,15 @@ __global__ __launch_bounds__(kBlock) void fill_f32_kernel(float *p, int n,
 }
 
 template <int KB>
-void launch_merge(const KnnLowdParams &p, int queries_per_lane,
-                  int tiles_bound, hipStream_t stream) {
+void launch_merge(const KnnLowdParams &p, int tile_queries, int tiles_bound,
+                  hipStream_t stream) {
   if constexpr (KB <= 32) {
-    if (queries_per_lane == 2) {
+    if (tile_queries == kMcQueries) {
+      hipLaunchKernelGGL((knn_merge_kernel<KB, kMcQueries>), dim3(tiles_bound),
+                         dim3(kBlock), 0, stream, p);
+      return;
+    }
+    if (tile_queries == 2 * kBlock) {
       hipLaunchKernelGGL((knn_merge_kernel<KB, 2 * kBlock>), dim3(tiles_bound),
                          dim3(kBlock), 0, stream, p);
       return;
@@ -75,6 +81,13 @@ KnnLowdConfig knn_lowd_config(int /*d*/, int k, int n, int m,
   (void)m;
   cfg.queries_per_lane = qpt;
   cfg.tile_queries = kBlock * qpt;
+  // Euclidean lists of up to 32 entries: pre-filter on the matrix cores
+  cfg.matrix_cores = !cosine && cfg.kbucket <= 32 &&
+                     env_int("PCA_KNN_LOWD_MATRIX_CORES", 1) != 0;
+  if (cfg.matrix_cores) {
+    cfg.queries_per_lane = 1;
+    cfg.tile_queries = kMcQueries;
+  }
 
   // Slices of x per segment: enough work items (~32 per CU) to even out
   // ragged segments, but slices of at least ~4 LDS tiles on average -- every
@@ -87,17 +100,69 @@ KnnLowdConfig knn_lowd_config(int /*d*/, int k, int n, int m,
   if (forced_chunks >= 1 && forced_chunks <= 64)
     chunks = forced_chunks;
   cfg.num_chunks = chunks;
+
+  // Bound-seeding pass: worth its ~sample/segment share of the scan once the
+  // segments are much longer than the sample.
+  cfg.sample_rows = 0;
+  const int sample = env_int("PCA_KNN_SAMPLE", 2048);
+  if (sample > 0 && !cosine && (n / num_segments) >= 16 * sample &&
+      sample >= 4 * k)
+    cfg.sample_rows = sample;
   return cfg;
 }
 
-size_t knn_lowd_scratch_bytes(const KnnLowdConfig &cfg, int m,
-                              int num_segments, int k) {
-  if (cfg.num_chunks <= 1)
+// packed operand rows of the matrix-core kernel
+size_t mc_split_bytes(const KnnLowdConfig &cfg, int n, int d) {
+  if (!cfg.matrix_cores)
     return 0;
-  const size_t tiles = plan_upper_bound(m, num_segments, cfg.tile_queries);
-  return align256(sizeof(float) * (size_t)m) +
-         align256(sizeof(double) * tiles * cfg.num_chunks * (size_t)k *
-                  cfg.tile_queries);
+  const int dim = padded_dim(d);
+  const int per_row = (dim + 1 + 3) / 4; // McShape<dim>::NI
+  return align256(sizeof(uint4) * (size_t)n * per_row);
+}
+
+size_t knn_lowd_scratch_bytes(const KnnLowdConfig &cfg, int n, int m, int d,
+                              int num_segments, int k) {
+  size_t bytes = align256(sizeof(float) * (size_t)m); // shared bounds
+  bytes += mc_split_bytes(cfg, n, d);
+  if (cfg.num_chunks > 1) {
+    const size_t tiles = plan_upper_bound(m, num_segments, cfg.tile_queries);
+    bytes += align256(sizeof(double) * tiles * cfg.num_chunks * (size_t)k *
+                      cfg.tile_queries);
+  }
+  return bytes;
+}
+
+// One launch of knn_lowd_kernel for the padded dimension and metric.
+hipError_t launch_lowd_pass(const KnnLowdParams &p, const KnnLowdConfig &cfg,
+                            int dim, bool cosine, int tiles_bound,
+                            hipStream_t stream) {
+  if (cfg.matrix_cores) {
+    const int grid = tiles_bound * p.num_chunks;
+    switch (dim) {
+    case 2:
+      return launch_knn_lowd_mc_dim<2>(p, cfg.kbucket, grid, stream);
+    case 3:
+      return launch_knn_lowd_mc_dim<3>(p, cfg.kbucket, grid, stream);
+    case 4:
+      return launch_knn_lowd_mc_dim<4>(p, cfg.kbucket, grid, stream);
+    case 8:
+      return launch_knn_lowd_mc_dim<8>(p, cfg.kbucket, grid, stream);
+    }
+    return hipErrorInvalidValue;
+  }
+#define PCA_DIM_CASE(D)                                                        \
+  case D:                                                                      \
+    return cosine ? launch_knn_lowd_dim<D, true>(p, cfg, tiles_bound, stream)  \
+                  : launch_knn_lowd_dim<D, false>(p, cfg, tiles_bound,         \
+                                                  stream);
+  switch (dim) {
+    PCA_DIM_CASE(2)
+    PCA_DIM_CASE(3)
+    PCA_DIM_CASE(4)
+    PCA_DIM_CASE(8)
+  }
+#undef PCA_DIM_CASE
+  return hipErrorInvalidValue;
 }
 
 hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
@@ -124,57 +189,84 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
   p.out_idx = out.idx;
   p.out_dist = out.dist;
   p.out_count = out.count;
-  if (cfg.num_chunks > 1) {
-    char *base = static_cast<char *>(scratch);
+  p.sample_rows = 0;
+  p.x_split = nullptr;
+  char *base = static_cast<char *>(scratch);
+  const size_t tau_bytes = align256(sizeof(float) * (size_t)in.m);
+  const size_t split_bytes = mc_split_bytes(cfg, in.n, in.d);
+  if (cfg.matrix_cores) {
+    uint4 *split = reinterpret_cast<uint4 *>(base + tau_bytes);
+    p.x_split = split;
+    hipError_t perr = hipErrorInvalidValue;
+    switch (padded_dim(in.d)) {
+    case 2:
+      perr = launch_mc_pack_rows<2>(p.x, in.n, in.d, split, stream);
+      break;
+    case 3:
+      perr = launch_mc_pack_rows<3>(p.x, in.n, in.d, split, stream);
+      break;
+    case 4:
+      perr = launch_mc_pack_rows<4>(p.x, in.n, in.d, split, stream);
+      break;
+    case 8:
+      perr = launch_mc_pack_rows<8>(p.x, in.n, in.d, split, stream);
+      break;
+    }
+    if (perr != hipSuccess)
+      return perr;
+  }
+  if (cfg.num_chunks > 1 || cfg.sample_rows > 0) {
     float *tau = reinterpret_cast<float *>(base);
-    p.partial = reinterpret_cast<double *>(
-        base + align256(sizeof(float) * (size_t)in.m));
+    if (cfg.num_chunks > 1)
+      p.partial =
+          reinterpret_cast<double *>(base + tau_bytes + split_bytes);
     p.tau = tau;
     hipLaunchKernelGGL(fill_f32_kernel, dim3((in.m + kBlock - 1) / kBlock),
                        dim3(kBlock), 0, stream, tau, in.m, kKnnSentinel);
   }
 
-  if (time_start)
-    (void)hipEventRecord(time_start, stream);
   hipError_t err = hipErrorInvalidValue;
-#define PCA_DIM_CASE(D)                                                        \
-  case D:                                                                      \
-    err = cosine ? launch_knn_lowd_dim<D, true>(p, cfg, tiles_bound, stream)   \
-                 : launch_knn_lowd_dim<D, false>(p, cfg, tiles_bound, stream); \
-    break;
-  switch (padded_dim(in.d)) {
-    PCA_DIM_CASE(2)
-    PCA_DIM_CASE(3)
-    PCA_DIM_CASE(4)
-    PCA_DIM_CASE(8)
+  for (int pass = cfg.sample_rows > 0 ? 0 : 1; pass < 2; ++pass) {
+    // pass 0 seeds the bounds from a sample of each segment, pass 1 is the
+    // search itself (the one the timing events bracket)
+    KnnLowdParams q = p;
+    if (pass == 0) {
+      q.sample_rows = cfg.sample_rows;
+      q.num_chunks = 1;
+    } else if (time_start) {
+      (void)hipEventRecord(time_start, stream);
+    }
+    err = launch_lowd_pass(q, cfg, padded_dim(in.d), cosine, tiles_bound,
+                           stream);
+    if (err != hipSuccess)
+      return err;
   }
-#undef PCA_DIM_CASE
   if (time_stop)
     (void)hipEventRecord(time_stop, stream);
-  if (err != hipSuccess || cfg.num_chunks <= 1)
+  if (cfg.num_chunks <= 1)
     return err;
 
   switch (cfg.kbucket) {
   case 8:
-    launch_merge<8>(p, cfg.queries_per_lane, tiles_bound, stream);
+    launch_merge<8>(p, cfg.tile_queries, tiles_bound, stream);
     break;
   case 16:
-    launch_merge<16>(p, cfg.queries_per_lane, tiles_bound, stream);
+    launch_merge<16>(p, cfg.tile_queries, tiles_bound, stream);
     break;
   case 24:
-    launch_merge<24>(p, cfg.queries_per_lane, tiles_bound, stream);
+    launch_merge<24>(p, cfg.tile_queries, tiles_bound, stream);
     break;
   case 32:
-    launch_merge<32>(p, cfg.queries_per_lane, tiles_bound, stream);
+    launch_merge<32>(p, cfg.tile_queries, tiles_bound, stream);
     break;
   case 48:
-    launch_merge<48>(p, cfg.queries_per_lane, tiles_bound, stream);
+    launch_merge<48>(p, cfg.tile_queries, tiles_bound, stream);
     break;
   case 64:
-    launch_merge<64>(p, cfg.queries_per_lane, tiles_bound, stream);
+    launch_merge<64>(p, cfg.tile_queries, tiles_bound, stream);
     break;
   case 100:
-    launch_merge<100>(p, cfg.queries_per_lane, tiles_bound, stream);
+    launch_merge<100>(p, cfg.tile_queries, tiles_bound, stream);
     break;
   default:
     return hipErrorInvalidValue;

@@ -41,6 +41,15 @@
 //     the merge), the slice's own k-th distance is a strict bound because all
 //     later candidates of the slice have higher rows.
 //
+// Bound-seeding pass (sample_rows > 0): the same kernel scans only every
+// stride-th x row of each segment (about sample_rows of them), keeps no
+// results and posts each query's k-th best sampled distance to `tau`.  The
+// k-th distance within any subset of the candidates bounds the final k-th
+// distance from above, so the full scan that follows starts with lists that
+// reject all but roughly k * stride candidates per query -- whatever order
+// the rows come in (a scan that approaches a query's neighbourhood gradually
+// would otherwise accept, and sort in, almost every candidate on the way).
+//
 // Results per query: rows [K-k, K) of the list = the k best (distance, row)
 // pairs in ascending order; slots never filled keep row -1 (segment smaller
 // than k, or candidates at distance >= 1e10 / NaN, which the reference never
@@ -65,7 +74,10 @@ struct KnnLowdParams {
   int n, m, d_in, num_segments, k;
   const int *work_start; // [num_segments + 1] first query tile of each segment
   int num_chunks;        // S: slices of every segment's x rows
-  float *tau;            // [m] shared pruning bounds (S > 1) or NULL
+  int sample_rows;       // > 0: bound-seeding pass over about this many
+                         // evenly spaced x rows per segment (see below)
+  const uint4 *x_split;  // matrix-core kernel: packed bf16 operand rows of x
+  float *tau;            // [m] shared pruning bounds or NULL
   double *partial;       // [S * tiles][k][tile queries] keys (S > 1) or NULL
   int *out_idx;          // dense results (written here only when S == 1)
   float *out_dist;
@@ -194,9 +206,14 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
   const int seg_len = x_end - x_begin;
   const int chunk_len =
       ((seg_len + p.num_chunks - 1) / p.num_chunks + TX - 1) / TX * TX;
-  const int c_begin = min(x_end, x_begin + chunk * chunk_len);
-  const int c_end = min(x_end, c_begin + chunk_len);
-  const int num_tiles = (c_end - c_begin + TX - 1) / TX;
+  // rows are addressed as c_begin + position * stride, position < c_count
+  const int stride = p.sample_rows > 0 ? max(1, seg_len / p.sample_rows) : 1;
+  const int c_begin =
+      p.sample_rows > 0 ? x_begin : min(x_end, x_begin + chunk * chunk_len);
+  const int c_count = p.sample_rows > 0
+                          ? (seg_len + stride - 1) / stride
+                          : min(x_end, c_begin + chunk_len) - c_begin;
+  const int num_tiles = (c_count + TX - 1) / TX;
 
   // ---- per-lane query state -------------------------------------------
   int q[QPT];
@@ -249,14 +266,15 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
   auto load_tile = [&](int t) {
 #pragma unroll
     for (int r = 0; r < PT; ++r) {
-      const int g = c_begin + t * TX + r * kBlock + tid;
+      const int pos = t * TX + r * kBlock + tid;
+      const size_t g = (size_t)c_begin + (size_t)pos * stride;
 #pragma unroll
       for (int c = 0; c < DIM; ++c) {
         // rows past the slice end become +inf: their distance is inf or
         // NaN and never passes a `<` test
         float v = __builtin_inff();
-        if (g < c_end)
-          v = c < d_in ? p.x[(size_t)g * d_in + c] : 0.0f;
+        if (pos < c_count)
+          v = c < d_in ? p.x[g * d_in + c] : 0.0f;
         stage[r][c] = v;
       }
     }
@@ -368,10 +386,12 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
     if (p.tau)
       sync_bounds();
 
+    // (row numbers only matter outside the bound-seeding pass: stride 1)
     const int g_base = c_begin + t * TX;
     // whole pairs of groups; rows between the slice end and the tile end are
     // +inf padding
-    const int limit = min(TX, (c_end - g_base + 2 * U - 1) & ~(2 * U - 1));
+    const int limit =
+        min(TX, (c_count - t * TX + 2 * U - 1) & ~(2 * U - 1));
 
     // one group of U candidates (component-major in `grp`) against this
     // lane's queries
@@ -467,6 +487,10 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
   }
 
   // ---- results --------------------------------------------------------
+  if (p.sample_rows > 0) {
+    sync_bounds(); // posts the k-th best sampled distance
+    return;
+  }
   if (p.num_chunks == 1) {
 #pragma unroll
     for (int qi = 0; qi < QPT; ++qi)

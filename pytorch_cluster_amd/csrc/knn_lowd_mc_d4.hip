@@ -1,0 +1,7 @@
+// Low-dimensional kNN with the pre-filter on the matrix cores: Euclidean
+// distance, 4 components per point.
+#include "knn_lowd_mc_impl.hpp"
+
+namespace pca {
+PCA_LOWD_MC_DEFINE(4)
+} // namespace pca

@@ -1,0 +1,544 @@
+// Brute-force Euclidean kNN for low-dimensional fp32 points (d <= 8, k <= 32)
+// with the pre-filter of knn_lowd_impl.hpp evaluated on the gfx950 matrix
+// cores.  Results are bit-identical to the reference's scalar loop
+// (csrc/cuda/knn_cuda.cu:52-78): the matrix cores only decide which
+// candidates are LOOKED AT, every distance that is kept is the exact fp32
+// chain of direct differences.
+//
+// The filter value of a (query, candidate) pair is
+//     t = w - 2 x.y,     w = fl(|x|^2) * (1 - eps),
+// the dot product of the augmented rows (x_0 .. x_{d-1}, w) and
+// (-2 y_0 .. -2 y_{d-1}, 1).  Every fp32 operand v is split into two bf16
+// numbers, v = hi + lo + r with |r| <= 2^-16 |v| (hi = bf16(v),
+// lo = bf16(v - hi); bf16 has the exponent range of fp32, so nothing
+// overflows or needs scaling), and the four partial products
+// hi*hi + lo*hi + hi*lo + lo*lo of up to four components fill the sixteen
+// accumulation slots of ONE v_mfma_f32_32x32x16_bf16 (products exact, fp32
+// accumulation): 32 candidates x 32 queries per instruction in a quarter of
+// the time the fp32 matrix instruction needs, and about a tenth of what the
+// vector ALU needs for the same 1,024 filter values.  The vector ALU is left
+// with one compare per pair.
+//
+// A candidate with t >= cut = thresh (1 + eps) - fl(|y|^2) (1 - eps) (+ a tiny
+// absolute term) can never have an exact distance below thresh, for
+// eps = 2^-14:  |t_computed - t| <= 2^-16 |w| + 2^-15 * 2 sum |x_c y_c| (the
+// split) + 50 u (|w| + 2 sum |x_c y_c|) (accumulation, u = 2^-24), the computed
+// norms are within (1 +- d u) of the true ones and the exact chain within
+// (1 +- (d + 2) u) of |x - y|^2; with 2 |x||y| <= |x|^2 + |y|^2 this gives
+//     t - cut <= |x|^2 (-eps + 2^-14.3 + (d + 1) u)
+//                + |y|^2 (-eps + 2^-14.9 + d u) + thresh ((d + 3) u - eps) < 0.
+// Operands below the bf16 normal range may be flushed to zero by the matrix
+// cores: at most 2^-126 per operand, times the other factor (below 2e15 for
+// operands of moderate norm); the absolute term of the cut covers it.  Rows
+// whose squared norm is not a moderate finite number enter with zero
+// coordinates and w = -1e38 (always looked at; an infinity would meet the
+// zero lo part of the query's 1 and turn into NaN), padding rows with w = NaN
+// (never pass a compare), queries with such a norm get cut = +inf and zero
+// coordinates (look at every real row).
+//
+// Mapping: a workgroup owns 128 queries of one segment (4 waves x 32) and one
+// slice of the segment's x rows; x streams through LDS in tiles of TX rows,
+// each row once as the packed bf16 operand and once as fp32 coordinates for
+// the exact distances.  Per 32-row step lane l supplies candidate row l % 32
+// (both lane halves the same 16 bytes) and the hi (l < 32) or lo (l >= 32)
+// parts of query l % 32; it receives the filter values of query l % 32
+// against the 16 rows 8 (v / 4) + 4 (l / 32) + v % 4.  So lanes l and l + 32
+// share a query and split its candidates: each keeps its own sorted list (its
+// rows arrive in ascending order, so its own k-th distance is a strict
+// bound), the two exchange their k-th distances after every drain, and the
+// lists are united at the end.  Candidates that pass the filter are parked
+// (position in the tile) in a per-lane LDS queue and resolved by all lanes
+// together, exactly, when a queue fills up or the tile ends -- as in
+// knn_lowd_impl.hpp.  Slices, shared bounds (`tau`) and the merge of partial
+// lists are those of knn_lowd_impl.hpp with tiles of 128 queries.
+//
+// Bound-seeding pass (sample_rows > 0): see knn_lowd_impl.hpp.
+#pragma once
+
+#include "knn_mfma_impl.hpp"
+
+namespace pca {
+
+constexpr int kMcQueries = 128; // queries per workgroup
+constexpr int kMcQueueCap = 32; // parked candidates per lane
+
+typedef __bf16 mc_bf16x8_t __attribute__((ext_vector_type(8)));
+
+template <int DIM> struct McShape {
+  // matrix instructions per 32-row step: four augmented components each
+  static constexpr int NI = (DIM + 1 + 3) / 4;
+  static constexpr int XF = DIM <= 4 ? 4 : 8; // fp32 coordinates per row
+  static constexpr int TX = DIM <= 4 ? 512 : 256; // rows per LDS tile
+};
+
+// bf16 nearest-even of a finite float of moderate size, as the upper half of
+// a float
+__device__ __forceinline__ uint32_t mc_bf16_bits(float v) {
+  const uint32_t u = __float_as_uint(v);
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+// v = hi + lo + r, |r| <= 2^-16 |v|
+__device__ __forceinline__ void mc_split(float v, uint32_t &hi, uint32_t &lo) {
+  hi = mc_bf16_bits(v);
+  lo = mc_bf16_bits(v - __uint_as_float(hi << 16)); // the difference is exact
+}
+
+constexpr float kMcEps = 1.0f / 16384.0f; // 2^-14
+
+// fl(|y|^2) (1 - eps) rounded towards -inf, or +inf for a norm that is not a
+// moderate finite number (the filter is then switched off for the query).
+__device__ __forceinline__ float mc_damped_norm(float ysq) {
+  if (!(ysq <= kFilterNormLimit))
+    return __builtin_inff();
+  const double c = (double)ysq * (1.0 - (double)kMcEps);
+  float f = (float)c;
+  if ((double)f > c)
+    f = __uint_as_float(__float_as_uint(f) - 1u); // f > c >= 0
+  return f;
+}
+
+// An upper bound of thresh (1 + eps) - ysq_damped + 2e-21 in three float
+// operations: the fused multiply-add is within half an ulp of the exact
+// value, the second one adds four ulps.  (2e-21: 48 accumulated terms, each
+// off by at most 2^-126 * 2e15 when the matrix cores flush an operand.)
+__device__ __forceinline__ float mc_filter_cut(float thresh,
+                                               float ysq_damped) {
+  if (ysq_damped == __builtin_inff())
+    return __builtin_inff(); // examine everything exactly
+  const float r = __builtin_fmaf(thresh, 1.0f + kMcEps, -ysq_damped);
+  return __builtin_fmaf(__builtin_fabsf(r), 2.384185791015625e-07f, r) +
+         2e-21f;
+}
+
+// The packed operand of one x row: per matrix instruction four hi parts and
+// four lo parts (bf16) of the augmented row (x_0 .. x_{d-1}, w, 0 ...).
+template <int DIM>
+__device__ __forceinline__ void mc_pack_row(const float (&x)[DIM],
+                                            uint4 (&out)[McShape<DIM>::NI]) {
+  constexpr int NI = McShape<DIM>::NI;
+  float s = x[0] * x[0];
+#pragma unroll
+  for (int c = 1; c < DIM; ++c)
+    s = __builtin_fmaf(x[c], x[c], s);
+  const bool moderate = s <= kFilterNormLimit;
+  // a row whose norm is not a moderate finite number always passes the
+  // filter and is judged by its exact distance alone
+  const float w = moderate ? s * (1.0f - kMcEps) : -1e38f;
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    uint32_t hi[4], lo[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int c = 4 * i + e;
+      hi[e] = 0;
+      lo[e] = 0;
+      if (c < DIM) {
+        if (moderate)
+          mc_split(x[c], hi[e], lo[e]);
+      } else if (c == DIM) {
+        if (moderate)
+          mc_split(w, hi[e], lo[e]);
+        else
+          hi[e] = __float_as_uint(w) >> 16;
+      }
+    }
+    out[i] = make_uint4(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16),
+                        lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16));
+  }
+}
+
+// Packs every x row once per call; the search kernel's workgroups, each of
+// which streams its whole segment through LDS, then just copy.
+template <int DIM>
+__global__ __launch_bounds__(kBlock) void mc_pack_rows_kernel(
+    const float *__restrict__ x, int n, int d_in, uint4 *__restrict__ out) {
+  constexpr int NI = McShape<DIM>::NI;
+  const int row = blockIdx.x * kBlock + threadIdx.x;
+  if (row >= n)
+    return;
+  float v[DIM];
+#pragma unroll
+  for (int c = 0; c < DIM; ++c)
+    v[c] = c < d_in ? x[(size_t)row * d_in + c] : 0.0f;
+  uint4 packed[NI];
+  mc_pack_row<DIM>(v, packed);
+#pragma unroll
+  for (int i = 0; i < NI; ++i)
+    out[(size_t)row * NI + i] = packed[i];
+}
+
+template <int DIM, int K>
+__global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
+  constexpr int NI = McShape<DIM>::NI;
+  constexpr int XF = McShape<DIM>::XF;
+  constexpr int TX = McShape<DIM>::TX;
+  constexpr int TQ = kMcQueries;
+  constexpr int QCAP = kMcQueueCap;
+  constexpr int PT = TX / kBlock; // rows staged per thread
+
+  // per row and matrix instruction: four hi parts, four lo parts (bf16)
+  __shared__ __attribute__((aligned(16))) uint4 xa[TX][NI];
+  __shared__ __attribute__((aligned(16))) float xf[TX][XF];
+  __shared__ uint16_t queue[QCAP][kBlock];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int half = lane >> 5;
+  const int col = lane & 31;
+
+  const int total_tiles = p.work_start[p.num_segments];
+  if (total_tiles == 0)
+    return;
+  const int chunk = blockIdx.x / total_tiles;
+  const int tile = blockIdx.x - chunk * total_tiles;
+  if (chunk >= p.num_chunks)
+    return;
+  const int seg = find_segment(p.work_start, p.num_segments, tile);
+  const int x_begin = p.ptr_x ? (int)p.ptr_x[seg] : 0;
+  const int x_end = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
+  const int y_begin = p.ptr_y ? (int)p.ptr_y[seg] : 0;
+  const int y_end = p.ptr_y ? (int)p.ptr_y[seg + 1] : p.m;
+  const int q = y_begin + (tile - p.work_start[seg]) * TQ + wave * 32 + col;
+  const bool valid = q < y_end;
+  const int d_in = p.d_in;
+  const int k = p.k;
+
+  const int seg_len = x_end - x_begin;
+  const int chunk_len =
+      ((seg_len + p.num_chunks - 1) / p.num_chunks + TX - 1) / TX * TX;
+  // rows are addressed as c_begin + position * stride, position < c_count
+  const int stride = p.sample_rows > 0 ? max(1, seg_len / p.sample_rows) : 1;
+  const int c_begin =
+      p.sample_rows > 0 ? x_begin : min(x_end, x_begin + chunk * chunk_len);
+  const int c_count = p.sample_rows > 0
+                          ? (seg_len + stride - 1) / stride
+                          : min(x_end, c_begin + chunk_len) - c_begin;
+  const int num_tiles = (c_count + TX - 1) / TX;
+
+
+  // ---- per-lane query state ---------------------------------------------
+  float yq[DIM];
+#pragma unroll
+  for (int c = 0; c < DIM; ++c)
+    yq[c] = (valid && c < d_in) ? p.y[(size_t)q * d_in + c] : 0.0f;
+  float ysq = yq[0] * yq[0];
+#pragma unroll
+  for (int c = 1; c < DIM; ++c)
+    ysq = __builtin_fmaf(yq[c], yq[c], ysq);
+  const bool y_moderate = ysq <= kFilterNormLimit;
+  // B operands: the hi (lanes 0-31) or lo (lanes 32-63) parts of
+  // (-2 y, 1, 0 ...), four components per instruction, given twice (against
+  // the hi and the lo parts of the row)
+  mc_bf16x8_t yb[NI];
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    uint32_t part[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int c = 4 * i + e;
+      float v = 0.0f;
+      if (c < DIM)
+        v = y_moderate ? -2.0f * yq[c] : 0.0f;
+      else if (c == DIM)
+        v = 1.0f;
+      uint32_t hi, lo;
+      mc_split(v, hi, lo);
+      part[e] = half ? lo : hi;
+    }
+    const uint32_t w0 = part[0] | (part[1] << 16);
+    const uint32_t w1 = part[2] | (part[3] << 16);
+    const uint4 packed = make_uint4(w0, w1, w0, w1);
+    yb[i] = __builtin_bit_cast(mc_bf16x8_t, packed);
+  }
+
+  double best[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j)
+    best[j] = (j < K - k) ? lowest_key() : empty_key();
+  // exact distances must be strictly below thresh; a lane without a query
+  // accepts nothing
+  const float ysq_damped = mc_damped_norm(ysq);
+  float thresh = valid ? kKnnSentinel : -__builtin_inff();
+  float cut = valid ? mc_filter_cut(thresh, ysq_damped) : -__builtin_inff();
+  float shared = kKnnSentinel; // bound inherited from other slices / partner
+  float posted = kKnnSentinel;
+  int qcount = 0;
+
+  auto set_thresh = [&](float v) {
+    if (valid) {
+      thresh = v;
+      cut = mc_filter_cut(v, ysq_damped);
+    }
+  };
+
+  // ---- tile staging -------------------------------------------------------
+  float stage[PT][DIM];
+  uint4 stage_op[PT][NI];
+  // the operand of a padding row: w = NaN (hi part of component DIM), never
+  // passes a compare
+  auto pad_op = [](int i) {
+    uint4 o = make_uint4(0u, 0u, 0u, 0u);
+    if (i == DIM / 4) {
+      const uint32_t nan_bits = 0x7fc0u << (16 * (DIM % 2));
+      if (DIM % 4 < 2)
+        o.x = nan_bits;
+      else
+        o.y = nan_bits;
+    }
+    return o;
+  };
+
+  auto load_tile = [&](int t) {
+#pragma unroll
+    for (int r = 0; r < PT; ++r) {
+      const int pos = t * TX + r * kBlock + tid;
+      const size_t g = (size_t)c_begin + (size_t)pos * stride;
+      const bool ok = pos < c_count;
+#pragma unroll
+      for (int c = 0; c < DIM; ++c)
+        stage[r][c] = (ok && c < d_in) ? p.x[g * d_in + c] : 0.0f;
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        stage_op[r][i] = ok ? p.x_split[g * NI + i] : pad_op(i);
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int r = 0; r < PT; ++r) {
+      const int pos = r * kBlock + tid;
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        xa[pos][i] = stage_op[r][i];
+#pragma unroll
+      for (int e = 0; e < XF; e += 4) {
+        float v[4];
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+          v[f] = (e + f < DIM) ? stage[r][e + f] : 0.0f;
+        *reinterpret_cast<float4 *>(&xf[pos][e]) =
+            make_float4(v[0], v[1], v[2], v[3]);
+      }
+    }
+  };
+
+  auto sync_bounds = [&]() {
+    if (valid) {
+      const float own = key_dist(best[K - 1]);
+      const float seen = __hip_atomic_load(&p.tau[q], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+      if (own < seen && own < posted) {
+        // squared distances are non-negative: floats order like their bits
+        __hip_atomic_fetch_min(reinterpret_cast<int *>(&p.tau[q]),
+                               (int)__float_as_uint(own), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        posted = own;
+      } else if (seen < posted) {
+        posted = seen;
+        // another list's k-th distance: equality must still pass
+        shared = __builtin_fminf(shared, next_up_positive(seen));
+        set_thresh(__builtin_fminf(thresh, shared));
+      }
+    }
+  };
+
+  // Resolves the parked candidates: all 64 lanes take the exact distance of
+  // their s-th parked row from the tile in LDS together.
+  auto drain = [&](int g_base, int rows) {
+    bool changed = false; // wave-uniform
+    for (int s = 0; s < QCAP; ++s) {
+      const bool has = s < qcount;
+      if (!__any(has))
+        break;
+      const int j = has ? (int)queue[s][tid] : 0;
+      float row[XF];
+#pragma unroll
+      for (int e = 0; e < XF; e += 4) {
+        const float4 v = *reinterpret_cast<const float4 *>(&xf[j][e]);
+        row[e] = v.x;
+        row[e + 1] = v.y;
+        row[e + 2] = v.z;
+        row[e + 3] = v.w;
+      }
+      const float d0 = row[0] - yq[0];
+      float d = d0 * d0;
+#pragma unroll
+      for (int c = 1; c < DIM; ++c) {
+        const float dc = row[c] - yq[c];
+        d = __builtin_fmaf(dc, dc, d);
+      }
+      // (j < rows: a padding row is never a candidate, whatever the filter
+      // made of it)
+      const bool ok = has && j < rows && d < thresh;
+      if (!__any(ok))
+        continue;
+      const double key =
+          ok ? make_key(d, (uint32_t)(g_base + j)) : empty_key();
+      sorted_insert<K>(best, key);
+      set_thresh(__builtin_fminf(key_dist(best[K - 1]), shared));
+      changed = true;
+    }
+    qcount = 0;
+    if (!changed)
+      return;
+    // the partner's k-th distance bounds the query's final k-th distance too
+    // (equality admitted: its rows interleave with this lane's)
+    const float own = key_dist(best[K - 1]);
+    const auto both = __builtin_amdgcn_permlane32_swap(
+        __float_as_uint(own), __float_as_uint(own), false, false);
+    const float partner = __uint_as_float(half ? both[0] : both[1]);
+    if (valid && partner < kKnnSentinel) {
+      shared = __builtin_fminf(shared, next_up_positive(partner));
+      if (shared < thresh)
+        set_thresh(shared);
+    }
+  };
+
+  if (num_tiles > 0)
+    load_tile(0);
+
+  for (int t = 0; t < num_tiles; ++t) {
+    // one LDS buffer: the next tile waits in registers while this one is
+    // scanned (other workgroups of the CU cover the two barriers)
+    __syncthreads();
+    store_tile();
+    __syncthreads();
+    if (t + 1 < num_tiles)
+      load_tile(t + 1);
+    if (p.tau)
+      sync_bounds();
+    // (row numbers only matter outside the bound-seeding pass: stride 1)
+    const int g_base = c_begin + t * TX;
+    const int rows = min(TX, c_count - t * TX);
+    const int steps32 = (rows + 31) / 32;
+
+    for (int rt = 0; rt < steps32; ++rt) {
+      mfma_acc_t acc = {0};
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const uint4 a = xa[rt * 32 + col][i];
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            __builtin_bit_cast(mc_bf16x8_t, a), yb[i], acc, 0, 0, 0);
+      }
+
+      // accumulator v = filter value of row 8 (v / 4) + 4 half + v % 4.
+      // All 16 compares are issued back to back into scalar masks; two
+      // masks that are empty (almost all are) then cost a scalar OR and
+      // branch, with no round trip between the vector and the scalar unit.
+      uint64_t hit[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        hit[v] = __ballot(acc[v] < cut);
+      const int base = rt * 32 + 4 * half;
+#pragma unroll
+      for (int v = 0; v < 16; v += 2) {
+        if (__builtin_expect((hit[v] | hit[v + 1]) != 0, 0)) {
+          // (the empty statement keeps this a branch of its own: merged with
+          // the per-lane tests below it would become predicated blocks that
+          // every step has to walk through)
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int u = v; u < v + 2; ++u) {
+            if (acc[u] < cut) {
+              queue[qcount][tid] = (uint16_t)(base + 8 * (u / 4) + (u % 4));
+              ++qcount;
+            }
+          }
+        }
+      }
+      if (__any(qcount > QCAP - 16))
+        drain(g_base, rows);
+    }
+    // parked positions refer to this tile: resolve them before it goes away
+    drain(g_base, rows);
+  }
+
+  // ---- results ----------------------------------------------------------
+  if (p.sample_rows > 0) {
+    if (p.tau)
+      sync_bounds(); // posts the k-th best sampled distance of either half
+    return;
+  }
+  // unite the two half lists of each query: every lane inserts its partner's
+  // keys (all read before any list changes)
+  double theirs[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    const auto hi = __builtin_amdgcn_permlane32_swap(
+        (unsigned)__double2hiint(best[j]), (unsigned)__double2hiint(best[j]),
+        false, false);
+    const auto lo = __builtin_amdgcn_permlane32_swap(
+        (unsigned)__double2loint(best[j]), (unsigned)__double2loint(best[j]),
+        false, false);
+    theirs[j] = half ? __hiloint2double((int)hi[0], (int)lo[0])
+                     : __hiloint2double((int)hi[1], (int)lo[1]);
+  }
+#pragma unroll
+  for (int j = 0; j < K; ++j)
+    if (j >= K - k) // slots below are padding, not keys
+      sorted_insert<K>(best, theirs[j]);
+
+  if (half == 0) {
+    if (p.num_chunks == 1) {
+      if (valid)
+        write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+    } else {
+      // sorted keys of this slice, [item][slot][query of the tile]
+      double *dst = p.partial + (size_t)blockIdx.x * k * TQ + wave * 32 + col;
+#pragma unroll
+      for (int j = 0; j < K; ++j) {
+        const int e = j - (K - k);
+        if (e >= 0)
+          dst[(size_t)e * TQ] = best[j];
+      }
+    }
+  }
+}
+
+// One padded dimension of the dispatch table (instantiated in its own
+// translation unit so the dimensions build in parallel).
+template <int DIM>
+hipError_t launch_knn_lowd_mc_dim(const KnnLowdParams &p, int kbucket,
+                                  int grid, hipStream_t stream);
+// Fills `out` (n * McShape<DIM>::NI entries) with the packed operand rows.
+template <int DIM>
+hipError_t launch_mc_pack_rows(const float *x, int n, int d_in, uint4 *out,
+                               hipStream_t stream);
+
+#define PCA_LOWD_MC_DEFINE(DIM_)                                               \
+  template <>                                                                  \
+  hipError_t launch_mc_pack_rows<DIM_>(const float *x, int n, int d_in,        \
+                                       uint4 *out, hipStream_t stream) {       \
+    hipLaunchKernelGGL((mc_pack_rows_kernel<DIM_>),                            \
+                       dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0,       \
+                       stream, x, n, d_in, out);                               \
+    return hipGetLastError();                                                  \
+  }                                                                            \
+  template <>                                                                  \
+  hipError_t launch_knn_lowd_mc_dim<DIM_>(const KnnLowdParams &p, int kbucket, \
+                                          int grid, hipStream_t stream) {      \
+    switch (kbucket) {                                                         \
+    case 8:                                                                    \
+      hipLaunchKernelGGL((knn_lowd_mc_kernel<DIM_, 8>), dim3(grid),            \
+                         dim3(kBlock), 0, stream, p);                          \
+      break;                                                                   \
+    case 16:                                                                   \
+      hipLaunchKernelGGL((knn_lowd_mc_kernel<DIM_, 16>), dim3(grid),           \
+                         dim3(kBlock), 0, stream, p);                          \
+      break;                                                                   \
+    case 24:                                                                   \
+      hipLaunchKernelGGL((knn_lowd_mc_kernel<DIM_, 24>), dim3(grid),           \
+                         dim3(kBlock), 0, stream, p);                          \
+      break;                                                                   \
+    case 32:                                                                   \
+      hipLaunchKernelGGL((knn_lowd_mc_kernel<DIM_, 32>), dim3(grid),           \
+                         dim3(kBlock), 0, stream, p);                          \
+      break;                                                                   \
+    default:                                                                   \
+      return hipErrorInvalidValue;                                             \
+    }                                                                          \
+    return hipGetLastError();                                                  \
+  }
+
+} // namespace pca

@@ -54,15 +54,17 @@ hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
 struct KnnLowdConfig {
   int kbucket;          // compiled list width (>= k)
   int queries_per_lane; // 1 or 2
-  int tile_queries;     // kBlock * queries_per_lane
+  int tile_queries;     // queries per work item
+  bool matrix_cores;    // pre-filter on the matrix cores (knn_lowd_mc_impl)
   int num_chunks;       // slices of every segment's x rows (>= 1)
+  int sample_rows;      // rows per segment of the bound-seeding pass, 0 = none
 };
 bool knn_lowd_supported(int d, int k, bool cosine);
 KnnLowdConfig knn_lowd_config(int d, int k, int n, int m, int num_segments,
                               bool cosine);
 // Scratch the launch needs beyond the dense result (shared bounds + partial
-// key lists; 0 when the segments are not sliced).
-size_t knn_lowd_scratch_bytes(const KnnLowdConfig &cfg, int m,
+// key lists of sliced segments).
+size_t knn_lowd_scratch_bytes(const KnnLowdConfig &cfg, int n, int m, int d,
                               int num_segments, int k);
 hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
                            const KnnLowdConfig &cfg, const int *work_start,
