@@ -116,7 +116,8 @@ size_t mc_split_bytes(const KnnLowdConfig &cfg, int n, int d) {
   if (!cfg.matrix_cores)
     return 0;
   const int dim = padded_dim(d);
-  const int per_row = (dim + 1 + 3) / 4; // McShape<dim>::NI
+  // McShape<dim>::REC: operand quads + coordinate quads
+  const int per_row = (dim + 1 + 3) / 4 + (dim <= 4 ? 1 : 2);
   return align256(sizeof(uint4) * (size_t)n * per_row);
 }
 

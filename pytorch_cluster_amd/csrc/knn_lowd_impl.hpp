@@ -76,7 +76,7 @@ struct KnnLowdParams {
   int num_chunks;        // S: slices of every segment's x rows
   int sample_rows;       // > 0: bound-seeding pass over about this many
                          // evenly spaced x rows per segment (see below)
-  const uint4 *x_split;  // matrix-core kernel: packed bf16 operand rows of x
+  const uint4 *x_split;  // matrix-core kernel: packed rows of x
   float *tau;            // [m] shared pruning bounds or NULL
   double *partial;       // [S * tiles][k][tile queries] keys (S > 1) or NULL
   int *out_idx;          // dense results (written here only when S == 1)

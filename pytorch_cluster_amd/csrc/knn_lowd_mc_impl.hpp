@@ -16,8 +16,12 @@
 // accumulation slots of ONE v_mfma_f32_32x32x16_bf16 (products exact, fp32
 // accumulation): 32 candidates x 32 queries per instruction in a quarter of
 // the time the fp32 matrix instruction needs, and about a tenth of what the
-// vector ALU needs for the same 1,024 filter values.  The vector ALU is left
-// with one compare per pair.
+// vector ALU needs for the same 1,024 filter values.  Two of the sixteen
+// slots would multiply w by the zero lo part of the query's 1; they carry
+// -cut instead (see below), so that the matrix cores deliver t - cut and the
+// vector ALU only has to collect SIGN BITS: one funnel shift per pair
+// (v_alignbit_b32, full rate) where a compare into a scalar mask costs twice
+// the issue cycles.
 //
 // A candidate with t >= cut = thresh (1 + eps) - fl(|y|^2) (1 - eps) (+ a tiny
 // absolute term) can never have an exact distance below thresh, for
@@ -26,7 +30,10 @@
 // norms are within (1 +- d u) of the true ones and the exact chain within
 // (1 +- (d + 2) u) of |x - y|^2; with 2 |x||y| <= |x|^2 + |y|^2 this gives
 //     t - cut <= |x|^2 (-eps + 2^-14.3 + (d + 1) u)
-//                + |y|^2 (-eps + 2^-14.9 + d u) + thresh ((d + 3) u - eps) < 0.
+//                + |y|^2 (-eps + 2^-14.9 + d u) + thresh ((d + 3) u - eps) < 0
+// with room left for the 50 u |cut| that accumulating -cut along with the
+// products adds.  -cut itself enters as the bf16 split of
+// -(cut + 2^-15 |cut|), which is never above -cut.
 // Operands below the bf16 normal range may be flushed to zero by the matrix
 // cores: at most 2^-126 per operand, times the other factor (below 2e15 for
 // operands of moderate norm); the absolute term of the cut covers it.  Rows
@@ -46,10 +53,10 @@
 // share a query and split its candidates: each keeps its own sorted list (its
 // rows arrive in ascending order, so its own k-th distance is a strict
 // bound), the two exchange their k-th distances after every drain, and the
-// lists are united at the end.  Candidates that pass the filter are parked
-// (position in the tile) in a per-lane LDS queue and resolved by all lanes
-// together, exactly, when a queue fills up or the tile ends -- as in
-// knn_lowd_impl.hpp.  Slices, shared bounds (`tau`) and the merge of partial
+// lists are united at the end.  A lane whose 16 sign bits of a step are not
+// all clear parks (step, sign mask) in a per-lane LDS queue; the parked rows
+// are resolved by all lanes together, exactly, when a queue fills up or the
+// tile ends -- as in knn_lowd_impl.hpp.  Slices, shared bounds (`tau`) and the merge of partial
 // lists are those of knn_lowd_impl.hpp with tiles of 128 queries.
 //
 // Bound-seeding pass (sample_rows > 0): see knn_lowd_impl.hpp.
@@ -60,7 +67,7 @@
 namespace pca {
 
 constexpr int kMcQueries = 128; // queries per workgroup
-constexpr int kMcQueueCap = 32; // parked candidates per lane
+constexpr int kMcQueueCap = 8; // parked steps per lane
 
 typedef __bf16 mc_bf16x8_t __attribute__((ext_vector_type(8)));
 
@@ -68,7 +75,9 @@ template <int DIM> struct McShape {
   // matrix instructions per 32-row step: four augmented components each
   static constexpr int NI = (DIM + 1 + 3) / 4;
   static constexpr int XF = DIM <= 4 ? 4 : 8; // fp32 coordinates per row
-  static constexpr int TX = DIM <= 4 ? 512 : 256; // rows per LDS tile
+  // a packed row: NI operand quads, then the coordinates (16-byte units)
+  static constexpr int REC = NI + XF / 4;
+  static constexpr int TX = DIM <= 4 ? 1024 : 256; // rows per LDS tile
 };
 
 // bf16 nearest-even of a finite float of moderate size, as the upper half of
@@ -111,12 +120,22 @@ __device__ __forceinline__ float mc_filter_cut(float thresh,
          2e-21f;
 }
 
-// The packed operand of one x row: per matrix instruction four hi parts and
-// four lo parts (bf16) of the augmented row (x_0 .. x_{d-1}, w, 0 ...).
+// One packed x row: per matrix instruction four hi parts and four lo parts
+// (bf16) of the augmented row (x_0 .. x_{d-1}, w, 0 ...), then the fp32
+// coordinates for the exact distances.
 template <int DIM>
 __device__ __forceinline__ void mc_pack_row(const float (&x)[DIM],
-                                            uint4 (&out)[McShape<DIM>::NI]) {
+                                            uint4 (&out)[McShape<DIM>::REC]) {
   constexpr int NI = McShape<DIM>::NI;
+  constexpr int XF = McShape<DIM>::XF;
+#pragma unroll
+  for (int e = 0; e < XF; e += 4) {
+    uint32_t v[4];
+#pragma unroll
+    for (int f = 0; f < 4; ++f)
+      v[f] = (e + f < DIM) ? __float_as_uint(x[e + f]) : 0u;
+    out[NI + e / 4] = make_uint4(v[0], v[1], v[2], v[3]);
+  }
   float s = x[0] * x[0];
 #pragma unroll
   for (int c = 1; c < DIM; ++c)
@@ -153,7 +172,7 @@ __device__ __forceinline__ void mc_pack_row(const float (&x)[DIM],
 template <int DIM>
 __global__ __launch_bounds__(kBlock) void mc_pack_rows_kernel(
     const float *__restrict__ x, int n, int d_in, uint4 *__restrict__ out) {
-  constexpr int NI = McShape<DIM>::NI;
+  constexpr int REC = McShape<DIM>::REC;
   const int row = blockIdx.x * kBlock + threadIdx.x;
   if (row >= n)
     return;
@@ -161,11 +180,11 @@ __global__ __launch_bounds__(kBlock) void mc_pack_rows_kernel(
 #pragma unroll
   for (int c = 0; c < DIM; ++c)
     v[c] = c < d_in ? x[(size_t)row * d_in + c] : 0.0f;
-  uint4 packed[NI];
+  uint4 packed[REC];
   mc_pack_row<DIM>(v, packed);
 #pragma unroll
-  for (int i = 0; i < NI; ++i)
-    out[(size_t)row * NI + i] = packed[i];
+  for (int i = 0; i < REC; ++i)
+    out[(size_t)row * REC + i] = packed[i];
 }
 
 template <int DIM, int K>
@@ -177,10 +196,11 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
   constexpr int QCAP = kMcQueueCap;
   constexpr int PT = TX / kBlock; // rows staged per thread
 
-  // per row and matrix instruction: four hi parts, four lo parts (bf16)
-  __shared__ __attribute__((aligned(16))) uint4 xa[TX][NI];
-  __shared__ __attribute__((aligned(16))) float xf[TX][XF];
-  __shared__ uint16_t queue[QCAP][kBlock];
+  constexpr int REC = McShape<DIM>::REC;
+  // packed rows as mc_pack_row leaves them
+  __shared__ __attribute__((aligned(16))) uint4 rows_lds[TX][REC];
+  // parked steps: (step << 16) | mask of the lane's 16 rows that passed
+  __shared__ uint32_t queue[QCAP][kBlock];
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -238,11 +258,13 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int c = 4 * i + e;
+      // (a lane without a query multiplies everything by zero and starts
+      // from a large positive value: nothing passes)
       float v = 0.0f;
       if (c < DIM)
-        v = y_moderate ? -2.0f * yq[c] : 0.0f;
+        v = (valid && y_moderate) ? -2.0f * yq[c] : 0.0f;
       else if (c == DIM)
-        v = 1.0f;
+        v = valid ? 1.0f : 0.0f;
       uint32_t hi, lo;
       mc_split(v, hi, lo);
       part[e] = half ? lo : hi;
@@ -261,10 +283,51 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
   // accepts nothing
   const float ysq_damped = mc_damped_norm(ysq);
   float thresh = valid ? kKnnSentinel : -__builtin_inff();
-  float cut = valid ? mc_filter_cut(thresh, ysq_damped) : -__builtin_inff();
+  float cut = valid ? mc_filter_cut(thresh, ysq_damped) : -1e38f;
   float shared = kKnnSentinel; // bound inherited from other slices / partner
   float posted = kKnnSentinel;
-  int qcount = 0;
+  // The filter tests the SIGN of t - cut: -cut rides along in the two
+  // accumulation slots that would otherwise multiply w by the (zero) lo part
+  // of the query's 1.  On the row side the upper lanes put 1 where they hold
+  // w_hi and w_lo (two operations per step, see the scan loop); on the query
+  // side they carry the hi and lo parts of -cut', cut' = cut + 2^-15 |cut|
+  // (so that the 2^-16 |cut'| the split may lose never lowers the cut).  An
+  // infinite cut (filter switched off) enters as the largest finite bf16.
+  constexpr int WI = DIM / 4;  // matrix instruction that holds component DIM
+  constexpr int WE = DIM % 4;  // ... as its WE-th component
+  const uint32_t one_keep =
+      half ? ~(0xffffu << (16 * (WE & 1))) : 0xffffffffu;
+  const uint32_t one_bits = half ? (0x3f80u << (16 * (WE & 1))) : 0u;
+  const uint4 yb_plain = __builtin_bit_cast(uint4, yb[WI]);
+  auto refresh_cut = [&]() {
+    if (half) {
+      float neg = -__builtin_fmaf(__builtin_fabsf(cut), 3.0517578125e-05f, cut);
+      uint32_t hi, lo;
+      if (__builtin_fabsf(neg) < 1e38f) {
+        mc_split(neg, hi, lo);
+      } else {
+        hi = neg < 0.0f ? 0xff7fu : 0x7f7fu;
+        lo = 0;
+      }
+      uint4 b = yb_plain;
+      const uint32_t keep = ~(0xffffu << (16 * (WE & 1)));
+      const uint32_t sh = 16 * (WE & 1);
+      if (WE < 2) {
+        b.x = (b.x & keep) | (hi << sh);
+        b.z = (b.z & keep) | (lo << sh);
+      } else {
+        b.y = (b.y & keep) | (hi << sh);
+        b.w = (b.w & keep) | (lo << sh);
+      }
+      yb[WI] = __builtin_bit_cast(mc_bf16x8_t, b);
+    }
+  };
+  refresh_cut();
+  // parked steps of this lane: queue[0 .. qcount)[tid]; qnext is the byte
+  // offset in `queue` at which the next one goes
+  constexpr int QROW = kBlock * (int)sizeof(uint32_t);
+  const int qfirst = tid * (int)sizeof(uint32_t);
+  int qnext = qfirst;
 
   auto set_thresh = [&](float v) {
     if (valid) {
@@ -274,11 +337,9 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
   };
 
   // ---- tile staging -------------------------------------------------------
-  float stage[PT][DIM];
-  uint4 stage_op[PT][NI];
-  // the operand of a padding row: w = NaN (hi part of component DIM), never
-  // passes a compare
-  auto pad_op = [](int i) {
+  uint4 stage[PT][REC];
+  // a padding row: w = NaN (hi part of component DIM), never passes a compare
+  auto pad_quad = [](int i) {
     uint4 o = make_uint4(0u, 0u, 0u, 0u);
     if (i == DIM / 4) {
       const uint32_t nan_bits = 0x7fc0u << (16 * (DIM % 2));
@@ -297,30 +358,16 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
       const size_t g = (size_t)c_begin + (size_t)pos * stride;
       const bool ok = pos < c_count;
 #pragma unroll
-      for (int c = 0; c < DIM; ++c)
-        stage[r][c] = (ok && c < d_in) ? p.x[g * d_in + c] : 0.0f;
-#pragma unroll
-      for (int i = 0; i < NI; ++i)
-        stage_op[r][i] = ok ? p.x_split[g * NI + i] : pad_op(i);
+      for (int i = 0; i < REC; ++i)
+        stage[r][i] = ok ? p.x_split[g * REC + i] : pad_quad(i);
     }
   };
   auto store_tile = [&]() {
 #pragma unroll
-    for (int r = 0; r < PT; ++r) {
-      const int pos = r * kBlock + tid;
+    for (int r = 0; r < PT; ++r)
 #pragma unroll
-      for (int i = 0; i < NI; ++i)
-        xa[pos][i] = stage_op[r][i];
-#pragma unroll
-      for (int e = 0; e < XF; e += 4) {
-        float v[4];
-#pragma unroll
-        for (int f = 0; f < 4; ++f)
-          v[f] = (e + f < DIM) ? stage[r][e + f] : 0.0f;
-        *reinterpret_cast<float4 *>(&xf[pos][e]) =
-            make_float4(v[0], v[1], v[2], v[3]);
-      }
-    }
+      for (int i = 0; i < REC; ++i)
+        rows_lds[r * kBlock + tid][i] = stage[r][i];
   };
 
   auto sync_bounds = [&]() {
@@ -341,25 +388,43 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
         set_thresh(__builtin_fminf(thresh, shared));
       }
     }
+    refresh_cut();
   };
 
-  // Resolves the parked candidates: all 64 lanes take the exact distance of
-  // their s-th parked row from the tile in LDS together.
+  // Resolves the parked candidates: in every round each lane takes the next
+  // row of its parked steps (steps in the order they were parked, rows in
+  // ascending order) and all 64 lanes evaluate their exact distances from the
+  // tile in LDS together.
   auto drain = [&](int g_base, int rows) {
     bool changed = false; // wave-uniform
-    for (int s = 0; s < QCAP; ++s) {
-      const bool has = s < qcount;
+    const int qcount = (qnext - qfirst) / QROW;
+    int taken = 0;         // parked steps this lane has started on
+    uint32_t pending = 0;  // rows of the current step still to look at
+    int step_base = 0;     // first of this lane's rows in that step
+    for (;;) {
+      if (pending == 0 && taken < qcount) {
+        const uint32_t word = queue[taken][tid];
+        ++taken;
+        pending = word & 0xffffu;
+        step_base = (int)(word >> 16) * 32 + 4 * half;
+      }
+      const bool has = pending != 0;
       if (!__any(has))
         break;
-      const int j = has ? (int)queue[s][tid] : 0;
+      // bit 15 - v of the mask stands for accumulator v = row
+      // 8 (v / 4) + v % 4 of the lane's rows: highest bit first
+      const int bit = 31 - __builtin_clz(has ? pending : 1u);
+      const int v = 15 - bit;
+      pending &= ~(1u << bit);
+      const int j = has ? step_base + 2 * (v & 12) + (v & 3) : 0;
       float row[XF];
 #pragma unroll
       for (int e = 0; e < XF; e += 4) {
-        const float4 v = *reinterpret_cast<const float4 *>(&xf[j][e]);
-        row[e] = v.x;
-        row[e + 1] = v.y;
-        row[e + 2] = v.z;
-        row[e + 3] = v.w;
+        const uint4 q4 = rows_lds[j][NI + e / 4];
+        row[e] = __uint_as_float(q4.x);
+        row[e + 1] = __uint_as_float(q4.y);
+        row[e + 2] = __uint_as_float(q4.z);
+        row[e + 3] = __uint_as_float(q4.w);
       }
       const float d0 = row[0] - yq[0];
       float d = d0 * d0;
@@ -379,7 +444,7 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
       set_thresh(__builtin_fminf(key_dist(best[K - 1]), shared));
       changed = true;
     }
-    qcount = 0;
+    qnext = qfirst;
     if (!changed)
       return;
     // the partner's k-th distance bounds the query's final k-th distance too
@@ -393,6 +458,7 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
       if (shared < thresh)
         set_thresh(shared);
     }
+    refresh_cut();
   };
 
   if (num_tiles > 0)
@@ -413,42 +479,52 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
     const int rows = min(TX, c_count - t * TX);
     const int steps32 = (rows + 31) / 32;
 
+    uint4 a_next[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+      a_next[i] = rows_lds[col][i];
     for (int rt = 0; rt < steps32; ++rt) {
       mfma_acc_t acc = {0};
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
-        const uint4 a = xa[rt * 32 + col][i];
+        uint4 a = a_next[i];
+        if (i == WI) {
+          // upper lanes: 1 in place of w_hi and w_lo (times -cut' parts)
+          if (WE < 2) {
+            a.x = (a.x & one_keep) | one_bits;
+            a.z = (a.z & one_keep) | one_bits;
+          } else {
+            a.y = (a.y & one_keep) | one_bits;
+            a.w = (a.w & one_keep) | one_bits;
+          }
+        }
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
             __builtin_bit_cast(mc_bf16x8_t, a), yb[i], acc, 0, 0, 0);
       }
+      // the next step's rows are on their way while this step is filtered
+      // (the last read stays inside the tile)
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        a_next[i] = rows_lds[min(rt + 1, TX / 32 - 1) * 32 + col][i];
 
-      // accumulator v = filter value of row 8 (v / 4) + 4 half + v % 4.
-      // All 16 compares are issued back to back into scalar masks; two
-      // masks that are empty (almost all are) then cost a scalar OR and
-      // branch, with no round trip between the vector and the scalar unit.
-      uint64_t hit[16];
+      // accumulator v = t - cut of row 8 (v / 4) + 4 half + v % 4: its sign
+      // bit says "look at this row".  One funnel shift per accumulator
+      // gathers the 16 signs of a lane (bit 15 - v); compares into scalar
+      // masks would cost twice as many issue cycles each.
+      uint32_t mask = 0;
 #pragma unroll
       for (int v = 0; v < 16; ++v)
-        hit[v] = __ballot(acc[v] < cut);
-      const int base = rt * 32 + 4 * half;
-#pragma unroll
-      for (int v = 0; v < 16; v += 2) {
-        if (__builtin_expect((hit[v] | hit[v + 1]) != 0, 0)) {
-          // (the empty statement keeps this a branch of its own: merged with
-          // the per-lane tests below it would become predicated blocks that
-          // every step has to walk through)
-          asm volatile("" ::: "memory");
-#pragma unroll
-          for (int u = v; u < v + 2; ++u) {
-            if (acc[u] < cut) {
-              queue[qcount][tid] = (uint16_t)(base + 8 * (u / 4) + (u % 4));
-              ++qcount;
-            }
-          }
+        mask = __builtin_amdgcn_alignbit(mask, __float_as_uint(acc[v]), 31);
+      if (__any(mask != 0)) {
+        if (mask != 0) {
+          *reinterpret_cast<uint32_t *>(
+              reinterpret_cast<char *>(&queue[0][0]) + qnext) =
+              ((uint32_t)rt << 16) | mask;
+          qnext += QROW;
         }
+        if (__any(qnext >= qfirst + QCAP * QROW))
+          drain(g_base, rows);
       }
-      if (__any(qcount > QCAP - 16))
-        drain(g_base, rows);
     }
     // parked positions refer to this tile: resolve them before it goes away
     drain(g_base, rows);
@@ -501,7 +577,7 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
 template <int DIM>
 hipError_t launch_knn_lowd_mc_dim(const KnnLowdParams &p, int kbucket,
                                   int grid, hipStream_t stream);
-// Fills `out` (n * McShape<DIM>::NI entries) with the packed operand rows.
+// Fills `out` (n * McShape<DIM>::REC entries) with the packed rows.
 template <int DIM>
 hipError_t launch_mc_pack_rows(const float *x, int n, int d_in, uint4 *out,
                                hipStream_t stream);
