@@ -93,21 +93,16 @@ KnnLowdConfig knn_lowd_config(int /*d*/, int k, int n, int m,
   // ragged segments, but slices of at least ~4 LDS tiles on average -- every
   // slice pays the start-up phase of its candidate lists again.
   const int tiles = plan_upper_bound(m, num_segments, cfg.tile_queries);
-  const int want = (8192 + tiles - 1) / tiles;
+  // (about 6,000 items measure best for the matrix-core kernel, whose
+  // workgroups hold half as many queries)
+  const int target = cfg.matrix_cores ? 6144 : 8192;
+  const int want = (target + tiles - 1) / tiles;
   const int by_length = (n / num_segments) / (4 * kLowdTileX);
   int chunks = std::max(1, std::min(std::min(want, 16), by_length));
   const int forced_chunks = env_int("PCA_KNN_SLICES", 0);
   if (forced_chunks >= 1 && forced_chunks <= 64)
     chunks = forced_chunks;
   cfg.num_chunks = chunks;
-
-  // Bound-seeding pass: worth its ~sample/segment share of the scan once the
-  // segments are much longer than the sample.
-  cfg.sample_rows = 0;
-  const int sample = env_int("PCA_KNN_SAMPLE", 2048);
-  if (sample > 0 && !cosine && (n / num_segments) >= 16 * sample &&
-      sample >= 4 * k)
-    cfg.sample_rows = sample;
   return cfg;
 }
 
@@ -190,7 +185,6 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
   p.out_idx = out.idx;
   p.out_dist = out.dist;
   p.out_count = out.count;
-  p.sample_rows = 0;
   p.x_split = nullptr;
   char *base = static_cast<char *>(scratch);
   const size_t tau_bytes = align256(sizeof(float) * (size_t)in.m);
@@ -216,32 +210,20 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
     if (perr != hipSuccess)
       return perr;
   }
-  if (cfg.num_chunks > 1 || cfg.sample_rows > 0) {
+  if (cfg.num_chunks > 1) {
     float *tau = reinterpret_cast<float *>(base);
-    if (cfg.num_chunks > 1)
-      p.partial =
-          reinterpret_cast<double *>(base + tau_bytes + split_bytes);
+    p.partial = reinterpret_cast<double *>(base + tau_bytes + split_bytes);
     p.tau = tau;
     hipLaunchKernelGGL(fill_f32_kernel, dim3((in.m + kBlock - 1) / kBlock),
                        dim3(kBlock), 0, stream, tau, in.m, kKnnSentinel);
   }
 
-  hipError_t err = hipErrorInvalidValue;
-  for (int pass = cfg.sample_rows > 0 ? 0 : 1; pass < 2; ++pass) {
-    // pass 0 seeds the bounds from a sample of each segment, pass 1 is the
-    // search itself (the one the timing events bracket)
-    KnnLowdParams q = p;
-    if (pass == 0) {
-      q.sample_rows = cfg.sample_rows;
-      q.num_chunks = 1;
-    } else if (time_start) {
-      (void)hipEventRecord(time_start, stream);
-    }
-    err = launch_lowd_pass(q, cfg, padded_dim(in.d), cosine, tiles_bound,
-                           stream);
-    if (err != hipSuccess)
-      return err;
-  }
+  if (time_start)
+    (void)hipEventRecord(time_start, stream);
+  const hipError_t err = launch_lowd_pass(p, cfg, padded_dim(in.d), cosine,
+                                          tiles_bound, stream);
+  if (err != hipSuccess)
+    return err;
   if (time_stop)
     (void)hipEventRecord(time_stop, stream);
   if (cfg.num_chunks <= 1)

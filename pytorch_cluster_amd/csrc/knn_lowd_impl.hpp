@@ -41,15 +41,6 @@
 //     the merge), the slice's own k-th distance is a strict bound because all
 //     later candidates of the slice have higher rows.
 //
-// Bound-seeding pass (sample_rows > 0): the same kernel scans only every
-// stride-th x row of each segment (about sample_rows of them), keeps no
-// results and posts each query's k-th best sampled distance to `tau`.  The
-// k-th distance within any subset of the candidates bounds the final k-th
-// distance from above, so the full scan that follows starts with lists that
-// reject all but roughly k * stride candidates per query -- whatever order
-// the rows come in (a scan that approaches a query's neighbourhood gradually
-// would otherwise accept, and sort in, almost every candidate on the way).
-//
 // Results per query: rows [K-k, K) of the list = the k best (distance, row)
 // pairs in ascending order; slots never filled keep row -1 (segment smaller
 // than k, or candidates at distance >= 1e10 / NaN, which the reference never
@@ -74,8 +65,6 @@ struct KnnLowdParams {
   int n, m, d_in, num_segments, k;
   const int *work_start; // [num_segments + 1] first query tile of each segment
   int num_chunks;        // S: slices of every segment's x rows
-  int sample_rows;       // > 0: bound-seeding pass over about this many
-                         // evenly spaced x rows per segment (see below)
   const uint4 *x_split;  // matrix-core kernel: packed rows of x
   float *tau;            // [m] shared pruning bounds or NULL
   double *partial;       // [S * tiles][k][tile queries] keys (S > 1) or NULL
@@ -206,13 +195,8 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
   const int seg_len = x_end - x_begin;
   const int chunk_len =
       ((seg_len + p.num_chunks - 1) / p.num_chunks + TX - 1) / TX * TX;
-  // rows are addressed as c_begin + position * stride, position < c_count
-  const int stride = p.sample_rows > 0 ? max(1, seg_len / p.sample_rows) : 1;
-  const int c_begin =
-      p.sample_rows > 0 ? x_begin : min(x_end, x_begin + chunk * chunk_len);
-  const int c_count = p.sample_rows > 0
-                          ? (seg_len + stride - 1) / stride
-                          : min(x_end, c_begin + chunk_len) - c_begin;
+  const int c_begin = min(x_end, x_begin + chunk * chunk_len);
+  const int c_count = min(x_end, c_begin + chunk_len) - c_begin;
   const int num_tiles = (c_count + TX - 1) / TX;
 
   // ---- per-lane query state -------------------------------------------
@@ -267,7 +251,7 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
 #pragma unroll
     for (int r = 0; r < PT; ++r) {
       const int pos = t * TX + r * kBlock + tid;
-      const size_t g = (size_t)c_begin + (size_t)pos * stride;
+      const size_t g = (size_t)c_begin + pos;
 #pragma unroll
       for (int c = 0; c < DIM; ++c) {
         // rows past the slice end become +inf: their distance is inf or
@@ -386,7 +370,6 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
     if (p.tau)
       sync_bounds();
 
-    // (row numbers only matter outside the bound-seeding pass: stride 1)
     const int g_base = c_begin + t * TX;
     // whole pairs of groups; rows between the slice end and the tile end are
     // +inf padding
@@ -487,10 +470,6 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
   }
 
   // ---- results --------------------------------------------------------
-  if (p.sample_rows > 0) {
-    sync_bounds(); // posts the k-th best sampled distance
-    return;
-  }
   if (p.num_chunks == 1) {
 #pragma unroll
     for (int qi = 0; qi < QPT; ++qi)

@@ -58,8 +58,6 @@
 // are resolved by all lanes together, exactly, when a queue fills up or the
 // tile ends -- as in knn_lowd_impl.hpp.  Slices, shared bounds (`tau`) and the merge of partial
 // lists are those of knn_lowd_impl.hpp with tiles of 128 queries.
-//
-// Bound-seeding pass (sample_rows > 0): see knn_lowd_impl.hpp.
 #pragma once
 
 #include "knn_mfma_impl.hpp"
@@ -228,13 +226,8 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
   const int seg_len = x_end - x_begin;
   const int chunk_len =
       ((seg_len + p.num_chunks - 1) / p.num_chunks + TX - 1) / TX * TX;
-  // rows are addressed as c_begin + position * stride, position < c_count
-  const int stride = p.sample_rows > 0 ? max(1, seg_len / p.sample_rows) : 1;
-  const int c_begin =
-      p.sample_rows > 0 ? x_begin : min(x_end, x_begin + chunk * chunk_len);
-  const int c_count = p.sample_rows > 0
-                          ? (seg_len + stride - 1) / stride
-                          : min(x_end, c_begin + chunk_len) - c_begin;
+  const int c_begin = min(x_end, x_begin + chunk * chunk_len);
+  const int c_count = min(x_end, c_begin + chunk_len) - c_begin;
   const int num_tiles = (c_count + TX - 1) / TX;
 
 
@@ -355,7 +348,7 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
 #pragma unroll
     for (int r = 0; r < PT; ++r) {
       const int pos = t * TX + r * kBlock + tid;
-      const size_t g = (size_t)c_begin + (size_t)pos * stride;
+      const size_t g = (size_t)c_begin + pos;
       const bool ok = pos < c_count;
 #pragma unroll
       for (int i = 0; i < REC; ++i)
@@ -474,7 +467,6 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
       load_tile(t + 1);
     if (p.tau)
       sync_bounds();
-    // (row numbers only matter outside the bound-seeding pass: stride 1)
     const int g_base = c_begin + t * TX;
     const int rows = min(TX, c_count - t * TX);
     const int steps32 = (rows + 31) / 32;
@@ -531,11 +523,6 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
   }
 
   // ---- results ----------------------------------------------------------
-  if (p.sample_rows > 0) {
-    if (p.tau)
-      sync_bounds(); // posts the k-th best sampled distance of either half
-    return;
-  }
   // unite the two half lists of each query: every lane inserts its partner's
   // keys (all read before any list changes)
   double theirs[K];

@@ -168,7 +168,6 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   mp.k = k;
   mp.work_start = work_start;
   mp.num_chunks = chunks;
-  mp.sample_rows = 0;
   mp.tau = nullptr;
   mp.partial = partial;
   mp.out_idx = out.idx;

@@ -57,7 +57,6 @@ struct KnnLowdConfig {
   int tile_queries;     // queries per work item
   bool matrix_cores;    // pre-filter on the matrix cores (knn_lowd_mc_impl)
   int num_chunks;       // slices of every segment's x rows (>= 1)
-  int sample_rows;      // rows per segment of the bound-seeding pass, 0 = none
 };
 bool knn_lowd_supported(int d, int k, bool cosine);
 KnnLowdConfig knn_lowd_config(int d, int k, int n, int m, int num_segments,
