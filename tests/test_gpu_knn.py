@@ -234,6 +234,60 @@ def test_prefilter_never_drops_a_neighbour(oracle, d, k, case):
     assert (gd == wd).all()
 
 
+@pytest.mark.parametrize("d,k", [(2, 8), (3, 16), (4, 24), (7, 32)])
+@pytest.mark.parametrize("case", ["full_mantissa", "binade_edges",
+                                  "norm_limit", "non_finite", "tiny_segments"])
+def test_split_bf16_filter_edge_cases(oracle, d, k, case):
+    # the matrix-core pre-filter works on bf16 hi/lo splits of the operands:
+    # values that round up across a power of two, rows around the norm above
+    # which the filter is switched off, non-finite rows and queries mixed in,
+    # and segments much shorter than a 32-row step
+    rng = np.random.default_rng(hash((d, k, case, "bf16")) % (2 ** 32))
+    n, m = 6000, 700
+    ptr_x = np.array([0, 2500, 6000])
+    ptr_y = np.array([0, 300, 700])
+    if case == "full_mantissa":
+        # every mantissa bit set, random exponents: the worst case of the
+        # split's rounding
+        bits = (rng.integers(100, 140, (n + m, d)).astype(np.uint32) << 23) \
+            | 0x7fffff | (rng.integers(0, 2, (n + m, d)).astype(np.uint32) << 31)
+        v = bits.view(np.float32)
+        x, y = v[:n], v[n:]
+    elif case == "binade_edges":
+        base = 2.0 ** rng.integers(-3, 8, (n + m, d))
+        v = base * (1.0 - rng.integers(0, 4, (n + m, d)) * 2.0 ** -24)
+        v = v * rng.choice([-1.0, 1.0], (n + m, d))
+        x, y = v[:n], v[n:]
+    elif case == "norm_limit":
+        # squared norms on both sides of 1e30
+        scale = 10.0 ** rng.uniform(14.5, 15.5, (n + m, 1))
+        v = scale * rng.standard_normal((n + m, d))
+        x, y = v[:n], v[n:]
+        y[:40] = x[:40]
+    elif case == "non_finite":
+        x = rng.standard_normal((n, d))
+        y = rng.standard_normal((m, d))
+        for arr, cnt in ((x, 300), (y, 40)):
+            idx = rng.integers(0, arr.shape[0], cnt)
+            arr[idx, rng.integers(0, d, cnt)] = rng.choice(
+                [np.inf, -np.inf, np.nan, 3e38, -3e38], cnt)
+    else:
+        x = 10.0 * rng.standard_normal((n, d))
+        y = 10.0 * rng.standard_normal((m, d))
+        cuts = np.sort(rng.choice(np.arange(1, n), 199, replace=False))
+        ptr_x = np.concatenate([[0], cuts, [n]])
+        cuts = np.sort(rng.choice(np.arange(1, m), 199, replace=False))
+        ptr_y = np.concatenate([[0], cuts, [m]])
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    with np.errstate(all="ignore"):
+        got, gd = gpu_knn(x, y, ptr_x, ptr_y, k)
+        want, wd = oracle_knn_edges(oracle, x, y, ptr_x, ptr_y, k)
+    assert got.shape == want.shape
+    assert (got == want).all()
+    assert (gd == wd).all()
+
+
 @pytest.mark.parametrize("d,k", [(3, 16), (24, 16), (128, 32), (100, 7)])
 @pytest.mark.parametrize("case", ["parallel", "random", "scaled_copies",
                                   "zero_rows"])
