@@ -10,16 +10,16 @@ template <int STEPS>
 hipError_t launch_knn_mfma_steps(const KnnMfmaParams &p, int kbucket,
                                  bool cosine, int grid, hipStream_t stream);
 template <>
-hipError_t launch_knn_mfma_steps<8>(const KnnMfmaParams &, int, bool, int,
+hipError_t launch_knn_mfma_steps<12>(const KnnMfmaParams &, int, bool, int,
                                     hipStream_t);
 template <>
-hipError_t launch_knn_mfma_steps<16>(const KnnMfmaParams &, int, bool, int,
+hipError_t launch_knn_mfma_steps<20>(const KnnMfmaParams &, int, bool, int,
                                      hipStream_t);
 template <>
-hipError_t launch_knn_mfma_steps<32>(const KnnMfmaParams &, int, bool, int,
+hipError_t launch_knn_mfma_steps<36>(const KnnMfmaParams &, int, bool, int,
                                      hipStream_t);
 template <>
-hipError_t launch_knn_mfma_steps<64>(const KnnMfmaParams &, int, bool, int,
+hipError_t launch_knn_mfma_steps<68>(const KnnMfmaParams &, int, bool, int,
                                      hipStream_t);
 
 // csrc/knn_generic_cos.hip
@@ -92,7 +92,7 @@ size_t knn_mfma_scratch_bytes(int n, int m, int num_segments, int k) {
   // the largest slice count a call may choose
   const int chunks = std::max(knn_mfma_slices(n, m, num_segments), 1);
   return align256(sizeof(float) * (size_t)n) +
-         align256(sizeof(float) * (size_t)m) +
+         2 * align256(sizeof(float) * (size_t)m) +
          align256(sizeof(double) * tiles * chunks * (size_t)k *
                   kMfmaQueries);
 }
@@ -109,12 +109,16 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   base += align256(sizeof(float) * (size_t)in.n);
   float *tau = reinterpret_cast<float *>(base);
   base += align256(sizeof(float) * (size_t)in.m);
+  float *y_norm = reinterpret_cast<float *>(base);
+  base += align256(sizeof(float) * (size_t)in.m);
   double *partial = reinterpret_cast<double *>(base);
 
-  if (cosine)
+  if (cosine) {
     (void)launch_row_norms(static_cast<const float *>(in.x), in.n, in.d, x_sq,
                            stream);
-  else
+    (void)launch_row_norms(static_cast<const float *>(in.y), in.m, in.d,
+                           y_norm, stream);
+  } else
     hipLaunchKernelGGL(row_sqnorm_kernel, dim3((in.n + kBlock - 1) / kBlock),
                        dim3(kBlock), 0, stream,
                        static_cast<const float *>(in.x), in.n, in.d, x_sq);
@@ -127,6 +131,7 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   p.ptr_x = in.ptr_x;
   p.ptr_y = in.ptr_y;
   p.x_sq = x_sq;
+  p.y_norm = y_norm;
   p.n = in.n;
   p.m = in.m;
   p.d = in.d;
@@ -134,22 +139,38 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   p.k = k;
   p.work_start = work_start;
   p.num_chunks = chunks;
+  p.sample_rows = 0;
   p.tau = tau;
   p.partial = partial;
 
   const int kb = k_bucket(k);
   const int grid = tiles_bound * chunks;
+  // 2 STEPS components per row: the d coordinates and two augmented ones
+  auto launch = [&](const KnnMfmaParams &pp, int g) {
+    if (in.d <= 22)
+      return launch_knn_mfma_steps<12>(pp, kb, cosine, g, stream);
+    if (in.d <= 38)
+      return launch_knn_mfma_steps<20>(pp, kb, cosine, g, stream);
+    if (in.d <= 70)
+      return launch_knn_mfma_steps<36>(pp, kb, cosine, g, stream);
+    return launch_knn_mfma_steps<68>(pp, kb, cosine, g, stream);
+  };
+  // Bound-seeding pass over a sample of every segment, worth its share of
+  // the scan once the segments are much longer than the sample.
+  int sample = 8192;
+  if (const char *env = std::getenv("PCA_KNN_SAMPLE"))
+    sample = std::atoi(env);
+  if (sample >= 8 * k && in.n / in.num_segments >= 8 * sample) {
+    KnnMfmaParams sp = p;
+    sp.sample_rows = sample;
+    sp.num_chunks = 1;
+    const hipError_t serr = launch(sp, tiles_bound);
+    if (serr != hipSuccess)
+      return serr;
+  }
   if (time_start)
     (void)hipEventRecord(time_start, stream);
-  hipError_t err;
-  if (in.d <= 16)
-    err = launch_knn_mfma_steps<8>(p, kb, cosine, grid, stream);
-  else if (in.d <= 32)
-    err = launch_knn_mfma_steps<16>(p, kb, cosine, grid, stream);
-  else if (in.d <= 64)
-    err = launch_knn_mfma_steps<32>(p, kb, cosine, grid, stream);
-  else
-    err = launch_knn_mfma_steps<64>(p, kb, cosine, grid, stream);
+  const hipError_t err = launch(p, grid);
   if (time_stop)
     (void)hipEventRecord(time_stop, stream);
   if (err != hipSuccess)

@@ -1,50 +1,67 @@
-// Feature-space kNN (8 < d <= 128, k <= 32, Euclidean or cosine) on the gfx950
+// Feature-space kNN (8 < d <= 134, k <= 32, Euclidean or cosine) on the gfx950
 // matrix cores, with results bit-identical to the reference's scalar loop
 // (csrc/cuda/knn_cuda.cu:52-78).
 //
-// The distance of a (query, candidate) pair is |x|^2 + |y|^2 - 2 x.y.  The
-// x.y of 32 candidates x 32 queries is one chain of v_mfma_f32_32x32x2_f32
-// (fp32 in, fp32 accumulate) over the components -- a dense contraction, the
-// one place on this path where the matrix cores apply.  The expanded form is
-// not accurate enough to rank neighbours by itself (|x - y| can be far below
-// |x|), so, exactly as in the low-dimensional kernel, it only REJECTS:
+// Filter.  The matrix cores decide which candidates are LOOKED AT; every
+// distance that is kept is evaluated exactly as the reference does.  For the
+// Euclidean metric the filter value of a (query, candidate) pair is
+//     t = w - 2 x.y,      w = fl(|x|^2) (1 - eps),
+// the dot product of the augmented rows (x, w) and (-2 y, 1): one chain of
+// v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate) over the components for 32
+// candidates x 32 queries.  The last component carries (1) . (-cut),
+//     cut = thresh (1 + eps) - fl(|y|^2) (1 - eps)   (rounded up),
+//     eps = (d + 32) 2^-22,
+// so the SIGN of a result says whether the candidate can still have an exact
+// distance below thresh: with the accumulated products within 2 u |x||y| per
+// term of the true ones (u = 2^-24), norms accumulated with one FMA per
+// component and the exact chain d_exact >= |x-y|^2 (1 - (d + 2) u), a
+// candidate with d_exact < thresh always has t - cut < 0.  Rows whose squared
+// norm is not a moderate finite number enter with zero coordinates and
+// w = -inf (always looked at), padding rows with w = NaN (never), queries with
+// such a norm use cut = +inf with zero coordinates (look at every real row).
 //
-//     t   = fl(|x|^2) * (1 - eps) - 2 * mfma_dot(x, y)
-//     cut = thresh * (1 + eps) - fl(|y|^2) * (1 - eps)      (rounded up)
-//     eps = (d + 32) * 2^-22
+// The cosine distance 1 - x.y / (|x| |y|) uses the same chain on normalised
+// rows: (x / |x|, 1) . (-y / |y|, 1) = 1 - cos, within (4 d + 72) u of the
+// exactly evaluated distance; the cut is thresh + that margin.
+// Rows of norm 0 or NaN have a NaN distance in the reference and are padding
+// here; a row or query of infinite norm is looked at / looks at everything.
 //
-// With the matrix-core dot product within 2 u |x||y| per accumulated term of
-// the true one (u = 2^-24), norms accumulated with one FMA per component and
-// the exact distance d_exact >= |x-y|^2 (1 - (d+2) u), a candidate with
-// d_exact < thresh always has t < cut.  Candidates with t >= cut are dropped
-// after one FMA and their share of a min/compare; the rest (true neighbours
-// plus a sliver) are parked, and before the tile leaves LDS all 64 lanes take
-// the exact distance of their parked candidates -- direct differences, one
-// FMA per component in ascending order, the candidate's components from the
-// tile in LDS, the query's from the B-operand registers of the lane and of
-// its partner lane (v_permlane32_swap) -- and feed the usual (distance, row)
-// key lists.  No memory latency is involved, and the vector work of one wave
-// overlaps the matrix-core chain of the other wave on the same SIMD.
-//
-// The cosine distance 1 - x.y / (|x| |y|) uses the same matrix-core dot
-// product: the filter value is 1 - mfma_dot * (1/|x|) * (1/|y|), within
-// (3d + 40) u of the exactly evaluated distance, and is tested against
-// thresh + (4d + 64) u; the exact value divides the sequentially accumulated
-// dot product by the product of the two norms like the reference does
-// (csrc/cuda/knn_cuda.cu:9-28,55-59).
+// Selection.  A lane gathers the 16 sign bits of a 32-row step with funnel
+// shifts and, if any is set, parks (step, mask) in its LDS queue -- one write.
+// Every kMfmaDrainSteps steps a wave resolves what its lanes have parked,
+// densely: the parked (query, row) pairs of all 64 lanes are compacted into
+// one list, lane i takes pair i, 64 + i, ... and evaluates its exact distance
+// -- direct differences, one FMA per component in ascending order
+// (csrc/cuda/knn_cuda.cu:9-28,55-66), both rows streamed from global memory
+// (they are L2 resident) -- and hands the (distance, row) key back through
+// LDS to the lane that owns the query, which runs the insertion network.  An
+// exact distance costs ~2 d vector instructions for the whole wave whether 1
+// or 64 lanes have work, so the dense list is what keeps the re-rank a few
+// percent of the matrix-core time even when a handful of queries collect most
+// of the candidates.
 //
 // Mapping: a workgroup owns 128 queries of one segment (4 waves x 32) and one
 // slice of the segment's x rows.  A = 32 candidates (rows i), B = 32 queries
 // (columns j): lane l supplies A[l%32][2s + l/32] and B[2s + l/32][l%32] for
-// step s, and receives, in 16 accumulator registers, the dot products of
-// query l%32 with the 16 candidate rows 8*(v/4) + 4*(l/32) + v%4.  So the two
-// lanes l and l+32 share a query and split its candidates; they hand each
-// other every key they accept (v_permlane32_swap) and so keep one identical
-// list.  The lists of a query's slices are merged by knn_merge_kernel and
-// exchange their pruning bound through `tau` like the slices of the
-// low-dimensional kernel do.
+// step s, and receives, in 16 accumulator registers, the results of query
+// l%32 against the 16 candidate rows 8*(v/4) + 4*(l/32) + v%4.  So lanes l and
+// l+32 share a query and split its candidates: each keeps its own sorted list
+// (its rows arrive in ascending order, so its own k-th distance is a strict
+// bound), the two exchange their k-th distances after every drain, and the
+// lists are united at the end.  The lists of a query's slices are merged by
+// knn_merge_kernel and exchange their pruning bound through `tau` like the
+// slices of the low-dimensional kernels do.
 //
-// The query operands stay in registers for the whole scan (d/2 per lane);
+// Bound-seeding pass (sample_rows > 0): the same kernel scans only every
+// stride-th x row of each segment (about sample_rows of them), keeps no
+// results and posts each query's k-th best sampled distance to `tau`.  The
+// k-th distance within any subset of the candidates bounds the final k-th
+// distance from above, so the slices of the full scan -- each of which would
+// otherwise accept and evaluate exactly its first k candidates and a good
+// many more before its own list is of any use -- start with a bound that
+// only about k * stride candidates per query pass at all.
+//
+// The query operands stay in registers for the whole scan (d/2 + 1 per lane);
 // candidate tiles stream through LDS, double-buffered, with the even and odd
 // components of a row stored as two contiguous halves so that a lane's
 // operands for 4 consecutive steps are one ds_read_b128.
@@ -56,9 +73,10 @@
 
 namespace pca {
 
-constexpr int kMfmaQueries = 128; // queries per workgroup
-constexpr int kMfmaRows = 32;     // candidates per tile
-constexpr int kMfmaSyncTiles = 8; // tiles between exchanges of bounds
+constexpr int kMfmaQueries = 128;   // queries per workgroup
+constexpr int kMfmaRows = 32;       // candidates per step
+constexpr int kMfmaDrainSteps = 8;  // steps between drains (= queue entries)
+constexpr int kMfmaPassPairs = 128; // pairs a wave evaluates per pass
 
 typedef float mfma_acc_t __attribute__((ext_vector_type(16)));
 
@@ -67,10 +85,12 @@ struct KnnMfmaParams {
   const float *y;
   const int64_t *ptr_x;
   const int64_t *ptr_y;
-  const float *x_sq; // [n] squared norms of the x rows (cosine: norms)
+  const float *x_sq;   // [n] squared norms of the x rows (cosine: norms)
+  const float *y_norm; // [m] norms of the y rows (cosine only)
   int n, m, d, num_segments, k;
   const int *work_start; // [num_segments + 1] first 128-query tile per segment
   int num_chunks;        // slices of every segment's x rows
+  int sample_rows;       // > 0: bound-seeding pass (see above)
   float *tau;            // [m] shared pruning bounds
   double *partial;       // [num_chunks * tiles][k][128] keys
 };
@@ -92,22 +112,33 @@ __device__ __forceinline__ float mfma_filter_cut(float thresh, float ysq,
   return f;
 }
 
-// STEPS = padded d / 2: matrix-core steps per tile.
+// A lane's walk over the rows it has parked, in ascending order.
+struct MfmaWalk {
+  int taken;        // queue entries started
+  uint32_t pending; // rows of the current entry still to visit
+  int base;         // the lane's first row of that entry's step
+};
+
+// STEPS = matrix-core steps per 32 rows: 2 STEPS >= d + 2 components (the
+// coordinates, w, and the last one for the cut).
 template <int STEPS, int K, bool COSINE>
 __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
-  constexpr int DP = 2 * STEPS;  // padded number of components
-  constexpr int RS = DP + 4;     // LDS row stride (floats), keeps b128 reads
-                                 // of 8 neighbouring rows on distinct banks
+  constexpr int DP = 2 * STEPS; // padded number of components (with w)
+  constexpr int RS = DP + 4;    // LDS row stride (floats), keeps b128 reads
+                                // of 8 neighbouring rows on distinct banks
   constexpr int TR = kMfmaRows;
   constexpr int TQ = kMfmaQueries;
   constexpr int PER_THREAD = TR * DP / kBlock; // floats staged per thread
+  constexpr int QCAP = kMfmaDrainSteps;
+  constexpr int CAP = kMfmaPassPairs;
+  static_assert(STEPS % 4 == 0 && (TR * DP) % kBlock == 0, "tile shape");
 
   __shared__ __attribute__((aligned(16))) float xs[2][TR][RS];
-  // per row: damped squared norm (Euclidean) or 1 / norm (cosine) ...
-  __shared__ __attribute__((aligned(16))) float wn[2][TR];
-  // ... and, for the cosine distance, the norm itself
-  __shared__ float xnorm[2][COSINE ? TR : 1];
-  __shared__ uint8_t queue[16][kBlock]; // parked rows of the current tile
+  // parked steps: (step within the batch << 16) | mask of the lane's rows
+  __shared__ uint32_t queue[QCAP][kBlock];
+  // dense re-rank, per wave: (query, row) pairs and their keys
+  __shared__ int2 pairs[kBlock / kWave][CAP];
+  __shared__ double results[kBlock / kWave][CAP];
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -136,98 +167,144 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   const int seg_len = x_end - x_begin;
   const int chunk_len =
       ((seg_len + p.num_chunks - 1) / p.num_chunks + TR - 1) / TR * TR;
-  const int c_begin = min(x_end, x_begin + chunk * chunk_len);
-  const int c_end = min(x_end, c_begin + chunk_len);
-  const int num_tiles = (c_end - c_begin + TR - 1) / TR;
+  // rows are addressed as c_begin + position * stride, position < c_count
+  const int stride = p.sample_rows > 0 ? max(1, seg_len / p.sample_rows) : 1;
+  const int c_begin =
+      p.sample_rows > 0 ? x_begin : min(x_end, x_begin + chunk * chunk_len);
+  const int c_count = p.sample_rows > 0
+                          ? (seg_len + stride - 1) / stride
+                          : min(x_end, c_begin + chunk_len) - c_begin;
+  const int num_steps = (c_count + TR - 1) / TR;
 
   const double eps = (double)(d + 32) * (1.0 / 4194304.0); // (d+32) * 2^-22
   const float damp = (float)(1.0 - eps);
+  const float cos_margin = (float)(4 * d + 72) * 5.9604644775390625e-08f;
 
-  // ---- per-lane state ---------------------------------------------------
-  float yb[STEPS]; // B operands: this lane's parity of the query's components
-#pragma unroll
-  for (int s = 0; s < STEPS; ++s) {
-    const int c = 2 * s + half;
-    yb[s] = (valid && c < d) ? yrow[c] : 0.0f;
-  }
+  // ---- per-lane query state ---------------------------------------------
   float ysq = 0.0f;
   for (int c = 0; c < d; ++c)
     ysq = __builtin_fmaf(yrow[c], yrow[c], ysq);
   const float ynorm = __builtin_sqrtf(ysq);
-  const float yrinv = 1.0f / ynorm;
-  const float cos_margin = (float)(4 * d + 64) * 5.9604644775390625e-08f;
+  // what the query contributes to the filter: coordinates (scaled), or
+  // nothing when the filter is switched off for it
+  bool y_filtered; // false: coordinates enter as zeros
+  bool y_blind;    // true: the query can have no neighbours at all
+  float y_scale;
+  if (COSINE) {
+    y_blind = !(ynorm > 0.0f); // 0 or NaN: every distance is NaN
+    y_filtered = !y_blind && ynorm < __builtin_inff();
+    y_scale = y_filtered ? -1.0f / ynorm : 0.0f;
+  } else {
+    y_blind = false;
+    y_filtered = ysq <= kFilterNormLimit;
+    y_scale = -2.0f;
+  }
+  const bool active = valid && !y_blind;
+  float yb[STEPS]; // B operands: this lane's parity of the augmented query
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    const int c = 2 * s + half;
+    float v = 0.0f;
+    if (active) {
+      if (c < d)
+        v = y_filtered ? yrow[c] * y_scale : 0.0f;
+      else if (c == d)
+        v = 1.0f;
+    }
+    yb[s] = v;
+  }
 
   double best[K];
 #pragma unroll
   for (int j = 0; j < K; ++j)
     best[j] = (j < K - k) ? lowest_key() : empty_key();
-  float thresh = kKnnSentinel;
-  float bound =
-      COSINE ? thresh + cos_margin : mfma_filter_cut(thresh, ysq, eps);
-  float shared = kKnnSentinel;
+  // exact distances must be strictly below thresh
+  float thresh = active ? kKnnSentinel : -__builtin_inff();
+  float shared = kKnnSentinel; // bound inherited from other slices / partner
   float posted = kKnnSentinel;
-
+  // the last component of the rows (odd: upper lanes) is 1; the upper lanes
+  // hold -cut there (a lane without a query holds zeros everywhere and never
+  // parks)
   auto set_thresh = [&](float v) {
+    if (!active)
+      return;
     thresh = v;
-    bound = COSINE ? v + cos_margin : mfma_filter_cut(v, ysq, eps);
+    float cut;
+    if (COSINE)
+      cut = y_filtered ? v + cos_margin : __builtin_inff();
+    else
+      cut = mfma_filter_cut(v, ysq, eps);
+    if (half)
+      yb[STEPS - 1] = -cut;
   };
+  set_thresh(thresh);
 
   // ---- tile staging -------------------------------------------------------
-  // thread -> row tid / 8, components [seg8 * DP/8, (seg8 + 1) * DP/8)
+  // thread -> row tid / 8, components tid % 8, tid % 8 + 8, ...
   const int st_row = tid >> 3;
-  const int st_c0 = (tid & 7) * (DP / 8);
-  float stage[PER_THREAD];
-  float stage_w = 0.0f;
-  float stage_norm = 0.0f;
+  const int st_c0 = tid & 7;
+  // load_tile only issues the global loads (they are in flight during the
+  // matrix-core chain of the current tile); store_tile turns what arrived
+  // into filter operands
+  float raw[PER_THREAD];
+  float raw_norm = 0.0f;
+  bool raw_real = false;
 
   auto load_tile = [&](int t) {
-    const int g = c_begin + t * TR + st_row;
+    const int pos = t * TR + st_row;
+    const size_t g = (size_t)c_begin + (size_t)pos * stride;
+    raw_real = pos < c_count;
+    // (rows past the end and padding components read a clamped address and
+    // are masked out later)
+    const size_t gl = raw_real ? g : (size_t)c_begin;
+    raw_norm = p.x_sq[gl];
+    const float *src = p.x + gl * d + st_c0;
 #pragma unroll
-    for (int e = 0; e < PER_THREAD; ++e) {
-      const int c = st_c0 + e;
-      // rows past the slice end and padding components are zero; such rows
-      // get w = +inf below and never pass the filter
-      stage[e] = (g < c_end && c < d) ? p.x[(size_t)g * d + c] : 0.0f;
-    }
-    if (tid < TR) {
-      const int gr = c_begin + t * TR + tid;
-      float w = __builtin_inff();
-      if (COSINE) {
-        // filter value = 1 - dot * w * (1 / |y|); padding rows: w = 0 and
-        // |x| = NaN, so that neither the filter (bound < 1 once a list is
-        // full) nor the exact distance (NaN) can accept them
-        float nx = __builtin_nanf("");
-        w = 0.0f;
-        if (gr < c_end) {
-          nx = p.x_sq[gr];
-          w = 1.0f / nx;
-        }
-        stage_norm = nx;
-      } else if (gr < c_end) {
-        const float s = p.x_sq[gr];
-        // norms that are not moderate finite numbers always pass the filter
-        w = (s <= kFilterNormLimit) ? s * damp : -__builtin_inff();
-      }
-      stage_w = w;
-    }
+    for (int e = 0; e < PER_THREAD; ++e)
+      raw[e] = (st_c0 + 8 * e < d) ? src[8 * e] : 0.0f;
   };
   auto store_tile = [&](int buf) {
+    const float nv = raw_norm;
+    // coordinates enter the filter scaled by `scale` (0: not at all); `aug`
+    // is the augmented component
+    float scale, aug;
+    if (COSINE) {
+      if (!raw_real || !(nv > 0.0f)) { // padding, or a NaN distance anyway
+        scale = 0.0f;
+        aug = __builtin_nanf("");
+      } else if (nv == __builtin_inff()) { // always looked at
+        scale = 0.0f;
+        aug = -__builtin_inff();
+      } else {
+        scale = 1.0f / nv;
+        aug = 1.0f;
+      }
+    } else {
+      if (!raw_real) {
+        scale = 0.0f;
+        aug = __builtin_nanf("");
+      } else if (!(nv <= kFilterNormLimit)) {
+        scale = 0.0f;
+        aug = -__builtin_inff();
+      } else {
+        scale = 1.0f;
+        aug = nv * damp;
+      }
+    }
 #pragma unroll
     for (int e = 0; e < PER_THREAD; ++e) {
-      const int c = st_c0 + e;
-      xs[buf][st_row][(c & 1) * STEPS + (c >> 1)] = stage[e];
-    }
-    if (tid < TR) {
-      wn[buf][tid] = stage_w;
-      if (COSINE)
-        xnorm[buf][tid] = stage_norm;
+      const int c = st_c0 + 8 * e;
+      float v = (scale != 0.0f && c < d) ? raw[e] * scale : 0.0f;
+      v = (c == d) ? aug : v;
+      v = (c == DP - 1) ? 1.0f : v; // times -cut
+      xs[buf][st_row][(c & 1) * STEPS + (c >> 1)] = v;
     }
   };
 
   // Exchange of pruning bounds between the slices of a query: the k-th best
   // distance any slice has reached bounds the final k-th distance from above.
   auto sync_bounds = [&]() {
-    if (valid) {
+    if (active) {
       // a (slightly) negative cosine distance is published as 0: still an
       // upper bound, and non-negative floats order like their bit patterns
       const float own = __builtin_fmaxf(key_dist(best[K - 1]), 0.0f);
@@ -241,95 +318,190 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
       } else if (seen < posted) {
         posted = seen;
         // another slice's k-th distance: equality must still pass
-        shared = next_up_positive(seen);
-        set_thresh(__builtin_fminf(thresh, shared));
+        shared = __builtin_fminf(shared, next_up_positive(seen));
+        if (shared < thresh)
+          set_thresh(shared);
       }
     }
   };
 
-  // Exact distances of the rows parked from the current tile, slot by slot
-  // for all lanes together.
-  int parked = 0;
-  auto drain = [&](int buf, int g_base) {
-    for (int s = 0; s < 16; ++s) {
-      const bool has = s < parked;
-      if (!__any(has))
-        break;
-      const int row = has ? (int)queue[s][tid] : 0;
-      const float *xr = &xs[buf][row][0];
-      float dist = 0.0f;
+  // ---- dense re-rank ------------------------------------------------------
+  int qn = 0; // parked steps of this lane: queue[0 .. qn)[tid]
+
+  // -> true and the next parked row of this lane (relative to the batch's
+  // first row) if one is left
+  auto walk_next = [&](MfmaWalk &w, int &row) {
+    if (w.pending == 0 && w.taken < qn) {
+      const uint32_t word = queue[w.taken][tid];
+      ++w.taken;
+      w.pending = word & 0xffffu;
+      w.base = (int)(word >> 16) * TR + 4 * half;
+    }
+    const bool has = w.pending != 0;
+    // bit 15 - v of the mask stands for accumulator v = row
+    // 8 (v / 4) + v % 4 of the lane's rows: highest bit first
+    const int bit = 31 - __builtin_clz(has ? w.pending : 1u);
+    const int v = 15 - bit;
+    w.pending &= ~(1u << bit);
+    row = w.base + 2 * (v & 12) + (v & 3);
+    return has;
+  };
+
+  auto exact_distance = [&](int qq, int g) {
+    const float *xr = p.x + (size_t)g * d;
+    const float *yr = p.y + (size_t)qq * d;
+    float acc = 0.0f;
+    if ((d & 3) == 0) {
+      const float4 *x4 = reinterpret_cast<const float4 *>(xr);
+      const float4 *y4 = reinterpret_cast<const float4 *>(yr);
+#pragma unroll 4
+      for (int c = 0; c < d / 4; ++c) {
+        const float4 a = x4[c];
+        const float4 b = y4[c];
+        if (COSINE) {
+          acc = __builtin_fmaf(a.x, b.x, acc);
+          acc = __builtin_fmaf(a.y, b.y, acc);
+          acc = __builtin_fmaf(a.z, b.z, acc);
+          acc = __builtin_fmaf(a.w, b.w, acc);
+        } else {
+          const float d0 = a.x - b.x, d1 = a.y - b.y;
+          const float d2 = a.z - b.z, d3 = a.w - b.w;
+          acc = __builtin_fmaf(d0, d0, acc);
+          acc = __builtin_fmaf(d1, d1, acc);
+          acc = __builtin_fmaf(d2, d2, acc);
+          acc = __builtin_fmaf(d3, d3, acc);
+        }
+      }
+    } else {
+      for (int c = 0; c < d; ++c) {
+        if (COSINE) {
+          acc = __builtin_fmaf(xr[c], yr[c], acc);
+        } else {
+          const float dc = xr[c] - yr[c];
+          acc = __builtin_fmaf(dc, dc, acc);
+        }
+      }
+    }
+    if (COSINE) {
+      acc = acc / (p.x_sq[g] * p.y_norm[qq]);
+      acc = 1.0f - acc;
+    }
+    return acc;
+  };
+
+  // Resolves everything parked since the last drain; pos0 = position of the
+  // batch's first row in the slice.
+  auto drain = [&](int pos0) {
+    // how many rows has each lane parked, and where do they go in the list
+    int count = 0;
+    for (int e = 0; e < QCAP; ++e)
+      if (e < qn)
+        count += __builtin_popcount(queue[e][tid] & 0xffffu);
+    int offset = count; // inclusive prefix sum over the wave
 #pragma unroll
-      for (int s4 = 0; s4 < STEPS / 4; ++s4) {
-        const float4 xe = *reinterpret_cast<const float4 *>(xr + 4 * s4);
-        const float4 xo =
-            *reinterpret_cast<const float4 *>(xr + STEPS + 4 * s4);
-        const float xev[4] = {xe.x, xe.y, xe.z, xe.w};
-        const float xov[4] = {xo.x, xo.y, xo.z, xo.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          // lanes 0-31 hold the even components of their query, lanes 32-63
-          // the odd ones: the swap hands every lane both
-          const auto both = __builtin_amdgcn_permlane32_swap(
-              __float_as_uint(yb[4 * s4 + e]), __float_as_uint(yb[4 * s4 + e]),
-              false, false);
-          if (COSINE) {
-            dist = __builtin_fmaf(xev[e], __uint_as_float(both[0]), dist);
-            dist = __builtin_fmaf(xov[e], __uint_as_float(both[1]), dist);
-          } else {
-            const float d0 = xev[e] - __uint_as_float(both[0]);
-            dist = __builtin_fmaf(d0, d0, dist);
-            const float d1 = xov[e] - __uint_as_float(both[1]);
-            dist = __builtin_fmaf(d1, d1, dist);
+    for (int sh = 1; sh < kWave; sh <<= 1) {
+      const int up = __shfl_up(offset, sh);
+      if (lane >= sh)
+        offset += up;
+    }
+    const int total = __shfl(offset, kWave - 1);
+    offset -= count;
+    bool changed = false; // wave-uniform
+
+    for (int pass0 = 0; pass0 < total; pass0 += CAP) {
+      // 1. the pairs of this pass, compacted
+      {
+        MfmaWalk w{0, 0u, 0};
+        int idx = offset;
+        for (;;) {
+          int row;
+          const bool has = walk_next(w, row);
+          if (!__any(has))
+            break;
+          if (has) {
+            if (idx >= pass0 && idx < pass0 + CAP)
+              pairs[wave][idx - pass0] =
+                  make_int2(q, pos0 + row < c_count
+                                   ? c_begin + (pos0 + row) * stride
+                                   : -1);
+            ++idx;
           }
         }
       }
-      if (COSINE) {
-        dist = dist / (xnorm[buf][row] * ynorm);
-        dist = 1.0f - dist;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      // 2. exact distances, one pair per lane and round
+      const int in_pass = min(CAP, total - pass0);
+      for (int i = lane; i < in_pass; i += kWave) {
+        const int2 pr = pairs[wave][i];
+        float dist = __builtin_nanf("");
+        if (pr.y >= 0) // (a padding row is never a candidate)
+          dist = exact_distance(pr.x, pr.y);
+        results[wave][i] = make_key(dist, (uint32_t)pr.y);
       }
-      // The two lanes that share a query keep ONE list between them: each
-      // hands its key to the other, both insert both, so the lists stay
-      // identical and the pruning bound is the k-th distance over all 32 rows
-      // of a tile, not over a lane's 16.  Rows of one lane reach its list in
-      // ascending order but the partner's rows interleave, so equality with
-      // the worst kept distance must pass (`<=`): the key order settles ties.
-      const bool ok = has && valid && dist <= thresh;
-      if (!__any(ok))
-        continue;
-      const double key =
-          ok ? make_key(dist, (uint32_t)(g_base + row)) : empty_key();
-      const auto hi = __builtin_amdgcn_permlane32_swap(
-          (unsigned)__double2hiint(key), (unsigned)__double2hiint(key), false,
-          false);
-      const auto lo = __builtin_amdgcn_permlane32_swap(
-          (unsigned)__double2loint(key), (unsigned)__double2loint(key), false,
-          false);
-      // element 0 = the lower lane's key, element 1 = the upper lane's
-      const double key_a = __hiloint2double((int)hi[0], (int)lo[0]);
-      const double key_b = __hiloint2double((int)hi[1], (int)lo[1]);
-      sorted_insert<K>(best, key_a);
-      sorted_insert<K>(best, key_b);
-      set_thresh(__builtin_fminf(key_dist(best[K - 1]), shared));
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      // 3. every lane collects the keys of its own rows, in order
+      {
+        MfmaWalk w{0, 0u, 0};
+        int idx = offset;
+        for (;;) {
+          int row;
+          const bool has = walk_next(w, row);
+          if (!__any(has))
+            break;
+          const bool mine = has && idx >= pass0 && idx < pass0 + CAP;
+          const double key = mine ? results[wave][idx - pass0] : empty_key();
+          if (has)
+            ++idx;
+          // NaN and sentinel distances fail the compare like in the
+          // reference (csrc/cuda/knn_cuda.cu:48,68)
+          const bool ok = mine && key_dist(key) < thresh;
+          if (!__any(ok))
+            continue;
+          sorted_insert<K>(best, ok ? key : empty_key());
+          if (active)
+            thresh = __builtin_fminf(key_dist(best[K - 1]), shared);
+          changed = true;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
     }
-    parked = 0;
+    qn = 0;
+    if (changed) {
+      // the partner's k-th distance bounds the query's final k-th distance
+      // too (equality admitted: its rows interleave with this lane's)
+      const float own = key_dist(best[K - 1]);
+      const auto both = __builtin_amdgcn_permlane32_swap(
+          __float_as_uint(own), __float_as_uint(own), false, false);
+      const float partner = __uint_as_float(half ? both[0] : both[1]);
+      if (active && partner < kKnnSentinel && !(partner < 0.0f))
+        shared = __builtin_fminf(shared, next_up_positive(partner));
+      set_thresh(__builtin_fminf(thresh, shared));
+    }
+    sync_bounds();
   };
 
-  if (num_tiles > 0) {
+  if (num_steps > 0) {
     load_tile(0);
     store_tile(0);
   }
   __syncthreads();
+  sync_bounds(); // what other slices (or the seeding pass) already know
 
-  for (int t = 0; t < num_tiles; ++t) {
+  // steps [batch_t0, t] are parked and not yet resolved; the first drains
+  // come early (after steps 0, 1 and 3), while the lists are still empty and
+  // every row passes
+  int batch_t0 = 0;
+  for (int t = 0; t < num_steps; ++t) {
     const int buf = t & 1;
-    const bool more = t + 1 < num_tiles;
+    const bool more = t + 1 < num_steps;
     if (more)
       load_tile(t + 1);
-    if ((t % kMfmaSyncTiles) == 0)
-      sync_bounds();
-    const int g_base = c_begin + t * TR;
 
-    // ---- 32 x 32 dot products on the matrix cores -----------------------
+    // ---- 32 x 32 filter values on the matrix cores ----------------------
     mfma_acc_t acc = {0};
     const float *arow = &xs[buf][col][half * STEPS];
 #pragma unroll
@@ -345,40 +517,19 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
                                                  0, 0);
     }
 
-    // ---- filter ---------------------------------------------------------
-    // accumulator v holds candidate row 8 * (v / 4) + 4 * half + v % 4
-    float score[16];
-    float lo = __builtin_inff();
+    // accumulator v belongs to candidate row 8 (v / 4) + 4 half + v % 4; its
+    // sign bit says "look at this row" (bit 15 - v of the mask)
+    uint32_t mask = 0;
 #pragma unroll
-    for (int v4 = 0; v4 < 4; ++v4) {
-      const float4 w =
-          *reinterpret_cast<const float4 *>(&wn[buf][8 * v4 + 4 * half]);
-      if (COSINE) {
-        score[4 * v4 + 0] = __builtin_fmaf(-acc[4 * v4 + 0], w.x * yrinv, 1.0f);
-        score[4 * v4 + 1] = __builtin_fmaf(-acc[4 * v4 + 1], w.y * yrinv, 1.0f);
-        score[4 * v4 + 2] = __builtin_fmaf(-acc[4 * v4 + 2], w.z * yrinv, 1.0f);
-        score[4 * v4 + 3] = __builtin_fmaf(-acc[4 * v4 + 3], w.w * yrinv, 1.0f);
-      } else {
-        score[4 * v4 + 0] = __builtin_fmaf(-2.0f, acc[4 * v4 + 0], w.x);
-        score[4 * v4 + 1] = __builtin_fmaf(-2.0f, acc[4 * v4 + 1], w.y);
-        score[4 * v4 + 2] = __builtin_fmaf(-2.0f, acc[4 * v4 + 2], w.z);
-        score[4 * v4 + 3] = __builtin_fmaf(-2.0f, acc[4 * v4 + 3], w.w);
-      }
-      lo = __builtin_fminf(
-          lo, __builtin_fminf(min3f(score[4 * v4], score[4 * v4 + 1],
-                                    score[4 * v4 + 2]),
-                              score[4 * v4 + 3]));
+    for (int v = 0; v < 16; ++v)
+      mask = __builtin_amdgcn_alignbit(mask, __float_as_uint(acc[v]), 31);
+    if (active && mask != 0) {
+      queue[qn][tid] = ((uint32_t)(t - batch_t0) << 16) | mask;
+      ++qn;
     }
-
-    if (__ballot(lo < bound) != 0) {
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        if (__ballot(score[v] < bound) != 0 && score[v] < bound) {
-          queue[parked][tid] = (uint8_t)(8 * (v / 4) + 4 * half + (v % 4));
-          ++parked;
-        }
-      }
-      drain(buf, g_base);
+    if (t - batch_t0 == QCAP - 1 || !more || t <= 1 || t == 3) {
+      drain(batch_t0 * TR);
+      batch_t0 = t + 1;
     }
 
     if (more)
@@ -386,7 +537,28 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
     __syncthreads();
   }
 
-  // ---- sorted keys of this slice (both lanes of a pair hold the same list)
+  // ---- results ------------------------------------------------------------
+  if (p.sample_rows > 0)
+    return; // the drains have posted the bounds
+  // unite the two half lists of each query: every lane inserts its partner's
+  // keys (all read before any list changes)
+  double theirs[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    const auto hi = __builtin_amdgcn_permlane32_swap(
+        (unsigned)__double2hiint(best[j]), (unsigned)__double2hiint(best[j]),
+        false, false);
+    const auto lo = __builtin_amdgcn_permlane32_swap(
+        (unsigned)__double2loint(best[j]), (unsigned)__double2loint(best[j]),
+        false, false);
+    theirs[j] = half ? __hiloint2double((int)hi[0], (int)lo[0])
+                     : __hiloint2double((int)hi[1], (int)lo[1]);
+  }
+#pragma unroll
+  for (int j = 0; j < K; ++j)
+    if (j >= K - k) // slots below are padding, not keys
+      sorted_insert<K>(best, theirs[j]);
+
   if (half == 0) {
     const size_t list = (size_t)chunk * total_tiles + tile;
     double *dst = p.partial + list * k * TQ + wave * 32 + col;

@@ -1,4 +1,4 @@
-// Matrix-core kNN kernels for up to 32 components per point.
+// Matrix-core kNN kernels for up to 38 components per point.
 #include "knn_mfma_impl.hpp"
 
 namespace pca {
@@ -19,21 +19,21 @@ void launch_one(const KnnMfmaParams &p, bool cosine, int grid,
 }
 
 template <>
-hipError_t launch_knn_mfma_steps<16>(const KnnMfmaParams &p, int kbucket,
+hipError_t launch_knn_mfma_steps<20>(const KnnMfmaParams &p, int kbucket,
                                      bool cosine, int grid,
                                      hipStream_t stream) {
   switch (kbucket) {
   case 8:
-    launch_one<16, 8>(p, cosine, grid, stream);
+    launch_one<20, 8>(p, cosine, grid, stream);
     break;
   case 16:
-    launch_one<16, 16>(p, cosine, grid, stream);
+    launch_one<20, 16>(p, cosine, grid, stream);
     break;
   case 24:
-    launch_one<16, 24>(p, cosine, grid, stream);
+    launch_one<20, 24>(p, cosine, grid, stream);
     break;
   case 32:
-    launch_one<16, 32>(p, cosine, grid, stream);
+    launch_one<20, 32>(p, cosine, grid, stream);
     break;
   default:
     return hipErrorInvalidValue;

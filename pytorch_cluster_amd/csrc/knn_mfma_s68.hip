@@ -1,4 +1,4 @@
-// Matrix-core kNN kernels for up to 128 components per point.
+// Matrix-core kNN kernels for up to 134 components per point.
 #include "knn_mfma_impl.hpp"
 
 namespace pca {
@@ -19,21 +19,21 @@ void launch_one(const KnnMfmaParams &p, bool cosine, int grid,
 }
 
 template <>
-hipError_t launch_knn_mfma_steps<64>(const KnnMfmaParams &p, int kbucket,
+hipError_t launch_knn_mfma_steps<68>(const KnnMfmaParams &p, int kbucket,
                                      bool cosine, int grid,
                                      hipStream_t stream) {
   switch (kbucket) {
   case 8:
-    launch_one<64, 8>(p, cosine, grid, stream);
+    launch_one<68, 8>(p, cosine, grid, stream);
     break;
   case 16:
-    launch_one<64, 16>(p, cosine, grid, stream);
+    launch_one<68, 16>(p, cosine, grid, stream);
     break;
   case 24:
-    launch_one<64, 24>(p, cosine, grid, stream);
+    launch_one<68, 24>(p, cosine, grid, stream);
     break;
   case 32:
-    launch_one<64, 32>(p, cosine, grid, stream);
+    launch_one<68, 32>(p, cosine, grid, stream);
     break;
   default:
     return hipErrorInvalidValue;
