@@ -157,7 +157,7 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   };
   // Bound-seeding pass over a sample of every segment, worth its share of
   // the scan once the segments are much longer than the sample.
-  int sample = 8192;
+  int sample = 4096;
   if (const char *env = std::getenv("PCA_KNN_SAMPLE"))
     sample = std::atoi(env);
   if (sample >= 8 * k && in.n / in.num_segments >= 8 * sample) {
