@@ -121,8 +121,12 @@ bool dtype_ok(int dtype) {
          dtype == PCA_BF16;
 }
 
-size_t radius_workspace(int64_t m, int64_t num_segments, int64_t slots) {
+size_t radius_workspace(int64_t n, int64_t m, int64_t d, int64_t num_segments,
+                        int64_t slots, int dtype) {
   size_t bytes = 0;
+  if (dtype == PCA_F32 &&
+      pca::radius_mc_supported((int)d, (int)n, (int)m, (int)num_segments))
+    bytes += pca::radius_mc_scratch_bytes((int)n, (int)d);
   bytes += align256(sizeof(int) * (size_t)(num_segments + 1));
   bytes += align256(sizeof(int) * (size_t)m * (size_t)slots);
   bytes += align256(sizeof(int) * (size_t)m);
@@ -326,8 +330,8 @@ size_t pca_radius_workspace_bytes(int64_t n, int64_t m, int64_t d,
   if (!sizes_ok(n, m, d, num_segments) || max_num_neighbors < 1 ||
       !dtype_ok(dtype))
     return 0;
-  return radius_workspace(m, num_segments,
-                          pca_radius_slots(n, max_num_neighbors));
+  return radius_workspace(n, m, d, num_segments,
+                          pca_radius_slots(n, max_num_neighbors), dtype);
 }
 
 int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
@@ -367,11 +371,19 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
     return fail(PCA_ERR_INVALID_ARGUMENT, "x, y or edges is NULL");
   const int64_t slots = pca_radius_slots(n, max_num_neighbors);
   if (workspace == nullptr || ((uintptr_t)workspace & 255) != 0 ||
-      workspace_bytes < radius_workspace(m, num_segments, slots))
+      workspace_bytes <
+          radius_workspace(n, m, d, num_segments, slots, dtype))
     return fail(PCA_ERR_WORKSPACE, "workspace needs %zu bytes, 256-aligned",
-                radius_workspace(m, num_segments, slots));
+                radius_workspace(n, m, d, num_segments, slots, dtype));
 
+  const bool matrix_cores =
+      dtype == PCA_F32 &&
+      pca::radius_mc_supported((int)d, (int)n, (int)m, (int)num_segments);
   Carver ws(workspace);
+  void *packed_rows = nullptr;
+  if (matrix_cores)
+    packed_rows =
+        ws.take<char>(pca::radius_mc_scratch_bytes((int)n, (int)d));
   int *work_start = ws.take<int>((size_t)num_segments + 1);
   pca::DenseResult dense;
   dense.idx = ws.take<int>((size_t)m * slots);
@@ -386,16 +398,22 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
 
   pca::SearchInput in{x,      y,      ptr_x,  ptr_y,
                       (int)n, (int)m, (int)d, (int)num_segments};
+  const int per_item = matrix_cores ? pca::kRadiusMcTileQueries
+                                    : pca::kRadiusQueriesPerWave;
   int rc = check_launch(pca::launch_plan(ptr_y, (int)m, (int)num_segments,
-                                         pca::kRadiusQueriesPerWave,
-                                         work_start, stream),
+                                         per_item, work_start, stream),
                         "plan_kernel");
   if (rc != PCA_OK)
     return rc;
-  const int bound = pca::plan_upper_bound((int)m, (int)num_segments,
-                                          pca::kRadiusQueriesPerWave);
+  const int bound =
+      pca::plan_upper_bound((int)m, (int)num_segments, per_item);
   timer.begin();
-  if (dtype == PCA_F32)
+  if (matrix_cores)
+    rc = check_launch(pca::launch_radius_mc(in, r2, ignore_same_index != 0,
+                                            work_start, bound, packed_rows,
+                                            dense, stream),
+                      "radius_mc_kernel");
+  else if (dtype == PCA_F32)
     rc = check_launch(pca::launch_radius(in, r2, ignore_same_index != 0,
                                          work_start, bound, dense, stream),
                       "radius_kernel");

@@ -108,6 +108,18 @@ hipError_t launch_radius_anytype(int dtype, const SearchInput &in, double r,
                                  const int *work_start, int task_bound,
                                  const DenseResult &out, hipStream_t stream);
 
+// --- radius_mc.hip ---------------------------------------------------------
+
+constexpr int kRadiusMcTileQueries = 128;
+bool radius_mc_supported(int d, int n, int m, int num_segments);
+// packed rows of x
+size_t radius_mc_scratch_bytes(int n, int d);
+// work_start: tiles of kRadiusMcTileQueries queries.
+hipError_t launch_radius_mc(const SearchInput &in, float r2,
+                            bool ignore_same_index, const int *work_start,
+                            int tiles_bound, void *scratch,
+                            const DenseResult &out, hipStream_t stream);
+
 // --- radius.hip ------------------------------------------------------------
 
 constexpr int kRadiusQueriesPerWave = 8;

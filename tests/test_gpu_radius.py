@@ -88,10 +88,17 @@ def test_radius_graph_large_vs_ckdtree():
 
 # ---- bit-exact parity against the oracle -----------------------------------
 
+@pytest.fixture(params=["0", "1"], ids=["wave_per_query", "matrix_cores"])
+def radius_path(request, monkeypatch):
+    # both fp32 kernels, whatever the problem size would select
+    monkeypatch.setenv("PCA_RADIUS_MATRIX_CORES", request.param)
+    return request.param
+
+
 @pytest.mark.parametrize("d", [1, 2, 3, 4, 7, 16])
 @pytest.mark.parametrize("cap,ignore", [(1, False), (5, True), (32, False),
                                         (64, True), (5000, False)])
-def test_parity_ragged(oracle, d, cap, ignore):
+def test_parity_ragged(oracle, radius_path, d, cap, ignore):
     rng = np.random.default_rng(31 * d + cap)
     n = 3000
     x = rng.random((n, d), dtype=np.float32)
@@ -105,7 +112,7 @@ def test_parity_ragged(oracle, d, cap, ignore):
     assert (got == want).all()
 
 
-def test_parity_bipartite_with_empty_segments(oracle):
+def test_parity_bipartite_with_empty_segments(oracle, radius_path):
     rng = np.random.default_rng(8)
     x = rng.random((5000, 3), dtype=np.float32)
     y = rng.random((777, 3), dtype=np.float32)
@@ -117,13 +124,55 @@ def test_parity_bipartite_with_empty_segments(oracle):
         assert (got == want).all()
 
 
-def test_strict_inequality_at_the_radius(oracle):
+def test_strict_inequality_at_the_radius(oracle, radius_path):
     # points exactly at distance r are excluded (dist < r*r, strict)
     x = np.array([[0, 0], [3, 4], [5, 0], [0, 4.9999995]], dtype=np.float32)
     y = np.array([[0, 0]], dtype=np.float32)
     got = gpu_radius(x, y, None, None, 5.0, 8)
     want = oracle.radius_op(x, y, None, None, 5.0, 8)
     assert got.tolist() == want.tolist() == [[0, 0], [0, 3]]
+
+
+@pytest.mark.parametrize("d", [2, 3, 5])
+@pytest.mark.parametrize("case", ["offset", "clusters", "non_finite",
+                                  "huge", "dense_early_exit"])
+def test_filter_never_drops_a_neighbour(oracle, radius_path, d, case):
+    # where the split-bf16 pre-filter is least accurate or switched off, and
+    # where queries fill up early and whole waves leave the scan
+    rng = np.random.default_rng(hash((d, case, "radius")) % (2 ** 32))
+    n, m, cap, r = 7000, 900, 16, 0.05
+    ptr_x = np.array([0, 3000, 7000])
+    ptr_y = np.array([0, 500, 900])
+    if case == "offset":
+        x = 300.0 + 0.2 * rng.random((n, d))
+        y = 300.0 + 0.2 * rng.random((m, d))
+    elif case == "clusters":
+        centres = 40.0 * rng.standard_normal((30, d))
+        x = centres[rng.integers(0, 30, n)] + 0.03 * rng.standard_normal((n, d))
+        y = centres[rng.integers(0, 30, m)] + 0.03 * rng.standard_normal((m, d))
+    elif case == "non_finite":
+        x = 0.3 * rng.random((n, d))
+        y = 0.3 * rng.random((m, d))
+        for arr, cnt in ((x, 400), (y, 50)):
+            idx = rng.integers(0, arr.shape[0], cnt)
+            arr[idx, rng.integers(0, d, cnt)] = rng.choice(
+                [np.inf, -np.inf, np.nan, 3e38], cnt)
+    elif case == "huge":
+        x = 1e16 * rng.standard_normal((n, d))
+        y = 1e16 * rng.standard_normal((m, d))
+        y[:60] = x[:60]
+        r = 1e15
+    else:
+        x = 0.1 * rng.random((n, d))
+        y = 0.1 * rng.random((m, d))
+        cap, r = 4, 0.08
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    with np.errstate(all="ignore"):
+        got = gpu_radius(x, y, ptr_x, ptr_y, r, cap)
+        want = oracle.radius_op(x, y, ptr_x, ptr_y, r, cap)
+    assert got.shape == want.shape
+    assert (got == want).all()
 
 
 def test_operator_errors():
