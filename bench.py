@@ -151,6 +151,10 @@ def main():
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the short timings of the other BASELINE "
                          "configurations")
+    ap.add_argument("--extras-only", action="store_true",
+                    help="run only the other BASELINE configurations and "
+                         "print their timings (for kernel traces of those "
+                         "paths)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy three times, so "
                          "that a counter profile of this command can scale "
@@ -168,6 +172,10 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+    if args.extras_only:
+        print(json.dumps({"other_configs":
+                          other_configs(torch, pca, testing, dev)}))
+        return
     data = testing.lidar_scans(0)
     B = data["batch_size"]
     ptr_x = testing.pointers(data["batch_x"], B)

@@ -139,7 +139,6 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   p.k = k;
   p.work_start = work_start;
   p.num_chunks = chunks;
-  p.sample_rows = 0;
   p.tau = tau;
   p.partial = partial;
 
@@ -155,19 +154,6 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
       return launch_knn_mfma_steps<36>(pp, kb, cosine, g, stream);
     return launch_knn_mfma_steps<68>(pp, kb, cosine, g, stream);
   };
-  // Bound-seeding pass over a sample of every segment, worth its share of
-  // the scan once the segments are much longer than the sample.
-  int sample = 4096;
-  if (const char *env = std::getenv("PCA_KNN_SAMPLE"))
-    sample = std::atoi(env);
-  if (sample >= 8 * k && in.n / in.num_segments >= 8 * sample) {
-    KnnMfmaParams sp = p;
-    sp.sample_rows = sample;
-    sp.num_chunks = 1;
-    const hipError_t serr = launch(sp, tiles_bound);
-    if (serr != hipSuccess)
-      return serr;
-  }
   if (time_start)
     (void)hipEventRecord(time_start, stream);
   const hipError_t err = launch(p, grid);

@@ -52,15 +52,6 @@
 // knn_merge_kernel and exchange their pruning bound through `tau` like the
 // slices of the low-dimensional kernels do.
 //
-// Bound-seeding pass (sample_rows > 0): the same kernel scans only every
-// stride-th x row of each segment (about sample_rows of them), keeps no
-// results and posts each query's k-th best sampled distance to `tau`.  The
-// k-th distance within any subset of the candidates bounds the final k-th
-// distance from above, so the slices of the full scan -- each of which would
-// otherwise accept and evaluate exactly its first k candidates and a good
-// many more before its own list is of any use -- start with a bound that
-// only about k * stride candidates per query pass at all.
-//
 // The query operands stay in registers for the whole scan (d/2 + 1 per lane);
 // candidate tiles stream through LDS, double-buffered, with the even and odd
 // components of a row stored as two contiguous halves so that a lane's
@@ -90,7 +81,6 @@ struct KnnMfmaParams {
   int n, m, d, num_segments, k;
   const int *work_start; // [num_segments + 1] first 128-query tile per segment
   int num_chunks;        // slices of every segment's x rows
-  int sample_rows;       // > 0: bound-seeding pass (see above)
   float *tau;            // [m] shared pruning bounds
   double *partial;       // [num_chunks * tiles][k][128] keys
 };
@@ -167,13 +157,9 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   const int seg_len = x_end - x_begin;
   const int chunk_len =
       ((seg_len + p.num_chunks - 1) / p.num_chunks + TR - 1) / TR * TR;
-  // rows are addressed as c_begin + position * stride, position < c_count
-  const int stride = p.sample_rows > 0 ? max(1, seg_len / p.sample_rows) : 1;
-  const int c_begin =
-      p.sample_rows > 0 ? x_begin : min(x_end, x_begin + chunk * chunk_len);
-  const int c_count = p.sample_rows > 0
-                          ? (seg_len + stride - 1) / stride
-                          : min(x_end, c_begin + chunk_len) - c_begin;
+  // the slice: rows c_begin + position, position < c_count
+  const int c_begin = min(x_end, x_begin + chunk * chunk_len);
+  const int c_count = min(x_end, c_begin + chunk_len) - c_begin;
   const int num_steps = (c_count + TR - 1) / TR;
 
   const double eps = (double)(d + 32) * (1.0 / 4194304.0); // (d+32) * 2^-22
@@ -252,7 +238,7 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
 
   auto load_tile = [&](int t) {
     const int pos = t * TR + st_row;
-    const size_t g = (size_t)c_begin + (size_t)pos * stride;
+    const size_t g = (size_t)c_begin + pos;
     raw_real = pos < c_count;
     // (rows past the end and padding components read a clamped address and
     // are masked out later)
@@ -422,7 +408,7 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
             if (idx >= pass0 && idx < pass0 + CAP)
               pairs[wave][idx - pass0] =
                   make_int2(q, pos0 + row < c_count
-                                   ? c_begin + (pos0 + row) * stride
+                                   ? c_begin + pos0 + row
                                    : -1);
             ++idx;
           }
@@ -489,7 +475,7 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
     store_tile(0);
   }
   __syncthreads();
-  sync_bounds(); // what other slices (or the seeding pass) already know
+  sync_bounds(); // what other slices already know
 
   // steps [batch_t0, t] are parked and not yet resolved; the first drains
   // come early (after steps 0, 1 and 3), while the lists are still empty and
@@ -538,8 +524,6 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   }
 
   // ---- results ------------------------------------------------------------
-  if (p.sample_rows > 0)
-    return; // the drains have posted the bounds
   // unite the two half lists of each query: every lane inserts its partner's
   // keys (all read before any list changes)
   double theirs[K];
