@@ -435,6 +435,39 @@ def test_config4_feature_space_reduced(oracle):
         assert (e == want).all()
 
 
+@pytest.mark.parametrize("cosine", [False, True])
+def test_config4_feature_space_full_size(oracle, cosine):
+    # 200,000 x 128 against 50,000 queries, k = 32: size-independent
+    # properties at full size, exact parity on a strided sample of the queries
+    data = testing.feature_space(0)
+    x, y = data["x"], data["y"]
+    e = pca.knn(x.to(DEV), y.to(DEV), 32, cosine=cosine).cpu().numpy()
+    m, n = y.shape[0], x.shape[0]
+    assert e.shape == (2, 32 * m)
+    assert (e[0] == np.repeat(np.arange(m), 32)).all()
+    cols = e[1].reshape(m, 32)
+    assert cols.min() >= 0 and cols.max() < n
+    # 32 different rows per query
+    assert (np.diff(np.sort(cols, axis=1), axis=1) > 0).all()
+    sample = np.arange(0, m, 250)
+    xs, ys = x.numpy().astype(np.float64), y.numpy()[sample].astype(np.float64)
+    if cosine:
+        xs = xs / np.linalg.norm(xs, axis=1, keepdims=True)
+        ys = ys / np.linalg.norm(ys, axis=1, keepdims=True)
+        dist = 1.0 - ys @ xs.T
+    else:
+        dist = ((ys ** 2).sum(1)[:, None] + (xs ** 2).sum(1)[None, :]
+                - 2.0 * ys @ xs.T)
+    got = np.take_along_axis(dist, cols[sample], 1)
+    # ascending, and nothing left out is closer than the k-th returned
+    assert (np.diff(got, axis=1) >= -1e-5).all()
+    kth = np.partition(dist, 31, axis=1)[:, 31]
+    assert (got[:, -1] <= kth + 1e-5).all()
+    want, _ = oracle_knn_edges(oracle, x.numpy(), y.numpy()[sample], None,
+                               None, 32, cosine)
+    assert (cols[sample] == want[1].reshape(len(sample), 32)).all()
+
+
 def test_config5_ragged_lidar_full_size(oracle):
     data = testing.lidar_scans(0)
     x, y = data["x"], data["y"]
