@@ -45,10 +45,10 @@
 // (columns j): lane l supplies A[l%32][2s + l/32] and B[2s + l/32][l%32] for
 // step s, and receives, in 16 accumulator registers, the results of query
 // l%32 against the 16 candidate rows 8*(v/4) + 4*(l/32) + v%4.  So lanes l and
-// l+32 share a query and split its candidates: each keeps its own sorted list
-// (its rows arrive in ascending order, so its own k-th distance is a strict
-// bound), the two exchange their k-th distances after every drain, and the
-// lists are united at the end.  The lists of a query's slices are merged by
+// l+32 share a query and split its candidates; the lower lane keeps the
+// query's list and collects the keys of both lanes' rows in ascending row
+// order (so the list's k-th distance is a strict bound), the upper lane
+// filters with the same bound.  The lists of a query's slices are merged by
 // knn_merge_kernel and exchange their pruning bound through `tau` like the
 // slices of the low-dimensional kernels do.
 //
@@ -314,23 +314,25 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   // ---- dense re-rank ------------------------------------------------------
   int qn = 0; // parked steps of this lane: queue[0 .. qn)[tid]
 
-  // -> true and the next parked row of this lane (relative to the batch's
-  // first row) if one is left
-  auto walk_next = [&](MfmaWalk &w, int &row) {
-    if (w.pending == 0 && w.taken < qn) {
-      const uint32_t word = queue[w.taken][tid];
+  // The next parked row of queue column `column` (relative to the batch's
+  // first row; row0 = first row of that lane within a step), or kNoRow.
+  constexpr int kNoRow = 1 << 30;
+  auto peek = [&](MfmaWalk &w, int column, int entries, int row0) {
+    if (w.pending == 0 && w.taken < entries) {
+      const uint32_t word = queue[w.taken][column];
       ++w.taken;
       w.pending = word & 0xffffu;
-      w.base = (int)(word >> 16) * TR + 4 * half;
+      w.base = (int)(word >> 16) * TR + row0;
     }
-    const bool has = w.pending != 0;
+    if (w.pending == 0)
+      return kNoRow;
     // bit 15 - v of the mask stands for accumulator v = row
     // 8 (v / 4) + v % 4 of the lane's rows: highest bit first
-    const int bit = 31 - __builtin_clz(has ? w.pending : 1u);
-    const int v = 15 - bit;
-    w.pending &= ~(1u << bit);
-    row = w.base + 2 * (v & 12) + (v & 3);
-    return has;
+    const int v = 15 - (31 - __builtin_clz(w.pending));
+    return w.base + 2 * (v & 12) + (v & 3);
+  };
+  auto pop = [&](MfmaWalk &w) { // (only after a successful peek)
+    w.pending &= ~(1u << (31 - __builtin_clz(w.pending)));
   };
 
   auto exact_distance = [&](int qq, int g) {
@@ -392,6 +394,14 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
     }
     const int total = __shfl(offset, kWave - 1);
     offset -= count;
+    // the lower lane of a pair collects the keys of both lanes
+    const auto qn_both = __builtin_amdgcn_permlane32_swap(
+        (unsigned)qn, (unsigned)qn, false, false);
+    const auto off_both = __builtin_amdgcn_permlane32_swap(
+        (unsigned)offset, (unsigned)offset, false, false);
+    const int qn_upper = (int)qn_both[1];
+    const int offset_upper = (int)off_both[1];
+    const bool owner = half == 0 && active;
     bool changed = false; // wave-uniform
 
     for (int pass0 = 0; pass0 < total; pass0 += CAP) {
@@ -400,16 +410,16 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
         MfmaWalk w{0, 0u, 0};
         int idx = offset;
         for (;;) {
-          int row;
-          const bool has = walk_next(w, row);
+          const int row = peek(w, tid, qn, 4 * half);
+          const bool has = row != kNoRow;
           if (!__any(has))
             break;
           if (has) {
+            pop(w);
             if (idx >= pass0 && idx < pass0 + CAP)
               pairs[wave][idx - pass0] =
-                  make_int2(q, pos0 + row < c_count
-                                   ? c_begin + pos0 + row
-                                   : -1);
+                  make_int2(q, pos0 + row < c_count ? c_begin + pos0 + row
+                                                    : -1);
             ++idx;
           }
         }
@@ -429,26 +439,43 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      // 3. every lane collects the keys of its own rows, in order
+      // 3. the lower lane of every pair takes the keys of both lanes' rows,
+      // in ascending row order
       {
-        MfmaWalk w{0, 0u, 0};
-        int idx = offset;
+        MfmaWalk lo{0, 0u, 0}, hi{0, 0u, 0};
+        int idx_lo = offset, idx_hi = offset_upper;
         for (;;) {
-          int row;
-          const bool has = walk_next(w, row);
+          int idx = -1;
+          bool has = false;
+          if (owner) {
+            const int a = peek(lo, tid, qn, 0);
+            const int b = peek(hi, tid + 32, qn_upper, 4);
+            has = min(a, b) != kNoRow;
+            if (has) {
+              if (a <= b) {
+                pop(lo);
+                idx = idx_lo++;
+              } else {
+                pop(hi);
+                idx = idx_hi++;
+              }
+            }
+          }
           if (!__any(has))
             break;
           const bool mine = has && idx >= pass0 && idx < pass0 + CAP;
           const double key = mine ? results[wave][idx - pass0] : empty_key();
-          if (has)
-            ++idx;
           // NaN and sentinel distances fail the compare like in the
-          // reference (csrc/cuda/knn_cuda.cu:48,68)
-          const bool ok = mine && key_dist(key) < thresh;
+          // reference (csrc/cuda/knn_cuda.cu:48,68).  Equality passes: a
+          // pass boundary can separate the two lanes' rows, so a row may
+          // arrive after higher rows of its partner -- the key order
+          // settles ties.
+          const bool ok = mine && key_dist(key) <= thresh &&
+                          key_dist(key) < kKnnSentinel;
           if (!__any(ok))
             continue;
           sorted_insert<K>(best, ok ? key : empty_key());
-          if (active)
+          if (owner)
             thresh = __builtin_fminf(key_dist(best[K - 1]), shared);
           changed = true;
         }
@@ -456,18 +483,13 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
       __builtin_amdgcn_wave_barrier();
     }
     qn = 0;
-    if (changed) {
-      // the partner's k-th distance bounds the query's final k-th distance
-      // too (equality admitted: its rows interleave with this lane's)
-      const float own = key_dist(best[K - 1]);
-      const auto both = __builtin_amdgcn_permlane32_swap(
-          __float_as_uint(own), __float_as_uint(own), false, false);
-      const float partner = __uint_as_float(half ? both[0] : both[1]);
-      if (active && partner < kKnnSentinel && !(partner < 0.0f))
-        shared = __builtin_fminf(shared, next_up_positive(partner));
-      set_thresh(__builtin_fminf(thresh, shared));
-    }
     sync_bounds();
+    // both lanes of a pair filter with the list's bound
+    const auto t_both = __builtin_amdgcn_permlane32_swap(
+        __float_as_uint(thresh), __float_as_uint(thresh), false, false);
+    const float pair_thresh = __uint_as_float(t_both[0]);
+    if (changed || pair_thresh < thresh)
+      set_thresh(__builtin_fminf(thresh, pair_thresh));
   };
 
   if (num_steps > 0) {
@@ -524,25 +546,6 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   }
 
   // ---- results ------------------------------------------------------------
-  // unite the two half lists of each query: every lane inserts its partner's
-  // keys (all read before any list changes)
-  double theirs[K];
-#pragma unroll
-  for (int j = 0; j < K; ++j) {
-    const auto hi = __builtin_amdgcn_permlane32_swap(
-        (unsigned)__double2hiint(best[j]), (unsigned)__double2hiint(best[j]),
-        false, false);
-    const auto lo = __builtin_amdgcn_permlane32_swap(
-        (unsigned)__double2loint(best[j]), (unsigned)__double2loint(best[j]),
-        false, false);
-    theirs[j] = half ? __hiloint2double((int)hi[0], (int)lo[0])
-                     : __hiloint2double((int)hi[1], (int)lo[1]);
-  }
-#pragma unroll
-  for (int j = 0; j < K; ++j)
-    if (j >= K - k) // slots below are padding, not keys
-      sorted_insert<K>(best, theirs[j]);
-
   if (half == 0) {
     const size_t list = (size_t)chunk * total_tiles + tile;
     double *dst = p.partial + list * k * TQ + wave * 32 + col;
