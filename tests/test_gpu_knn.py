@@ -79,9 +79,17 @@ def test_knn_graph_large_vs_ckdtree():
 
 # ---- bit-exact parity against the oracle -----------------------------------
 
+@pytest.fixture(params=["1", "0"], ids=["matrix_cores", "vector_alu"])
+def lowd_path(request, monkeypatch):
+    # both low-dimensional Euclidean kernels (lists of more than 32 entries
+    # and the cosine distance always run on the vector-ALU kernel)
+    monkeypatch.setenv("PCA_KNN_LOWD_MATRIX_CORES", request.param)
+    return request.param
+
+
 @pytest.mark.parametrize("d", [1, 2, 3, 4, 5, 8])
 @pytest.mark.parametrize("k", [1, 7, 16, 17, 32, 33, 64, 100])
-def test_parity_single_segment(oracle, d, k):
+def test_parity_single_segment(oracle, lowd_path, d, k):
     rng = np.random.default_rng(100 * d + k)
     n = int(rng.choice([1023, 1024, 1025, 2500]))
     m = int(rng.choice([255, 256, 257, 700]))
@@ -96,7 +104,7 @@ def test_parity_single_segment(oracle, d, k):
 
 @pytest.mark.parametrize("d,k,segments", [(3, 5, 2), (3, 21, 16), (2, 16, 7),
                                           (4, 9, 33), (8, 24, 5), (3, 48, 3)])
-def test_parity_ragged_segments(oracle, d, k, segments):
+def test_parity_ragged_segments(oracle, lowd_path, d, k, segments):
     rng = np.random.default_rng(d * 1000 + k * 10 + segments)
     n, m = 6000, 1900
     x = rng.standard_normal((n, d)).astype(np.float32)
@@ -110,7 +118,7 @@ def test_parity_ragged_segments(oracle, d, k, segments):
     assert (gd == wd).all()
 
 
-def test_k_larger_than_segment_and_empty_segments(oracle):
+def test_k_larger_than_segment_and_empty_segments(oracle, lowd_path):
     rng = np.random.default_rng(5)
     x = rng.random((40, 3), dtype=np.float32)
     y = rng.random((600, 3), dtype=np.float32)
@@ -124,7 +132,7 @@ def test_k_larger_than_segment_and_empty_segments(oracle):
     assert (counts[310:599] == 5).all() and counts[599] == 0
 
 
-def test_exact_ties_keep_lowest_rows(oracle):
+def test_exact_ties_keep_lowest_rows(oracle, lowd_path):
     # integer grid: many exactly equal distances; order must be by
     # (distance, row) -- float64 stable brute force is the independent check
     rng = np.random.default_rng(11)
@@ -146,7 +154,7 @@ def test_duplicate_points(oracle):
     assert (gd == 0).all()
 
 
-def test_sentinel_and_nan_candidates(oracle):
+def test_sentinel_and_nan_candidates(oracle, lowd_path):
     # distance >= 1e10 or NaN is never returned
     # (csrc/cuda/knn_cuda.cu:48,68 in the reference)
     x = np.array([[0.0, 0.0], [1.0, 0.0], [2e5, 0.0], [np.nan, 0.0],
@@ -199,7 +207,7 @@ def test_parity_high_dimension(oracle, d, k, cosine):
                                  (128, 32)])
 @pytest.mark.parametrize("case", ["offset", "huge", "tiny", "mixed_scale",
                                   "clustered"])
-def test_prefilter_never_drops_a_neighbour(oracle, d, k, case):
+def test_prefilter_never_drops_a_neighbour(oracle, lowd_path, d, k, case):
     # the expanded-form pre-filter must stay conservative where it is least
     # accurate: tight clusters far from the origin, coordinates near the
     # overflow / underflow ends of fp32, wildly mixed scales
@@ -323,6 +331,7 @@ def test_cosine_prefilter_never_drops_a_neighbour(oracle, d, k, case):
 
 
 def test_two_queries_per_lane_path(oracle, monkeypatch):
+    monkeypatch.setenv("PCA_KNN_LOWD_MATRIX_CORES", "0")
     rng = np.random.default_rng(77)
     x = rng.random((5000, 3), dtype=np.float32)
     y = rng.random((1500, 3), dtype=np.float32)
@@ -336,14 +345,18 @@ def test_two_queries_per_lane_path(oracle, monkeypatch):
 
 
 @pytest.mark.parametrize("slices", [1, 2, 3, 5, 8, 16])
-@pytest.mark.parametrize("qpt", ["1", "2"])
+@pytest.mark.parametrize("qpt", ["1", "2", "matrix_cores"])
 def test_sliced_segments_merge_exactly(oracle, monkeypatch, slices, qpt):
     # every segment's x rows cut into `slices` parts that share pruning
     # bounds and are merged by key: same bits as the unsliced scan, including
     # exact distance ties across slices (integer grid) and slices shorter
     # than k
     monkeypatch.setenv("PCA_KNN_SLICES", str(slices))
-    monkeypatch.setenv("PCA_KNN_QUERIES_PER_LANE", qpt)
+    if qpt == "matrix_cores":
+        monkeypatch.setenv("PCA_KNN_LOWD_MATRIX_CORES", "1")
+    else:
+        monkeypatch.setenv("PCA_KNN_LOWD_MATRIX_CORES", "0")
+        monkeypatch.setenv("PCA_KNN_QUERIES_PER_LANE", qpt)
     rng = np.random.default_rng(slices)
     x = rng.integers(0, 7, (9000, 3)).astype(np.float32)
     y = rng.integers(0, 7, (1100, 3)).astype(np.float32)
