@@ -66,8 +66,8 @@ namespace pca {
 
 constexpr int kMfmaQueries = 128;   // queries per workgroup
 constexpr int kMfmaRows = 32;       // candidates per step
-constexpr int kMfmaDrainSteps = 8;  // steps between drains (= queue entries)
-constexpr int kMfmaPassPairs = 128; // pairs a wave evaluates per pass
+constexpr int kMfmaDrainSteps = 16; // steps between drains (= queue entries)
+constexpr int kMfmaPassPairs = 256; // pairs a wave evaluates per pass
 
 typedef float mfma_acc_t __attribute__((ext_vector_type(16)));
 
