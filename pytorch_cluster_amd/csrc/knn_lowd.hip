@@ -45,12 +45,12 @@ __global__ __launch_bounds__(kBlock) void fill_f32_kernel(float *p, int n,
 template <int KB>
 void launch_merge(const KnnLowdParams &p, int tile_queries, int tiles_bound,
                   hipStream_t stream) {
+  if (tile_queries == kMcQueries) {
+    hipLaunchKernelGGL((knn_merge_kernel<KB, kMcQueries>), dim3(tiles_bound),
+                       dim3(kBlock), 0, stream, p);
+    return;
+  }
   if constexpr (KB <= 32) {
-    if (tile_queries == kMcQueries) {
-      hipLaunchKernelGGL((knn_merge_kernel<KB, kMcQueries>), dim3(tiles_bound),
-                         dim3(kBlock), 0, stream, p);
-      return;
-    }
     if (tile_queries == 2 * kBlock) {
       hipLaunchKernelGGL((knn_merge_kernel<KB, 2 * kBlock>), dim3(tiles_bound),
                          dim3(kBlock), 0, stream, p);
@@ -82,6 +82,8 @@ KnnLowdConfig knn_lowd_config(int /*d*/, int k, int n, int m,
   cfg.queries_per_lane = qpt;
   cfg.tile_queries = kBlock * qpt;
   // Euclidean lists of up to 32 entries: pre-filter on the matrix cores
+  // (longer lists were tried there too: three to four times slower than the
+  // vector-ALU kernel, whose queues hold single candidates)
   cfg.matrix_cores = !cosine && cfg.kbucket <= 32 &&
                      env_int("PCA_KNN_LOWD_MATRIX_CORES", 1) != 0;
   if (cfg.matrix_cores) {
