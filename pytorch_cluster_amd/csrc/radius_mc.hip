@@ -41,11 +41,11 @@ bool radius_mc_supported(int d, int n, int m, int num_segments) {
     if (env[0] == '1')
       return true;
   }
-  // one workgroup per 128 queries scans a whole segment: worth it once there
-  // are enough of them to fill the chip (the wave-per-query kernel of
-  // radius.hip spreads a small problem over more workgroups)
+  // one workgroup per 128 queries scans a whole segment; measured faster
+  // than the wave-per-query kernel of radius.hip from 128 workgroups on
+  // (half a workgroup per CU), the small problems below stay there
   (void)n;
-  return plan_upper_bound(m, num_segments, kRadiusMcTileQueries) >= 512;
+  return plan_upper_bound(m, num_segments, kRadiusMcTileQueries) >= 64;
 }
 
 size_t radius_mc_scratch_bytes(int n, int d) {
