@@ -162,8 +162,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not "
-                 "supported (the path shards by segment without "
-                 "communication, see DESIGN.md)" % args.gpus)
+                 "supported (the path would shard by segment, without "
+                 "communication)" % args.gpus)
 
     import torch
     import pytorch_cluster_amd as pca

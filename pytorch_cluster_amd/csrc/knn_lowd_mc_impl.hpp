@@ -514,7 +514,10 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
               ((uint32_t)rt << 16) | mask;
           qnext += QROW;
         }
-        if (__any(qnext >= qfirst + QCAP * QROW))
+        // (the first drains of a scan come early -- after steps 0, 1 and 3
+        // -- while the lists are empty and every row passes)
+        if (__any(qnext >= qfirst + QCAP * QROW) ||
+            (t == 0 && (rt <= 1 || rt == 3)))
           drain(g_base, rows);
       }
     }
