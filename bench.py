@@ -89,7 +89,7 @@ def cpu_baseline(data, ptr_x, ptr_y):
 
 
 def other_configs(torch, pca, testing, dev):
-    """End-to-end times of the other BASELINE configurations (median of a few
+    """End-to-end times of the other benchmark configurations (median of a few
     calls, inputs resident in HBM); reported beside the headline number, they
     are parity-test cases, not the benchmark."""
     def median_ms(fn, reps):
@@ -149,10 +149,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
-                    help="skip the short timings of the other BASELINE "
+                    help="skip the short timings of the other benchmark "
                          "configurations")
     ap.add_argument("--extras-only", action="store_true",
-                    help="run only the other BASELINE configurations and "
+                    help="run only the other benchmark configurations and "
                          "print their timings (for kernel traces of those "
                          "paths)")
     ap.add_argument("--copy-calibration", action="store_true",

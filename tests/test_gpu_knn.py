@@ -416,7 +416,7 @@ def test_runs_on_the_current_stream(oracle):
     assert (e.cpu().numpy() == want).all()
 
 
-# ---- BASELINE configurations -----------------------------------------------
+# ---- the benchmark configurations -----------------------------------------------
 
 def test_config1_knn_graph_1024(oracle):
     data = testing.uniform_cloud(0)

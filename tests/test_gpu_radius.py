@@ -186,7 +186,7 @@ def test_operator_errors():
         op(x, x.cpu(), None, None, 1.0, 4, 1, False)
 
 
-# ---- BASELINE configuration 3 ------------------------------------------------
+# ---- benchmark configuration 3 -------------------------------------------------
 
 def test_config3_gaussian_mixture_radius_graph(oracle):
     data = testing.gaussian_mixture_batched(0)
