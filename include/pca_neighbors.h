@@ -75,7 +75,8 @@ const char *pca_status_string(int status);
 const char *pca_last_error(void);
 
 /*
- * Measurement hook: the next pca_knn / pca_radius call of the calling thread
+ * Measurement hook: the next pca_knn / pca_radius / pca_nearest call of the
+ * calling thread
  * records `start_event` immediately before and `stop_event` immediately after
  * its search kernel (the dominant kernel; planning and compaction kernels stay
  * outside) on that call's stream.  Both are hipEvent_t created by the caller
@@ -148,6 +149,39 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
                int ignore_same_index, int dtype, int64_t *edges,
                int64_t *num_edges, void *workspace, size_t workspace_bytes,
                void *stream);
+
+/* -------------------------------------------------------------- nearest -- */
+
+/*
+ * NOTE the roles: as in the reference operator, here the rows of x SEARCH and
+ * the rows of y ARE SEARCHED (the opposite of pca_knn / pca_radius).
+ *   x      [n, d] rows that look for their nearest row of y
+ *   y      [m, d] candidates
+ *   ptr_x  [num_segments + 1] segments of x, ptr_y those of y (as above;
+ *          every row of x must lie in a segment: ptr_x[last] = n)
+ *   out    [n] int64: for every row of x the global number of the row of y
+ *          of the same segment with the smallest squared distance.
+ *
+ * Stands under the reference operator
+ *   torch_cluster::nearest(x, y, ptr_x, ptr_y)
+ *   csrc/nearest.cpp:22-39 -> nearest_cuda, csrc/cuda/nearest_cuda.cu:68-94
+ * and reproduces nearest_kernel (csrc/cuda/nearest_cuda.cu:10-66) including
+ * its two corner rules: a candidate counts only if its distance is strictly
+ * below 1e38 (narrowed to the element type: +inf for fp16), and a row with no
+ * such candidate (empty segment of y, NaN, overflow) gets 0; among candidates
+ * of equal distance the one with the smallest (row - segment start) % 1024
+ * wins, then the smallest row (what that kernel's block of 1,024 threads and
+ * its pairwise reduction return).
+ * dtype: PCA_F32, PCA_F64 or PCA_F16 (the types the reference instantiates,
+ * csrc/cuda/nearest_cuda.cu:85); PCA_BF16 returns PCA_ERR_UNSUPPORTED.
+ */
+size_t pca_nearest_workspace_bytes(int64_t n, int64_t m, int64_t d,
+                                   int64_t num_segments, int dtype);
+
+int pca_nearest(const void *x, const void *y, const int64_t *ptr_x,
+                const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+                int64_t num_segments, int dtype, int64_t *out,
+                void *workspace, size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -249,6 +249,80 @@ def radius_op16(x_bits, y_bits, ptr_x, ptr_y, r, max_num_neighbors,
 
 
 # --------------------------------------------------------------------------
+# nearest (csrc/cuda/nearest_cuda.cu, torch_cluster/nearest.py)
+# --------------------------------------------------------------------------
+
+def nearest_op(x, y, ptr_x, ptr_y, fma_mode=1):
+    """``torch_cluster::nearest`` (csrc/cuda/nearest_cuda.cu:68-94): for every
+    row of ``x`` the row of ``y`` of its example that is nearest.  ``x``/``y``
+    float32 or float64 arrays, or uint16 / float16 arrays for IEEE half."""
+    lib = _load()
+    x, y = np.ascontiguousarray(x), np.ascontiguousarray(y)
+    # x.view({x.size(0), -1}) (:76-77)
+    x = x.reshape(x.shape[0], -1)
+    y = y.reshape(y.shape[0], -1)
+    if x.dtype != y.dtype or x.shape[1] != y.shape[1]:
+        raise RuntimeError("Input mismatch")
+    ptr_x, ptr_y = _as_ptr(ptr_x), _as_ptr(ptr_y)
+    nseg = ptr_x.size - 1
+    out = np.empty(x.shape[0], dtype=np.int64)
+    if x.dtype == np.float16:
+        x, y = x.view(np.uint16), y.view(np.uint16)
+    if x.dtype == np.uint16:
+        fn, mode = lib.oracle_nearest_16, 0
+    elif x.dtype in _DTYPE_CODE:
+        fn, mode = getattr(lib, "oracle_nearest_" + _suffix(x.dtype)), fma_mode
+    else:
+        raise TypeError(f"oracle nearest: unsupported dtype {x.dtype}")
+    rc = fn(_ptr(x), _ptr(y), _ptr(ptr_x), _ptr(ptr_y),
+            ctypes.c_int64(x.shape[0]), ctypes.c_int64(y.shape[0]),
+            ctypes.c_int64(x.shape[1]), ctypes.c_int64(nseg),
+            ctypes.c_int(int(mode)), _ptr(out))
+    if rc != 0:
+        raise RuntimeError("a row of x lies in no example of ptr_x")
+    return out
+
+
+def _counts_to_ptr(batch):
+    """torch_cluster/nearest.py:57-63: scatter_add of ones, then cumsum."""
+    batch = np.asarray(batch, dtype=np.int64)
+    batch_size = int(batch.max()) + 1
+    deg = np.bincount(batch, minlength=batch_size)
+    return np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+
+
+def nearest(x, y, batch_x=None, batch_y=None, fma_mode=1):
+    """The GPU branch of torch_cluster/nearest.py:7-91."""
+    x, y = np.asarray(x), np.asarray(y)
+    x = x.reshape(-1, 1) if x.ndim == 1 else x
+    y = y.reshape(-1, 1) if y.ndim == 1 else y
+    assert x.shape[1] == y.shape[1]
+    if batch_x is not None and (np.diff(np.asarray(batch_x)) < 0).any():
+        raise ValueError("'batch_x' is not sorted")
+    if batch_y is not None and (np.diff(np.asarray(batch_y)) < 0).any():
+        raise ValueError("'batch_y' is not sorted")
+    if batch_x is not None:
+        assert x.shape[0] == np.asarray(batch_x).size
+        ptr_x = _counts_to_ptr(batch_x)
+    else:
+        ptr_x = np.array([0, x.shape[0]], dtype=np.int64)
+    if batch_y is not None:
+        assert y.shape[0] == np.asarray(batch_y).size
+        ptr_y = _counts_to_ptr(batch_y)
+    else:
+        ptr_y = np.array([0, y.shape[0]], dtype=np.int64)
+    # an example that is non-empty in x must be non-empty in y (:80-86);
+    # torch.equal is False for different shapes
+    nonempty_x = np.diff(ptr_x) > 0
+    nonempty_y = np.diff(ptr_y) > 0
+    if nonempty_x.shape != nonempty_y.shape or \
+            not np.array_equal(nonempty_x, nonempty_y):
+        raise ValueError("Some batch indices occur in 'batch_x' "
+                         "that do not occur in 'batch_y'")
+    return nearest_op(x, y, ptr_x, ptr_y, fma_mode)
+
+
+# --------------------------------------------------------------------------
 # Python entry points (torch_cluster/knn.py, torch_cluster/radius.py)
 # --------------------------------------------------------------------------
 

@@ -17,6 +17,12 @@
  *   oracle_compact         csrc/cuda/knn_cuda.cu:133-134 and
  *                          csrc/cuda/radius_cuda.cu:94-95 (mask on -1, two
  *                          masked_selects, stack)
+ *   oracle_nearest_*       csrc/cuda/nearest_cuda.cu:10-66 (nearest_kernel):
+ *                          the block of 1,024 threads is played through
+ *                          literally -- strided scan per thread (:31-44),
+ *                          then the pairwise reduction over shared memory
+ *                          (:46-59) -- so that the candidate chosen among
+ *                          equal distances is the reference's
  *
  * Arithmetic: `fma_mode` = 1 evaluates every `acc += a * b` of the reference
  * kernels as one fused multiply-add (what a GPU compiler emits for that
@@ -29,7 +35,11 @@
  * test/test_knn.py:16-52,57-75, test/test_radius.py:25-116, the ordered README
  * outputs README.md:188-191,217-220, the reference's compiled CPU operators
  * (oracle/_ref), scipy's cKDTree as in test/test_knn.py:84-88 and
- * test/test_radius.py:129-133, and float64 brute force.
+ * test/test_radius.py:129-133, and float64 brute force.  oracle_nearest_*:
+ * the fixture test/test_nearest.py:11-35, scipy.cluster.vq.vq (the
+ * reference's own CPU route, torch_cluster/nearest.py:122-124), float64
+ * brute force, and a closed form of the tie rule (smallest distance, then
+ * smallest (row - segment start) % 1024, then smallest row).
  */
 #include <math.h>
 #include <stdint.h>
@@ -199,6 +209,97 @@ static int64_t example_idx(int64_t idx, const int64_t *ptr,
 
 DEFINE_ORACLE(f32, float, fmaf, sqrtf)
 DEFINE_ORACLE(f64, double, fma, sqrt)
+
+/* ------------------------------------------------------------------------
+ * nearest_kernel (csrc/cuda/nearest_cuda.cu:10-66): for every row of x the
+ * row of y of the same example with the smallest squared distance.  One
+ * block of NEAREST_THREADS threads per x row; thread t looks at the y rows
+ * y_start + t, y_start + t + 1024, ... and keeps the first strictly smaller
+ * distance (:31-44; `best` starts at 1e38 narrowed to scalar_t and
+ * `best_idx` at 0, so a row whose candidates all fail `dist < best` --
+ * NaN, overflow, an empty example of y -- yields index 0); the block then
+ * halves the number of live entries ten times, an entry taking its right
+ * neighbour's value only when that one is strictly smaller (:46-59).
+ * The loops below run in exactly that order.
+ * ------------------------------------------------------------------------ */
+#define NEAREST_THREADS 1024
+
+/* :17-23 -- the example whose range of ptr_x holds the row; -1 if none (the
+ * reference then reads an uninitialised variable). */
+static int64_t nearest_example(int64_t n_x, const int64_t *ptr_x,
+                               int64_t batch_size) {
+  for (int64_t b = 0; b < batch_size; b++) {
+    if (n_x >= ptr_x[b] && n_x < ptr_x[b + 1])
+      return b;
+  }
+  return -1;
+}
+
+#define DEFINE_NEAREST(SUFFIX, T, XT, DIST_EXPR, LIMIT_EXPR)                   \
+  int oracle_nearest_##SUFFIX(const XT *x, const XT *y, const int64_t *ptr_x,  \
+                              const int64_t *ptr_y, int64_t n, int64_t m,      \
+                              int64_t dim, int64_t batch_size, int mode,       \
+                              int64_t *out) {                                  \
+    int64_t default_ptr_x[2] = {0, n}, default_ptr_y[2] = {0, m};              \
+    if (ptr_x == NULL || ptr_y == NULL) {                                      \
+      ptr_x = default_ptr_x;                                                   \
+      ptr_y = default_ptr_y;                                                   \
+      batch_size = 1;                                                          \
+    }                                                                          \
+    int bad = 0;                                                               \
+    _Pragma("omp parallel") {                                                  \
+      T *best_dist = (T *)malloc(sizeof(T) * NEAREST_THREADS);                 \
+      int64_t *best_dist_idx =                                                 \
+          (int64_t *)malloc(sizeof(int64_t) * NEAREST_THREADS);                \
+      _Pragma("omp for schedule(dynamic, 16)") for (int64_t n_x = 0; n_x < n;  \
+                                                    n_x++) {                   \
+        const int64_t batch_idx = nearest_example(n_x, ptr_x, batch_size);     \
+        if (batch_idx < 0) {                                                   \
+          bad = 1;                                                             \
+          out[n_x] = -1;                                                       \
+          continue;                                                            \
+        }                                                                      \
+        const int64_t y_start_idx = ptr_y[batch_idx];                          \
+        const int64_t y_end_idx = ptr_y[batch_idx + 1];                        \
+        for (int64_t thread_idx = 0; thread_idx < NEAREST_THREADS;             \
+             thread_idx++) {                                                   \
+          T best = (LIMIT_EXPR);                                               \
+          int64_t best_idx = 0;                                                \
+          for (int64_t n_y = y_start_idx + thread_idx; n_y < y_end_idx;        \
+               n_y += NEAREST_THREADS) {                                       \
+            T dist = (DIST_EXPR);                                              \
+            if (dist < best) {                                                 \
+              best = dist;                                                     \
+              best_idx = n_y;                                                  \
+            }                                                                  \
+          }                                                                    \
+          best_dist[thread_idx] = best;                                        \
+          best_dist_idx[thread_idx] = best_idx;                                \
+        }                                                                      \
+        for (int64_t u = 0; (1 << u) < NEAREST_THREADS; u++) {                 \
+          for (int64_t thread_idx = 0;                                         \
+               thread_idx < (NEAREST_THREADS >> (u + 1)); thread_idx++) {      \
+            int64_t idx_1 = (thread_idx * 2) << u;                             \
+            int64_t idx_2 = (thread_idx * 2 + 1) << u;                         \
+            if (best_dist[idx_1] > best_dist[idx_2]) {                         \
+              best_dist[idx_1] = best_dist[idx_2];                             \
+              best_dist_idx[idx_1] = best_dist_idx[idx_2];                     \
+            }                                                                  \
+          }                                                                    \
+        }                                                                      \
+        out[n_x] = best_dist_idx[0];                                           \
+      }                                                                        \
+      free(best_dist);                                                         \
+      free(best_dist_idx);                                                     \
+    }                                                                          \
+    return bad;                                                                \
+  }
+
+/* mode: fma_mode for the float and double versions */
+DEFINE_NEAREST(f32, float, float, sqdist_f32(x, y, n_x, n_y, dim, mode),
+               (float)1e38)
+DEFINE_NEAREST(f64, double, double, sqdist_f64(x, y, n_x, n_y, dim, mode),
+               (double)1e38)
 
 /* ------------------------------------------------------------------------
  * 16-bit element types (IEEE half, bfloat16).
@@ -439,6 +540,12 @@ int oracle_radius_dense_16(const uint16_t *x, const uint16_t *y,
   }
   return 0;
 }
+
+/* nearest_kernel with scalar_t = c10::Half (mode: kind, 0 = IEEE half; the
+ * reference does not instantiate it for bfloat16, csrc/cuda/nearest_cuda.cu:
+ * 87); `best = 1e38` narrows to +inf. */
+DEFINE_NEAREST(16, float, uint16_t, sqdist16(x, y, n_x, n_y, dim, mode),
+               round16(1e38f, mode))
 
 /* Host-wrapper epilogue: keep the slots whose `mask_src` entry is not -1, in
  * slot order, and stack them as [2, E] (row-major, leading dimension E).

@@ -119,3 +119,29 @@ def radius_edges(x, y, ptr_x=None, ptr_y=None, r: float = 1.0,
                                           ignore_same_index, stream)
     e = int(num_edges.item())
     return edges[:2 * e].view(2, e)
+
+
+def nearest_launch(x, y, ptr_x=None, ptr_y=None, stream=None):
+    """Queues ``pca_nearest``: for every row of ``x`` the nearest row of ``y``
+    of the same segment.  Returns (out [n] int64, workspace); nothing is
+    synchronised."""
+    assert x.is_cuda and y.is_cuda and x.is_contiguous() and y.is_contiguous()
+    assert x.dtype == y.dtype and x.dtype in _DTYPE_CODE
+    dtype = _DTYPE_CODE[x.dtype]
+    n, d = x.shape
+    m = y.shape[0]
+    ptr_x, ptr_y, nseg = _segments(ptr_x, ptr_y)
+    ws_bytes = capi.pca_nearest_workspace_bytes(n, m, d, nseg, dtype)
+    if ws_bytes == 0:
+        ws_bytes = 256
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    out = torch.empty(n, dtype=torch.long, device=x.device)
+    _check(capi.pca_nearest(_dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x),
+                            _dev_ptr(ptr_y), n, m, d, nseg, dtype,
+                            _dev_ptr(out), _dev_ptr(ws), ws_bytes,
+                            _stream_handle(stream, x.device)))
+    return out, ws
+
+
+def nearest_rows(x, y, ptr_x=None, ptr_y=None, stream=None) -> torch.Tensor:
+    return nearest_launch(x, y, ptr_x, ptr_y, stream)[0]

@@ -1,7 +1,9 @@
 // kNN and radius search for the element types other than fp32: fp64, fp16,
 // bf16.  Completeness path -- same results as the reference's kernels
 // instantiated for these `scalar_t` (csrc/cuda/knn_cuda.cu:125,
-// csrc/cuda/radius_cuda.cu:84-85), no tuning beyond LDS tiling.
+// csrc/cuda/radius_cuda.cu:84-85), no tuning beyond LDS tiling.  Also the
+// `nearest` search (csrc/cuda/nearest_cuda.cu:10-66) for fp64, fp16 and for
+// fp32 points of more than 8 dimensions.
 //
 // Arithmetic per element type (`Traits`):
 //   fp64        everything in double, `acc += a * b` as one fused multiply-add
@@ -78,7 +80,24 @@ struct F64Traits {
     return 1.0 - dot / (xn * yn);
   }
   static __device__ __forceinline__ calc_t sentinel() { return 1e10; }
+  static __device__ __forceinline__ calc_t nearest_limit() { return 1e38; }
   static calc_t narrow_r2(double r2) { return r2; }
+};
+
+// fp32 with fused multiply-adds (the `nearest` search only; kNN and radius
+// have their own fp32 kernels)
+struct F32Traits {
+  typedef float store_t;
+  typedef float calc_t;
+  static __device__ __forceinline__ calc_t load(store_t v) { return v; }
+  static __device__ __forceinline__ calc_t sq_step(calc_t x, calc_t y,
+                                                   calc_t acc) {
+    const calc_t d = x - y;
+    return __builtin_fmaf(d, d, acc);
+  }
+  static __device__ __forceinline__ calc_t nearest_limit() {
+    return kNearestLimit;
+  }
 };
 
 template <bool BF16> struct R16Traits {
@@ -121,6 +140,10 @@ template <bool BF16> struct R16Traits {
   }
   static __device__ __forceinline__ calc_t sentinel() {
     return round16(1e10f);
+  }
+  // `scalar_t best = 1e38`: +inf in fp16
+  static __device__ __forceinline__ calc_t nearest_limit() {
+    return round16(1e38f);
   }
   // (scalar_t)(r * r): double -> float -> 16 bits
   static calc_t narrow_r2(double r2) {
@@ -333,6 +356,95 @@ __global__ __launch_bounds__(kBlock) void knn_any_kernel(
   }
 }
 
+// The `nearest` search with the mapping of knn_any_kernel: one searching row
+// (a row of y here) per lane, candidates (rows of x) through LDS.  A lane
+// keeps the candidate that is smallest by (distance, (row - start) % 1024,
+// row) -- the one the reference's block reduction returns -- and the result
+// is 0 when no distance is below the limit (csrc/cuda/nearest_cuda.cu:31-64).
+template <typename Tr>
+__global__ __launch_bounds__(kBlock) void nearest_any_kernel(
+    const typename Tr::store_t *__restrict__ x,
+    const typename Tr::store_t *__restrict__ y,
+    const int64_t *__restrict__ ptr_x, const int64_t *__restrict__ ptr_y,
+    int n, int m, int d, int num_segments, const int *__restrict__ work_start,
+    int64_t *__restrict__ out) {
+  typedef typename Tr::calc_t calc_t;
+  constexpr int TG = kAnyTile;
+  __shared__ calc_t xs[TG][kAnySlab];
+
+  const int tid = threadIdx.x;
+  const int tile = blockIdx.x;
+  if (tile >= work_start[num_segments])
+    return;
+  const int seg = find_segment(work_start, num_segments, tile);
+  const int x_begin = ptr_x ? (int)ptr_x[seg] : 0;
+  const int x_end = ptr_x ? (int)ptr_x[seg + 1] : n;
+  const int y_begin = ptr_y ? (int)ptr_y[seg] : 0;
+  const int y_end = ptr_y ? (int)ptr_y[seg + 1] : m;
+  const int q = y_begin + (tile - work_start[seg]) * kBlock + tid;
+  const bool valid = q < y_end;
+  const typename Tr::store_t *yrow = y + (size_t)(valid ? q : y_begin) * d;
+
+  constexpr uint32_t kNone = 0xffffffffu;
+  const calc_t limit = Tr::nearest_limit();
+  calc_t best = limit;
+  uint32_t best_tie = kNone;
+
+  for (int base = x_begin; base < x_end; base += TG) {
+    const int rows = min(TG, x_end - base);
+    calc_t acc[TG];
+#pragma unroll
+    for (int j = 0; j < TG; ++j)
+      acc[j] = 0;
+
+    for (int slab = 0; slab < d; slab += kAnySlab) {
+      const int width = min(kAnySlab, d - slab);
+      __syncthreads();
+      for (int i = tid; i < TG * width; i += kBlock) {
+        const int r = i / width;
+        const int c = i - r * width;
+        xs[r][c] = r < rows ? Tr::load(x[(size_t)(base + r) * d + slab + c])
+                            : (calc_t)0;
+      }
+      __syncthreads();
+
+      for (int c0 = 0; c0 < width; c0 += kAnyChunk) {
+        calc_t yv[kAnyChunk];
+#pragma unroll
+        for (int c = 0; c < kAnyChunk; ++c)
+          yv[c] = (c0 + c < width) ? Tr::load(yrow[slab + c0 + c]) : (calc_t)0;
+        const int count = min(kAnyChunk, width - c0);
+#pragma unroll
+        for (int j = 0; j < TG; ++j) {
+#pragma unroll
+          for (int c = 0; c < kAnyChunk; ++c) {
+            if (c < count)
+              acc[j] = Tr::sq_step(xs[j][c0 + c], yv[c], acc[j]);
+          }
+        }
+      }
+    }
+
+#pragma unroll
+    for (int j = 0; j < TG; ++j) {
+      if (j < rows) { // uniform
+        const calc_t dist = acc[j];
+        const uint32_t tie = nearest_tie((uint32_t)(base + j - x_begin));
+        // (best < limit exactly when a candidate has been kept)
+        const bool take =
+            dist < limit && (dist < best || (dist == best && tie < best_tie));
+        best = take ? dist : best;
+        best_tie = take ? tie : best_tie;
+      }
+    }
+  }
+
+  if (valid)
+    out[q] = best_tie != kNone
+                 ? (int64_t)x_begin + (int64_t)nearest_rel(best_tie)
+                 : 0;
+}
+
 constexpr int QW = kRadiusQueriesPerWave;
 constexpr int kWavesPerBlock = kBlock / kWave;
 
@@ -482,7 +594,38 @@ hipError_t launch_radius_any_t(const SearchInput &in, double r,
   return hipGetLastError();
 }
 
+template <typename Tr>
+hipError_t launch_nearest_any_t(const SearchInput &in, const int *work_start,
+                                int grid, int64_t *out, hipStream_t stream) {
+  typedef typename Tr::store_t store_t;
+  if (grid <= 0)
+    return hipSuccess;
+  hipLaunchKernelGGL((nearest_any_kernel<Tr>), dim3(grid), dim3(kBlock), 0,
+                     stream, static_cast<const store_t *>(in.x),
+                     static_cast<const store_t *>(in.y), in.ptr_x, in.ptr_y,
+                     in.n, in.m, in.d, in.num_segments, work_start, out);
+  return hipGetLastError();
+}
+
 } // namespace
+
+hipError_t launch_nearest_any(int dtype, const SearchInput &in,
+                              const int *work_start, int grid_bound,
+                              int64_t *out, hipStream_t stream) {
+  switch (dtype) {
+  case 0:
+    return launch_nearest_any_t<F32Traits>(in, work_start, grid_bound, out,
+                                           stream);
+  case 1:
+    return launch_nearest_any_t<F64Traits>(in, work_start, grid_bound, out,
+                                           stream);
+  case 2:
+    return launch_nearest_any_t<R16Traits<false>>(in, work_start, grid_bound,
+                                                  out, stream);
+  default:
+    return hipErrorInvalidValue;
+  }
+}
 
 size_t anytype_norm_bytes(int n) { return sizeof(double) * (size_t)n; }
 

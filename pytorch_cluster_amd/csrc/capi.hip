@@ -64,6 +64,12 @@ struct Carver {
 
 __global__ void set_i64_kernel(int64_t *p, int64_t v) { *p = v; }
 
+__global__ void fill_i64_kernel(int64_t *p, int64_t count, int64_t v) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count)
+    p[i] = v;
+}
+
 constexpr int64_t kMaxRows = 2147483646; // n, m < 2^31 - 1
 
 bool sizes_ok(int64_t n, int64_t m, int64_t d, int64_t num_segments) {
@@ -131,6 +137,25 @@ size_t radius_workspace(int64_t n, int64_t m, int64_t d, int64_t num_segments,
   bytes += align256(sizeof(int) * (size_t)m * (size_t)slots);
   bytes += align256(sizeof(int) * (size_t)m);
   bytes += pca::compact_workspace_bytes((int)m);
+  return bytes;
+}
+
+bool nearest_dtype_ok(int dtype) {
+  return dtype == PCA_F32 || dtype == PCA_F64 || dtype == PCA_F16;
+}
+
+// (searching rows n, candidates m)
+bool nearest_low_d(int64_t d, int dtype) { return dtype == PCA_F32 && d <= 8; }
+
+size_t nearest_workspace(int64_t n, int64_t m, int64_t d,
+                         int64_t num_segments, int dtype) {
+  size_t bytes = align256(sizeof(int) * (size_t)(num_segments + 1));
+  if (nearest_low_d(d, dtype)) {
+    const pca::KnnLowdConfig cfg =
+        pca::nearest_lowd_config((int)d, (int)m, (int)n, (int)num_segments);
+    bytes += pca::knn_lowd_scratch_bytes(cfg, (int)m, (int)n, (int)d,
+                                         (int)num_segments, 1);
+  }
   return bytes;
 }
 
@@ -429,6 +454,93 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
   return check_launch(pca::launch_compact(dense, (int)m, edges, num_edges,
                                           nullptr, compact_ws, stream),
                       "compaction kernels");
+}
+
+size_t pca_nearest_workspace_bytes(int64_t n, int64_t m, int64_t d,
+                                   int64_t num_segments, int dtype) {
+  if (num_segments < 1)
+    num_segments = 1;
+  if (!sizes_ok(n, m, d, num_segments) || !nearest_dtype_ok(dtype))
+    return 0;
+  return nearest_workspace(n, m, d, num_segments, dtype);
+}
+
+int pca_nearest(const void *x, const void *y, const int64_t *ptr_x,
+                const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+                int64_t num_segments, int dtype, int64_t *out,
+                void *workspace, size_t workspace_bytes, void *stream_) {
+  g_last_error[0] = 0;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  SearchTimer timer(stream);
+  if ((ptr_x == nullptr) != (ptr_y == nullptr))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "ptr_x and ptr_y must both be given or both be NULL");
+  if (ptr_x == nullptr)
+    num_segments = 1;
+  if (!sizes_ok(n, m, d, num_segments))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "bad sizes n=%lld m=%lld d=%lld num_segments=%lld",
+                (long long)n, (long long)m, (long long)d,
+                (long long)num_segments);
+  if (!dtype_ok(dtype))
+    return fail(PCA_ERR_INVALID_ARGUMENT, "unknown element type %d", dtype);
+  if (!nearest_dtype_ok(dtype))
+    return fail(PCA_ERR_UNSUPPORTED,
+                "nearest is built for fp32, fp64 and fp16 points");
+  if (n == 0)
+    return PCA_OK;
+  if (out == nullptr || x == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "x or out is NULL");
+  if (m == 0) {
+    // no candidate anywhere: every row keeps the reference's initial index
+    hipLaunchKernelGGL(fill_i64_kernel, dim3((unsigned)((n + 255) / 256)),
+                       dim3(256), 0, stream, out, n, (int64_t)0);
+    return check_launch(hipGetLastError(), "fill_i64_kernel");
+  }
+  if (y == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "y is NULL");
+  const size_t need = nearest_workspace(n, m, d, num_segments, dtype);
+  if (workspace == nullptr || ((uintptr_t)workspace & 255) != 0 ||
+      workspace_bytes < need)
+    return fail(PCA_ERR_WORKSPACE, "workspace needs %zu bytes, 256-aligned",
+                need);
+
+  // the search kernels call the searched rows x and the searching rows y
+  pca::SearchInput in{y,      x,      ptr_y,  ptr_x,
+                      (int)m, (int)n, (int)d, (int)num_segments};
+  Carver ws(workspace);
+  int *work_start = ws.take<int>((size_t)num_segments + 1);
+  const bool low_d = nearest_low_d(d, dtype);
+  pca::KnnLowdConfig cfg;
+  int per_item = pca::kBlock;
+  if (low_d) {
+    cfg = pca::nearest_lowd_config((int)d, (int)m, (int)n, (int)num_segments);
+    per_item = cfg.tile_queries;
+  }
+  int rc = check_launch(pca::launch_plan(ptr_x, (int)n, (int)num_segments,
+                                         per_item, work_start, stream),
+                        "plan_kernel");
+  if (rc != PCA_OK)
+    return rc;
+  if (low_d) {
+    void *scratch = ws.take<char>(pca::knn_lowd_scratch_bytes(
+        cfg, (int)m, (int)n, (int)d, (int)num_segments, 1));
+    const pca::DenseResult none{nullptr, nullptr, nullptr, 1};
+    rc = check_launch(pca::launch_knn_lowd(in, 1, false, cfg, work_start,
+                                           scratch, none, timer.start,
+                                           timer.stop, stream, out),
+                      "knn_lowd_mc_kernel (nearest)");
+    timer.stop = nullptr;
+    return rc;
+  }
+  const int bound =
+      pca::plan_upper_bound((int)n, (int)num_segments, per_item);
+  timer.begin();
+  rc = check_launch(pca::launch_nearest_any(dtype, in, work_start, bound, out,
+                                            stream),
+                    "nearest_any_kernel");
+  timer.done();
+  return rc;
 }
 
 } // extern "C"

@@ -60,6 +60,33 @@ __device__ __forceinline__ double empty_key() {
   return __hiloint2double((int)(0x501502F9u /* 1e10f */ + kKeyBias), -1);
 }
 
+// The `nearest` operator (csrc/cuda/nearest_cuda.cu:10-66 in the reference)
+// is a search for one neighbour with two differences: a candidate must be
+// strictly below 1e38 instead of 1e10 (:31,41), and among candidates of equal
+// distance the reference's block of 1,024 threads -- thread t scans the rows
+// start + t, start + t + 1024, ... and keeps its first minimum (:33-44), the
+// pairwise reduction keeps the lower thread on ties (:46-59) -- returns the
+// one with the smallest (row - start) % 1024, then the smallest row.  With
+// that pair in the low word of the key (10 bits of slot, 22 bits of
+// (row - start) / 1024; rows stay below 2^31) the key order is that rule.
+constexpr float kNearestLimit = 1e38f;
+
+__device__ __forceinline__ uint32_t nearest_tie(uint32_t rel) {
+  return ((rel & 1023u) << 22) | (rel >> 10);
+}
+
+__device__ __forceinline__ uint32_t nearest_rel(uint32_t tie) {
+  return ((tie & 0x3fffffu) << 10) | (tie >> 22);
+}
+
+// Limit and empty-slot key of a search: the kNN ones, or those of `nearest`.
+template <bool NEAREST> struct SearchLimit {
+  static constexpr float value = NEAREST ? kNearestLimit : kKnnSentinel;
+  static __device__ __forceinline__ double empty() {
+    return __hiloint2double((int)(__float_as_uint(value) + kKeyBias), -1);
+  }
+};
+
 // Key below every real key: fills the slots of a K-wide list that the caller
 // did not ask for (k < K), so that they never take part in the selection.
 __device__ __forceinline__ double lowest_key() {

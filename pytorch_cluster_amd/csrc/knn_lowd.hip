@@ -105,6 +105,20 @@ KnnLowdConfig knn_lowd_config(int /*d*/, int k, int n, int m,
   if (forced_chunks >= 1 && forced_chunks <= 64)
     chunks = forced_chunks;
   cfg.num_chunks = chunks;
+  cfg.nearest = false;
+  return cfg;
+}
+
+KnnLowdConfig nearest_lowd_config(int d, int n, int m, int num_segments) {
+  // the slices of a one-neighbour kNN search on the matrix cores
+  KnnLowdConfig cfg = knn_lowd_config(d, 1, n, m, num_segments, false);
+  if (!cfg.matrix_cores) {
+    cfg.matrix_cores = true; // the only kernel with the `nearest` rules
+    cfg.queries_per_lane = 1;
+    cfg.tile_queries = kMcQueries;
+  }
+  cfg.kbucket = 1;
+  cfg.nearest = true;
   return cfg;
 }
 
@@ -167,7 +181,7 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
                            const KnnLowdConfig &cfg, const int *work_start,
                            void *scratch, const DenseResult &out,
                            hipEvent_t time_start, hipEvent_t time_stop,
-                           hipStream_t stream) {
+                           hipStream_t stream, int64_t *nearest_out) {
   const int tiles_bound =
       plan_upper_bound(in.m, in.num_segments, cfg.tile_queries);
   KnnLowdParams p;
@@ -187,6 +201,7 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
   p.out_idx = out.idx;
   p.out_dist = out.dist;
   p.out_count = out.count;
+  p.out_nearest = nearest_out;
   p.x_split = nullptr;
   char *base = static_cast<char *>(scratch);
   const size_t tau_bytes = align256(sizeof(float) * (size_t)in.m);
@@ -217,7 +232,8 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
     p.partial = reinterpret_cast<double *>(base + tau_bytes + split_bytes);
     p.tau = tau;
     hipLaunchKernelGGL(fill_f32_kernel, dim3((in.m + kBlock - 1) / kBlock),
-                       dim3(kBlock), 0, stream, tau, in.m, kKnnSentinel);
+                       dim3(kBlock), 0, stream, tau, in.m,
+                       cfg.nearest ? kNearestLimit : kKnnSentinel);
   }
 
   if (time_start)
@@ -232,6 +248,10 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
     return err;
 
   switch (cfg.kbucket) {
+  case 1:
+    hipLaunchKernelGGL((knn_merge_kernel<1, kMcQueries, true>),
+                       dim3(tiles_bound), dim3(kBlock), 0, stream, p);
+    break;
   case 8:
     launch_merge<8>(p, cfg.tile_queries, tiles_bound, stream);
     break;

@@ -71,6 +71,7 @@ struct KnnLowdParams {
   int *out_idx;          // dense results (written here only when S == 1)
   float *out_dist;
   int *out_count;
+  int64_t *out_nearest;  // [m] result of the `nearest` search, else unused
 };
 
 __device__ __forceinline__ float next_up_positive(float v) {
@@ -95,6 +96,16 @@ __device__ __forceinline__ void write_dense(const double (&best)[K], int k,
     }
   }
   out_count[q] = found;
+}
+
+// Result of a `nearest` search: the row behind the smallest key, or 0 when no
+// candidate was below the limit (csrc/cuda/nearest_cuda.cu:32,64 in the
+// reference: `best_idx` starts at 0).
+__device__ __forceinline__ void write_nearest(double best, int q, int x_begin,
+                                              int64_t *out) {
+  const bool found = best < SearchLimit<true>::empty();
+  const uint32_t tie = (uint32_t)__double2loint(best);
+  out[q] = found ? (int64_t)x_begin + (int64_t)nearest_rel(tie) : 0;
 }
 
 // Squared distance exactly as the reference accumulates it: direct
@@ -495,7 +506,7 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
 // workgroup per tile; list c of the tile's query at position `pos` starts at
 // partial[((c * tiles + tile) * k) * TQ + pos], consecutive slots TQ apart).
 // p.num_chunks is the number of lists per query.
-template <int K, int TQ>
+template <int K, int TQ, bool NEAREST = false>
 __global__ __launch_bounds__(kBlock) void knn_merge_kernel(KnnLowdParams p) {
   const int tid = threadIdx.x;
   const int total_tiles = p.work_start[p.num_segments];
@@ -514,7 +525,7 @@ __global__ __launch_bounds__(kBlock) void knn_merge_kernel(KnnLowdParams p) {
     double best[K];
 #pragma unroll
     for (int j = 0; j < K; ++j)
-      best[j] = (j < K - k) ? lowest_key() : empty_key();
+      best[j] = (j < K - k) ? lowest_key() : SearchLimit<NEAREST>::empty();
     for (int c = 0; c < p.num_chunks; ++c) {
       const double *src =
           p.partial + (size_t)(c * total_tiles + tile) * k * TQ + pos;
@@ -527,8 +538,13 @@ __global__ __launch_bounds__(kBlock) void knn_merge_kernel(KnnLowdParams p) {
         sorted_insert<K>(best, key);
       }
     }
-    if (q < y_end)
-      write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+    if (q < y_end) {
+      if constexpr (NEAREST)
+        write_nearest(best[0], q, p.ptr_x ? (int)p.ptr_x[seg] : 0,
+                      p.out_nearest);
+      else
+        write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+    }
   }
 }
 

@@ -185,8 +185,13 @@ __global__ __launch_bounds__(kBlock) void mc_pack_rows_kernel(
     out[(size_t)row * REC + i] = packed[i];
 }
 
-template <int DIM, int K>
+// NEAREST: the search of the `nearest` operator -- one neighbour, limit 1e38,
+// the reference's order among equal distances (see device_utils.hpp) -- whose
+// result goes to p.out_nearest as a row number (0 when nothing qualified).
+template <int DIM, int K, bool NEAREST = false>
 __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
+  static_assert(!NEAREST || K == 1, "nearest keeps one neighbour");
+  constexpr float kLimit = SearchLimit<NEAREST>::value;
   constexpr int NI = McShape<DIM>::NI;
   constexpr int XF = McShape<DIM>::XF;
   constexpr int TX = McShape<DIM>::TX;
@@ -271,14 +276,14 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
   double best[K];
 #pragma unroll
   for (int j = 0; j < K; ++j)
-    best[j] = (j < K - k) ? lowest_key() : empty_key();
+    best[j] = (j < K - k) ? lowest_key() : SearchLimit<NEAREST>::empty();
   // exact distances must be strictly below thresh; a lane without a query
   // accepts nothing
   const float ysq_damped = mc_damped_norm(ysq);
-  float thresh = valid ? kKnnSentinel : -__builtin_inff();
+  float thresh = valid ? kLimit : -__builtin_inff();
   float cut = valid ? mc_filter_cut(thresh, ysq_damped) : -1e38f;
-  float shared = kKnnSentinel; // bound inherited from other slices / partner
-  float posted = kKnnSentinel;
+  float shared = kLimit; // bound inherited from other slices / partner
+  float posted = kLimit;
   // The filter tests the SIGN of t - cut: -cut rides along in the two
   // accumulation slots that would otherwise multiply w by the (zero) lo part
   // of the query's 1.  On the row side the upper lanes put 1 where they hold
@@ -431,10 +436,17 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
       const bool ok = has && j < rows && d < thresh;
       if (!__any(ok))
         continue;
+      const uint32_t row_id = NEAREST
+                                  ? nearest_tie((uint32_t)(g_base + j - x_begin))
+                                  : (uint32_t)(g_base + j);
       const double key =
-          ok ? make_key(d, (uint32_t)(g_base + j)) : empty_key();
+          ok ? make_key(d, row_id) : SearchLimit<NEAREST>::empty();
       sorted_insert<K>(best, key);
-      set_thresh(__builtin_fminf(key_dist(best[K - 1]), shared));
+      float own_bound = key_dist(best[K - 1]);
+      // (`nearest`: a later row of EQUAL distance can still win the tie)
+      if (NEAREST && own_bound < kLimit)
+        own_bound = next_up_positive(own_bound);
+      set_thresh(__builtin_fminf(own_bound, shared));
       changed = true;
     }
     qnext = qfirst;
@@ -446,7 +458,7 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
     const auto both = __builtin_amdgcn_permlane32_swap(
         __float_as_uint(own), __float_as_uint(own), false, false);
     const float partner = __uint_as_float(half ? both[0] : both[1]);
-    if (valid && partner < kKnnSentinel) {
+    if (valid && partner < kLimit) {
       shared = __builtin_fminf(shared, next_up_positive(partner));
       if (shared < thresh)
         set_thresh(shared);
@@ -539,13 +551,17 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
         (unsigned)__double2loint(best[j]), (unsigned)__double2loint(best[j]),
         false, false);
     const double upper = __hiloint2double((int)hi[1], (int)lo[1]);
-    sorted_insert<K>(best, half ? empty_key() : upper);
+    sorted_insert<K>(best, half ? SearchLimit<NEAREST>::empty() : upper);
   }
 
   if (half == 0) {
     if (p.num_chunks == 1) {
-      if (valid)
-        write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+      if (valid) {
+        if constexpr (NEAREST)
+          write_nearest(best[0], q, x_begin, p.out_nearest);
+        else
+          write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+      }
     } else {
       // sorted keys of this slice, [item][slot][query of the tile]
       double *dst = p.partial + (size_t)blockIdx.x * k * TQ + wave * 32 + col;
@@ -596,6 +612,10 @@ hipError_t launch_mc_pack_rows(const float *x, int n, int d_in, uint4 *out,
       break;                                                                   \
     case 32:                                                                   \
       hipLaunchKernelGGL((knn_lowd_mc_kernel<DIM_, 32>), dim3(grid),           \
+                         dim3(kBlock), 0, stream, p);                          \
+      break;                                                                   \
+    case 1: /* the `nearest` search */                                         \
+      hipLaunchKernelGGL((knn_lowd_mc_kernel<DIM_, 1, true>), dim3(grid),      \
                          dim3(kBlock), 0, stream, p);                          \
       break;                                                                   \
     default:                                                                   \

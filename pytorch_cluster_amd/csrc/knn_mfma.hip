@@ -180,6 +180,8 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   mp.out_idx = out.idx;
   mp.out_dist = out.dist;
   mp.out_count = out.count;
+  mp.out_nearest = nullptr;
+  mp.x_split = nullptr;
   switch (kb) {
   case 8:
     launch_mfma_merge<8>(mp, tiles_bound, stream);

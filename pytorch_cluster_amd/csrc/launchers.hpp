@@ -57,19 +57,25 @@ struct KnnLowdConfig {
   int tile_queries;     // queries per work item
   bool matrix_cores;    // pre-filter on the matrix cores (knn_lowd_mc_impl)
   int num_chunks;       // slices of every segment's x rows (>= 1)
+  bool nearest;         // the `nearest` search (kbucket 1, matrix cores)
 };
 bool knn_lowd_supported(int d, int k, bool cosine);
 KnnLowdConfig knn_lowd_config(int d, int k, int n, int m, int num_segments,
                               bool cosine);
+// The `nearest` search over fp32 points of up to 8 dimensions: in.x are the
+// candidates, in.y the rows that look for their nearest candidate.
+KnnLowdConfig nearest_lowd_config(int d, int n, int m, int num_segments);
 // Scratch the launch needs beyond the dense result (shared bounds + partial
 // key lists of sliced segments).
 size_t knn_lowd_scratch_bytes(const KnnLowdConfig &cfg, int n, int m, int d,
                               int num_segments, int k);
+// cfg.nearest: `out` is unused and nearest_out [m] receives the rows.
 hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
                            const KnnLowdConfig &cfg, const int *work_start,
                            void *scratch, const DenseResult &out,
                            hipEvent_t time_start, hipEvent_t time_stop,
-                           hipStream_t stream);
+                           hipStream_t stream,
+                           int64_t *nearest_out = nullptr);
 
 // --- knn_mfma*.hip ---------------------------------------------------------
 
@@ -107,6 +113,14 @@ hipError_t launch_radius_anytype(int dtype, const SearchInput &in, double r,
                                  bool ignore_same_index,
                                  const int *work_start, int task_bound,
                                  const DenseResult &out, hipStream_t stream);
+
+// --- anytype.hip: the `nearest` search, any element type and dimension ------
+
+// work_start: tiles of kBlock rows of in.y (the rows that search); in.x are
+// the candidates.  dtype: PCA_F32, PCA_F64 or PCA_F16.
+hipError_t launch_nearest_any(int dtype, const SearchInput &in,
+                              const int *work_start, int grid_bound,
+                              int64_t *out, hipStream_t stream);
 
 // --- radius_mc.hip ---------------------------------------------------------
 

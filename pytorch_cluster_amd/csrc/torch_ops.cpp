@@ -1,6 +1,7 @@
-// TorchScript operator binding: registers `torch_cluster::knn` and
-// `torch_cluster::radius` with the reference's operator signatures
-// (csrc/knn.cpp:22-40, csrc/radius.cpp:22-39) on top of the C ABI in
+// TorchScript operator binding: registers `torch_cluster::knn`,
+// `torch_cluster::radius` and `torch_cluster::nearest` with the reference's
+// operator signatures (csrc/knn.cpp:22-40, csrc/radius.cpp:22-39,
+// csrc/nearest.cpp:22-39) on top of the C ABI in
 // include/pca_neighbors.h.  Tensor validation, allocation through PyTorch's
 // caching allocator, the current HIP stream and the single host read of the
 // edge count live here; the kernels never see a torch type.
@@ -198,6 +199,49 @@ at::Tensor radius(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
   return finish(edges, num_edges);
 }
 
+// csrc/nearest.cpp:22-36 -> nearest_cuda (csrc/cuda/nearest_cuda.cu:68-94):
+// both pointer tensors are required, x and y are flattened to [N, -1].
+at::Tensor nearest(at::Tensor x, at::Tensor y, at::Tensor ptr_x,
+                   at::Tensor ptr_y) {
+  TORCH_CHECK(x.device().is_cuda(), "No CPU version supported");
+  PCA_CHECK_GPU(x);
+  PCA_CHECK_GPU(y);
+  PCA_CHECK_GPU(ptr_x);
+  PCA_CHECK_GPU(ptr_y);
+  PCA_CHECK_INPUT(x.dim() >= 1 && y.dim() >= 1);
+  PCA_CHECK_INPUT(x.scalar_type() == y.scalar_type());
+  PCA_CHECK_INPUT(x.get_device() == y.get_device());
+  PCA_CHECK_INPUT(ptr_x.dim() == 1 && ptr_y.dim() == 1);
+  PCA_CHECK_INPUT(ptr_x.numel() == ptr_y.numel() && ptr_x.numel() >= 2);
+  DeviceScope scope(x.get_device());
+  x = x.view({x.size(0), -1}).contiguous();
+  y = y.view({y.size(0), -1}).contiguous();
+  PCA_CHECK_INPUT(x.size(0) == 0 || y.size(0) == 0 ||
+                  x.size(1) == y.size(1));
+  auto out = at::empty({x.size(0)}, ptr_x.options().dtype(at::kLong));
+  const int64_t n = x.size(0), m = y.size(0);
+  if (n == 0)
+    return out;
+  const int64_t d = x.size(1);
+  at::Tensor px = ptr_x.to(at::kLong).contiguous();
+  at::Tensor py = ptr_y.to(at::kLong).contiguous();
+  const int64_t segments = px.numel() - 1;
+  const int dtype = dtype_code(x);
+  TORCH_CHECK(dtype != PCA_BF16,
+              "nearest is not implemented for 'BFloat16'");
+  const size_t ws_bytes =
+      pca_nearest_workspace_bytes(n, m, d, segments, dtype);
+  TORCH_CHECK(ws_bytes > 0, "problem size not supported");
+  auto workspace =
+      at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+  hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
+  check_status(pca_nearest(x.data_ptr(), m > 0 ? y.data_ptr() : nullptr,
+                           px.data_ptr<int64_t>(), py.data_ptr<int64_t>(), n,
+                           m, d, segments, dtype, out.data_ptr<int64_t>(),
+                           workspace.data_ptr(), ws_bytes, stream));
+  return out;
+}
+
 // The stock loader of the reference package calls this
 // (torch_cluster/__init__.py:23, csrc/version.cpp:26-41).
 int64_t cuda_version() { return HIP_VERSION; }
@@ -212,5 +256,7 @@ TORCH_LIBRARY(torch_cluster, m) {
         "int max_num_neighbors, int num_workers, bool ignore_same_index) "
         "-> Tensor",
         &radius);
+  m.def("nearest(Tensor x, Tensor y, Tensor ptr_x, Tensor ptr_y) -> Tensor",
+        &nearest);
   m.def("cuda_version() -> int", &cuda_version);
 }
