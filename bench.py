@@ -126,6 +126,30 @@ def other_configs(torch, pca, testing, dev):
                % cosine] = {
             "ms": ms, "queries_per_s": y.shape[0] / ms * 1e3,
             "gemm_tflops": 2 * 128 * x.shape[0] * y.shape[0] / ms / 1e9}
+    # nearest: every point of the LiDAR-like scans looks for the nearest of
+    # its scan's every-8th point (the operator that follows the neighbour
+    # searches in the reference's list; 3 * D flop per pair as above)
+    from pytorch_cluster_amd._native import capi
+    lidar = testing.lidar_scans(0, query_stride=8)
+    x, y = lidar["x"].to(dev), lidar["y"].to(dev)
+    bx, by = lidar["batch_x"].to(dev), lidar["batch_y"].to(dev)
+    sizes_x = torch.bincount(lidar["batch_x"])
+    sizes_y = torch.bincount(lidar["batch_y"])
+    pairs = int((sizes_x * sizes_y).sum())
+    ms, out = median_ms(lambda: pca.nearest(x, y, bx, by), 10)
+    events = HipEvents(torch)
+    start, stop = events.create(), events.create()
+    capi.pca_time_next_search(start, stop)
+    pca.nearest(x, y, bx, by)
+    torch.cuda.synchronize()
+    kernel_ms = events.elapsed_ms(start, stop)
+    events.destroy(start)
+    events.destroy(stop)
+    report["nearest: %d scan points -> their scan's every 8th point (%d)"
+           % (x.shape[0], y.shape[0])] = {
+        "ms": ms, "rows_per_s": x.shape[0] / ms * 1e3,
+        "kernel_ms": kernel_ms,
+        "kernel_tflops": 9 * pairs / kernel_ms / 1e9}
     return report
 
 
