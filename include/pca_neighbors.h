@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define PCA_ABI_VERSION 1
+#define PCA_ABI_VERSION 2
 
 enum pca_status {
   PCA_OK = 0,
@@ -64,6 +64,21 @@ enum pca_dtype {
   PCA_F16 = 2,
   PCA_BF16 = 3
 };
+
+/*
+ * Edge options of pca_knn / pca_radius (`edge_flags`, 0 = the operators'
+ * output as described above).  They fold the epilogue of the reference's
+ * graph entry points (torch_cluster/knn.py:135-144,
+ * torch_cluster/radius.py:143-148) into the pass that writes `edges`:
+ *   PCA_EDGES_DROP_SELF  leave out the pairs whose x row number equals the
+ *                        query's (the `row != col` mask of knn_graph when x
+ *                        and y are the same rows; for pca_radius the same as
+ *                        ignore_same_index)
+ *   PCA_EDGES_X_FIRST    edges[0 .. E) are the x rows, edges[E .. 2E) the
+ *                        query rows (flow "source_to_target")
+ */
+#define PCA_EDGES_DROP_SELF 1
+#define PCA_EDGES_X_FIRST 2
 
 /* ABI version of the loaded library (== PCA_ABI_VERSION it was built with). */
 int pca_abi_version(void);
@@ -113,8 +128,8 @@ size_t pca_knn_workspace_bytes(int64_t n, int64_t m, int64_t d,
 int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
             const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
             int64_t num_segments, int64_t k, int cosine, int dtype,
-            int64_t *edges, int64_t *num_edges, void *dist, void *workspace,
-            size_t workspace_bytes, void *stream);
+            int edge_flags, int64_t *edges, int64_t *num_edges, void *dist,
+            void *workspace, size_t workspace_bytes, void *stream);
 
 /* --------------------------------------------------------------- radius -- */
 
@@ -146,9 +161,9 @@ size_t pca_radius_workspace_bytes(int64_t n, int64_t m, int64_t d,
 int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
                const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
                int64_t num_segments, double r, int64_t max_num_neighbors,
-               int ignore_same_index, int dtype, int64_t *edges,
-               int64_t *num_edges, void *workspace, size_t workspace_bytes,
-               void *stream);
+               int ignore_same_index, int dtype, int edge_flags,
+               int64_t *edges, int64_t *num_edges, void *workspace,
+               size_t workspace_bytes, void *stream);
 
 /* -------------------------------------------------------------- nearest -- */
 

@@ -22,6 +22,7 @@ _BUILD_HINT = ("build it with `python pytorch_cluster_amd/build.py` "
                "(or `python -c 'import __graft_entry__ as g; g.build()'`)")
 
 PCA_F32, PCA_F64, PCA_F16, PCA_BF16 = 0, 1, 2, 3
+PCA_EDGES_DROP_SELF, PCA_EDGES_X_FIRST = 1, 2
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -36,7 +37,7 @@ C_ABI = {
                                 [_i64, _i64, _i64, _i64, _i64, ctypes.c_int]),
     "pca_knn": (ctypes.c_int,
                 [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
-                 ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp,
+                 ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp,
                  ctypes.c_size_t, _vp]),
     "pca_radius_slots": (_i64, [_i64, _i64]),
     "pca_radius_workspace_bytes": (ctypes.c_size_t,
@@ -44,8 +45,8 @@ C_ABI = {
                                     ctypes.c_int]),
     "pca_radius": (ctypes.c_int,
                    [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
-                    ctypes.c_double, _i64, ctypes.c_int, ctypes.c_int, _vp,
-                    _vp, _vp, ctypes.c_size_t, _vp]),
+                    ctypes.c_double, _i64, ctypes.c_int, ctypes.c_int,
+                    ctypes.c_int, _vp, _vp, _vp, ctypes.c_size_t, _vp]),
     "pca_nearest_workspace_bytes": (ctypes.c_size_t,
                                     [_i64, _i64, _i64, _i64, ctypes.c_int]),
     "pca_nearest": (ctypes.c_int,

@@ -54,10 +54,12 @@ def segment_pointers(
     return torch.bucketize(ids, batch_x), torch.bucketize(ids, batch_y)
 
 
-def orient(edge_index: torch.Tensor, flow: str) -> torch.Tensor:
-    """The search operators return (query, neighbour) pairs.  With
-    ``source_to_target`` messages flow from the neighbour to the query, so the
-    neighbour row comes first."""
-    if flow == 'source_to_target':
-        return edge_index.flip(0)
-    return edge_index
+def graph_pointers(x: torch.Tensor, batch: Optional[torch.Tensor],
+                   batch_size: Optional[int]) -> Optional[torch.Tensor]:
+    """:func:`segment_pointers` of a graph entry point, where both sides are
+    the same rows: one pointer array, computed once."""
+    b = num_examples(x, x, batch, None, batch_size)
+    if b <= 1:
+        return None
+    assert batch is not None
+    return torch.bucketize(torch.arange(b + 1, device=x.device), batch)

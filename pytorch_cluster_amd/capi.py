@@ -9,7 +9,8 @@ from typing import Optional, Tuple
 
 import torch
 
-from ._native import PCA_BF16, PCA_F16, PCA_F32, PCA_F64, capi
+from ._native import (PCA_BF16, PCA_EDGES_DROP_SELF, PCA_EDGES_X_FIRST, PCA_F16,
+                      PCA_F32, PCA_F64, capi)
 
 _DTYPE_CODE = {torch.float32: PCA_F32, torch.float64: PCA_F64,
                torch.float16: PCA_F16, torch.bfloat16: PCA_BF16}
@@ -47,8 +48,14 @@ def _segments(ptr_x, ptr_y):
     return ptr_x, ptr_y, ptr_x.numel() - 1
 
 
+def _edge_flags(drop_self: bool, x_first: bool) -> int:
+    return ((PCA_EDGES_DROP_SELF if drop_self else 0)
+            | (PCA_EDGES_X_FIRST if x_first else 0))
+
+
 def knn_launch(x, y, ptr_x, ptr_y, k: int, cosine: bool = False,
-               want_dist: bool = False, stream=None):
+               want_dist: bool = False, stream=None, drop_self: bool = False,
+               x_first: bool = False):
     """Queues ``pca_knn``; returns (edges buffer [2*m*k], num_edges [1] on the
     device, dist buffer or None, workspace).  Nothing is synchronised."""
     assert x.is_cuda and y.is_cuda and x.is_contiguous() and y.is_contiguous()
@@ -69,25 +76,29 @@ def knn_launch(x, y, ptr_x, ptr_y, k: int, cosine: bool = False,
                         device=x.device) if want_dist else None)
     _check(capi.pca_knn(_dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x),
                         _dev_ptr(ptr_y), n, m, d, nseg, k, int(cosine),
-                        dtype, _dev_ptr(edges), _dev_ptr(num_edges),
+                        dtype, _edge_flags(drop_self, x_first),
+                        _dev_ptr(edges), _dev_ptr(num_edges),
                         _dev_ptr(dist), _dev_ptr(ws), ws_bytes,
                         _stream_handle(stream, x.device)))
     return edges, num_edges, dist, ws
 
 
 def knn_edges(x, y, ptr_x=None, ptr_y=None, k: int = 1, cosine: bool = False,
-              want_dist: bool = False,
-              stream=None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+              want_dist: bool = False, stream=None, drop_self: bool = False,
+              x_first: bool = False
+              ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """``[2, E]`` edges (and the ``[E]`` distances when asked for)."""
     edges, num_edges, dist, _ws = knn_launch(x, y, ptr_x, ptr_y, k, cosine,
-                                             want_dist, stream)
+                                             want_dist, stream, drop_self,
+                                             x_first)
     e = int(num_edges.item())
     out = edges[:2 * e].view(2, e)
     return out, (dist[:e] if dist is not None else None)
 
 
 def radius_launch(x, y, ptr_x, ptr_y, r: float, max_num_neighbors: int,
-                  ignore_same_index: bool = False, stream=None):
+                  ignore_same_index: bool = False, stream=None,
+                  x_first: bool = False):
     assert x.is_cuda and y.is_cuda and x.is_contiguous() and y.is_contiguous()
     assert x.dtype == y.dtype and x.dtype in _DTYPE_CODE
     dtype = _DTYPE_CODE[x.dtype]
@@ -106,6 +117,7 @@ def radius_launch(x, y, ptr_x, ptr_y, r: float, max_num_neighbors: int,
     _check(capi.pca_radius(_dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x),
                            _dev_ptr(ptr_y), n, m, d, nseg, float(r),
                            max_num_neighbors, int(ignore_same_index), dtype,
+                           _edge_flags(False, x_first),
                            _dev_ptr(edges), _dev_ptr(num_edges), _dev_ptr(ws),
                            ws_bytes, _stream_handle(stream, x.device)))
     return edges, num_edges, ws
@@ -113,10 +125,10 @@ def radius_launch(x, y, ptr_x, ptr_y, r: float, max_num_neighbors: int,
 
 def radius_edges(x, y, ptr_x=None, ptr_y=None, r: float = 1.0,
                  max_num_neighbors: int = 32, ignore_same_index: bool = False,
-                 stream=None) -> torch.Tensor:
+                 stream=None, x_first: bool = False) -> torch.Tensor:
     edges, num_edges, _ws = radius_launch(x, y, ptr_x, ptr_y, r,
                                           max_num_neighbors,
-                                          ignore_same_index, stream)
+                                          ignore_same_index, stream, x_first)
     e = int(num_edges.item())
     return edges[:2 * e].view(2, e)
 

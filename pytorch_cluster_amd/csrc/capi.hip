@@ -140,6 +140,10 @@ size_t radius_workspace(int64_t n, int64_t m, int64_t d, int64_t num_segments,
   return bytes;
 }
 
+bool edge_flags_ok(int flags) {
+  return (flags & ~(PCA_EDGES_DROP_SELF | PCA_EDGES_X_FIRST)) == 0;
+}
+
 bool nearest_dtype_ok(int dtype) {
   return dtype == PCA_F32 || dtype == PCA_F64 || dtype == PCA_F16;
 }
@@ -216,8 +220,8 @@ size_t pca_knn_workspace_bytes(int64_t n, int64_t m, int64_t d,
 int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
             const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
             int64_t num_segments, int64_t k, int cosine, int dtype,
-            int64_t *edges, int64_t *num_edges, void *dist, void *workspace,
-            size_t workspace_bytes, void *stream_) {
+            int edge_flags, int64_t *edges, int64_t *num_edges, void *dist,
+            void *workspace, size_t workspace_bytes, void *stream_) {
   g_last_error[0] = 0;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   SearchTimer timer(stream);
@@ -244,6 +248,8 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
   if (dtype != PCA_F32 && dist != nullptr)
     return fail(PCA_ERR_UNSUPPORTED,
                 "per-edge distances are returned for fp32 points only");
+  if (!edge_flags_ok(edge_flags))
+    return fail(PCA_ERR_INVALID_ARGUMENT, "unknown edge flags %d", edge_flags);
 
   if (n == 0 || m == 0) {
     hipLaunchKernelGGL(set_i64_kernel, dim3(1), dim3(1), 0, stream, num_edges,
@@ -335,10 +341,12 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
   }
   if (rc != PCA_OK)
     return rc;
-  return check_launch(pca::launch_compact(dense, (int)m, edges, num_edges,
-                                          static_cast<float *>(dist),
-                                          compact_ws, stream),
-                      "compaction kernels");
+  return check_launch(
+      pca::launch_compact(dense, (int)m, edges, num_edges,
+                          static_cast<float *>(dist), compact_ws, stream,
+                          (edge_flags & PCA_EDGES_DROP_SELF) != 0,
+                          (edge_flags & PCA_EDGES_X_FIRST) != 0),
+      "compaction kernels");
 }
 
 int64_t pca_radius_slots(int64_t n, int64_t max_num_neighbors) {
@@ -362,9 +370,9 @@ size_t pca_radius_workspace_bytes(int64_t n, int64_t m, int64_t d,
 int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
                const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
                int64_t num_segments, double r, int64_t max_num_neighbors,
-               int ignore_same_index, int dtype, int64_t *edges,
-               int64_t *num_edges, void *workspace, size_t workspace_bytes,
-               void *stream_) {
+               int ignore_same_index, int dtype, int edge_flags,
+               int64_t *edges, int64_t *num_edges, void *workspace,
+               size_t workspace_bytes, void *stream_) {
   g_last_error[0] = 0;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   SearchTimer timer(stream);
@@ -382,6 +390,11 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
     return fail(PCA_ERR_INVALID_ARGUMENT,
                 "max_num_neighbors must be >= 1, got %lld",
                 (long long)max_num_neighbors);
+  if (!edge_flags_ok(edge_flags))
+    return fail(PCA_ERR_INVALID_ARGUMENT, "unknown edge flags %d", edge_flags);
+  // (the search itself skips the row; it must not count towards the limit)
+  if (edge_flags & PCA_EDGES_DROP_SELF)
+    ignore_same_index = 1;
   if (num_edges == nullptr)
     return fail(PCA_ERR_INVALID_ARGUMENT, "num_edges is NULL");
   if (!dtype_ok(dtype))
@@ -451,9 +464,11 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
   timer.done();
   if (rc != PCA_OK)
     return rc;
-  return check_launch(pca::launch_compact(dense, (int)m, edges, num_edges,
-                                          nullptr, compact_ws, stream),
-                      "compaction kernels");
+  return check_launch(
+      pca::launch_compact(dense, (int)m, edges, num_edges, nullptr,
+                          compact_ws, stream, false,
+                          (edge_flags & PCA_EDGES_X_FIRST) != 0),
+      "compaction kernels");
 }
 
 size_t pca_nearest_workspace_bytes(int64_t n, int64_t m, int64_t d,

@@ -44,9 +44,12 @@ inline int plan_upper_bound(int m, int num_segments, int per_item) {
 size_t compact_workspace_bytes(int m);
 
 // count -> exclusive offsets -> edges [2, E] (+ optional distances) and E.
+// drop_self: the slot holding the query's own row number is left out;
+// x_first: x rows in the first half of `edges`, query rows in the second.
 hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
                           int64_t *num_edges, float *dist_out, void *workspace,
-                          hipStream_t stream);
+                          hipStream_t stream, bool drop_self = false,
+                          bool x_first = false);
 
 // --- knn_lowd_*.hip --------------------------------------------------------
 

@@ -7,7 +7,11 @@
 //   * the reference's post-kernel epilogue `mask = col != -1`,
 //     2x masked_select, stack (csrc/cuda/knn_cuda.cu:133-134,
 //     csrc/cuda/radius_cuda.cu:94-95): per-query counts -> exclusive scan ->
-//     scatter into a contiguous [2, E] matrix, E left in device memory.
+//     scatter into a contiguous [2, E] matrix, E left in device memory;
+//   * on request the epilogue of the graph entry points as well
+//     (torch_cluster/knn.py:135-144, torch_cluster/radius.py:143-148): pairs
+//     of a row with itself are left out and the x row is written first, in
+//     the same pass.
 #include "device_utils.hpp"
 #include "launchers.hpp"
 
@@ -117,15 +121,52 @@ __global__ __launch_bounds__(kPlanThreads) void scan_block_sums_kernel(
     *num_edges = partial[tid];
 }
 
+// 2^group_shift consecutive threads walk the slots of one query, so that
+// reads of the slot rows and writes of the edge columns stay contiguous.
+//
+// find_self_kernel: position of the slot that holds the query's own row
+// number (at most one: the rows of a query are distinct), or -1, and the
+// number of slots without it.
+__global__ __launch_bounds__(kBlock) void find_self_kernel(
+    const int *__restrict__ idx, const int *__restrict__ count, int m,
+    int slots, int group_shift, int *__restrict__ self_pos,
+    int *__restrict__ kept) {
+  __shared__ int s_self[kCompactQueries];
+  const int tid = threadIdx.x;
+  const int q0 = blockIdx.x * kCompactQueries;
+  const int nq = min(kCompactQueries, m - q0);
+  s_self[tid] = -1;
+  __syncthreads();
+  const int group = 1 << group_shift;
+  const int sub = tid & (group - 1);
+  const int rows_per_pass = kBlock >> group_shift;
+  for (int ql = tid >> group_shift; ql < nq; ql += rows_per_pass) {
+    const int cq = count[q0 + ql];
+    const int64_t row_base = (int64_t)(q0 + ql) * slots;
+    for (int s = sub; s < cq; s += group)
+      if (idx[row_base + s] == q0 + ql)
+        s_self[ql] = s;
+  }
+  __syncthreads();
+  if (tid < nq) {
+    self_pos[q0 + tid] = s_self[tid];
+    kept[q0 + tid] = count[q0 + tid] - (s_self[tid] >= 0 ? 1 : 0);
+  }
+}
+
+// count: slots to write per query (without the self slot when self_pos is
+// given).  x_first: the x row goes to the first half of `edges`.
 __global__ __launch_bounds__(kBlock) void scatter_kernel(
     const int *__restrict__ idx, const float *__restrict__ dist,
-    const int *__restrict__ count, int m, int slots, int group_shift,
+    const int *__restrict__ count, const int *__restrict__ self_pos, int m,
+    int slots, int group_shift, int x_first,
     const int64_t *__restrict__ block_offsets,
     const int64_t *__restrict__ num_edges, int64_t *__restrict__ edges,
     float *__restrict__ dist_out) {
   __shared__ int lds[kBlock];
   __shared__ int s_count[kCompactQueries];
   __shared__ int s_offset[kCompactQueries];
+  __shared__ int s_self[kCompactQueries];
   const int tid = threadIdx.x;
   const int q0 = blockIdx.x * kCompactQueries;
   const int q = q0 + tid;
@@ -134,6 +175,8 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
   const int off = block_exclusive_scan(c, lds, &total);
   s_count[tid] = c;
   s_offset[tid] = off;
+  // (a position no slot has when nothing is left out)
+  s_self[tid] = (self_pos && q < m && self_pos[q] >= 0) ? self_pos[q] : slots;
   __syncthreads();
   if (total == 0)
     return;
@@ -141,20 +184,23 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
   const int64_t E = *num_edges;
   const int64_t base = block_offsets[blockIdx.x];
   const int nq = min(kCompactQueries, m - q0);
-  // 2^group_shift consecutive threads walk the slots of one query, so that
-  // reads of the slot rows and writes of the edge columns stay contiguous.
+  int64_t *first = x_first ? edges + E : edges;  // receives the query rows
+  int64_t *second = x_first ? edges : edges + E; // receives the x rows
   const int group = 1 << group_shift;
   const int sub = tid & (group - 1);
   const int rows_per_pass = kBlock >> group_shift;
   for (int ql = tid >> group_shift; ql < nq; ql += rows_per_pass) {
     const int cq = s_count[ql];
+    const int skip = s_self[ql];
     const int64_t row_base = (int64_t)(q0 + ql) * slots;
     const int64_t e0 = base + s_offset[ql];
+    // output position s reads slot s, or s + 1 from the left-out slot on
     for (int s = sub; s < cq; s += group) {
-      edges[e0 + s] = q0 + ql;
-      edges[E + e0 + s] = idx[row_base + s];
+      const int src = s + (s >= skip ? 1 : 0);
+      first[e0 + s] = q0 + ql;
+      second[e0 + s] = idx[row_base + src];
       if (dist_out)
-        dist_out[e0 + s] = dist[row_base + s];
+        dist_out[e0 + s] = dist[row_base + src];
     }
   }
 }
@@ -172,24 +218,39 @@ hipError_t launch_plan(const int64_t *ptr_y, int m, int num_segments,
 
 size_t compact_workspace_bytes(int m) {
   const int blocks = (m + kCompactQueries - 1) / kCompactQueries;
-  return align256(sizeof(int64_t) * (size_t)(blocks + 1));
+  // block sums, then the two per-query arrays of find_self_kernel
+  return align256(sizeof(int64_t) * (size_t)(blocks + 1)) +
+         2 * align256(sizeof(int) * (size_t)m);
 }
 
 hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
                           int64_t *num_edges, float *dist_out, void *workspace,
-                          hipStream_t stream) {
+                          hipStream_t stream, bool drop_self, bool x_first) {
   const int blocks = (m + kCompactQueries - 1) / kCompactQueries;
-  int64_t *block_sums = static_cast<int64_t *>(workspace);
+  char *ws = static_cast<char *>(workspace);
+  int64_t *block_sums = reinterpret_cast<int64_t *>(ws);
+  ws += align256(sizeof(int64_t) * (size_t)(blocks + 1));
+  int *self_pos = reinterpret_cast<int *>(ws);
+  int *kept = reinterpret_cast<int *>(ws + align256(sizeof(int) * (size_t)m));
   int group_shift = 0;
   while ((1 << group_shift) < dense.slots && group_shift < 8)
     ++group_shift;
+  const int *count = dense.count;
+  if (drop_self) {
+    hipLaunchKernelGGL(find_self_kernel, dim3(blocks), dim3(kBlock), 0, stream,
+                       dense.idx, dense.count, m, dense.slots, group_shift,
+                       self_pos, kept);
+    count = kept;
+  }
   hipLaunchKernelGGL(block_sum_kernel, dim3(blocks), dim3(kBlock), 0, stream,
-                     dense.count, m, block_sums);
+                     count, m, block_sums);
   hipLaunchKernelGGL(scan_block_sums_kernel, dim3(1), dim3(kPlanThreads), 0,
                      stream, block_sums, blocks, num_edges);
   hipLaunchKernelGGL(scatter_kernel, dim3(blocks), dim3(kBlock), 0, stream,
-                     dense.idx, dense.dist, dense.count, m, dense.slots,
-                     group_shift, block_sums, num_edges, edges, dist_out);
+                     dense.idx, dense.dist, count,
+                     drop_self ? self_pos : (const int *)nullptr, m,
+                     dense.slots, group_shift, x_first ? 1 : 0, block_sums,
+                     num_edges, edges, dist_out);
   return hipGetLastError();
 }
 

@@ -115,10 +115,15 @@ at::Tensor finish(const at::Tensor &edges, const at::Tensor &num_edges) {
   return edges.narrow(0, 0, 2 * E).view({2, E});
 }
 
-at::Tensor knn(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
-               std::optional<at::Tensor> ptr_y, int64_t k, bool cosine,
-               int64_t num_workers) {
-  (void)num_workers; // unused by the reference as well (csrc/cpu/knn_cpu.cpp)
+int edge_flags(bool drop_self, bool x_first) {
+  return (drop_self ? PCA_EDGES_DROP_SELF : 0) |
+         (x_first ? PCA_EDGES_X_FIRST : 0);
+}
+
+at::Tensor knn_search(at::Tensor x, at::Tensor y,
+                      std::optional<at::Tensor> ptr_x,
+                      std::optional<at::Tensor> ptr_y, int64_t k, bool cosine,
+                      int flags) {
   PCA_CHECK_GPU(x);
   PCA_CHECK_CONTIGUOUS(x);
   PCA_CHECK_INPUT(x.dim() == 2);
@@ -148,18 +153,36 @@ at::Tensor knn(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
 
   hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
   check_status(pca_knn(x.data_ptr(), y.data_ptr(), seg.ptr_x, seg.ptr_y, n, m,
-                       d, seg.count, k, cosine ? 1 : 0, dtype,
+                       d, seg.count, k, cosine ? 1 : 0, dtype, flags,
                        edges.data_ptr<int64_t>(),
                        num_edges.data_ptr<int64_t>(), nullptr,
                        workspace.data_ptr(), ws_bytes, stream));
   return finish(edges, num_edges);
 }
 
-at::Tensor radius(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
-                  std::optional<at::Tensor> ptr_y, double r,
-                  int64_t max_num_neighbors, int64_t num_workers,
-                  bool ignore_same_index) {
-  (void)num_workers;
+at::Tensor knn(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
+               std::optional<at::Tensor> ptr_y, int64_t k, bool cosine,
+               int64_t num_workers) {
+  (void)num_workers; // unused by the reference as well (csrc/cpu/knn_cpu.cpp)
+  return knn_search(x, y, ptr_x, ptr_y, k, cosine, 0);
+}
+
+// The search of knn_graph with its epilogue (torch_cluster/knn.py:135-144)
+// folded into the pass that writes the edges: no pairs of a row with itself
+// (drop_self), neighbour row first (x_first).
+at::Tensor knn_edges(at::Tensor x, at::Tensor y,
+                     std::optional<at::Tensor> ptr_x,
+                     std::optional<at::Tensor> ptr_y, int64_t k, bool cosine,
+                     bool drop_self, bool x_first) {
+  return knn_search(x, y, ptr_x, ptr_y, k, cosine,
+                    edge_flags(drop_self, x_first));
+}
+
+at::Tensor radius_search(at::Tensor x, at::Tensor y,
+                         std::optional<at::Tensor> ptr_x,
+                         std::optional<at::Tensor> ptr_y, double r,
+                         int64_t max_num_neighbors, bool ignore_same_index,
+                         int flags) {
   PCA_CHECK_GPU(x);
   PCA_CHECK_CONTIGUOUS(x);
   PCA_CHECK_INPUT(x.dim() == 2);
@@ -192,11 +215,31 @@ at::Tensor radius(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
   hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
   check_status(pca_radius(x.data_ptr(), y.data_ptr(), seg.ptr_x, seg.ptr_y, n,
                           m, d, seg.count, r, max_num_neighbors,
-                          ignore_same_index ? 1 : 0, dtype,
+                          ignore_same_index ? 1 : 0, dtype, flags,
                           edges.data_ptr<int64_t>(),
                           num_edges.data_ptr<int64_t>(), workspace.data_ptr(),
                           ws_bytes, stream));
   return finish(edges, num_edges);
+}
+
+at::Tensor radius(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
+                  std::optional<at::Tensor> ptr_y, double r,
+                  int64_t max_num_neighbors, int64_t num_workers,
+                  bool ignore_same_index) {
+  (void)num_workers;
+  return radius_search(x, y, ptr_x, ptr_y, r, max_num_neighbors,
+                       ignore_same_index, 0);
+}
+
+// The search of radius_graph with the flow flip of
+// torch_cluster/radius.py:143-148 folded in.
+at::Tensor radius_edges(at::Tensor x, at::Tensor y,
+                        std::optional<at::Tensor> ptr_x,
+                        std::optional<at::Tensor> ptr_y, double r,
+                        int64_t max_num_neighbors, bool ignore_same_index,
+                        bool x_first) {
+  return radius_search(x, y, ptr_x, ptr_y, r, max_num_neighbors,
+                       ignore_same_index, edge_flags(false, x_first));
 }
 
 // csrc/nearest.cpp:22-36 -> nearest_cuda (csrc/cuda/nearest_cuda.cu:68-94):
@@ -259,4 +302,16 @@ TORCH_LIBRARY(torch_cluster, m) {
   m.def("nearest(Tensor x, Tensor y, Tensor ptr_x, Tensor ptr_y) -> Tensor",
         &nearest);
   m.def("cuda_version() -> int", &cuda_version);
+}
+
+// Operators without a counterpart in the reference: the graph entry points of
+// this package call them to get their edges in one pass.
+TORCH_LIBRARY(pytorch_cluster_amd, m) {
+  m.def("knn_edges(Tensor x, Tensor y, Tensor? ptr_x, Tensor? ptr_y, int k, "
+        "bool cosine, bool drop_self, bool x_first) -> Tensor",
+        &knn_edges);
+  m.def("radius_edges(Tensor x, Tensor y, Tensor? ptr_x, Tensor? ptr_y, "
+        "float r, int max_num_neighbors, bool ignore_same_index, "
+        "bool x_first) -> Tensor",
+        &radius_edges);
 }

@@ -505,3 +505,29 @@ def test_config5_ragged_lidar_full_size(oracle):
     want, _ = oracle_knn_edges(oracle, x.numpy(), ys, ptr_x, ptr_ys, 16)
     got = e[1].reshape(m, 16)[sample]
     assert (got == want[1].reshape(len(sample), 16)).all()
+
+
+@pytest.mark.parametrize("flow", ["source_to_target", "target_to_source"])
+@pytest.mark.parametrize("loop", [False, True])
+def test_graph_epilogue_in_the_output_pass(oracle, flow, loop):
+    """knn_graph drops self-pairs and orients the edges while they are
+    written (edge flags of pca_knn); order and content are those of the
+    reference's mask + stack (torch_cluster/knn.py:135-144), including the
+    rows that keep k + 1 edges because duplicates precede them."""
+    rng = np.random.default_rng(5)
+    x = rng.integers(0, 6, (3000, 3)).astype(np.float32)  # many duplicates
+    batch = np.sort(rng.integers(0, 5, 3000))
+    batch[batch == 2] = 3  # an example without rows
+    for k in (1, 7, 20):
+        want = oracle.knn_graph(x, k, batch, loop=loop, flow=flow)
+        got = pca.knn_graph(dev(x), k, dev(batch), loop=loop, flow=flow)
+        assert got.cpu().numpy().tolist() == want.tolist()
+    # the C entry point with distances: they follow the kept edges
+    ptr = np.searchsorted(batch, np.arange(6)).astype(np.int64)
+    e, d = capi.knn_edges(dev(x), dev(x), dev(ptr), dev(ptr), 8,
+                          want_dist=True, drop_self=True, x_first=True)
+    e, d = e.cpu().numpy(), d.cpu().numpy()
+    full, dfull = gpu_knn(x, x, ptr, ptr, 8)
+    keep = full[0] != full[1]
+    assert e.tolist() == full[::-1][:, keep].tolist()
+    assert (d == dfull[keep]).all()

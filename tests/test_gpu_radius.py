@@ -199,3 +199,18 @@ def test_config3_gaussian_mixture_radius_graph(oracle):
     assert e.shape == want.shape
     assert (e.cpu().numpy() == want).all()
     assert (batch.numpy()[want[0]] == batch.numpy()[want[1]]).all()
+
+
+@pytest.mark.parametrize("flow", ["source_to_target", "target_to_source"])
+@pytest.mark.parametrize("loop", [False, True])
+def test_graph_orientation_in_the_output_pass(oracle, radius_path, flow, loop):
+    """radius_graph's flow flip (torch_cluster/radius.py:143-148) is applied
+    while the edges are written (edge flags of pca_radius)."""
+    rng = np.random.default_rng(8)
+    x = rng.random((2500, 3)).astype(np.float32)
+    batch = np.sort(rng.integers(0, 4, 2500))
+    want = oracle.radius_graph(x, 0.12, batch, loop=loop, flow=flow,
+                               max_num_neighbors=9)
+    got = pca.radius_graph(dev(x), 0.12, dev(batch), loop=loop, flow=flow,
+                           max_num_neighbors=9)
+    assert got.cpu().numpy().tolist() == want.tolist()

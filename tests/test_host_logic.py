@@ -26,31 +26,31 @@ def test_header_symbols_are_exported():
     for name in sorted(declared):
         assert hasattr(lib, name), "missing export: " + name
     assert declared == set(_native.C_ABI), "ctypes table out of date"
-    assert lib.pca_abi_version() == 1
+    assert lib.pca_abi_version() == 2
 
 
 def test_capi_validation_needs_no_gpu():
     capi = _native.capi
     one = ctypes.c_void_p(256)  # never dereferenced on these paths
     # k > 100 -> the reference's message (csrc/cuda/knn_cuda.cu:98)
-    rc = capi.pca_knn(one, one, None, None, 10, 10, 3, 1, 101, 0, 0, one, one,
+    rc = capi.pca_knn(one, one, None, None, 10, 10, 3, 1, 101, 0, 0, 0, one, one,
                       None, one, 1 << 20, None)
     assert rc == -2
     assert b"smaller than or equal to 100" in capi.pca_last_error()
-    rc = capi.pca_knn(one, one, one, None, 10, 10, 3, 1, 4, 0, 0, one, one,
+    rc = capi.pca_knn(one, one, one, None, 10, 10, 3, 1, 4, 0, 0, 0, one, one,
                       None, one, 1 << 20, None)
     assert rc == -1  # only one ptr given
-    rc = capi.pca_knn(one, one, None, None, 10, 10, 3, 1, 4, 0, 0, one, one,
+    rc = capi.pca_knn(one, one, None, None, 10, 10, 3, 1, 4, 0, 0, 0, one, one,
                       None, one, 16, None)
     assert rc == -3  # workspace too small
-    rc = capi.pca_knn(one, one, None, None, 10, 10, 3, 1, 4, 0, 7, one, one,
+    rc = capi.pca_knn(one, one, None, None, 10, 10, 3, 1, 4, 0, 7, 0, one, one,
                       None, one, 1 << 20, None)
     assert rc == -5  # no such element type
-    rc = capi.pca_knn(one, one, None, None, 10, 10, 3, 1, 4, 0, 1, one, one,
+    rc = capi.pca_knn(one, one, None, None, 10, 10, 3, 1, 4, 0, 1, 0, one, one,
                       one, one, 1 << 20, None)
     assert rc == -5  # distances are written for fp32 points only
     rc = capi.pca_radius(one, one, None, None, 10, 10, 3, 1, 0.5, 0, 0, 0,
-                         one, one, one, 1 << 20, None)
+                         0, one, one, one, 1 << 20, None)
     assert rc == -1  # max_num_neighbors must be >= 1
     assert capi.pca_knn_workspace_bytes(100, 100, 3, 1, 101, 0) == 0
     assert capi.pca_knn_workspace_bytes(100, 100, 3, 1, 16, 0) > 100 * 16 * 8
@@ -75,6 +75,8 @@ def test_cpu_tensors_fail_loudly():
         pca.knn(x, x, 2)
     with pytest.raises(RuntimeError, match="must be CUDA tensor"):
         pca.radius_graph(x, 0.5)
+    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
+        pca.knn_graph(x, 2)
     with pytest.raises(RuntimeError, match="must be CUDA tensor"):
         torch.ops.torch_cluster.knn(x, x, None, None, 2, False, 1)
 
@@ -109,8 +111,27 @@ def oracle_ops(monkeypatch, oracle):
         return torch.from_numpy(oracle.radius_op(x.numpy(), y.numpy(), px, py,
                                                  r, max_nn, 1, ignore))
 
+    # the variants the graph entry points call: the operator's edges without
+    # self-pairs and / or with the x row first
+    def finish(edges, drop_self, x_first):
+        if drop_self:
+            edges = edges[:, edges[0] != edges[1]]
+        return edges.flip(0) if x_first else edges
+
+    def fake_knn_edges(x, y, ptr_x, ptr_y, k, cosine, drop_self, x_first):
+        return finish(fake_knn(x, y, ptr_x, ptr_y, k, cosine, 1), drop_self,
+                      x_first)
+
+    def fake_radius_edges(x, y, ptr_x, ptr_y, r, max_nn, ignore, x_first):
+        return finish(fake_radius(x, y, ptr_x, ptr_y, r, max_nn, 1, ignore),
+                      False, x_first)
+
     monkeypatch.setattr(torch.ops.torch_cluster, "knn", fake_knn)
     monkeypatch.setattr(torch.ops.torch_cluster, "radius", fake_radius)
+    monkeypatch.setattr(torch.ops.pytorch_cluster_amd, "knn_edges",
+                        fake_knn_edges)
+    monkeypatch.setattr(torch.ops.pytorch_cluster_amd, "radius_edges",
+                        fake_radius_edges)
     return calls
 
 
