@@ -95,7 +95,7 @@ KnnLayout knn_layout(int64_t n, int64_t m, int64_t d, int64_t num_segments,
   } else if (d > 8) {
     w.x_norm = align256(sizeof(float) * (size_t)n);
     if (pca::knn_mfma_supported((int)d, (int)k, false))
-      w.sliced = pca::knn_mfma_scratch_bytes((int)n, (int)m,
+      w.sliced = pca::knn_mfma_scratch_bytes((int)n, (int)m, (int)d,
                                              (int)num_segments, (int)k);
   } else {
     // the larger of the two metrics' needs, so one size query serves both

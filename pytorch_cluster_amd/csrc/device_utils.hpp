@@ -116,6 +116,22 @@ __device__ __forceinline__ void sorted_insert(double (&b)[K], double key) {
   b[0] = key_min(b[0], key);
 }
 
+// ---- fp32 values as sums of two bf16 numbers (matrix-core pre-filters) -----
+typedef __bf16 mc_bf16x8_t __attribute__((ext_vector_type(8)));
+
+// bf16 nearest-even of a finite float of moderate size, as the upper half of
+// a float
+__device__ __forceinline__ uint32_t mc_bf16_bits(float v) {
+  const uint32_t u = __float_as_uint(v);
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+// v = hi + lo + r, |r| <= 2^-16 |v|
+__device__ __forceinline__ void mc_split(float v, uint32_t &hi, uint32_t &lo) {
+  hi = mc_bf16_bits(v);
+  lo = mc_bf16_bits(v - __uint_as_float(hi << 16)); // the difference is exact
+}
+
 __device__ __forceinline__ float min3f(float a, float b, float c) {
   return __builtin_fminf(__builtin_fminf(a, b), c);
 }

@@ -67,8 +67,6 @@ namespace pca {
 constexpr int kMcQueries = 128; // queries per workgroup
 constexpr int kMcQueueCap = 8; // parked steps per lane
 
-typedef __bf16 mc_bf16x8_t __attribute__((ext_vector_type(8)));
-
 template <int DIM> struct McShape {
   // matrix instructions per 32-row step: four augmented components each
   static constexpr int NI = (DIM + 1 + 3) / 4;
@@ -77,19 +75,6 @@ template <int DIM> struct McShape {
   static constexpr int REC = NI + XF / 4;
   static constexpr int TX = DIM <= 4 ? 1024 : 256; // rows per LDS tile
 };
-
-// bf16 nearest-even of a finite float of moderate size, as the upper half of
-// a float
-__device__ __forceinline__ uint32_t mc_bf16_bits(float v) {
-  const uint32_t u = __float_as_uint(v);
-  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-}
-
-// v = hi + lo + r, |r| <= 2^-16 |v|
-__device__ __forceinline__ void mc_split(float v, uint32_t &hi, uint32_t &lo) {
-  hi = mc_bf16_bits(v);
-  lo = mc_bf16_bits(v - __uint_as_float(hi << 16)); // the difference is exact
-}
 
 constexpr float kMcEps = 1.0f / 16384.0f; // 2^-14
 

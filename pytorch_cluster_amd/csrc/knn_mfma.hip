@@ -6,21 +6,27 @@
 
 namespace pca {
 
-template <int STEPS>
-hipError_t launch_knn_mfma_steps(const KnnMfmaParams &p, int kbucket,
-                                 bool cosine, int grid, hipStream_t stream);
-template <>
-hipError_t launch_knn_mfma_steps<12>(const KnnMfmaParams &, int, bool, int,
-                                    hipStream_t);
-template <>
-hipError_t launch_knn_mfma_steps<20>(const KnnMfmaParams &, int, bool, int,
-                                     hipStream_t);
-template <>
-hipError_t launch_knn_mfma_steps<36>(const KnnMfmaParams &, int, bool, int,
-                                     hipStream_t);
-template <>
-hipError_t launch_knn_mfma_steps<68>(const KnnMfmaParams &, int, bool, int,
-                                     hipStream_t);
+// One number of component blocks per translation unit (knn_mfma_b*.hip):
+// the search kernels and the kernel that packs the x rows for them.
+template <int NB>
+hipError_t launch_knn_mfma_blocks(const KnnMfmaParams &p, int kbucket,
+                                  bool cosine, int grid, hipStream_t stream);
+template <int NB>
+hipError_t launch_mfma_pack_rows(const float *x, const float *norms, int n,
+                                 int d, bool cosine, uint4 *out,
+                                 hipStream_t stream);
+#define PCA_DECLARE_BLOCKS(NB)                                                 \
+  template <>                                                                  \
+  hipError_t launch_knn_mfma_blocks<NB>(const KnnMfmaParams &, int, bool,      \
+                                        int, hipStream_t);                     \
+  template <>                                                                  \
+  hipError_t launch_mfma_pack_rows<NB>(const float *, const float *, int,      \
+                                       int, bool, uint4 *, hipStream_t);
+PCA_DECLARE_BLOCKS(2)
+PCA_DECLARE_BLOCKS(3)
+PCA_DECLARE_BLOCKS(5)
+PCA_DECLARE_BLOCKS(9)
+#undef PCA_DECLARE_BLOCKS
 
 // csrc/knn_generic_cos.hip
 hipError_t launch_row_norms(const float *x, int n, int d, float *norm,
@@ -64,6 +70,23 @@ void launch_mfma_merge(const KnnLowdParams &p, int tiles_bound,
                      dim3(kBlock), 0, stream, p);
 }
 
+// blocks of 16 components: the coordinates and one augmented block
+int mfma_blocks(int d) {
+  if (d <= 16)
+    return 2;
+  if (d <= 32)
+    return 3;
+  if (d <= 64)
+    return 5;
+  return 9;
+}
+
+size_t mfma_pack_bytes(int n, int d) {
+  const int nb = mfma_blocks(d);
+  const size_t units = 2 * nb + 2 * (nb - 1); // MfmaShape<nb>::UNITS
+  return align256(sizeof(uint4) * units * (size_t)n);
+}
+
 } // namespace
 
 bool knn_mfma_supported(int d, int k, bool cosine) {
@@ -87,11 +110,11 @@ int knn_mfma_slices(int n, int m, int num_segments) {
   return chunks;
 }
 
-size_t knn_mfma_scratch_bytes(int n, int m, int num_segments, int k) {
+size_t knn_mfma_scratch_bytes(int n, int m, int d, int num_segments, int k) {
   const size_t tiles = plan_upper_bound(m, num_segments, kMfmaQueries);
   // the largest slice count a call may choose
   const int chunks = std::max(knn_mfma_slices(n, m, num_segments), 1);
-  return align256(sizeof(float) * (size_t)n) +
+  return mfma_pack_bytes(n, d) + align256(sizeof(float) * (size_t)n) +
          2 * align256(sizeof(float) * (size_t)m) +
          align256(sizeof(double) * tiles * chunks * (size_t)k *
                   kMfmaQueries);
@@ -105,6 +128,8 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
       plan_upper_bound(in.m, in.num_segments, kMfmaQueries);
   const int chunks = knn_mfma_slices(in.n, in.m, in.num_segments);
   char *base = static_cast<char *>(scratch);
+  uint4 *x_pack = reinterpret_cast<uint4 *>(base);
+  base += mfma_pack_bytes(in.n, in.d);
   float *x_sq = reinterpret_cast<float *>(base);
   base += align256(sizeof(float) * (size_t)in.n);
   float *tau = reinterpret_cast<float *>(base);
@@ -124,6 +149,30 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
                        static_cast<const float *>(in.x), in.n, in.d, x_sq);
   hipLaunchKernelGGL(fill_tau_kernel, dim3((in.m + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, tau, in.m, kKnnSentinel);
+  {
+    const float *xf = static_cast<const float *>(in.x);
+    hipError_t perr;
+    switch (mfma_blocks(in.d)) {
+    case 2:
+      perr = launch_mfma_pack_rows<2>(xf, x_sq, in.n, in.d, cosine, x_pack,
+                                      stream);
+      break;
+    case 3:
+      perr = launch_mfma_pack_rows<3>(xf, x_sq, in.n, in.d, cosine, x_pack,
+                                      stream);
+      break;
+    case 5:
+      perr = launch_mfma_pack_rows<5>(xf, x_sq, in.n, in.d, cosine, x_pack,
+                                      stream);
+      break;
+    default:
+      perr = launch_mfma_pack_rows<9>(xf, x_sq, in.n, in.d, cosine, x_pack,
+                                      stream);
+      break;
+    }
+    if (perr != hipSuccess)
+      return perr;
+  }
 
   KnnMfmaParams p;
   p.x = static_cast<const float *>(in.x);
@@ -132,6 +181,7 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   p.ptr_y = in.ptr_y;
   p.x_sq = x_sq;
   p.y_norm = y_norm;
+  p.x_pack = x_pack;
   p.n = in.n;
   p.m = in.m;
   p.d = in.d;
@@ -144,15 +194,17 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
 
   const int kb = k_bucket(k);
   const int grid = tiles_bound * chunks;
-  // 2 STEPS components per row: the d coordinates and two augmented ones
   auto launch = [&](const KnnMfmaParams &pp, int g) {
-    if (in.d <= 22)
-      return launch_knn_mfma_steps<12>(pp, kb, cosine, g, stream);
-    if (in.d <= 38)
-      return launch_knn_mfma_steps<20>(pp, kb, cosine, g, stream);
-    if (in.d <= 70)
-      return launch_knn_mfma_steps<36>(pp, kb, cosine, g, stream);
-    return launch_knn_mfma_steps<68>(pp, kb, cosine, g, stream);
+    switch (mfma_blocks(in.d)) {
+    case 2:
+      return launch_knn_mfma_blocks<2>(pp, kb, cosine, g, stream);
+    case 3:
+      return launch_knn_mfma_blocks<3>(pp, kb, cosine, g, stream);
+    case 5:
+      return launch_knn_mfma_blocks<5>(pp, kb, cosine, g, stream);
+    default:
+      return launch_knn_mfma_blocks<9>(pp, kb, cosine, g, stream);
+    }
   };
   if (time_start)
     (void)hipEventRecord(time_start, stream);

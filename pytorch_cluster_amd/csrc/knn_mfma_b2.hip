@@ -1,0 +1,17 @@
+// Matrix-core kNN kernels for points of up to 16 components (2 blocks
+// of 16: the coordinates and one block of augmented components).
+#include "knn_mfma_impl.hpp"
+
+namespace pca {
+
+template <int NB>
+hipError_t launch_knn_mfma_blocks(const KnnMfmaParams &p, int kbucket,
+                                  bool cosine, int grid, hipStream_t stream);
+template <int NB>
+hipError_t launch_mfma_pack_rows(const float *x, const float *norms, int n,
+                                 int d, bool cosine, uint4 *out,
+                                 hipStream_t stream);
+
+PCA_KNN_MFMA_DEFINE(2)
+
+} // namespace pca

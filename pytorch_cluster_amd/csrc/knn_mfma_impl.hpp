@@ -1,4 +1,4 @@
-// Feature-space kNN (8 < d <= 134, k <= 32, Euclidean or cosine) on the gfx950
+// Feature-space kNN (8 < d <= 128, k <= 32, Euclidean or cosine) on the gfx950
 // matrix cores, with results bit-identical to the reference's scalar loop
 // (csrc/cuda/knn_cuda.cu:52-78).
 //
@@ -6,22 +6,31 @@
 // distance that is kept is evaluated exactly as the reference does.  For the
 // Euclidean metric the filter value of a (query, candidate) pair is
 //     t = w - 2 x.y,      w = fl(|x|^2) (1 - eps),
-// the dot product of the augmented rows (x, w) and (-2 y, 1): one chain of
-// v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate) over the components for 32
-// candidates x 32 queries.  The last component carries (1) . (-cut),
+// the dot product of the augmented rows (x, w) and (-2 y, 1).  Every fp32
+// operand v is split into two bf16 numbers, v = hi + lo + r with
+// |r| <= 2^-18 |v| (bf16 keeps the exponent range of fp32), and the products
+// hi*hi + hi*lo + lo*hi of 16 components at a time are one
+// v_mfma_f32_32x32x16_bf16 each (exact products, fp32 accumulation): 32
+// candidates x 32 queries x 16 components in 8 passes, where the fp32 matrix
+// instruction needs 16 passes for 2 components.  A last block of components
+// holds w (two parts, times 1) and 1 (twice, times the two parts of -cut),
 //     cut = thresh (1 + eps) - fl(|y|^2) (1 - eps)   (rounded up),
-//     eps = (d + 32) 2^-22,
 // so the SIGN of a result says whether the candidate can still have an exact
-// distance below thresh: with the accumulated products within 2 u |x||y| per
-// term of the true ones (u = 2^-24), norms accumulated with one FMA per
-// component and the exact chain d_exact >= |x-y|^2 (1 - (d + 2) u), a
-// candidate with d_exact < thresh always has t - cut < 0.  Rows whose squared
-// norm is not a moderate finite number enter with zero coordinates and
-// w = -inf (always looked at), padding rows with w = NaN (never), queries with
-// such a norm use cut = +inf with zero coordinates (look at every real row).
+// distance below thresh.  Error budget, relative to |x|^2 + |y|^2 + thresh:
+// the dropped lo*lo products and the split residuals 2^-16.4; accumulating
+// 3 d + 4 terms, each step within 2^-23 of the running magnitude (which stays
+// below 2 (|x|^2 + |y|^2) + thresh), (3 d + 4) 2^-22; norms and the exact
+// chain (d + 2) 2^-24 each.  eps = 2^-15 + (3 d + 8) 2^-21 covers twice that.
+// Rows whose squared norm is not a moderate finite number enter with zero
+// coordinates and w = -1e38 (always looked at; an infinity would meet a zero
+// part of another operand and turn into NaN), padding rows with a huge
+// positive w and are never candidates whatever the filter says, queries with
+// such a norm use the largest finite cut with zero coordinates (look at every
+// real row).
 //
 // The cosine distance 1 - x.y / (|x| |y|) uses the same chain on normalised
-// rows: (x / |x|, 1) . (-y / |y|, 1) = 1 - cos, within (4 d + 72) u of the
+// rows: (x / |x|, 1) . (-y / |y|, 1) = 1 - cos, within (4 d + 72) 2^-24 (the
+// normalisations) + eps (split and accumulation, magnitudes below 4) of the
 // exactly evaluated distance; the cut is thresh + that margin.
 // Rows of norm 0 or NaN have a NaN distance in the reference and are padding
 // here; a row or query of infinite norm is looked at / looks at everything.
@@ -36,14 +45,14 @@
 // (they are L2 resident) -- and hands the (distance, row) key back through
 // LDS to the lane that owns the query, which runs the insertion network.  An
 // exact distance costs ~2 d vector instructions for the whole wave whether 1
-// or 64 lanes have work, so the dense list is what keeps the re-rank a few
-// percent of the matrix-core time even when a handful of queries collect most
-// of the candidates.
+// or 64 lanes have work, so the dense list is what keeps the re-rank cheap
+// even when a handful of queries collect most of the candidates.
 //
 // Mapping: a workgroup owns 128 queries of one segment (4 waves x 32) and one
 // slice of the segment's x rows.  A = 32 candidates (rows i), B = 32 queries
-// (columns j): lane l supplies A[l%32][2s + l/32] and B[2s + l/32][l%32] for
-// step s, and receives, in 16 accumulator registers, the results of query
+// (columns j): for the block of components 16 b .. 16 b + 15 lane l supplies
+// the 8 components 16 b + 8 (l / 32) + 0..7 of candidate l % 32 and of query
+// l % 32, and receives, in 16 accumulator registers, the results of query
 // l%32 against the 16 candidate rows 8*(v/4) + 4*(l/32) + v%4.  So lanes l and
 // l+32 share a query and split its candidates; the lower lane keeps the
 // query's list and collects the keys of both lanes' rows in ascending row
@@ -52,10 +61,12 @@
 // knn_merge_kernel and exchange their pruning bound through `tau` like the
 // slices of the low-dimensional kernels do.
 //
-// The query operands stay in registers for the whole scan (d/2 + 1 per lane);
-// candidate tiles stream through LDS, double-buffered, with the even and odd
-// components of a row stored as two contiguous halves so that a lane's
-// operands for 4 consecutive steps are one ds_read_b128.
+// The query operands stay in registers for the whole scan; the candidate rows
+// are split once per call (mfma_pack_rows_kernel: per row the hi parts of all
+// blocks, then the lo parts of the coordinate blocks, 16 bytes per lane and
+// block) and stream through LDS as they are, double-buffered, with an odd row
+// stride so that the 16-byte reads of neighbouring rows fall on distinct
+// banks.
 #pragma once
 
 #include "device_utils.hpp"
@@ -78,6 +89,7 @@ struct KnnMfmaParams {
   const int64_t *ptr_y;
   const float *x_sq;   // [n] squared norms of the x rows (cosine: norms)
   const float *y_norm; // [m] norms of the y rows (cosine only)
+  const uint4 *x_pack; // [n] packed filter operands (mfma_pack_rows_kernel)
   int n, m, d, num_segments, k;
   const int *work_start; // [num_segments + 1] first 128-query tile per segment
   int num_chunks;        // slices of every segment's x rows
@@ -89,17 +101,99 @@ struct KnnMfmaParams {
 __global__ __launch_bounds__(kBlock) void row_sqnorm_kernel(
     const float *__restrict__ x, int n, int d, float *__restrict__ out);
 
+// Shape of a packed row for NB blocks of 16 components (the last block holds
+// the augmented components): 16-byte units of 8 bf16 numbers.
+template <int NB> struct MfmaShape {
+  static constexpr int P = 16 * NB;          // components with the padding
+  static constexpr int HI = 2 * NB;          // units of hi parts
+  static constexpr int LO = 2 * (NB - 1);    // units of lo parts (coordinates)
+  static constexpr int UNITS = HI + LO;      // per row in global memory
+  static constexpr int RSU = UNITS + 1;      // LDS row stride (odd)
+  static constexpr int MAX_D = 16 * (NB - 1);
+};
+
+__host__ __device__ __forceinline__ double mfma_filter_eps(int d) {
+  return 1.0 / 32768.0 + (double)(3 * d + 8) * (1.0 / 2097152.0);
+}
+
 __device__ __forceinline__ float mfma_filter_cut(float thresh, float ysq,
                                                  double eps) {
   if (!(ysq <= kFilterNormLimit))
     return __builtin_inff(); // examine everything exactly
+  // (1e-20: operands below the bf16 normal range may be flushed to zero by
+  // the matrix cores, 400 terms of at most 2^-126 * 2e15 each)
   const double c =
-      (double)thresh * (1.0 + eps) - (double)ysq * (1.0 - eps) + 1e-30;
+      (double)thresh * (1.0 + eps) - (double)ysq * (1.0 - eps) + 1e-20;
   float f = (float)c;
   if ((double)f < c) // round towards +inf
     f = __uint_as_float(f >= 0.0f ? __float_as_uint(f) + 1u
                                   : __float_as_uint(f) - 1u);
   return f;
+}
+
+// Packs the filter operands of the x rows: one thread per 16-byte unit.
+// norms: squared norms (Euclidean) or norms (cosine) of the rows.
+template <int NB, bool COSINE>
+__global__ __launch_bounds__(kBlock) void mfma_pack_rows_kernel(
+    const float *__restrict__ x, const float *__restrict__ norms, int n, int d,
+    uint4 *__restrict__ out) {
+  typedef MfmaShape<NB> S;
+  const size_t id = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  if (id >= (size_t)n * S::UNITS)
+    return;
+  const int row = (int)(id / S::UNITS);
+  const int unit = (int)(id - (size_t)row * S::UNITS);
+  const bool lo_part = unit >= S::HI;
+  const int c0 = 8 * (lo_part ? unit - S::HI : unit);
+  const float nv = norms[row];
+  // coordinates enter scaled by `scale` (0: not at all); `aug` is w
+  float scale, aug;
+  if (COSINE) {
+    if (!(nv > 0.0f)) { // a NaN distance anyway: never a candidate
+      scale = 0.0f;
+      aug = 1.7e38f;
+    } else if (nv == __builtin_inff()) { // always looked at
+      scale = 0.0f;
+      aug = -1e38f;
+    } else {
+      scale = 1.0f / nv;
+      aug = 1.0f;
+    }
+  } else {
+    if (!(nv <= kFilterNormLimit)) {
+      scale = 0.0f;
+      aug = -1e38f;
+    } else {
+      scale = 1.0f;
+      aug = nv * (float)(1.0 - mfma_filter_eps(d));
+    }
+  }
+  uint32_t part[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int c = c0 + e;
+    float v = 0.0f;
+    if (c < d)
+      v = scale != 0.0f ? x[(size_t)row * d + c] * scale : 0.0f;
+    uint32_t hi, lo;
+    mc_split(v, hi, lo);
+    if (!lo_part) {
+      // the augmented components: w in two parts, then 1 twice
+      if (c == S::P - 4 || c == S::P - 3) {
+        uint32_t whi, wlo = 0;
+        if (__builtin_fabsf(aug) < 1e37f)
+          mc_split(aug, whi, wlo);
+        else
+          whi = __float_as_uint(aug) >> 16;
+        hi = (c == S::P - 4) ? whi : wlo;
+      } else if (c >= S::P - 2) {
+        hi = 0x3f80u;
+      }
+    }
+    part[e] = lo_part ? lo : hi;
+  }
+  out[id] = make_uint4(part[0] | (part[1] << 16), part[2] | (part[3] << 16),
+                       part[4] | (part[5] << 16), part[6] | (part[7] << 16));
 }
 
 // A lane's walk over the rows it has parked, in ascending order.
@@ -109,21 +203,21 @@ struct MfmaWalk {
   int base;         // the lane's first row of that entry's step
 };
 
-// STEPS = matrix-core steps per 32 rows: 2 STEPS >= d + 2 components (the
-// coordinates, w, and the last one for the cut).
-template <int STEPS, int K, bool COSINE>
+// NB = blocks of 16 components per row: the coordinates (d <= 16 (NB - 1)) and
+// one block with the augmented components.
+template <int NB, int K, bool COSINE>
 __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
-  constexpr int DP = 2 * STEPS; // padded number of components (with w)
-  constexpr int RS = DP + 4;    // LDS row stride (floats), keeps b128 reads
-                                // of 8 neighbouring rows on distinct banks
+  typedef MfmaShape<NB> S;
+  constexpr int UNITS = S::UNITS;
+  constexpr int RSU = S::RSU;
   constexpr int TR = kMfmaRows;
   constexpr int TQ = kMfmaQueries;
-  constexpr int PER_THREAD = TR * DP / kBlock; // floats staged per thread
+  constexpr int TILE_UNITS = TR * UNITS;
+  constexpr int PER_THREAD = (TILE_UNITS + kBlock - 1) / kBlock;
   constexpr int QCAP = kMfmaDrainSteps;
   constexpr int CAP = kMfmaPassPairs;
-  static_assert(STEPS % 4 == 0 && (TR * DP) % kBlock == 0, "tile shape");
 
-  __shared__ __attribute__((aligned(16))) float xs[2][TR][RS];
+  __shared__ __attribute__((aligned(16))) uint4 xs[2][TR * RSU];
   // parked steps: (step within the batch << 16) | mask of the lane's rows
   __shared__ uint32_t queue[QCAP][kBlock];
   // dense re-rank, per wave: (query, row) pairs and their keys
@@ -133,7 +227,7 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
-  const int half = lane >> 5; // which components (parity) / which rows
+  const int half = lane >> 5; // which 8 components of a block / which rows
   const int col = lane & 31;  // query column of B, candidate row of A
 
   const int total_tiles = p.work_start[p.num_segments];
@@ -162,14 +256,31 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   const int c_count = min(x_end, c_begin + chunk_len) - c_begin;
   const int num_steps = (c_count + TR - 1) / TR;
 
-  const double eps = (double)(d + 32) * (1.0 / 4194304.0); // (d+32) * 2^-22
-  const float damp = (float)(1.0 - eps);
-  const float cos_margin = (float)(4 * d + 72) * 5.9604644775390625e-08f;
+  const double eps = mfma_filter_eps(d);
+  const float cos_margin =
+      (float)(4 * d + 72) * 5.9604644775390625e-08f + (float)eps;
 
   // ---- per-lane query state ---------------------------------------------
+  // (rows of a multiple of four components are read in 16-byte pieces, many
+  // at a time: one dependent load per component would cost a memory round
+  // trip each)
+  const bool vec4 = (d & 3) == 0;
   float ysq = 0.0f;
-  for (int c = 0; c < d; ++c)
-    ysq = __builtin_fmaf(yrow[c], yrow[c], ysq);
+  if (vec4) {
+    const float4 *y4 = reinterpret_cast<const float4 *>(yrow);
+#pragma unroll 8
+    for (int c = 0; c < d / 4; ++c) {
+      const float4 v = y4[c];
+      ysq = __builtin_fmaf(v.x, v.x, ysq);
+      ysq = __builtin_fmaf(v.y, v.y, ysq);
+      ysq = __builtin_fmaf(v.z, v.z, ysq);
+      ysq = __builtin_fmaf(v.w, v.w, ysq);
+    }
+  } else {
+#pragma unroll 8
+    for (int c = 0; c < d; ++c)
+      ysq = __builtin_fmaf(yrow[c], yrow[c], ysq);
+  }
   const float ynorm = __builtin_sqrtf(ysq);
   // what the query contributes to the filter: coordinates (scaled), or
   // nothing when the filter is switched off for it
@@ -186,19 +297,55 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
     y_scale = -2.0f;
   }
   const bool active = valid && !y_blind;
-  float yb[STEPS]; // B operands: this lane's parity of the augmented query
+  // B operands: this lane's 8 components of every block of the augmented
+  // query, hi parts (all blocks) and lo parts (coordinate blocks).  In the
+  // last block the upper lanes hold (0, 0, 0, 0, 1, 1, -cut_hi, -cut_lo); its
+  // last word is kept apart (cut_word) and put in place at the instruction.
+  mc_bf16x8_t yh[NB];
+  mc_bf16x8_t yl[NB - 1];
 #pragma unroll
-  for (int s = 0; s < STEPS; ++s) {
-    const int c = 2 * s + half;
-    float v = 0.0f;
-    if (active) {
-      if (c < d)
-        v = y_filtered ? yrow[c] * y_scale : 0.0f;
-      else if (c == d)
-        v = 1.0f;
+  for (int i = 0; i < NB; ++i) {
+    // the lane's 8 components of this block, read from clamped addresses
+    // (no load depends on a branch) and masked afterwards
+    const int cb = 16 * i + 8 * half;
+    float comp[8];
+    if (i < NB - 1) {
+      if (vec4) {
+        const float4 a =
+            *reinterpret_cast<const float4 *>(yrow + min(cb, d - 4));
+        const float4 b =
+            *reinterpret_cast<const float4 *>(yrow + min(cb + 4, d - 4));
+        comp[0] = a.x, comp[1] = a.y, comp[2] = a.z, comp[3] = a.w;
+        comp[4] = b.x, comp[5] = b.y, comp[6] = b.z, comp[7] = b.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          comp[e] = yrow[min(cb + e, d - 1)];
+      }
     }
-    yb[s] = v;
+    uint32_t hi[8], lo[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int c = cb + e;
+      float v = 0.0f;
+      if (active) {
+        if (i < NB - 1 && c < d)
+          v = y_filtered ? comp[e] * y_scale : 0.0f;
+        else if (c == S::P - 4 || c == S::P - 3)
+          v = 1.0f;
+      }
+      mc_split(v, hi[e], lo[e]);
+    }
+    yh[i] = __builtin_bit_cast(
+        mc_bf16x8_t, make_uint4(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16),
+                                hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16)));
+    if (i < NB - 1)
+      yl[i < NB - 1 ? i : 0] = __builtin_bit_cast(
+          mc_bf16x8_t,
+          make_uint4(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16),
+                     lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16)));
   }
+  uint32_t cut_word = 0; // (-cut_hi, -cut_lo) of the upper lanes
 
   double best[K];
 #pragma unroll
@@ -208,9 +355,10 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   float thresh = active ? kKnnSentinel : -__builtin_inff();
   float shared = kKnnSentinel; // bound inherited from other slices / partner
   float posted = kKnnSentinel;
-  // the last component of the rows (odd: upper lanes) is 1; the upper lanes
-  // hold -cut there (a lane without a query holds zeros everywhere and never
-  // parks)
+  // the rows' last two components are 1; the upper lanes hold the two parts
+  // of -cut', cut' = cut + 2^-15 |cut| (what the split may lose never lowers
+  // the cut), there; an infinite cut enters as the largest finite bf16 (a
+  // lane without a query holds zeros everywhere and never parks)
   auto set_thresh = [&](float v) {
     if (!active)
       return;
@@ -220,70 +368,51 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
       cut = y_filtered ? v + cos_margin : __builtin_inff();
     else
       cut = mfma_filter_cut(v, ysq, eps);
-    if (half)
-      yb[STEPS - 1] = -cut;
+    if (half) {
+      const float neg =
+          -__builtin_fmaf(__builtin_fabsf(cut), 3.0517578125e-05f, cut);
+      uint32_t hi, lo;
+      if (__builtin_fabsf(neg) < 1e38f) {
+        mc_split(neg, hi, lo);
+      } else {
+        hi = neg < 0.0f ? 0xff7fu : 0x7f7fu;
+        lo = 0;
+      }
+      cut_word = hi | (lo << 16);
+    }
   };
   set_thresh(thresh);
 
   // ---- tile staging -------------------------------------------------------
-  // thread -> row tid / 8, components tid % 8, tid % 8 + 8, ...
-  const int st_row = tid >> 3;
-  const int st_c0 = tid & 7;
-  // load_tile only issues the global loads (they are in flight during the
-  // matrix-core chain of the current tile); store_tile turns what arrived
-  // into filter operands
-  float raw[PER_THREAD];
-  float raw_norm = 0.0f;
-  bool raw_real = false;
-
-  auto load_tile = [&](int t) {
-    const int pos = t * TR + st_row;
-    const size_t g = (size_t)c_begin + pos;
-    raw_real = pos < c_count;
-    // (rows past the end and padding components read a clamped address and
-    // are masked out later)
-    const size_t gl = raw_real ? g : (size_t)c_begin;
-    raw_norm = p.x_sq[gl];
-    const float *src = p.x + gl * d + st_c0;
-#pragma unroll
-    for (int e = 0; e < PER_THREAD; ++e)
-      raw[e] = (st_c0 + 8 * e < d) ? src[8 * e] : 0.0f;
+  // a tile is TR packed rows, contiguous in global memory; load_tile only
+  // issues the loads (they are in flight during the matrix-core chain of the
+  // current tile), store_tile puts what arrived into LDS
+  uint4 raw[PER_THREAD];
+  // a padding row: zero coordinates and a huge w
+  auto pad_unit = [](int unit) {
+    return unit == S::HI - 1 ? make_uint4(0u, 0u, 0x7f00u, 0x3f803f80u)
+                             : make_uint4(0u, 0u, 0u, 0u);
   };
-  auto store_tile = [&](int buf) {
-    const float nv = raw_norm;
-    // coordinates enter the filter scaled by `scale` (0: not at all); `aug`
-    // is the augmented component
-    float scale, aug;
-    if (COSINE) {
-      if (!raw_real || !(nv > 0.0f)) { // padding, or a NaN distance anyway
-        scale = 0.0f;
-        aug = __builtin_nanf("");
-      } else if (nv == __builtin_inff()) { // always looked at
-        scale = 0.0f;
-        aug = -__builtin_inff();
-      } else {
-        scale = 1.0f / nv;
-        aug = 1.0f;
-      }
-    } else {
-      if (!raw_real) {
-        scale = 0.0f;
-        aug = __builtin_nanf("");
-      } else if (!(nv <= kFilterNormLimit)) {
-        scale = 0.0f;
-        aug = -__builtin_inff();
-      } else {
-        scale = 1.0f;
-        aug = nv * damp;
-      }
-    }
+  auto load_tile = [&](int t) {
+    const uint4 *src = p.x_pack + ((size_t)c_begin + (size_t)t * TR) * UNITS;
+    const int rows = min(TR, c_count - t * TR);
 #pragma unroll
     for (int e = 0; e < PER_THREAD; ++e) {
-      const int c = st_c0 + 8 * e;
-      float v = (scale != 0.0f && c < d) ? raw[e] * scale : 0.0f;
-      v = (c == d) ? aug : v;
-      v = (c == DP - 1) ? 1.0f : v; // times -cut
-      xs[buf][st_row][(c & 1) * STEPS + (c >> 1)] = v;
+      const int u = tid + e * kBlock;
+      if (u < TILE_UNITS) {
+        const int row = u / UNITS;
+        raw[e] = row < rows ? src[u] : pad_unit(u - row * UNITS);
+      }
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int e = 0; e < PER_THREAD; ++e) {
+      const int u = tid + e * kBlock;
+      if (u < TILE_UNITS) {
+        const int row = u / UNITS;
+        xs[buf][row * RSU + (u - row * UNITS)] = raw[e];
+      }
     }
   };
 
@@ -342,7 +471,7 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
     if ((d & 3) == 0) {
       const float4 *x4 = reinterpret_cast<const float4 *>(xr);
       const float4 *y4 = reinterpret_cast<const float4 *>(yr);
-#pragma unroll 4
+#pragma unroll 8
       for (int c = 0; c < d / 4; ++c) {
         const float4 a = x4[c];
         const float4 b = y4[c];
@@ -511,18 +640,23 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
 
     // ---- 32 x 32 filter values on the matrix cores ----------------------
     mfma_acc_t acc = {0};
-    const float *arow = &xs[buf][col][half * STEPS];
+    const uint4 *arow = &xs[buf][col * RSU + half];
 #pragma unroll
-    for (int s4 = 0; s4 < STEPS / 4; ++s4) {
-      const float4 a = *reinterpret_cast<const float4 *>(arow + 4 * s4);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, yb[4 * s4 + 0], acc, 0,
-                                                 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, yb[4 * s4 + 1], acc, 0,
-                                                 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, yb[4 * s4 + 2], acc, 0,
-                                                 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, yb[4 * s4 + 3], acc, 0,
-                                                 0, 0);
+    for (int i = 0; i < NB; ++i) {
+      const mc_bf16x8_t ah = __builtin_bit_cast(mc_bf16x8_t, arow[2 * i]);
+      if (i < NB - 1) {
+        const mc_bf16x8_t al =
+            __builtin_bit_cast(mc_bf16x8_t, arow[S::HI + 2 * i]);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, yh[i], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            ah, yl[i < NB - 1 ? i : 0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, yh[i], acc, 0, 0, 0);
+      } else {
+        uint4 b = __builtin_bit_cast(uint4, yh[i]);
+        b.w = cut_word;
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            ah, __builtin_bit_cast(mc_bf16x8_t, b), acc, 0, 0, 0);
+      }
     }
 
     // accumulator v belongs to candidate row 8 (v / 4) + 4 half + v % 4; its
@@ -557,5 +691,55 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
     }
   }
 }
+
+// Everything for one number of blocks (instantiated in its own translation
+// unit so the sizes build in parallel).
+#define PCA_KNN_MFMA_DEFINE(NB_)                                               \
+  template <int KB>                                                            \
+  static void launch_one_##NB_(const KnnMfmaParams &p, bool cosine, int grid,  \
+                               hipStream_t stream) {                           \
+    if (cosine)                                                                \
+      hipLaunchKernelGGL((knn_mfma_kernel<NB_, KB, true>), dim3(grid),         \
+                         dim3(kBlock), 0, stream, p);                          \
+    else                                                                       \
+      hipLaunchKernelGGL((knn_mfma_kernel<NB_, KB, false>), dim3(grid),        \
+                         dim3(kBlock), 0, stream, p);                          \
+  }                                                                            \
+  template <>                                                                  \
+  hipError_t launch_knn_mfma_blocks<NB_>(const KnnMfmaParams &p, int kbucket,  \
+                                         bool cosine, int grid,                \
+                                         hipStream_t stream) {                 \
+    switch (kbucket) {                                                         \
+    case 8:                                                                    \
+      launch_one_##NB_<8>(p, cosine, grid, stream);                            \
+      break;                                                                   \
+    case 16:                                                                   \
+      launch_one_##NB_<16>(p, cosine, grid, stream);                           \
+      break;                                                                   \
+    case 24:                                                                   \
+      launch_one_##NB_<24>(p, cosine, grid, stream);                           \
+      break;                                                                   \
+    case 32:                                                                   \
+      launch_one_##NB_<32>(p, cosine, grid, stream);                           \
+      break;                                                                   \
+    default:                                                                   \
+      return hipErrorInvalidValue;                                             \
+    }                                                                          \
+    return hipGetLastError();                                                  \
+  }                                                                            \
+  template <>                                                                  \
+  hipError_t launch_mfma_pack_rows<NB_>(const float *x, const float *norms,    \
+                                        int n, int d, bool cosine, uint4 *out, \
+                                        hipStream_t stream) {                  \
+    const size_t units = (size_t)n * MfmaShape<NB_>::UNITS;                    \
+    const unsigned grid = (unsigned)((units + kBlock - 1) / kBlock);           \
+    if (cosine)                                                                \
+      hipLaunchKernelGGL((mfma_pack_rows_kernel<NB_, true>), dim3(grid),       \
+                         dim3(kBlock), 0, stream, x, norms, n, d, out);        \
+    else                                                                       \
+      hipLaunchKernelGGL((mfma_pack_rows_kernel<NB_, false>), dim3(grid),      \
+                         dim3(kBlock), 0, stream, x, norms, n, d, out);        \
+    return hipGetLastError();                                                  \
+  }
 
 } // namespace pca

@@ -84,7 +84,7 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
 
 constexpr int kMfmaTileQueries = 128;
 bool knn_mfma_supported(int d, int k, bool cosine);
-size_t knn_mfma_scratch_bytes(int n, int m, int num_segments, int k);
+size_t knn_mfma_scratch_bytes(int n, int m, int d, int num_segments, int k);
 // work_start: tiles of kMfmaTileQueries queries.
 hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
                            const int *work_start, void *scratch,
