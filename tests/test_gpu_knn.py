@@ -242,11 +242,13 @@ def test_prefilter_never_drops_a_neighbour(oracle, lowd_path, d, k, case):
     assert (gd == wd).all()
 
 
-@pytest.mark.parametrize("d,k", [(2, 8), (3, 16), (4, 24), (7, 32)])
+@pytest.mark.parametrize("d,k", [(2, 8), (3, 16), (4, 24), (7, 32), (12, 8),
+                                 (16, 24), (40, 16), (128, 32)])
 @pytest.mark.parametrize("case", ["full_mantissa", "binade_edges",
                                   "norm_limit", "non_finite", "tiny_segments"])
 def test_split_bf16_filter_edge_cases(oracle, d, k, case):
-    # the matrix-core pre-filter works on bf16 hi/lo splits of the operands:
+    # the matrix-core pre-filters (low-dimensional and feature-space kernels)
+    # work on bf16 hi/lo splits of the operands:
     # values that round up across a power of two, rows around the norm above
     # which the filter is switched off, non-finite rows and queries mixed in,
     # and segments much shorter than a 32-row step
