@@ -198,6 +198,43 @@ int pca_nearest(const void *x, const void *y, const int64_t *ptr_x,
                 int64_t num_segments, int dtype, int64_t *out,
                 void *workspace, size_t workspace_bytes, void *stream);
 
+/* ------------------------------------------------------------------ fps -- */
+
+/*
+ * Farthest point sampling per segment.
+ *   src      [n, d] row-major points
+ *   ptr      [num_segments + 1] segments of src (required)
+ *   out_ptr  [num_segments + 1] first output position of every segment
+ *            (out_ptr[0] = 0); segment b receives out_ptr[b+1] - out_ptr[b]
+ *            samples.  The reference computes it as the running sum of
+ *            ceil(segment size * ratio) (csrc/cuda/fps_cuda.cu:80-83).
+ *   start    [num_segments] offset of every segment's first sample within
+ *            the segment, or NULL = its first row (random_start = false)
+ *   out      [out_ptr[num_segments]] int64 row numbers of src, per segment in
+ *            sampling order
+ *   max_segment_rows  an upper bound of the segment sizes known to the caller
+ *            (it selects the kernel: fp32 points of up to 4 dimensions in
+ *            segments of up to 16,384 rows are sampled from registers), or 0
+ *            = unknown.
+ *
+ * Stands under the reference operator
+ *   torch_cluster::fps(src, ptr, ratio, random_start)
+ *   csrc/fps.cpp:22-38 -> fps_cuda, csrc/cuda/fps_cuda.cu:68-109
+ * and reproduces fps_kernel (csrc/cuda/fps_cuda.cu:10-66): running minimum
+ * squared distances that start at 5e4 (larger distances count as 5e4), the
+ * next sample = the row with the largest running minimum, among equal ones
+ * the smallest (row - segment start) % 256, then the smallest row (what that
+ * kernel's block of 256 threads returns); row 0 when every value is NaN.
+ * dtype: PCA_F32, PCA_F64 or PCA_F16 (csrc/cuda/fps_cuda.cu:100).
+ */
+size_t pca_fps_workspace_bytes(int64_t n, int64_t d, int64_t num_segments,
+                               int64_t max_segment_rows, int dtype);
+
+int pca_fps(const void *src, const int64_t *ptr, const int64_t *out_ptr,
+            const int64_t *start, int64_t n, int64_t d, int64_t num_segments,
+            int64_t max_segment_rows, int dtype, int64_t *out, void *workspace,
+            size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

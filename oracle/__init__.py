@@ -323,6 +323,78 @@ def nearest(x, y, batch_x=None, batch_y=None, fma_mode=1):
 
 
 # --------------------------------------------------------------------------
+# fps (csrc/cuda/fps_cuda.cu, torch_cluster/fps.py)
+# --------------------------------------------------------------------------
+
+def fps_out_ptr(ptr, ratio, dtype):
+    """csrc/cuda/fps_cuda.cu:80-83: samples per example = ceil(deg * ratio)
+    evaluated in the ratio's element type (``dtype``), then the running sum
+    with a leading zero.  ``ratio``: scalar or one value per example."""
+    ptr = np.asarray(ptr, dtype=np.int64)
+    deg = np.diff(ptr)
+    ratio = np.asarray(ratio, dtype=dtype)
+    with np.errstate(over="ignore"):
+        per = np.ceil(deg.astype(dtype) * ratio).astype(np.int64)
+    return np.concatenate([[0], np.cumsum(per)]).astype(np.int64)
+
+
+def fps_op(src, ptr, ratio, start=None, fma_mode=1):
+    """``torch_cluster::fps`` (csrc/cuda/fps_cuda.cu:68-109) with
+    ``random_start=False``, or with the given start offsets per example.
+    ``src`` float32 / float64 / float16 (or uint16 bit patterns of halves)."""
+    lib = _load()
+    src = np.ascontiguousarray(src)
+    src = src.reshape(src.shape[0], -1)
+    ptr = _as_ptr(ptr)
+    nseg = ptr.size - 1
+    if src.dtype == np.uint16:
+        ratio_dtype = np.float16
+    else:
+        ratio_dtype = src.dtype
+    out_ptr = fps_out_ptr(ptr, ratio, ratio_dtype)
+    if start is None:
+        start = np.zeros(nseg, dtype=np.int64)
+    start = np.ascontiguousarray(start, dtype=np.int64)
+    out = np.empty(int(out_ptr[-1]), dtype=np.int64)
+    if src.dtype == np.float16:
+        src = src.view(np.uint16)
+    if src.dtype == np.uint16:
+        fn, mode = lib.oracle_fps_16, 0
+    elif src.dtype in _DTYPE_CODE:
+        fn, mode = getattr(lib, "oracle_fps_" + _suffix(src.dtype)), fma_mode
+    else:
+        raise TypeError(f"oracle fps: unsupported dtype {src.dtype}")
+    rc = fn(_ptr(src), _ptr(ptr), _ptr(out_ptr), _ptr(start),
+            ctypes.c_int64(src.shape[0]), ctypes.c_int64(src.shape[1]),
+            ctypes.c_int64(nseg), ctypes.c_int(int(mode)), _ptr(out))
+    if rc != 0:
+        raise RuntimeError("oracle_fps failed")
+    return out
+
+
+def fps(src, batch=None, ratio=None, random_start=True, batch_size=None,
+        ptr=None, fma_mode=1):
+    """torch_cluster/fps.py:35-108 (random_start must be False here: the
+    reference draws its start rows from the device's generator)."""
+    assert not random_start, "the oracle has no random start"
+    src = np.asarray(src)
+    if ratio is None:
+        ratio = 0.5
+    if ptr is not None:
+        return fps_op(src, np.asarray(ptr), ratio, None, fma_mode)
+    if batch is not None:
+        batch = np.asarray(batch)
+        assert src.shape[0] == batch.size
+        if batch_size is None:
+            batch_size = int(batch.max()) + 1
+        deg = np.bincount(batch, minlength=batch_size)
+        ptr_vec = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    else:
+        ptr_vec = np.array([0, src.shape[0]], dtype=np.int64)
+    return fps_op(src, ptr_vec, ratio, None, fma_mode)
+
+
+# --------------------------------------------------------------------------
 # Python entry points (torch_cluster/knn.py, torch_cluster/radius.py)
 # --------------------------------------------------------------------------
 
@@ -462,3 +534,22 @@ def ref_radius(x, y, ptr_x, ptr_y, r, max_num_neighbors,
     if e < 0:
         raise RuntimeError("reference radius_cpu raised")
     return out[:2 * e].reshape(2, e).copy()
+
+
+def ref_fps(src, ptr, ratio):
+    """The reference's CPU operator ``fps_cpu`` (csrc/cpu/fps_cpu.cpp:13-68),
+    first row of every example as start."""
+    lib = _load_ref()
+    src = _as_points(src)
+    ptr = _as_ptr(ptr)
+    out = np.empty(src.shape[0] + ptr.size, dtype=np.int64)
+    lib.ref_fps_cpu.restype = ctypes.c_int64
+    count = lib.ref_fps_cpu(_ptr(src), _ptr(ptr), ctypes.c_int64(src.shape[0]),
+                            ctypes.c_int64(src.shape[1]),
+                            ctypes.c_int64(ptr.size - 1),
+                            ctypes.c_double(float(ratio)),
+                            ctypes.c_int(_DTYPE_CODE[src.dtype]),
+                            _ptr(out), ctypes.c_int64(out.size))
+    if count < 0:
+        raise RuntimeError("ref_fps_cpu failed")
+    return out[:count].copy()

@@ -23,6 +23,11 @@
  *                          then the pairwise reduction over shared memory
  *                          (:46-59) -- so that the candidate chosen among
  *                          equal distances is the reference's
+ *   oracle_fps_*           csrc/cuda/fps_cuda.cu:10-66 (fps_kernel): the block
+ *                          of 256 threads played through in the same way, per
+ *                          sample: strided scan with the running minimum
+ *                          distances (:35-47), then the reduction over shared
+ *                          memory (:52-59), read as lock-step rounds
  *
  * Arithmetic: `fma_mode` = 1 evaluates every `acc += a * b` of the reference
  * kernels as one fused multiply-add (what a GPU compiler emits for that
@@ -40,6 +45,11 @@
  * reference's own CPU route, torch_cluster/nearest.py:122-124), float64
  * brute force, and a closed form of the tie rule (smallest distance, then
  * smallest (row - segment start) % 1024, then smallest row).
+ * oracle_fps_*: the fixture test/test_fps.py:16-63, float64 brute-force
+ * farthest point sampling on data without ties, the reference's compiled CPU
+ * operator (oracle/_ref, csrc/cpu/fps_cpu.cpp) on such data, and a closed form
+ * of the tie rule (largest clipped distance, then smallest
+ * (row - start) % 256, then smallest row).
  */
 #include <math.h>
 #include <stdint.h>
@@ -546,6 +556,87 @@ int oracle_radius_dense_16(const uint16_t *x, const uint16_t *y,
  * 87); `best = 1e38` narrows to +inf. */
 DEFINE_NEAREST(16, float, uint16_t, sqdist16(x, y, n_x, n_y, dim, mode),
                round16(1e38f, mode))
+
+/* ------------------------------------------------------------------------
+ * fps_kernel (csrc/cuda/fps_cuda.cu:10-66): farthest point sampling, one block
+ * of FPS_THREADS threads per example.  out[out_ptr[b]] is the start row
+ * (:26-28); for every further sample the threads update the running minimum
+ * distance of their rows n = start + t, start + t + 256, ... to the last
+ * sample (`dist`, initialised to 5e4 by the host wrapper, :91; squared
+ * distance by `dd += tmp * tmp` per dimension) and keep the first strictly
+ * larger value, `best` starting at -1 and `best_idx` at 0 (:32-47); the block
+ * then takes, in rounds i = 1, 2, 4, .., 128, for every t with t + i < 256
+ * the entry t + i when it is strictly larger (:52-59).  Within a round the
+ * reference's threads read and write the shared arrays without a barrier in
+ * between; the rounds are played here with all reads before all writes (the
+ * race-free reading, which is also what a block running in lock step does).
+ * `min(dist[n], dd)` is fmin (a NaN distance leaves `dist` as it is and is
+ * never `> best`).
+ * ------------------------------------------------------------------------ */
+#define FPS_THREADS 256
+
+#define DEFINE_FPS(SUFFIX, T, XT, DIST_EXPR, MIN_EXPR, INIT_EXPR)              \
+  int oracle_fps_##SUFFIX(const XT *src, const int64_t *ptr,                   \
+                          const int64_t *out_ptr, const int64_t *start,        \
+                          int64_t n_rows, int64_t dim, int64_t batch_size,     \
+                          int mode, int64_t *out) {                            \
+    T *dist = (T *)malloc(sizeof(T) * (size_t)(n_rows > 0 ? n_rows : 1));      \
+    for (int64_t i = 0; i < n_rows; i++)                                       \
+      dist[i] = (INIT_EXPR);                                                   \
+    _Pragma("omp parallel for schedule(dynamic, 1)") for (                     \
+        int64_t batch_idx = 0; batch_idx < batch_size; batch_idx++) {          \
+      T best_dist[FPS_THREADS], next_dist[FPS_THREADS];                        \
+      int64_t best_dist_idx[FPS_THREADS], next_idx[FPS_THREADS];               \
+      const int64_t start_idx = ptr[batch_idx];                                \
+      const int64_t end_idx = ptr[batch_idx + 1];                              \
+      if (out_ptr[batch_idx] >= out_ptr[batch_idx + 1])                        \
+        continue; /* (the reference writes one entry even then) */             \
+      out[out_ptr[batch_idx]] = start_idx + start[batch_idx];                  \
+      for (int64_t m = out_ptr[batch_idx] + 1; m < out_ptr[batch_idx + 1];     \
+           m++) {                                                              \
+        const int64_t old = out[m - 1];                                        \
+        for (int64_t thread_idx = 0; thread_idx < FPS_THREADS; thread_idx++) { \
+          T best = (T)-1.;                                                     \
+          int64_t best_idx = 0;                                                \
+          for (int64_t n = start_idx + thread_idx; n < end_idx;                \
+               n += FPS_THREADS) {                                             \
+            T dd = (DIST_EXPR);                                                \
+            dd = (MIN_EXPR);                                                   \
+            dist[n] = dd;                                                      \
+            if (dd > best) {                                                   \
+              best = dd;                                                       \
+              best_idx = n;                                                    \
+            }                                                                  \
+          }                                                                    \
+          best_dist[thread_idx] = best;                                        \
+          best_dist_idx[thread_idx] = best_idx;                                \
+        }                                                                      \
+        for (int64_t i = 1; i < FPS_THREADS; i *= 2) {                         \
+          for (int64_t t = 0; t < FPS_THREADS; t++) {                          \
+            next_dist[t] = best_dist[t];                                       \
+            next_idx[t] = best_dist_idx[t];                                    \
+            if ((t + i) < FPS_THREADS && best_dist[t] < best_dist[t + i]) {    \
+              next_dist[t] = best_dist[t + i];                                 \
+              next_idx[t] = best_dist_idx[t + i];                              \
+            }                                                                  \
+          }                                                                    \
+          memcpy(best_dist, next_dist, sizeof(best_dist));                     \
+          memcpy(best_dist_idx, next_idx, sizeof(best_dist_idx));              \
+        }                                                                      \
+        out[m] = best_dist_idx[0];                                             \
+      }                                                                        \
+    }                                                                          \
+    free(dist);                                                                \
+    return 0;                                                                  \
+  }
+
+/* mode: fma_mode (float, double) or the 16-bit kind (0 = IEEE half) */
+DEFINE_FPS(f32, float, float, sqdist_f32(src, src, old, n, dim, mode),
+           fminf(dist[n], dd), (float)5e4)
+DEFINE_FPS(f64, double, double, sqdist_f64(src, src, old, n, dim, mode),
+           fmin(dist[n], dd), (double)5e4)
+DEFINE_FPS(16, float, uint16_t, sqdist16(src, src, old, n, dim, mode),
+           fminf(dist[n], dd), round16(5e4f, mode))
 
 /* Host-wrapper epilogue: keep the slots whose `mask_src` entry is not -1, in
  * slot order, and stack them as [2, E] (row-major, leading dimension E).

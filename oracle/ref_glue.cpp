@@ -10,8 +10,10 @@
 // reference sources where they lie:
 //   /root/reference/csrc/cpu/knn_cpu.cpp     (knn_cpu,    :7-105)
 //   /root/reference/csrc/cpu/radius_cpu.cpp  (radius_cpu, :7-117)
+//   /root/reference/csrc/cpu/fps_cpu.cpp     (fps_cpu,    :13-68)
 // whose prototypes come from the reference headers included below
-// (csrc/cpu/knn_cpu.h:5-8, csrc/cpu/radius_cpu.h:5-9).
+// (csrc/cpu/knn_cpu.h:5-8, csrc/cpu/radius_cpu.h:5-9, csrc/cpu/fps_cpu.h).
+#include "cpu/fps_cpu.h"
 #include "cpu/knn_cpu.h"
 #include "cpu/radius_cpu.h"
 
@@ -90,6 +92,24 @@ int64_t ref_radius_cpu(const void *x, const void *y, const int64_t *ptr_x,
                         wrap_ptr(ptr_y, num_segments), r, max_num_neighbors,
                         /*num_workers=*/1, ignore_same_index != 0);
     return emit(e, out, capacity);
+  } catch (const std::exception &) {
+    return -1;
+  }
+}
+
+// fps_cpu with random_start = false; returns the number of samples or -1.
+int64_t ref_fps_cpu(const void *src, const int64_t *ptr, int64_t n, int64_t d,
+                    int64_t num_segments, double ratio, int dtype,
+                    int64_t *out, int64_t capacity) {
+  try {
+    auto r = torch::tensor(ratio, torch::TensorOptions().dtype(torch::kFloat));
+    auto idx = fps_cpu(wrap(src, n, d, dtype), *wrap_ptr(ptr, num_segments), r,
+                       /*random_start=*/false)
+                   .contiguous();
+    const int64_t count = idx.numel();
+    if (out != nullptr && count <= capacity && count > 0)
+      std::memcpy(out, idx.data_ptr<int64_t>(), sizeof(int64_t) * count);
+    return count;
   } catch (const std::exception &) {
     return -1;
   }

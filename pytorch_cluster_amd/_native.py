@@ -3,7 +3,7 @@
 * ``libpca_neighbors.so`` -- HIP kernels behind the C ABI declared in
   ``include/pca_neighbors.h`` (bound with ctypes as :data:`capi`).
 * ``_torch_ops.so`` -- registers ``torch.ops.torch_cluster.knn`` /
-  ``radius`` / ``nearest`` / ``cuda_version``, the operators the reference package loads from
+  ``radius`` / ``nearest`` / ``fps`` / ``cuda_version``, the operators the reference package loads from
   its per-operator shared objects (``torch_cluster/__init__.py:8-21``).
 
 There is no fallback: if a library is missing the import fails and says how to
@@ -52,6 +52,11 @@ C_ABI = {
     "pca_nearest": (ctypes.c_int,
                     [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_int,
                      _vp, _vp, ctypes.c_size_t, _vp]),
+    "pca_fps_workspace_bytes": (ctypes.c_size_t,
+                                [_i64, _i64, _i64, _i64, ctypes.c_int]),
+    "pca_fps": (ctypes.c_int,
+                [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_int,
+                 _vp, _vp, ctypes.c_size_t, _vp]),
 }
 
 

@@ -157,3 +157,26 @@ def nearest_launch(x, y, ptr_x=None, ptr_y=None, stream=None):
 
 def nearest_rows(x, y, ptr_x=None, ptr_y=None, stream=None) -> torch.Tensor:
     return nearest_launch(x, y, ptr_x, ptr_y, stream)[0]
+
+
+def fps_launch(src, ptr, out_ptr, num_samples: int, start=None,
+               max_segment_rows: int = 0, stream=None):
+    """Queues ``pca_fps``.  ``out_ptr``: int64 ``[B + 1]`` output positions on
+    the device, ``num_samples`` = its last entry (known to the caller).
+    Returns (out [num_samples] int64, workspace); nothing is synchronised."""
+    assert src.is_cuda and src.is_contiguous() and src.dtype in _DTYPE_CODE
+    assert ptr.dtype == torch.long and out_ptr.dtype == torch.long
+    dtype = _DTYPE_CODE[src.dtype]
+    n, d = src.shape
+    nseg = ptr.numel() - 1
+    ws_bytes = capi.pca_fps_workspace_bytes(n, d, nseg, max_segment_rows,
+                                            dtype)
+    if ws_bytes == 0:
+        ws_bytes = 256
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=src.device)
+    out = torch.empty(num_samples, dtype=torch.long, device=src.device)
+    _check(capi.pca_fps(_dev_ptr(src), _dev_ptr(ptr), _dev_ptr(out_ptr),
+                        _dev_ptr(start), n, d, nseg, max_segment_rows, dtype,
+                        _dev_ptr(out), _dev_ptr(ws), ws_bytes,
+                        _stream_handle(stream, src.device)))
+    return out, ws

@@ -558,4 +558,48 @@ int pca_nearest(const void *x, const void *y, const int64_t *ptr_x,
   return rc;
 }
 
+size_t pca_fps_workspace_bytes(int64_t n, int64_t d, int64_t num_segments,
+                               int64_t max_segment_rows, int dtype) {
+  if (n < 0 || n > kMaxRows || d < 1 || d > (1 << 20) || num_segments < 1 ||
+      !nearest_dtype_ok(dtype))
+    return 0;
+  if (pca::fps_in_registers(dtype, (int)d, max_segment_rows))
+    return 256;
+  return align256(pca::fps_dist_bytes(n)) + 256;
+}
+
+int pca_fps(const void *src, const int64_t *ptr, const int64_t *out_ptr,
+            const int64_t *start, int64_t n, int64_t d, int64_t num_segments,
+            int64_t max_segment_rows, int dtype, int64_t *out, void *workspace,
+            size_t workspace_bytes, void *stream_) {
+  g_last_error[0] = 0;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (n < 0 || n > kMaxRows || d < 1 || d > (1 << 20) || num_segments < 1 ||
+      num_segments > kMaxRows)
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "bad sizes n=%lld d=%lld num_segments=%lld", (long long)n,
+                (long long)d, (long long)num_segments);
+  if (!dtype_ok(dtype))
+    return fail(PCA_ERR_INVALID_ARGUMENT, "unknown element type %d", dtype);
+  if (!nearest_dtype_ok(dtype))
+    return fail(PCA_ERR_UNSUPPORTED,
+                "fps is built for fp32, fp64 and fp16 points");
+  if (ptr == nullptr || out_ptr == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "ptr or out_ptr is NULL");
+  if (n == 0)
+    return PCA_OK;
+  if (src == nullptr || out == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "src or out is NULL");
+  const size_t need =
+      pca_fps_workspace_bytes(n, d, num_segments, max_segment_rows, dtype);
+  if (workspace == nullptr || ((uintptr_t)workspace & 255) != 0 ||
+      workspace_bytes < need)
+    return fail(PCA_ERR_WORKSPACE, "workspace needs %zu bytes, 256-aligned",
+                need);
+  return check_launch(pca::launch_fps(dtype, src, ptr, out_ptr, start, (int)d,
+                                      (int)num_segments, max_segment_rows,
+                                      workspace, out, stream),
+                      "fps kernel");
+}
+
 } // extern "C"

@@ -1,0 +1,396 @@
+// Farthest point sampling: the `fps` operator of the reference
+// (csrc/cuda/fps_cuda.cu:10-66, fps_kernel), one workgroup of 1,024 threads
+// per example.
+//
+// What the reference computes, and what is reproduced bit for bit: the first
+// sample of an example is its start row; every further sample is the row with
+// the largest running minimum distance to the samples so far, where
+//   * distances are squared, accumulated with one fused multiply-add per
+//     dimension (`dd += tmp * tmp`; every operator rounds to 16 bits for
+//     fp16), and the running minimum starts at 5e4 for every row (the `dist`
+//     array of the host wrapper, :91) -- larger distances count as 5e4;
+//   * among rows of equal value the reference's block of 256 threads returns
+//     the one with the smallest (row - start) % 256, then the smallest row:
+//     thread t scans rows start + t, start + t + 256, ... and keeps its first
+//     strict maximum (:35-47), the reduction keeps the lower thread on ties
+//     (:52-59, read as lock-step rounds);
+//   * `best` starts at -1 and `best_idx` at 0: when no row has a value above
+//     -1 (every distance NaN) the sample is row 0.
+//
+// The sampling is a chain of dependent steps, each a pass over the example's
+// rows plus a workgroup-wide arg-max, so the time per sample is what counts.
+// fps_reg_kernel keeps the rows and their running minima in REGISTERS (up to
+// 16 rows per thread: examples of up to 16,384 rows of up to 4 dimensions),
+// reads the last sample's coordinates from LDS, and needs one barrier per
+// sample: every wave reduces (value, tie, coordinates of its best row) with
+// DPP shuffles, writes them to LDS, and after the barrier every thread picks
+// the winner among the 16 wave results.  fps_any_kernel (any size, dimension
+// and element type) streams the rows and a `dist` array from memory instead.
+#include "device_utils.hpp"
+#include "launchers.hpp"
+
+#include <hip/hip_fp16.h>
+
+namespace pca {
+
+namespace {
+
+constexpr int kFpsThreads = 1024;
+constexpr int kFpsWaves = kFpsThreads / kWave;
+constexpr uint32_t kFpsNoTie = 0xffffffffu;
+
+// Order among equal values: (row - start) % 256 first, then the row
+__device__ __forceinline__ uint32_t fps_tie(uint32_t rel) {
+  return ((rel & 255u) << 24) | (rel >> 8);
+}
+__device__ __forceinline__ uint32_t fps_rel(uint32_t tie) {
+  return ((tie & 0xffffffu) << 8) | (tie >> 24);
+}
+
+// (value, tie) a beats b
+template <typename T>
+__device__ __forceinline__ bool fps_better(T ad, uint32_t at, T bd,
+                                           uint32_t bt) {
+  return ad > bd || (ad == bd && at < bt);
+}
+
+__device__ __forceinline__ float shfl_xor_t(float v, int m) {
+  return __shfl_xor(v, m);
+}
+__device__ __forceinline__ double shfl_xor_t(double v, int m) {
+  return __shfl_xor(v, m);
+}
+
+// ---- element types ----------------------------------------------------------
+
+struct FpsF32 {
+  typedef float store_t;
+  typedef float calc_t;
+  static __device__ __forceinline__ calc_t load(store_t v) { return v; }
+  static __device__ __forceinline__ calc_t step(calc_t a, calc_t b,
+                                                calc_t acc) {
+    const calc_t t = a - b;
+    return __builtin_fmaf(t, t, acc);
+  }
+  static __device__ __forceinline__ calc_t lower(calc_t a, calc_t b) {
+    return __builtin_fminf(a, b);
+  }
+  static __device__ __forceinline__ calc_t limit() { return 5e4f; }
+};
+
+struct FpsF64 {
+  typedef double store_t;
+  typedef double calc_t;
+  static __device__ __forceinline__ calc_t load(store_t v) { return v; }
+  static __device__ __forceinline__ calc_t step(calc_t a, calc_t b,
+                                                calc_t acc) {
+    const calc_t t = a - b;
+    return __builtin_fma(t, t, acc);
+  }
+  static __device__ __forceinline__ calc_t lower(calc_t a, calc_t b) {
+    return __builtin_fmin(a, b);
+  }
+  static __device__ __forceinline__ calc_t limit() { return 5e4; }
+};
+
+// c10::Half arithmetic: every operator computes in float and rounds to 16
+// bits; values travel as floats that are representable halves
+struct FpsF16 {
+  typedef uint16_t store_t;
+  typedef float calc_t;
+  static __device__ __forceinline__ float r16(float v) {
+    return __half2float(__float2half_rn(v));
+  }
+  static __device__ __forceinline__ calc_t load(store_t v) {
+    return __half2float(__ushort_as_half(v));
+  }
+  static __device__ __forceinline__ calc_t step(calc_t a, calc_t b,
+                                                calc_t acc) {
+    const float t = r16(a - b);
+    const float p = r16(t * t);
+    return r16(acc + p);
+  }
+  static __device__ __forceinline__ calc_t lower(calc_t a, calc_t b) {
+    return __builtin_fminf(a, b);
+  }
+  static __device__ __forceinline__ calc_t limit() { return r16(5e4f); }
+};
+
+// ---- any size, dimension and element type -------------------------------------
+
+// dist: [n] running minima (initialised here); one workgroup per example.
+template <typename Tr>
+__global__ __launch_bounds__(kFpsThreads) void fps_any_kernel(
+    const typename Tr::store_t *__restrict__ src,
+    const int64_t *__restrict__ ptr, const int64_t *__restrict__ out_ptr,
+    const int64_t *__restrict__ start, int d,
+    typename Tr::calc_t *__restrict__ dist, int64_t *__restrict__ out) {
+  typedef typename Tr::calc_t calc_t;
+  __shared__ calc_t s_d[2][kFpsWaves];
+  __shared__ uint32_t s_t[2][kFpsWaves];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int b = blockIdx.x;
+  const int64_t start_idx = ptr[b];
+  const int64_t end_idx = ptr[b + 1];
+  const int64_t o_begin = out_ptr[b];
+  const int64_t o_end = out_ptr[b + 1];
+  if (o_begin >= o_end)
+    return;
+
+  for (int64_t n = start_idx + tid; n < end_idx; n += kFpsThreads)
+    dist[n] = Tr::limit();
+  int64_t old = start_idx + (start ? start[b] : 0);
+  if (tid == 0)
+    out[o_begin] = old;
+
+  for (int64_t m = o_begin + 1; m < o_end; ++m) {
+    const int par = (int)(m & 1);
+    const typename Tr::store_t *cur = src + (size_t)old * d;
+    calc_t best = (calc_t)-1;
+    uint32_t best_tie = kFpsNoTie;
+    // a thread's rows share (row - start) % 256, so its first strict
+    // maximum is its best by the tie rule as well
+    for (int64_t n = start_idx + tid; n < end_idx; n += kFpsThreads) {
+      const typename Tr::store_t *row = src + (size_t)n * d;
+      calc_t dd = 0;
+      for (int c = 0; c < d; ++c)
+        dd = Tr::step(Tr::load(cur[c]), Tr::load(row[c]), dd);
+      dd = Tr::lower(dist[n], dd);
+      dist[n] = dd;
+      if (dd > best) {
+        best = dd;
+        best_tie = fps_tie((uint32_t)(n - start_idx));
+      }
+    }
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1) {
+      const calc_t od = shfl_xor_t(best, sh);
+      const uint32_t ot = __shfl_xor(best_tie, sh);
+      if (fps_better(od, ot, best, best_tie)) {
+        best = od;
+        best_tie = ot;
+      }
+    }
+    if (lane == 0) {
+      s_d[par][wave] = best;
+      s_t[par][wave] = best_tie;
+    }
+    __syncthreads();
+    best = s_d[par][0];
+    best_tie = s_t[par][0];
+#pragma unroll
+    for (int w = 1; w < kFpsWaves; ++w) {
+      const calc_t od = s_d[par][w];
+      const uint32_t ot = s_t[par][w];
+      if (fps_better(od, ot, best, best_tie)) {
+        best = od;
+        best_tie = ot;
+      }
+    }
+    // nothing above -1: the reference's `best_idx` is still 0
+    old = best_tie != kFpsNoTie ? start_idx + (int64_t)fps_rel(best_tie) : 0;
+    if (tid == 0)
+      out[m] = old;
+  }
+}
+
+// ---- fp32, up to 4 dimensions, up to 1024 * P rows per example ----------------
+
+template <int DIM, int P>
+__global__ __launch_bounds__(kFpsThreads) void fps_reg_kernel(
+    const float *__restrict__ src, const int64_t *__restrict__ ptr,
+    const int64_t *__restrict__ out_ptr, const int64_t *__restrict__ start,
+    int d, int64_t *__restrict__ out) {
+  // per wave and parity: value, tie and coordinates of the wave's best row
+  __shared__ float s_d[2][kFpsWaves];
+  __shared__ uint32_t s_t[2][kFpsWaves];
+  __shared__ float s_x[2][kFpsWaves][DIM];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int b = blockIdx.x;
+  const int64_t start_idx = ptr[b];
+  const int count = (int)(ptr[b + 1] - start_idx);
+  const int64_t o_begin = out_ptr[b];
+  const int64_t o_end = out_ptr[b + 1];
+  if (o_begin >= o_end)
+    return;
+
+  float px[P][DIM];
+  float dist[P];
+#pragma unroll
+  for (int i = 0; i < P; ++i) {
+    const int rel = tid + i * kFpsThreads;
+#pragma unroll
+    for (int c = 0; c < DIM; ++c)
+      px[i][c] = (rel < count && c < d)
+                     ? src[(size_t)(start_idx + rel) * d + c]
+                     : 0.0f;
+    dist[i] = 5e4f;
+  }
+  const int64_t first = start_idx + (start ? start[b] : 0);
+  if (tid == 0)
+    out[o_begin] = first;
+  float cur[DIM];
+#pragma unroll
+  for (int c = 0; c < DIM; ++c)
+    cur[c] = c < d ? src[(size_t)first * d + c] : 0.0f;
+
+  for (int64_t m = o_begin + 1; m < o_end; ++m) {
+    const int par = (int)(m & 1);
+    float best = -1.0f;
+    int best_i = -1;
+    float bx[DIM];
+#pragma unroll
+    for (int c = 0; c < DIM; ++c)
+      bx[c] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < P; ++i) {
+      // (zero components beyond d add fma(0, 0, acc) = acc)
+      const float t0 = cur[0] - px[i][0];
+      float dd = t0 * t0;
+#pragma unroll
+      for (int c = 1; c < DIM; ++c) {
+        const float tc = cur[c] - px[i][c];
+        dd = __builtin_fmaf(tc, tc, dd);
+      }
+      dd = __builtin_fminf(dist[i], dd);
+      dist[i] = dd;
+      // rows of a thread share (row - start) % 256 and come in ascending
+      // order: the first strict maximum is the thread's best
+      const bool take = tid + i * kFpsThreads < count && dd > best;
+      best = take ? dd : best;
+      best_i = take ? i : best_i;
+#pragma unroll
+      for (int c = 0; c < DIM; ++c)
+        bx[c] = take ? px[i][c] : bx[c];
+    }
+    uint32_t best_tie =
+        best_i >= 0 ? fps_tie((uint32_t)(tid + best_i * kFpsThreads))
+                    : kFpsNoTie;
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1) {
+      const float od = __shfl_xor(best, sh);
+      const uint32_t ot = __shfl_xor(best_tie, sh);
+      float ox[DIM];
+#pragma unroll
+      for (int c = 0; c < DIM; ++c)
+        ox[c] = __shfl_xor(bx[c], sh);
+      const bool take = fps_better(od, ot, best, best_tie);
+      best = take ? od : best;
+      best_tie = take ? ot : best_tie;
+#pragma unroll
+      for (int c = 0; c < DIM; ++c)
+        bx[c] = take ? ox[c] : bx[c];
+    }
+    if (lane == 0) {
+      s_d[par][wave] = best;
+      s_t[par][wave] = best_tie;
+#pragma unroll
+      for (int c = 0; c < DIM; ++c)
+        s_x[par][wave][c] = bx[c];
+    }
+    __syncthreads();
+    int win = 0;
+    best = s_d[par][0];
+    best_tie = s_t[par][0];
+#pragma unroll
+    for (int w = 1; w < kFpsWaves; ++w) {
+      const float od = s_d[par][w];
+      const uint32_t ot = s_t[par][w];
+      const bool take = fps_better(od, ot, best, best_tie);
+      best = take ? od : best;
+      best_tie = take ? ot : best_tie;
+      win = take ? w : win;
+    }
+    int64_t chosen;
+    if (best_tie != kFpsNoTie) {
+      chosen = start_idx + (int64_t)fps_rel(best_tie);
+#pragma unroll
+      for (int c = 0; c < DIM; ++c)
+        cur[c] = s_x[par][win][c];
+    } else {
+      // nothing above -1: the reference's `best_idx` is still 0
+      chosen = 0;
+#pragma unroll
+      for (int c = 0; c < DIM; ++c)
+        cur[c] = c < d ? src[c] : 0.0f;
+    }
+    if (tid == 0)
+      out[m] = chosen;
+  }
+}
+
+template <int DIM>
+hipError_t launch_fps_reg(const float *src, const int64_t *ptr,
+                          const int64_t *out_ptr, const int64_t *start, int d,
+                          int num_segments, int64_t max_rows, int64_t *out,
+                          hipStream_t stream) {
+  if (max_rows <= 4 * kFpsThreads)
+    hipLaunchKernelGGL((fps_reg_kernel<DIM, 4>), dim3(num_segments),
+                       dim3(kFpsThreads), 0, stream, src, ptr, out_ptr, start,
+                       d, out);
+  else
+    hipLaunchKernelGGL((fps_reg_kernel<DIM, 16>), dim3(num_segments),
+                       dim3(kFpsThreads), 0, stream, src, ptr, out_ptr, start,
+                       d, out);
+  return hipGetLastError();
+}
+
+template <typename Tr>
+hipError_t launch_fps_any(const void *src, const int64_t *ptr,
+                          const int64_t *out_ptr, const int64_t *start, int d,
+                          int num_segments, void *dist, int64_t *out,
+                          hipStream_t stream) {
+  hipLaunchKernelGGL((fps_any_kernel<Tr>), dim3(num_segments),
+                     dim3(kFpsThreads), 0, stream,
+                     static_cast<const typename Tr::store_t *>(src), ptr,
+                     out_ptr, start, d,
+                     static_cast<typename Tr::calc_t *>(dist), out);
+  return hipGetLastError();
+}
+
+} // namespace
+
+bool fps_in_registers(int dtype, int d, int64_t max_rows) {
+  return dtype == 0 && d >= 1 && d <= 4 && max_rows >= 1 &&
+         max_rows <= 16 * kFpsThreads;
+}
+
+size_t fps_dist_bytes(int64_t n) { return sizeof(double) * (size_t)n; }
+
+hipError_t launch_fps(int dtype, const void *src, const int64_t *ptr,
+                      const int64_t *out_ptr, const int64_t *start, int d,
+                      int num_segments, int64_t max_rows, void *dist,
+                      int64_t *out, hipStream_t stream) {
+  if (fps_in_registers(dtype, d, max_rows)) {
+    const float *s = static_cast<const float *>(src);
+    if (d <= 2)
+      return launch_fps_reg<2>(s, ptr, out_ptr, start, d, num_segments,
+                               max_rows, out, stream);
+    if (d == 3)
+      return launch_fps_reg<3>(s, ptr, out_ptr, start, d, num_segments,
+                               max_rows, out, stream);
+    return launch_fps_reg<4>(s, ptr, out_ptr, start, d, num_segments, max_rows,
+                             out, stream);
+  }
+  switch (dtype) {
+  case 0:
+    return launch_fps_any<FpsF32>(src, ptr, out_ptr, start, d, num_segments,
+                                  dist, out, stream);
+  case 1:
+    return launch_fps_any<FpsF64>(src, ptr, out_ptr, start, d, num_segments,
+                                  dist, out, stream);
+  case 2:
+    return launch_fps_any<FpsF16>(src, ptr, out_ptr, start, d, num_segments,
+                                  dist, out, stream);
+  default:
+    return hipErrorInvalidValue;
+  }
+}
+
+} // namespace pca

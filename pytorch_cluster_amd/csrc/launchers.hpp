@@ -125,6 +125,19 @@ hipError_t launch_nearest_any(int dtype, const SearchInput &in,
                               const int *work_start, int grid_bound,
                               int64_t *out, hipStream_t stream);
 
+// --- fps.hip ---------------------------------------------------------------
+
+// fp32 rows of up to 4 dimensions in examples of up to 16,384 rows are sampled
+// from registers; everything else streams `dist` ([n], fps_dist_bytes) and
+// the rows from memory.
+bool fps_in_registers(int dtype, int d, int64_t max_rows);
+size_t fps_dist_bytes(int64_t n);
+// One workgroup per example.  start: NULL = first row of every example.
+hipError_t launch_fps(int dtype, const void *src, const int64_t *ptr,
+                      const int64_t *out_ptr, const int64_t *start, int d,
+                      int num_segments, int64_t max_rows, void *dist,
+                      int64_t *out, hipStream_t stream);
+
 // --- radius_mc.hip ---------------------------------------------------------
 
 constexpr int kRadiusMcTileQueries = 128;

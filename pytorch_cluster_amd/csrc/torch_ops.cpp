@@ -1,7 +1,8 @@
 // TorchScript operator binding: registers `torch_cluster::knn`,
-// `torch_cluster::radius` and `torch_cluster::nearest` with the reference's
-// operator signatures (csrc/knn.cpp:22-40, csrc/radius.cpp:22-39,
-// csrc/nearest.cpp:22-39) on top of the C ABI in
+// `torch_cluster::radius`, `torch_cluster::nearest` and `torch_cluster::fps`
+// with the reference's operator signatures (csrc/knn.cpp:22-40,
+// csrc/radius.cpp:22-39, csrc/nearest.cpp:22-39, csrc/fps.cpp:22-41) on top of
+// the C ABI in
 // include/pca_neighbors.h.  Tensor validation, allocation through PyTorch's
 // caching allocator, the current HIP stream and the single host read of the
 // edge count live here; the kernels never see a torch type.
@@ -285,6 +286,61 @@ at::Tensor nearest(at::Tensor x, at::Tensor y, at::Tensor ptr_x,
   return out;
 }
 
+// csrc/fps.cpp:22-36 -> fps_cuda (csrc/cuda/fps_cuda.cu:68-109): samples per
+// example = ceil(deg * ratio) in the ratio's element type, random start rows
+// from the device generator, one host read for the output size (here the
+// largest example comes with it and selects the kernel).
+at::Tensor fps(at::Tensor src, at::Tensor ptr, at::Tensor ratio,
+               bool random_start) {
+  PCA_CHECK_GPU(src);
+  PCA_CHECK_GPU(ptr);
+  PCA_CHECK_GPU(ratio);
+  PCA_CHECK_INPUT(ptr.dim() == 1);
+  PCA_CHECK_INPUT(ptr.numel() >= 2);
+  PCA_CHECK_INPUT(src.dim() >= 1);
+  DeviceScope scope(src.get_device());
+  src = src.view({src.size(0), -1}).contiguous();
+  ptr = ptr.to(at::kLong).contiguous();
+  const int64_t batch_size = ptr.numel() - 1;
+
+  auto deg = ptr.narrow(0, 1, batch_size) - ptr.narrow(0, 0, batch_size);
+  auto out_ptr = deg.toType(ratio.scalar_type()) * ratio;
+  out_ptr = out_ptr.ceil().toType(at::kLong).cumsum(0);
+  out_ptr = at::cat({at::zeros({1}, ptr.options()), out_ptr}, 0).contiguous();
+
+  at::Tensor start;
+  if (random_start) {
+    start = at::rand({batch_size}, src.options());
+    start = (start * deg.toType(ratio.scalar_type())).toType(at::kLong);
+    start = start.contiguous();
+  }
+
+  // [number of samples, largest example] in one read
+  auto sizes = at::stack({out_ptr[-1], deg.max()}).cpu();
+  const int64_t out_size = sizes[0].item<int64_t>();
+  const int64_t max_rows = sizes[1].item<int64_t>();
+  auto out = at::empty({out_size}, ptr.options());
+  const int64_t n = src.size(0);
+  if (n == 0 || out_size == 0)
+    return out;
+  const int64_t d = src.size(1);
+  const int dtype = dtype_code(src);
+  TORCH_CHECK(dtype != PCA_BF16, "fps is not implemented for 'BFloat16'");
+  const size_t ws_bytes =
+      pca_fps_workspace_bytes(n, d, batch_size, max_rows, dtype);
+  TORCH_CHECK(ws_bytes > 0, "problem size not supported");
+  auto workspace =
+      at::empty({(int64_t)ws_bytes}, src.options().dtype(at::kByte));
+  hipStream_t stream =
+      c10::hip::getCurrentHIPStream(src.get_device()).stream();
+  check_status(pca_fps(src.data_ptr(), ptr.data_ptr<int64_t>(),
+                       out_ptr.data_ptr<int64_t>(),
+                       random_start ? start.data_ptr<int64_t>() : nullptr, n,
+                       d, batch_size, max_rows, dtype, out.data_ptr<int64_t>(),
+                       workspace.data_ptr(), ws_bytes, stream));
+  return out;
+}
+
 // The stock loader of the reference package calls this
 // (torch_cluster/__init__.py:23, csrc/version.cpp:26-41).
 int64_t cuda_version() { return HIP_VERSION; }
@@ -301,6 +357,9 @@ TORCH_LIBRARY(torch_cluster, m) {
         &radius);
   m.def("nearest(Tensor x, Tensor y, Tensor ptr_x, Tensor ptr_y) -> Tensor",
         &nearest);
+  m.def("fps(Tensor src, Tensor ptr, Tensor ratio, bool random_start) -> "
+        "Tensor",
+        &fps);
   m.def("cuda_version() -> int", &cuda_version);
 }
 
