@@ -150,6 +150,17 @@ def other_configs(torch, pca, testing, dev):
         "ms": ms, "rows_per_s": x.shape[0] / ms * 1e3,
         "kernel_ms": kernel_ms,
         "kernel_tflops": 9 * pairs / kernel_ms / 1e9}
+    # fps: the sampling step that precedes radius / knn in a set-abstraction
+    # layer; a quarter of every cloud, first row as start
+    for clouds, points in ((16, 4096), (8, 16384)):
+        pts = testing.uniform_batched(0, clouds, points)["x"].to(dev)
+        ptr = (torch.arange(clouds + 1) * points).to(dev)
+        ratio = torch.tensor(0.25, device=dev)
+        ms, out = median_ms(
+            lambda: torch.ops.torch_cluster.fps(pts, ptr, ratio, False), 5)
+        report["fps %dx%d ratio 0.25" % (clouds, points)] = {
+            "ms": ms, "samples": int(out.numel()),
+            "us_per_sample_step": ms * 1e3 / (points // 4)}
     return report
 
 

@@ -21,11 +21,13 @@
 // rows plus a workgroup-wide arg-max, so the time per sample is what counts.
 // fps_reg_kernel keeps the rows and their running minima in REGISTERS (up to
 // 16 rows per thread: examples of up to 16,384 rows of up to 4 dimensions),
-// reads the last sample's coordinates from LDS, and needs one barrier per
-// sample: every wave reduces (value, tie, coordinates of its best row) with
-// DPP shuffles, writes them to LDS, and after the barrier every thread picks
-// the winner among the 16 wave results.  fps_any_kernel (any size, dimension
-// and element type) streams the rows and a `dist` array from memory instead.
+// and needs one barrier per sample: every wave finds its best row with two
+// reductions of 32-bit keys by data-parallel lane shifts (value, then tie),
+// the lane that holds it writes value, tie and coordinates to LDS, and after
+// the barrier every row of 16 lanes picks the winner among the 16 wave
+// results the same way and reads its coordinates.  fps_any_kernel (any size,
+// dimension and element type) streams the rows and a `dist` array from memory
+// instead.
 #include "device_utils.hpp"
 #include "launchers.hpp"
 
@@ -60,6 +62,27 @@ __device__ __forceinline__ float shfl_xor_t(float v, int m) {
 __device__ __forceinline__ double shfl_xor_t(double v, int m) {
   return __shfl_xor(v, m);
 }
+
+// Largest value of a wave / of every row of 16 lanes, by data-parallel
+// primitives (one fused shift-and-max instruction per step; lanes without a
+// source take 0, the smallest value).  The wave's result is uniform.
+#define PCA_DPP_UMAX(v, ctrl, rows)                                            \
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(v), ctrl, rows,    \
+                                                   0xf, false))
+__device__ __forceinline__ uint32_t row16_umax(uint32_t v) {
+  PCA_DPP_UMAX(v, 0x111, 0xf); // row_shr:1
+  PCA_DPP_UMAX(v, 0x112, 0xf); // row_shr:2
+  PCA_DPP_UMAX(v, 0x114, 0xf); // row_shr:4
+  PCA_DPP_UMAX(v, 0x118, 0xf); // row_shr:8
+  return v; // lane 15 of every row holds the row's maximum
+}
+__device__ __forceinline__ uint32_t wave_umax(uint32_t v) {
+  v = row16_umax(v);
+  PCA_DPP_UMAX(v, 0x142, 0xa); // row_bcast:15 into rows 1 and 3
+  PCA_DPP_UMAX(v, 0x143, 0xc); // row_bcast:31 into rows 2 and 3
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+#undef PCA_DPP_UMAX
 
 // ---- element types ----------------------------------------------------------
 
@@ -204,10 +227,12 @@ __global__ __launch_bounds__(kFpsThreads) void fps_reg_kernel(
     const float *__restrict__ src, const int64_t *__restrict__ ptr,
     const int64_t *__restrict__ out_ptr, const int64_t *__restrict__ start,
     int d, int64_t *__restrict__ out) {
-  // per wave and parity: value, tie and coordinates of the wave's best row
-  __shared__ float s_d[2][kFpsWaves];
-  __shared__ uint32_t s_t[2][kFpsWaves];
+  // per wave and parity: value (as an ordered unsigned number, 0 = none),
+  // complemented tie and coordinates of the wave's best row
+  __shared__ uint32_t s_v[2][kFpsWaves];
+  __shared__ uint32_t s_nt[2][kFpsWaves];
   __shared__ float s_x[2][kFpsWaves][DIM];
+  static_assert(kFpsWaves == 16, "one row of 16 lanes picks the winner");
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -269,47 +294,36 @@ __global__ __launch_bounds__(kFpsThreads) void fps_reg_kernel(
       for (int c = 0; c < DIM; ++c)
         bx[c] = take ? px[i][c] : bx[c];
     }
-    uint32_t best_tie =
-        best_i >= 0 ? fps_tie((uint32_t)(tid + best_i * kFpsThreads))
-                    : kFpsNoTie;
-#pragma unroll
-    for (int sh = 1; sh < kWave; sh <<= 1) {
-      const float od = __shfl_xor(best, sh);
-      const uint32_t ot = __shfl_xor(best_tie, sh);
-      float ox[DIM];
-#pragma unroll
-      for (int c = 0; c < DIM; ++c)
-        ox[c] = __shfl_xor(bx[c], sh);
-      const bool take = fps_better(od, ot, best, best_tie);
-      best = take ? od : best;
-      best_tie = take ? ot : best_tie;
-#pragma unroll
-      for (int c = 0; c < DIM; ++c)
-        bx[c] = take ? ox[c] : bx[c];
-    }
-    if (lane == 0) {
-      s_d[par][wave] = best;
-      s_t[par][wave] = best_tie;
+    // values are -1 (nothing) or >= 0: their bit patterns, with the top bit
+    // set, order like the values; ties go to the smallest tie number, i.e.
+    // the largest complement
+    const uint32_t key =
+        best_i >= 0 ? (__float_as_uint(best) | 0x80000000u) : 0u;
+    const uint32_t ntie =
+        best_i >= 0 ? ~fps_tie((uint32_t)(tid + best_i * kFpsThreads)) : 0u;
+    const uint32_t wave_key = wave_umax(key);
+    const uint32_t wave_ntie = wave_umax(key == wave_key ? ntie : 0u);
+    // (tie numbers are unique: exactly one lane matches when there is a key)
+    if (wave_key != 0u ? (key == wave_key && ntie == wave_ntie) : lane == 0) {
+      s_v[par][wave] = wave_key;
+      s_nt[par][wave] = wave_ntie;
 #pragma unroll
       for (int c = 0; c < DIM; ++c)
         s_x[par][wave][c] = bx[c];
     }
     __syncthreads();
-    int win = 0;
-    best = s_d[par][0];
-    best_tie = s_t[par][0];
-#pragma unroll
-    for (int w = 1; w < kFpsWaves; ++w) {
-      const float od = s_d[par][w];
-      const uint32_t ot = s_t[par][w];
-      const bool take = fps_better(od, ot, best, best_tie);
-      best = take ? od : best;
-      best_tie = take ? ot : best_tie;
-      win = take ? w : win;
-    }
+    // every row of 16 lanes looks at the 16 wave results
+    const uint32_t ev = s_v[par][lane & 15];
+    const uint32_t ent = s_nt[par][lane & 15];
+    const uint32_t top_key =
+        (uint32_t)__builtin_amdgcn_readlane((int)row16_umax(ev), 15);
+    const uint32_t top_ntie = (uint32_t)__builtin_amdgcn_readlane(
+        (int)row16_umax(ev == top_key ? ent : 0u), 15);
     int64_t chosen;
-    if (best_tie != kFpsNoTie) {
-      chosen = start_idx + (int64_t)fps_rel(best_tie);
+    if (top_key != 0u) {
+      const uint64_t who = __ballot(ev == top_key && ent == top_ntie);
+      const int win = (__builtin_ctzll(who)) & 15;
+      chosen = start_idx + (int64_t)fps_rel(~top_ntie);
 #pragma unroll
       for (int c = 0; c < DIM; ++c)
         cur[c] = s_x[par][win][c];
