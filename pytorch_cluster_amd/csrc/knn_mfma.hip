@@ -83,8 +83,9 @@ int mfma_blocks(int d) {
 
 size_t mfma_pack_bytes(int n, int d) {
   const int nb = mfma_blocks(d);
-  const size_t units = 2 * nb + 2 * (nb - 1); // MfmaShape<nb>::UNITS
-  return align256(sizeof(uint4) * units * (size_t)n);
+  const size_t units = 2 * nb + 2 * (nb - 1) + 1; // MfmaShape<nb>::RSU
+  // (one tile of spare rows: the last tile of a slice is read in full)
+  return align256(sizeof(uint4) * units * ((size_t)n + kMfmaRows));
 }
 
 } // namespace

@@ -77,7 +77,7 @@ namespace pca {
 
 constexpr int kMfmaQueries = 128;   // queries per workgroup
 constexpr int kMfmaRows = 32;       // candidates per step
-constexpr int kMfmaDrainSteps = 16; // steps between drains (= queue entries)
+constexpr int kMfmaDrainSteps = 8;  // steps between drains (= queue entries)
 constexpr int kMfmaPassPairs = 256; // pairs a wave evaluates per pass
 
 typedef float mfma_acc_t __attribute__((ext_vector_type(16)));
@@ -192,8 +192,10 @@ __global__ __launch_bounds__(kBlock) void mfma_pack_rows_kernel(
     }
     part[e] = lo_part ? lo : hi;
   }
-  out[id] = make_uint4(part[0] | (part[1] << 16), part[2] | (part[3] << 16),
-                       part[4] | (part[5] << 16), part[6] | (part[7] << 16));
+  // (rows are RSU units apart, like in LDS: a tile is copied as it is)
+  out[(size_t)row * S::RSU + unit] =
+      make_uint4(part[0] | (part[1] << 16), part[2] | (part[3] << 16),
+                 part[4] | (part[5] << 16), part[6] | (part[7] << 16));
 }
 
 // A lane's walk over the rows it has parked, in ascending order.
@@ -212,12 +214,16 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   constexpr int RSU = S::RSU;
   constexpr int TR = kMfmaRows;
   constexpr int TQ = kMfmaQueries;
-  constexpr int TILE_UNITS = TR * UNITS;
-  constexpr int PER_THREAD = (TILE_UNITS + kBlock - 1) / kBlock;
+  constexpr int TILE_UNITS = TR * RSU; // a tile in global memory and in LDS
+  // 1 KB pieces of a tile (one LDS-direct load of a wave each), dealt to the
+  // four waves in turn
+  constexpr int PIECES = (TILE_UNITS + kWave - 1) / kWave;
+  constexpr int MAX_PIECES_PER_WAVE = (PIECES + 3) / 4;
+  constexpr int RING = 3; // tile buffers
   constexpr int QCAP = kMfmaDrainSteps;
   constexpr int CAP = kMfmaPassPairs;
 
-  __shared__ __attribute__((aligned(16))) uint4 xs[2][TR * RSU];
+  __shared__ __attribute__((aligned(16))) uint4 xs[RING][TR * RSU];
   // parked steps: (step within the batch << 16) | mask of the lane's rows
   __shared__ uint32_t queue[QCAP][kBlock];
   // dense re-rank, per wave: (query, row) pairs and their keys
@@ -384,36 +390,43 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   set_thresh(thresh);
 
   // ---- tile staging -------------------------------------------------------
-  // a tile is TR packed rows, contiguous in global memory; load_tile only
-  // issues the loads (they are in flight during the matrix-core chain of the
-  // current tile), store_tile puts what arrived into LDS
-  uint4 raw[PER_THREAD];
-  // a padding row: zero coordinates and a huge w
-  auto pad_unit = [](int unit) {
-    return unit == S::HI - 1 ? make_uint4(0u, 0u, 0x7f00u, 0x3f803f80u)
-                             : make_uint4(0u, 0u, 0u, 0u);
-  };
-  auto load_tile = [&](int t) {
-    const uint4 *src = p.x_pack + ((size_t)c_begin + (size_t)t * TR) * UNITS;
-    const int rows = min(TR, c_count - t * TR);
+  // A tile is TR packed rows, contiguous in global memory, and goes to LDS as
+  // it is: LDS-direct loads (16 bytes per lane, a wave fills 1 KB from the
+  // address in M0 on), no registers in between.  Tiles are requested two
+  // steps ahead; a wave's requests complete in order, so "at most the
+  // requests of one tile outstanding" means the older tile has arrived.
+  // Rows past the end of the slice are whatever follows in memory (the packed
+  // array has TR spare rows); the drain never takes them for candidates.
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  auto request_tile = [&](int t) {
+    const uint4 *src = p.x_pack + ((size_t)c_begin + (size_t)t * TR) * RSU;
+    const uint32_t dst =
+        (uint32_t)(uintptr_t)&xs[t % RING][0]; // byte offset within LDS
 #pragma unroll
-    for (int e = 0; e < PER_THREAD; ++e) {
-      const int u = tid + e * kBlock;
-      if (u < TILE_UNITS) {
-        const int row = u / UNITS;
-        raw[e] = row < rows ? src[u] : pad_unit(u - row * UNITS);
+    for (int e = 0; e < MAX_PIECES_PER_WAVE; ++e) {
+      const int piece = wave_u + 4 * e;
+      const int u = piece * kWave + lane;
+      if (piece < PIECES && u < TILE_UNITS) {
+        const uint4 *g = src + u;
+        const uint32_t base = dst + (uint32_t)piece * (kWave * 16);
+        // (M0 is written and used inside one statement; the compiler keeps
+        // nothing in it across statements)
+        asm volatile("s_mov_b32 m0, %1\n\t"
+                     "s_nop 0\n\t"
+                     "global_load_lds_dwordx4 %0, off"
+                     :
+                     : "v"(g), "s"(base)
+                     : "memory");
       }
     }
   };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int e = 0; e < PER_THREAD; ++e) {
-      const int u = tid + e * kBlock;
-      if (u < TILE_UNITS) {
-        const int row = u / UNITS;
-        xs[buf][row * RSU + (u - row * UNITS)] = raw[e];
-      }
-    }
+  // all but the newest tile's requests of this wave have completed
+  auto await_tile = [&](bool newer_in_flight) {
+    if (newer_in_flight)
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(MAX_PIECES_PER_WAVE - 1)
+                   : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
 
   // Exchange of pruning bounds between the slices of a query: the k-th best
@@ -621,11 +634,10 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
       set_thresh(__builtin_fminf(thresh, pair_thresh));
   };
 
-  if (num_steps > 0) {
-    load_tile(0);
-    store_tile(0);
-  }
-  __syncthreads();
+  if (num_steps > 0)
+    request_tile(0);
+  if (num_steps > 1)
+    request_tile(1);
   sync_bounds(); // what other slices already know
 
   // steps [batch_t0, t] are parked and not yet resolved; the first drains
@@ -633,10 +645,15 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   // every row passes
   int batch_t0 = 0;
   for (int t = 0; t < num_steps; ++t) {
-    const int buf = t & 1;
+    const int buf = t % RING;
     const bool more = t + 1 < num_steps;
-    if (more)
-      load_tile(t + 1);
+    // this wave's pieces of tile t have arrived; after the barrier so have
+    // everybody's, and everybody is done with tile t - 1, whose buffer tile
+    // t + 2 may now overwrite
+    await_tile(more);
+    __syncthreads();
+    if (t + 2 < num_steps)
+      request_tile(t + 2);
 
     // ---- 32 x 32 filter values on the matrix cores ----------------------
     mfma_acc_t acc = {0};
@@ -674,9 +691,6 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
       batch_t0 = t + 1;
     }
 
-    if (more)
-      store_tile(buf ^ 1);
-    __syncthreads();
   }
 
   // ---- results ------------------------------------------------------------
