@@ -37,8 +37,8 @@
 //
 // Selection.  A lane gathers the 16 sign bits of a 32-row step with funnel
 // shifts and, if any is set, parks (step, mask) in its LDS queue -- one write.
-// Every kMfmaDrainSteps steps a wave resolves what its lanes have parked,
-// densely: the parked (query, row) pairs of all 64 lanes are compacted into
+// When a lane runs out of queue entries (and every kMfmaMaxBatch steps at the
+// latest) a wave resolves what its lanes have parked, densely: the parked (query, row) pairs of all 64 lanes are compacted into
 // one list, lane i takes pair i, 64 + i, ... and evaluates its exact distance
 // -- direct differences, one FMA per component in ascending order
 // (csrc/cuda/knn_cuda.cu:9-28,55-66), both rows streamed from global memory
@@ -77,7 +77,8 @@ namespace pca {
 
 constexpr int kMfmaQueries = 128;   // queries per workgroup
 constexpr int kMfmaRows = 32;       // candidates per step
-constexpr int kMfmaDrainSteps = 8;  // steps between drains (= queue entries)
+constexpr int kMfmaDrainSteps = 8;  // queue entries (parked steps) per lane
+constexpr int kMfmaMaxBatch = 128;  // steps between drains at most
 constexpr int kMfmaPassPairs = 256; // pairs a wave evaluates per pass
 
 typedef float mfma_acc_t __attribute__((ext_vector_type(16)));
@@ -226,6 +227,10 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   __shared__ __attribute__((aligned(16))) uint4 xs[RING][TR * RSU];
   // parked steps: (step within the batch << 16) | mask of the lane's rows
   __shared__ uint32_t queue[QCAP][kBlock];
+  // the step after which every wave of the workgroup drains: written by
+  // lanes that are about to run out of queue entries (waves that drain
+  // together also wait for memory together)
+  __shared__ int drain_at;
   // dense re-rank, per wave: (query, row) pairs and their keys
   __shared__ int2 pairs[kBlock / kWave][CAP];
   __shared__ double results[kBlock / kWave][CAP];
@@ -638,6 +643,8 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
     request_tile(0);
   if (num_steps > 1)
     request_tile(1);
+  if (tid == 0)
+    drain_at = -1;
   sync_bounds(); // what other slices already know
 
   // steps [batch_t0, t] are parked and not yet resolved; the first drains
@@ -652,6 +659,7 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
     // t + 2 may now overwrite
     await_tile(more);
     __syncthreads();
+    const bool drain_ordered = drain_at == t;
     if (t + 2 < num_steps)
       request_tile(t + 2);
 
@@ -685,8 +693,17 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
     if (active && mask != 0) {
       queue[qn][tid] = ((uint32_t)(t - batch_t0) << 16) | mask;
       ++qn;
+      // one entry left: everybody drains after the next step
+      if (qn == QCAP - 1)
+        drain_at = t + 1;
     }
-    if (t - batch_t0 == QCAP - 1 || !more || t <= 1 || t == 3) {
+    // Parked steps are resolved when a lane of this wave has no entry left,
+    // when some lane of the workgroup announced it one step ago, after
+    // kMfmaMaxBatch steps, and at the end.  While lists fill, that is every
+    // few steps; later, when hits are rare, a drain (four memory round trips
+    // whether it holds 1 pair or 64) comes only every kMfmaMaxBatch steps.
+    if (__any(qn == QCAP) || drain_ordered ||
+        t - batch_t0 == kMfmaMaxBatch - 1 || !more || t <= 1 || t == 3) {
       drain(batch_t0 * TR);
       batch_t0 = t + 1;
     }
