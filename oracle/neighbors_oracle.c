@@ -50,6 +50,14 @@
  * operator (oracle/_ref, csrc/cpu/fps_cpu.cpp) on such data, and a closed form
  * of the tie rule (largest clipped distance, then smallest
  * (row - start) % 256, then smallest row).
+ * PARITY UNPINNED, two details of oracle_fps_*: the reference's reduction
+ * (csrc/cuda/fps_cuda.cu:52-59) reads and writes its shared arrays within a
+ * round without a barrier, so which of several rows of EQUAL value it returns
+ * can depend on the timing of its warps -- the lock-step reading restated here
+ * is one of its possible outcomes (the reference's own test sorts the result
+ * where ties occur, test/test_fps.py:46-60); and `min` with a NaN operand for
+ * fp16 (restated as fmin, as for the other element types).  Neither can be
+ * checked without an NVIDIA toolchain.
  */
 #include <math.h>
 #include <stdint.h>
