@@ -121,36 +121,38 @@ __global__ __launch_bounds__(kPlanThreads) void scan_block_sums_kernel(
     *num_edges = partial[tid];
 }
 
-// 2^group_shift consecutive threads walk the slots of one query, so that
-// reads of the slot rows and writes of the edge columns stay contiguous.
+// Both kernels below walk the slot rows of a block of queries as ONE flat
+// range (element e = slot e % slots of query e / slots): reads are contiguous
+// and independent of each other, so many are in flight per thread.
 //
 // find_self_kernel: position of the slot that holds the query's own row
 // number (at most one: the rows of a query are distinct), or -1, and the
 // number of slots without it.
 __global__ __launch_bounds__(kBlock) void find_self_kernel(
     const int *__restrict__ idx, const int *__restrict__ count, int m,
-    int slots, int group_shift, int *__restrict__ self_pos,
-    int *__restrict__ kept) {
+    int slots, int *__restrict__ self_pos, int *__restrict__ kept) {
   __shared__ int s_self[kCompactQueries];
+  __shared__ int s_count[kCompactQueries];
   const int tid = threadIdx.x;
   const int q0 = blockIdx.x * kCompactQueries;
   const int nq = min(kCompactQueries, m - q0);
   s_self[tid] = -1;
+  s_count[tid] = tid < nq ? count[q0 + tid] : 0;
   __syncthreads();
-  const int group = 1 << group_shift;
-  const int sub = tid & (group - 1);
-  const int rows_per_pass = kBlock >> group_shift;
-  for (int ql = tid >> group_shift; ql < nq; ql += rows_per_pass) {
-    const int cq = count[q0 + ql];
-    const int64_t row_base = (int64_t)(q0 + ql) * slots;
-    for (int s = sub; s < cq; s += group)
-      if (idx[row_base + s] == q0 + ql)
-        s_self[ql] = s;
+  const int *rows = idx + (size_t)q0 * slots;
+  const int total = nq * slots;
+#pragma unroll 4
+  for (int e = tid; e < total; e += kBlock) {
+    const int ql = e / slots;
+    const int sl = e - ql * slots;
+    const int v = rows[e];
+    if (sl < s_count[ql] && v == q0 + ql)
+      s_self[ql] = sl;
   }
   __syncthreads();
   if (tid < nq) {
     self_pos[q0 + tid] = s_self[tid];
-    kept[q0 + tid] = count[q0 + tid] - (s_self[tid] >= 0 ? 1 : 0);
+    kept[q0 + tid] = s_count[tid] - (s_self[tid] >= 0 ? 1 : 0);
   }
 }
 
@@ -159,8 +161,7 @@ __global__ __launch_bounds__(kBlock) void find_self_kernel(
 __global__ __launch_bounds__(kBlock) void scatter_kernel(
     const int *__restrict__ idx, const float *__restrict__ dist,
     const int *__restrict__ count, const int *__restrict__ self_pos, int m,
-    int slots, int group_shift, int x_first,
-    const int64_t *__restrict__ block_offsets,
+    int slots, int x_first, const int64_t *__restrict__ block_offsets,
     const int64_t *__restrict__ num_edges, int64_t *__restrict__ edges,
     float *__restrict__ dist_out) {
   __shared__ int lds[kBlock];
@@ -186,21 +187,22 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
   const int nq = min(kCompactQueries, m - q0);
   int64_t *first = x_first ? edges + E : edges;  // receives the query rows
   int64_t *second = x_first ? edges : edges + E; // receives the x rows
-  const int group = 1 << group_shift;
-  const int sub = tid & (group - 1);
-  const int rows_per_pass = kBlock >> group_shift;
-  for (int ql = tid >> group_shift; ql < nq; ql += rows_per_pass) {
-    const int cq = s_count[ql];
+  const int *rows = idx + (size_t)q0 * slots;
+  const float *row_dist = dist ? dist + (size_t)q0 * slots : nullptr;
+  const int span = nq * slots;
+#pragma unroll 4
+  for (int e = tid; e < span; e += kBlock) {
+    const int ql = e / slots;
+    const int sl = e - ql * slots;
     const int skip = s_self[ql];
-    const int64_t row_base = (int64_t)(q0 + ql) * slots;
-    const int64_t e0 = base + s_offset[ql];
-    // output position s reads slot s, or s + 1 from the left-out slot on
-    for (int s = sub; s < cq; s += group) {
-      const int src = s + (s >= skip ? 1 : 0);
-      first[e0 + s] = q0 + ql;
-      second[e0 + s] = idx[row_base + src];
+    // slot sl goes to position sl, or sl - 1 behind the left-out slot
+    const int pos = sl - (sl > skip ? 1 : 0);
+    if (sl != skip && pos < s_count[ql]) {
+      const int64_t o = base + s_offset[ql] + pos;
+      first[o] = q0 + ql;
+      second[o] = rows[e];
       if (dist_out)
-        dist_out[e0 + s] = dist[row_base + src];
+        dist_out[o] = row_dist[e];
     }
   }
 }
@@ -232,14 +234,10 @@ hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
   ws += align256(sizeof(int64_t) * (size_t)(blocks + 1));
   int *self_pos = reinterpret_cast<int *>(ws);
   int *kept = reinterpret_cast<int *>(ws + align256(sizeof(int) * (size_t)m));
-  int group_shift = 0;
-  while ((1 << group_shift) < dense.slots && group_shift < 8)
-    ++group_shift;
   const int *count = dense.count;
   if (drop_self) {
     hipLaunchKernelGGL(find_self_kernel, dim3(blocks), dim3(kBlock), 0, stream,
-                       dense.idx, dense.count, m, dense.slots, group_shift,
-                       self_pos, kept);
+                       dense.idx, dense.count, m, dense.slots, self_pos, kept);
     count = kept;
   }
   hipLaunchKernelGGL(block_sum_kernel, dim3(blocks), dim3(kBlock), 0, stream,
@@ -249,8 +247,8 @@ hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
   hipLaunchKernelGGL(scatter_kernel, dim3(blocks), dim3(kBlock), 0, stream,
                      dense.idx, dense.dist, count,
                      drop_self ? self_pos : (const int *)nullptr, m,
-                     dense.slots, group_shift, x_first ? 1 : 0, block_sums,
-                     num_edges, edges, dist_out);
+                     dense.slots, x_first ? 1 : 0, block_sums, num_edges,
+                     edges, dist_out);
   return hipGetLastError();
 }
 
