@@ -255,7 +255,8 @@ __global__ __launch_bounds__(kFpsThreads) void fps_reg_kernel(
       px[i][c] = (rel < count && c < d)
                      ? src[(size_t)(start_idx + rel) * d + c]
                      : 0.0f;
-    dist[i] = 5e4f;
+    // (a slot without a row holds -1: never above `best`, which starts there)
+    dist[i] = rel < count ? 5e4f : -1.0f;
   }
   const int64_t first = start_idx + (start ? start[b] : 0);
   if (tid == 0)
@@ -269,10 +270,6 @@ __global__ __launch_bounds__(kFpsThreads) void fps_reg_kernel(
     const int par = (int)(m & 1);
     float best = -1.0f;
     int best_i = -1;
-    float bx[DIM];
-#pragma unroll
-    for (int c = 0; c < DIM; ++c)
-      bx[c] = 0.0f;
 #pragma unroll
     for (int i = 0; i < P; ++i) {
       // (zero components beyond d add fma(0, 0, acc) = acc)
@@ -287,12 +284,9 @@ __global__ __launch_bounds__(kFpsThreads) void fps_reg_kernel(
       dist[i] = dd;
       // rows of a thread share (row - start) % 256 and come in ascending
       // order: the first strict maximum is the thread's best
-      const bool take = tid + i * kFpsThreads < count && dd > best;
+      const bool take = dd > best;
       best = take ? dd : best;
       best_i = take ? i : best_i;
-#pragma unroll
-      for (int c = 0; c < DIM; ++c)
-        bx[c] = take ? px[i][c] : bx[c];
     }
     // values are -1 (nothing) or >= 0: their bit patterns, with the top bit
     // set, order like the values; ties go to the smallest tie number, i.e.
@@ -304,7 +298,26 @@ __global__ __launch_bounds__(kFpsThreads) void fps_reg_kernel(
     const uint32_t wave_key = wave_umax(key);
     const uint32_t wave_ntie = wave_umax(key == wave_key ? ntie : 0u);
     // (tie numbers are unique: exactly one lane matches when there is a key)
-    if (wave_key != 0u ? (key == wave_key && ntie == wave_ntie) : lane == 0) {
+    const bool writer =
+        wave_key != 0u ? (key == wave_key && ntie == wave_ntie) : lane == 0;
+    // which of its rows the writer means: a uniform number, so every lane
+    // picks that slot of its own registers with a scalar branch (no per-row
+    // bookkeeping of coordinates in the loop above)
+    const int slot = __builtin_amdgcn_readlane(
+        best_i, (int)__builtin_ctzll(__ballot(writer)));
+    float bx[DIM];
+#pragma unroll
+    for (int c = 0; c < DIM; ++c)
+      bx[c] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < P; ++i)
+      if (slot == i) {
+        asm volatile(""); // (keeps this a branch: P - 1 of the bodies are skipped)
+#pragma unroll
+        for (int c = 0; c < DIM; ++c)
+          bx[c] = px[i][c];
+      }
+    if (writer) {
       s_v[par][wave] = wave_key;
       s_nt[par][wave] = wave_ntie;
 #pragma unroll
