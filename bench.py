@@ -150,6 +150,25 @@ def other_configs(torch, pca, testing, dev):
         "ms": ms, "rows_per_s": x.shape[0] / ms * 1e3,
         "kernel_ms": kernel_ms,
         "kernel_tflops": 9 * pairs / kernel_ms / 1e9}
+    # nearest in feature space: a code-book assignment (1M rows of 64
+    # components to 4,096 code vectors, one segment; 2 * D flop per pair)
+    g = torch.Generator().manual_seed(0)
+    codes = torch.randn(4096, 64, generator=g)
+    feats = (codes[torch.randint(0, 4096, (1 << 20,), generator=g)]
+             + 0.5 * torch.randn(1 << 20, 64, generator=g)).to(dev)
+    codes = codes.to(dev)
+    ms, out = median_ms(lambda: pca.nearest(feats, codes), 5)
+    start, stop = events.create(), events.create()
+    capi.pca_time_next_search(start, stop)
+    pca.nearest(feats, codes)
+    torch.cuda.synchronize()
+    kernel_ms = events.elapsed_ms(start, stop)
+    events.destroy(start)
+    events.destroy(stop)
+    report["nearest: 1048576 x 64 features -> 4096 code vectors"] = {
+        "ms": ms, "rows_per_s": feats.shape[0] / ms * 1e3,
+        "kernel_ms": kernel_ms,
+        "kernel_tflops": 2 * 64 * feats.shape[0] * 4096 / kernel_ms / 1e9}
     # fps: the sampling step that precedes radius / knn in a set-abstraction
     # layer; a quarter of every cloud, first row as start
     for clouds, points in ((16, 4096), (8, 16384)):

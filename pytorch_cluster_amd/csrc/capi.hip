@@ -151,9 +151,18 @@ bool nearest_dtype_ok(int dtype) {
 // (searching rows n, candidates m)
 bool nearest_low_d(int64_t d, int dtype) { return dtype == PCA_F32 && d <= 8; }
 
+// fp32, 8 < d <= 128: the matrix-core kernel of the feature-space kNN
+bool nearest_mfma(int64_t d, int dtype) {
+  return dtype == PCA_F32 && d > 8 &&
+         pca::knn_mfma_supported((int)d, 1, false);
+}
+
 size_t nearest_workspace(int64_t n, int64_t m, int64_t d,
                          int64_t num_segments, int dtype) {
   size_t bytes = align256(sizeof(int) * (size_t)(num_segments + 1));
+  if (nearest_mfma(d, dtype))
+    bytes += pca::knn_mfma_scratch_bytes((int)m, (int)n, (int)d,
+                                         (int)num_segments, 1);
   if (nearest_low_d(d, dtype)) {
     const pca::KnnLowdConfig cfg =
         pca::nearest_lowd_config((int)d, (int)m, (int)n, (int)num_segments);
@@ -526,8 +535,9 @@ int pca_nearest(const void *x, const void *y, const int64_t *ptr_x,
   Carver ws(workspace);
   int *work_start = ws.take<int>((size_t)num_segments + 1);
   const bool low_d = nearest_low_d(d, dtype);
+  const bool mfma = nearest_mfma(d, dtype);
   pca::KnnLowdConfig cfg;
-  int per_item = pca::kBlock;
+  int per_item = mfma ? pca::kMfmaTileQueries : pca::kBlock;
   if (low_d) {
     cfg = pca::nearest_lowd_config((int)d, (int)m, (int)n, (int)num_segments);
     per_item = cfg.tile_queries;
@@ -545,6 +555,17 @@ int pca_nearest(const void *x, const void *y, const int64_t *ptr_x,
                                            scratch, none, timer.start,
                                            timer.stop, stream, out),
                       "knn_lowd_mc_kernel (nearest)");
+    timer.stop = nullptr;
+    return rc;
+  }
+  if (mfma) {
+    void *scratch = ws.take<char>(pca::knn_mfma_scratch_bytes(
+        (int)m, (int)n, (int)d, (int)num_segments, 1));
+    const pca::DenseResult none{nullptr, nullptr, nullptr, 1};
+    rc = check_launch(pca::launch_knn_mfma(in, 1, false, work_start, scratch,
+                                           none, timer.start, timer.stop,
+                                           stream, out),
+                      "knn_mfma_kernel (nearest)");
     timer.stop = nullptr;
     return rc;
   }

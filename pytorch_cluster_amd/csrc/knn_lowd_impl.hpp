@@ -539,8 +539,8 @@ __global__ __launch_bounds__(kBlock) void knn_merge_kernel(KnnLowdParams p) {
       }
     }
     if (q < y_end) {
-      if constexpr (NEAREST)
-        write_nearest(best[0], q, p.ptr_x ? (int)p.ptr_x[seg] : 0,
+      if constexpr (NEAREST) // (k = 1: the one real slot is the last)
+        write_nearest(best[K - 1], q, p.ptr_x ? (int)p.ptr_x[seg] : 0,
                       p.out_nearest);
       else
         write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);

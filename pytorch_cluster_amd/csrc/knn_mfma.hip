@@ -124,7 +124,9 @@ size_t knn_mfma_scratch_bytes(int n, int m, int d, int num_segments, int k) {
 hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
                            const int *work_start, void *scratch,
                            const DenseResult &out, hipEvent_t time_start,
-                           hipEvent_t time_stop, hipStream_t stream) {
+                           hipEvent_t time_stop, hipStream_t stream,
+                           int64_t *nearest_out) {
+  const bool nearest = nearest_out != nullptr;
   const int tiles_bound =
       plan_upper_bound(in.m, in.num_segments, kMfmaQueries);
   const int chunks = knn_mfma_slices(in.n, in.m, in.num_segments);
@@ -149,7 +151,8 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
                        dim3(kBlock), 0, stream,
                        static_cast<const float *>(in.x), in.n, in.d, x_sq);
   hipLaunchKernelGGL(fill_tau_kernel, dim3((in.m + kBlock - 1) / kBlock),
-                     dim3(kBlock), 0, stream, tau, in.m, kKnnSentinel);
+                     dim3(kBlock), 0, stream, tau, in.m,
+                     nearest ? kNearestLimit : kKnnSentinel);
   {
     const float *xf = static_cast<const float *>(in.x);
     hipError_t perr;
@@ -193,7 +196,7 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   p.tau = tau;
   p.partial = partial;
 
-  const int kb = k_bucket(k);
+  const int kb = nearest ? 1 : k_bucket(k);
   const int grid = tiles_bound * chunks;
   auto launch = [&](const KnnMfmaParams &pp, int g) {
     switch (mfma_blocks(in.d)) {
@@ -233,9 +236,13 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   mp.out_idx = out.idx;
   mp.out_dist = out.dist;
   mp.out_count = out.count;
-  mp.out_nearest = nullptr;
+  mp.out_nearest = nearest_out;
   mp.x_split = nullptr;
   switch (kb) {
+  case 1:
+    hipLaunchKernelGGL((knn_merge_kernel<8, kMfmaQueries, true>),
+                       dim3(tiles_bound), dim3(kBlock), 0, stream, mp);
+    break;
   case 8:
     launch_mfma_merge<8>(mp, tiles_bound, stream);
     break;

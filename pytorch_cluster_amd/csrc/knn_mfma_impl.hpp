@@ -208,8 +208,13 @@ struct MfmaWalk {
 
 // NB = blocks of 16 components per row: the coordinates (d <= 16 (NB - 1)) and
 // one block with the augmented components.
-template <int NB, int K, bool COSINE>
+// NEAREST: the search of the `nearest` operator (one neighbour, limit 1e38,
+// the reference's order among equal distances: see device_utils.hpp); the
+// lists go through knn_merge_kernel like those of the kNN.
+template <int NB, int K, bool COSINE, bool NEAREST = false>
 __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
+  static_assert(!NEAREST || !COSINE, "nearest is Euclidean");
+  constexpr float kLimit = SearchLimit<NEAREST>::value;
   typedef MfmaShape<NB> S;
   constexpr int UNITS = S::UNITS;
   constexpr int RSU = S::RSU;
@@ -361,11 +366,11 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   double best[K];
 #pragma unroll
   for (int j = 0; j < K; ++j)
-    best[j] = (j < K - k) ? lowest_key() : empty_key();
+    best[j] = (j < K - k) ? lowest_key() : SearchLimit<NEAREST>::empty();
   // exact distances must be strictly below thresh
-  float thresh = active ? kKnnSentinel : -__builtin_inff();
-  float shared = kKnnSentinel; // bound inherited from other slices / partner
-  float posted = kKnnSentinel;
+  float thresh = active ? kLimit : -__builtin_inff();
+  float shared = kLimit; // bound inherited from other slices / partner
+  float posted = kLimit;
   // the rows' last two components are 1; the upper lanes hold the two parts
   // of -cut', cut' = cut + 2^-15 |cut| (what the split may lose never lowers
   // the cut), there; an infinite cut enters as the largest finite bf16 (a
@@ -377,8 +382,9 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
     float cut;
     if (COSINE)
       cut = y_filtered ? v + cos_margin : __builtin_inff();
-    else
-      cut = mfma_filter_cut(v, ysq, eps);
+    else // (`nearest`: a later row of EQUAL distance can still win the tie)
+      cut = mfma_filter_cut(
+          NEAREST && v < kLimit ? next_up_positive(v) : v, ysq, eps);
     if (half) {
       const float neg =
           -__builtin_fmaf(__builtin_fabsf(cut), 3.0517578125e-05f, cut);
@@ -581,7 +587,9 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
         float dist = __builtin_nanf("");
         if (pr.y >= 0) // (a padding row is never a candidate)
           dist = exact_distance(pr.x, pr.y);
-        results[wave][i] = make_key(dist, (uint32_t)pr.y);
+        results[wave][i] = make_key(
+            dist, NEAREST ? nearest_tie((uint32_t)(pr.y - x_begin))
+                          : (uint32_t)pr.y);
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
@@ -611,17 +619,18 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
           if (!__any(has))
             break;
           const bool mine = has && idx >= pass0 && idx < pass0 + CAP;
-          const double key = mine ? results[wave][idx - pass0] : empty_key();
+          const double key = mine ? results[wave][idx - pass0]
+                                  : SearchLimit<NEAREST>::empty();
           // NaN and sentinel distances fail the compare like in the
           // reference (csrc/cuda/knn_cuda.cu:48,68).  Equality passes: a
           // pass boundary can separate the two lanes' rows, so a row may
           // arrive after higher rows of its partner -- the key order
           // settles ties.
           const bool ok = mine && key_dist(key) <= thresh &&
-                          key_dist(key) < kKnnSentinel;
+                          key_dist(key) < kLimit;
           if (!__any(ok))
             continue;
-          sorted_insert<K>(best, ok ? key : empty_key());
+          sorted_insert<K>(best, ok ? key : SearchLimit<NEAREST>::empty());
           if (owner)
             thresh = __builtin_fminf(key_dist(best[K - 1]), shared);
           changed = true;
@@ -741,6 +750,10 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
                                          bool cosine, int grid,                \
                                          hipStream_t stream) {                 \
     switch (kbucket) {                                                         \
+    case 1: /* the `nearest` search: one entry of an 8-wide list */            \
+      hipLaunchKernelGGL((knn_mfma_kernel<NB_, 8, false, true>), dim3(grid),   \
+                         dim3(kBlock), 0, stream, p);                          \
+      break;                                                                   \
     case 8:                                                                    \
       launch_one_##NB_<8>(p, cosine, grid, stream);                            \
       break;                                                                   \

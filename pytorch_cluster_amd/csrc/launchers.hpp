@@ -85,11 +85,13 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
 constexpr int kMfmaTileQueries = 128;
 bool knn_mfma_supported(int d, int k, bool cosine);
 size_t knn_mfma_scratch_bytes(int n, int m, int d, int num_segments, int k);
-// work_start: tiles of kMfmaTileQueries queries.
+// work_start: tiles of kMfmaTileQueries queries.  nearest_out: the `nearest`
+// search (k = 1, Euclidean; `out` unused, [m] rows written there).
 hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
                            const int *work_start, void *scratch,
                            const DenseResult &out, hipEvent_t time_start,
-                           hipEvent_t time_stop, hipStream_t stream);
+                           hipEvent_t time_stop, hipStream_t stream,
+                           int64_t *nearest_out = nullptr);
 
 // --- knn_generic_*.hip -----------------------------------------------------
 

@@ -33,7 +33,7 @@ def matched_ptrs(rng, n, m, segments):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16])
-@pytest.mark.parametrize("d", [1, 2, 3, 4, 5, 8, 9, 16, 130])
+@pytest.mark.parametrize("d", [1, 2, 3, 4, 5, 8, 9, 16, 33, 64, 128, 130])
 @pytest.mark.parametrize("segments", [1, 5])
 def test_random_points(oracle, dtype, d, segments):
     rng = np.random.default_rng(1000 * d + segments)
@@ -50,6 +50,8 @@ def test_random_points(oracle, dtype, d, segments):
 
 @pytest.mark.parametrize("dtype,d", [(np.float32, 3), (np.float32, 2),
                                      (np.float32, 8), (np.float32, 12),
+                                     (np.float32, 40), (np.float32, 128),
+                                     (np.float32, 200),
                                      (np.float64, 3), (np.float16, 3)])
 def test_ties_follow_the_reference_block(oracle, dtype, d):
     """Integer grids: exact ties everywhere; candidate segments longer than
@@ -59,9 +61,13 @@ def test_ties_follow_the_reference_block(oracle, dtype, d):
     sizes_x = [700, 0, 64, 900]
     ptr_y = np.concatenate([[0], np.cumsum(sizes_y)]).astype(np.int64)
     ptr_x = np.concatenate([[0], np.cumsum(sizes_x)]).astype(np.int64)
-    hi = 4 if d <= 3 else 2  # few enough grid cells for duplicates
-    y = rng.integers(0, hi, (ptr_y[-1], d)).astype(dtype)
-    x = rng.integers(0, hi, (ptr_x[-1], d)).astype(dtype)
+    if d <= 3:
+        y = rng.integers(0, 4, (ptr_y[-1], d)).astype(dtype)
+        x = rng.integers(0, 4, (ptr_x[-1], d)).astype(dtype)
+    else:  # rows drawn from a small pool: duplicates in any dimension
+        pool = rng.integers(0, 3, (48, d)).astype(dtype)
+        y = pool[rng.integers(0, 48, ptr_y[-1])]
+        x = pool[rng.integers(0, 48, ptr_x[-1])]
     got = gpu_nearest(x, y, ptr_x, ptr_y)
     want = oracle.nearest_op(x, y, ptr_x, ptr_y)
     assert (got == want).all()
@@ -117,13 +123,25 @@ def test_limit_nan_and_empty_candidates(oracle):
     assert gpu_nearest(x16[:1], y16[:1], None, None).tolist() == [0]
 
 
-def test_far_apart_clusters(oracle):
+@pytest.mark.parametrize("d", [3, 32])
+def test_far_apart_clusters(oracle, d):
     """Squared distances beyond 1e10 (the kNN limit) are ordinary here."""
     rng = np.random.default_rng(3)
-    y = (rng.standard_normal((4000, 3)) * 10 + 5e6).astype(np.float32)
-    x = (rng.standard_normal((2500, 3)) * 10).astype(np.float32)
+    y = (rng.standard_normal((4000, d)) * 10 + 5e6).astype(np.float32)
+    x = (rng.standard_normal((2500, d)) * 10).astype(np.float32)
     got = gpu_nearest(x, y, None, None)
     assert (got == oracle.nearest_op(x, y, [0, 2500], [0, 4000])).all()
+
+
+def test_codebook_assignment_in_feature_space(oracle):
+    """20,000 feature rows of 64 components to the nearest of 4,096 code
+    vectors, several slices of the code book (matrix-core kernel, merge)."""
+    rng = np.random.default_rng(12)
+    y = rng.standard_normal((4096 * 5, 64)).astype(np.float32)
+    x = (y[rng.integers(0, len(y), 20000)]
+         + 0.3 * rng.standard_normal((20000, 64))).astype(np.float32)
+    got = gpu_nearest(x, y, None, None)
+    assert (got == oracle.nearest_op(x, y, [0, len(x)], [0, len(y)])).all()
 
 
 def test_unsupported_and_invalid():
