@@ -49,7 +49,7 @@ namespace {
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 int k_bucket(int k) {
-  static const int buckets[] = {8, 16, 24, 32};
+  static const int buckets[] = {8, 16, 24, 32, 48, 64};
   for (int b : buckets)
     if (k <= b)
       return b;
@@ -95,7 +95,7 @@ bool knn_mfma_supported(int d, int k, bool cosine) {
     if (env[0] == '1')
       return false;
   (void)cosine;
-  return d > 8 && d <= 128 && k >= 1 && k <= 32;
+  return d > 8 && d <= 128 && k >= 1 && k <= 64;
 }
 
 int knn_mfma_slices(int n, int m, int num_segments) {
@@ -254,6 +254,12 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
     break;
   case 32:
     launch_mfma_merge<32>(mp, tiles_bound, stream);
+    break;
+  case 48:
+    launch_mfma_merge<48>(mp, tiles_bound, stream);
+    break;
+  case 64:
+    launch_mfma_merge<64>(mp, tiles_bound, stream);
     break;
   default:
     return hipErrorInvalidValue;

@@ -1,4 +1,4 @@
-// Feature-space kNN (8 < d <= 128, k <= 32, Euclidean or cosine) on the gfx950
+// Feature-space kNN (8 < d <= 128, k <= 64, Euclidean or cosine) on the gfx950
 // matrix cores, with results bit-identical to the reference's scalar loop
 // (csrc/cuda/knn_cuda.cu:52-78).
 //
@@ -765,6 +765,12 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
       break;                                                                   \
     case 32:                                                                   \
       launch_one_##NB_<32>(p, cosine, grid, stream);                           \
+      break;                                                                   \
+    case 48:                                                                   \
+      launch_one_##NB_<48>(p, cosine, grid, stream);                           \
+      break;                                                                   \
+    case 64: /* (one wave per SIMD: the list takes 128 registers) */           \
+      launch_one_##NB_<64>(p, cosine, grid, stream);                           \
       break;                                                                   \
     default:                                                                   \
       return hipErrorInvalidValue;                                             \

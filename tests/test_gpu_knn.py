@@ -188,6 +188,9 @@ def test_cosine_parity(oracle, d, k):
 @pytest.mark.parametrize("d,k,cosine", [(9, 5, False), (16, 16, False),
                                         (17, 33, True), (33, 8, False),
                                         (128, 32, False), (128, 32, True),
+                                        (40, 33, False), (128, 48, True),
+                                        (100, 50, False), (64, 64, True),
+                                        (128, 64, False), (128, 65, False),
                                         (300, 7, False), (515, 3, True)])
 def test_parity_high_dimension(oracle, d, k, cosine):
     rng = np.random.default_rng(d * 7 + k)
