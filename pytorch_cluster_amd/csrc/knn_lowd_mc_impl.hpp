@@ -374,6 +374,42 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
     refresh_cut();
   };
 
+  // What the two lanes of a query tell each other about its final k-th
+  // distance (equality admitted: their rows interleave).
+  auto partner_bounds = [&]() {
+    // the partner's k-th distance bounds the query's final k-th distance too
+    // (equality admitted: its rows interleave with this lane's)
+    const float own = key_dist(best[K - 1]);
+    const auto both = __builtin_amdgcn_permlane32_swap(
+        __float_as_uint(own), __float_as_uint(own), false, false);
+    float partner = __uint_as_float(half ? both[0] : both[1]);
+    // So does the larger of the two lanes' (k - c)-th distances for any
+    // c <= k / 2: together the lists hold 2 (k - c) >= k rows at or below it.
+    // The lanes see every other group of rows, so with c = k / 2 this is close
+    // to the k-th distance of both lists united -- about half as many rows
+    // get past it as past a lane's own k-th distance.  (The entry is picked
+    // by a uniform branch: c takes one of five values for a list width.)
+    if (K >= 2) {
+      const int c = k >> 1;
+      float mid = kLimit;
+#pragma unroll
+      for (int cc = (K >= 8 ? K / 2 - 4 : 0); cc <= K / 2; ++cc)
+        if (cc >= 1 && cc == c) {
+          asm volatile(""); // (keeps this a branch)
+          mid = key_dist(best[K - 1 - cc]);
+        }
+      const auto mids = __builtin_amdgcn_permlane32_swap(
+          __float_as_uint(mid), __float_as_uint(mid), false, false);
+      const float partner_mid = __uint_as_float(half ? mids[0] : mids[1]);
+      partner = __builtin_fminf(partner, __builtin_fmaxf(mid, partner_mid));
+    }
+    if (valid && partner < kLimit) {
+      shared = __builtin_fminf(shared, next_up_positive(partner));
+      if (shared < thresh)
+        set_thresh(shared);
+    }
+  };
+
   // Resolves the parked candidates: in every round each lane takes the next
   // row of its parked steps (steps in the order they were parked, rows in
   // ascending order) and all 64 lanes evaluate their exact distances from the
@@ -437,17 +473,7 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
     qnext = qfirst;
     if (!changed)
       return;
-    // the partner's k-th distance bounds the query's final k-th distance too
-    // (equality admitted: its rows interleave with this lane's)
-    const float own = key_dist(best[K - 1]);
-    const auto both = __builtin_amdgcn_permlane32_swap(
-        __float_as_uint(own), __float_as_uint(own), false, false);
-    const float partner = __uint_as_float(half ? both[0] : both[1]);
-    if (valid && partner < kLimit) {
-      shared = __builtin_fminf(shared, next_up_positive(partner));
-      if (shared < thresh)
-        set_thresh(shared);
-    }
+    partner_bounds();
     refresh_cut();
   };
 
