@@ -6,24 +6,34 @@ Same signature, argument checks and errors.  The search itself is
 library; the reference's route for CPU tensors (scipy's ``vq``,
 ``torch_cluster/nearest.py:93-124``) has no counterpart here: the operator
 rejects them ("No CPU version supported", as ``csrc/nearest.cpp:33``).
+
+The reference reads from the device five times before it calls the operator
+(two sortedness tests, two ``batch.max()``, one comparison of the non-empty
+examples).  Here the same facts come back in two reads: the last entries of
+the batch vectors (their maxima if they are sorted) size the pointer arrays,
+and one vector of three flags carries the outcome of all three checks.
 """
 from typing import Optional
 
 import torch
 
 
-def _pointers(batch: Optional[torch.Tensor], rows: torch.Tensor) -> torch.Tensor:
-    """``[B + 1]`` CSR pointers of a sorted batch vector: counts per example,
-    then their running sum (``torch_cluster/nearest.py:55-63``)."""
+def _unsorted(batch: Optional[torch.Tensor], like: torch.Tensor) -> torch.Tensor:
+    """0-d bool tensor: the batch vector decreases somewhere."""
+    if batch is None or batch.numel() < 2:
+        return torch.zeros((), dtype=torch.bool, device=like.device)
+    return (batch[1:] < batch[:-1]).any()
+
+
+def _pointers(batch: Optional[torch.Tensor], rows: torch.Tensor,
+              batch_size: int) -> torch.Tensor:
+    """``[B + 1]`` CSR pointers of a sorted batch vector: ``ptr[b]`` is the
+    first row whose example id is ``>= b`` -- the running sum of the counts
+    per example that the reference forms (``torch_cluster/nearest.py:55-63``)."""
     if batch is None:
         return torch.tensor([0, rows.size(0)], device=rows.device)
-    assert rows.size(0) == batch.numel()
-    batch_size = int(batch.max()) + 1
-    deg = rows.new_zeros(batch_size, dtype=torch.long)
-    deg.scatter_add_(0, batch, torch.ones_like(batch))
-    ptr = deg.new_zeros(batch_size + 1)
-    torch.cumsum(deg, 0, out=ptr[1:])
-    return ptr
+    ids = torch.arange(batch_size + 1, device=rows.device)
+    return torch.bucketize(ids, batch)
 
 
 def nearest(
@@ -48,18 +58,44 @@ def nearest(
     x = x.view(-1, 1) if x.dim() == 1 else x
     y = y.view(-1, 1) if y.dim() == 1 else y
     assert x.size(1) == y.size(1)
+    if batch_x is not None:
+        assert x.size(0) == batch_x.numel()
+    if batch_y is not None:
+        assert y.size(0) == batch_y.numel()
 
-    if batch_x is not None and (batch_x[1:] - batch_x[:-1] < 0).any():
+    # first read: the number of examples on each side (the last entry of a
+    # sorted vector is its maximum; if it is not sorted the check below fails
+    # before the pointers are used)
+    size_x, size_y = 1, 1
+    lasts = []
+    if batch_x is not None and batch_x.numel() > 0:
+        lasts.append(batch_x[-1])
+    if batch_y is not None and batch_y.numel() > 0:
+        lasts.append(batch_y[-1])
+    if len(lasts) > 0:
+        values = torch.stack(lasts).tolist()
+        if batch_x is not None and batch_x.numel() > 0:
+            size_x = int(values[0]) + 1
+        if batch_y is not None and batch_y.numel() > 0:
+            size_y = int(values[-1]) + 1
+    bad_sizes = size_x < 1 or size_y < 1
+
+    ptr_x = _pointers(batch_x, x, max(size_x, 1))
+    ptr_y = _pointers(batch_y, y, max(size_y, 1))
+
+    # second read: the three checks of the reference, in its order
+    if ptr_x.numel() == ptr_y.numel():
+        mismatch = (((ptr_x[1:] - ptr_x[:-1]) > 0)
+                    != ((ptr_y[1:] - ptr_y[:-1]) > 0)).any()
+    else:
+        mismatch = torch.ones((), dtype=torch.bool, device=x.device)
+    flags = torch.stack([_unsorted(batch_x, x), _unsorted(batch_y, y),
+                         mismatch]).tolist()
+    if flags[0]:
         raise ValueError("'batch_x' is not sorted")
-    if batch_y is not None and (batch_y[1:] - batch_y[:-1] < 0).any():
+    if flags[1]:
         raise ValueError("'batch_y' is not sorted")
-
-    ptr_x = _pointers(batch_x, x)
-    ptr_y = _pointers(batch_y, y)
-
-    nonempty_x = (ptr_x[1:] - ptr_x[:-1]) > 0
-    nonempty_y = (ptr_y[1:] - ptr_y[:-1]) > 0
-    if not torch.equal(nonempty_x, nonempty_y):
+    if flags[2] or bad_sizes:
         raise ValueError("Some batch indices occur in 'batch_x' "
                          "that do not occur in 'batch_y'")
 
