@@ -64,9 +64,9 @@
 // The query operands stay in registers for the whole scan; the candidate rows
 // are split once per call (mfma_pack_rows_kernel: per row the hi parts of all
 // blocks, then the lo parts of the coordinate blocks, 16 bytes per lane and
-// block) and stream through LDS as they are, double-buffered, with an odd row
-// stride so that the 16-byte reads of neighbouring rows fall on distinct
-// banks.
+// block, rows an odd number of 16-byte units apart so that the reads of
+// neighbouring rows fall on distinct LDS banks) and go to a ring of three LDS
+// buffers as they are, by LDS-direct loads issued two steps ahead.
 #pragma once
 
 #include "device_utils.hpp"
@@ -108,8 +108,9 @@ template <int NB> struct MfmaShape {
   static constexpr int P = 16 * NB;          // components with the padding
   static constexpr int HI = 2 * NB;          // units of hi parts
   static constexpr int LO = 2 * (NB - 1);    // units of lo parts (coordinates)
-  static constexpr int UNITS = HI + LO;      // per row in global memory
-  static constexpr int RSU = UNITS + 1;      // LDS row stride (odd)
+  static constexpr int UNITS = HI + LO;      // units of a row that hold data
+  static constexpr int RSU = UNITS + 1;      // row stride, in memory and in LDS
+                                             // (odd: see the header)
   static constexpr int MAX_D = 16 * (NB - 1);
 };
 
@@ -216,7 +217,6 @@ __global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
   static_assert(!NEAREST || !COSINE, "nearest is Euclidean");
   constexpr float kLimit = SearchLimit<NEAREST>::value;
   typedef MfmaShape<NB> S;
-  constexpr int UNITS = S::UNITS;
   constexpr int RSU = S::RSU;
   constexpr int TR = kMfmaRows;
   constexpr int TQ = kMfmaQueries;
