@@ -220,23 +220,35 @@ __global__ __launch_bounds__(kFpsThreads) void fps_any_kernel(
   }
 }
 
-// ---- fp32, up to 4 dimensions, up to 1024 * P rows per example ----------------
+// ---- fp32, up to 4 dimensions, up to T * P rows per example -------------------
 
-template <int DIM, int P>
-__global__ __launch_bounds__(kFpsThreads) void fps_reg_kernel(
+// T = 256 S threads hold P rows each: thread t has the rows
+// t / S + 256 * ((t % S) * P + i), i < P, of its example.  Among equal values
+// the reference's order is "(row - start) % 256, then the row", which in this
+// layout reads "t, then i": the first thread wins, and inside it the first
+// slot.  Every "first of the equal ones" is therefore a count of trailing
+// zeros of a ballot, and only the values themselves go through a reduction.
+// A step costs every wave the same few dozen instructions of reduction and
+// hand-over on top of its 10 P of distances, and the waves of a SIMD take
+// turns: the launcher picks the shape that measured fastest for the row count.
+template <int DIM, int P, int T>
+__global__ __launch_bounds__(T) void fps_reg_kernel(
     const float *__restrict__ src, const int64_t *__restrict__ ptr,
     const int64_t *__restrict__ out_ptr, const int64_t *__restrict__ start,
     int d, int64_t *__restrict__ out) {
-  // per wave and parity: value (as an ordered unsigned number, 0 = none),
-  // complemented tie and coordinates of the wave's best row
+  // per wave and parity: value (as an ordered unsigned number,
+  // 0 = none), row (relative to the example) and coordinates of the wave's best
   __shared__ uint32_t s_v[2][kFpsWaves];
-  __shared__ uint32_t s_nt[2][kFpsWaves];
-  __shared__ float s_x[2][kFpsWaves][DIM];
-  static_assert(kFpsWaves == 16, "one row of 16 lanes picks the winner");
+  __shared__ uint32_t s_rel[2][kFpsWaves];
+  __shared__ float s_x[2][DIM][kFpsWaves];
+  static_assert(kFpsWaves == 16 && T % 256 == 0 && T <= kFpsThreads,
+                "one row of 16 lanes picks the winner among up to 16 waves");
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
+  constexpr int S = T / 256;
+  const int rel0 = tid / S + 256 * ((tid % S) * P);
   const int b = blockIdx.x;
   const int64_t start_idx = ptr[b];
   const int count = (int)(ptr[b + 1] - start_idx);
@@ -244,19 +256,31 @@ __global__ __launch_bounds__(kFpsThreads) void fps_reg_kernel(
   const int64_t o_end = out_ptr[b + 1];
   if (o_begin >= o_end)
     return;
+  if (T < kFpsThreads) {
+    // the entries of waves that do not run stay "nothing"
+    if (tid < 2 * kFpsWaves)
+      s_v[tid / kFpsWaves][tid % kFpsWaves] = 0u;
+    __syncthreads();
+  }
 
   float px[P][DIM];
-  float dist[P];
+  // A slot's running minimum is the high word of a 64-bit pattern whose low
+  // word is 15 - i.  Minima are -1 (no row) or in [0, 5e4]: read as doubles,
+  // the patterns of rows order by minimum first and smaller slot second, and
+  // none is a NaN or an infinity, so one 64-bit maximum per slot tracks the
+  // thread's best (the first of its largest minima) and where it is.
+  double slot_key[P];
+  static_assert(P <= 16, "low words 15 - i");
 #pragma unroll
   for (int i = 0; i < P; ++i) {
-    const int rel = tid + i * kFpsThreads;
+    const int rel = rel0 + 256 * i;
 #pragma unroll
     for (int c = 0; c < DIM; ++c)
       px[i][c] = (rel < count && c < d)
                      ? src[(size_t)(start_idx + rel) * d + c]
                      : 0.0f;
-    // (a slot without a row holds -1: never above `best`, which starts there)
-    dist[i] = rel < count ? 5e4f : -1.0f;
+    slot_key[i] = __hiloint2double(
+        __float_as_int(rel < count ? 5e4f : -1.0f), 15 - i);
   }
   const int64_t first = start_idx + (start ? start[b] : 0);
   if (tid == 0)
@@ -268,8 +292,8 @@ __global__ __launch_bounds__(kFpsThreads) void fps_reg_kernel(
 
   for (int64_t m = o_begin + 1; m < o_end; ++m) {
     const int par = (int)(m & 1);
-    float best = -1.0f;
-    int best_i = -1;
+    // (below every slot's pattern: -1 with the largest low word)
+    double best_key = __hiloint2double(__float_as_int(-1.0f), -1);
 #pragma unroll
     for (int i = 0; i < P; ++i) {
       // (zero components beyond d add fma(0, 0, acc) = acc)
@@ -280,66 +304,77 @@ __global__ __launch_bounds__(kFpsThreads) void fps_reg_kernel(
         const float tc = cur[c] - px[i][c];
         dd = __builtin_fmaf(tc, tc, dd);
       }
-      dd = __builtin_fminf(dist[i], dd);
-      dist[i] = dd;
-      // rows of a thread share (row - start) % 256 and come in ascending
-      // order: the first strict maximum is the thread's best
-      const bool take = dd > best;
-      best = take ? dd : best;
-      best_i = take ? i : best_i;
+      // fminf without its quieting of signalling NaNs, which neither operand
+      // can be (5e4, -1, or the result of arithmetic): a NaN loses to a number
+      const float before = __int_as_float(__double2hiint(slot_key[i]));
+      asm("v_min_f32 %0, %1, %2" : "=v"(dd) : "v"(before), "v"(dd));
+      slot_key[i] =
+          __hiloint2double(__float_as_int(dd), __double2loint(slot_key[i]));
+      asm("v_max_f64 %0, %1, %2"
+          : "=v"(best_key)
+          : "v"(best_key), "v"(slot_key[i]));
     }
+    const uint32_t best_bits = (uint32_t)__double2hiint(best_key);
+    const int best_i = best_bits != __float_as_uint(-1.0f)
+                           ? 15 - __double2loint(best_key)
+                           : -1;
     // values are -1 (nothing) or >= 0: their bit patterns, with the top bit
-    // set, order like the values; ties go to the smallest tie number, i.e.
-    // the largest complement
-    const uint32_t key =
-        best_i >= 0 ? (__float_as_uint(best) | 0x80000000u) : 0u;
-    const uint32_t ntie =
-        best_i >= 0 ? ~fps_tie((uint32_t)(tid + best_i * kFpsThreads)) : 0u;
+    // set, order like the values
+    const uint32_t key = best_i >= 0 ? (best_bits | 0x80000000u) : 0u;
     const uint32_t wave_key = wave_umax(key);
-    const uint32_t wave_ntie = wave_umax(key == wave_key ? ntie : 0u);
-    // (tie numbers are unique: exactly one lane matches when there is a key)
-    const bool writer =
-        wave_key != 0u ? (key == wave_key && ntie == wave_ntie) : lane == 0;
-    // which of its rows the writer means: a uniform number, so every lane
-    // picks that slot of its own registers with a scalar branch (no per-row
+    const int src_lane = (int)__builtin_ctzll(__ballot(key == wave_key));
+    // which of its rows that lane means: a uniform number, so every lane
+    // picks that slot of its own registers with scalar branches (no per-row
     // bookkeeping of coordinates in the loop above)
-    const int slot = __builtin_amdgcn_readlane(
-        best_i, (int)__builtin_ctzll(__ballot(writer)));
+    const int slot = __builtin_amdgcn_readlane(best_i, src_lane);
     float bx[DIM];
 #pragma unroll
     for (int c = 0; c < DIM; ++c)
       bx[c] = 0.0f;
-#pragma unroll
-    for (int i = 0; i < P; ++i)
-      if (slot == i) {
-        asm volatile(""); // (keeps this a branch: P - 1 of the bodies are skipped)
-#pragma unroll
-        for (int c = 0; c < DIM; ++c)
-          bx[c] = px[i][c];
-      }
-    if (writer) {
+    switch (slot) {
+#define PCA_FPS_SLOT(i_)                                                       \
+  case i_:                                                                     \
+    if (i_ < P) {                                                              \
+      _Pragma("unroll") for (int c = 0; c < DIM; ++c) bx[c] =                  \
+          px[i_ < P ? i_ : 0][c];                                              \
+    }                                                                          \
+    break;
+      PCA_FPS_SLOT(0) PCA_FPS_SLOT(1) PCA_FPS_SLOT(2) PCA_FPS_SLOT(3)
+      PCA_FPS_SLOT(4) PCA_FPS_SLOT(5) PCA_FPS_SLOT(6) PCA_FPS_SLOT(7)
+      PCA_FPS_SLOT(8) PCA_FPS_SLOT(9) PCA_FPS_SLOT(10) PCA_FPS_SLOT(11)
+      PCA_FPS_SLOT(12) PCA_FPS_SLOT(13) PCA_FPS_SLOT(14) PCA_FPS_SLOT(15)
+#undef PCA_FPS_SLOT
+    default:
+      break;
+    }
+    static_assert(P <= 16, "slots of the switch above");
+    if (lane == src_lane) {
       s_v[par][wave] = wave_key;
-      s_nt[par][wave] = wave_ntie;
+      s_rel[par][wave] = (uint32_t)(rel0 + 256 * slot);
 #pragma unroll
       for (int c = 0; c < DIM; ++c)
-        s_x[par][wave][c] = bx[c];
+        s_x[par][c][wave] = bx[c];
     }
     __syncthreads();
     // every row of 16 lanes looks at the 16 wave results
     const uint32_t ev = s_v[par][lane & 15];
-    const uint32_t ent = s_nt[par][lane & 15];
+    const uint32_t erel = s_rel[par][lane & 15];
+    float ex[DIM];
+#pragma unroll
+    for (int c = 0; c < DIM; ++c) {
+      ex[c] = s_x[par][c][lane & 15];
+      asm volatile("" : "+v"(ex[c])); // (read now, not after the reduction)
+    }
     const uint32_t top_key =
         (uint32_t)__builtin_amdgcn_readlane((int)row16_umax(ev), 15);
-    const uint32_t top_ntie = (uint32_t)__builtin_amdgcn_readlane(
-        (int)row16_umax(ev == top_key ? ent : 0u), 15);
     int64_t chosen;
     if (top_key != 0u) {
-      const uint64_t who = __ballot(ev == top_key && ent == top_ntie);
-      const int win = (__builtin_ctzll(who)) & 15;
-      chosen = start_idx + (int64_t)fps_rel(~top_ntie);
+      const int win = (int)__builtin_ctzll(__ballot(ev == top_key));
+      chosen = start_idx + (int64_t)__builtin_amdgcn_readlane((int)erel, win);
 #pragma unroll
       for (int c = 0; c < DIM; ++c)
-        cur[c] = s_x[par][win][c];
+        cur[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+            (int)__float_as_uint(ex[c]), win));
     } else {
       // nothing above -1: the reference's `best_idx` is still 0
       chosen = 0;
@@ -349,6 +384,10 @@ __global__ __launch_bounds__(kFpsThreads) void fps_reg_kernel(
     }
     if (tid == 0)
       out[m] = chosen;
+    // (in vector registers: the distance code then interleaves its rows)
+#pragma unroll
+    for (int c = 0; c < DIM; ++c)
+      asm volatile("" : "+v"(cur[c]));
   }
 }
 
@@ -357,14 +396,25 @@ hipError_t launch_fps_reg(const float *src, const int64_t *ptr,
                           const int64_t *out_ptr, const int64_t *start, int d,
                           int num_segments, int64_t max_rows, int64_t *out,
                           hipStream_t stream) {
-  if (max_rows <= 4 * kFpsThreads)
-    hipLaunchKernelGGL((fps_reg_kernel<DIM, 4>), dim3(num_segments),
-                       dim3(kFpsThreads), 0, stream, src, ptr, out_ptr, start,
-                       d, out);
+#define PCA_FPS_REG(P_, T_)                                                    \
+  hipLaunchKernelGGL((fps_reg_kernel<DIM, P_, T_>), dim3(num_segments),        \
+                     dim3(T_), 0, stream, src, ptr, out_ptr, start, d, out)
+  // (shapes by measurement: 16 examples of each size on one device)
+  if (max_rows <= 256)
+    PCA_FPS_REG(1, 256);
+  else if (max_rows <= 512)
+    PCA_FPS_REG(2, 256);
+  else if (max_rows <= 1024)
+    PCA_FPS_REG(2, 512);
+  else if (max_rows <= 2048)
+    PCA_FPS_REG(4, 512);
+  else if (max_rows <= 4096)
+    PCA_FPS_REG(8, 512);
+  else if (max_rows <= 8192)
+    PCA_FPS_REG(16, 512);
   else
-    hipLaunchKernelGGL((fps_reg_kernel<DIM, 16>), dim3(num_segments),
-                       dim3(kFpsThreads), 0, stream, src, ptr, out_ptr, start,
-                       d, out);
+    PCA_FPS_REG(16, 1024);
+#undef PCA_FPS_REG
   return hipGetLastError();
 }
 

@@ -56,6 +56,25 @@ def test_ties_and_clipping_follow_the_reference_block(oracle, dtype, d):
     assert (got == want).all()
 
 
+@pytest.mark.parametrize("rows", [1, 200, 256, 257, 512, 1000, 1024, 2047,
+                                  2048, 3000, 4096, 4097, 8192, 8193, 12000,
+                                  16384])
+@pytest.mark.parametrize("d", [2, 3, 4])
+def test_every_register_shape_resolves_ties_like_the_reference(oracle, rows, d):
+    """The register kernel's launch shape follows the largest example; points
+    on a coarse integer grid make most maxima ties, which go by
+    (row - start) % 256 first and the row second."""
+    rng = np.random.default_rng(rows + d)
+    small = max(1, rows // 3)
+    ptr = np.array([0, small, small + rows], dtype=np.int64)
+    x = rng.integers(0, 4, (ptr[-1], d)).astype(np.float32)
+    ratio = np.array([0.5, min(1.0, 150.0 / rows)])
+    start = np.array([small - 1, rows // 2], dtype=np.int64)
+    got = gpu_fps(oracle, x, ptr, ratio, start)
+    want = oracle.fps_op(x, ptr, ratio, start)
+    assert (got == want).all()
+
+
 def test_register_and_streaming_kernels_agree(oracle):
     """Examples of up to 4,096 / 16,384 rows are sampled from registers,
     larger ones (or an unknown bound) from memory: same samples."""
