@@ -222,15 +222,18 @@ __global__ __launch_bounds__(kFpsThreads) void fps_any_kernel(
 
 // ---- fp32, up to 4 dimensions, up to T * P rows per example -------------------
 
-// T = 256 S threads hold P rows each: thread t has the rows
-// t / S + 256 * ((t % S) * P + i), i < P, of its example.  Among equal values
-// the reference's order is "(row - start) % 256, then the row", which in this
-// layout reads "t, then i": the first thread wins, and inside it the first
-// slot.  Every "first of the equal ones" is therefore a count of trailing
-// zeros of a ballot, and only the values themselves go through a reduction.
-// A step costs every wave the same few dozen instructions of reduction and
-// hand-over on top of its 10 P of distances, and the waves of a SIMD take
-// turns: the launcher picks the shape that measured fastest for the row count.
+// T threads hold P rows each.  With T = 256 S, thread t has the rows
+// t / S + 256 * ((t % S) * P + i), i < P, of its example; a single wave
+// (T = 64) gives thread t the rows 4 t + i / (P / 4) + 256 * (i % (P / 4)).
+// Among equal values the reference's order is "(row - start) % 256, then the
+// row", which in these layouts reads "t, then i": the first thread wins, and
+// inside it the first slot.  Every "first of the equal ones" is therefore a
+// count of trailing zeros of a ballot, and only the values themselves go
+// through a reduction.  A step costs every wave the same few dozen
+// instructions of reduction and hand-over on top of its 8 P of distances,
+// and the waves of a SIMD take turns: the launcher picks the shape that
+// measured fastest for the row count.  The single wave needs neither the
+// hand-over through shared memory nor a barrier.
 template <int DIM, int P, int T>
 __global__ __launch_bounds__(T) void fps_reg_kernel(
     const float *__restrict__ src, const int64_t *__restrict__ ptr,
@@ -241,14 +244,20 @@ __global__ __launch_bounds__(T) void fps_reg_kernel(
   __shared__ uint32_t s_v[2][kFpsWaves];
   __shared__ uint32_t s_rel[2][kFpsWaves];
   __shared__ float s_x[2][DIM][kFpsWaves];
-  static_assert(kFpsWaves == 16 && T % 256 == 0 && T <= kFpsThreads,
+  static_assert(kFpsWaves == 16 && (T % 256 == 0 || T == kWave) &&
+                    T <= kFpsThreads,
                 "one row of 16 lanes picks the winner among up to 16 waves");
+  static_assert(T != kWave || P % 4 == 0, "four tie classes per lane");
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
-  constexpr int S = T / 256;
-  const int rel0 = tid / S + 256 * ((tid % S) * P);
+  constexpr int S = T >= 256 ? T / 256 : 1; // threads per tie class
+  constexpr int C = T >= 256 ? 1 : 256 / T; // tie classes per thread
+  constexpr int PARTS = P / C;              // slots per tie class
+  const int rel0 = (tid / S) * C + 256 * ((tid % S) * P);
+  // row of slot i, relative to rel0
+  auto slot_row = [](int i) { return i / PARTS + 256 * (i % PARTS); };
   const int b = blockIdx.x;
   const int64_t start_idx = ptr[b];
   const int count = (int)(ptr[b + 1] - start_idx);
@@ -256,7 +265,7 @@ __global__ __launch_bounds__(T) void fps_reg_kernel(
   const int64_t o_end = out_ptr[b + 1];
   if (o_begin >= o_end)
     return;
-  if (T < kFpsThreads) {
+  if (T < kFpsThreads && T > kWave) {
     // the entries of waves that do not run stay "nothing"
     if (tid < 2 * kFpsWaves)
       s_v[tid / kFpsWaves][tid % kFpsWaves] = 0u;
@@ -273,7 +282,7 @@ __global__ __launch_bounds__(T) void fps_reg_kernel(
   static_assert(P <= 16, "low words 15 - i");
 #pragma unroll
   for (int i = 0; i < P; ++i) {
-    const int rel = rel0 + 256 * i;
+    const int rel = rel0 + slot_row(i);
 #pragma unroll
     for (int c = 0; c < DIM; ++c)
       px[i][c] = (rel < count && c < d)
@@ -294,26 +303,41 @@ __global__ __launch_bounds__(T) void fps_reg_kernel(
     const int par = (int)(m & 1);
     // (below every slot's pattern: -1 with the largest low word)
     double best_key = __hiloint2double(__float_as_int(-1.0f), -1);
+    // (component by component over all slots: independent instructions
+    // follow each other, a slot's own chain is spread out)
+    float dd[P];
 #pragma unroll
     for (int i = 0; i < P; ++i) {
-      // (zero components beyond d add fma(0, 0, acc) = acc)
       const float t0 = cur[0] - px[i][0];
-      float dd = t0 * t0;
+      dd[i] = t0 * t0;
+    }
 #pragma unroll
-      for (int c = 1; c < DIM; ++c) {
+    for (int c = 1; c < DIM; ++c) {
+#pragma unroll
+      for (int i = 0; i < P; ++i) {
+        // (zero components beyond d add fma(0, 0, acc) = acc)
         const float tc = cur[c] - px[i][c];
-        dd = __builtin_fmaf(tc, tc, dd);
+        dd[i] = __builtin_fmaf(tc, tc, dd[i]);
       }
+    }
+#pragma unroll
+    for (int i = 0; i < P; ++i) {
       // fminf without its quieting of signalling NaNs, which neither operand
       // can be (5e4, -1, or the result of arithmetic): a NaN loses to a number
       const float before = __int_as_float(__double2hiint(slot_key[i]));
-      asm("v_min_f32 %0, %1, %2" : "=v"(dd) : "v"(before), "v"(dd));
-      slot_key[i] =
-          __hiloint2double(__float_as_int(dd), __double2loint(slot_key[i]));
-      asm("v_max_f64 %0, %1, %2"
-          : "=v"(best_key)
-          : "v"(best_key), "v"(slot_key[i]));
+      asm("v_min_f32 %0, %1, %2" : "=v"(dd[i]) : "v"(before), "v"(dd[i]));
+      slot_key[i] = __hiloint2double(__float_as_int(dd[i]),
+                                     __double2loint(slot_key[i]));
     }
+    double part_key[2] = {best_key, best_key};
+#pragma unroll
+    for (int i = 0; i < P; ++i)
+      asm("v_max_f64 %0, %1, %2"
+          : "=v"(part_key[i & 1])
+          : "v"(part_key[i & 1]), "v"(slot_key[i]));
+    asm("v_max_f64 %0, %1, %2"
+        : "=v"(best_key)
+        : "v"(part_key[0]), "v"(part_key[1]));
     const uint32_t best_bits = (uint32_t)__double2hiint(best_key);
     const int best_i = best_bits != __float_as_uint(-1.0f)
                            ? 15 - __double2loint(best_key)
@@ -348,39 +372,57 @@ __global__ __launch_bounds__(T) void fps_reg_kernel(
       break;
     }
     static_assert(P <= 16, "slots of the switch above");
-    if (lane == src_lane) {
-      s_v[par][wave] = wave_key;
-      s_rel[par][wave] = (uint32_t)(rel0 + 256 * slot);
-#pragma unroll
-      for (int c = 0; c < DIM; ++c)
-        s_x[par][c][wave] = bx[c];
-    }
-    __syncthreads();
-    // every row of 16 lanes looks at the 16 wave results
-    const uint32_t ev = s_v[par][lane & 15];
-    const uint32_t erel = s_rel[par][lane & 15];
-    float ex[DIM];
-#pragma unroll
-    for (int c = 0; c < DIM; ++c) {
-      ex[c] = s_x[par][c][lane & 15];
-      asm volatile("" : "+v"(ex[c])); // (read now, not after the reduction)
-    }
-    const uint32_t top_key =
-        (uint32_t)__builtin_amdgcn_readlane((int)row16_umax(ev), 15);
     int64_t chosen;
-    if (top_key != 0u) {
-      const int win = (int)__builtin_ctzll(__ballot(ev == top_key));
-      chosen = start_idx + (int64_t)__builtin_amdgcn_readlane((int)erel, win);
+    if (T == kWave) {
+      if (wave_key != 0u) {
+        chosen = start_idx + __builtin_amdgcn_readlane(rel0, src_lane) +
+                 slot_row(slot);
 #pragma unroll
-      for (int c = 0; c < DIM; ++c)
-        cur[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
-            (int)__float_as_uint(ex[c]), win));
+        for (int c = 0; c < DIM; ++c)
+          cur[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+              (int)__float_as_uint(bx[c]), src_lane));
+      } else {
+        // nothing above -1: the reference's `best_idx` is still 0
+        chosen = 0;
+#pragma unroll
+        for (int c = 0; c < DIM; ++c)
+          cur[c] = c < d ? src[c] : 0.0f;
+      }
     } else {
-      // nothing above -1: the reference's `best_idx` is still 0
-      chosen = 0;
+      if (lane == src_lane) {
+        s_v[par][wave] = wave_key;
+        s_rel[par][wave] = (uint32_t)(rel0 + slot_row(slot));
 #pragma unroll
-      for (int c = 0; c < DIM; ++c)
-        cur[c] = c < d ? src[c] : 0.0f;
+        for (int c = 0; c < DIM; ++c)
+          s_x[par][c][wave] = bx[c];
+      }
+      __syncthreads();
+      // every row of 16 lanes looks at the 16 wave results
+      const uint32_t ev = s_v[par][lane & 15];
+      const uint32_t erel = s_rel[par][lane & 15];
+      float ex[DIM];
+#pragma unroll
+      for (int c = 0; c < DIM; ++c) {
+        ex[c] = s_x[par][c][lane & 15];
+        asm volatile("" : "+v"(ex[c])); // (read now, not after the reduction)
+      }
+      const uint32_t top_key =
+          (uint32_t)__builtin_amdgcn_readlane((int)row16_umax(ev), 15);
+      if (top_key != 0u) {
+        const int win = (int)__builtin_ctzll(__ballot(ev == top_key));
+        chosen =
+            start_idx + (int64_t)__builtin_amdgcn_readlane((int)erel, win);
+#pragma unroll
+        for (int c = 0; c < DIM; ++c)
+          cur[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+              (int)__float_as_uint(ex[c]), win));
+      } else {
+        // nothing above -1: the reference's `best_idx` is still 0
+        chosen = 0;
+#pragma unroll
+        for (int c = 0; c < DIM; ++c)
+          cur[c] = c < d ? src[c] : 0.0f;
+      }
     }
     if (tid == 0)
       out[m] = chosen;
@@ -401,9 +443,9 @@ hipError_t launch_fps_reg(const float *src, const int64_t *ptr,
                      dim3(T_), 0, stream, src, ptr, out_ptr, start, d, out)
   // (shapes by measurement: 16 examples of each size on one device)
   if (max_rows <= 256)
-    PCA_FPS_REG(1, 256);
+    PCA_FPS_REG(4, 64);
   else if (max_rows <= 512)
-    PCA_FPS_REG(2, 256);
+    PCA_FPS_REG(8, 64);
   else if (max_rows <= 1024)
     PCA_FPS_REG(2, 512);
   else if (max_rows <= 2048)
