@@ -131,6 +131,27 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
             int edge_flags, int64_t *edges, int64_t *num_edges, void *dist,
             void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * pca_knn for fp32 points of up to 3 dimensions, Euclidean distance and
+ * k <= 32 (PCA_ERR_UNSUPPORTED otherwise) over spatially binned rows: the x
+ * rows of every segment are ordered along a space-filling curve (the voxel
+ * numbers of the reference's grid clustering, csrc/cuda/grid_cuda.cu:10-25,
+ * bit-interleaved), cut into tiles with bounding boxes, and a query scans only
+ * the tiles whose box is within its current k-th distance.  Stands under the
+ * same operator as pca_knn (csrc/knn.cpp:22-40 -> csrc/cuda/knn_cuda.cu:86-135)
+ * and returns the same edges, bit for bit, in the same order; only the work
+ * differs (rows looked at per query: tens to hundreds instead of the whole
+ * segment).  Arguments as for pca_knn.
+ */
+size_t pca_knn_binned_workspace_bytes(int64_t n, int64_t m, int64_t d,
+                                      int64_t num_segments, int64_t k);
+
+int pca_knn_binned(const void *x, const void *y, const int64_t *ptr_x,
+                   const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+                   int64_t num_segments, int64_t k, int edge_flags,
+                   int64_t *edges, int64_t *num_edges, void *dist,
+                   void *workspace, size_t workspace_bytes, void *stream);
+
 /* --------------------------------------------------------------- radius -- */
 
 /*

@@ -39,6 +39,12 @@ C_ABI = {
                 [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                  ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp,
                  ctypes.c_size_t, _vp]),
+    "pca_knn_binned_workspace_bytes": (ctypes.c_size_t,
+                                       [_i64, _i64, _i64, _i64, _i64]),
+    "pca_knn_binned": (ctypes.c_int,
+                       [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
+                        ctypes.c_int, _vp, _vp, _vp, _vp, ctypes.c_size_t,
+                        _vp]),
     "pca_radius_slots": (_i64, [_i64, _i64]),
     "pca_radius_workspace_bytes": (ctypes.c_size_t,
                                    [_i64, _i64, _i64, _i64, _i64,

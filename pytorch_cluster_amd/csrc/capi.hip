@@ -122,6 +122,16 @@ size_t knn_workspace(int64_t n, int64_t m, int64_t d, int64_t num_segments,
   return knn_layout(n, m, d, num_segments, k, dtype).total();
 }
 
+size_t binned_workspace(int64_t n, int64_t m, int64_t num_segments,
+                        int64_t k) {
+  return align256(pca::knn_binned_scratch_bytes((int)n, (int)m,
+                                                (int)num_segments)) +
+         align256(sizeof(int) * (size_t)m * (size_t)k) +
+         align256(sizeof(float) * (size_t)m * (size_t)k) +
+         align256(sizeof(int) * (size_t)m) +
+         pca::compact_workspace_bytes((int)m);
+}
+
 bool dtype_ok(int dtype) {
   return dtype == PCA_F32 || dtype == PCA_F64 || dtype == PCA_F16 ||
          dtype == PCA_BF16;
@@ -348,6 +358,90 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
                       "knn_generic_kernel");
     timer.done();
   }
+  if (rc != PCA_OK)
+    return rc;
+  return check_launch(
+      pca::launch_compact(dense, (int)m, edges, num_edges,
+                          static_cast<float *>(dist), compact_ws, stream,
+                          (edge_flags & PCA_EDGES_DROP_SELF) != 0,
+                          (edge_flags & PCA_EDGES_X_FIRST) != 0),
+      "compaction kernels");
+}
+
+size_t pca_knn_binned_workspace_bytes(int64_t n, int64_t m, int64_t d,
+                                      int64_t num_segments, int64_t k) {
+  if (num_segments < 1)
+    num_segments = 1;
+  if (!sizes_ok(n, m, d, num_segments) || n == 0 || m == 0 ||
+      !pca::knn_binned_supported((int)d, (int)k, false))
+    return 0;
+  return binned_workspace(n, m, num_segments, k);
+}
+
+int pca_knn_binned(const void *x, const void *y, const int64_t *ptr_x,
+                   const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+                   int64_t num_segments, int64_t k, int edge_flags,
+                   int64_t *edges, int64_t *num_edges, void *dist,
+                   void *workspace, size_t workspace_bytes, void *stream_) {
+  g_last_error[0] = 0;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  SearchTimer timer(stream);
+  if ((ptr_x == nullptr) != (ptr_y == nullptr))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "ptr_x and ptr_y must both be given or both be NULL");
+  if (ptr_x == nullptr)
+    num_segments = 1;
+  if (!sizes_ok(n, m, d, num_segments))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "bad sizes n=%lld m=%lld d=%lld num_segments=%lld",
+                (long long)n, (long long)m, (long long)d,
+                (long long)num_segments);
+  if (k < 1)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "k must be >= 1, got %lld",
+                (long long)k);
+  if (k > PCA_KNN_MAX_K)
+    return fail(PCA_ERR_K_TOO_LARGE, "%s",
+                pca_status_string(PCA_ERR_K_TOO_LARGE));
+  if (!pca::knn_binned_supported((int)d, (int)k, false))
+    return fail(PCA_ERR_UNSUPPORTED,
+                "binned search: fp32 points of up to 3 dimensions and k <= 32, "
+                "got d=%lld k=%lld",
+                (long long)d, (long long)k);
+  if (num_edges == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "num_edges is NULL");
+  if (!edge_flags_ok(edge_flags))
+    return fail(PCA_ERR_INVALID_ARGUMENT, "unknown edge flags %d", edge_flags);
+  if (n == 0 || m == 0) {
+    hipLaunchKernelGGL(set_i64_kernel, dim3(1), dim3(1), 0, stream, num_edges,
+                       (int64_t)0);
+    return check_launch(hipGetLastError(), "set_i64_kernel");
+  }
+  if (x == nullptr || y == nullptr || edges == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "x, y or edges is NULL");
+  const size_t need = binned_workspace(n, m, num_segments, k);
+  if (workspace == nullptr || ((uintptr_t)workspace & 255) != 0 ||
+      workspace_bytes < need)
+    return fail(PCA_ERR_WORKSPACE, "workspace needs %zu bytes, 256-aligned",
+                need);
+
+  Carver carve(workspace);
+  void *scratch = carve.take<char>(pca::knn_binned_scratch_bytes(
+      (int)n, (int)m, (int)num_segments));
+  pca::DenseResult dense;
+  dense.idx = carve.take<int>((size_t)m * (size_t)k);
+  dense.dist = carve.take<float>((size_t)m * (size_t)k);
+  dense.count = carve.take<int>((size_t)m);
+  dense.slots = (int)k;
+  void *compact_ws = carve.take<char>(pca::compact_workspace_bytes((int)m));
+  if (dist == nullptr)
+    dense.dist = nullptr;
+
+  pca::SearchInput in{x,      y,      ptr_x,  ptr_y,
+                      (int)n, (int)m, (int)d, (int)num_segments};
+  int rc = check_launch(pca::launch_knn_binned(in, (int)k, scratch, dense,
+                                               timer.start, timer.stop, stream),
+                        "binned search");
+  timer.stop = nullptr;
   if (rc != PCA_OK)
     return rc;
   return check_launch(

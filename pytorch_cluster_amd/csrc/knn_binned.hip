@@ -1,0 +1,607 @@
+// Exact Euclidean kNN over spatially binned rows: fp32 points of up to three
+// dimensions, k <= 32.  Same results, bit for bit, as the reference's scan of
+// every row of the segment (csrc/cuda/knn_cuda.cu:52-78: distances as chains
+// of direct differences and fused multiply-adds, neighbours by ascending
+// distance, ties by ascending row, strictly below 1e10), but a query looks only
+// at rows near it.
+//
+// Per call: every segment's x rows are ordered along a space-filling curve
+// (30-bit Morton codes inside the segment's bounding box - the voxel number of
+// the reference's grid clustering, csrc/cuda/grid_cuda.cu:10-25, with its bits
+// interleaved - sorted by rocPRIM's radix sort), copied in that order together
+// with their row numbers, and cut into tiles of 32 rows with a bounding box
+// each.  The queries are ordered the same way, so the 64 queries of a wave
+// (one per lane) are neighbours in space and share one bounding box.
+//
+// A wave first scans the tiles around its queries' position in the order of x
+// (that fills the lists and gives every query a k-th distance), then sweeps
+// the segment's tile boxes 64 at a time, one per lane, outwards from that
+// position: a tile is scanned only if the smallest distance between its box
+// and the wave's box is not above the largest k-th distance among the wave's
+// queries.  That box distance is computed with the operations of the exact
+// chain (one difference per axis, product, fused multiply-adds in the same
+// order) applied to per-axis gaps that are not above any row's difference:
+// rounding is monotone, so the value is never above the computed distance of
+// any (query, row) pair of the two boxes, and a skipped tile cannot hold a
+// neighbour.  Rows of a scanned tile are uniform over the wave (scalar
+// loads); a lane whose distance passes its own bound parks (distance, row) in
+// a queue in LDS, and the queues are emptied into the sorted lists by all
+// lanes together when one fills up, as in the scanning kernels.  Rows arrive
+// out of row order here, so a row of EQUAL distance may still displace a
+// neighbour with a larger row number: a full list admits d <= its k-th
+// distance and the 64-bit (distance, row) keys decide.
+#include "device_utils.hpp"
+#include "knn_lowd_impl.hpp"
+#include "launchers.hpp"
+
+#include <climits>
+#include <cstring>
+
+#include <rocprim/device/device_radix_sort.hpp>
+
+namespace pca {
+
+namespace {
+
+constexpr int kBinTile = 32;      // rows per tile
+constexpr int kBinQueueCap = 16;  // parked rows per lane
+constexpr int kBinSeedTiles = 16; // most tiles scanned before the sweep
+constexpr int kCodeBits = 30;
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// floats as integers of the same order (for atomic min / max)
+__device__ __forceinline__ int ordered_int(float f) {
+  const int i = __float_as_int(f);
+  return i >= 0 ? i : i ^ 0x7fffffff;
+}
+__device__ __forceinline__ float from_ordered_int(int i) {
+  return __int_as_float(i >= 0 ? i : i ^ 0x7fffffff);
+}
+
+__device__ __forceinline__ int find_segment64(const int64_t *__restrict__ ptr,
+                                              int num_segments, int64_t v) {
+  if (ptr == nullptr)
+    return 0;
+  int lo = 0, hi = num_segments;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (ptr[mid] <= v)
+      lo = mid;
+    else
+      hi = mid;
+  }
+  return lo;
+}
+
+// seg_box: [num_segments][6] = lower corner, upper corner (ordered integers)
+__global__ void seg_box_init_kernel(int *seg_box, int count) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count)
+    seg_box[i] = (i % 6) < 3 ? INT_MAX : INT_MIN;
+}
+
+// Bounding box of the finite coordinates of every segment; grid (parts,
+// up to 65,535 segments at a time).
+__global__ __launch_bounds__(kBlock) void seg_box_kernel(
+    const float *__restrict__ x, const int64_t *__restrict__ ptr_x, int n,
+    int d, int seg_count, int *__restrict__ seg_box) {
+  for (int seg = blockIdx.y; seg < seg_count; seg += gridDim.y) {
+    const int64_t begin = ptr_x ? ptr_x[seg] : 0;
+    const int64_t end = ptr_x ? ptr_x[seg + 1] : n;
+    float lo[3], hi[3];
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      lo[c] = __builtin_inff();
+      hi[c] = -__builtin_inff();
+    }
+    for (int64_t i = begin + (int64_t)blockIdx.x * kBlock + threadIdx.x;
+         i < end; i += (int64_t)gridDim.x * kBlock) {
+#pragma unroll
+      for (int c = 0; c < 3; ++c)
+        if (c < d) {
+          const float v = x[(size_t)i * d + c];
+          if (__builtin_fabsf(v) < __builtin_inff()) {
+            lo[c] = __builtin_fminf(lo[c], v);
+            hi[c] = __builtin_fmaxf(hi[c], v);
+          }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+#pragma unroll
+      for (int sh = 1; sh < kWave; sh <<= 1) {
+        lo[c] = __builtin_fminf(lo[c], __shfl_xor(lo[c], sh));
+        hi[c] = __builtin_fmaxf(hi[c], __shfl_xor(hi[c], sh));
+      }
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+#pragma unroll
+      for (int c = 0; c < 3; ++c) {
+        atomicMin(&seg_box[seg * 6 + c], ordered_int(lo[c]));
+        atomicMax(&seg_box[seg * 6 + 3 + c], ordered_int(hi[c]));
+      }
+    }
+  }
+}
+
+// 10 bits spread to every third position
+__device__ __forceinline__ uint32_t spread3(uint32_t v) {
+  v &= 0x3ffu;
+  v = (v | (v << 16)) & 0x030000ffu;
+  v = (v | (v << 8)) & 0x0300f00fu;
+  v = (v | (v << 4)) & 0x030c30c3u;
+  v = (v | (v << 2)) & 0x09249249u;
+  return v;
+}
+
+// keys[i] = (segment << 30) | Morton code of row i inside its segment's box of
+// x rows (coordinates outside the box, NaN and missing axes go to its border);
+// vals[i] = i.
+__global__ __launch_bounds__(kBlock) void morton_keys_kernel(
+    const float *__restrict__ pts, const int64_t *__restrict__ ptr, int count,
+    int d, int num_segments, const int *__restrict__ seg_box,
+    uint64_t *__restrict__ keys, uint32_t *__restrict__ vals) {
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= count)
+    return;
+  const int seg = find_segment64(ptr, num_segments, i);
+  uint32_t code = 0;
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    uint32_t cell = 0;
+    if (c < d) {
+      const float lo = from_ordered_int(seg_box[seg * 6 + c]);
+      const float hi = from_ordered_int(seg_box[seg * 6 + 3 + c]);
+      const float v = pts[(size_t)i * d + c];
+      const float t = (v - lo) / (hi - lo) * 1024.0f;
+      // (NaN, also from an empty or flat box, fails the first comparison)
+      cell = t >= 0.0f ? (uint32_t)__builtin_fminf(t, 1023.0f) : 0u;
+    }
+    code |= spread3(cell) << c;
+  }
+  keys[i] = ((uint64_t)seg << kCodeBits) | code;
+  vals[i] = (uint32_t)i;
+}
+
+// Rows in curve order with their row numbers, and the box of every tile of 32:
+// half a wave per tile.  box: [6][box_stride], lower then upper corner.
+__global__ __launch_bounds__(kBlock) void gather_tiles_kernel(
+    const float *__restrict__ x, const int64_t *__restrict__ ptr_x, int n,
+    int d, int num_segments, const int *__restrict__ tile_start,
+    const uint32_t *__restrict__ perm, float4 *__restrict__ rows,
+    float *__restrict__ box, int box_stride) {
+  const int gt = (blockIdx.x * kBlock + threadIdx.x) / kBinTile;
+  const int r = threadIdx.x & (kBinTile - 1);
+  if (gt >= tile_start[num_segments])
+    return;
+  const int seg = find_segment(tile_start, num_segments, gt);
+  const int x_begin = ptr_x ? (int)ptr_x[seg] : 0;
+  const int x_end = ptr_x ? (int)ptr_x[seg + 1] : n;
+  const int j = x_begin + (gt - tile_start[seg]) * kBinTile + r;
+  const bool ok = j < x_end;
+  const uint32_t id = ok ? perm[j] : 0u;
+  float v[3];
+#pragma unroll
+  for (int c = 0; c < 3; ++c)
+    v[c] = (ok && c < d) ? x[(size_t)id * d + c] : 0.0f;
+  if (ok)
+    rows[j] = make_float4(v[0], v[1], v[2], __uint_as_float(id));
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    // (fminf / fmaxf drop a NaN operand: a NaN coordinate is in no box, and
+    // such a row has no distance below the limit either)
+    float lo = ok ? v[c] : __builtin_inff();
+    float hi = ok ? v[c] : -__builtin_inff();
+#pragma unroll
+    for (int sh = 1; sh < kBinTile; sh <<= 1) {
+      lo = __builtin_fminf(lo, __shfl_xor(lo, sh));
+      hi = __builtin_fmaxf(hi, __shfl_xor(hi, sh));
+    }
+    if (r == 0) {
+      box[(size_t)c * box_stride + gt] = lo;
+      box[(size_t)(3 + c) * box_stride + gt] = hi;
+    }
+  }
+}
+
+struct BinnedParams {
+  const float *y;
+  const int64_t *ptr_x;
+  const int64_t *ptr_y;
+  int n, m, d, num_segments, k;
+  const int *tile_start;    // first tile of every segment
+  const int *wave_start;    // first wave task of every segment
+  const uint64_t *keys_x;   // sorted keys of the x rows
+  const uint64_t *keys_y;   // sorted keys of the queries
+  const uint32_t *perm_y;   // query behind every sorted position
+  const float4 *rows;       // x rows in curve order, .w = row number
+  const float *box;         // [6][box_stride]
+  int box_stride;
+  int *out_idx;
+  float *out_dist;
+  int *out_count;
+};
+
+// First position in [lo, hi) whose key is not below `key` (hi if none); the
+// wave probes 64 positions per round.
+__device__ __forceinline__ int wave_lower_bound(
+    const uint64_t *__restrict__ keys, int lo, int hi, uint64_t key,
+    int lane) {
+  while (hi - lo > kWave) {
+    const int step = (hi - lo) / kWave;
+    const int probe = lo + (lane + 1) * step - 1;
+    const int below = __popcll(__ballot(keys[probe] < key));
+    // probes 0 .. below-1 are below the key, probe `below` (if any) is not
+    const int new_lo = lo + below * step;
+    if (below < kWave)
+      hi = lo + (below + 1) * step - 1;
+    lo = new_lo;
+  }
+  const int probe = lo + lane;
+  const bool below = probe < hi && keys[probe] < key;
+  return lo + __popcll(__ballot(below));
+}
+
+template <int K>
+__global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
+  // parked rows: distance and row number, [slot][thread]
+  __shared__ float queue_d[kBinQueueCap][kBlock];
+  __shared__ uint32_t queue_id[kBinQueueCap][kBlock];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int task = blockIdx.x * (kBlock / kWave) +
+                   __builtin_amdgcn_readfirstlane(tid / kWave);
+  if (task >= p.wave_start[p.num_segments])
+    return; // (whole waves leave; no barrier below)
+  const int seg = find_segment(p.wave_start, p.num_segments, task);
+  const int x_begin = p.ptr_x ? (int)p.ptr_x[seg] : 0;
+  const int x_end = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
+  const int y_begin = p.ptr_y ? (int)p.ptr_y[seg] : 0;
+  const int y_end = p.ptr_y ? (int)p.ptr_y[seg + 1] : p.m;
+  const int jq = y_begin + (task - p.wave_start[seg]) * kWave + lane;
+  const bool valid = jq < y_end;
+  const int q = valid ? (int)p.perm_y[jq] : 0;
+  const int k = p.k;
+  const int d_in = p.d;
+
+  float yq[3];
+#pragma unroll
+  for (int c = 0; c < 3; ++c)
+    yq[c] = (valid && c < d_in) ? p.y[(size_t)q * d_in + c] : 0.0f;
+  // a query with a coordinate that is not finite has no distance below the
+  // limit: it looks at nothing and returns nothing
+  const bool searching = valid && __builtin_fabsf(yq[0]) < __builtin_inff() &&
+                         __builtin_fabsf(yq[1]) < __builtin_inff() &&
+                         __builtin_fabsf(yq[2]) < __builtin_inff();
+
+  // the wave's box (lanes that do not search stay out)
+  float q_lo[3], q_hi[3];
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    float lo = searching ? yq[c] : __builtin_inff();
+    float hi = searching ? yq[c] : -__builtin_inff();
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1) {
+      lo = __builtin_fminf(lo, __shfl_xor(lo, sh));
+      hi = __builtin_fmaxf(hi, __shfl_xor(hi, sh));
+    }
+    q_lo[c] = lo;
+    q_hi[c] = hi;
+  }
+
+  double best[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j)
+    best[j] = (j < K - k) ? lowest_key() : empty_key();
+  // a row is parked when its distance is strictly below `admit`: the limit
+  // while the list has room, just above the k-th distance afterwards (a row of
+  // equal distance and smaller number still gets in); nothing for a lane
+  // that does not search
+  float admit = searching ? kKnnSentinel : -__builtin_inff();
+  // largest k-th distance among the wave's queries (the limit while any list
+  // has room): tiles whose box is farther away are skipped
+  float reach = kKnnSentinel;
+  int parked = 0;
+
+  auto drain = [&]() {
+    for (;;) {
+      const bool has = parked > 0;
+      if (!__any(has))
+        break;
+      parked -= has ? 1 : 0;
+      const float d = queue_d[has ? parked : 0][tid];
+      const uint32_t id = queue_id[has ? parked : 0][tid];
+      // (parked under an older bound: the keys sort it out)
+      const double key = (has && d < admit) ? make_key(d, id) : empty_key();
+      sorted_insert<K>(best, key);
+      const float kth = key_dist(best[K - 1]);
+      if (searching && kth < kKnnSentinel)
+        admit = next_up_positive(kth);
+    }
+    float r = searching ? key_dist(best[K - 1]) : 0.0f;
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1)
+      r = __builtin_fmaxf(r, __shfl_xor(r, sh));
+    reach = r;
+  };
+
+  // rows of one tile against every lane's query
+  auto scan_tile = [&](int tile) {
+    const int j0 = x_begin + tile * kBinTile;
+    const int rows = min(kBinTile, x_end - j0);
+    const float4 *__restrict__ src = p.rows + j0;
+    for (int r = 0; r < rows; ++r) {
+      const float4 row = src[r]; // (uniform address)
+      const float d0 = row.x - yq[0];
+      float dd = d0 * d0;
+      const float d1 = row.y - yq[1];
+      dd = __builtin_fmaf(d1, d1, dd);
+      const float d2 = row.z - yq[2];
+      dd = __builtin_fmaf(d2, d2, dd);
+      const bool hit = dd < admit;
+      if (hit) {
+        queue_d[parked][tid] = dd;
+        queue_id[parked][tid] = __float_as_uint(row.w);
+        ++parked;
+      }
+      if (__any(parked == kBinQueueCap))
+        drain();
+    }
+  };
+
+  const int tile0 = p.tile_start[seg];
+  const int num_tiles = p.tile_start[seg + 1] - tile0;
+  int seed_lo = 0, seed_hi = -1; // tiles seed_lo .. seed_hi scanned up front
+  if (num_tiles > 0) {
+    // where the wave's first and last query fall in the order of x
+    const int last_lane = min(kWave, y_end - (jq - lane)) - 1;
+    const uint64_t key_first =
+        p.keys_y[__builtin_amdgcn_readfirstlane(jq - lane)];
+    const uint64_t key_last =
+        p.keys_y[__builtin_amdgcn_readfirstlane(jq - lane + last_lane)];
+    const int pos_first =
+        wave_lower_bound(p.keys_x, x_begin, x_end, key_first, lane);
+    const int pos_last =
+        wave_lower_bound(p.keys_x, x_begin, x_end, key_last, lane);
+    const int t_first = min(num_tiles - 1, (pos_first - x_begin) / kBinTile);
+    const int t_last = min(num_tiles - 1, (pos_last - x_begin) / kBinTile);
+    seed_lo = max(0, t_first - 1);
+    seed_hi = min(num_tiles - 1, max(t_last, t_first) + 1);
+    if (seed_hi - seed_lo + 1 > kBinSeedTiles) {
+      // queries far apart in the order of x: the middle of their range
+      const int mid = (seed_lo + seed_hi) / 2;
+      seed_lo = max(0, mid - kBinSeedTiles / 2);
+      seed_hi = min(num_tiles - 1, seed_lo + kBinSeedTiles - 1);
+    }
+    for (int t = seed_lo; t <= seed_hi; ++t)
+      scan_tile(t);
+    drain();
+
+    // sweep of the tile boxes, 64 per round, outwards from the seed tiles
+    const int num_rounds = (num_tiles + kWave - 1) / kWave;
+    const int centre = ((seed_lo + seed_hi) / 2) / kWave;
+    for (int i = 0; i < 2 * num_rounds; ++i) {
+      const int round = centre + ((i & 1) ? -((i + 1) >> 1) : (i >> 1));
+      if (round < 0 || round >= num_rounds)
+        continue;
+      const int t = round * kWave + lane;
+      float gap2 = __builtin_inff();
+      if (t < num_tiles && !(t >= seed_lo && t <= seed_hi)) {
+        const size_t g = (size_t)(tile0 + t);
+        float acc = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+          const float lo = p.box[(size_t)c * p.box_stride + g];
+          const float hi = p.box[(size_t)(3 + c) * p.box_stride + g];
+          // not above |row - query| along this axis for any pair of the boxes
+          // (a NaN, from an infinite or empty box, survives to the test below)
+          const float gap =
+              __builtin_fmaxf(__builtin_fmaxf(lo - q_hi[c], q_lo[c] - hi), 0.0f);
+          acc = c == 0 ? gap * gap : __builtin_fmaf(gap, gap, acc);
+        }
+        gap2 = acc;
+      }
+      // (!(a > b): a NaN box distance never skips a tile)
+      uint64_t todo = __ballot(t < num_tiles &&
+                               !(t >= seed_lo && t <= seed_hi) &&
+                               !(gap2 > reach));
+      while (todo != 0) {
+        const int src_lane = (int)__builtin_ctzll(todo);
+        todo &= todo - 1;
+        const float g2 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+            (int)__float_as_uint(gap2), src_lane));
+        if (g2 > reach)
+          continue; // the bound has moved since the ballot
+        scan_tile(round * kWave + src_lane);
+        if (__any(parked > 0))
+          drain();
+      }
+    }
+  }
+
+  if (valid)
+    write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+}
+
+struct BinnedLayout {
+  size_t seg_box, keys_a, keys_x, keys_y, vals_a, perm_x, perm_y, rows, box,
+      tile_start, wave_start, sort_temp;
+  int box_stride;
+  size_t total() const {
+    return seg_box + keys_a + keys_x + keys_y + vals_a + perm_x + perm_y +
+           rows + box + tile_start + wave_start + sort_temp;
+  }
+};
+
+int key_bits(int num_segments) {
+  int bits = kCodeBits;
+  while (bits < 62 && ((int64_t)1 << (bits - kCodeBits)) < num_segments)
+    ++bits;
+  return bits;
+}
+
+hipError_t sort_pairs(void *temp, size_t &temp_bytes, const uint64_t *keys_in,
+                      uint64_t *keys_out, const uint32_t *vals_in,
+                      uint32_t *vals_out, int count, int num_segments,
+                      hipStream_t stream) {
+  return rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out,
+                                   vals_in, vals_out, (unsigned int)count, 0u,
+                                   (unsigned int)key_bits(num_segments),
+                                   stream, false);
+}
+
+BinnedLayout binned_layout(int n, int m, int num_segments) {
+  BinnedLayout w;
+  const size_t big = (size_t)std::max(n, m);
+  w.seg_box = align256(sizeof(int) * 6 * (size_t)num_segments);
+  w.keys_a = align256(sizeof(uint64_t) * big);
+  w.keys_x = align256(sizeof(uint64_t) * (size_t)n);
+  w.keys_y = align256(sizeof(uint64_t) * (size_t)m);
+  w.vals_a = align256(sizeof(uint32_t) * big);
+  w.perm_x = align256(sizeof(uint32_t) * (size_t)n);
+  w.perm_y = align256(sizeof(uint32_t) * (size_t)m);
+  w.rows = align256(sizeof(float4) * (size_t)n);
+  w.box_stride = plan_upper_bound(n, num_segments, kBinTile);
+  w.box = align256(sizeof(float) * 6 * (size_t)w.box_stride);
+  w.tile_start = align256(sizeof(int) * (size_t)(num_segments + 1));
+  w.wave_start = align256(sizeof(int) * (size_t)(num_segments + 1));
+  size_t tx = 0, ty = 0;
+  const hipError_t ex = sort_pairs(nullptr, tx, nullptr, nullptr, nullptr,
+                                   nullptr, n, num_segments, nullptr);
+  const hipError_t ey = sort_pairs(nullptr, ty, nullptr, nullptr, nullptr,
+                                   nullptr, m, num_segments, nullptr);
+  // (a failed size query leaves a size no workspace can meet)
+  w.sort_temp = (ex == hipSuccess && ey == hipSuccess)
+                    ? align256(std::max(tx, ty))
+                    : ~(size_t)0 / 2;
+  return w;
+}
+
+} // namespace
+
+bool knn_binned_supported(int d, int k, bool cosine) {
+  return !cosine && d >= 1 && d <= 3 && k >= 1 && k <= 32;
+}
+
+size_t knn_binned_scratch_bytes(int n, int m, int num_segments) {
+  return binned_layout(n, m, num_segments).total();
+}
+
+hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
+                             const DenseResult &out, hipEvent_t time_start,
+                             hipEvent_t time_stop, hipStream_t stream) {
+  const BinnedLayout lay = binned_layout(in.n, in.m, in.num_segments);
+  char *cursor = static_cast<char *>(scratch);
+  auto take = [&cursor](size_t bytes) {
+    char *piece = cursor;
+    cursor += bytes;
+    return static_cast<void *>(piece);
+  };
+  int *seg_box = static_cast<int *>(take(lay.seg_box));
+  uint64_t *keys_a = static_cast<uint64_t *>(take(lay.keys_a));
+  uint64_t *keys_x = static_cast<uint64_t *>(take(lay.keys_x));
+  uint64_t *keys_y = static_cast<uint64_t *>(take(lay.keys_y));
+  uint32_t *vals_a = static_cast<uint32_t *>(take(lay.vals_a));
+  uint32_t *perm_x = static_cast<uint32_t *>(take(lay.perm_x));
+  uint32_t *perm_y = static_cast<uint32_t *>(take(lay.perm_y));
+  float4 *rows = static_cast<float4 *>(take(lay.rows));
+  float *box = static_cast<float *>(take(lay.box));
+  int *tile_start = static_cast<int *>(take(lay.tile_start));
+  int *wave_start = static_cast<int *>(take(lay.wave_start));
+  void *sort_temp = take(lay.sort_temp);
+  size_t sort_bytes = lay.sort_temp;
+
+  const float *x = static_cast<const float *>(in.x);
+  const float *y = static_cast<const float *>(in.y);
+  const int nseg = in.num_segments;
+
+  if (time_start)
+    (void)hipEventRecord(time_start, stream);
+  hipError_t err;
+  if ((err = launch_plan(in.ptr_x, in.n, nseg, kBinTile, tile_start, stream)) !=
+      hipSuccess)
+    return err;
+  if ((err = launch_plan(in.ptr_y, in.m, nseg, kWave, wave_start, stream)) !=
+      hipSuccess)
+    return err;
+  hipLaunchKernelGGL(seg_box_init_kernel, dim3((6 * nseg + kBlock - 1) / kBlock),
+                     dim3(kBlock), 0, stream, seg_box, 6 * nseg);
+  {
+    // enough workgroups per segment to fill the device when segments are few
+    const int parts = std::max(
+        1, std::min((in.n / nseg + 8 * kBlock - 1) / (8 * kBlock),
+                    std::max(1, 2048 / nseg)));
+    hipLaunchKernelGGL(seg_box_kernel, dim3(parts, std::min(nseg, 65535)),
+                       dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
+                       seg_box);
+  }
+  hipLaunchKernelGGL(morton_keys_kernel, dim3((in.n + kBlock - 1) / kBlock),
+                     dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
+                     seg_box, keys_a, vals_a);
+  if ((err = hipGetLastError()) != hipSuccess)
+    return err;
+  if ((err = sort_pairs(sort_temp, sort_bytes, keys_a, keys_x, vals_a, perm_x,
+                        in.n, nseg, stream)) != hipSuccess)
+    return err;
+  hipLaunchKernelGGL(morton_keys_kernel, dim3((in.m + kBlock - 1) / kBlock),
+                     dim3(kBlock), 0, stream, y, in.ptr_y, in.m, in.d, nseg,
+                     seg_box, keys_a, vals_a);
+  if ((err = hipGetLastError()) != hipSuccess)
+    return err;
+  sort_bytes = lay.sort_temp;
+  if ((err = sort_pairs(sort_temp, sort_bytes, keys_a, keys_y, vals_a, perm_y,
+                        in.m, nseg, stream)) != hipSuccess)
+    return err;
+  {
+    const int tiles = lay.box_stride;
+    const int per_block = kBlock / kBinTile;
+    hipLaunchKernelGGL(gather_tiles_kernel,
+                       dim3((tiles + per_block - 1) / per_block), dim3(kBlock),
+                       0, stream, x, in.ptr_x, in.n, in.d, nseg, tile_start,
+                       perm_x, rows, box, lay.box_stride);
+  }
+  if ((err = hipGetLastError()) != hipSuccess)
+    return err;
+
+  BinnedParams p;
+  p.y = y;
+  p.ptr_x = in.ptr_x;
+  p.ptr_y = in.ptr_y;
+  p.n = in.n;
+  p.m = in.m;
+  p.d = in.d;
+  p.num_segments = nseg;
+  p.k = k;
+  p.tile_start = tile_start;
+  p.wave_start = wave_start;
+  p.keys_x = keys_x;
+  p.keys_y = keys_y;
+  p.perm_y = perm_y;
+  p.rows = rows;
+  p.box = box;
+  p.box_stride = lay.box_stride;
+  p.out_idx = out.idx;
+  p.out_dist = out.dist;
+  p.out_count = out.count;
+  const int waves = plan_upper_bound(in.m, nseg, kWave);
+  const int grid = (waves + kBlock / kWave - 1) / (kBlock / kWave);
+  if (k <= 8)
+    hipLaunchKernelGGL((knn_binned_kernel<8>), dim3(grid), dim3(kBlock), 0,
+                       stream, p);
+  else if (k <= 16)
+    hipLaunchKernelGGL((knn_binned_kernel<16>), dim3(grid), dim3(kBlock), 0,
+                       stream, p);
+  else if (k <= 24)
+    hipLaunchKernelGGL((knn_binned_kernel<24>), dim3(grid), dim3(kBlock), 0,
+                       stream, p);
+  else
+    hipLaunchKernelGGL((knn_binned_kernel<32>), dim3(grid), dim3(kBlock), 0,
+                       stream, p);
+  if (time_stop)
+    (void)hipEventRecord(time_stop, stream);
+  return hipGetLastError();
+}
+
+} // namespace pca

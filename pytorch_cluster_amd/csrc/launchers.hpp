@@ -80,6 +80,17 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
                            hipStream_t stream,
                            int64_t *nearest_out = nullptr);
 
+// --- knn_binned.hip --------------------------------------------------------
+
+// Exact Euclidean kNN for fp32 points of up to 3 dimensions, k <= 32, over
+// rows binned along a space-filling curve (same results as the scans).
+bool knn_binned_supported(int d, int k, bool cosine);
+size_t knn_binned_scratch_bytes(int n, int m, int num_segments);
+// The events bracket everything from binning to the search kernel.
+hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
+                             const DenseResult &out, hipEvent_t time_start,
+                             hipEvent_t time_stop, hipStream_t stream);
+
 // --- knn_mfma*.hip ---------------------------------------------------------
 
 constexpr int kMfmaTileQueries = 128;

@@ -1,0 +1,159 @@
+"""GPU parity of the binned kNN search (pca_knn_binned through the C ABI).
+
+It stands under the same operator as pca_knn and must return the same edges
+and distances, bit for bit and in the same order: checked against the CPU
+oracle (the reference kernel's scan, csrc/cuda/knn_cuda.cu:30-84, evaluated
+with fused multiply-adds) at sizes the oracle finishes in seconds, and against
+the scanning kernels of pca_knn at full size.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from pytorch_cluster_amd import capi, testing  # noqa: E402
+from gpu_common import DEV, dev, gpu_knn, oracle_knn_edges, ragged_ptrs  # noqa
+
+
+def gpu_knn_binned(x, y, ptr_x, ptr_y, k, want_dist=True, **kw):
+    e, d = capi.knn_edges(dev(x), dev(y), dev(ptr_x, torch.long),
+                          dev(ptr_y, torch.long), k, False, want_dist,
+                          binned=True, **kw)
+    torch.cuda.synchronize()
+    return e.cpu().numpy(), (None if d is None else d.cpu().numpy())
+
+
+def check(oracle, x, y, ptr_x, ptr_y, k):
+    want_e, want_d = oracle_knn_edges(oracle, x, y, ptr_x, ptr_y, k)
+    got_e, got_d = gpu_knn_binned(x, y, ptr_x, ptr_y, k)
+    assert got_e.shape == want_e.shape
+    assert (got_e == want_e).all()
+    assert (got_d.view(np.uint32) == want_d.view(np.uint32)).all()
+
+
+@pytest.mark.parametrize("d", [1, 2, 3])
+@pytest.mark.parametrize("k", [1, 5, 8, 16, 17, 32])
+def test_random_clouds(oracle, d, k):
+    rng = np.random.default_rng(10 * d + k)
+    x = rng.standard_normal((5000, d)).astype(np.float32)
+    y = rng.standard_normal((700, d)).astype(np.float32)
+    check(oracle, x, y, None, None, k)
+
+
+@pytest.mark.parametrize("segments", [2, 5, 40])
+@pytest.mark.parametrize("k", [3, 16, 24])
+def test_ragged_segments(oracle, segments, k):
+    """Segments of uneven size, one of them empty, some shorter than k."""
+    rng = np.random.default_rng(segments + k)
+    n, m = 6000, 1500
+    ptr_x = ragged_ptrs(rng, n, segments)
+    ptr_y = ragged_ptrs(rng, m, segments)
+    x = rng.random((n, 3)).astype(np.float32)
+    y = rng.random((m, 3)).astype(np.float32)
+    check(oracle, x, y, ptr_x, ptr_y, k)
+
+
+@pytest.mark.parametrize("d", [2, 3])
+@pytest.mark.parametrize("k", [4, 16, 32])
+def test_ties_go_to_the_lower_row(oracle, d, k):
+    """Points on a coarse integer grid: most k-th distances are shared by
+    several rows, which the binned search meets out of row order."""
+    rng = np.random.default_rng(d * 100 + k)
+    x = rng.integers(0, 6, (4000, d)).astype(np.float32)
+    y = rng.integers(0, 6, (500, d)).astype(np.float32)
+    ptr_x = np.array([0, 2500, 4000], dtype=np.int64)
+    ptr_y = np.array([0, 200, 500], dtype=np.int64)
+    check(oracle, x, y, ptr_x, ptr_y, k)
+
+
+def test_all_rows_equal(oracle):
+    x = np.ones((3000, 3), dtype=np.float32)
+    y = np.ones((130, 3), dtype=np.float32)
+    check(oracle, x, y, None, None, 16)
+
+
+def test_self_search_lidar_like(oracle):
+    """Queries that are rows of x (every 4th), strongly varying density."""
+    c = testing.lidar_scans(0, scans=2, min_points=4000, max_points=6000)
+    x, y = c["x"].numpy(), c["y"].numpy()
+    ptr_x = testing.pointers(c["batch_x"], 2).numpy()
+    ptr_y = testing.pointers(c["batch_y"], 2).numpy()
+    check(oracle, x, y, ptr_x, ptr_y, 16)
+
+
+def test_queries_far_from_the_rows(oracle):
+    rng = np.random.default_rng(7)
+    x = rng.random((3000, 3)).astype(np.float32)
+    y = (rng.random((300, 3)) * 50 - 25).astype(np.float32)
+    check(oracle, x, y, None, None, 10)
+
+
+def test_rows_and_queries_that_are_not_finite(oracle):
+    """NaN and infinite coordinates never make a neighbour (their distances
+    are not below 1e10); neither do rows farther than 1e5 away."""
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((2000, 3)).astype(np.float32)
+    y = rng.standard_normal((200, 3)).astype(np.float32)
+    x[5, 1] = np.nan
+    x[64:96] = np.nan          # a whole tile's worth, wherever they land
+    x[700, 0] = np.inf
+    x[701, 2] = -np.inf
+    x[900] = 3e5               # squared distance 2.7e11 >= 1e10
+    y[3, 0] = np.nan
+    y[4, 2] = np.inf
+    y[5] = 3e5                 # finds only x[900]
+    check(oracle, x, y, None, None, 8)
+
+
+def test_fewer_rows_than_k_and_single_rows(oracle):
+    rng = np.random.default_rng(9)
+    ptr_x = np.array([0, 1, 4, 4, 40, 300], dtype=np.int64)
+    ptr_y = np.array([0, 3, 5, 9, 9, 100], dtype=np.int64)
+    x = rng.random((300, 2)).astype(np.float32)
+    y = rng.random((100, 2)).astype(np.float32)
+    check(oracle, x, y, ptr_x, ptr_y, 12)
+
+
+def test_edge_options_match_the_scanning_search():
+    g = torch.Generator().manual_seed(4)
+    x = torch.rand(5000, 3, generator=g).to(DEV)
+    ptr = torch.tensor([0, 1000, 5000], device=DEV)
+    for drop_self, x_first in ((True, False), (False, True), (True, True)):
+        a, _ = capi.knn_edges(x, x, ptr, ptr, 9, drop_self=drop_self,
+                              x_first=x_first)
+        b, _ = capi.knn_edges(x, x, ptr, ptr, 9, drop_self=drop_self,
+                              x_first=x_first, binned=True)
+        assert torch.equal(a, b)
+
+
+def test_full_size_against_the_scanning_kernels():
+    """The ragged LiDAR-like workload at full size (1M points, 258k queries):
+    identical edges and distances from both searches."""
+    c = testing.lidar_scans(0)
+    x, y = c["x"].to(DEV), c["y"].to(DEV)
+    px = testing.pointers(c["batch_x"], c["batch_size"]).to(DEV)
+    py = testing.pointers(c["batch_y"], c["batch_size"]).to(DEV)
+    a, da = capi.knn_edges(x, y, px, py, 16, want_dist=True)
+    b, db = capi.knn_edges(x, y, px, py, 16, want_dist=True, binned=True)
+    assert torch.equal(a, b)
+    assert torch.equal(da.view(torch.int32), db.view(torch.int32))
+
+
+def test_uniform_clouds_against_the_scanning_kernels():
+    c = testing.uniform_batched(0)
+    x = c["x"].to(DEV)
+    ptr = (torch.arange(17) * 4096).to(DEV)
+    a, da = capi.knn_edges(x, x, ptr, ptr, 21, want_dist=True)
+    b, db = capi.knn_edges(x, x, ptr, ptr, 21, want_dist=True, binned=True)
+    assert torch.equal(a, b)
+    assert torch.equal(da.view(torch.int32), db.view(torch.int32))
+
+
+def test_unsupported_shapes_are_refused():
+    x = torch.rand(100, 4, device=DEV)
+    with pytest.raises(RuntimeError, match="binned search"):
+        capi.knn_edges(x, x, None, None, 4, binned=True)
+    x = torch.rand(100, 3, device=DEV)
+    with pytest.raises(RuntimeError, match="binned search"):
+        capi.knn_edges(x, x, None, None, 33, binned=True)
