@@ -14,22 +14,26 @@
 // (one per lane) are neighbours in space and share one bounding box.
 //
 // A wave first scans the tiles around its queries' position in the order of x
-// (that fills the lists and gives every query a k-th distance), then sweeps
-// the segment's tile boxes 64 at a time, one per lane, outwards from that
-// position: a tile is scanned only if the smallest distance between its box
-// and the wave's box is not above the largest k-th distance among the wave's
-// queries.  That box distance is computed with the operations of the exact
-// chain (one difference per axis, product, fused multiply-adds in the same
-// order) applied to per-axis gaps that are not above any row's difference:
-// rounding is monotone, so the value is never above the computed distance of
-// any (query, row) pair of the two boxes, and a skipped tile cannot hold a
-// neighbour.  Rows of a scanned tile are uniform over the wave (scalar
-// loads); a lane whose distance passes its own bound parks (distance, row) in
-// a queue in LDS, and the queues are emptied into the sorted lists by all
-// lanes together when one fills up, as in the scanning kernels.  Rows arrive
-// out of row order here, so a row of EQUAL distance may still displace a
-// neighbour with a larger row number: a full list admits d <= its k-th
-// distance and the 64-bit (distance, row) keys decide.
+// (that fills the lists and gives every query a k-th distance), then goes
+// through the segment's groups of 64 tiles outwards from that position: a
+// group, and inside it a tile, is looked into only if for SOME lane the
+// distance from its query to the box is not above that query's k-th distance
+// (the boxes are uniform over the wave: scalar loads; the test is a dozen
+// vector instructions per box for all 64 queries).  That box distance is
+// computed with the operations of the exact chain (one difference per axis,
+// product, fused multiply-adds in the same order) applied to per-axis gaps
+// that are not above any row's difference: rounding is monotone, so the value
+// is never above the computed distance of any row of the box, and a skipped
+// tile cannot hold a neighbour.  Testing per query, not per wave, bounds the
+// work of a wave whose queries straddle a jump of the curve: it pays for the
+// neighbourhoods of its queries, not for the space between them.
+// Rows of a scanned tile are uniform over the wave as well; a lane whose
+// distance passes its own bound parks (distance, row) in a queue in LDS, and
+// the queues are emptied into the sorted lists by all lanes together when one
+// fills up, as in the scanning kernels.  Rows arrive out of row order here, so
+// a row of EQUAL distance may still displace a neighbour with a larger row
+// number: a full list admits d <= its k-th distance and the 64-bit
+// (distance, row) keys decide.
 #include "device_utils.hpp"
 #include "knn_lowd_impl.hpp"
 #include "launchers.hpp"
@@ -44,6 +48,7 @@ namespace pca {
 namespace {
 
 constexpr int kBinTile = 32;      // rows per tile
+constexpr int kBinGroup = 64;     // tiles per group (a box of their own)
 constexpr int kBinQueueCap = 16;  // parked rows per lane
 constexpr int kBinSeedTiles = 16; // most tiles scanned before the sweep
 constexpr int kCodeBits = 30;
@@ -164,13 +169,21 @@ __global__ __launch_bounds__(kBlock) void morton_keys_kernel(
   vals[i] = (uint32_t)i;
 }
 
+// A box: lower corner, upper corner, two words of padding (one 32-byte scalar
+// load).
+struct Box {
+  float lo[3];
+  float hi[3];
+  float pad[2];
+};
+
 // Rows in curve order with their row numbers, and the box of every tile of 32:
-// half a wave per tile.  box: [6][box_stride], lower then upper corner.
+// half a wave per tile.
 __global__ __launch_bounds__(kBlock) void gather_tiles_kernel(
     const float *__restrict__ x, const int64_t *__restrict__ ptr_x, int n,
     int d, int num_segments, const int *__restrict__ tile_start,
     const uint32_t *__restrict__ perm, float4 *__restrict__ rows,
-    float *__restrict__ box, int box_stride) {
+    Box *__restrict__ box) {
   const int gt = (blockIdx.x * kBlock + threadIdx.x) / kBinTile;
   const int r = threadIdx.x & (kBinTile - 1);
   if (gt >= tile_start[num_segments])
@@ -199,8 +212,39 @@ __global__ __launch_bounds__(kBlock) void gather_tiles_kernel(
       hi = __builtin_fmaxf(hi, __shfl_xor(hi, sh));
     }
     if (r == 0) {
-      box[(size_t)c * box_stride + gt] = lo;
-      box[(size_t)(3 + c) * box_stride + gt] = hi;
+      box[gt].lo[c] = lo;
+      box[gt].hi[c] = hi;
+    }
+  }
+}
+
+// Boxes of the groups of kBinGroup consecutive tiles of a segment: one wave
+// per group.
+__global__ __launch_bounds__(kBlock) void group_boxes_kernel(
+    int num_segments, const int *__restrict__ tile_start,
+    const int *__restrict__ group_start, const Box *__restrict__ box,
+    Box *__restrict__ group_box) {
+  const int gg = (blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  if (gg >= group_start[num_segments])
+    return;
+  const int seg = find_segment(group_start, num_segments, gg);
+  const int t = (gg - group_start[seg]) * kBinGroup + lane;
+  const int tiles = tile_start[seg + 1] - tile_start[seg];
+  const bool ok = t < tiles;
+  static_assert(kBinGroup == kWave, "one tile per lane");
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    float lo = ok ? box[tile_start[seg] + t].lo[c] : __builtin_inff();
+    float hi = ok ? box[tile_start[seg] + t].hi[c] : -__builtin_inff();
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1) {
+      lo = __builtin_fminf(lo, __shfl_xor(lo, sh));
+      hi = __builtin_fmaxf(hi, __shfl_xor(hi, sh));
+    }
+    if (lane == 0) {
+      group_box[gg].lo[c] = lo;
+      group_box[gg].hi[c] = hi;
     }
   }
 }
@@ -216,8 +260,9 @@ struct BinnedParams {
   const uint64_t *keys_y;   // sorted keys of the queries
   const uint32_t *perm_y;   // query behind every sorted position
   const float4 *rows;       // x rows in curve order, .w = row number
-  const float *box;         // [6][box_stride]
-  int box_stride;
+  const Box *box;           // of every tile
+  const int *group_start;   // first group of tiles of every segment
+  const Box *group_box;     // of every group
   int *out_idx;
   float *out_dist;
   int *out_count;
@@ -298,11 +343,11 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
   // a row is parked when its distance is strictly below `admit`: the limit
   // while the list has room, just above the k-th distance afterwards (a row of
   // equal distance and smaller number still gets in); nothing for a lane
-  // that does not search
+  // that does not search.  `kth`: the k-th distance (the limit while the list
+  // has room; below every distance for a lane that does not search): a box
+  // farther away than that holds no neighbour of this lane's query.
   float admit = searching ? kKnnSentinel : -__builtin_inff();
-  // largest k-th distance among the wave's queries (the limit while any list
-  // has room): tiles whose box is farther away are skipped
-  float reach = kKnnSentinel;
+  float kth = searching ? kKnnSentinel : -1.0f;
   int parked = 0;
 
   auto drain = [&]() {
@@ -316,44 +361,62 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
       // (parked under an older bound: the keys sort it out)
       const double key = (has && d < admit) ? make_key(d, id) : empty_key();
       sorted_insert<K>(best, key);
-      const float kth = key_dist(best[K - 1]);
-      if (searching && kth < kKnnSentinel)
-        admit = next_up_positive(kth);
+      const float now = key_dist(best[K - 1]);
+      if (searching && now < kKnnSentinel) {
+        kth = now;
+        admit = next_up_positive(now);
+      }
     }
-    float r = searching ? key_dist(best[K - 1]) : 0.0f;
-#pragma unroll
-    for (int sh = 1; sh < kWave; sh <<= 1)
-      r = __builtin_fmaxf(r, __shfl_xor(r, sh));
-    reach = r;
   };
 
-  // rows of one tile against every lane's query
+  // rows of one tile against every lane's query, four rows per step (the
+  // copy of the rows is padded, so a step may read past the tile's rows)
   auto scan_tile = [&](int tile) {
     const int j0 = x_begin + tile * kBinTile;
     const int rows = min(kBinTile, x_end - j0);
     const float4 *__restrict__ src = p.rows + j0;
-    for (int r = 0; r < rows; ++r) {
-      const float4 row = src[r]; // (uniform address)
-      const float d0 = row.x - yq[0];
-      float dd = d0 * d0;
-      const float d1 = row.y - yq[1];
-      dd = __builtin_fmaf(d1, d1, dd);
-      const float d2 = row.z - yq[2];
-      dd = __builtin_fmaf(d2, d2, dd);
-      const bool hit = dd < admit;
-      if (hit) {
-        queue_d[parked][tid] = dd;
-        queue_id[parked][tid] = __float_as_uint(row.w);
-        ++parked;
+    for (int r = 0; r < rows; r += 4) {
+      float4 row[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        row[u] = src[r + u]; // (uniform addresses)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float d0 = row[u].x - yq[0];
+        float dd = d0 * d0;
+        const float d1 = row[u].y - yq[1];
+        dd = __builtin_fmaf(d1, d1, dd);
+        const float d2 = row[u].z - yq[2];
+        dd = __builtin_fmaf(d2, d2, dd);
+        const bool hit = dd < admit && r + u < rows;
+        if (hit) {
+          queue_d[parked][tid] = dd;
+          queue_id[parked][tid] = __float_as_uint(row[u].w);
+          ++parked;
+        }
       }
-      if (__any(parked == kBinQueueCap))
+      if (__any(parked > kBinQueueCap - 4))
         drain();
     }
   };
 
+  // Squared distance from the lane's query to a box, with the operations of
+  // the exact chain on per-axis gaps that are not above |row - query| for any
+  // row of the box: never above the computed distance of any of its rows.  (A
+  // NaN - from an infinite or empty box - never rules a box out.)
+  auto box_reachable = [&](const Box &b) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      const float gap = __builtin_fmaxf(
+          __builtin_fmaxf(b.lo[c] - yq[c], yq[c] - b.hi[c]), 0.0f);
+      acc = c == 0 ? gap * gap : __builtin_fmaf(gap, gap, acc);
+    }
+    return !(acc > kth);
+  };
+
   const int tile0 = p.tile_start[seg];
   const int num_tiles = p.tile_start[seg + 1] - tile0;
-  int seed_lo = 0, seed_hi = -1; // tiles seed_lo .. seed_hi scanned up front
   if (num_tiles > 0) {
     // where the wave's first and last query fall in the order of x
     const int last_lane = min(kWave, y_end - (jq - lane)) - 1;
@@ -367,8 +430,9 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
         wave_lower_bound(p.keys_x, x_begin, x_end, key_last, lane);
     const int t_first = min(num_tiles - 1, (pos_first - x_begin) / kBinTile);
     const int t_last = min(num_tiles - 1, (pos_last - x_begin) / kBinTile);
-    seed_lo = max(0, t_first - 1);
-    seed_hi = min(num_tiles - 1, max(t_last, t_first) + 1);
+    // tiles seed_lo .. seed_hi are scanned up front
+    int seed_lo = max(0, t_first - 1);
+    int seed_hi = min(num_tiles - 1, max(t_last, t_first) + 1);
     if (seed_hi - seed_lo + 1 > kBinSeedTiles) {
       // queries far apart in the order of x: the middle of their range
       const int mid = (seed_lo + seed_hi) / 2;
@@ -379,45 +443,27 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
       scan_tile(t);
     drain();
 
-    // sweep of the tile boxes, 64 per round, outwards from the seed tiles
-    const int num_rounds = (num_tiles + kWave - 1) / kWave;
-    const int centre = ((seed_lo + seed_hi) / 2) / kWave;
-    for (int i = 0; i < 2 * num_rounds; ++i) {
-      const int round = centre + ((i & 1) ? -((i + 1) >> 1) : (i >> 1));
-      if (round < 0 || round >= num_rounds)
+    // groups of tiles outwards from the seed tiles; a group, then a tile, is
+    // looked into only if some lane's query can reach its box
+    const int group0 = p.group_start[seg];
+    const int num_groups = (num_tiles + kBinGroup - 1) / kBinGroup;
+    const int centre = ((seed_lo + seed_hi) / 2) / kBinGroup;
+    for (int i = 0; i < 2 * num_groups; ++i) {
+      const int group = centre + ((i & 1) ? -((i + 1) >> 1) : (i >> 1));
+      if (group < 0 || group >= num_groups)
         continue;
-      const int t = round * kWave + lane;
-      float gap2 = __builtin_inff();
-      if (t < num_tiles && !(t >= seed_lo && t <= seed_hi)) {
-        const size_t g = (size_t)(tile0 + t);
-        float acc = 0.0f;
-#pragma unroll
-        for (int c = 0; c < 3; ++c) {
-          const float lo = p.box[(size_t)c * p.box_stride + g];
-          const float hi = p.box[(size_t)(3 + c) * p.box_stride + g];
-          // not above |row - query| along this axis for any pair of the boxes
-          // (a NaN, from an infinite or empty box, survives to the test below)
-          const float gap =
-              __builtin_fmaxf(__builtin_fmaxf(lo - q_hi[c], q_lo[c] - hi), 0.0f);
-          acc = c == 0 ? gap * gap : __builtin_fmaf(gap, gap, acc);
-        }
-        gap2 = acc;
+      if (!__any(box_reachable(p.group_box[group0 + group])))
+        continue;
+      const int t_end = min(num_tiles, (group + 1) * kBinGroup);
+      for (int t = group * kBinGroup; t < t_end; ++t) {
+        if (t >= seed_lo && t <= seed_hi)
+          continue;
+        if (!__any(box_reachable(p.box[tile0 + t])))
+          continue;
+        scan_tile(t);
       }
-      // (!(a > b): a NaN box distance never skips a tile)
-      uint64_t todo = __ballot(t < num_tiles &&
-                               !(t >= seed_lo && t <= seed_hi) &&
-                               !(gap2 > reach));
-      while (todo != 0) {
-        const int src_lane = (int)__builtin_ctzll(todo);
-        todo &= todo - 1;
-        const float g2 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
-            (int)__float_as_uint(gap2), src_lane));
-        if (g2 > reach)
-          continue; // the bound has moved since the ballot
-        scan_tile(round * kWave + src_lane);
-        if (__any(parked > 0))
-          drain();
-      }
+      if (__any(parked > 0))
+        drain();
     }
   }
 
@@ -427,11 +473,12 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
 
 struct BinnedLayout {
   size_t seg_box, keys_a, keys_x, keys_y, vals_a, perm_x, perm_y, rows, box,
-      tile_start, wave_start, sort_temp;
-  int box_stride;
+      group_box, tile_start, group_start, wave_start, sort_temp;
+  int tiles_bound, groups_bound;
   size_t total() const {
     return seg_box + keys_a + keys_x + keys_y + vals_a + perm_x + perm_y +
-           rows + box + tile_start + wave_start + sort_temp;
+           rows + box + group_box + tile_start + group_start + wave_start +
+           sort_temp;
   }
 };
 
@@ -462,10 +509,14 @@ BinnedLayout binned_layout(int n, int m, int num_segments) {
   w.vals_a = align256(sizeof(uint32_t) * big);
   w.perm_x = align256(sizeof(uint32_t) * (size_t)n);
   w.perm_y = align256(sizeof(uint32_t) * (size_t)m);
-  w.rows = align256(sizeof(float4) * (size_t)n);
-  w.box_stride = plan_upper_bound(n, num_segments, kBinTile);
-  w.box = align256(sizeof(float) * 6 * (size_t)w.box_stride);
+  // (padded: the search reads rows four at a time)
+  w.rows = align256(sizeof(float4) * ((size_t)n + kBinTile));
+  w.tiles_bound = plan_upper_bound(n, num_segments, kBinTile);
+  w.groups_bound = plan_upper_bound(n, num_segments, kBinTile * kBinGroup);
+  w.box = align256(sizeof(Box) * (size_t)w.tiles_bound);
+  w.group_box = align256(sizeof(Box) * (size_t)w.groups_bound);
   w.tile_start = align256(sizeof(int) * (size_t)(num_segments + 1));
+  w.group_start = align256(sizeof(int) * (size_t)(num_segments + 1));
   w.wave_start = align256(sizeof(int) * (size_t)(num_segments + 1));
   size_t tx = 0, ty = 0;
   const hipError_t ex = sort_pairs(nullptr, tx, nullptr, nullptr, nullptr,
@@ -507,8 +558,10 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
   uint32_t *perm_x = static_cast<uint32_t *>(take(lay.perm_x));
   uint32_t *perm_y = static_cast<uint32_t *>(take(lay.perm_y));
   float4 *rows = static_cast<float4 *>(take(lay.rows));
-  float *box = static_cast<float *>(take(lay.box));
+  Box *box = static_cast<Box *>(take(lay.box));
+  Box *group_box = static_cast<Box *>(take(lay.group_box));
   int *tile_start = static_cast<int *>(take(lay.tile_start));
+  int *group_start = static_cast<int *>(take(lay.group_start));
   int *wave_start = static_cast<int *>(take(lay.wave_start));
   void *sort_temp = take(lay.sort_temp);
   size_t sort_bytes = lay.sort_temp;
@@ -522,6 +575,9 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
   hipError_t err;
   if ((err = launch_plan(in.ptr_x, in.n, nseg, kBinTile, tile_start, stream)) !=
       hipSuccess)
+    return err;
+  if ((err = launch_plan(in.ptr_x, in.n, nseg, kBinTile * kBinGroup,
+                         group_start, stream)) != hipSuccess)
     return err;
   if ((err = launch_plan(in.ptr_y, in.m, nseg, kWave, wave_start, stream)) !=
       hipSuccess)
@@ -555,12 +611,17 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
                         in.m, nseg, stream)) != hipSuccess)
     return err;
   {
-    const int tiles = lay.box_stride;
     const int per_block = kBlock / kBinTile;
     hipLaunchKernelGGL(gather_tiles_kernel,
-                       dim3((tiles + per_block - 1) / per_block), dim3(kBlock),
-                       0, stream, x, in.ptr_x, in.n, in.d, nseg, tile_start,
-                       perm_x, rows, box, lay.box_stride);
+                       dim3((lay.tiles_bound + per_block - 1) / per_block),
+                       dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
+                       tile_start, perm_x, rows, box);
+    const int groups_per_block = kBlock / kWave;
+    hipLaunchKernelGGL(
+        group_boxes_kernel,
+        dim3((lay.groups_bound + groups_per_block - 1) / groups_per_block),
+        dim3(kBlock), 0, stream, nseg, tile_start, group_start, box,
+        group_box);
   }
   if ((err = hipGetLastError()) != hipSuccess)
     return err;
@@ -581,7 +642,8 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
   p.perm_y = perm_y;
   p.rows = rows;
   p.box = box;
-  p.box_stride = lay.box_stride;
+  p.group_start = group_start;
+  p.group_box = group_box;
   p.out_idx = out.idx;
   p.out_dist = out.dist;
   p.out_count = out.count;
