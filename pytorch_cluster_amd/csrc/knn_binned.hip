@@ -17,9 +17,11 @@
 // (that fills the lists and gives every query a k-th distance), then goes
 // through the segment's groups of 64 tiles outwards from that position: a
 // group, and inside it a tile, is looked into only if for SOME lane the
-// distance from its query to the box is not above that query's k-th distance
-// (the boxes are uniform over the wave: scalar loads; the test is a dozen
-// vector instructions per box for all 64 queries).  That box distance is
+// distance from its query to the box is not above that query's k-th distance.
+// Boxes are tested 64 at a time first (one per lane, against the box around
+// the wave's queries and the wave's largest k-th distance); the few that pass
+// are broadcast lane by lane for the per-query test (a dozen vector
+// instructions per box for all 64 queries).  That box distance is
 // computed with the operations of the exact chain (one difference per axis,
 // product, fused multiply-adds in the same order) applied to per-axis gaps
 // that are not above any row's difference: rounding is monotone, so the value
@@ -51,7 +53,6 @@ constexpr int kBinTile = 32;      // rows per tile
 constexpr int kBinGroup = 64;     // tiles per group (a box of their own)
 constexpr int kBinQueueCap = 16;  // parked rows per lane
 constexpr int kBinSeedTiles = 16; // most tiles scanned before the sweep
-constexpr int kCodeBits = 30;
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
@@ -91,6 +92,7 @@ __global__ void seg_box_init_kernel(int *seg_box, int count) {
 __global__ __launch_bounds__(kBlock) void seg_box_kernel(
     const float *__restrict__ x, const int64_t *__restrict__ ptr_x, int n,
     int d, int seg_count, int *__restrict__ seg_box) {
+  __shared__ float part[kBlock / kWave][6];
   for (int seg = blockIdx.y; seg < seg_count; seg += gridDim.y) {
     const int64_t begin = ptr_x ? ptr_x[seg] : 0;
     const int64_t end = ptr_x ? ptr_x[seg + 1] : n;
@@ -120,12 +122,25 @@ __global__ __launch_bounds__(kBlock) void seg_box_kernel(
         hi[c] = __builtin_fmaxf(hi[c], __shfl_xor(hi[c], sh));
       }
     }
+    // one set of atomic updates per workgroup
+    __syncthreads(); // (the previous segment's values have been read)
     if ((threadIdx.x & (kWave - 1)) == 0) {
 #pragma unroll
       for (int c = 0; c < 3; ++c) {
-        atomicMin(&seg_box[seg * 6 + c], ordered_int(lo[c]));
-        atomicMax(&seg_box[seg * 6 + 3 + c], ordered_int(hi[c]));
+        part[threadIdx.x / kWave][c] = lo[c];
+        part[threadIdx.x / kWave][3 + c] = hi[c];
       }
+    }
+    __syncthreads();
+    if (threadIdx.x < 6) {
+      float v = part[0][threadIdx.x];
+      for (int w = 1; w < kBlock / kWave; ++w)
+        v = threadIdx.x < 3 ? __builtin_fminf(v, part[w][threadIdx.x])
+                            : __builtin_fmaxf(v, part[w][threadIdx.x]);
+      if (threadIdx.x < 3)
+        atomicMin(&seg_box[seg * 6 + threadIdx.x], ordered_int(v));
+      else
+        atomicMax(&seg_box[seg * 6 + threadIdx.x], ordered_int(v));
     }
   }
 }
@@ -140,13 +155,14 @@ __device__ __forceinline__ uint32_t spread3(uint32_t v) {
   return v;
 }
 
-// keys[i] = (segment << 30) | Morton code of row i inside its segment's box of
-// x rows (coordinates outside the box, NaN and missing axes go to its border);
-// vals[i] = i.
+// keys[i] = (segment << 3 axis_bits) | Morton code of row i inside its
+// segment's box of x rows, axis_bits bits per axis (coordinates outside the
+// box, NaN and missing axes go to its border); vals[i] = i.
 __global__ __launch_bounds__(kBlock) void morton_keys_kernel(
     const float *__restrict__ pts, const int64_t *__restrict__ ptr, int count,
     int d, int num_segments, const int *__restrict__ seg_box,
-    uint64_t *__restrict__ keys, uint32_t *__restrict__ vals) {
+    int axis_bits, uint32_t *__restrict__ keys,
+    uint32_t *__restrict__ vals) {
   const int i = blockIdx.x * kBlock + threadIdx.x;
   if (i >= count)
     return;
@@ -159,13 +175,14 @@ __global__ __launch_bounds__(kBlock) void morton_keys_kernel(
       const float lo = from_ordered_int(seg_box[seg * 6 + c]);
       const float hi = from_ordered_int(seg_box[seg * 6 + 3 + c]);
       const float v = pts[(size_t)i * d + c];
-      const float t = (v - lo) / (hi - lo) * 1024.0f;
+      const float cells = (float)(1 << axis_bits);
+      const float t = (v - lo) / (hi - lo) * cells;
       // (NaN, also from an empty or flat box, fails the first comparison)
-      cell = t >= 0.0f ? (uint32_t)__builtin_fminf(t, 1023.0f) : 0u;
+      cell = t >= 0.0f ? (uint32_t)__builtin_fminf(t, cells - 1.0f) : 0u;
     }
     code |= spread3(cell) << c;
   }
-  keys[i] = ((uint64_t)seg << kCodeBits) | code;
+  keys[i] = ((uint32_t)seg << (3 * axis_bits)) | code;
   vals[i] = (uint32_t)i;
 }
 
@@ -256,8 +273,8 @@ struct BinnedParams {
   int n, m, d, num_segments, k;
   const int *tile_start;    // first tile of every segment
   const int *wave_start;    // first wave task of every segment
-  const uint64_t *keys_x;   // sorted keys of the x rows
-  const uint64_t *keys_y;   // sorted keys of the queries
+  const uint32_t *keys_x;   // sorted keys of the x rows
+  const uint32_t *keys_y;   // sorted keys of the queries
   const uint32_t *perm_y;   // query behind every sorted position
   const float4 *rows;       // x rows in curve order, .w = row number
   const Box *box;           // of every tile
@@ -271,7 +288,7 @@ struct BinnedParams {
 // First position in [lo, hi) whose key is not below `key` (hi if none); the
 // wave probes 64 positions per round.
 __device__ __forceinline__ int wave_lower_bound(
-    const uint64_t *__restrict__ keys, int lo, int hi, uint64_t key,
+    const uint32_t *__restrict__ keys, int lo, int hi, uint32_t key,
     int lane) {
   while (hi - lo > kWave) {
     const int step = (hi - lo) / kWave;
@@ -400,19 +417,50 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
     }
   };
 
-  // Squared distance from the lane's query to a box, with the operations of
-  // the exact chain on per-axis gaps that are not above |row - query| for any
-  // row of the box: never above the computed distance of any of its rows.  (A
-  // NaN - from an infinite or empty box - never rules a box out.)
-  auto box_reachable = [&](const Box &b) {
+  // Squared distance between two boxes (a query is a box of one point), with
+  // the operations of the exact chain on per-axis gaps that are not above
+  // |row - query| for any row and query of the boxes: never above the computed
+  // distance of any such pair.
+  auto box_gap2 = [](const float (&alo)[3], const float (&ahi)[3],
+                     const float (&blo)[3], const float (&bhi)[3]) {
     float acc = 0.0f;
 #pragma unroll
     for (int c = 0; c < 3; ++c) {
       const float gap = __builtin_fmaxf(
-          __builtin_fmaxf(b.lo[c] - yq[c], yq[c] - b.hi[c]), 0.0f);
+          __builtin_fmaxf(alo[c] - bhi[c], blo[c] - ahi[c]), 0.0f);
       acc = c == 0 ? gap * gap : __builtin_fmaf(gap, gap, acc);
     }
-    return !(acc > kth);
+    return acc;
+  };
+  // largest k-th distance among the wave's queries
+  auto wave_reach = [&]() {
+    float r = kth;
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1)
+      r = __builtin_fmaxf(r, __shfl_xor(r, sh));
+    return r;
+  };
+  // Of the 64 boxes the lanes hold (lane l: box l, `mine` = it exists), is
+  // the box of lane `src` within reach of some lane's query?  (A NaN - from an
+  // infinite or empty box - never rules a box out.)
+  auto reachable = [&](const Box &held, int src) {
+    float lo[3], hi[3];
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      lo[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+          (int)__float_as_uint(held.lo[c]), src));
+      hi[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+          (int)__float_as_uint(held.hi[c]), src));
+    }
+    return __any(!(box_gap2(lo, hi, yq, yq) > kth));
+  };
+  // the set bit of `mask` nearest to position `at` (mask != 0)
+  auto nearest_bit = [](uint64_t mask, int at) {
+    const uint64_t up = mask >> at;
+    const uint64_t down = at > 0 ? mask & (~(uint64_t)0 >> (64 - at)) : 0;
+    const int d_up = up ? (int)__builtin_ctzll(up) : 128;
+    const int d_down = down ? at - (63 - (int)__builtin_clzll(down)) : 128;
+    return d_up <= d_down ? at + d_up : at - d_down;
   };
 
   const int tile0 = p.tile_start[seg];
@@ -420,9 +468,9 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
   if (num_tiles > 0) {
     // where the wave's first and last query fall in the order of x
     const int last_lane = min(kWave, y_end - (jq - lane)) - 1;
-    const uint64_t key_first =
+    const uint32_t key_first =
         p.keys_y[__builtin_amdgcn_readfirstlane(jq - lane)];
-    const uint64_t key_last =
+    const uint32_t key_last =
         p.keys_y[__builtin_amdgcn_readfirstlane(jq - lane + last_lane)];
     const int pos_first =
         wave_lower_bound(p.keys_x, x_begin, x_end, key_first, lane);
@@ -442,28 +490,56 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
     for (int t = seed_lo; t <= seed_hi; ++t)
       scan_tile(t);
     drain();
+    float reach = wave_reach();
 
-    // groups of tiles outwards from the seed tiles; a group, then a tile, is
-    // looked into only if some lane's query can reach its box
+    // Groups of tiles, 64 at a time (one box per lane), nearest to the seed
+    // tiles first.  A group, then a tile, is looked into if its box is within
+    // the wave's largest k-th distance of the box around the wave's queries
+    // (all 64 boxes at once), and then within some query's own k-th distance
+    // of that query (a dozen instructions per box).
     const int group0 = p.group_start[seg];
     const int num_groups = (num_tiles + kBinGroup - 1) / kBinGroup;
     const int centre = ((seed_lo + seed_hi) / 2) / kBinGroup;
-    for (int i = 0; i < 2 * num_groups; ++i) {
-      const int group = centre + ((i & 1) ? -((i + 1) >> 1) : (i >> 1));
-      if (group < 0 || group >= num_groups)
+    const int num_rounds = (num_groups + kWave - 1) / kWave;
+    const int centre_round = centre / kWave;
+    for (int i = 0; i < 2 * num_rounds; ++i) {
+      const int round = centre_round + ((i & 1) ? -((i + 1) >> 1) : (i >> 1));
+      if (round < 0 || round >= num_rounds)
         continue;
-      if (!__any(box_reachable(p.group_box[group0 + group])))
-        continue;
-      const int t_end = min(num_tiles, (group + 1) * kBinGroup);
-      for (int t = group * kBinGroup; t < t_end; ++t) {
-        if (t >= seed_lo && t <= seed_hi)
+      const int g_mine = round * kWave + lane;
+      Box g_box = {};
+      if (g_mine < num_groups)
+        g_box = p.group_box[group0 + g_mine];
+      uint64_t g_todo =
+          __ballot(g_mine < num_groups &&
+                   !(box_gap2(g_box.lo, g_box.hi, q_lo, q_hi) > reach));
+      const int g_at = min(max(centre - round * kWave, 0), kWave - 1);
+      while (g_todo != 0) {
+        const int g_lane = nearest_bit(g_todo, g_at);
+        g_todo &= ~((uint64_t)1 << g_lane);
+        if (!reachable(g_box, g_lane))
           continue;
-        if (!__any(box_reachable(p.box[tile0 + t])))
-          continue;
-        scan_tile(t);
+        const int group = round * kWave + g_lane;
+        const int t_mine = group * kBinGroup + lane;
+        const bool t_ok =
+            t_mine < num_tiles && !(t_mine >= seed_lo && t_mine <= seed_hi);
+        Box t_box = {};
+        if (t_ok)
+          t_box = p.box[tile0 + t_mine];
+        uint64_t t_todo = __ballot(
+            t_ok && !(box_gap2(t_box.lo, t_box.hi, q_lo, q_hi) > reach));
+        while (t_todo != 0) {
+          const int t_lane = (int)__builtin_ctzll(t_todo);
+          t_todo &= t_todo - 1;
+          if (!reachable(t_box, t_lane))
+            continue;
+          scan_tile(group * kBinGroup + t_lane);
+        }
+        if (__any(parked > 0)) {
+          drain();
+          reach = wave_reach();
+        }
       }
-      if (__any(parked > 0))
-        drain();
     }
   }
 
@@ -482,30 +558,36 @@ struct BinnedLayout {
   }
 };
 
-int key_bits(int num_segments) {
-  int bits = kCodeBits;
-  while (bits < 62 && ((int64_t)1 << (bits - kCodeBits)) < num_segments)
+// Keys are 32 bits: the segment above the Morton code, whose bits per axis
+// (at most 10) shrink as the segments get more (and with that smaller).
+int segment_bits(int num_segments) {
+  int bits = 0;
+  while (bits < 31 && ((int64_t)1 << bits) < num_segments)
     ++bits;
   return bits;
 }
+int axis_bits(int num_segments) {
+  return std::min(10, (32 - segment_bits(num_segments)) / 3);
+}
 
-hipError_t sort_pairs(void *temp, size_t &temp_bytes, const uint64_t *keys_in,
-                      uint64_t *keys_out, const uint32_t *vals_in,
+hipError_t sort_pairs(void *temp, size_t &temp_bytes, const uint32_t *keys_in,
+                      uint32_t *keys_out, const uint32_t *vals_in,
                       uint32_t *vals_out, int count, int num_segments,
                       hipStream_t stream) {
+  const int bits = segment_bits(num_segments) + 3 * axis_bits(num_segments);
   return rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out,
                                    vals_in, vals_out, (unsigned int)count, 0u,
-                                   (unsigned int)key_bits(num_segments),
-                                   stream, false);
+                                   (unsigned int)std::max(bits, 1), stream,
+                                   false);
 }
 
 BinnedLayout binned_layout(int n, int m, int num_segments) {
   BinnedLayout w;
   const size_t big = (size_t)std::max(n, m);
   w.seg_box = align256(sizeof(int) * 6 * (size_t)num_segments);
-  w.keys_a = align256(sizeof(uint64_t) * big);
-  w.keys_x = align256(sizeof(uint64_t) * (size_t)n);
-  w.keys_y = align256(sizeof(uint64_t) * (size_t)m);
+  w.keys_a = align256(sizeof(uint32_t) * big);
+  w.keys_x = align256(sizeof(uint32_t) * (size_t)n);
+  w.keys_y = align256(sizeof(uint32_t) * (size_t)m);
   w.vals_a = align256(sizeof(uint32_t) * big);
   w.perm_x = align256(sizeof(uint32_t) * (size_t)n);
   w.perm_y = align256(sizeof(uint32_t) * (size_t)m);
@@ -551,9 +633,9 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
     return static_cast<void *>(piece);
   };
   int *seg_box = static_cast<int *>(take(lay.seg_box));
-  uint64_t *keys_a = static_cast<uint64_t *>(take(lay.keys_a));
-  uint64_t *keys_x = static_cast<uint64_t *>(take(lay.keys_x));
-  uint64_t *keys_y = static_cast<uint64_t *>(take(lay.keys_y));
+  uint32_t *keys_a = static_cast<uint32_t *>(take(lay.keys_a));
+  uint32_t *keys_x = static_cast<uint32_t *>(take(lay.keys_x));
+  uint32_t *keys_y = static_cast<uint32_t *>(take(lay.keys_y));
   uint32_t *vals_a = static_cast<uint32_t *>(take(lay.vals_a));
   uint32_t *perm_x = static_cast<uint32_t *>(take(lay.perm_x));
   uint32_t *perm_y = static_cast<uint32_t *>(take(lay.perm_y));
@@ -587,15 +669,15 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
   {
     // enough workgroups per segment to fill the device when segments are few
     const int parts = std::max(
-        1, std::min((in.n / nseg + 8 * kBlock - 1) / (8 * kBlock),
-                    std::max(1, 2048 / nseg)));
+        1, std::min((in.n / nseg + 16 * kBlock - 1) / (16 * kBlock),
+                    std::max(1, 1024 / nseg)));
     hipLaunchKernelGGL(seg_box_kernel, dim3(parts, std::min(nseg, 65535)),
                        dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
                        seg_box);
   }
   hipLaunchKernelGGL(morton_keys_kernel, dim3((in.n + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
-                     seg_box, keys_a, vals_a);
+                     seg_box, axis_bits(nseg), keys_a, vals_a);
   if ((err = hipGetLastError()) != hipSuccess)
     return err;
   if ((err = sort_pairs(sort_temp, sort_bytes, keys_a, keys_x, vals_a, perm_x,
@@ -603,7 +685,7 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
     return err;
   hipLaunchKernelGGL(morton_keys_kernel, dim3((in.m + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, y, in.ptr_y, in.m, in.d, nseg,
-                     seg_box, keys_a, vals_a);
+                     seg_box, axis_bits(nseg), keys_a, vals_a);
   if ((err = hipGetLastError()) != hipSuccess)
     return err;
   sort_bytes = lay.sort_temp;
