@@ -11,7 +11,25 @@ from .knn import knn, knn_graph
 from .nearest import nearest
 from .radius import radius, radius_graph
 
+import torch as _torch
+
 __version__ = "0.1.0"
 
+
+def set_knn_strategy(name: str) -> None:
+    """How ``knn`` / ``knn_graph`` search fp32 points of up to 3 dimensions
+    (Euclidean, k <= 32): ``"scan"`` (default) looks at every row of the
+    example, ``"binned"`` orders the rows along a space-filling curve first and
+    looks only at rows near the query.  Same edges either way; ``"binned"``
+    wins on large examples (10^5 rows and more).  Process-wide; the
+    environment variable ``PCA_KNN_STRATEGY`` sets the initial value.  No
+    counterpart in the reference."""
+    _torch.ops.pytorch_cluster_amd.set_knn_strategy(name)
+
+
+def get_knn_strategy() -> str:
+    return _torch.ops.pytorch_cluster_amd.get_knn_strategy()
+
+
 __all__ = ["knn", "knn_graph", "radius", "radius_graph", "nearest", "fps",
-           "__version__"]
+           "set_knn_strategy", "get_knn_strategy", "__version__"]

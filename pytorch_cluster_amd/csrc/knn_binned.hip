@@ -541,6 +541,7 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
         }
       }
     }
+    drain();
   }
 
   if (valid)

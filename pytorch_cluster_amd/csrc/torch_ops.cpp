@@ -17,7 +17,11 @@
 #include <hip/hip_version.h>
 #include <torch/library.h>
 
+#include <atomic>
+#include <cstdlib>
+#include <cstring>
 #include <optional>
+#include <string>
 
 #include "../../include/pca_neighbors.h"
 
@@ -121,6 +125,26 @@ int edge_flags(bool drop_self, bool x_first) {
          (x_first ? PCA_EDGES_X_FIRST : 0);
 }
 
+// How a low-dimensional Euclidean kNN search goes about it: "scan" looks at
+// every row of the segment (pca_knn), "binned" at the rows near the query
+// (pca_knn_binned; fp32, up to 3 dimensions, k <= 32 - anything else is
+// scanned).  Same edges either way.  Process-wide; starts from the environment
+// variable PCA_KNN_STRATEGY.
+std::atomic<int> g_knn_binned{[] {
+  const char *e = std::getenv("PCA_KNN_STRATEGY");
+  return (e != nullptr && std::strcmp(e, "binned") == 0) ? 1 : 0;
+}()};
+
+void set_knn_strategy(std::string name) {
+  TORCH_CHECK(name == "scan" || name == "binned",
+              "knn strategy is 'scan' or 'binned', got '", name, "'");
+  g_knn_binned.store(name == "binned" ? 1 : 0);
+}
+
+std::string get_knn_strategy() {
+  return g_knn_binned.load() ? "binned" : "scan";
+}
+
 at::Tensor knn_search(at::Tensor x, at::Tensor y,
                       std::optional<at::Tensor> ptr_x,
                       std::optional<at::Tensor> ptr_y, int64_t k, bool cosine,
@@ -145,7 +169,11 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
     return at::empty({2, 0}, long_opts);
 
   const int dtype = dtype_code(x);
-  const size_t ws_bytes = pca_knn_workspace_bytes(n, m, d, seg.count, k, dtype);
+  const bool binned = g_knn_binned.load() != 0 && dtype == PCA_F32 &&
+                      !cosine && d <= 3 && k <= 32;
+  const size_t ws_bytes =
+      binned ? pca_knn_binned_workspace_bytes(n, m, d, seg.count, k)
+             : pca_knn_workspace_bytes(n, m, d, seg.count, k, dtype);
   TORCH_CHECK(ws_bytes > 0, "problem size not supported");
   auto workspace =
       at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
@@ -153,6 +181,14 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
   auto num_edges = at::empty({1}, long_opts);
 
   hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
+  if (binned) {
+    check_status(pca_knn_binned(x.data_ptr(), y.data_ptr(), seg.ptr_x,
+                                seg.ptr_y, n, m, d, seg.count, k, flags,
+                                edges.data_ptr<int64_t>(),
+                                num_edges.data_ptr<int64_t>(), nullptr,
+                                workspace.data_ptr(), ws_bytes, stream));
+    return finish(edges, num_edges);
+  }
   check_status(pca_knn(x.data_ptr(), y.data_ptr(), seg.ptr_x, seg.ptr_y, n, m,
                        d, seg.count, k, cosine ? 1 : 0, dtype, flags,
                        edges.data_ptr<int64_t>(),
@@ -373,4 +409,6 @@ TORCH_LIBRARY(pytorch_cluster_amd, m) {
         "float r, int max_num_neighbors, bool ignore_same_index, "
         "bool x_first) -> Tensor",
         &radius_edges);
+  m.def("set_knn_strategy(str name) -> ()", &set_knn_strategy);
+  m.def("get_knn_strategy() -> str", &get_knn_strategy);
 }

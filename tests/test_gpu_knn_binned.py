@@ -157,3 +157,46 @@ def test_unsupported_shapes_are_refused():
     x = torch.rand(100, 3, device=DEV)
     with pytest.raises(RuntimeError, match="binned search"):
         capi.knn_edges(x, x, None, None, 33, binned=True)
+
+
+def test_strategy_switch_of_the_entry_points():
+    """`set_knn_strategy("binned")` sends knn / knn_graph of low-dimensional
+    fp32 points through the binned search (same edges), leaves everything
+    else on the scanning kernels, and can be switched back."""
+    import pytorch_cluster_amd as pca
+    g = torch.Generator().manual_seed(5)
+    x = torch.rand(6000, 3, generator=g).to(DEV)
+    y = torch.rand(900, 3, generator=g).to(DEV)
+    bx = torch.arange(3).repeat_interleave(2000).to(DEV)
+    by = torch.arange(3).repeat_interleave(300).to(DEV)
+    hi = torch.rand(500, 16, generator=g).to(DEV)
+    assert pca.get_knn_strategy() == "scan"
+    want = (pca.knn(x, y, 7, bx, by), pca.knn_graph(x, 6, bx, loop=False),
+            pca.knn_graph(x, 6, bx, loop=True, flow="target_to_source"),
+            pca.knn(hi, hi, 4), pca.knn(x, y, 5, bx, by, cosine=True))
+    try:
+        pca.set_knn_strategy("binned")
+        assert pca.get_knn_strategy() == "binned"
+        got = (pca.knn(x, y, 7, bx, by), pca.knn_graph(x, 6, bx, loop=False),
+               pca.knn_graph(x, 6, bx, loop=True, flow="target_to_source"),
+               pca.knn(hi, hi, 4), pca.knn(x, y, 5, bx, by, cosine=True))
+        jit = torch.jit.script(pca.knn)
+        assert torch.equal(jit(x, y, 7, bx, by), want[0])
+    finally:
+        pca.set_knn_strategy("scan")
+    for a, b in zip(want, got):
+        assert torch.equal(a, b)
+    with pytest.raises(RuntimeError, match="scan.*binned"):
+        pca.set_knn_strategy("tree")
+    assert pca.get_knn_strategy() == "scan"
+
+
+def test_many_small_segments(oracle):
+    rng = np.random.default_rng(11)
+    sizes_x = rng.integers(0, 70, 300)
+    sizes_y = rng.integers(0, 20, 300)
+    ptr_x = np.concatenate([[0], np.cumsum(sizes_x)]).astype(np.int64)
+    ptr_y = np.concatenate([[0], np.cumsum(sizes_y)]).astype(np.int64)
+    x = rng.random((ptr_x[-1], 3)).astype(np.float32)
+    y = rng.random((ptr_y[-1], 3)).astype(np.float32)
+    check(oracle, x, y, ptr_x, ptr_y, 6)
