@@ -180,6 +180,35 @@ def other_configs(torch, pca, testing, dev):
         report["fps %dx%d ratio 0.25" % (clouds, points)] = {
             "ms": ms, "samples": int(out.numel()),
             "us_per_sample_step": ms * 1e3 / (points // 4)}
+    # the headline workload and one large cloud through the binned search
+    # (rows ordered along a space-filling curve, exact pruning by tile boxes):
+    # same edges as the scan; `search_ms` covers binning and search
+    lidar = testing.lidar_scans(0)
+    x, y = lidar["x"].to(dev), lidar["y"].to(dev)
+    bx, by = lidar["batch_x"].to(dev), lidar["batch_y"].to(dev)
+    big = torch.rand(1000000, 3, generator=torch.Generator().manual_seed(1))
+    big = big.to(dev)
+    cases = (("configs[4] ragged LiDAR-like knn k=16",
+              lambda: pca.knn(x, y, 16, bx, by, batch_size=8), y.shape[0]),
+             ("knn 1000000 uniform points onto themselves k=16",
+              lambda: pca.knn(big, big, 16), big.shape[0]))
+    for name, fn, queries in cases:
+        for strategy in ("scan", "binned"):
+            pca.set_knn_strategy(strategy)
+            try:
+                ms, out = median_ms(fn, 5)
+                start, stop = events.create(), events.create()
+                capi.pca_time_next_search(start, stop)
+                fn()
+                torch.cuda.synchronize()
+                search_ms = events.elapsed_ms(start, stop)
+                events.destroy(start)
+                events.destroy(stop)
+            finally:
+                pca.set_knn_strategy("scan")
+            report["%s, strategy %s" % (name, strategy)] = {
+                "ms": ms, "queries_per_s": queries / ms * 1e3,
+                "search_ms": search_ms, "edges": int(out.shape[1])}
     return report
 
 
