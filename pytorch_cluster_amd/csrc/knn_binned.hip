@@ -42,6 +42,7 @@
 
 #include <climits>
 #include <cstring>
+#include <type_traits>
 
 #include <rocprim/device/device_radix_sort.hpp>
 
@@ -308,8 +309,7 @@ __device__ __forceinline__ int wave_lower_bound(
 template <int K>
 __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
   // parked rows: distance and row number, [slot][thread]
-  __shared__ float queue_d[kBinQueueCap][kBlock];
-  __shared__ uint32_t queue_id[kBinQueueCap][kBlock];
+  __shared__ float queue_d[2 * kBinQueueCap][kBlock];
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -365,16 +365,20 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
   // farther away than that holds no neighbour of this lane's query.
   float admit = searching ? kKnnSentinel : -__builtin_inff();
   float kth = searching ? kKnnSentinel : -1.0f;
-  int parked = 0;
+  // byte offset in the queue at which the lane's next row goes
+  const int park_first = tid * (int)sizeof(float);
+  int park_at = park_first;
 
   auto drain = [&]() {
     for (;;) {
-      const bool has = parked > 0;
+      const bool has = park_at > park_first;
       if (!__any(has))
         break;
-      parked -= has ? 1 : 0;
-      const float d = queue_d[has ? parked : 0][tid];
-      const uint32_t id = queue_id[has ? parked : 0][tid];
+      park_at -= has ? kBlock * (int)sizeof(float) : 0;
+      const float *slot = reinterpret_cast<const float *>(
+          reinterpret_cast<const char *>(&queue_d[0][0]) + park_at);
+      const float d = slot[0];
+      const uint32_t id = __float_as_uint(slot[kBinQueueCap * kBlock]);
       // (parked under an older bound: the keys sort it out)
       const double key = (has && d < admit) ? make_key(d, id) : empty_key();
       sorted_insert<K>(best, key);
@@ -387,12 +391,12 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
   };
 
   // rows of one tile against every lane's query, four rows per step (the
-  // copy of the rows is padded, so a step may read past the tile's rows)
-  auto scan_tile = [&](int tile) {
-    const int j0 = x_begin + tile * kBinTile;
-    const int rows = min(kBinTile, x_end - j0);
-    const float4 *__restrict__ src = p.rows + j0;
-    for (int r = 0; r < rows; r += 4) {
+  // copy of the rows is padded, so a step may read past the tile's rows;
+  // FULL: the tile has all its 32 rows, no step needs a bound)
+  auto scan_rows = [&](const float4 *__restrict__ src, int rows,
+                       auto full) {
+    constexpr bool FULL = decltype(full)::value;
+    for (int r = 0; r < (FULL ? kBinTile : rows); r += 4) {
       float4 row[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u)
@@ -405,16 +409,29 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
         dd = __builtin_fmaf(d1, d1, dd);
         const float d2 = row[u].z - yq[2];
         dd = __builtin_fmaf(d2, d2, dd);
-        const bool hit = dd < admit && r + u < rows;
+        const bool hit = dd < admit && (FULL || r + u < rows);
         if (hit) {
-          queue_d[parked][tid] = dd;
-          queue_id[parked][tid] = __float_as_uint(row[u].w);
-          ++parked;
+          // (one address for both queues: the row numbers sit a fixed
+          // distance behind the distances)
+          float *slot = reinterpret_cast<float *>(
+              reinterpret_cast<char *>(&queue_d[0][0]) + park_at);
+          slot[0] = dd;
+          slot[kBinQueueCap * kBlock] = row[u].w;
+          park_at += kBlock * (int)sizeof(float);
         }
       }
-      if (__any(parked > kBinQueueCap - 4))
+      if (__any(park_at > park_first + (kBinQueueCap - 4) * kBlock *
+                                          (int)sizeof(float)))
         drain();
     }
+  };
+  auto scan_tile = [&](int tile) {
+    const int j0 = x_begin + tile * kBinTile;
+    const int rows = min(kBinTile, x_end - j0);
+    if (rows == kBinTile)
+      scan_rows(p.rows + j0, rows, std::true_type{});
+    else
+      scan_rows(p.rows + j0, rows, std::false_type{});
   };
 
   // Squared distance between two boxes (a query is a box of one point), with
@@ -535,7 +552,7 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
             continue;
           scan_tile(group * kBinGroup + t_lane);
         }
-        if (__any(parked > 0)) {
+        if (__any(park_at > park_first)) {
           drain();
           reach = wave_reach();
         }
