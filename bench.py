@@ -194,7 +194,7 @@ def other_configs(torch, pca, testing, dev):
               lambda: pca.knn(big, big, 16), big.shape[0]))
     for name, fn, queries in cases:
         for strategy in ("scan", "binned"):
-            pca.set_knn_strategy(strategy)
+            pca.set_search_strategy(strategy)
             try:
                 ms, out = median_ms(fn, 5)
                 start, stop = events.create(), events.create()
@@ -205,7 +205,7 @@ def other_configs(torch, pca, testing, dev):
                 events.destroy(start)
                 events.destroy(stop)
             finally:
-                pca.set_knn_strategy("scan")
+                pca.set_search_strategy("scan")
             report["%s, strategy %s" % (name, strategy)] = {
                 "ms": ms, "queries_per_s": queries / ms * 1e3,
                 "search_ms": search_ms, "edges": int(out.shape[1])}

@@ -186,6 +186,26 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
                int64_t *edges, int64_t *num_edges, void *workspace,
                size_t workspace_bytes, void *stream);
 
+/*
+ * pca_radius for fp32 points of up to 3 dimensions and at most 32 neighbours
+ * per query (pca_radius_slots; PCA_ERR_UNSUPPORTED otherwise) over the
+ * spatially binned rows of pca_knn_binned: a query scans only the tiles whose
+ * box is closer than r, and of the rows found keeps the max_num_neighbors
+ * with the smallest row numbers.  Stands under the same operator as
+ * pca_radius (csrc/radius.cpp:22-39 -> csrc/cuda/radius_cuda.cu:44-96) and
+ * returns the same edges in the same order.  Arguments as for pca_radius.
+ */
+size_t pca_radius_binned_workspace_bytes(int64_t n, int64_t m, int64_t d,
+                                         int64_t num_segments,
+                                         int64_t max_num_neighbors);
+
+int pca_radius_binned(const void *x, const void *y, const int64_t *ptr_x,
+                      const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+                      int64_t num_segments, double r,
+                      int64_t max_num_neighbors, int ignore_same_index,
+                      int edge_flags, int64_t *edges, int64_t *num_edges,
+                      void *workspace, size_t workspace_bytes, void *stream);
+
 /* -------------------------------------------------------------- nearest -- */
 
 /*

@@ -16,20 +16,21 @@ import torch as _torch
 __version__ = "0.1.0"
 
 
-def set_knn_strategy(name: str) -> None:
-    """How ``knn`` / ``knn_graph`` search fp32 points of up to 3 dimensions
-    (Euclidean, k <= 32): ``"scan"`` (default) looks at every row of the
+def set_search_strategy(name: str) -> None:
+    """How ``knn`` / ``knn_graph`` (Euclidean, k <= 32) and ``radius`` /
+    ``radius_graph`` (at most 32 neighbours per query) search fp32 points of
+    up to 3 dimensions: ``"scan"`` (default) looks at every row of the
     example, ``"binned"`` orders the rows along a space-filling curve first and
     looks only at rows near the query.  Same edges either way; ``"binned"``
     wins on large examples (10^5 rows and more).  Process-wide; the
-    environment variable ``PCA_KNN_STRATEGY`` sets the initial value.  No
+    environment variable ``PCA_SEARCH_STRATEGY`` sets the initial value.  No
     counterpart in the reference."""
-    _torch.ops.pytorch_cluster_amd.set_knn_strategy(name)
+    _torch.ops.pytorch_cluster_amd.set_search_strategy(name)
 
 
-def get_knn_strategy() -> str:
-    return _torch.ops.pytorch_cluster_amd.get_knn_strategy()
+def get_search_strategy() -> str:
+    return _torch.ops.pytorch_cluster_amd.get_search_strategy()
 
 
 __all__ = ["knn", "knn_graph", "radius", "radius_graph", "nearest", "fps",
-           "set_knn_strategy", "get_knn_strategy", "__version__"]
+           "set_search_strategy", "get_search_strategy", "__version__"]

@@ -53,6 +53,12 @@ C_ABI = {
                    [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                     ctypes.c_double, _i64, ctypes.c_int, ctypes.c_int,
                     ctypes.c_int, _vp, _vp, _vp, ctypes.c_size_t, _vp]),
+    "pca_radius_binned_workspace_bytes": (ctypes.c_size_t,
+                                          [_i64, _i64, _i64, _i64, _i64]),
+    "pca_radius_binned": (ctypes.c_int,
+                          [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
+                           ctypes.c_double, _i64, ctypes.c_int, ctypes.c_int,
+                           _vp, _vp, _vp, ctypes.c_size_t, _vp]),
     "pca_nearest_workspace_bytes": (ctypes.c_size_t,
                                     [_i64, _i64, _i64, _i64, ctypes.c_int]),
     "pca_nearest": (ctypes.c_int,

@@ -111,15 +111,20 @@ def knn_edges(x, y, ptr_x=None, ptr_y=None, k: int = 1, cosine: bool = False,
 
 def radius_launch(x, y, ptr_x, ptr_y, r: float, max_num_neighbors: int,
                   ignore_same_index: bool = False, stream=None,
-                  x_first: bool = False):
+                  x_first: bool = False, binned: bool = False):
     assert x.is_cuda and y.is_cuda and x.is_contiguous() and y.is_contiguous()
     assert x.dtype == y.dtype and x.dtype in _DTYPE_CODE
     dtype = _DTYPE_CODE[x.dtype]
     n, d = x.shape
     m = y.shape[0]
     ptr_x, ptr_y, nseg = _segments(ptr_x, ptr_y)
-    ws_bytes = capi.pca_radius_workspace_bytes(n, m, d, nseg,
-                                               max_num_neighbors, dtype)
+    if binned:
+        assert dtype == 0
+        ws_bytes = capi.pca_radius_binned_workspace_bytes(
+            n, m, d, nseg, max_num_neighbors)
+    else:
+        ws_bytes = capi.pca_radius_workspace_bytes(n, m, d, nseg,
+                                                   max_num_neighbors, dtype)
     if ws_bytes == 0:
         ws_bytes = 256
     slots = capi.pca_radius_slots(n, max_num_neighbors)
@@ -127,6 +132,13 @@ def radius_launch(x, y, ptr_x, ptr_y, r: float, max_num_neighbors: int,
     edges = torch.empty(max(2 * m * slots, 1), dtype=torch.long,
                         device=x.device)
     num_edges = torch.empty(1, dtype=torch.long, device=x.device)
+    if binned:
+        _check(capi.pca_radius_binned(
+            _dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x), _dev_ptr(ptr_y), n, m,
+            d, nseg, float(r), max_num_neighbors, int(ignore_same_index),
+            _edge_flags(False, x_first), _dev_ptr(edges), _dev_ptr(num_edges),
+            _dev_ptr(ws), ws_bytes, _stream_handle(stream, x.device)))
+        return edges, num_edges, ws
     _check(capi.pca_radius(_dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x),
                            _dev_ptr(ptr_y), n, m, d, nseg, float(r),
                            max_num_neighbors, int(ignore_same_index), dtype,
@@ -138,10 +150,12 @@ def radius_launch(x, y, ptr_x, ptr_y, r: float, max_num_neighbors: int,
 
 def radius_edges(x, y, ptr_x=None, ptr_y=None, r: float = 1.0,
                  max_num_neighbors: int = 32, ignore_same_index: bool = False,
-                 stream=None, x_first: bool = False) -> torch.Tensor:
+                 stream=None, x_first: bool = False,
+                 binned: bool = False) -> torch.Tensor:
     edges, num_edges, _ws = radius_launch(x, y, ptr_x, ptr_y, r,
                                           max_num_neighbors,
-                                          ignore_same_index, stream, x_first)
+                                          ignore_same_index, stream, x_first,
+                                          binned)
     e = int(num_edges.item())
     return edges[:2 * e].view(2, e)
 

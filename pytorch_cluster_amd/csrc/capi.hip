@@ -132,6 +132,15 @@ size_t binned_workspace(int64_t n, int64_t m, int64_t num_segments,
          pca::compact_workspace_bytes((int)m);
 }
 
+size_t radius_binned_workspace(int64_t n, int64_t m, int64_t num_segments,
+                               int64_t slots) {
+  return align256(pca::knn_binned_scratch_bytes((int)n, (int)m,
+                                                (int)num_segments)) +
+         align256(sizeof(int) * (size_t)m * (size_t)slots) +
+         align256(sizeof(int) * (size_t)m) +
+         pca::compact_workspace_bytes((int)m);
+}
+
 bool dtype_ok(int dtype) {
   return dtype == PCA_F32 || dtype == PCA_F64 || dtype == PCA_F16 ||
          dtype == PCA_BF16;
@@ -564,6 +573,96 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
                                                  work_start, bound, dense,
                                                  stream),
                       "radius_any_kernel");
+  timer.done();
+  if (rc != PCA_OK)
+    return rc;
+  return check_launch(
+      pca::launch_compact(dense, (int)m, edges, num_edges, nullptr,
+                          compact_ws, stream, false,
+                          (edge_flags & PCA_EDGES_X_FIRST) != 0),
+      "compaction kernels");
+}
+
+size_t pca_radius_binned_workspace_bytes(int64_t n, int64_t m, int64_t d,
+                                         int64_t num_segments,
+                                         int64_t max_num_neighbors) {
+  if (num_segments < 1)
+    num_segments = 1;
+  const int64_t slots = pca_radius_slots(n, max_num_neighbors);
+  if (!sizes_ok(n, m, d, num_segments) || n == 0 || m == 0 ||
+      !pca::radius_binned_supported((int)d, (int)slots))
+    return 0;
+  return radius_binned_workspace(n, m, num_segments, slots);
+}
+
+int pca_radius_binned(const void *x, const void *y, const int64_t *ptr_x,
+                      const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+                      int64_t num_segments, double r,
+                      int64_t max_num_neighbors, int ignore_same_index,
+                      int edge_flags, int64_t *edges, int64_t *num_edges,
+                      void *workspace, size_t workspace_bytes, void *stream_) {
+  g_last_error[0] = 0;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  SearchTimer timer(stream);
+  if ((ptr_x == nullptr) != (ptr_y == nullptr))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "ptr_x and ptr_y must both be given or both be NULL");
+  if (ptr_x == nullptr)
+    num_segments = 1;
+  if (!sizes_ok(n, m, d, num_segments))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "bad sizes n=%lld m=%lld d=%lld num_segments=%lld",
+                (long long)n, (long long)m, (long long)d,
+                (long long)num_segments);
+  if (max_num_neighbors < 1)
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "max_num_neighbors must be >= 1, got %lld",
+                (long long)max_num_neighbors);
+  if (!edge_flags_ok(edge_flags))
+    return fail(PCA_ERR_INVALID_ARGUMENT, "unknown edge flags %d", edge_flags);
+  if (edge_flags & PCA_EDGES_DROP_SELF)
+    ignore_same_index = 1;
+  if (num_edges == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "num_edges is NULL");
+  if (n == 0 || m == 0) {
+    hipLaunchKernelGGL(set_i64_kernel, dim3(1), dim3(1), 0, stream, num_edges,
+                       (int64_t)0);
+    return check_launch(hipGetLastError(), "set_i64_kernel");
+  }
+  const int64_t slots = pca_radius_slots(n, max_num_neighbors);
+  if (!pca::radius_binned_supported((int)d, (int)slots))
+    return fail(PCA_ERR_UNSUPPORTED,
+                "binned search: fp32 points of up to 3 dimensions and at most "
+                "32 neighbours per query, got d=%lld slots=%lld",
+                (long long)d, (long long)slots);
+  if (x == nullptr || y == nullptr || edges == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "x, y or edges is NULL");
+  const size_t need = radius_binned_workspace(n, m, num_segments, slots);
+  if (workspace == nullptr || ((uintptr_t)workspace & 255) != 0 ||
+      workspace_bytes < need)
+    return fail(PCA_ERR_WORKSPACE, "workspace needs %zu bytes, 256-aligned",
+                need);
+
+  Carver carve(workspace);
+  void *scratch = carve.take<char>(pca::knn_binned_scratch_bytes(
+      (int)n, (int)m, (int)num_segments));
+  pca::DenseResult dense;
+  dense.idx = carve.take<int>((size_t)m * (size_t)slots);
+  dense.dist = nullptr;
+  dense.count = carve.take<int>((size_t)m);
+  dense.slots = (int)slots;
+  void *compact_ws = carve.take<char>(pca::compact_workspace_bytes((int)m));
+
+  // r * r in double, narrowed to the element type at the launch
+  // (csrc/cuda/radius_cuda.cu:90)
+  const float r2 = (float)(r * r);
+  pca::SearchInput in{x,      y,      ptr_x,  ptr_y,
+                      (int)n, (int)m, (int)d, (int)num_segments};
+  timer.begin();
+  int rc = check_launch(pca::launch_radius_binned(in, r2,
+                                                  ignore_same_index != 0,
+                                                  scratch, dense, stream),
+                        "binned search");
   timer.done();
   if (rc != PCA_OK)
     return rc;

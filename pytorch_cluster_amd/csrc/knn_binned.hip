@@ -565,6 +565,192 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
     write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
 }
 
+// The radius search over the same bins (reference: radius_kernel,
+// csrc/cuda/radius_cuda.cu:9-42): every row with a squared distance strictly
+// below r2, at most `slots` of them - the ones with the smallest row numbers,
+// in ascending order.  The radius is known from the start, so there are no
+// seed tiles: boxes at r2 or farther from every query are skipped, rows that
+// qualify are parked by number, and the lists keep the `slots` smallest
+// numbers (as doubles; a full list admits only smaller numbers).
+template <int K>
+__global__ __launch_bounds__(kBlock) void radius_binned_kernel(
+    BinnedParams p, float r2, int ignore_same_index) {
+  __shared__ uint32_t queue[kBinQueueCap][kBlock];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int task = blockIdx.x * (kBlock / kWave) +
+                   __builtin_amdgcn_readfirstlane(tid / kWave);
+  if (task >= p.wave_start[p.num_segments])
+    return; // (whole waves leave; no barrier below)
+  const int seg = find_segment(p.wave_start, p.num_segments, task);
+  const int x_begin = p.ptr_x ? (int)p.ptr_x[seg] : 0;
+  const int x_end = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
+  const int y_begin = p.ptr_y ? (int)p.ptr_y[seg] : 0;
+  const int y_end = p.ptr_y ? (int)p.ptr_y[seg + 1] : p.m;
+  const int jq = y_begin + (task - p.wave_start[seg]) * kWave + lane;
+  const bool valid = jq < y_end;
+  const int q = valid ? (int)p.perm_y[jq] : 0;
+  const int slots = p.k;
+  const int d_in = p.d;
+
+  float yq[3];
+#pragma unroll
+  for (int c = 0; c < 3; ++c)
+    yq[c] = (valid && c < d_in) ? p.y[(size_t)q * d_in + c] : 0.0f;
+  // (a coordinate that is not finite: no distance below r2)
+  const bool searching = valid && __builtin_fabsf(yq[0]) < __builtin_inff() &&
+                         __builtin_fabsf(yq[1]) < __builtin_inff() &&
+                         __builtin_fabsf(yq[2]) < __builtin_inff();
+  float q_lo[3], q_hi[3];
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    float lo = searching ? yq[c] : __builtin_inff();
+    float hi = searching ? yq[c] : -__builtin_inff();
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1) {
+      lo = __builtin_fminf(lo, __shfl_xor(lo, sh));
+      hi = __builtin_fmaxf(hi, __shfl_xor(hi, sh));
+    }
+    q_lo[c] = lo;
+    q_hi[c] = hi;
+  }
+
+  double best[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j)
+    best[j] = (j < K - slots) ? -__builtin_inf() : __builtin_inf();
+  // rows with a number below `below` are parked: all while the list has
+  // room, those under its largest number afterwards; none for a lane that
+  // does not search
+  uint32_t below = searching ? 0xffffffffu : 0u;
+  const uint32_t self = ignore_same_index ? (uint32_t)q : 0xffffffffu;
+  // a lane without a query never passes d < limit
+  const float limit = searching ? r2 : -__builtin_inff();
+  int parked = 0;
+
+  auto drain = [&]() {
+    for (;;) {
+      const bool has = parked > 0;
+      if (!__any(has))
+        break;
+      parked -= has ? 1 : 0;
+      const uint32_t id = queue[has ? parked : 0][tid];
+      const double key = (has && id < below) ? (double)id : __builtin_inf();
+      sorted_insert<K>(best, key);
+      if (searching && best[K - 1] < __builtin_inf())
+        below = (uint32_t)best[K - 1];
+    }
+  };
+
+  auto scan_tile = [&](int tile) {
+    const int j0 = x_begin + tile * kBinTile;
+    const int rows = min(kBinTile, x_end - j0);
+    const float4 *__restrict__ src = p.rows + j0;
+    for (int r = 0; r < rows; r += 4) {
+      float4 row[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        row[u] = src[r + u]; // (uniform addresses; the copy is padded)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float d0 = row[u].x - yq[0];
+        float dd = d0 * d0;
+        const float d1 = row[u].y - yq[1];
+        dd = __builtin_fmaf(d1, d1, dd);
+        const float d2 = row[u].z - yq[2];
+        dd = __builtin_fmaf(d2, d2, dd);
+        const uint32_t id = __float_as_uint(row[u].w);
+        const bool hit = dd < limit && id < below && id != self &&
+                         r + u < rows;
+        if (hit) {
+          queue[parked][tid] = id;
+          ++parked;
+        }
+      }
+      if (__any(parked > kBinQueueCap - 4))
+        drain();
+    }
+  };
+
+  auto box_gap2 = [](const float (&alo)[3], const float (&ahi)[3],
+                     const float (&blo)[3], const float (&bhi)[3]) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      const float gap = __builtin_fmaxf(
+          __builtin_fmaxf(alo[c] - bhi[c], blo[c] - ahi[c]), 0.0f);
+      acc = c == 0 ? gap * gap : __builtin_fmaf(gap, gap, acc);
+    }
+    return acc;
+  };
+  // is the box of lane `src` closer than the radius to some lane's query?
+  // (A NaN - from an infinite or empty box - never rules a box out.)
+  auto reachable = [&](const Box &held, int src) {
+    float lo[3], hi[3];
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      lo[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+          (int)__float_as_uint(held.lo[c]), src));
+      hi[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+          (int)__float_as_uint(held.hi[c]), src));
+    }
+    return __any(searching && !(box_gap2(lo, hi, yq, yq) >= r2));
+  };
+
+  const int tile0 = p.tile_start[seg];
+  const int num_tiles = p.tile_start[seg + 1] - tile0;
+  const int group0 = p.group_start[seg];
+  const int num_groups = (num_tiles + kBinGroup - 1) / kBinGroup;
+  if (__any(searching)) {
+    for (int g_base = 0; g_base < num_groups; g_base += kWave) {
+      const int g_mine = g_base + lane;
+      Box g_box = {};
+      if (g_mine < num_groups)
+        g_box = p.group_box[group0 + g_mine];
+      uint64_t g_todo =
+          __ballot(g_mine < num_groups &&
+                   !(box_gap2(g_box.lo, g_box.hi, q_lo, q_hi) >= r2));
+      while (g_todo != 0) {
+        const int g_lane = (int)__builtin_ctzll(g_todo);
+        g_todo &= g_todo - 1;
+        if (!reachable(g_box, g_lane))
+          continue;
+        const int group = g_base + g_lane;
+        const int t_mine = group * kBinGroup + lane;
+        Box t_box = {};
+        if (t_mine < num_tiles)
+          t_box = p.box[tile0 + t_mine];
+        uint64_t t_todo =
+            __ballot(t_mine < num_tiles &&
+                     !(box_gap2(t_box.lo, t_box.hi, q_lo, q_hi) >= r2));
+        while (t_todo != 0) {
+          const int t_lane = (int)__builtin_ctzll(t_todo);
+          t_todo &= t_todo - 1;
+          if (reachable(t_box, t_lane))
+            scan_tile(group * kBinGroup + t_lane);
+        }
+        if (__any(parked > 0))
+          drain();
+      }
+    }
+  }
+
+  if (valid) {
+    const size_t row = (size_t)q * slots;
+    int found = 0;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      const int e = j - (K - slots);
+      if (e >= 0 && best[j] < __builtin_inf()) {
+        p.out_idx[row + e] = (int)best[j];
+        ++found;
+      }
+    }
+    p.out_count[q] = found;
+  }
+}
+
 struct BinnedLayout {
   size_t seg_box, keys_a, keys_x, keys_y, vals_a, perm_x, perm_y, rows, box,
       group_box, tile_start, group_start, wave_start, sort_temp;
@@ -630,19 +816,17 @@ BinnedLayout binned_layout(int n, int m, int num_segments) {
   return w;
 }
 
-} // namespace
+// Everything a binned search reads, as prepare_bins leaves it in the scratch.
+struct Bins {
+  const int *tile_start, *group_start, *wave_start;
+  const uint32_t *keys_x, *keys_y, *perm_y;
+  const float4 *rows;
+  const Box *box, *group_box;
+};
 
-bool knn_binned_supported(int d, int k, bool cosine) {
-  return !cosine && d >= 1 && d <= 3 && k >= 1 && k <= 32;
-}
-
-size_t knn_binned_scratch_bytes(int n, int m, int num_segments) {
-  return binned_layout(n, m, num_segments).total();
-}
-
-hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
-                             const DenseResult &out, hipEvent_t time_start,
-                             hipEvent_t time_stop, hipStream_t stream) {
+// Orders rows and queries along the curve, copies the rows, builds the boxes.
+hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
+                        hipStream_t stream) {
   const BinnedLayout lay = binned_layout(in.n, in.m, in.num_segments);
   char *cursor = static_cast<char *>(scratch);
   auto take = [&cursor](size_t bytes) {
@@ -670,8 +854,6 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
   const float *y = static_cast<const float *>(in.y);
   const int nseg = in.num_segments;
 
-  if (time_start)
-    (void)hipEventRecord(time_start, stream);
   hipError_t err;
   if ((err = launch_plan(in.ptr_x, in.n, nseg, kBinTile, tile_start, stream)) !=
       hipSuccess)
@@ -726,28 +908,64 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
   if ((err = hipGetLastError()) != hipSuccess)
     return err;
 
-  BinnedParams p;
-  p.y = y;
+  bins.tile_start = tile_start;
+  bins.group_start = group_start;
+  bins.wave_start = wave_start;
+  bins.keys_x = keys_x;
+  bins.keys_y = keys_y;
+  bins.perm_y = perm_y;
+  bins.rows = rows;
+  bins.box = box;
+  bins.group_box = group_box;
+  return hipSuccess;
+}
+
+void fill_params(BinnedParams &p, const SearchInput &in, const Bins &bins,
+                 const DenseResult &out) {
+  p.y = static_cast<const float *>(in.y);
   p.ptr_x = in.ptr_x;
   p.ptr_y = in.ptr_y;
   p.n = in.n;
   p.m = in.m;
   p.d = in.d;
-  p.num_segments = nseg;
-  p.k = k;
-  p.tile_start = tile_start;
-  p.wave_start = wave_start;
-  p.keys_x = keys_x;
-  p.keys_y = keys_y;
-  p.perm_y = perm_y;
-  p.rows = rows;
-  p.box = box;
-  p.group_start = group_start;
-  p.group_box = group_box;
+  p.num_segments = in.num_segments;
+  p.tile_start = bins.tile_start;
+  p.wave_start = bins.wave_start;
+  p.keys_x = bins.keys_x;
+  p.keys_y = bins.keys_y;
+  p.perm_y = bins.perm_y;
+  p.rows = bins.rows;
+  p.box = bins.box;
+  p.group_start = bins.group_start;
+  p.group_box = bins.group_box;
   p.out_idx = out.idx;
   p.out_dist = out.dist;
   p.out_count = out.count;
-  const int waves = plan_upper_bound(in.m, nseg, kWave);
+}
+
+} // namespace
+
+bool knn_binned_supported(int d, int k, bool cosine) {
+  return !cosine && d >= 1 && d <= 3 && k >= 1 && k <= 32;
+}
+
+size_t knn_binned_scratch_bytes(int n, int m, int num_segments) {
+  return binned_layout(n, m, num_segments).total();
+}
+
+hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
+                             const DenseResult &out, hipEvent_t time_start,
+                             hipEvent_t time_stop, hipStream_t stream) {
+  if (time_start)
+    (void)hipEventRecord(time_start, stream);
+  Bins bins;
+  const hipError_t err = prepare_bins(in, scratch, bins, stream);
+  if (err != hipSuccess)
+    return err;
+  BinnedParams p;
+  fill_params(p, in, bins, out);
+  p.k = k;
+  const int waves = plan_upper_bound(in.m, in.num_segments, kWave);
   const int grid = (waves + kBlock / kWave - 1) / (kBlock / kWave);
   if (k <= 8)
     hipLaunchKernelGGL((knn_binned_kernel<8>), dim3(grid), dim3(kBlock), 0,
@@ -763,6 +981,38 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
                        stream, p);
   if (time_stop)
     (void)hipEventRecord(time_stop, stream);
+  return hipGetLastError();
+}
+
+bool radius_binned_supported(int d, int slots) {
+  return d >= 1 && d <= 3 && slots >= 1 && slots <= 32;
+}
+
+hipError_t launch_radius_binned(const SearchInput &in, float r2,
+                                bool ignore_same_index, void *scratch,
+                                const DenseResult &out, hipStream_t stream) {
+  Bins bins;
+  const hipError_t err = prepare_bins(in, scratch, bins, stream);
+  if (err != hipSuccess)
+    return err;
+  BinnedParams p;
+  fill_params(p, in, bins, out);
+  p.k = out.slots;
+  const int waves = plan_upper_bound(in.m, in.num_segments, kWave);
+  const int grid = (waves + kBlock / kWave - 1) / (kBlock / kWave);
+  const int same = ignore_same_index ? 1 : 0;
+  if (out.slots <= 8)
+    hipLaunchKernelGGL((radius_binned_kernel<8>), dim3(grid), dim3(kBlock), 0,
+                       stream, p, r2, same);
+  else if (out.slots <= 16)
+    hipLaunchKernelGGL((radius_binned_kernel<16>), dim3(grid), dim3(kBlock),
+                       0, stream, p, r2, same);
+  else if (out.slots <= 24)
+    hipLaunchKernelGGL((radius_binned_kernel<24>), dim3(grid), dim3(kBlock),
+                       0, stream, p, r2, same);
+  else
+    hipLaunchKernelGGL((radius_binned_kernel<32>), dim3(grid), dim3(kBlock),
+                       0, stream, p, r2, same);
   return hipGetLastError();
 }
 

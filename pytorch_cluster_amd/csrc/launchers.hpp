@@ -91,6 +91,13 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
                              const DenseResult &out, hipEvent_t time_start,
                              hipEvent_t time_stop, hipStream_t stream);
 
+// The radius search over the same bins: fp32 points of up to 3 dimensions,
+// up to 32 slots per query (out.slots; out.dist unused).
+bool radius_binned_supported(int d, int slots);
+hipError_t launch_radius_binned(const SearchInput &in, float r2,
+                                bool ignore_same_index, void *scratch,
+                                const DenseResult &out, hipStream_t stream);
+
 // --- knn_mfma*.hip ---------------------------------------------------------
 
 constexpr int kMfmaTileQueries = 128;

@@ -125,24 +125,25 @@ int edge_flags(bool drop_self, bool x_first) {
          (x_first ? PCA_EDGES_X_FIRST : 0);
 }
 
-// How a low-dimensional Euclidean kNN search goes about it: "scan" looks at
-// every row of the segment (pca_knn), "binned" at the rows near the query
-// (pca_knn_binned; fp32, up to 3 dimensions, k <= 32 - anything else is
-// scanned).  Same edges either way.  Process-wide; starts from the environment
-// variable PCA_KNN_STRATEGY.
-std::atomic<int> g_knn_binned{[] {
-  const char *e = std::getenv("PCA_KNN_STRATEGY");
+// How a search over fp32 points of up to 3 dimensions goes about it: "scan"
+// looks at every row of the segment (pca_knn, pca_radius), "binned" at the
+// rows near the query (pca_knn_binned: Euclidean, k <= 32; pca_radius_binned:
+// at most 32 neighbours per query - anything else is scanned).  Same edges
+// either way.  Process-wide; starts from the environment variable
+// PCA_SEARCH_STRATEGY.
+std::atomic<int> g_binned{[] {
+  const char *e = std::getenv("PCA_SEARCH_STRATEGY");
   return (e != nullptr && std::strcmp(e, "binned") == 0) ? 1 : 0;
 }()};
 
-void set_knn_strategy(std::string name) {
+void set_search_strategy(std::string name) {
   TORCH_CHECK(name == "scan" || name == "binned",
-              "knn strategy is 'scan' or 'binned', got '", name, "'");
-  g_knn_binned.store(name == "binned" ? 1 : 0);
+              "search strategy is 'scan' or 'binned', got '", name, "'");
+  g_binned.store(name == "binned" ? 1 : 0);
 }
 
-std::string get_knn_strategy() {
-  return g_knn_binned.load() ? "binned" : "scan";
+std::string get_search_strategy() {
+  return g_binned.load() ? "binned" : "scan";
 }
 
 at::Tensor knn_search(at::Tensor x, at::Tensor y,
@@ -169,8 +170,8 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
     return at::empty({2, 0}, long_opts);
 
   const int dtype = dtype_code(x);
-  const bool binned = g_knn_binned.load() != 0 && dtype == PCA_F32 &&
-                      !cosine && d <= 3 && k <= 32;
+  const bool binned = g_binned.load() != 0 && dtype == PCA_F32 && !cosine &&
+                      d <= 3 && k <= 32;
   const size_t ws_bytes =
       binned ? pca_knn_binned_workspace_bytes(n, m, d, seg.count, k)
              : pca_knn_workspace_bytes(n, m, d, seg.count, k, dtype);
@@ -240,16 +241,29 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
     return at::empty({2, 0}, long_opts);
 
   const int dtype = dtype_code(x);
-  const size_t ws_bytes = pca_radius_workspace_bytes(n, m, d, seg.count,
-                                                     max_num_neighbors, dtype);
+  const int64_t slots = pca_radius_slots(n, max_num_neighbors);
+  const bool binned =
+      g_binned.load() != 0 && dtype == PCA_F32 && d <= 3 && slots <= 32;
+  const size_t ws_bytes =
+      binned ? pca_radius_binned_workspace_bytes(n, m, d, seg.count,
+                                                 max_num_neighbors)
+             : pca_radius_workspace_bytes(n, m, d, seg.count,
+                                          max_num_neighbors, dtype);
   TORCH_CHECK(ws_bytes > 0, "problem size not supported");
   auto workspace =
       at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
-  const int64_t slots = pca_radius_slots(n, max_num_neighbors);
   auto edges = at::empty({2 * m * slots}, long_opts);
   auto num_edges = at::empty({1}, long_opts);
 
   hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
+  if (binned) {
+    check_status(pca_radius_binned(
+        x.data_ptr(), y.data_ptr(), seg.ptr_x, seg.ptr_y, n, m, d, seg.count,
+        r, max_num_neighbors, ignore_same_index ? 1 : 0, flags,
+        edges.data_ptr<int64_t>(), num_edges.data_ptr<int64_t>(),
+        workspace.data_ptr(), ws_bytes, stream));
+    return finish(edges, num_edges);
+  }
   check_status(pca_radius(x.data_ptr(), y.data_ptr(), seg.ptr_x, seg.ptr_y, n,
                           m, d, seg.count, r, max_num_neighbors,
                           ignore_same_index ? 1 : 0, dtype, flags,
@@ -409,6 +423,6 @@ TORCH_LIBRARY(pytorch_cluster_amd, m) {
         "float r, int max_num_neighbors, bool ignore_same_index, "
         "bool x_first) -> Tensor",
         &radius_edges);
-  m.def("set_knn_strategy(str name) -> ()", &set_knn_strategy);
-  m.def("get_knn_strategy() -> str", &get_knn_strategy);
+  m.def("set_search_strategy(str name) -> ()", &set_search_strategy);
+  m.def("get_search_strategy() -> str", &get_search_strategy);
 }

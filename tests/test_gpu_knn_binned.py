@@ -160,7 +160,7 @@ def test_unsupported_shapes_are_refused():
 
 
 def test_strategy_switch_of_the_entry_points():
-    """`set_knn_strategy("binned")` sends knn / knn_graph of low-dimensional
+    """`set_search_strategy("binned")` sends knn / knn_graph of low-dimensional
     fp32 points through the binned search (same edges), leaves everything
     else on the scanning kernels, and can be switched back."""
     import pytorch_cluster_amd as pca
@@ -170,25 +170,25 @@ def test_strategy_switch_of_the_entry_points():
     bx = torch.arange(3).repeat_interleave(2000).to(DEV)
     by = torch.arange(3).repeat_interleave(300).to(DEV)
     hi = torch.rand(500, 16, generator=g).to(DEV)
-    assert pca.get_knn_strategy() == "scan"
+    assert pca.get_search_strategy() == "scan"
     want = (pca.knn(x, y, 7, bx, by), pca.knn_graph(x, 6, bx, loop=False),
             pca.knn_graph(x, 6, bx, loop=True, flow="target_to_source"),
             pca.knn(hi, hi, 4), pca.knn(x, y, 5, bx, by, cosine=True))
     try:
-        pca.set_knn_strategy("binned")
-        assert pca.get_knn_strategy() == "binned"
+        pca.set_search_strategy("binned")
+        assert pca.get_search_strategy() == "binned"
         got = (pca.knn(x, y, 7, bx, by), pca.knn_graph(x, 6, bx, loop=False),
                pca.knn_graph(x, 6, bx, loop=True, flow="target_to_source"),
                pca.knn(hi, hi, 4), pca.knn(x, y, 5, bx, by, cosine=True))
         jit = torch.jit.script(pca.knn)
         assert torch.equal(jit(x, y, 7, bx, by), want[0])
     finally:
-        pca.set_knn_strategy("scan")
+        pca.set_search_strategy("scan")
     for a, b in zip(want, got):
         assert torch.equal(a, b)
     with pytest.raises(RuntimeError, match="scan.*binned"):
-        pca.set_knn_strategy("tree")
-    assert pca.get_knn_strategy() == "scan"
+        pca.set_search_strategy("tree")
+    assert pca.get_search_strategy() == "scan"
 
 
 def test_many_small_segments(oracle):
