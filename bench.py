@@ -188,10 +188,18 @@ def other_configs(torch, pca, testing, dev):
     bx, by = lidar["batch_x"].to(dev), lidar["batch_y"].to(dev)
     big = torch.rand(1000000, 3, generator=torch.Generator().manual_seed(1))
     big = big.to(dev)
+    c3 = testing.gaussian_mixture_batched(0)
+    x3, b3 = c3["x"].to(dev), c3["batch"].to(dev)
     cases = (("configs[4] ragged LiDAR-like knn k=16",
               lambda: pca.knn(x, y, 16, bx, by, batch_size=8), y.shape[0]),
              ("knn 1000000 uniform points onto themselves k=16",
-              lambda: pca.knn(big, big, 16), big.shape[0]))
+              lambda: pca.knn(big, big, 16), big.shape[0]),
+             ("configs[2] radius_graph 8x16384 r=0.05 max 32",
+              lambda: pca.radius_graph(x3, 0.05, b3, max_num_neighbors=32,
+                                       batch_size=8), x3.shape[0]),
+             ("radius 1000000 uniform points onto themselves r=0.01 max 32",
+              lambda: pca.radius(big, big, 0.01, max_num_neighbors=32),
+              big.shape[0]))
     for name, fn, queries in cases:
         for strategy in ("scan", "binned"):
             pca.set_search_strategy(strategy)

@@ -17,6 +17,7 @@
 #include <hip/hip_version.h>
 #include <torch/library.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cstdlib>
 #include <cstring>
@@ -129,21 +130,46 @@ int edge_flags(bool drop_self, bool x_first) {
 // looks at every row of the segment (pca_knn, pca_radius), "binned" at the
 // rows near the query (pca_knn_binned: Euclidean, k <= 32; pca_radius_binned:
 // at most 32 neighbours per query - anything else is scanned).  Same edges
-// either way.  Process-wide; starts from the environment variable
-// PCA_SEARCH_STRATEGY.
-std::atomic<int> g_binned{[] {
+// either way.  "auto" bins when the segments average kAutoBinRows rows or
+// more, where binning has paid off in measurements (the scan grows with the
+// square of the segment size).  Process-wide; starts from the environment
+// variable PCA_SEARCH_STRATEGY.
+enum Strategy { kScan = 0, kBinned = 1, kAuto = 2 };
+constexpr int64_t kAutoBinRows = 65536;
+
+int strategy_code(const std::string &name) {
+  if (name == "scan")
+    return kScan;
+  if (name == "binned")
+    return kBinned;
+  if (name == "auto")
+    return kAuto;
+  return -1;
+}
+
+std::atomic<int> g_strategy{[] {
   const char *e = std::getenv("PCA_SEARCH_STRATEGY");
-  return (e != nullptr && std::strcmp(e, "binned") == 0) ? 1 : 0;
+  const int code = e != nullptr ? strategy_code(e) : kScan;
+  return code < 0 ? (int)kScan : code;
 }()};
 
 void set_search_strategy(std::string name) {
-  TORCH_CHECK(name == "scan" || name == "binned",
-              "search strategy is 'scan' or 'binned', got '", name, "'");
-  g_binned.store(name == "binned" ? 1 : 0);
+  const int code = strategy_code(name);
+  TORCH_CHECK(code >= 0, "search strategy is 'scan', 'binned' or 'auto', got '",
+              name, "'");
+  g_strategy.store(code);
 }
 
 std::string get_search_strategy() {
-  return g_binned.load() ? "binned" : "scan";
+  const int code = g_strategy.load();
+  return code == kBinned ? "binned" : code == kAuto ? "auto" : "scan";
+}
+
+bool bins_wanted(int64_t n, int64_t num_segments) {
+  const int code = g_strategy.load();
+  return code == kBinned ||
+         (code == kAuto && n / std::max<int64_t>(num_segments, 1) >=
+                               kAutoBinRows);
 }
 
 at::Tensor knn_search(at::Tensor x, at::Tensor y,
@@ -170,8 +196,8 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
     return at::empty({2, 0}, long_opts);
 
   const int dtype = dtype_code(x);
-  const bool binned = g_binned.load() != 0 && dtype == PCA_F32 && !cosine &&
-                      d <= 3 && k <= 32;
+  const bool binned = bins_wanted(n, seg.count) && dtype == PCA_F32 &&
+                      !cosine && d <= 3 && k <= 32;
   const size_t ws_bytes =
       binned ? pca_knn_binned_workspace_bytes(n, m, d, seg.count, k)
              : pca_knn_workspace_bytes(n, m, d, seg.count, k, dtype);
@@ -242,8 +268,8 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
 
   const int dtype = dtype_code(x);
   const int64_t slots = pca_radius_slots(n, max_num_neighbors);
-  const bool binned =
-      g_binned.load() != 0 && dtype == PCA_F32 && d <= 3 && slots <= 32;
+  const bool binned = bins_wanted(n, seg.count) && dtype == PCA_F32 &&
+                      d <= 3 && slots <= 32;
   const size_t ws_bytes =
       binned ? pca_radius_binned_workspace_bytes(n, m, d, seg.count,
                                                  max_num_neighbors)

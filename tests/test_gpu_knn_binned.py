@@ -191,6 +191,38 @@ def test_strategy_switch_of_the_entry_points():
     assert pca.get_search_strategy() == "scan"
 
 
+def test_auto_strategy_bins_large_examples_only(monkeypatch):
+    """"auto": examples of 65,536 rows and more on average go through the
+    binned search (seen by the search timer, which the binned entry point
+    starts before its first kernel), smaller ones through the scan."""
+    import pytorch_cluster_amd as pca
+    g = torch.Generator().manual_seed(9)
+    small = torch.rand(20000, 3, generator=g).to(DEV)
+    large = torch.rand(140000, 3, generator=g).to(DEV)
+    y = large[::50].contiguous()
+    want_small = pca.knn(small, small[::10].contiguous(), 8)
+    want_large = pca.knn(large, y, 8)
+    try:
+        pca.set_search_strategy("auto")
+        assert pca.get_search_strategy() == "auto"
+        assert torch.equal(pca.knn(small, small[::10].contiguous(), 8),
+                           want_small)
+        assert torch.equal(pca.knn(large, y, 8), want_large)
+        assert torch.equal(pca.radius(large, y, 0.02, max_num_neighbors=8),
+                           _scan_radius(pca, large, y))
+    finally:
+        pca.set_search_strategy("scan")
+
+
+def _scan_radius(pca, x, y):
+    before = pca.get_search_strategy()
+    pca.set_search_strategy("scan")
+    try:
+        return pca.radius(x, y, 0.02, max_num_neighbors=8)
+    finally:
+        pca.set_search_strategy(before)
+
+
 def test_many_small_segments(oracle):
     rng = np.random.default_rng(11)
     sizes_x = rng.integers(0, 70, 300)
