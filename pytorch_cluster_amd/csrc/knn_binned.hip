@@ -37,10 +37,12 @@
 // number: a full list admits d <= its k-th distance and the 64-bit
 // (distance, row) keys decide.
 #include "device_utils.hpp"
+#include "knn_binned_mc_impl.hpp"
 #include "knn_lowd_impl.hpp"
 #include "launchers.hpp"
 
 #include <climits>
+#include <cstdlib>
 #include <cstring>
 #include <type_traits>
 
@@ -50,10 +52,7 @@ namespace pca {
 
 namespace {
 
-constexpr int kBinTile = 32;      // rows per tile
-constexpr int kBinGroup = 64;     // tiles per group (a box of their own)
 constexpr int kBinQueueCap = 16;  // parked rows per lane
-constexpr int kBinSeedTiles = 16; // most tiles scanned before the sweep
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
@@ -187,21 +186,13 @@ __global__ __launch_bounds__(kBlock) void morton_keys_kernel(
   vals[i] = (uint32_t)i;
 }
 
-// A box: lower corner, upper corner, two words of padding (one 32-byte scalar
-// load).
-struct Box {
-  float lo[3];
-  float hi[3];
-  float pad[2];
-};
-
-// Rows in curve order with their row numbers, and the box of every tile of 32:
-// half a wave per tile.
+// Rows in curve order with their row numbers (plain and as the matrix-core
+// filter takes them), and the box of every tile of 32: half a wave per tile.
 __global__ __launch_bounds__(kBlock) void gather_tiles_kernel(
     const float *__restrict__ x, const int64_t *__restrict__ ptr_x, int n,
     int d, int num_segments, const int *__restrict__ tile_start,
     const uint32_t *__restrict__ perm, float4 *__restrict__ rows,
-    Box *__restrict__ box) {
+    uint4 *__restrict__ packed, Box *__restrict__ box) {
   const int gt = (blockIdx.x * kBlock + threadIdx.x) / kBinTile;
   const int r = threadIdx.x & (kBinTile - 1);
   if (gt >= tile_start[num_segments])
@@ -216,8 +207,15 @@ __global__ __launch_bounds__(kBlock) void gather_tiles_kernel(
 #pragma unroll
   for (int c = 0; c < 3; ++c)
     v[c] = (ok && c < d) ? x[(size_t)id * d + c] : 0.0f;
-  if (ok)
+  if (ok) {
     rows[j] = make_float4(v[0], v[1], v[2], __uint_as_float(id));
+    // the operand of the matrix-core filter, then coordinates and row number
+    uint4 rec[McShape<3>::REC];
+    mc_pack_row<3>(v, rec);
+    rec[1].w = id;
+    packed[(size_t)j * 2] = rec[0];
+    packed[(size_t)j * 2 + 1] = rec[1];
+  }
 #pragma unroll
   for (int c = 0; c < 3; ++c) {
     // (fminf / fmaxf drop a NaN operand: a NaN coordinate is in no box, and
@@ -233,6 +231,16 @@ __global__ __launch_bounds__(kBlock) void gather_tiles_kernel(
       box[gt].lo[c] = lo;
       box[gt].hi[c] = hi;
     }
+  }
+}
+
+// A tile of rows behind the last one that never pass the filter (operand
+// w = NaN), so that a fetch of a whole tile stays inside the copy.
+__global__ void pad_packed_kernel(uint4 *__restrict__ packed, int n) {
+  const int r = threadIdx.x;
+  if (r < kBinTile) {
+    packed[(size_t)(n + r) * 2] = make_uint4(0u, 0x7fc00000u, 0u, 0u);
+    packed[(size_t)(n + r) * 2 + 1] = make_uint4(0u, 0u, 0u, 0u);
   }
 }
 
@@ -265,45 +273,6 @@ __global__ __launch_bounds__(kBlock) void group_boxes_kernel(
       group_box[gg].hi[c] = hi;
     }
   }
-}
-
-struct BinnedParams {
-  const float *y;
-  const int64_t *ptr_x;
-  const int64_t *ptr_y;
-  int n, m, d, num_segments, k;
-  const int *tile_start;    // first tile of every segment
-  const int *wave_start;    // first wave task of every segment
-  const uint32_t *keys_x;   // sorted keys of the x rows
-  const uint32_t *keys_y;   // sorted keys of the queries
-  const uint32_t *perm_y;   // query behind every sorted position
-  const float4 *rows;       // x rows in curve order, .w = row number
-  const Box *box;           // of every tile
-  const int *group_start;   // first group of tiles of every segment
-  const Box *group_box;     // of every group
-  int *out_idx;
-  float *out_dist;
-  int *out_count;
-};
-
-// First position in [lo, hi) whose key is not below `key` (hi if none); the
-// wave probes 64 positions per round.
-__device__ __forceinline__ int wave_lower_bound(
-    const uint32_t *__restrict__ keys, int lo, int hi, uint32_t key,
-    int lane) {
-  while (hi - lo > kWave) {
-    const int step = (hi - lo) / kWave;
-    const int probe = lo + (lane + 1) * step - 1;
-    const int below = __popcll(__ballot(keys[probe] < key));
-    // probes 0 .. below-1 are below the key, probe `below` (if any) is not
-    const int new_lo = lo + below * step;
-    if (below < kWave)
-      hi = lo + (below + 1) * step - 1;
-    lo = new_lo;
-  }
-  const int probe = lo + lane;
-  const bool below = probe < hi && keys[probe] < key;
-  return lo + __popcll(__ballot(below));
 }
 
 template <int K>
@@ -434,21 +403,6 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
       scan_rows(p.rows + j0, rows, std::false_type{});
   };
 
-  // Squared distance between two boxes (a query is a box of one point), with
-  // the operations of the exact chain on per-axis gaps that are not above
-  // |row - query| for any row and query of the boxes: never above the computed
-  // distance of any such pair.
-  auto box_gap2 = [](const float (&alo)[3], const float (&ahi)[3],
-                     const float (&blo)[3], const float (&bhi)[3]) {
-    float acc = 0.0f;
-#pragma unroll
-    for (int c = 0; c < 3; ++c) {
-      const float gap = __builtin_fmaxf(
-          __builtin_fmaxf(alo[c] - bhi[c], blo[c] - ahi[c]), 0.0f);
-      acc = c == 0 ? gap * gap : __builtin_fmaf(gap, gap, acc);
-    }
-    return acc;
-  };
   // largest k-th distance among the wave's queries
   auto wave_reach = [&]() {
     float r = kth;
@@ -471,15 +425,6 @@ __global__ __launch_bounds__(kBlock) void knn_binned_kernel(BinnedParams p) {
     }
     return __any(!(box_gap2(lo, hi, yq, yq) > kth));
   };
-  // the set bit of `mask` nearest to position `at` (mask != 0)
-  auto nearest_bit = [](uint64_t mask, int at) {
-    const uint64_t up = mask >> at;
-    const uint64_t down = at > 0 ? mask & (~(uint64_t)0 >> (64 - at)) : 0;
-    const int d_up = up ? (int)__builtin_ctzll(up) : 128;
-    const int d_down = down ? at - (63 - (int)__builtin_clzll(down)) : 128;
-    return d_up <= d_down ? at + d_up : at - d_down;
-  };
-
   const int tile0 = p.tile_start[seg];
   const int num_tiles = p.tile_start[seg + 1] - tile0;
   if (num_tiles > 0) {
@@ -673,17 +618,6 @@ __global__ __launch_bounds__(kBlock) void radius_binned_kernel(
     }
   };
 
-  auto box_gap2 = [](const float (&alo)[3], const float (&ahi)[3],
-                     const float (&blo)[3], const float (&bhi)[3]) {
-    float acc = 0.0f;
-#pragma unroll
-    for (int c = 0; c < 3; ++c) {
-      const float gap = __builtin_fmaxf(
-          __builtin_fmaxf(alo[c] - bhi[c], blo[c] - ahi[c]), 0.0f);
-      acc = c == 0 ? gap * gap : __builtin_fmaf(gap, gap, acc);
-    }
-    return acc;
-  };
   // is the box of lane `src` closer than the radius to some lane's query?
   // (A NaN - from an infinite or empty box - never rules a box out.)
   auto reachable = [&](const Box &held, int src) {
@@ -752,13 +686,14 @@ __global__ __launch_bounds__(kBlock) void radius_binned_kernel(
 }
 
 struct BinnedLayout {
-  size_t seg_box, keys_a, keys_x, keys_y, vals_a, perm_x, perm_y, rows, box,
-      group_box, tile_start, group_start, wave_start, sort_temp;
+  size_t seg_box, keys_a, keys_x, keys_y, vals_a, perm_x, perm_y, rows, packed,
+      box, group_box, tile_start, group_start, wave_start, half_start,
+      sort_temp;
   int tiles_bound, groups_bound;
   size_t total() const {
     return seg_box + keys_a + keys_x + keys_y + vals_a + perm_x + perm_y +
-           rows + box + group_box + tile_start + group_start + wave_start +
-           sort_temp;
+           rows + packed + box + group_box + tile_start + group_start +
+           wave_start + half_start + sort_temp;
   }
 };
 
@@ -797,6 +732,7 @@ BinnedLayout binned_layout(int n, int m, int num_segments) {
   w.perm_y = align256(sizeof(uint32_t) * (size_t)m);
   // (padded: the search reads rows four at a time)
   w.rows = align256(sizeof(float4) * ((size_t)n + kBinTile));
+  w.packed = align256(sizeof(uint4) * 2 * ((size_t)n + kBinTile));
   w.tiles_bound = plan_upper_bound(n, num_segments, kBinTile);
   w.groups_bound = plan_upper_bound(n, num_segments, kBinTile * kBinGroup);
   w.box = align256(sizeof(Box) * (size_t)w.tiles_bound);
@@ -804,6 +740,7 @@ BinnedLayout binned_layout(int n, int m, int num_segments) {
   w.tile_start = align256(sizeof(int) * (size_t)(num_segments + 1));
   w.group_start = align256(sizeof(int) * (size_t)(num_segments + 1));
   w.wave_start = align256(sizeof(int) * (size_t)(num_segments + 1));
+  w.half_start = align256(sizeof(int) * (size_t)(num_segments + 1));
   size_t tx = 0, ty = 0;
   const hipError_t ex = sort_pairs(nullptr, tx, nullptr, nullptr, nullptr,
                                    nullptr, n, num_segments, nullptr);
@@ -818,9 +755,12 @@ BinnedLayout binned_layout(int n, int m, int num_segments) {
 
 // Everything a binned search reads, as prepare_bins leaves it in the scratch.
 struct Bins {
-  const int *tile_start, *group_start, *wave_start;
+  const int *tile_start, *group_start;
+  const int *wave_start; // tasks of 64 queries
+  const int *half_start; // tasks of 32 queries
   const uint32_t *keys_x, *keys_y, *perm_y;
   const float4 *rows;
+  const uint4 *packed;
   const Box *box, *group_box;
 };
 
@@ -842,11 +782,13 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
   uint32_t *perm_x = static_cast<uint32_t *>(take(lay.perm_x));
   uint32_t *perm_y = static_cast<uint32_t *>(take(lay.perm_y));
   float4 *rows = static_cast<float4 *>(take(lay.rows));
+  uint4 *packed = static_cast<uint4 *>(take(lay.packed));
   Box *box = static_cast<Box *>(take(lay.box));
   Box *group_box = static_cast<Box *>(take(lay.group_box));
   int *tile_start = static_cast<int *>(take(lay.tile_start));
   int *group_start = static_cast<int *>(take(lay.group_start));
   int *wave_start = static_cast<int *>(take(lay.wave_start));
+  int *half_start = static_cast<int *>(take(lay.half_start));
   void *sort_temp = take(lay.sort_temp);
   size_t sort_bytes = lay.sort_temp;
 
@@ -863,6 +805,9 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
     return err;
   if ((err = launch_plan(in.ptr_y, in.m, nseg, kWave, wave_start, stream)) !=
       hipSuccess)
+    return err;
+  if ((err = launch_plan(in.ptr_y, in.m, nseg, kWave / 2, half_start,
+                         stream)) != hipSuccess)
     return err;
   hipLaunchKernelGGL(seg_box_init_kernel, dim3((6 * nseg + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, seg_box, 6 * nseg);
@@ -897,7 +842,9 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
     hipLaunchKernelGGL(gather_tiles_kernel,
                        dim3((lay.tiles_bound + per_block - 1) / per_block),
                        dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
-                       tile_start, perm_x, rows, box);
+                       tile_start, perm_x, rows, packed, box);
+    hipLaunchKernelGGL(pad_packed_kernel, dim3(1), dim3(kWave), 0, stream,
+                       packed, in.n);
     const int groups_per_block = kBlock / kWave;
     hipLaunchKernelGGL(
         group_boxes_kernel,
@@ -911,10 +858,12 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
   bins.tile_start = tile_start;
   bins.group_start = group_start;
   bins.wave_start = wave_start;
+  bins.half_start = half_start;
   bins.keys_x = keys_x;
   bins.keys_y = keys_y;
   bins.perm_y = perm_y;
   bins.rows = rows;
+  bins.packed = packed;
   bins.box = box;
   bins.group_box = group_box;
   return hipSuccess;
@@ -935,6 +884,7 @@ void fill_params(BinnedParams &p, const SearchInput &in, const Bins &bins,
   p.keys_y = bins.keys_y;
   p.perm_y = bins.perm_y;
   p.rows = bins.rows;
+  p.packed = bins.packed;
   p.box = bins.box;
   p.group_start = bins.group_start;
   p.group_box = bins.group_box;
@@ -965,20 +915,32 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
   BinnedParams p;
   fill_params(p, in, bins, out);
   p.k = k;
-  const int waves = plan_upper_bound(in.m, in.num_segments, kWave);
+  // (diagnostic switch: the vector-ALU scan instead of the matrix-core one)
+  const char *env = getenv("PCA_KNN_BINNED_MATRIX_CORES");
+  const bool matrix_cores = !(env != nullptr && env[0] == '0');
+  const int per_task = matrix_cores ? kWave / 2 : kWave;
+  if (matrix_cores)
+    p.wave_start = bins.half_start;
+  const int waves = plan_upper_bound(in.m, in.num_segments, per_task);
   const int grid = (waves + kBlock / kWave - 1) / (kBlock / kWave);
+#define PCA_BINNED_LAUNCH(K_)                                                  \
+  do {                                                                         \
+    if (matrix_cores)                                                          \
+      hipLaunchKernelGGL((knn_binned_mc_kernel<K_>), dim3(grid), dim3(kBlock), \
+                         0, stream, p);                                        \
+    else                                                                       \
+      hipLaunchKernelGGL((knn_binned_kernel<K_>), dim3(grid), dim3(kBlock), 0, \
+                         stream, p);                                           \
+  } while (0)
   if (k <= 8)
-    hipLaunchKernelGGL((knn_binned_kernel<8>), dim3(grid), dim3(kBlock), 0,
-                       stream, p);
+    PCA_BINNED_LAUNCH(8);
   else if (k <= 16)
-    hipLaunchKernelGGL((knn_binned_kernel<16>), dim3(grid), dim3(kBlock), 0,
-                       stream, p);
+    PCA_BINNED_LAUNCH(16);
   else if (k <= 24)
-    hipLaunchKernelGGL((knn_binned_kernel<24>), dim3(grid), dim3(kBlock), 0,
-                       stream, p);
+    PCA_BINNED_LAUNCH(24);
   else
-    hipLaunchKernelGGL((knn_binned_kernel<32>), dim3(grid), dim3(kBlock), 0,
-                       stream, p);
+    PCA_BINNED_LAUNCH(32);
+#undef PCA_BINNED_LAUNCH
   if (time_stop)
     (void)hipEventRecord(time_stop, stream);
   return hipGetLastError();

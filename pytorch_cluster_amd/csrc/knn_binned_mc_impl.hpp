@@ -1,0 +1,496 @@
+// The binned kNN search (knn_binned.hip) with the scan of a tile done by the
+// matrix-core pre-filter of knn_lowd_mc_impl.hpp: one
+// v_mfma_f32_32x32x16_bf16 gives the signs of t - cut for the 32 rows of a
+// tile against 32 queries, 16 funnel shifts per lane gather them, and only the
+// flagged rows get their exact fp32 distance (from a copy of the tile's
+// coordinates in LDS).  Results are those of the reference's scan
+// (csrc/cuda/knn_cuda.cu:52-78) bit for bit, as for the other kernels.
+//
+// A wave owns 32 curve-consecutive queries: lanes l and l + 32 share query
+// l % 32 (hi and lo parts of its operand) and split every tile's rows, 16
+// each, with a sorted list of their own; the two lists are united at the end.
+// The coordinates of the last kBinRing scanned tiles stay in a per-wave ring
+// in LDS; a lane parks at most one word (ring slot, sign mask) per tile, and
+// the parked rows are resolved exactly, by all lanes together, when the ring
+// has gone round.  Rows are met out of row order, so every bound admits an
+// equal distance (the 64-bit (distance, row) keys decide), as in the `nearest`
+// mode of the scanning kernel.
+#pragma once
+
+#include "knn_lowd_mc_impl.hpp"
+
+namespace pca {
+
+constexpr int kBinTile = 32;  // rows per tile
+constexpr int kBinGroup = 64; // tiles per group (a box of their own)
+constexpr int kBinRing = 8;   // tiles whose coordinates stay in LDS
+constexpr int kBinSeedTiles = 16; // most tiles scanned before the sweep
+
+// A box: lower corner, upper corner, two words of padding (32 bytes).
+struct Box {
+  float lo[3];
+  float hi[3];
+  float pad[2];
+};
+
+struct BinnedParams {
+  const float *y;
+  const int64_t *ptr_x;
+  const int64_t *ptr_y;
+  int n, m, d, num_segments, k;
+  const int *tile_start;    // first tile of every segment
+  const int *wave_start;    // first wave task of every segment
+  const uint32_t *keys_x;   // sorted keys of the x rows
+  const uint32_t *keys_y;   // sorted keys of the queries
+  const uint32_t *perm_y;   // query behind every sorted position
+  const float4 *rows;       // x rows in curve order, .w = row number
+  const uint4 *packed;      // the same rows as mc_pack_row<3> leaves them,
+                            // the fourth coordinate word = row number
+  const Box *box;           // of every tile
+  const int *group_start;   // first group of tiles of every segment
+  const Box *group_box;     // of every group
+  int *out_idx;
+  float *out_dist;
+  int *out_count;
+};
+
+// First position in [lo, hi) whose key is not below `key` (hi if none); the
+// wave probes 64 positions per round.
+__device__ __forceinline__ int wave_lower_bound(
+    const uint32_t *__restrict__ keys, int lo, int hi, uint32_t key,
+    int lane) {
+  while (hi - lo > kWave) {
+    const int step = (hi - lo) / kWave;
+    const int probe = lo + (lane + 1) * step - 1;
+    const int below = __popcll(__ballot(keys[probe] < key));
+    // probes 0 .. below-1 are below the key, probe `below` (if any) is not
+    const int new_lo = lo + below * step;
+    if (below < kWave)
+      hi = lo + (below + 1) * step - 1;
+    lo = new_lo;
+  }
+  const int probe = lo + lane;
+  const bool below = probe < hi && keys[probe] < key;
+  return lo + __popcll(__ballot(below));
+}
+
+// Squared distance between two boxes (a query is a box of one point), with
+// the operations of the exact chain on per-axis gaps that are not above
+// |row - query| for any row and query of the boxes: never above the computed
+// distance of any such pair.
+__device__ __forceinline__ float box_gap2(const float (&alo)[3],
+                                          const float (&ahi)[3],
+                                          const float (&blo)[3],
+                                          const float (&bhi)[3]) {
+  float acc = 0.0f;
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    const float gap = __builtin_fmaxf(
+        __builtin_fmaxf(alo[c] - bhi[c], blo[c] - ahi[c]), 0.0f);
+    acc = c == 0 ? gap * gap : __builtin_fmaf(gap, gap, acc);
+  }
+  return acc;
+}
+
+// the set bit of `mask` nearest to position `at` (mask != 0)
+__device__ __forceinline__ int nearest_bit(uint64_t mask, int at) {
+  const uint64_t up = mask >> at;
+  const uint64_t down = at > 0 ? mask & (~(uint64_t)0 >> (64 - at)) : 0;
+  const int d_up = up ? (int)__builtin_ctzll(up) : 128;
+  const int d_down = down ? at - (63 - (int)__builtin_clzll(down)) : 128;
+  return d_up <= d_down ? at + d_up : at - d_down;
+}
+
+// p.wave_start counts tasks of 32 queries.
+template <int K>
+__global__ __launch_bounds__(kBlock) void knn_binned_mc_kernel(BinnedParams p) {
+  constexpr int DIM = 3;
+  constexpr int REC = McShape<DIM>::REC; // operand quad, coordinate quad
+  static_assert(McShape<DIM>::NI == 1 && REC == 2, "one instruction per tile");
+  constexpr float kLimit = kKnnSentinel;
+  constexpr int kWaves = kBlock / kWave;
+
+  // coordinates and row numbers of the last kBinRing tiles of every wave
+  __shared__ __attribute__((aligned(16))) uint4 ring[kWaves][kBinRing][kBinTile];
+  // parked words: (ring slot << 16) | mask of the lane's 16 rows that passed
+  __shared__ uint32_t queue[kBinRing][kBlock];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int half = lane >> 5;
+  const int col = lane & 31;
+  const int task = blockIdx.x * kWaves + wave;
+  if (task >= p.wave_start[p.num_segments])
+    return; // (whole waves leave; no barrier below)
+  const int seg = find_segment(p.wave_start, p.num_segments, task);
+  const int x_begin = p.ptr_x ? (int)p.ptr_x[seg] : 0;
+  const int x_end = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
+  const int y_begin = p.ptr_y ? (int)p.ptr_y[seg] : 0;
+  const int y_end = p.ptr_y ? (int)p.ptr_y[seg + 1] : p.m;
+  const int jq0 = y_begin + (task - p.wave_start[seg]) * 32;
+  const int jq = jq0 + col;
+  const bool valid = jq < y_end;
+  const int q = valid ? (int)p.perm_y[jq] : 0;
+  const int k = p.k;
+  const int d_in = p.d;
+
+  float yq[DIM];
+#pragma unroll
+  for (int c = 0; c < DIM; ++c)
+    yq[c] = (valid && c < d_in) ? p.y[(size_t)q * d_in + c] : 0.0f;
+  // a query with a coordinate that is not finite has no distance below the
+  // limit: it looks at nothing and returns nothing
+  const bool searching = valid && __builtin_fabsf(yq[0]) < __builtin_inff() &&
+                         __builtin_fabsf(yq[1]) < __builtin_inff() &&
+                         __builtin_fabsf(yq[2]) < __builtin_inff();
+  float ysq = yq[0] * yq[0];
+#pragma unroll
+  for (int c = 1; c < DIM; ++c)
+    ysq = __builtin_fmaf(yq[c], yq[c], ysq);
+  const bool y_moderate = ysq <= kFilterNormLimit;
+
+  // the wave's box (lanes that do not search stay out)
+  float q_lo[3], q_hi[3];
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    float lo = searching ? yq[c] : __builtin_inff();
+    float hi = searching ? yq[c] : -__builtin_inff();
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1) {
+      lo = __builtin_fminf(lo, __shfl_xor(lo, sh));
+      hi = __builtin_fmaxf(hi, __shfl_xor(hi, sh));
+    }
+    q_lo[c] = lo;
+    q_hi[c] = hi;
+  }
+
+  // B operand: the hi (lanes 0-31) or lo (lanes 32-63) parts of
+  // (-2 y_0, -2 y_1, -2 y_2, 1), given twice (against the hi and the lo parts
+  // of the row); see knn_lowd_mc_impl.hpp
+  uint4 yb_plain;
+  {
+    uint32_t part[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float v = 0.0f;
+      if (e < DIM)
+        v = (searching && y_moderate) ? -2.0f * yq[e] : 0.0f;
+      else
+        v = searching ? 1.0f : 0.0f;
+      uint32_t hi, lo;
+      mc_split(v, hi, lo);
+      part[e] = half ? lo : hi;
+    }
+    const uint32_t w0 = part[0] | (part[1] << 16);
+    const uint32_t w1 = part[2] | (part[3] << 16);
+    yb_plain = make_uint4(w0, w1, w0, w1);
+  }
+  mc_bf16x8_t yb = __builtin_bit_cast(mc_bf16x8_t, yb_plain);
+
+  double best[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j)
+    best[j] = (j < K - k) ? lowest_key() : empty_key();
+  // exact distances must be strictly below thresh: the limit, or just above
+  // the smaller of this lane's and the query's k-th distance (equality still
+  // passes); a lane that does not search accepts nothing
+  const float ysq_damped = mc_damped_norm(ysq);
+  float thresh = searching ? kLimit : -__builtin_inff();
+  float cut = searching ? mc_filter_cut(thresh, ysq_damped) : -1e38f;
+  float shared = kLimit; // bound learnt from the partner lane
+  // -cut rides in the two accumulation slots of w that the zero lo part of
+  // the query's 1 would leave unused (component 3 of the one instruction)
+  const uint32_t one_keep = half ? ~(0xffffu << 16) : 0xffffffffu;
+  const uint32_t one_bits = half ? (0x3f80u << 16) : 0u;
+  auto refresh_cut = [&]() {
+    if (half) {
+      float neg = -__builtin_fmaf(__builtin_fabsf(cut), 3.0517578125e-05f, cut);
+      uint32_t hi, lo;
+      if (__builtin_fabsf(neg) < 1e38f) {
+        mc_split(neg, hi, lo);
+      } else {
+        hi = neg < 0.0f ? 0xff7fu : 0x7f7fu;
+        lo = 0;
+      }
+      uint4 b = yb_plain;
+      b.y = (b.y & 0x0000ffffu) | (hi << 16);
+      b.w = (b.w & 0x0000ffffu) | (lo << 16);
+      yb = __builtin_bit_cast(mc_bf16x8_t, b);
+    }
+  };
+  refresh_cut();
+  auto set_thresh = [&](float v) {
+    if (searching) {
+      thresh = v;
+      cut = mc_filter_cut(v, ysq_damped);
+    }
+  };
+
+  int qn = 0; // parked words of this lane
+
+  // What the two lanes of a query tell each other about its final k-th
+  // distance (see knn_lowd_mc_impl.hpp; equality admitted).
+  auto partner_bounds = [&]() {
+    const float own = key_dist(best[K - 1]);
+    const auto both = __builtin_amdgcn_permlane32_swap(
+        __float_as_uint(own), __float_as_uint(own), false, false);
+    float partner = __uint_as_float(half ? both[0] : both[1]);
+    if (K >= 2) {
+      const int c = k >> 1;
+      float mid = kLimit;
+#pragma unroll
+      for (int cc = (K >= 8 ? K / 2 - 4 : 0); cc <= K / 2; ++cc)
+        if (cc >= 1 && cc == c) {
+          asm volatile(""); // (keeps this a branch)
+          mid = key_dist(best[K - 1 - cc]);
+        }
+      const auto mids = __builtin_amdgcn_permlane32_swap(
+          __float_as_uint(mid), __float_as_uint(mid), false, false);
+      const float partner_mid = __uint_as_float(half ? mids[0] : mids[1]);
+      partner = __builtin_fminf(partner, __builtin_fmaxf(mid, partner_mid));
+    }
+    if (searching && partner < kLimit) {
+      shared = __builtin_fminf(shared, next_up_positive(partner));
+      if (shared < thresh)
+        set_thresh(shared);
+    }
+  };
+
+  // Resolves the parked rows exactly: in every round each lane takes the next
+  // row of its parked words and all lanes evaluate theirs together.
+  auto drain = [&]() {
+    bool changed = false; // wave-uniform
+    int taken = 0;
+    uint32_t pending = 0;
+    int slot_base = 0;
+    for (;;) {
+      if (pending == 0 && taken < qn) {
+        const uint32_t word = queue[taken][tid];
+        ++taken;
+        pending = word & 0xffffu;
+        slot_base = (int)(word >> 16) * kBinTile + 4 * half;
+      }
+      const bool has = pending != 0;
+      if (!__any(has))
+        break;
+      // bit 15 - v of the mask stands for accumulator v = row
+      // 8 (v / 4) + 4 half + v % 4 of the tile
+      const int bit = 31 - __builtin_clz(has ? pending : 1u);
+      const int v = 15 - bit;
+      pending &= ~(1u << bit);
+      const int j = has ? slot_base + 2 * (v & 12) + (v & 3) : 0;
+      const uint4 r4 = (&ring[wave][0][0])[j];
+      const float d0 = __uint_as_float(r4.x) - yq[0];
+      float d = d0 * d0;
+      const float d1 = __uint_as_float(r4.y) - yq[1];
+      d = __builtin_fmaf(d1, d1, d);
+      const float d2 = __uint_as_float(r4.z) - yq[2];
+      d = __builtin_fmaf(d2, d2, d);
+      const bool ok = has && d < thresh;
+      if (!__any(ok))
+        continue;
+      const double key = ok ? make_key(d, r4.w) : empty_key();
+      sorted_insert<K>(best, key);
+      float own_bound = key_dist(best[K - 1]);
+      // (a row of EQUAL distance and smaller number can still get in)
+      if (own_bound < kLimit)
+        own_bound = next_up_positive(own_bound);
+      set_thresh(__builtin_fminf(own_bound, shared));
+      changed = true;
+    }
+    qn = 0;
+    if (!changed)
+      return;
+    partner_bounds();
+    refresh_cut();
+  };
+
+  // largest bound among the wave's queries
+  auto wave_reach = [&]() {
+    float r = searching ? thresh : -1.0f;
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1)
+      r = __builtin_fmaxf(r, __shfl_xor(r, sh));
+    return r;
+  };
+
+  const int tile0 = p.tile_start[seg];
+  const int num_tiles = p.tile_start[seg + 1] - tile0;
+  int scanned = 0; // tiles since the start: slot = scanned % kBinRing
+
+  // The rows of a tile as the lanes fetch them: the operand quad of row
+  // `col` (both halves), the coordinate quad of row `col` (lower half).
+  struct Fetched {
+    uint4 operand, coords;
+  };
+  auto fetch = [&](int tile) {
+    const size_t j = (size_t)(x_begin + tile * kBinTile + col);
+    Fetched f;
+    // (the packed copy is padded by a tile of rows that never pass)
+    f.operand = p.packed[j * REC];
+    f.coords = half ? make_uint4(0u, 0u, 0u, 0u) : p.packed[j * REC + 1];
+    return f;
+  };
+  auto scan = [&](int tile, const Fetched &f) {
+    const int slot = scanned % kBinRing;
+    if (!half)
+      ring[wave][slot][col] = f.coords;
+    uint4 a = f.operand;
+    // upper lanes: 1 in place of w_hi and w_lo (times the parts of -cut)
+    a.y = (a.y & one_keep) | one_bits;
+    a.w = (a.w & one_keep) | one_bits;
+    mfma_acc_t acc = {0};
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+        __builtin_bit_cast(mc_bf16x8_t, a), yb, acc, 0, 0, 0);
+    uint32_t mask = 0;
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      mask = __builtin_amdgcn_alignbit(mask, __float_as_uint(acc[v]), 31);
+    const int rows = min(kBinTile, x_end - (x_begin + tile * kBinTile));
+    if (rows < kBinTile) {
+      // the segment's last tile: rows past its end belong to the next one
+      uint32_t real = 0;
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        real |= (8 * (v / 4) + 4 * half + v % 4 < rows) ? (1u << (15 - v)) : 0u;
+      mask &= real;
+    }
+    if (mask != 0) {
+      queue[qn][tid] = ((uint32_t)slot << 16) | mask;
+      ++qn;
+    }
+    ++scanned;
+    if (scanned % kBinRing == 0)
+      drain();
+  };
+
+  if (num_tiles > 0) {
+    // where the wave's first and last query fall in the order of x
+    const int last_col = min(32, y_end - jq0) - 1;
+    const uint32_t key_first = p.keys_y[jq0];
+    const uint32_t key_last = p.keys_y[jq0 + last_col];
+    const int pos_first =
+        wave_lower_bound(p.keys_x, x_begin, x_end, key_first, lane);
+    const int pos_last =
+        wave_lower_bound(p.keys_x, x_begin, x_end, key_last, lane);
+    const int t_first = min(num_tiles - 1, (pos_first - x_begin) / kBinTile);
+    const int t_last = min(num_tiles - 1, (pos_last - x_begin) / kBinTile);
+    // tiles seed_lo .. seed_hi are scanned up front
+    int seed_lo = max(0, t_first - 1);
+    int seed_hi = min(num_tiles - 1, max(t_last, t_first) + 1);
+    if (seed_hi - seed_lo + 1 > kBinSeedTiles) {
+      const int mid = (seed_lo + seed_hi) / 2;
+      seed_lo = max(0, mid - kBinSeedTiles / 2);
+      seed_hi = min(num_tiles - 1, seed_lo + kBinSeedTiles - 1);
+    }
+    {
+      Fetched next = fetch(seed_lo);
+      for (int t = seed_lo; t <= seed_hi; ++t) {
+        const Fetched cur = next;
+        if (t < seed_hi)
+          next = fetch(t + 1);
+        scan(t, cur);
+      }
+    }
+    drain();
+    float reach = wave_reach();
+
+    // is the box of lane `src` within reach of some lane's query?  (A NaN -
+    // from an infinite or empty box - never rules a box out.)
+    auto reachable = [&](const Box &held, int src) {
+      float lo[3], hi[3];
+#pragma unroll
+      for (int c = 0; c < 3; ++c) {
+        lo[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+            (int)__float_as_uint(held.lo[c]), src));
+        hi[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+            (int)__float_as_uint(held.hi[c]), src));
+      }
+      return __any(searching && !(box_gap2(lo, hi, yq, yq) >= thresh));
+    };
+
+    // Groups of tiles, 64 at a time (one box per lane), nearest to the seed
+    // tiles first; a group, then a tile, is looked into if its box is within
+    // the wave's largest bound of the box around the wave's queries, and then
+    // within some query's own bound of that query.
+    const int group0 = p.group_start[seg];
+    const int num_groups = (num_tiles + kBinGroup - 1) / kBinGroup;
+    const int centre = ((seed_lo + seed_hi) / 2) / kBinGroup;
+    const int num_rounds = (num_groups + kWave - 1) / kWave;
+    const int centre_round = centre / kWave;
+    for (int i = 0; i < 2 * num_rounds; ++i) {
+      const int round = centre_round + ((i & 1) ? -((i + 1) >> 1) : (i >> 1));
+      if (round < 0 || round >= num_rounds)
+        continue;
+      const int g_mine = round * kWave + lane;
+      Box g_box = {};
+      if (g_mine < num_groups)
+        g_box = p.group_box[group0 + g_mine];
+      uint64_t g_todo =
+          __ballot(g_mine < num_groups &&
+                   !(box_gap2(g_box.lo, g_box.hi, q_lo, q_hi) >= reach));
+      const int g_at = min(max(centre - round * kWave, 0), kWave - 1);
+      while (g_todo != 0) {
+        const int g_lane = nearest_bit(g_todo, g_at);
+        g_todo &= ~((uint64_t)1 << g_lane);
+        if (!reachable(g_box, g_lane))
+          continue;
+        const int group = round * kWave + g_lane;
+        const int t_mine = group * kBinGroup + lane;
+        const bool t_ok =
+            t_mine < num_tiles && !(t_mine >= seed_lo && t_mine <= seed_hi);
+        Box t_box = {};
+        if (t_ok)
+          t_box = p.box[tile0 + t_mine];
+        uint64_t t_todo = __ballot(
+            t_ok && !(box_gap2(t_box.lo, t_box.hi, q_lo, q_hi) >= reach));
+        // the tiles of the group that some query can reach, by its bound of
+        // now; their rows are fetched one tile ahead of the scan
+        uint64_t t_pass = 0;
+        while (t_todo != 0) {
+          const int t_lane = (int)__builtin_ctzll(t_todo);
+          t_todo &= t_todo - 1;
+          if (reachable(t_box, t_lane))
+            t_pass |= (uint64_t)1 << t_lane;
+        }
+        if (t_pass != 0) {
+          Fetched next = fetch(group * kBinGroup + (int)__builtin_ctzll(t_pass));
+          while (t_pass != 0) {
+            const int t_lane = (int)__builtin_ctzll(t_pass);
+            t_pass &= t_pass - 1;
+            const Fetched cur = next;
+            if (t_pass != 0)
+              next =
+                  fetch(group * kBinGroup + (int)__builtin_ctzll(t_pass));
+            scan(group * kBinGroup + t_lane, cur);
+          }
+          if (__any(qn > 0)) {
+            drain();
+            reach = wave_reach();
+          }
+        }
+      }
+    }
+    drain();
+  }
+
+  // unite the two half lists of each query in the lower lane
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    if (j < K - k)
+      continue; // slots below are padding, not keys
+    const auto hi = __builtin_amdgcn_permlane32_swap(
+        (unsigned)__double2hiint(best[j]), (unsigned)__double2hiint(best[j]),
+        false, false);
+    const auto lo = __builtin_amdgcn_permlane32_swap(
+        (unsigned)__double2loint(best[j]), (unsigned)__double2loint(best[j]),
+        false, false);
+    const double upper = __hiloint2double((int)hi[1], (int)lo[1]);
+    sorted_insert<K>(best, half ? empty_key() : upper);
+  }
+  if (half == 0 && valid)
+    write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+}
+
+} // namespace pca

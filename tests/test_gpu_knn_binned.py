@@ -16,6 +16,14 @@ from pytorch_cluster_amd import capi, testing  # noqa: E402
 from gpu_common import DEV, dev, gpu_knn, oracle_knn_edges, ragged_ptrs  # noqa
 
 
+@pytest.fixture(autouse=True, params=["1", "0"],
+                ids=["matrix_cores", "vector_alu"])
+def scan_kind(request, monkeypatch):
+    # both scans of a tile, whichever is the default
+    monkeypatch.setenv("PCA_KNN_BINNED_MATRIX_CORES", request.param)
+    return request.param
+
+
 def gpu_knn_binned(x, y, ptr_x, ptr_y, k, want_dist=True, **kw):
     e, d = capi.knn_edges(dev(x), dev(y), dev(ptr_x, torch.long),
                           dev(ptr_y, torch.long), k, False, want_dist,
