@@ -714,7 +714,14 @@ hipError_t sort_pairs(void *temp, size_t &temp_bytes, const uint32_t *keys_in,
                       uint32_t *vals_out, int count, int num_segments,
                       hipStream_t stream) {
   const int bits = segment_bits(num_segments) + 3 * axis_bits(num_segments);
-  return rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out,
+  // (rocPRIM's default turns to merge sort up to 2^20 items - 19 launches for
+  // a million rows; measured here, its one-sweep radix sort is quicker from a
+  // few hundred thousand rows on and slower below)
+  using Config =
+      rocprim::radix_sort_config<rocprim::default_config,
+                                 rocprim::default_config,
+                                 rocprim::default_config, 300000>;
+  return rocprim::radix_sort_pairs<Config>(temp, temp_bytes, keys_in, keys_out,
                                    vals_in, vals_out, (unsigned int)count, 0u,
                                    (unsigned int)std::max(bits, 1), stream,
                                    false);
