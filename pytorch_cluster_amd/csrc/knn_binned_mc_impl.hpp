@@ -103,7 +103,8 @@ __device__ __forceinline__ int nearest_bit(uint64_t mask, int at) {
 
 // p.wave_start counts tasks of 32 queries.
 template <int K>
-__global__ __launch_bounds__(kBlock) void knn_binned_mc_kernel(BinnedParams p) {
+__global__ __launch_bounds__(kBlock, K <= 16 ? 4 : 1) void knn_binned_mc_kernel(
+    BinnedParams p) {
   constexpr int DIM = 3;
   constexpr int REC = McShape<DIM>::REC; // operand quad, coordinate quad
   static_assert(McShape<DIM>::NI == 1 && REC == 2, "one instruction per tile");
