@@ -933,8 +933,8 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
 #define PCA_BINNED_LAUNCH(K_)                                                  \
   do {                                                                         \
     if (matrix_cores)                                                          \
-      hipLaunchKernelGGL((knn_binned_mc_kernel<K_>), dim3(grid), dim3(kBlock), \
-                         0, stream, p);                                        \
+      hipLaunchKernelGGL((knn_binned_mc_kernel<K_>), dim3(waves),              \
+                         dim3(kBinMcBlock), 0, stream, p);                     \
     else                                                                       \
       hipLaunchKernelGGL((knn_binned_kernel<K_>), dim3(grid), dim3(kBlock), 0, \
                          stream, p);                                           \

@@ -101,20 +101,25 @@ __device__ __forceinline__ int nearest_bit(uint64_t mask, int at) {
   return d_up <= d_down ? at + d_up : at - d_down;
 }
 
+// Waves work on their own (no barrier): a workgroup is one wave, so that its
+// place on the SIMD frees up the moment it is done - the tasks differ a lot in
+// length.
+constexpr int kBinMcBlock = kWave;
+
 // p.wave_start counts tasks of 32 queries.
 template <int K>
-__global__ __launch_bounds__(kBlock, K <= 16 ? 4 : 1) void knn_binned_mc_kernel(
-    BinnedParams p) {
+__global__ __launch_bounds__(kBinMcBlock, K <= 16 ? 4 : 1) void
+knn_binned_mc_kernel(BinnedParams p) {
   constexpr int DIM = 3;
   constexpr int REC = McShape<DIM>::REC; // operand quad, coordinate quad
   static_assert(McShape<DIM>::NI == 1 && REC == 2, "one instruction per tile");
   constexpr float kLimit = kKnnSentinel;
-  constexpr int kWaves = kBlock / kWave;
+  constexpr int kWaves = kBinMcBlock / kWave;
 
   // coordinates and row numbers of the last kBinRing tiles of every wave
   __shared__ __attribute__((aligned(16))) uint4 ring[kWaves][kBinRing][kBinTile];
   // parked words: (ring slot << 16) | mask of the lane's 16 rows that passed
-  __shared__ uint32_t queue[kBinRing][kBlock];
+  __shared__ uint32_t queue[kBinRing][kBinMcBlock];
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
