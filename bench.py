@@ -246,6 +246,12 @@ def main():
                     help="run only the other benchmark configurations and "
                          "print their timings (for kernel traces of those "
                          "paths)")
+    ap.add_argument("--strategy", choices=("scan", "binned", "auto"),
+                    default="scan",
+                    help="search strategy of the timed steps: scan (default, "
+                         "the kernel the roofline figure is about), binned or "
+                         "auto (rows ordered along a space-filling curve, "
+                         "exact pruning; same edges)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy three times, so "
                          "that a counter profile of this command can scale "
@@ -275,6 +281,9 @@ def main():
     bx, by = data["batch_x"].to(dev), data["batch_y"].to(dev)
     n, m = x.shape[0], y.shape[0]
     pairs = int(((ptr_x[1:] - ptr_x[:-1]) * (ptr_y[1:] - ptr_y[:-1])).sum())
+
+    pca.set_search_strategy(args.strategy)
+    binned = args.strategy != "scan"
 
     def step():
         return pca.knn(x, y, K, bx, by, batch_size=B)
@@ -341,6 +350,13 @@ def main():
             "traffic": measured_traffic(),
         },
     }
+    if binned:
+        # the events bracket binning + search here, and the work is not the
+        # 9 flop x all pairs the roofline figure prices: no roofline claim
+        result["config"]["strategy"] = args.strategy
+        result["roofline"] = None
+        result["search_ms"] = kernel_s * 1e3
+    pca.set_search_strategy("scan")
     if not args.no_extras:
         result["other_configs"] = other_configs(torch, pca, testing, dev)
     if args.copy_calibration:
