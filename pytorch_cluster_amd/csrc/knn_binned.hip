@@ -232,6 +232,14 @@ __global__ __launch_bounds__(kBlock) void gather_tiles_kernel(
       box[gt].hi[c] = hi;
     }
   }
+  uint32_t min_row = ok ? id : 0xffffffffu;
+#pragma unroll
+  for (int sh = 1; sh < kBinTile; sh <<= 1)
+    min_row = min(min_row, (uint32_t)__shfl_xor((int)min_row, sh));
+  if (r == 0) {
+    box[gt].min_row = min_row;
+    box[gt].pad = 0u;
+  }
 }
 
 // A tile of rows behind the last one that never pass the filter (operand
@@ -272,6 +280,14 @@ __global__ __launch_bounds__(kBlock) void group_boxes_kernel(
       group_box[gg].lo[c] = lo;
       group_box[gg].hi[c] = hi;
     }
+  }
+  uint32_t min_row = ok ? box[tile_start[seg] + t].min_row : 0xffffffffu;
+#pragma unroll
+  for (int sh = 1; sh < kWave; sh <<= 1)
+    min_row = min(min_row, (uint32_t)__shfl_xor((int)min_row, sh));
+  if (lane == 0) {
+    group_box[gg].min_row = min_row;
+    group_box[gg].pad = 0u;
   }
 }
 
@@ -967,21 +983,33 @@ hipError_t launch_radius_binned(const SearchInput &in, float r2,
   BinnedParams p;
   fill_params(p, in, bins, out);
   p.k = out.slots;
-  const int waves = plan_upper_bound(in.m, in.num_segments, kWave);
-  const int grid = (waves + kBlock / kWave - 1) / (kBlock / kWave);
   const int same = ignore_same_index ? 1 : 0;
+  // (diagnostic switch: the vector-ALU scan instead of the matrix-core one)
+  const char *env = getenv("PCA_RADIUS_BINNED_MATRIX_CORES");
+  const bool matrix_cores = !(env != nullptr && env[0] == '0');
+  const int per_task = matrix_cores ? kWave / 2 : kWave;
+  if (matrix_cores)
+    p.wave_start = bins.half_start;
+  const int waves = plan_upper_bound(in.m, in.num_segments, per_task);
+  const int grid = (waves + kBlock / kWave - 1) / (kBlock / kWave);
+#define PCA_BINNED_LAUNCH(K_)                                                  \
+  do {                                                                         \
+    if (matrix_cores)                                                          \
+      hipLaunchKernelGGL((radius_binned_mc_kernel<K_>), dim3(waves),           \
+                         dim3(kBinMcBlock), 0, stream, p, r2, same);           \
+    else                                                                       \
+      hipLaunchKernelGGL((radius_binned_kernel<K_>), dim3(grid), dim3(kBlock), \
+                         0, stream, p, r2, same);                              \
+  } while (0)
   if (out.slots <= 8)
-    hipLaunchKernelGGL((radius_binned_kernel<8>), dim3(grid), dim3(kBlock), 0,
-                       stream, p, r2, same);
+    PCA_BINNED_LAUNCH(8);
   else if (out.slots <= 16)
-    hipLaunchKernelGGL((radius_binned_kernel<16>), dim3(grid), dim3(kBlock),
-                       0, stream, p, r2, same);
+    PCA_BINNED_LAUNCH(16);
   else if (out.slots <= 24)
-    hipLaunchKernelGGL((radius_binned_kernel<24>), dim3(grid), dim3(kBlock),
-                       0, stream, p, r2, same);
+    PCA_BINNED_LAUNCH(24);
   else
-    hipLaunchKernelGGL((radius_binned_kernel<32>), dim3(grid), dim3(kBlock),
-                       0, stream, p, r2, same);
+    PCA_BINNED_LAUNCH(32);
+#undef PCA_BINNED_LAUNCH
   return hipGetLastError();
 }
 

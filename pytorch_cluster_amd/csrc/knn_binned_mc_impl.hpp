@@ -26,11 +26,13 @@ constexpr int kBinGroup = 64; // tiles per group (a box of their own)
 constexpr int kBinRing = 8;   // tiles whose coordinates stay in LDS
 constexpr int kBinSeedTiles = 16; // most tiles scanned before the sweep
 
-// A box: lower corner, upper corner, two words of padding (32 bytes).
+// A box: lower corner, upper corner, the smallest row number inside, a word
+// of padding (32 bytes).
 struct Box {
   float lo[3];
   float hi[3];
-  float pad[2];
+  uint32_t min_row;
+  uint32_t pad;
 };
 
 struct BinnedParams {
@@ -497,6 +499,313 @@ knn_binned_mc_kernel(BinnedParams p) {
   }
   if (half == 0 && valid)
     write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+}
+
+// The binned radius search with the same scan (reference: radius_kernel,
+// csrc/cuda/radius_cuda.cu:9-42): every row with a squared distance strictly
+// below r2, at most `slots` (= p.k) of them - the ones with the smallest row
+// numbers, ascending.  The bound of the filter is fixed (r2), so the query
+// operand is built once and there are no seed tiles; flagged rows get their
+// exact distance from the ring, and those in range whose number is below the
+// largest one of a full list go into the list (row numbers as doubles).
+// p.wave_start counts tasks of 32 queries.
+template <int K>
+__global__ __launch_bounds__(kBinMcBlock, K <= 16 ? 4 : 1) void
+radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
+  constexpr int DIM = 3;
+  constexpr int REC = McShape<DIM>::REC;
+  __shared__ __attribute__((aligned(16))) uint4 ring[kBinRing][kBinTile];
+  __shared__ uint32_t queue[kBinRing][kBinMcBlock];
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int tid = lane;
+  const int half = lane >> 5;
+  const int col = lane & 31;
+  const int task = blockIdx.x;
+  if (task >= p.wave_start[p.num_segments])
+    return;
+  const int seg = find_segment(p.wave_start, p.num_segments, task);
+  const int x_begin = p.ptr_x ? (int)p.ptr_x[seg] : 0;
+  const int x_end = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
+  const int y_begin = p.ptr_y ? (int)p.ptr_y[seg] : 0;
+  const int y_end = p.ptr_y ? (int)p.ptr_y[seg + 1] : p.m;
+  const int jq = y_begin + (task - p.wave_start[seg]) * 32 + col;
+  const bool valid = jq < y_end;
+  const int q = valid ? (int)p.perm_y[jq] : 0;
+  const int slots = p.k;
+  const int d_in = p.d;
+
+  float yq[DIM];
+#pragma unroll
+  for (int c = 0; c < DIM; ++c)
+    yq[c] = (valid && c < d_in) ? p.y[(size_t)q * d_in + c] : 0.0f;
+  // (a coordinate that is not finite: no distance below r2)
+  const bool searching = valid && __builtin_fabsf(yq[0]) < __builtin_inff() &&
+                         __builtin_fabsf(yq[1]) < __builtin_inff() &&
+                         __builtin_fabsf(yq[2]) < __builtin_inff();
+  float ysq = yq[0] * yq[0];
+#pragma unroll
+  for (int c = 1; c < DIM; ++c)
+    ysq = __builtin_fmaf(yq[c], yq[c], ysq);
+  const bool y_moderate = ysq <= kFilterNormLimit;
+
+  float q_lo[3], q_hi[3];
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    float lo = searching ? yq[c] : __builtin_inff();
+    float hi = searching ? yq[c] : -__builtin_inff();
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1) {
+      lo = __builtin_fminf(lo, __shfl_xor(lo, sh));
+      hi = __builtin_fmaxf(hi, __shfl_xor(hi, sh));
+    }
+    q_lo[c] = lo;
+    q_hi[c] = hi;
+  }
+
+  // the query operand with -cut for the fixed bound r2 in place (see
+  // knn_binned_mc_kernel); a lane that does not search passes nothing
+  mc_bf16x8_t yb;
+  {
+    uint32_t part[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float v = 0.0f;
+      if (e < DIM)
+        v = (searching && y_moderate) ? -2.0f * yq[e] : 0.0f;
+      else
+        v = searching ? 1.0f : 0.0f;
+      uint32_t hi, lo;
+      mc_split(v, hi, lo);
+      part[e] = half ? lo : hi;
+    }
+    const uint32_t w0 = part[0] | (part[1] << 16);
+    const uint32_t w1 = part[2] | (part[3] << 16);
+    uint4 b = make_uint4(w0, w1, w0, w1);
+    if (half) {
+      const float cut =
+          searching ? mc_filter_cut(r2, mc_damped_norm(ysq)) : -1e38f;
+      float neg = -__builtin_fmaf(__builtin_fabsf(cut), 3.0517578125e-05f, cut);
+      uint32_t hi, lo;
+      if (__builtin_fabsf(neg) < 1e38f) {
+        mc_split(neg, hi, lo);
+      } else {
+        hi = neg < 0.0f ? 0xff7fu : 0x7f7fu;
+        lo = 0;
+      }
+      b.y = (b.y & 0x0000ffffu) | (hi << 16);
+      b.w = (b.w & 0x0000ffffu) | (lo << 16);
+    }
+    yb = __builtin_bit_cast(mc_bf16x8_t, b);
+  }
+  const uint32_t one_keep = half ? ~(0xffffu << 16) : 0xffffffffu;
+  const uint32_t one_bits = half ? (0x3f80u << 16) : 0u;
+
+  double best[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j)
+    best[j] = (j < K - slots) ? -__builtin_inf() : __builtin_inf();
+  // rows with a number below `below` can still get in: all while neither of
+  // the query's two lists is full, those under the smaller of their largest
+  // numbers afterwards
+  uint32_t below = searching ? 0xffffffffu : 0u;
+  const uint32_t self = ignore_same_index ? (uint32_t)q : 0xffffffffu;
+  const float limit = searching ? r2 : -__builtin_inff();
+  int qn = 0;
+  int scanned = 0;
+
+  auto drain = [&]() {
+    bool changed = false;
+    int taken = 0;
+    uint32_t pending = 0;
+    int slot_base = 0;
+    for (;;) {
+      if (pending == 0 && taken < qn) {
+        const uint32_t word = queue[taken][tid];
+        ++taken;
+        pending = word & 0xffffu;
+        slot_base = (int)(word >> 16) * kBinTile + 4 * half;
+      }
+      const bool has = pending != 0;
+      if (!__any(has))
+        break;
+      const int bit = 31 - __builtin_clz(has ? pending : 1u);
+      const int v = 15 - bit;
+      pending &= ~(1u << bit);
+      const int j = has ? slot_base + 2 * (v & 12) + (v & 3) : 0;
+      const uint4 r4 = (&ring[0][0])[j];
+      const float d0 = __uint_as_float(r4.x) - yq[0];
+      float d = d0 * d0;
+      const float d1 = __uint_as_float(r4.y) - yq[1];
+      d = __builtin_fmaf(d1, d1, d);
+      const float d2 = __uint_as_float(r4.z) - yq[2];
+      d = __builtin_fmaf(d2, d2, d);
+      const bool ok = has && d < limit && r4.w < below && r4.w != self;
+      if (!__any(ok))
+        continue;
+      sorted_insert<K>(best, ok ? (double)r4.w : __builtin_inf());
+      if (searching && best[K - 1] < __builtin_inf())
+        below = min(below, (uint32_t)best[K - 1]);
+      changed = true;
+    }
+    qn = 0;
+    if (!changed)
+      return;
+    // the partner's list bounds the query's final largest number as well
+    const auto both = __builtin_amdgcn_permlane32_swap(below, below, false,
+                                                       false);
+    below = min(below, half ? both[0] : both[1]);
+  };
+
+  struct Fetched {
+    uint4 operand, coords;
+  };
+  auto fetch = [&](int tile) {
+    const size_t j = (size_t)(x_begin + tile * kBinTile + col);
+    Fetched f;
+    f.operand = p.packed[j * REC];
+    f.coords = half ? make_uint4(0u, 0u, 0u, 0u) : p.packed[j * REC + 1];
+    return f;
+  };
+  auto scan = [&](int tile, const Fetched &f) {
+    const int slot = scanned % kBinRing;
+    if (!half)
+      ring[slot][col] = f.coords;
+    uint4 a = f.operand;
+    a.y = (a.y & one_keep) | one_bits;
+    a.w = (a.w & one_keep) | one_bits;
+    mfma_acc_t acc = {0};
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+        __builtin_bit_cast(mc_bf16x8_t, a), yb, acc, 0, 0, 0);
+    uint32_t mask = 0;
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      mask = __builtin_amdgcn_alignbit(mask, __float_as_uint(acc[v]), 31);
+    const int rows = min(kBinTile, x_end - (x_begin + tile * kBinTile));
+    if (rows < kBinTile) {
+      uint32_t real = 0;
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        real |= (8 * (v / 4) + 4 * half + v % 4 < rows) ? (1u << (15 - v)) : 0u;
+      mask &= real;
+    }
+    if (mask != 0) {
+      queue[qn][tid] = ((uint32_t)slot << 16) | mask;
+      ++qn;
+    }
+    ++scanned;
+    if (scanned % kBinRing == 0)
+      drain();
+  };
+
+  // is the box of lane `src` closer than the radius to the query of some
+  // lane that could still use one of its rows (a full list takes only smaller
+  // row numbers than it holds)?  (A NaN - from an infinite or empty box -
+  // never rules a box out.)
+  auto reachable = [&](const Box &held, int src) {
+    float lo[3], hi[3];
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      lo[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+          (int)__float_as_uint(held.lo[c]), src));
+      hi[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+          (int)__float_as_uint(held.hi[c]), src));
+    }
+    const uint32_t min_row =
+        (uint32_t)__builtin_amdgcn_readlane((int)held.min_row, src);
+    return __any(searching && min_row < below &&
+                 !(box_gap2(lo, hi, yq, yq) >= r2));
+  };
+  // largest row number any of the wave's queries could still take
+  auto wave_below = [&]() {
+    uint32_t b = below;
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1)
+      b = max(b, (uint32_t)__shfl_xor((int)b, sh));
+    return b;
+  };
+
+  const int tile0 = p.tile_start[seg];
+  const int num_tiles = p.tile_start[seg + 1] - tile0;
+  const int group0 = p.group_start[seg];
+  const int num_groups = (num_tiles + kBinGroup - 1) / kBinGroup;
+  uint32_t any_below = 0xffffffffu;
+  if (__any(searching)) {
+    for (int g_base = 0; g_base < num_groups; g_base += kWave) {
+      const int g_mine = g_base + lane;
+      Box g_box = {};
+      if (g_mine < num_groups)
+        g_box = p.group_box[group0 + g_mine];
+      uint64_t g_todo =
+          __ballot(g_mine < num_groups &&
+                   !(box_gap2(g_box.lo, g_box.hi, q_lo, q_hi) >= r2));
+      while (g_todo != 0) {
+        const int g_lane = (int)__builtin_ctzll(g_todo);
+        g_todo &= g_todo - 1;
+        if (!reachable(g_box, g_lane))
+          continue;
+        const int group = g_base + g_lane;
+        const int t_mine = group * kBinGroup + lane;
+        Box t_box = {};
+        if (t_mine < num_tiles)
+          t_box = p.box[tile0 + t_mine];
+        uint64_t t_todo =
+            __ballot(t_mine < num_tiles && t_box.min_row < any_below &&
+                     !(box_gap2(t_box.lo, t_box.hi, q_lo, q_hi) >= r2));
+        uint64_t t_pass = 0;
+        while (t_todo != 0) {
+          const int t_lane = (int)__builtin_ctzll(t_todo);
+          t_todo &= t_todo - 1;
+          if (reachable(t_box, t_lane))
+            t_pass |= (uint64_t)1 << t_lane;
+        }
+        if (t_pass != 0) {
+          Fetched next = fetch(group * kBinGroup + (int)__builtin_ctzll(t_pass));
+          while (t_pass != 0) {
+            const int t_lane = (int)__builtin_ctzll(t_pass);
+            t_pass &= t_pass - 1;
+            const Fetched cur = next;
+            if (t_pass != 0)
+              next =
+                  fetch(group * kBinGroup + (int)__builtin_ctzll(t_pass));
+            scan(group * kBinGroup + t_lane, cur);
+          }
+          if (__any(qn > 0))
+            drain();
+          any_below = wave_below();
+        }
+      }
+    }
+    drain();
+  }
+
+  // unite the two half lists of each query in the lower lane
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    if (j < K - slots)
+      continue;
+    const auto hi = __builtin_amdgcn_permlane32_swap(
+        (unsigned)__double2hiint(best[j]), (unsigned)__double2hiint(best[j]),
+        false, false);
+    const auto lo = __builtin_amdgcn_permlane32_swap(
+        (unsigned)__double2loint(best[j]), (unsigned)__double2loint(best[j]),
+        false, false);
+    const double upper = __hiloint2double((int)hi[1], (int)lo[1]);
+    sorted_insert<K>(best, half ? __builtin_inf() : upper);
+  }
+  if (half == 0 && valid) {
+    const size_t row = (size_t)q * slots;
+    int found = 0;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      const int e = j - (K - slots);
+      if (e >= 0 && best[j] < __builtin_inf()) {
+        p.out_idx[row + e] = (int)best[j];
+        ++found;
+      }
+    }
+    p.out_count[q] = found;
+  }
 }
 
 } // namespace pca

@@ -15,6 +15,14 @@ from pytorch_cluster_amd import capi, testing  # noqa: E402
 from gpu_common import DEV, dev, ragged_ptrs  # noqa: E402
 
 
+@pytest.fixture(autouse=True, params=["1", "0"],
+                ids=["matrix_cores", "vector_alu"])
+def scan_kind(request, monkeypatch):
+    # both scans of a tile, whichever is the default
+    monkeypatch.setenv("PCA_RADIUS_BINNED_MATRIX_CORES", request.param)
+    return request.param
+
+
 def gpu_radius_binned(x, y, ptr_x, ptr_y, r, max_nn, ignore_same=False):
     e = capi.radius_edges(dev(x), dev(y), dev(ptr_x, torch.long),
                           dev(ptr_y, torch.long), r, max_nn, ignore_same,
