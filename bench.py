@@ -356,6 +356,21 @@ def main():
         result["config"]["strategy"] = args.strategy
         result["roofline"] = None
         result["search_ms"] = kernel_s * 1e3
+    if not binned:
+        # the same steps with the binned search (same edges; the library's
+        # default stays the scan, which the roofline figure is about)
+        pca.set_search_strategy("binned")
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        result["with_binned_strategy"] = {
+            "value": m * args.steps / dt, "unit": "queries/s",
+            "ms_per_step": dt / args.steps * 1e3}
     pca.set_search_strategy("scan")
     if not args.no_extras:
         result["other_configs"] = other_configs(torch, pca, testing, dev)
