@@ -239,6 +239,23 @@ int pca_nearest(const void *x, const void *y, const int64_t *ptr_x,
                 int64_t num_segments, int dtype, int64_t *out,
                 void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * pca_nearest for fp32 points of up to 3 dimensions (PCA_ERR_UNSUPPORTED
+ * otherwise) over spatially binned rows of y, as pca_knn_binned bins the rows
+ * of x: every row of x looks only at rows of y near it.  Stands under the same
+ * operator as pca_nearest (csrc/nearest.cpp:22-36 ->
+ * csrc/cuda/nearest_cuda.cu:68-94) and returns the same rows, the reference's
+ * order among equal distances included.  Arguments as for pca_nearest, without
+ * dtype.
+ */
+size_t pca_nearest_binned_workspace_bytes(int64_t n, int64_t m, int64_t d,
+                                          int64_t num_segments);
+
+int pca_nearest_binned(const void *x, const void *y, const int64_t *ptr_x,
+                       const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+                       int64_t num_segments, int64_t *out, void *workspace,
+                       size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------ fps -- */
 
 /*

@@ -64,6 +64,11 @@ C_ABI = {
     "pca_nearest": (ctypes.c_int,
                     [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_int,
                      _vp, _vp, ctypes.c_size_t, _vp]),
+    "pca_nearest_binned_workspace_bytes": (ctypes.c_size_t,
+                                           [_i64, _i64, _i64, _i64]),
+    "pca_nearest_binned": (ctypes.c_int,
+                           [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp,
+                            _vp, ctypes.c_size_t, _vp]),
     "pca_fps_workspace_bytes": (ctypes.c_size_t,
                                 [_i64, _i64, _i64, _i64, ctypes.c_int]),
     "pca_fps": (ctypes.c_int,

@@ -160,7 +160,8 @@ def radius_edges(x, y, ptr_x=None, ptr_y=None, r: float = 1.0,
     return edges[:2 * e].view(2, e)
 
 
-def nearest_launch(x, y, ptr_x=None, ptr_y=None, stream=None):
+def nearest_launch(x, y, ptr_x=None, ptr_y=None, stream=None,
+                   binned: bool = False):
     """Queues ``pca_nearest``: for every row of ``x`` the nearest row of ``y``
     of the same segment.  Returns (out [n] int64, workspace); nothing is
     synchronised."""
@@ -170,11 +171,21 @@ def nearest_launch(x, y, ptr_x=None, ptr_y=None, stream=None):
     n, d = x.shape
     m = y.shape[0]
     ptr_x, ptr_y, nseg = _segments(ptr_x, ptr_y)
-    ws_bytes = capi.pca_nearest_workspace_bytes(n, m, d, nseg, dtype)
+    if binned:
+        assert dtype == 0
+        ws_bytes = capi.pca_nearest_binned_workspace_bytes(n, m, d, nseg)
+    else:
+        ws_bytes = capi.pca_nearest_workspace_bytes(n, m, d, nseg, dtype)
     if ws_bytes == 0:
         ws_bytes = 256
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
     out = torch.empty(n, dtype=torch.long, device=x.device)
+    if binned:
+        _check(capi.pca_nearest_binned(
+            _dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x), _dev_ptr(ptr_y), n, m,
+            d, nseg, _dev_ptr(out), _dev_ptr(ws), ws_bytes,
+            _stream_handle(stream, x.device)))
+        return out, ws
     _check(capi.pca_nearest(_dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x),
                             _dev_ptr(ptr_y), n, m, d, nseg, dtype,
                             _dev_ptr(out), _dev_ptr(ws), ws_bytes,
@@ -182,8 +193,9 @@ def nearest_launch(x, y, ptr_x=None, ptr_y=None, stream=None):
     return out, ws
 
 
-def nearest_rows(x, y, ptr_x=None, ptr_y=None, stream=None) -> torch.Tensor:
-    return nearest_launch(x, y, ptr_x, ptr_y, stream)[0]
+def nearest_rows(x, y, ptr_x=None, ptr_y=None, stream=None,
+                 binned: bool = False) -> torch.Tensor:
+    return nearest_launch(x, y, ptr_x, ptr_y, stream, binned)[0]
 
 
 def fps_launch(src, ptr, out_ptr, num_samples: int, start=None,

@@ -772,6 +772,67 @@ int pca_nearest(const void *x, const void *y, const int64_t *ptr_x,
   return rc;
 }
 
+size_t pca_nearest_binned_workspace_bytes(int64_t n, int64_t m, int64_t d,
+                                          int64_t num_segments) {
+  if (num_segments < 1)
+    num_segments = 1;
+  if (!sizes_ok(n, m, d, num_segments) || n == 0 || m == 0 || d > 3)
+    return 0;
+  // (the searched rows, m of them, are the ones that get binned)
+  return align256(
+      pca::knn_binned_scratch_bytes((int)m, (int)n, (int)num_segments));
+}
+
+int pca_nearest_binned(const void *x, const void *y, const int64_t *ptr_x,
+                       const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+                       int64_t num_segments, int64_t *out, void *workspace,
+                       size_t workspace_bytes, void *stream_) {
+  g_last_error[0] = 0;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  SearchTimer timer(stream);
+  if ((ptr_x == nullptr) != (ptr_y == nullptr))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "ptr_x and ptr_y must both be given or both be NULL");
+  if (ptr_x == nullptr)
+    num_segments = 1;
+  if (!sizes_ok(n, m, d, num_segments))
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "bad sizes n=%lld m=%lld d=%lld num_segments=%lld",
+                (long long)n, (long long)m, (long long)d,
+                (long long)num_segments);
+  if (d > 3)
+    return fail(PCA_ERR_UNSUPPORTED,
+                "binned search: fp32 points of up to 3 dimensions, got d=%lld",
+                (long long)d);
+  if (n == 0)
+    return PCA_OK;
+  if (out == nullptr || x == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "x or out is NULL");
+  if (m == 0) {
+    // no candidate anywhere: every row keeps the reference's initial index
+    hipLaunchKernelGGL(fill_i64_kernel, dim3((unsigned)((n + 255) / 256)),
+                       dim3(256), 0, stream, out, n, (int64_t)0);
+    return check_launch(hipGetLastError(), "fill_i64_kernel");
+  }
+  if (y == nullptr)
+    return fail(PCA_ERR_INVALID_ARGUMENT, "y is NULL");
+  const size_t need = align256(
+      pca::knn_binned_scratch_bytes((int)m, (int)n, (int)num_segments));
+  if (workspace == nullptr || ((uintptr_t)workspace & 255) != 0 ||
+      workspace_bytes < need)
+    return fail(PCA_ERR_WORKSPACE, "workspace needs %zu bytes, 256-aligned",
+                need);
+  // the search kernels call the searched rows x and the searching rows y
+  pca::SearchInput in{y,      x,      ptr_y,  ptr_x,
+                      (int)m, (int)n, (int)d, (int)num_segments};
+  const int rc = check_launch(
+      pca::launch_nearest_binned(in, workspace, out, timer.start, timer.stop,
+                                 stream),
+      "binned search (nearest)");
+  timer.stop = nullptr;
+  return rc;
+}
+
 size_t pca_fps_workspace_bytes(int64_t n, int64_t d, int64_t num_segments,
                                int64_t max_segment_rows, int dtype) {
   if (n < 0 || n > kMaxRows || d < 1 || d > (1 << 20) || num_segments < 1 ||

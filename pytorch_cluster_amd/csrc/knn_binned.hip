@@ -914,6 +914,7 @@ void fill_params(BinnedParams &p, const SearchInput &in, const Bins &bins,
   p.out_idx = out.idx;
   p.out_dist = out.dist;
   p.out_count = out.count;
+  p.out_nearest = nullptr;
 }
 
 } // namespace
@@ -964,6 +965,29 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
   else
     PCA_BINNED_LAUNCH(32);
 #undef PCA_BINNED_LAUNCH
+  if (time_stop)
+    (void)hipEventRecord(time_stop, stream);
+  return hipGetLastError();
+}
+
+hipError_t launch_nearest_binned(const SearchInput &in, void *scratch,
+                                 int64_t *out, hipEvent_t time_start,
+                                 hipEvent_t time_stop, hipStream_t stream) {
+  if (time_start)
+    (void)hipEventRecord(time_start, stream);
+  Bins bins;
+  const hipError_t err = prepare_bins(in, scratch, bins, stream);
+  if (err != hipSuccess)
+    return err;
+  BinnedParams p;
+  const DenseResult none{nullptr, nullptr, nullptr, 1};
+  fill_params(p, in, bins, none);
+  p.k = 1;
+  p.out_nearest = out;
+  p.wave_start = bins.half_start;
+  const int waves = plan_upper_bound(in.m, in.num_segments, kWave / 2);
+  hipLaunchKernelGGL((knn_binned_mc_kernel<1, true>), dim3(waves),
+                     dim3(kBinMcBlock), 0, stream, p);
   if (time_stop)
     (void)hipEventRecord(time_stop, stream);
   return hipGetLastError();

@@ -54,6 +54,7 @@ struct BinnedParams {
   int *out_idx;
   float *out_dist;
   int *out_count;
+  int64_t *out_nearest; // the `nearest` search: [m] rows
 };
 
 // First position in [lo, hi) whose key is not below `key` (hi if none); the
@@ -108,14 +109,18 @@ __device__ __forceinline__ int nearest_bit(uint64_t mask, int at) {
 // length.
 constexpr int kBinMcBlock = kWave;
 
-// p.wave_start counts tasks of 32 queries.
-template <int K>
+// p.wave_start counts tasks of 32 queries.  NEAREST: the search of the
+// `nearest` operator - one neighbour, limit 1e38, the reference's order among
+// equal distances (device_utils.hpp) - whose result goes to p.out_nearest as
+// a row number (0 when nothing qualified).
+template <int K, bool NEAREST = false>
 __global__ __launch_bounds__(kBinMcBlock, K <= 16 ? 4 : 1) void
 knn_binned_mc_kernel(BinnedParams p) {
+  static_assert(!NEAREST || K == 1, "nearest keeps one neighbour");
   constexpr int DIM = 3;
   constexpr int REC = McShape<DIM>::REC; // operand quad, coordinate quad
   static_assert(McShape<DIM>::NI == 1 && REC == 2, "one instruction per tile");
-  constexpr float kLimit = kKnnSentinel;
+  constexpr float kLimit = SearchLimit<NEAREST>::value;
   constexpr int kWaves = kBinMcBlock / kWave;
 
   // coordinates and row numbers of the last kBinRing tiles of every wave
@@ -199,7 +204,7 @@ knn_binned_mc_kernel(BinnedParams p) {
   double best[K];
 #pragma unroll
   for (int j = 0; j < K; ++j)
-    best[j] = (j < K - k) ? lowest_key() : empty_key();
+    best[j] = (j < K - k) ? lowest_key() : SearchLimit<NEAREST>::empty();
   // exact distances must be strictly below thresh: the limit, or just above
   // the smaller of this lane's and the query's k-th distance (equality still
   // passes); a lane that does not search accepts nothing
@@ -298,7 +303,10 @@ knn_binned_mc_kernel(BinnedParams p) {
       const bool ok = has && d < thresh;
       if (!__any(ok))
         continue;
-      const double key = ok ? make_key(d, r4.w) : empty_key();
+      const uint32_t row_id =
+          NEAREST ? nearest_tie(r4.w - (uint32_t)x_begin) : r4.w;
+      const double key =
+          ok ? make_key(d, row_id) : SearchLimit<NEAREST>::empty();
       sorted_insert<K>(best, key);
       float own_bound = key_dist(best[K - 1]);
       // (a row of EQUAL distance and smaller number can still get in)
@@ -495,10 +503,14 @@ knn_binned_mc_kernel(BinnedParams p) {
         (unsigned)__double2loint(best[j]), (unsigned)__double2loint(best[j]),
         false, false);
     const double upper = __hiloint2double((int)hi[1], (int)lo[1]);
-    sorted_insert<K>(best, half ? empty_key() : upper);
+    sorted_insert<K>(best, half ? SearchLimit<NEAREST>::empty() : upper);
   }
-  if (half == 0 && valid)
-    write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+  if (half == 0 && valid) {
+    if constexpr (NEAREST)
+      write_nearest(best[0], q, x_begin, p.out_nearest);
+    else
+      write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+  }
 }
 
 // The binned radius search with the same scan (reference: radius_kernel,

@@ -91,6 +91,13 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
                              const DenseResult &out, hipEvent_t time_start,
                              hipEvent_t time_stop, hipStream_t stream);
 
+// The `nearest` search over the same bins (fp32, up to 3 dimensions): in.x
+// are the candidates, in.y the rows that look for their nearest candidate;
+// out [in.m] receives the rows.  The events bracket binning and search.
+hipError_t launch_nearest_binned(const SearchInput &in, void *scratch,
+                                 int64_t *out, hipEvent_t time_start,
+                                 hipEvent_t time_stop, hipStream_t stream);
+
 // The radius search over the same bins: fp32 points of up to 3 dimensions,
 // up to 32 slots per query (out.slots; out.dist unused).
 bool radius_binned_supported(int d, int slots);

@@ -349,12 +349,23 @@ at::Tensor nearest(at::Tensor x, at::Tensor y, at::Tensor ptr_x,
   const int dtype = dtype_code(x);
   TORCH_CHECK(dtype != PCA_BF16,
               "nearest is not implemented for 'BFloat16'");
+  // (the searched rows, y, are the ones a binned search orders)
+  const bool binned =
+      bins_wanted(m, segments) && dtype == PCA_F32 && d <= 3 && m > 0;
   const size_t ws_bytes =
-      pca_nearest_workspace_bytes(n, m, d, segments, dtype);
+      binned ? pca_nearest_binned_workspace_bytes(n, m, d, segments)
+             : pca_nearest_workspace_bytes(n, m, d, segments, dtype);
   TORCH_CHECK(ws_bytes > 0, "problem size not supported");
   auto workspace =
       at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
   hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
+  if (binned) {
+    check_status(pca_nearest_binned(
+        x.data_ptr(), y.data_ptr(), px.data_ptr<int64_t>(),
+        py.data_ptr<int64_t>(), n, m, d, segments, out.data_ptr<int64_t>(),
+        workspace.data_ptr(), ws_bytes, stream));
+    return out;
+  }
   check_status(pca_nearest(x.data_ptr(), m > 0 ? y.data_ptr() : nullptr,
                            px.data_ptr<int64_t>(), py.data_ptr<int64_t>(), n,
                            m, d, segments, dtype, out.data_ptr<int64_t>(),
