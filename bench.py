@@ -217,6 +217,18 @@ def other_configs(torch, pca, testing, dev):
             report["%s, strategy %s" % (name, strategy)] = {
                 "ms": ms, "queries_per_s": queries / ms * 1e3,
                 "search_ms": search_ms, "edges": int(out.shape[1])}
+    # nearest on the LiDAR-like points again, through both strategies
+    lidar8 = testing.lidar_scans(0, query_stride=8)
+    nx, ny = lidar8["x"].to(dev), lidar8["y"].to(dev)
+    nbx, nby = lidar8["batch_x"].to(dev), lidar8["batch_y"].to(dev)
+    for strategy in ("scan", "binned"):
+        pca.set_search_strategy(strategy)
+        try:
+            ms, out = median_ms(lambda: pca.nearest(nx, ny, nbx, nby), 5)
+        finally:
+            pca.set_search_strategy("scan")
+        report["nearest on the LiDAR-like points, strategy %s" % strategy] = {
+            "ms": ms, "rows_per_s": nx.shape[0] / ms * 1e3}
     return report
 
 
