@@ -704,12 +704,12 @@ __global__ __launch_bounds__(kBlock) void radius_binned_kernel(
 struct BinnedLayout {
   size_t seg_box, keys_a, keys_x, keys_y, vals_a, perm_x, perm_y, rows, packed,
       box, group_box, tile_start, group_start, wave_start, half_start,
-      sort_temp;
+      task_keys, sort_temp;
   int tiles_bound, groups_bound;
   size_t total() const {
     return seg_box + keys_a + keys_x + keys_y + vals_a + perm_x + perm_y +
            rows + packed + box + group_box + tile_start + group_start +
-           wave_start + half_start + sort_temp;
+           wave_start + half_start + task_keys + sort_temp;
   }
 };
 
@@ -764,6 +764,9 @@ BinnedLayout binned_layout(int n, int m, int num_segments) {
   w.group_start = align256(sizeof(int) * (size_t)(num_segments + 1));
   w.wave_start = align256(sizeof(int) * (size_t)(num_segments + 1));
   w.half_start = align256(sizeof(int) * (size_t)(num_segments + 1));
+  // span keys and task numbers, unsorted and sorted
+  w.task_keys = align256(sizeof(uint32_t) * 4 *
+                         (size_t)plan_upper_bound(m, num_segments, kWave / 2));
   size_t tx = 0, ty = 0;
   const hipError_t ex = sort_pairs(nullptr, tx, nullptr, nullptr, nullptr,
                                    nullptr, n, num_segments, nullptr);
@@ -781,6 +784,9 @@ struct Bins {
   const int *tile_start, *group_start;
   const int *wave_start; // tasks of 64 queries
   const int *half_start; // tasks of 32 queries
+  uint32_t *task_keys;   // 4 arrays of a word per task of 32 queries
+  void *sort_temp;
+  size_t sort_bytes;
   const uint32_t *keys_x, *keys_y, *perm_y;
   const float4 *rows;
   const uint4 *packed;
@@ -812,6 +818,7 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
   int *group_start = static_cast<int *>(take(lay.group_start));
   int *wave_start = static_cast<int *>(take(lay.wave_start));
   int *half_start = static_cast<int *>(take(lay.half_start));
+  uint32_t *task_keys = static_cast<uint32_t *>(take(lay.task_keys));
   void *sort_temp = take(lay.sort_temp);
   size_t sort_bytes = lay.sort_temp;
 
@@ -882,6 +889,9 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
   bins.group_start = group_start;
   bins.wave_start = wave_start;
   bins.half_start = half_start;
+  bins.task_keys = task_keys;
+  bins.sort_temp = sort_temp;
+  bins.sort_bytes = lay.sort_temp;
   bins.keys_x = keys_x;
   bins.keys_y = keys_y;
   bins.perm_y = perm_y;
@@ -915,9 +925,27 @@ void fill_params(BinnedParams &p, const SearchInput &in, const Bins &bins,
   p.out_dist = out.dist;
   p.out_count = out.count;
   p.out_nearest = nullptr;
+  p.task_order = nullptr;
 }
 
 } // namespace
+
+// p.wave_start = tasks of 32 queries; leaves p.task_order set.
+hipError_t order_tasks(BinnedParams &p, const Bins &bins, int waves,
+                       hipStream_t stream) {
+  uint32_t *keys_in = bins.task_keys;
+  uint32_t *vals_in = keys_in + waves;
+  uint32_t *keys_out = vals_in + waves;
+  uint32_t *vals_out = keys_out + waves;
+  hipLaunchKernelGGL(task_span_kernel, dim3((waves + kBlock - 1) / kBlock),
+                     dim3(kBlock), 0, stream, p, waves, keys_in, vals_in);
+  size_t bytes = bins.sort_bytes;
+  const hipError_t err = rocprim::radix_sort_pairs(
+      bins.sort_temp, bytes, keys_in, keys_out, vals_in, vals_out,
+      (unsigned int)waves, 0u, 32u, stream, false);
+  p.task_order = vals_out;
+  return err;
+}
 
 bool knn_binned_supported(int d, int k, bool cosine) {
   return !cosine && d >= 1 && d <= 3 && k >= 1 && k <= 32;
@@ -947,6 +975,11 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
     p.wave_start = bins.half_start;
   const int waves = plan_upper_bound(in.m, in.num_segments, per_task);
   const int grid = (waves + kBlock / kWave - 1) / (kBlock / kWave);
+  if (matrix_cores) {
+    const hipError_t order_err = order_tasks(p, bins, waves, stream);
+    if (order_err != hipSuccess)
+      return order_err;
+  }
 #define PCA_BINNED_LAUNCH(K_)                                                  \
   do {                                                                         \
     if (matrix_cores)                                                          \
@@ -986,6 +1019,9 @@ hipError_t launch_nearest_binned(const SearchInput &in, void *scratch,
   p.out_nearest = out;
   p.wave_start = bins.half_start;
   const int waves = plan_upper_bound(in.m, in.num_segments, kWave / 2);
+  const hipError_t order_err = order_tasks(p, bins, waves, stream);
+  if (order_err != hipSuccess)
+    return order_err;
   hipLaunchKernelGGL((knn_binned_mc_kernel<1, true>), dim3(waves),
                      dim3(kBinMcBlock), 0, stream, p);
   if (time_stop)

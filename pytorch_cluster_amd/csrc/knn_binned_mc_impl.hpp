@@ -48,6 +48,7 @@ struct BinnedParams {
   const float4 *rows;       // x rows in curve order, .w = row number
   const uint4 *packed;      // the same rows as mc_pack_row<3> leaves them,
                             // the fourth coordinate word = row number
+  const uint32_t *task_order; // tasks of 32 queries, the longest first
   const Box *box;           // of every tile
   const int *group_start;   // first group of tiles of every segment
   const Box *group_box;     // of every group
@@ -104,6 +105,31 @@ __device__ __forceinline__ int nearest_bit(uint64_t mask, int at) {
   return d_up <= d_down ? at + d_up : at - d_down;
 }
 
+// Sort key of a task of 32 queries for the order in which the tasks start:
+// the complement of the span of its queries' curve keys.  Where the points
+// are sparse 32 consecutive queries span a long piece of the curve, their
+// neighbours are far apart, and the task looks at many more boxes and tiles
+// than a task in a dense region; started last, such tasks would be the tail
+// of the launch.
+__global__ __launch_bounds__(kBlock) void task_span_kernel(
+    BinnedParams p, int bound, uint32_t *__restrict__ keys,
+    uint32_t *__restrict__ vals) {
+  const int task = blockIdx.x * kBlock + threadIdx.x;
+  if (task >= bound)
+    return;
+  uint32_t key = 0xffffffffu; // (no such task: sorts last, leaves at once)
+  if (task < p.wave_start[p.num_segments]) {
+    const int seg = find_segment(p.wave_start, p.num_segments, task);
+    const int y_begin = p.ptr_y ? (int)p.ptr_y[seg] : 0;
+    const int y_end = p.ptr_y ? (int)p.ptr_y[seg + 1] : p.m;
+    const int jq0 = y_begin + (task - p.wave_start[seg]) * 32;
+    const int last = min(32, y_end - jq0) - 1;
+    key = ~(p.keys_y[jq0 + last] - p.keys_y[jq0]);
+  }
+  keys[task] = key;
+  vals[task] = (uint32_t)task;
+}
+
 // Waves work on their own (no barrier): a workgroup is one wave, so that its
 // place on the SIMD frees up the moment it is done - the tasks differ a lot in
 // length.
@@ -133,7 +159,7 @@ knn_binned_mc_kernel(BinnedParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int half = lane >> 5;
   const int col = lane & 31;
-  const int task = blockIdx.x * kWaves + wave;
+  const int task = (int)p.task_order[blockIdx.x * kWaves + wave];
   if (task >= p.wave_start[p.num_segments])
     return; // (whole waves leave; no barrier below)
   const int seg = find_segment(p.wave_start, p.num_segments, task);
