@@ -240,3 +240,17 @@ def test_many_small_segments(oracle):
     x = rng.random((ptr_x[-1], 3)).astype(np.float32)
     y = rng.random((ptr_y[-1], 3)).astype(np.float32)
     check(oracle, x, y, ptr_x, ptr_y, 6)
+
+
+def test_three_million_rows_against_the_scanning_kernels(scan_kind):
+    """One large segment (positions and tile numbers far beyond 16 bits) and
+    coordinates with a large common offset."""
+    if scan_kind == "0":
+        pytest.skip("one scan kind is enough at this size")
+    g = torch.Generator().manual_seed(12)
+    x = (torch.rand(3000000, 3, generator=g) * 100.0 + 5000.0).to(DEV)
+    y = x[::37].contiguous()
+    a, da = capi.knn_edges(x, y, None, None, 8, want_dist=True)
+    b, db = capi.knn_edges(x, y, None, None, 8, want_dist=True, binned=True)
+    assert torch.equal(a, b)
+    assert torch.equal(da.view(torch.int32), db.view(torch.int32))
