@@ -452,6 +452,19 @@ knn_binned_mc_kernel(BinnedParams p) {
       return __any(searching && !(box_gap2(lo, hi, yq, yq) >= thresh));
     };
 
+    // the same for the boxes of lanes `a` (tested by lanes 0-31) and `b`
+    // (lanes 32-63) at once: the ballot of the lanes whose query reaches
+    auto reachable_pair = [&](const Box &held, int a, int b) {
+      const int src = half ? b : a;
+      float lo[3], hi[3];
+#pragma unroll
+      for (int c = 0; c < 3; ++c) {
+        lo[c] = __shfl(held.lo[c], src);
+        hi[c] = __shfl(held.hi[c], src);
+      }
+      return __ballot(searching && !(box_gap2(lo, hi, yq, yq) >= thresh));
+    };
+
     // Groups of tiles, 64 at a time (one box per lane), nearest to the seed
     // tiles first; a group, then a tile, is looked into if its box is within
     // the wave's largest bound of the box around the wave's queries, and then
@@ -491,10 +504,18 @@ knn_binned_mc_kernel(BinnedParams p) {
         // now; their rows are fetched one tile ahead of the scan
         uint64_t t_pass = 0;
         while (t_todo != 0) {
-          const int t_lane = (int)__builtin_ctzll(t_todo);
+          // two boxes per step: the two halves of the wave hold the same 32
+          // queries, so the lower half tests one box and the upper half the
+          // next (a lone last box is tested by both)
+          const int t_a = (int)__builtin_ctzll(t_todo);
           t_todo &= t_todo - 1;
-          if (reachable(t_box, t_lane))
-            t_pass |= (uint64_t)1 << t_lane;
+          const int t_b = t_todo != 0 ? (int)__builtin_ctzll(t_todo) : t_a;
+          t_todo &= t_todo - 1;
+          const uint64_t both = reachable_pair(t_box, t_a, t_b);
+          if (both & 0xffffffffull)
+            t_pass |= (uint64_t)1 << t_a;
+          if (both >> 32)
+            t_pass |= (uint64_t)1 << t_b;
         }
         if (t_pass != 0) {
           Fetched next = fetch(group * kBinGroup + (int)__builtin_ctzll(t_pass));
