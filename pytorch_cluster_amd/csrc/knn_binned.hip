@@ -743,6 +743,16 @@ hipError_t sort_pairs(void *temp, size_t &temp_bytes, const uint32_t *keys_in,
                                    false);
 }
 
+// Task slots for `blocks` blocks of 32 queries: one each, and half as many
+// again for the parts of split blocks - while the blocks are not many more
+// than the waves the device holds at once (256 CUs x 4 SIMDs x 4 waves).  With
+// several rounds of waves the long tasks, started first, are covered by the
+// others, and splitting only adds work (measured: it gains 15-25 % up to
+// ~4,000 blocks and loses 5 % at 8,000).
+int task_slots(int blocks) {
+  return blocks <= 6144 ? blocks + (blocks / 6) * 3 : blocks;
+}
+
 BinnedLayout binned_layout(int n, int m, int num_segments) {
   BinnedLayout w;
   const size_t big = (size_t)std::max(n, m);
@@ -764,18 +774,28 @@ BinnedLayout binned_layout(int n, int m, int num_segments) {
   w.group_start = align256(sizeof(int) * (size_t)(num_segments + 1));
   w.wave_start = align256(sizeof(int) * (size_t)(num_segments + 1));
   w.half_start = align256(sizeof(int) * (size_t)(num_segments + 1));
-  // span keys and task numbers, unsorted and sorted
-  w.task_keys = align256(sizeof(uint32_t) * 4 *
-                         (size_t)plan_upper_bound(m, num_segments, kWave / 2));
-  size_t tx = 0, ty = 0;
+  // per task slot: descriptor (2 words), span key and slot number, unsorted
+  // and sorted (4 words)
+  w.task_keys = align256(
+      sizeof(uint32_t) *
+      (6 * (size_t)task_slots(plan_upper_bound(m, num_segments, kWave / 2)) +
+       64));
+  size_t tx = 0, ty = 0, tt = 0;
   const hipError_t ex = sort_pairs(nullptr, tx, nullptr, nullptr, nullptr,
                                    nullptr, n, num_segments, nullptr);
   const hipError_t ey = sort_pairs(nullptr, ty, nullptr, nullptr, nullptr,
                                    nullptr, m, num_segments, nullptr);
+  // (the task slots, sorted on all 32 bits by order_tasks)
+  const hipError_t et = rocprim::radix_sort_pairs(
+      nullptr, tt, (const uint32_t *)nullptr, (uint32_t *)nullptr,
+      (const uint32_t *)nullptr, (uint32_t *)nullptr,
+      (unsigned int)task_slots(plan_upper_bound(m, num_segments, kWave / 2)),
+      0u, 32u, nullptr, false);
   // (a failed size query leaves a size no workspace can meet)
-  w.sort_temp = (ex == hipSuccess && ey == hipSuccess)
-                    ? align256(std::max(tx, ty))
-                    : ~(size_t)0 / 2;
+  w.sort_temp =
+      (ex == hipSuccess && ey == hipSuccess && et == hipSuccess)
+          ? align256(std::max(std::max(tx, ty), tt))
+          : ~(size_t)0 / 2;
   return w;
 }
 
@@ -784,7 +804,7 @@ struct Bins {
   const int *tile_start, *group_start;
   const int *wave_start; // tasks of 64 queries
   const int *half_start; // tasks of 32 queries
-  uint32_t *task_keys;   // 4 arrays of a word per task of 32 queries
+  uint32_t *task_keys;   // 6 words per task slot
   void *sort_temp;
   size_t sort_bytes;
   const uint32_t *keys_x, *keys_y, *perm_y;
@@ -926,23 +946,36 @@ void fill_params(BinnedParams &p, const SearchInput &in, const Bins &bins,
   p.out_count = out.count;
   p.out_nearest = nullptr;
   p.task_order = nullptr;
+  p.task_desc = nullptr;
+  p.code_bits = 0;
 }
 
 } // namespace
 
-// p.wave_start = tasks of 32 queries; leaves p.task_order set.
-hipError_t order_tasks(BinnedParams &p, const Bins &bins, int waves,
-                       hipStream_t stream) {
-  uint32_t *keys_in = bins.task_keys;
-  uint32_t *vals_in = keys_in + waves;
-  uint32_t *keys_out = vals_in + waves;
-  uint32_t *vals_out = keys_out + waves;
-  hipLaunchKernelGGL(task_span_kernel, dim3((waves + kBlock - 1) / kBlock),
-                     dim3(kBlock), 0, stream, p, waves, keys_in, vals_in);
+// p.wave_start = blocks of 32 queries (`blocks`: their upper bound); leaves
+// p.task_desc and p.task_order set and returns the number of task slots.
+hipError_t order_tasks(BinnedParams &p, const Bins &bins, int blocks,
+                       int num_segments, int &slots, hipStream_t stream) {
+  slots = task_slots(blocks);
+  const int extra = slots - blocks;
+  int *extra_used = reinterpret_cast<int *>(bins.task_keys);
+  int2 *desc = reinterpret_cast<int2 *>(bins.task_keys + 64);
+  uint32_t *keys_in = bins.task_keys + 64 + 2 * (size_t)slots;
+  uint32_t *vals_in = keys_in + slots;
+  uint32_t *keys_out = vals_in + slots;
+  uint32_t *vals_out = keys_out + slots;
+  p.code_bits = 3 * axis_bits(num_segments);
+  hipLaunchKernelGGL(task_slots_clear_kernel,
+                     dim3((extra + kBlock) / kBlock), dim3(kBlock), 0, stream,
+                     blocks, extra, extra_used, desc, keys_in, vals_in);
+  hipLaunchKernelGGL(task_span_kernel, dim3((blocks + kBlock - 1) / kBlock),
+                     dim3(kBlock), 0, stream, p, blocks, extra, extra_used,
+                     desc, keys_in, vals_in);
   size_t bytes = bins.sort_bytes;
   const hipError_t err = rocprim::radix_sort_pairs(
       bins.sort_temp, bytes, keys_in, keys_out, vals_in, vals_out,
-      (unsigned int)waves, 0u, 32u, stream, false);
+      (unsigned int)slots, 0u, 32u, stream, false);
+  p.task_desc = desc;
   p.task_order = vals_out;
   return err;
 }
@@ -975,15 +1008,17 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
     p.wave_start = bins.half_start;
   const int waves = plan_upper_bound(in.m, in.num_segments, per_task);
   const int grid = (waves + kBlock / kWave - 1) / (kBlock / kWave);
+  int slots = 0;
   if (matrix_cores) {
-    const hipError_t order_err = order_tasks(p, bins, waves, stream);
+    const hipError_t order_err =
+        order_tasks(p, bins, waves, in.num_segments, slots, stream);
     if (order_err != hipSuccess)
       return order_err;
   }
 #define PCA_BINNED_LAUNCH(K_)                                                  \
   do {                                                                         \
     if (matrix_cores)                                                          \
-      hipLaunchKernelGGL((knn_binned_mc_kernel<K_>), dim3(waves),              \
+      hipLaunchKernelGGL((knn_binned_mc_kernel<K_>), dim3(slots),              \
                          dim3(kBinMcBlock), 0, stream, p);                     \
     else                                                                       \
       hipLaunchKernelGGL((knn_binned_kernel<K_>), dim3(grid), dim3(kBlock), 0, \
@@ -1019,10 +1054,12 @@ hipError_t launch_nearest_binned(const SearchInput &in, void *scratch,
   p.out_nearest = out;
   p.wave_start = bins.half_start;
   const int waves = plan_upper_bound(in.m, in.num_segments, kWave / 2);
-  const hipError_t order_err = order_tasks(p, bins, waves, stream);
+  int slots = 0;
+  const hipError_t order_err =
+      order_tasks(p, bins, waves, in.num_segments, slots, stream);
   if (order_err != hipSuccess)
     return order_err;
-  hipLaunchKernelGGL((knn_binned_mc_kernel<1, true>), dim3(waves),
+  hipLaunchKernelGGL((knn_binned_mc_kernel<1, true>), dim3(slots),
                      dim3(kBinMcBlock), 0, stream, p);
   if (time_stop)
     (void)hipEventRecord(time_stop, stream);

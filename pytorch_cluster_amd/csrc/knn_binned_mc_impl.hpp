@@ -48,7 +48,9 @@ struct BinnedParams {
   const float4 *rows;       // x rows in curve order, .w = row number
   const uint4 *packed;      // the same rows as mc_pack_row<3> leaves them,
                             // the fourth coordinate word = row number
-  const uint32_t *task_order; // tasks of 32 queries, the longest first
+  const uint32_t *task_order; // task slots, the longest tasks first
+  const int2 *task_desc;      // per slot: first query position, queries
+  int code_bits;              // bits of the curve code inside a key
   const Box *box;           // of every tile
   const int *group_start;   // first group of tiles of every segment
   const Box *group_box;     // of every group
@@ -105,29 +107,68 @@ __device__ __forceinline__ int nearest_bit(uint64_t mask, int at) {
   return d_up <= d_down ? at + d_up : at - d_down;
 }
 
-// Sort key of a task of 32 queries for the order in which the tasks start:
-// the complement of the span of its queries' curve keys.  Where the points
-// are sparse 32 consecutive queries span a long piece of the curve, their
-// neighbours are far apart, and the task looks at many more boxes and tiles
-// than a task in a dense region; started last, such tasks would be the tail
-// of the launch.
+// Tasks of the matrix-core searches.  Normally a block of 32
+// curve-consecutive queries is one task (slot = block number).  A block whose
+// queries span much more of the curve than the segment's average lies where
+// the points are sparse: its queries are far apart, each with a neighbourhood
+// of its own, and one wave would look at several times as many boxes and
+// tiles as a wave in a dense region - the tail of the launch.  Such a block is
+// split into four tasks of 8 queries: its own slot and three extra slots
+// behind the blocks' ones, handed out by an atomic counter while they last
+// (`extra` slots; `*extra_used` starts at 0).  The sort key of a slot is the
+// complement of its span, so that the longest tasks start first and unused
+// extra slots come last (their waves leave at once).
 __global__ __launch_bounds__(kBlock) void task_span_kernel(
-    BinnedParams p, int bound, uint32_t *__restrict__ keys,
+    BinnedParams p, int bound, int extra, int *__restrict__ extra_used,
+    int2 *__restrict__ desc, uint32_t *__restrict__ keys,
     uint32_t *__restrict__ vals) {
-  const int task = blockIdx.x * kBlock + threadIdx.x;
-  if (task >= bound)
+  const int block = blockIdx.x * kBlock + threadIdx.x;
+  if (block >= bound)
     return;
-  uint32_t key = 0xffffffffu; // (no such task: sorts last, leaves at once)
-  if (task < p.wave_start[p.num_segments]) {
-    const int seg = find_segment(p.wave_start, p.num_segments, task);
+  int2 mine = make_int2(0, 0);
+  uint32_t key = 0xffffffffu;
+  if (block < p.wave_start[p.num_segments]) {
+    const int seg = find_segment(p.wave_start, p.num_segments, block);
     const int y_begin = p.ptr_y ? (int)p.ptr_y[seg] : 0;
     const int y_end = p.ptr_y ? (int)p.ptr_y[seg + 1] : p.m;
-    const int jq0 = y_begin + (task - p.wave_start[seg]) * 32;
-    const int last = min(32, y_end - jq0) - 1;
-    key = ~(p.keys_y[jq0 + last] - p.keys_y[jq0]);
+    const int jq0 = y_begin + (block - p.wave_start[seg]) * 32;
+    const int count = min(32, y_end - jq0);
+    const uint32_t span = p.keys_y[jq0 + count - 1] - p.keys_y[jq0];
+    const int blocks = p.wave_start[seg + 1] - p.wave_start[seg];
+    const uint64_t average = ((uint64_t)1 << p.code_bits) / (uint64_t)blocks;
+    mine = make_int2(jq0, count);
+    key = min(~span, 0xfffffffeu);
+    if (count == 32 && (uint64_t)span > 8 * average) {
+      const int at = atomicAdd(extra_used, 3);
+      if (at + 3 <= extra) {
+        mine = make_int2(jq0, 8);
+        key = min(~(span / 4), 0xfffffffeu);
+        for (int i = 0; i < 3; ++i) {
+          desc[bound + at + i] = make_int2(jq0 + 8 * (i + 1), 8);
+          keys[bound + at + i] = key;
+          vals[bound + at + i] = (uint32_t)(bound + at + i);
+        }
+      }
+    }
   }
-  keys[task] = key;
-  vals[task] = (uint32_t)task;
+  desc[block] = mine;
+  keys[block] = key;
+  vals[block] = (uint32_t)block;
+}
+
+// Extra slots start out unused (before task_span_kernel).
+__global__ __launch_bounds__(kBlock) void task_slots_clear_kernel(
+    int bound, int extra, int *__restrict__ extra_used,
+    int2 *__restrict__ desc, uint32_t *__restrict__ keys,
+    uint32_t *__restrict__ vals) {
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i == 0)
+    *extra_used = 0;
+  if (i < extra) {
+    desc[bound + i] = make_int2(0, 0);
+    keys[bound + i] = 0xffffffffu;
+    vals[bound + i] = (uint32_t)(bound + i);
+  }
 }
 
 // Waves work on their own (no barrier): a workgroup is one wave, so that its
@@ -135,7 +176,8 @@ __global__ __launch_bounds__(kBlock) void task_span_kernel(
 // length.
 constexpr int kBinMcBlock = kWave;
 
-// p.wave_start counts tasks of 32 queries.  NEAREST: the search of the
+// p.wave_start counts blocks of 32 queries, p.task_desc / p.task_order are
+// task_span_kernel's.  NEAREST: the search of the
 // `nearest` operator - one neighbour, limit 1e38, the reference's order among
 // equal distances (device_utils.hpp) - whose result goes to p.out_nearest as
 // a row number (0 when nothing qualified).
@@ -159,17 +201,28 @@ knn_binned_mc_kernel(BinnedParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int half = lane >> 5;
   const int col = lane & 31;
-  const int task = (int)p.task_order[blockIdx.x * kWaves + wave];
-  if (task >= p.wave_start[p.num_segments])
-    return; // (whole waves leave; no barrier below)
-  const int seg = find_segment(p.wave_start, p.num_segments, task);
+  const int slot = (int)p.task_order[blockIdx.x * kWaves + wave];
+  const int2 task = p.task_desc[slot]; // (first query position, queries)
+  if (task.y == 0)
+    return; // (an unused slot; whole waves leave, no barrier below)
+  // (the segment of the task's first query)
+  int seg = 0;
+  if (p.ptr_y) {
+    int lo = 0, hi = p.num_segments;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (p.ptr_y[mid] <= task.x)
+        lo = mid;
+      else
+        hi = mid;
+    }
+    seg = lo;
+  }
   const int x_begin = p.ptr_x ? (int)p.ptr_x[seg] : 0;
   const int x_end = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
-  const int y_begin = p.ptr_y ? (int)p.ptr_y[seg] : 0;
-  const int y_end = p.ptr_y ? (int)p.ptr_y[seg + 1] : p.m;
-  const int jq0 = y_begin + (task - p.wave_start[seg]) * 32;
+  const int jq0 = task.x;
   const int jq = jq0 + col;
-  const bool valid = jq < y_end;
+  const bool valid = col < task.y;
   const int q = valid ? (int)p.perm_y[jq] : 0;
   const int k = p.k;
   const int d_in = p.d;
@@ -409,7 +462,7 @@ knn_binned_mc_kernel(BinnedParams p) {
 
   if (num_tiles > 0) {
     // where the wave's first and last query fall in the order of x
-    const int last_col = min(32, y_end - jq0) - 1;
+    const int last_col = task.y - 1;
     const uint32_t key_first = p.keys_y[jq0];
     const uint32_t key_last = p.keys_y[jq0 + last_col];
     const int pos_first =
