@@ -107,6 +107,165 @@ __device__ __forceinline__ int nearest_bit(uint64_t mask, int at) {
   return d_up <= d_down ? at + d_up : at - d_down;
 }
 
+// ---- pieces shared by the matrix-core searches ------------------------------
+
+// A lane's query: coordinates (zero beyond d and for a lane without one),
+// whether it searches at all (a coordinate that is not finite has no distance
+// below any limit), its squared norm, and the box around the wave's searching
+// queries.
+struct BinQuery {
+  float y[3];
+  bool searching;
+  float ysq;
+  float lo[3], hi[3];
+};
+
+__device__ __forceinline__ BinQuery bin_load_query(const BinnedParams &p,
+                                                   bool valid, int q) {
+  BinQuery r;
+#pragma unroll
+  for (int c = 0; c < 3; ++c)
+    r.y[c] = (valid && c < p.d) ? p.y[(size_t)q * p.d + c] : 0.0f;
+  r.searching = valid && __builtin_fabsf(r.y[0]) < __builtin_inff() &&
+                __builtin_fabsf(r.y[1]) < __builtin_inff() &&
+                __builtin_fabsf(r.y[2]) < __builtin_inff();
+  r.ysq = r.y[0] * r.y[0];
+#pragma unroll
+  for (int c = 1; c < 3; ++c)
+    r.ysq = __builtin_fmaf(r.y[c], r.y[c], r.ysq);
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    float lo = r.searching ? r.y[c] : __builtin_inff();
+    float hi = r.searching ? r.y[c] : -__builtin_inff();
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1) {
+      lo = __builtin_fminf(lo, __shfl_xor(lo, sh));
+      hi = __builtin_fmaxf(hi, __shfl_xor(hi, sh));
+    }
+    r.lo[c] = lo;
+    r.hi[c] = hi;
+  }
+  return r;
+}
+
+// B operand of the filter without the cut: the hi (lanes 0-31) or lo (lanes
+// 32-63) parts of (-2 y_0, -2 y_1, -2 y_2, 1), given twice (against the hi
+// and the lo parts of the row); see knn_lowd_mc_impl.hpp.  A lane that does
+// not search multiplies everything by zero.
+__device__ __forceinline__ uint4 bin_query_operand(const BinQuery &q,
+                                                   int half) {
+  const bool moderate = q.ysq <= kFilterNormLimit;
+  uint32_t part[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float v = 0.0f;
+    if (e < 3)
+      v = (q.searching && moderate) ? -2.0f * q.y[e] : 0.0f;
+    else
+      v = q.searching ? 1.0f : 0.0f;
+    uint32_t hi, lo;
+    mc_split(v, hi, lo);
+    part[e] = half ? lo : hi;
+  }
+  const uint32_t w0 = part[0] | (part[1] << 16);
+  const uint32_t w1 = part[2] | (part[3] << 16);
+  return make_uint4(w0, w1, w0, w1);
+}
+
+// ... with -cut riding in the two accumulation slots of w that the zero lo
+// part of the query's 1 would leave unused (upper lanes, component 3 of the
+// one instruction): -cut' split, cut' = cut + 2^-15 |cut|, so that what the
+// split may lose never lowers the cut; an infinite cut (filter switched off)
+// enters as the largest finite bf16.
+__device__ __forceinline__ mc_bf16x8_t bin_operand_with_cut(uint4 plain,
+                                                            float cut,
+                                                            int half) {
+  if (half) {
+    float neg = -__builtin_fmaf(__builtin_fabsf(cut), 3.0517578125e-05f, cut);
+    uint32_t hi, lo;
+    if (__builtin_fabsf(neg) < 1e38f) {
+      mc_split(neg, hi, lo);
+    } else {
+      hi = neg < 0.0f ? 0xff7fu : 0x7f7fu;
+      lo = 0;
+    }
+    plain.y = (plain.y & 0x0000ffffu) | (hi << 16);
+    plain.w = (plain.w & 0x0000ffffu) | (lo << 16);
+  }
+  return __builtin_bit_cast(mc_bf16x8_t, plain);
+}
+
+// The rows of a tile as the lanes fetch them: the operand quad of row `col`
+// (both halves), the coordinate quad of row `col` (lower half).  (The packed
+// copy is padded by a tile of rows that never pass.)
+struct BinFetched {
+  uint4 operand, coords;
+};
+
+__device__ __forceinline__ BinFetched bin_fetch(const uint4 *__restrict__ packed,
+                                                int first_row, int col,
+                                                int half) {
+  const size_t j = (size_t)(first_row + col);
+  BinFetched f;
+  f.operand = packed[j * 2];
+  f.coords = half ? make_uint4(0u, 0u, 0u, 0u) : packed[j * 2 + 1];
+  return f;
+}
+
+// Sign mask of t - cut for the lane's 16 rows of a tile (bit 15 - v stands for
+// accumulator v = row 8 (v / 4) + 4 half + v % 4): one matrix instruction and
+// 16 funnel shifts.  rows < 32: the segment's last tile, whose rows past the
+// end belong to the next segment and are masked out.
+__device__ __forceinline__ uint32_t bin_tile_signs(uint4 operand,
+                                                   mc_bf16x8_t yb, int half,
+                                                   int rows) {
+  // upper lanes: 1 in place of w_hi and w_lo (times the parts of -cut)
+  if (half) {
+    operand.y = (operand.y & 0x0000ffffu) | (0x3f80u << 16);
+    operand.w = (operand.w & 0x0000ffffu) | (0x3f80u << 16);
+  }
+  mfma_acc_t acc = {0};
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+      __builtin_bit_cast(mc_bf16x8_t, operand), yb, acc, 0, 0, 0);
+  uint32_t mask = 0;
+#pragma unroll
+  for (int v = 0; v < 16; ++v)
+    mask = __builtin_amdgcn_alignbit(mask, __float_as_uint(acc[v]), 31);
+  if (rows < kBinTile) {
+    uint32_t real = 0;
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      real |= (8 * (v / 4) + 4 * half + v % 4 < rows) ? (1u << (15 - v)) : 0u;
+    mask &= real;
+  }
+  return mask;
+}
+
+// Exact squared distance of a ring entry (coordinates, row number) to the
+// lane's query, as the reference accumulates it.
+__device__ __forceinline__ float bin_exact_distance(const uint4 &r4,
+                                                    const float (&y)[3]) {
+  const float d0 = __uint_as_float(r4.x) - y[0];
+  float d = d0 * d0;
+  const float d1 = __uint_as_float(r4.y) - y[1];
+  d = __builtin_fmaf(d1, d1, d);
+  const float d2 = __uint_as_float(r4.z) - y[2];
+  return __builtin_fmaf(d2, d2, d);
+}
+
+// The box that lane `src` holds, broadcast to the wave.
+__device__ __forceinline__ void bin_box_of_lane(const Box &held, int src,
+                                                float (&lo)[3],
+                                                float (&hi)[3]) {
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    lo[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+        (int)__float_as_uint(held.lo[c]), src));
+    hi[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+        (int)__float_as_uint(held.hi[c]), src));
+  }
+}
+
 // Tasks of the matrix-core searches.  Normally a block of 32
 // curve-consecutive queries is one task (slot = block number).  A block whose
 // queries span much more of the curve than the segment's average lies where
@@ -225,60 +384,14 @@ knn_binned_mc_kernel(BinnedParams p) {
   const bool valid = col < task.y;
   const int q = valid ? (int)p.perm_y[jq] : 0;
   const int k = p.k;
-  const int d_in = p.d;
 
-  float yq[DIM];
-#pragma unroll
-  for (int c = 0; c < DIM; ++c)
-    yq[c] = (valid && c < d_in) ? p.y[(size_t)q * d_in + c] : 0.0f;
-  // a query with a coordinate that is not finite has no distance below the
-  // limit: it looks at nothing and returns nothing
-  const bool searching = valid && __builtin_fabsf(yq[0]) < __builtin_inff() &&
-                         __builtin_fabsf(yq[1]) < __builtin_inff() &&
-                         __builtin_fabsf(yq[2]) < __builtin_inff();
-  float ysq = yq[0] * yq[0];
-#pragma unroll
-  for (int c = 1; c < DIM; ++c)
-    ysq = __builtin_fmaf(yq[c], yq[c], ysq);
-  const bool y_moderate = ysq <= kFilterNormLimit;
-
-  // the wave's box (lanes that do not search stay out)
-  float q_lo[3], q_hi[3];
-#pragma unroll
-  for (int c = 0; c < 3; ++c) {
-    float lo = searching ? yq[c] : __builtin_inff();
-    float hi = searching ? yq[c] : -__builtin_inff();
-#pragma unroll
-    for (int sh = 1; sh < kWave; sh <<= 1) {
-      lo = __builtin_fminf(lo, __shfl_xor(lo, sh));
-      hi = __builtin_fmaxf(hi, __shfl_xor(hi, sh));
-    }
-    q_lo[c] = lo;
-    q_hi[c] = hi;
-  }
-
-  // B operand: the hi (lanes 0-31) or lo (lanes 32-63) parts of
-  // (-2 y_0, -2 y_1, -2 y_2, 1), given twice (against the hi and the lo parts
-  // of the row); see knn_lowd_mc_impl.hpp
-  uint4 yb_plain;
-  {
-    uint32_t part[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float v = 0.0f;
-      if (e < DIM)
-        v = (searching && y_moderate) ? -2.0f * yq[e] : 0.0f;
-      else
-        v = searching ? 1.0f : 0.0f;
-      uint32_t hi, lo;
-      mc_split(v, hi, lo);
-      part[e] = half ? lo : hi;
-    }
-    const uint32_t w0 = part[0] | (part[1] << 16);
-    const uint32_t w1 = part[2] | (part[3] << 16);
-    yb_plain = make_uint4(w0, w1, w0, w1);
-  }
-  mc_bf16x8_t yb = __builtin_bit_cast(mc_bf16x8_t, yb_plain);
+  const BinQuery me = bin_load_query(p, valid, q);
+  const float (&yq)[3] = me.y;
+  const float (&q_lo)[3] = me.lo;
+  const float (&q_hi)[3] = me.hi;
+  const bool searching = me.searching;
+  const float ysq = me.ysq;
+  const uint4 yb_plain = bin_query_operand(me, half);
 
   double best[K];
 #pragma unroll
@@ -291,27 +404,8 @@ knn_binned_mc_kernel(BinnedParams p) {
   float thresh = searching ? kLimit : -__builtin_inff();
   float cut = searching ? mc_filter_cut(thresh, ysq_damped) : -1e38f;
   float shared = kLimit; // bound learnt from the partner lane
-  // -cut rides in the two accumulation slots of w that the zero lo part of
-  // the query's 1 would leave unused (component 3 of the one instruction)
-  const uint32_t one_keep = half ? ~(0xffffu << 16) : 0xffffffffu;
-  const uint32_t one_bits = half ? (0x3f80u << 16) : 0u;
-  auto refresh_cut = [&]() {
-    if (half) {
-      float neg = -__builtin_fmaf(__builtin_fabsf(cut), 3.0517578125e-05f, cut);
-      uint32_t hi, lo;
-      if (__builtin_fabsf(neg) < 1e38f) {
-        mc_split(neg, hi, lo);
-      } else {
-        hi = neg < 0.0f ? 0xff7fu : 0x7f7fu;
-        lo = 0;
-      }
-      uint4 b = yb_plain;
-      b.y = (b.y & 0x0000ffffu) | (hi << 16);
-      b.w = (b.w & 0x0000ffffu) | (lo << 16);
-      yb = __builtin_bit_cast(mc_bf16x8_t, b);
-    }
-  };
-  refresh_cut();
+  mc_bf16x8_t yb = bin_operand_with_cut(yb_plain, cut, half);
+  auto refresh_cut = [&]() { yb = bin_operand_with_cut(yb_plain, cut, half); };
   auto set_thresh = [&](float v) {
     if (searching) {
       thresh = v;
@@ -373,12 +467,7 @@ knn_binned_mc_kernel(BinnedParams p) {
       pending &= ~(1u << bit);
       const int j = has ? slot_base + 2 * (v & 12) + (v & 3) : 0;
       const uint4 r4 = (&ring[wave][0][0])[j];
-      const float d0 = __uint_as_float(r4.x) - yq[0];
-      float d = d0 * d0;
-      const float d1 = __uint_as_float(r4.y) - yq[1];
-      d = __builtin_fmaf(d1, d1, d);
-      const float d2 = __uint_as_float(r4.z) - yq[2];
-      d = __builtin_fmaf(d2, d2, d);
+      const float d = bin_exact_distance(r4, yq);
       const bool ok = has && d < thresh;
       if (!__any(ok))
         continue;
@@ -414,43 +503,16 @@ knn_binned_mc_kernel(BinnedParams p) {
   const int num_tiles = p.tile_start[seg + 1] - tile0;
   int scanned = 0; // tiles since the start: slot = scanned % kBinRing
 
-  // The rows of a tile as the lanes fetch them: the operand quad of row
-  // `col` (both halves), the coordinate quad of row `col` (lower half).
-  struct Fetched {
-    uint4 operand, coords;
-  };
+  typedef BinFetched Fetched;
   auto fetch = [&](int tile) {
-    const size_t j = (size_t)(x_begin + tile * kBinTile + col);
-    Fetched f;
-    // (the packed copy is padded by a tile of rows that never pass)
-    f.operand = p.packed[j * REC];
-    f.coords = half ? make_uint4(0u, 0u, 0u, 0u) : p.packed[j * REC + 1];
-    return f;
+    return bin_fetch(p.packed, x_begin + tile * kBinTile, col, half);
   };
   auto scan = [&](int tile, const Fetched &f) {
     const int slot = scanned % kBinRing;
     if (!half)
       ring[wave][slot][col] = f.coords;
-    uint4 a = f.operand;
-    // upper lanes: 1 in place of w_hi and w_lo (times the parts of -cut)
-    a.y = (a.y & one_keep) | one_bits;
-    a.w = (a.w & one_keep) | one_bits;
-    mfma_acc_t acc = {0};
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-        __builtin_bit_cast(mc_bf16x8_t, a), yb, acc, 0, 0, 0);
-    uint32_t mask = 0;
-#pragma unroll
-    for (int v = 0; v < 16; ++v)
-      mask = __builtin_amdgcn_alignbit(mask, __float_as_uint(acc[v]), 31);
     const int rows = min(kBinTile, x_end - (x_begin + tile * kBinTile));
-    if (rows < kBinTile) {
-      // the segment's last tile: rows past its end belong to the next one
-      uint32_t real = 0;
-#pragma unroll
-      for (int v = 0; v < 16; ++v)
-        real |= (8 * (v / 4) + 4 * half + v % 4 < rows) ? (1u << (15 - v)) : 0u;
-      mask &= real;
-    }
+    const uint32_t mask = bin_tile_signs(f.operand, yb, half, rows);
     if (mask != 0) {
       queue[qn][tid] = ((uint32_t)slot << 16) | mask;
       ++qn;
@@ -495,16 +557,9 @@ knn_binned_mc_kernel(BinnedParams p) {
     // from an infinite or empty box - never rules a box out.)
     auto reachable = [&](const Box &held, int src) {
       float lo[3], hi[3];
-#pragma unroll
-      for (int c = 0; c < 3; ++c) {
-        lo[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
-            (int)__float_as_uint(held.lo[c]), src));
-        hi[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
-            (int)__float_as_uint(held.hi[c]), src));
-      }
+      bin_box_of_lane(held, src, lo, hi);
       return __any(searching && !(box_gap2(lo, hi, yq, yq) >= thresh));
     };
-
     // the same for the boxes of lanes `a` (tested by lanes 0-31) and `b`
     // (lanes 32-63) at once: the ballot of the lanes whose query reaches
     auto reachable_pair = [&](const Box &held, int a, int b) {
@@ -624,8 +679,6 @@ knn_binned_mc_kernel(BinnedParams p) {
 template <int K>
 __global__ __launch_bounds__(kBinMcBlock, K <= 16 ? 4 : 1) void
 radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
-  constexpr int DIM = 3;
-  constexpr int REC = McShape<DIM>::REC;
   __shared__ __attribute__((aligned(16))) uint4 ring[kBinRing][kBinTile];
   __shared__ uint32_t queue[kBinRing][kBinMcBlock];
 
@@ -645,73 +698,17 @@ radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
   const bool valid = jq < y_end;
   const int q = valid ? (int)p.perm_y[jq] : 0;
   const int slots = p.k;
-  const int d_in = p.d;
 
-  float yq[DIM];
-#pragma unroll
-  for (int c = 0; c < DIM; ++c)
-    yq[c] = (valid && c < d_in) ? p.y[(size_t)q * d_in + c] : 0.0f;
-  // (a coordinate that is not finite: no distance below r2)
-  const bool searching = valid && __builtin_fabsf(yq[0]) < __builtin_inff() &&
-                         __builtin_fabsf(yq[1]) < __builtin_inff() &&
-                         __builtin_fabsf(yq[2]) < __builtin_inff();
-  float ysq = yq[0] * yq[0];
-#pragma unroll
-  for (int c = 1; c < DIM; ++c)
-    ysq = __builtin_fmaf(yq[c], yq[c], ysq);
-  const bool y_moderate = ysq <= kFilterNormLimit;
-
-  float q_lo[3], q_hi[3];
-#pragma unroll
-  for (int c = 0; c < 3; ++c) {
-    float lo = searching ? yq[c] : __builtin_inff();
-    float hi = searching ? yq[c] : -__builtin_inff();
-#pragma unroll
-    for (int sh = 1; sh < kWave; sh <<= 1) {
-      lo = __builtin_fminf(lo, __shfl_xor(lo, sh));
-      hi = __builtin_fmaxf(hi, __shfl_xor(hi, sh));
-    }
-    q_lo[c] = lo;
-    q_hi[c] = hi;
-  }
-
-  // the query operand with -cut for the fixed bound r2 in place (see
-  // knn_binned_mc_kernel); a lane that does not search passes nothing
-  mc_bf16x8_t yb;
-  {
-    uint32_t part[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float v = 0.0f;
-      if (e < DIM)
-        v = (searching && y_moderate) ? -2.0f * yq[e] : 0.0f;
-      else
-        v = searching ? 1.0f : 0.0f;
-      uint32_t hi, lo;
-      mc_split(v, hi, lo);
-      part[e] = half ? lo : hi;
-    }
-    const uint32_t w0 = part[0] | (part[1] << 16);
-    const uint32_t w1 = part[2] | (part[3] << 16);
-    uint4 b = make_uint4(w0, w1, w0, w1);
-    if (half) {
-      const float cut =
-          searching ? mc_filter_cut(r2, mc_damped_norm(ysq)) : -1e38f;
-      float neg = -__builtin_fmaf(__builtin_fabsf(cut), 3.0517578125e-05f, cut);
-      uint32_t hi, lo;
-      if (__builtin_fabsf(neg) < 1e38f) {
-        mc_split(neg, hi, lo);
-      } else {
-        hi = neg < 0.0f ? 0xff7fu : 0x7f7fu;
-        lo = 0;
-      }
-      b.y = (b.y & 0x0000ffffu) | (hi << 16);
-      b.w = (b.w & 0x0000ffffu) | (lo << 16);
-    }
-    yb = __builtin_bit_cast(mc_bf16x8_t, b);
-  }
-  const uint32_t one_keep = half ? ~(0xffffu << 16) : 0xffffffffu;
-  const uint32_t one_bits = half ? (0x3f80u << 16) : 0u;
+  const BinQuery me = bin_load_query(p, valid, q);
+  const float (&yq)[3] = me.y;
+  const float (&q_lo)[3] = me.lo;
+  const float (&q_hi)[3] = me.hi;
+  const bool searching = me.searching;
+  // the query operand with -cut for the fixed bound r2 in place; a lane that
+  // does not search passes nothing
+  const mc_bf16x8_t yb = bin_operand_with_cut(
+      bin_query_operand(me, half),
+      searching ? mc_filter_cut(r2, mc_damped_norm(me.ysq)) : -1e38f, half);
 
   double best[K];
 #pragma unroll
@@ -746,12 +743,7 @@ radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
       pending &= ~(1u << bit);
       const int j = has ? slot_base + 2 * (v & 12) + (v & 3) : 0;
       const uint4 r4 = (&ring[0][0])[j];
-      const float d0 = __uint_as_float(r4.x) - yq[0];
-      float d = d0 * d0;
-      const float d1 = __uint_as_float(r4.y) - yq[1];
-      d = __builtin_fmaf(d1, d1, d);
-      const float d2 = __uint_as_float(r4.z) - yq[2];
-      d = __builtin_fmaf(d2, d2, d);
+      const float d = bin_exact_distance(r4, yq);
       const bool ok = has && d < limit && r4.w < below && r4.w != self;
       if (!__any(ok))
         continue;
@@ -769,38 +761,16 @@ radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
     below = min(below, half ? both[0] : both[1]);
   };
 
-  struct Fetched {
-    uint4 operand, coords;
-  };
+  typedef BinFetched Fetched;
   auto fetch = [&](int tile) {
-    const size_t j = (size_t)(x_begin + tile * kBinTile + col);
-    Fetched f;
-    f.operand = p.packed[j * REC];
-    f.coords = half ? make_uint4(0u, 0u, 0u, 0u) : p.packed[j * REC + 1];
-    return f;
+    return bin_fetch(p.packed, x_begin + tile * kBinTile, col, half);
   };
   auto scan = [&](int tile, const Fetched &f) {
     const int slot = scanned % kBinRing;
     if (!half)
       ring[slot][col] = f.coords;
-    uint4 a = f.operand;
-    a.y = (a.y & one_keep) | one_bits;
-    a.w = (a.w & one_keep) | one_bits;
-    mfma_acc_t acc = {0};
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-        __builtin_bit_cast(mc_bf16x8_t, a), yb, acc, 0, 0, 0);
-    uint32_t mask = 0;
-#pragma unroll
-    for (int v = 0; v < 16; ++v)
-      mask = __builtin_amdgcn_alignbit(mask, __float_as_uint(acc[v]), 31);
     const int rows = min(kBinTile, x_end - (x_begin + tile * kBinTile));
-    if (rows < kBinTile) {
-      uint32_t real = 0;
-#pragma unroll
-      for (int v = 0; v < 16; ++v)
-        real |= (8 * (v / 4) + 4 * half + v % 4 < rows) ? (1u << (15 - v)) : 0u;
-      mask &= real;
-    }
+    const uint32_t mask = bin_tile_signs(f.operand, yb, half, rows);
     if (mask != 0) {
       queue[qn][tid] = ((uint32_t)slot << 16) | mask;
       ++qn;
@@ -816,13 +786,7 @@ radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
   // never rules a box out.)
   auto reachable = [&](const Box &held, int src) {
     float lo[3], hi[3];
-#pragma unroll
-    for (int c = 0; c < 3; ++c) {
-      lo[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
-          (int)__float_as_uint(held.lo[c]), src));
-      hi[c] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
-          (int)__float_as_uint(held.hi[c]), src));
-    }
+    bin_box_of_lane(held, src, lo, hi);
     const uint32_t min_row =
         (uint32_t)__builtin_amdgcn_readlane((int)held.min_row, src);
     return __any(searching && min_row < below &&
