@@ -21,9 +21,10 @@ def set_search_strategy(name: str) -> None:
     ``radius_graph`` (at most 32 neighbours per query) search fp32 points of
     up to 3 dimensions: ``"scan"`` (default) looks at every row of the
     example, ``"binned"`` orders the rows along a space-filling curve first and
-    looks only at rows near the query, ``"auto"`` bins when the examples
-    average 65,536 rows or more.  Same edges either way; binning wins on large
-    examples (10^5 rows and more).  Process-wide; the environment variable
+    looks only at rows near the query, ``"auto"`` bins when its estimate of
+    the two costs says so (from some ten thousand rows per example on, unless
+    the queries are few).  Same edges either way; binning wins on large
+    examples.  Process-wide; the environment variable
     ``PCA_SEARCH_STRATEGY`` sets the initial value.  No counterpart in the
     reference."""
     _torch.ops.pytorch_cluster_amd.set_search_strategy(name)

@@ -130,12 +130,9 @@ int edge_flags(bool drop_self, bool x_first) {
 // looks at every row of the segment (pca_knn, pca_radius), "binned" at the
 // rows near the query (pca_knn_binned: Euclidean, k <= 32; pca_radius_binned:
 // at most 32 neighbours per query - anything else is scanned).  Same edges
-// either way.  "auto" bins when the segments average kAutoBinRows rows or
-// more, where binning has paid off in measurements (the scan grows with the
-// square of the segment size).  Process-wide; starts from the environment
-// variable PCA_SEARCH_STRATEGY.
+// either way.  "auto" bins when that is expected to pay off (bins_wanted).
+// Process-wide; starts from the environment variable PCA_SEARCH_STRATEGY.
 enum Strategy { kScan = 0, kBinned = 1, kAuto = 2 };
-constexpr int64_t kAutoBinRows = 65536;
 
 int strategy_code(const std::string &name) {
   if (name == "scan")
@@ -165,11 +162,24 @@ std::string get_search_strategy() {
   return code == kBinned ? "binned" : code == kAuto ? "auto" : "scan";
 }
 
-bool bins_wanted(int64_t n, int64_t num_segments) {
+// searched: rows that get binned (x of knn / radius, y of nearest);
+// searching: the rows that look for neighbours.  "auto" compares two rough
+// estimates fitted to measurements on an MI355X, in ms: the scan looks at
+// every pair of a segment (segments taken as equal; ~5 G pairs per ms between
+// the small-cloud and the large-cloud rate), binning costs a sort of both
+// sides and a search that grows with their sizes.  It picks the scan for
+// clouds of a few thousand points and for a handful of queries against many
+// rows, bins from some ten thousand rows per segment on.
+bool bins_wanted(int64_t searched, int64_t searching, int64_t num_segments) {
   const int code = g_strategy.load();
-  return code == kBinned ||
-         (code == kAuto && n / std::max<int64_t>(num_segments, 1) >=
-                               kAutoBinRows);
+  if (code != kAuto)
+    return code == kBinned;
+  const double pairs = (double)searched * (double)searching /
+                       (double)std::max<int64_t>(num_segments, 1);
+  const double scan_ms = 0.1 + pairs / 5e9;
+  const double binned_ms =
+      0.2 + 1e-6 * ((double)searched + 2.0 * (double)searching);
+  return scan_ms > binned_ms;
 }
 
 at::Tensor knn_search(at::Tensor x, at::Tensor y,
@@ -196,7 +206,7 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
     return at::empty({2, 0}, long_opts);
 
   const int dtype = dtype_code(x);
-  const bool binned = bins_wanted(n, seg.count) && dtype == PCA_F32 &&
+  const bool binned = bins_wanted(n, m, seg.count) && dtype == PCA_F32 &&
                       !cosine && d <= 3 && k <= 32;
   const size_t ws_bytes =
       binned ? pca_knn_binned_workspace_bytes(n, m, d, seg.count, k)
@@ -268,7 +278,7 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
 
   const int dtype = dtype_code(x);
   const int64_t slots = pca_radius_slots(n, max_num_neighbors);
-  const bool binned = bins_wanted(n, seg.count) && dtype == PCA_F32 &&
+  const bool binned = bins_wanted(n, m, seg.count) && dtype == PCA_F32 &&
                       d <= 3 && slots <= 32;
   const size_t ws_bytes =
       binned ? pca_radius_binned_workspace_bytes(n, m, d, seg.count,
@@ -351,7 +361,7 @@ at::Tensor nearest(at::Tensor x, at::Tensor y, at::Tensor ptr_x,
               "nearest is not implemented for 'BFloat16'");
   // (the searched rows, y, are the ones a binned search orders)
   const bool binned =
-      bins_wanted(m, segments) && dtype == PCA_F32 && d <= 3 && m > 0;
+      bins_wanted(m, n, segments) && dtype == PCA_F32 && d <= 3 && m > 0;
   const size_t ws_bytes =
       binned ? pca_nearest_binned_workspace_bytes(n, m, d, segments)
              : pca_nearest_workspace_bytes(n, m, d, segments, dtype);
