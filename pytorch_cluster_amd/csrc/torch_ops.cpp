@@ -165,20 +165,23 @@ std::string get_search_strategy() {
 // searched: rows that get binned (x of knn / radius, y of nearest);
 // searching: the rows that look for neighbours.  "auto" compares two rough
 // estimates fitted to measurements on an MI355X, in ms: the scan looks at
-// every pair of a segment (segments taken as equal; ~5 G pairs per ms between
-// the small-cloud and the large-cloud rate), binning costs a sort of both
-// sides and a search that grows with their sizes.  It picks the scan for
+// every pair of a segment (segments taken as equal) at scan_rate pairs per
+// ms - kNN ~3 G (between its small-cloud and large-cloud rates), radius and
+// nearest ~10 G (the radius scan stops at max_num_neighbors, nearest keeps
+// one neighbour) -, binning costs a sort of both sides and a search that
+// grows with their sizes (query_us per searching row).  It picks the scan for
 // clouds of a few thousand points and for a handful of queries against many
 // rows, bins from some ten thousand rows per segment on.
-bool bins_wanted(int64_t searched, int64_t searching, int64_t num_segments) {
+bool bins_wanted(int64_t searched, int64_t searching, int64_t num_segments,
+                 double scan_rate, double query_us) {
   const int code = g_strategy.load();
   if (code != kAuto)
     return code == kBinned;
   const double pairs = (double)searched * (double)searching /
                        (double)std::max<int64_t>(num_segments, 1);
-  const double scan_ms = 0.1 + pairs / 5e9;
+  const double scan_ms = 0.1 + pairs / scan_rate;
   const double binned_ms =
-      0.2 + 1e-6 * ((double)searched + 2.0 * (double)searching);
+      0.2 + 1e-6 * (double)searched + 1e-3 * query_us * (double)searching;
   return scan_ms > binned_ms;
 }
 
@@ -206,8 +209,8 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
     return at::empty({2, 0}, long_opts);
 
   const int dtype = dtype_code(x);
-  const bool binned = bins_wanted(n, m, seg.count) && dtype == PCA_F32 &&
-                      !cosine && d <= 3 && k <= 32;
+  const bool binned = bins_wanted(n, m, seg.count, 3e9, 2e-3) &&
+                      dtype == PCA_F32 && !cosine && d <= 3 && k <= 32;
   const size_t ws_bytes =
       binned ? pca_knn_binned_workspace_bytes(n, m, d, seg.count, k)
              : pca_knn_workspace_bytes(n, m, d, seg.count, k, dtype);
@@ -278,8 +281,8 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
 
   const int dtype = dtype_code(x);
   const int64_t slots = pca_radius_slots(n, max_num_neighbors);
-  const bool binned = bins_wanted(n, m, seg.count) && dtype == PCA_F32 &&
-                      d <= 3 && slots <= 32;
+  const bool binned = bins_wanted(n, m, seg.count, 1e10, 2e-3) &&
+                      dtype == PCA_F32 && d <= 3 && slots <= 32;
   const size_t ws_bytes =
       binned ? pca_radius_binned_workspace_bytes(n, m, d, seg.count,
                                                  max_num_neighbors)
@@ -361,7 +364,8 @@ at::Tensor nearest(at::Tensor x, at::Tensor y, at::Tensor ptr_x,
               "nearest is not implemented for 'BFloat16'");
   // (the searched rows, y, are the ones a binned search orders)
   const bool binned =
-      bins_wanted(m, n, segments) && dtype == PCA_F32 && d <= 3 && m > 0;
+      bins_wanted(m, n, segments, 1e10, 0.5e-3) && dtype == PCA_F32 &&
+      d <= 3 && m > 0;
   const size_t ws_bytes =
       binned ? pca_nearest_binned_workspace_bytes(n, m, d, segments)
              : pca_nearest_workspace_bytes(n, m, d, segments, dtype);
