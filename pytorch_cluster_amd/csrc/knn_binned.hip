@@ -878,15 +878,24 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
   if ((err = sort_pairs(sort_temp, sort_bytes, keys_a, keys_x, vals_a, perm_x,
                         in.n, nseg, stream)) != hipSuccess)
     return err;
-  hipLaunchKernelGGL(morton_keys_kernel, dim3((in.m + kBlock - 1) / kBlock),
-                     dim3(kBlock), 0, stream, y, in.ptr_y, in.m, in.d, nseg,
-                     seg_box, axis_bits(nseg), keys_a, vals_a);
-  if ((err = hipGetLastError()) != hipSuccess)
-    return err;
-  sort_bytes = lay.sort_temp;
-  if ((err = sort_pairs(sort_temp, sort_bytes, keys_a, keys_y, vals_a, perm_y,
-                        in.m, nseg, stream)) != hipSuccess)
-    return err;
+  // the rows searching for themselves (the graph entry points): one order
+  // serves both sides
+  const bool self_search = in.y == in.x && in.m == in.n &&
+                           (in.ptr_y == in.ptr_x || in.ptr_x == nullptr);
+  if (self_search) {
+    keys_y = keys_x;
+    perm_y = perm_x;
+  } else {
+    hipLaunchKernelGGL(morton_keys_kernel, dim3((in.m + kBlock - 1) / kBlock),
+                       dim3(kBlock), 0, stream, y, in.ptr_y, in.m, in.d, nseg,
+                       seg_box, axis_bits(nseg), keys_a, vals_a);
+    if ((err = hipGetLastError()) != hipSuccess)
+      return err;
+    sort_bytes = lay.sort_temp;
+    if ((err = sort_pairs(sort_temp, sort_bytes, keys_a, keys_y, vals_a,
+                          perm_y, in.m, nseg, stream)) != hipSuccess)
+      return err;
+  }
   {
     const int per_block = kBlock / kBinTile;
     hipLaunchKernelGGL(gather_tiles_kernel,

@@ -252,3 +252,19 @@ def test_three_million_rows_against_the_scanning_kernels(scan_kind):
     b, db = capi.knn_edges(x, y, None, None, 8, want_dist=True, binned=True)
     assert torch.equal(a, b)
     assert torch.equal(da.view(torch.int32), db.view(torch.int32))
+
+
+def test_rows_searching_for_themselves_share_one_order(oracle):
+    """x and y the same buffer (the graph entry points): the order along the
+    curve is computed once and serves both sides."""
+    rng = np.random.default_rng(21)
+    x = rng.integers(0, 7, (5000, 3)).astype(np.float32)   # ties everywhere
+    ptr = np.array([0, 1200, 1200, 5000], dtype=np.int64)
+    xt, pt = dev(x), dev(ptr, torch.long)
+    e, d = capi.knn_edges(xt, xt, pt, pt, 9, want_dist=True, binned=True)
+    want_e, want_d = oracle_knn_edges(oracle, x, x, ptr, ptr, 9)
+    assert (e.cpu().numpy() == want_e).all()
+    assert (d.cpu().numpy().view(np.uint32) == want_d.view(np.uint32)).all()
+    r = capi.radius_edges(xt, xt, pt, pt, 1.5, 12, True, binned=True)
+    want_r = oracle.radius_op(x, x, ptr, ptr, 1.5, 12, 1, True)
+    assert (r.cpu().numpy() == want_r).all()
