@@ -133,7 +133,7 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
 
 /*
  * pca_knn for fp32 points of up to 3 dimensions, Euclidean distance and
- * k <= 32 (PCA_ERR_UNSUPPORTED otherwise) over spatially binned rows: the x
+ * k <= 64 (PCA_ERR_UNSUPPORTED otherwise) over spatially binned rows: the x
  * rows of every segment are ordered along a space-filling curve (the voxel
  * numbers of the reference's grid clustering, csrc/cuda/grid_cuda.cu:10-25,
  * bit-interleaved), cut into tiles with bounding boxes, and a query scans only

@@ -413,7 +413,7 @@ int pca_knn_binned(const void *x, const void *y, const int64_t *ptr_x,
                 pca_status_string(PCA_ERR_K_TOO_LARGE));
   if (!pca::knn_binned_supported((int)d, (int)k, false))
     return fail(PCA_ERR_UNSUPPORTED,
-                "binned search: fp32 points of up to 3 dimensions and k <= 32, "
+                "binned search: fp32 points of up to 3 dimensions and k <= 64, "
                 "got d=%lld k=%lld",
                 (long long)d, (long long)k);
   if (num_edges == nullptr)

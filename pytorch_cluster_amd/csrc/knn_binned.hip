@@ -990,7 +990,7 @@ hipError_t order_tasks(BinnedParams &p, const Bins &bins, int blocks,
 }
 
 bool knn_binned_supported(int d, int k, bool cosine) {
-  return !cosine && d >= 1 && d <= 3 && k >= 1 && k <= 32;
+  return !cosine && d >= 1 && d <= 3 && k >= 1 && k <= 64;
 }
 
 size_t knn_binned_scratch_bytes(int n, int m, int num_segments) {
@@ -1010,8 +1010,9 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
   fill_params(p, in, bins, out);
   p.k = k;
   // (diagnostic switch: the vector-ALU scan instead of the matrix-core one)
+  // (lists of more than 32 entries exist for the matrix-core scan only)
   const char *env = getenv("PCA_KNN_BINNED_MATRIX_CORES");
-  const bool matrix_cores = !(env != nullptr && env[0] == '0');
+  const bool matrix_cores = k > 32 || !(env != nullptr && env[0] == '0');
   const int per_task = matrix_cores ? kWave / 2 : kWave;
   if (matrix_cores)
     p.wave_start = bins.half_start;
@@ -1033,14 +1034,28 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
       hipLaunchKernelGGL((knn_binned_kernel<K_>), dim3(grid), dim3(kBlock), 0, \
                          stream, p);                                           \
   } while (0)
+#define PCA_BINNED_LAUNCH_WIDE(K_)                                             \
+  hipLaunchKernelGGL((knn_binned_mc_kernel<K_>), dim3(slots),                  \
+                     dim3(kBinMcBlock), 0, stream, p)
+  // (list widths in steps of 8: the bound shared by the two lanes of a query
+  // reads one of the five middle entries of a list)
   if (k <= 8)
     PCA_BINNED_LAUNCH(8);
   else if (k <= 16)
     PCA_BINNED_LAUNCH(16);
   else if (k <= 24)
     PCA_BINNED_LAUNCH(24);
-  else
+  else if (k <= 32)
     PCA_BINNED_LAUNCH(32);
+  else if (k <= 40)
+    PCA_BINNED_LAUNCH_WIDE(40);
+  else if (k <= 48)
+    PCA_BINNED_LAUNCH_WIDE(48);
+  else if (k <= 56)
+    PCA_BINNED_LAUNCH_WIDE(56);
+  else
+    PCA_BINNED_LAUNCH_WIDE(64);
+#undef PCA_BINNED_LAUNCH_WIDE
 #undef PCA_BINNED_LAUNCH
   if (time_stop)
     (void)hipEventRecord(time_stop, stream);

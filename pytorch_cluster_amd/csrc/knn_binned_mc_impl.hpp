@@ -266,6 +266,61 @@ __device__ __forceinline__ void bin_box_of_lane(const Box &held, int src,
   }
 }
 
+// Unites the sorted lists of the two lanes of a query (l and l + 32) in the
+// lower lane: afterwards its slots K - k .. K - 1 hold the k smallest keys of
+// both lists, ascending (slots below K - k: the padding they held before).
+// Entry i of the lower lane meets the upper lane's entry K - 1 - (i - s),
+// s = K - k: the minimum of an ascending and a descending sequence holds the
+// k smallest of both and is bitonic, and a bitonic merge network (over the
+// next power of two, the padding in front staying where it is) sorts it:
+// K + K log2(K) minimum / maximum operations instead of the K (2 K - 1) of K
+// insertions.  s takes one of eight values for a list width (k is uniform),
+// picked by a branch so that every register index is a constant.
+template <int K>
+__device__ __forceinline__ void bin_unite_halves(double (&best)[K], int k,
+                                                 int half) {
+  constexpr int P = K <= 8 ? 8 : K <= 16 ? 16 : K <= 32 ? 32 : 64;
+  static_assert(K <= 64 && K % 8 == 0 || K < 8, "list widths in steps of 8");
+  const int s_now = K - k;
+#pragma unroll
+  for (int s = 0; s < (K < 8 ? K : 8); ++s) {
+    if (s != s_now)
+      continue;
+    asm volatile(""); // (keeps this a branch)
+#pragma unroll
+    for (int i = s; i < K; ++i) {
+      const int j = K - 1 - (i - s); // the partner's entry for slot i
+      const auto hi = __builtin_amdgcn_permlane32_swap(
+          (unsigned)__double2hiint(best[j]), (unsigned)__double2hiint(best[j]),
+          false, false);
+      const auto lo = __builtin_amdgcn_permlane32_swap(
+          (unsigned)__double2loint(best[j]), (unsigned)__double2loint(best[j]),
+          false, false);
+      // (element 1 of a swap: in a lower lane, the upper lane's value)
+      const double upper = __hiloint2double((int)hi[1], (int)lo[1]);
+      // (the upper lanes' lists stay as they are: later slots still read
+      // them)
+      const double united = key_min(best[i], upper);
+      best[i] = half ? best[i] : united;
+    }
+  }
+  // entry e of the network is slot e - (P - K); entries in front of it are
+  // padding below every key and never move
+#pragma unroll
+  for (int stride = P / 2; stride >= 1; stride >>= 1) {
+#pragma unroll
+    for (int e = 0; e < P; ++e) {
+      if ((e & stride) != 0 || e < P - K)
+        continue;
+      const int a = e - (P - K), b = a + stride;
+      const double lo = key_min(best[a], best[b]);
+      const double hi = key_max(best[a], best[b]);
+      best[a] = lo;
+      best[b] = hi;
+    }
+  }
+}
+
 // Tasks of the matrix-core searches.  Normally a block of 32
 // curve-consecutive queries is one task (slot = block number).  A block whose
 // queries span much more of the curve than the segment's average lies where
@@ -405,8 +460,8 @@ knn_binned_mc_kernel(BinnedParams p) {
   float cut = searching ? mc_filter_cut(thresh, ysq_damped) : -1e38f;
   float shared = kLimit; // bound learnt from the partner lane
   mc_bf16x8_t yb = bin_operand_with_cut(yb_plain, cut, half);
-  auto refresh_cut = [&]() { yb = bin_operand_with_cut(yb_plain, cut, half); };
-  auto set_thresh = [&](float v) {
+  auto refresh_cut = [&]() __attribute__((always_inline)) { yb = bin_operand_with_cut(yb_plain, cut, half); };
+  auto set_thresh = [&](float v) __attribute__((always_inline)) {
     if (searching) {
       thresh = v;
       cut = mc_filter_cut(v, ysq_damped);
@@ -417,7 +472,7 @@ knn_binned_mc_kernel(BinnedParams p) {
 
   // What the two lanes of a query tell each other about its final k-th
   // distance (see knn_lowd_mc_impl.hpp; equality admitted).
-  auto partner_bounds = [&]() {
+  auto partner_bounds = [&]() __attribute__((always_inline)) {
     const float own = key_dist(best[K - 1]);
     const auto both = __builtin_amdgcn_permlane32_swap(
         __float_as_uint(own), __float_as_uint(own), false, false);
@@ -445,7 +500,7 @@ knn_binned_mc_kernel(BinnedParams p) {
 
   // Resolves the parked rows exactly: in every round each lane takes the next
   // row of its parked words and all lanes evaluate theirs together.
-  auto drain = [&]() {
+  auto drain = [&]() __attribute__((always_inline)) {
     bool changed = false; // wave-uniform
     int taken = 0;
     uint32_t pending = 0;
@@ -491,7 +546,7 @@ knn_binned_mc_kernel(BinnedParams p) {
   };
 
   // largest bound among the wave's queries
-  auto wave_reach = [&]() {
+  auto wave_reach = [&]() __attribute__((always_inline)) {
     float r = searching ? thresh : -1.0f;
 #pragma unroll
     for (int sh = 1; sh < kWave; sh <<= 1)
@@ -504,10 +559,10 @@ knn_binned_mc_kernel(BinnedParams p) {
   int scanned = 0; // tiles since the start: slot = scanned % kBinRing
 
   typedef BinFetched Fetched;
-  auto fetch = [&](int tile) {
+  auto fetch = [&](int tile) __attribute__((always_inline)) {
     return bin_fetch(p.packed, x_begin + tile * kBinTile, col, half);
   };
-  auto scan = [&](int tile, const Fetched &f) {
+  auto scan = [&](int tile, const Fetched &f) __attribute__((always_inline)) {
     const int slot = scanned % kBinRing;
     if (!half)
       ring[wave][slot][col] = f.coords;
@@ -555,14 +610,14 @@ knn_binned_mc_kernel(BinnedParams p) {
 
     // is the box of lane `src` within reach of some lane's query?  (A NaN -
     // from an infinite or empty box - never rules a box out.)
-    auto reachable = [&](const Box &held, int src) {
+    auto reachable = [&](const Box &held, int src) __attribute__((always_inline)) {
       float lo[3], hi[3];
       bin_box_of_lane(held, src, lo, hi);
       return __any(searching && !(box_gap2(lo, hi, yq, yq) >= thresh));
     };
     // the same for the boxes of lanes `a` (tested by lanes 0-31) and `b`
     // (lanes 32-63) at once: the ballot of the lanes whose query reaches
-    auto reachable_pair = [&](const Box &held, int a, int b) {
+    auto reachable_pair = [&](const Box &held, int a, int b) __attribute__((always_inline)) {
       const int src = half ? b : a;
       float lo[3], hi[3];
 #pragma unroll
@@ -646,20 +701,7 @@ knn_binned_mc_kernel(BinnedParams p) {
     drain();
   }
 
-  // unite the two half lists of each query in the lower lane
-#pragma unroll
-  for (int j = 0; j < K; ++j) {
-    if (j < K - k)
-      continue; // slots below are padding, not keys
-    const auto hi = __builtin_amdgcn_permlane32_swap(
-        (unsigned)__double2hiint(best[j]), (unsigned)__double2hiint(best[j]),
-        false, false);
-    const auto lo = __builtin_amdgcn_permlane32_swap(
-        (unsigned)__double2loint(best[j]), (unsigned)__double2loint(best[j]),
-        false, false);
-    const double upper = __hiloint2double((int)hi[1], (int)lo[1]);
-    sorted_insert<K>(best, half ? SearchLimit<NEAREST>::empty() : upper);
-  }
+  bin_unite_halves<K>(best, k, half);
   if (half == 0 && valid) {
     if constexpr (NEAREST)
       write_nearest(best[0], q, x_begin, p.out_nearest);
@@ -723,7 +765,7 @@ radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
   int qn = 0;
   int scanned = 0;
 
-  auto drain = [&]() {
+  auto drain = [&]() __attribute__((always_inline)) {
     bool changed = false;
     int taken = 0;
     uint32_t pending = 0;
@@ -762,10 +804,10 @@ radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
   };
 
   typedef BinFetched Fetched;
-  auto fetch = [&](int tile) {
+  auto fetch = [&](int tile) __attribute__((always_inline)) {
     return bin_fetch(p.packed, x_begin + tile * kBinTile, col, half);
   };
-  auto scan = [&](int tile, const Fetched &f) {
+  auto scan = [&](int tile, const Fetched &f) __attribute__((always_inline)) {
     const int slot = scanned % kBinRing;
     if (!half)
       ring[slot][col] = f.coords;
@@ -784,7 +826,7 @@ radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
   // lane that could still use one of its rows (a full list takes only smaller
   // row numbers than it holds)?  (A NaN - from an infinite or empty box -
   // never rules a box out.)
-  auto reachable = [&](const Box &held, int src) {
+  auto reachable = [&](const Box &held, int src) __attribute__((always_inline)) {
     float lo[3], hi[3];
     bin_box_of_lane(held, src, lo, hi);
     const uint32_t min_row =
@@ -793,7 +835,7 @@ radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
                  !(box_gap2(lo, hi, yq, yq) >= r2));
   };
   // largest row number any of the wave's queries could still take
-  auto wave_below = [&]() {
+  auto wave_below = [&]() __attribute__((always_inline)) {
     uint32_t b = below;
 #pragma unroll
     for (int sh = 1; sh < kWave; sh <<= 1)
@@ -855,20 +897,7 @@ radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
     drain();
   }
 
-  // unite the two half lists of each query in the lower lane
-#pragma unroll
-  for (int j = 0; j < K; ++j) {
-    if (j < K - slots)
-      continue;
-    const auto hi = __builtin_amdgcn_permlane32_swap(
-        (unsigned)__double2hiint(best[j]), (unsigned)__double2hiint(best[j]),
-        false, false);
-    const auto lo = __builtin_amdgcn_permlane32_swap(
-        (unsigned)__double2loint(best[j]), (unsigned)__double2loint(best[j]),
-        false, false);
-    const double upper = __hiloint2double((int)hi[1], (int)lo[1]);
-    sorted_insert<K>(best, half ? __builtin_inf() : upper);
-  }
+  bin_unite_halves<K>(best, slots, half);
   if (half == 0 && valid) {
     const size_t row = (size_t)q * slots;
     int found = 0;

@@ -128,7 +128,7 @@ int edge_flags(bool drop_self, bool x_first) {
 
 // How a search over fp32 points of up to 3 dimensions goes about it: "scan"
 // looks at every row of the segment (pca_knn, pca_radius), "binned" at the
-// rows near the query (pca_knn_binned: Euclidean, k <= 32; pca_radius_binned:
+// rows near the query (pca_knn_binned: Euclidean, k <= 64; pca_radius_binned:
 // at most 32 neighbours per query - anything else is scanned).  Same edges
 // either way.  "auto" bins when that is expected to pay off (bins_wanted).
 // Process-wide; starts from the environment variable PCA_SEARCH_STRATEGY.
@@ -210,7 +210,7 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
 
   const int dtype = dtype_code(x);
   const bool binned = bins_wanted(n, m, seg.count, 3e9, 2e-3) &&
-                      dtype == PCA_F32 && !cosine && d <= 3 && k <= 32;
+                      dtype == PCA_F32 && !cosine && d <= 3 && k <= 64;
   const size_t ws_bytes =
       binned ? pca_knn_binned_workspace_bytes(n, m, d, seg.count, k)
              : pca_knn_workspace_bytes(n, m, d, seg.count, k, dtype);

@@ -164,7 +164,21 @@ def test_unsupported_shapes_are_refused():
         capi.knn_edges(x, x, None, None, 4, binned=True)
     x = torch.rand(100, 3, device=DEV)
     with pytest.raises(RuntimeError, match="binned search"):
-        capi.knn_edges(x, x, None, None, 33, binned=True)
+        capi.knn_edges(x, x, None, None, 65, binned=True)
+
+
+@pytest.mark.parametrize("k", [33, 40, 41, 50, 57, 64])
+def test_more_than_32_neighbours(oracle, k, scan_kind):
+    """Lists of 40 to 64 entries (matrix-core scan only)."""
+    if scan_kind == "0":
+        pytest.skip("wide lists exist for the matrix-core scan only")
+    rng = np.random.default_rng(k)
+    x = rng.random((4000, 3)).astype(np.float32)
+    x[:500] = np.round(x[:500] * 4) / 4      # some exact ties
+    y = rng.random((300, 3)).astype(np.float32)
+    ptr_x = np.array([0, 45, 2000, 4000], dtype=np.int64)   # 45 rows < k
+    ptr_y = np.array([0, 20, 150, 300], dtype=np.int64)
+    check(oracle, x, y, ptr_x, ptr_y, k)
 
 
 def test_strategy_switch_of_the_entry_points():
