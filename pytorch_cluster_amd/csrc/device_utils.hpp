@@ -116,6 +116,61 @@ __device__ __forceinline__ void sorted_insert(double (&b)[K], double key) {
   b[0] = key_min(b[0], key);
 }
 
+// Unites the sorted lists of the two lanes of a query (l and l + 32) in the
+// lower lane: afterwards its slots K - k .. K - 1 hold the k smallest keys of
+// both lists, ascending (slots below K - k: the padding they held before).
+// Entry i of the lower lane meets the upper lane's entry K - 1 - (i - s),
+// s = K - k: the minimum of an ascending and a descending sequence holds the
+// k smallest of both and is bitonic, and a bitonic merge network (over the
+// next power of two, the padding in front staying where it is) sorts it:
+// K + K log2(K) minimum / maximum operations instead of the K (2 K - 1) of K
+// insertions.  s takes one of eight values for a list width (k is uniform),
+// picked by a branch so that every register index is a constant.
+template <int K>
+__device__ __forceinline__ void unite_halves(double (&best)[K], int k,
+                                                 int half) {
+  constexpr int P = K <= 8 ? 8 : K <= 16 ? 16 : K <= 32 ? 32 : 64;
+  static_assert(K <= 64 && K % 8 == 0 || K < 8, "list widths in steps of 8");
+  const int s_now = K - k;
+#pragma unroll
+  for (int s = 0; s < (K < 8 ? K : 8); ++s) {
+    if (s != s_now)
+      continue;
+    asm volatile(""); // (keeps this a branch)
+#pragma unroll
+    for (int i = s; i < K; ++i) {
+      const int j = K - 1 - (i - s); // the partner's entry for slot i
+      const auto hi = __builtin_amdgcn_permlane32_swap(
+          (unsigned)__double2hiint(best[j]), (unsigned)__double2hiint(best[j]),
+          false, false);
+      const auto lo = __builtin_amdgcn_permlane32_swap(
+          (unsigned)__double2loint(best[j]), (unsigned)__double2loint(best[j]),
+          false, false);
+      // (element 1 of a swap: in a lower lane, the upper lane's value)
+      const double upper = __hiloint2double((int)hi[1], (int)lo[1]);
+      // (the upper lanes' lists stay as they are: later slots still read
+      // them)
+      const double united = key_min(best[i], upper);
+      best[i] = half ? best[i] : united;
+    }
+  }
+  // entry e of the network is slot e - (P - K); entries in front of it are
+  // padding below every key and never move
+#pragma unroll
+  for (int stride = P / 2; stride >= 1; stride >>= 1) {
+#pragma unroll
+    for (int e = 0; e < P; ++e) {
+      if ((e & stride) != 0 || e < P - K)
+        continue;
+      const int a = e - (P - K), b = a + stride;
+      const double lo = key_min(best[a], best[b]);
+      const double hi = key_max(best[a], best[b]);
+      best[a] = lo;
+      best[b] = hi;
+    }
+  }
+}
+
 // ---- fp32 values as sums of two bf16 numbers (matrix-core pre-filters) -----
 typedef __bf16 mc_bf16x8_t __attribute__((ext_vector_type(8)));
 

@@ -549,21 +549,8 @@ __global__ __launch_bounds__(kBlock) void knn_lowd_mc_kernel(KnnLowdParams p) {
   }
 
   // ---- results ----------------------------------------------------------
-  // unite the two half lists of each query in the lower lane: it inserts the
-  // upper lane's keys one by one (the upper lane's list stays as it is)
-#pragma unroll
-  for (int j = 0; j < K; ++j) {
-    if (j < K - k)
-      continue; // slots below are padding, not keys
-    const auto hi = __builtin_amdgcn_permlane32_swap(
-        (unsigned)__double2hiint(best[j]), (unsigned)__double2hiint(best[j]),
-        false, false);
-    const auto lo = __builtin_amdgcn_permlane32_swap(
-        (unsigned)__double2loint(best[j]), (unsigned)__double2loint(best[j]),
-        false, false);
-    const double upper = __hiloint2double((int)hi[1], (int)lo[1]);
-    sorted_insert<K>(best, half ? SearchLimit<NEAREST>::empty() : upper);
-  }
+  // unite the two half lists of each query in the lower lane
+  unite_halves<K>(best, k, half);
 
   if (half == 0) {
     if (p.num_chunks == 1) {
