@@ -104,6 +104,8 @@ def other_configs(torch, pca, testing, dev):
         return statistics.median(times), out
 
     report = {}
+    # (the scanning kernels unless an entry names its strategy)
+    pca.set_search_strategy("scan")
     c2 = testing.uniform_batched(0)
     x, b = c2["x"].to(dev), c2["batch"].to(dev)
     ms, out = median_ms(lambda: pca.knn_graph(x, 20, b, batch_size=16), 10)
@@ -229,6 +231,7 @@ def other_configs(torch, pca, testing, dev):
             pca.set_search_strategy("scan")
         report["nearest on the LiDAR-like points, strategy %s" % strategy] = {
             "ms": ms, "rows_per_s": nx.shape[0] / ms * 1e3}
+    pca.set_search_strategy("auto")
     return report
 
 
@@ -260,9 +263,10 @@ def main():
                          "paths)")
     ap.add_argument("--strategy", choices=("scan", "binned", "auto"),
                     default="scan",
-                    help="search strategy of the timed steps: scan (default, "
-                         "the kernel the roofline figure is about), binned or "
-                         "auto (rows ordered along a space-filling curve, "
+                    help="search strategy of the timed steps: scan (default "
+                         "here: the brute-force kernel the metric's roofline "
+                         "figure is about), binned or auto (the library's "
+                         "default; rows ordered along a space-filling curve, "
                          "exact pruning; same edges)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy three times, so "
@@ -341,6 +345,7 @@ def main():
             "workload": "configs[4]: ragged LiDAR-like knn(x, y, k=16, "
                         "batch_x, batch_y), 8 scans of 60k-200k points, "
                         "y = every 4th point",
+            "strategy": args.strategy,
             "points": n, "queries": m, "k": K, "dim": 3, "segments": B,
             "pairs": pairs, "seed": 0,
         },
@@ -365,7 +370,6 @@ def main():
     if binned:
         # the events bracket binning + search here, and the work is not the
         # 9 flop x all pairs the roofline figure prices: no roofline claim
-        result["config"]["strategy"] = args.strategy
         result["roofline"] = None
         result["search_ms"] = kernel_s * 1e3
     if not binned:
@@ -383,7 +387,6 @@ def main():
         result["with_binned_strategy"] = {
             "value": m * args.steps / dt, "unit": "queries/s",
             "ms_per_step": dt / args.steps * 1e3}
-    pca.set_search_strategy("scan")
     if not args.no_extras:
         result["other_configs"] = other_configs(torch, pca, testing, dev)
     if args.copy_calibration:

@@ -19,11 +19,11 @@ __version__ = "0.1.0"
 def set_search_strategy(name: str) -> None:
     """How ``knn`` / ``knn_graph`` (Euclidean, k <= 64) and ``radius`` /
     ``radius_graph`` (at most 32 neighbours per query) search fp32 points of
-    up to 3 dimensions: ``"scan"`` (default) looks at every row of the
-    example, ``"binned"`` orders the rows along a space-filling curve first and
-    looks only at rows near the query, ``"auto"`` bins when its estimate of
-    the two costs says so (from some ten thousand rows per example on, unless
-    the queries are few).  Same edges either way; binning wins on large
+    up to 3 dimensions: ``"scan"`` looks at every row of the example,
+    ``"binned"`` orders the rows along a space-filling curve first and looks
+    only at rows near the query, ``"auto"`` (the default) bins when its
+    estimate of the two costs says so (from some ten thousand rows per example
+    on, unless the queries are few).  Same edges either way; binning wins on large
     examples.  Process-wide; the environment variable
     ``PCA_SEARCH_STRATEGY`` sets the initial value.  No counterpart in the
     reference."""

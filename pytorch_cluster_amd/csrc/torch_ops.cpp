@@ -130,8 +130,9 @@ int edge_flags(bool drop_self, bool x_first) {
 // looks at every row of the segment (pca_knn, pca_radius), "binned" at the
 // rows near the query (pca_knn_binned: Euclidean, k <= 64; pca_radius_binned:
 // at most 32 neighbours per query - anything else is scanned).  Same edges
-// either way.  "auto" bins when that is expected to pay off (bins_wanted).
-// Process-wide; starts from the environment variable PCA_SEARCH_STRATEGY.
+// either way.  "auto" - the default - bins when that is expected to pay off
+// (bins_wanted).  Process-wide; the environment variable PCA_SEARCH_STRATEGY
+// sets the initial value.
 enum Strategy { kScan = 0, kBinned = 1, kAuto = 2 };
 
 int strategy_code(const std::string &name) {
@@ -146,8 +147,8 @@ int strategy_code(const std::string &name) {
 
 std::atomic<int> g_strategy{[] {
   const char *e = std::getenv("PCA_SEARCH_STRATEGY");
-  const int code = e != nullptr ? strategy_code(e) : kScan;
-  return code < 0 ? (int)kScan : code;
+  const int code = e != nullptr ? strategy_code(e) : kAuto;
+  return code < 0 ? (int)kAuto : code;
 }()};
 
 void set_search_strategy(std::string name) {

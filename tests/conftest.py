@@ -3,6 +3,11 @@ import sys
 
 import pytest
 
+# The tests name the search strategy they mean; everything else runs on the
+# scanning kernels, whatever the size (the library's own default would bin
+# the large cases).
+os.environ.setdefault("PCA_SEARCH_STRATEGY", "scan")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
