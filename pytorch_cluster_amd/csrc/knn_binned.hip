@@ -956,6 +956,7 @@ void fill_params(BinnedParams &p, const SearchInput &in, const Bins &bins,
   p.out_nearest = nullptr;
   p.task_order = nullptr;
   p.task_desc = nullptr;
+  p.task_slots = 0;
   p.code_bits = 0;
 }
 
@@ -986,6 +987,9 @@ hipError_t order_tasks(BinnedParams &p, const Bins &bins, int blocks,
       (unsigned int)slots, 0u, 32u, stream, false);
   p.task_desc = desc;
   p.task_order = vals_out;
+  p.task_slots = slots;
+  // (the search kernels' grid: whole runs of 8 tasks on each of 8 XCDs)
+  slots = (slots + 63) / 64 * 64;
   return err;
 }
 

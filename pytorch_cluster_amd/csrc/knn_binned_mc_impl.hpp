@@ -50,6 +50,7 @@ struct BinnedParams {
                             // the fourth coordinate word = row number
   const uint32_t *task_order; // task slots, the longest tasks first
   const int2 *task_desc;      // per slot: first query position, queries
+  int task_slots;             // entries of task_order
   int code_bits;              // bits of the curve code inside a key
   const Box *box;           // of every tile
   const int *group_start;   // first group of tiles of every segment
@@ -277,6 +278,14 @@ __device__ __forceinline__ void bin_box_of_lane(const Box &held, int src,
 // (`extra` slots; `*extra_used` starts at 0).  The sort key of a slot is the
 // complement of its span, so that the longest tasks start first and unused
 // extra slots come last (their waves leave at once).
+// Octave of the span first (longest first), position along the curve second:
+// tasks of about the same length keep their neighbours next to them, and
+// neighbours look at the same tiles.
+__device__ __forceinline__ uint32_t bin_task_key(uint32_t span, int block) {
+  const uint32_t octave = span != 0 ? (uint32_t)__builtin_clz(span) : 32u;
+  return (octave << 25) | min((uint32_t)block, (1u << 25) - 1u);
+}
+
 __global__ __launch_bounds__(kBlock) void task_span_kernel(
     BinnedParams p, int bound, int extra, int *__restrict__ extra_used,
     int2 *__restrict__ desc, uint32_t *__restrict__ keys,
@@ -296,12 +305,12 @@ __global__ __launch_bounds__(kBlock) void task_span_kernel(
     const int blocks = p.wave_start[seg + 1] - p.wave_start[seg];
     const uint64_t average = ((uint64_t)1 << p.code_bits) / (uint64_t)blocks;
     mine = make_int2(jq0, count);
-    key = min(~span, 0xfffffffeu);
+    key = bin_task_key(span, block);
     if (count == 32 && (uint64_t)span > 8 * average) {
       const int at = atomicAdd(extra_used, 3);
       if (at + 3 <= extra) {
         mine = make_int2(jq0, 8);
-        key = min(~(span / 4), 0xfffffffeu);
+        key = bin_task_key(span / 4, block);
         for (int i = 0; i < 3; ++i) {
           desc[bound + at + i] = make_int2(jq0 + 8 * (i + 1), 8);
           keys[bound + at + i] = key;
@@ -360,7 +369,15 @@ knn_binned_mc_kernel(BinnedParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int half = lane >> 5;
   const int col = lane & 31;
-  const int slot = (int)p.task_order[blockIdx.x * kWaves + wave];
+  // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2:
+  // runs of 8 consecutive tasks of the order (neighbours along the curve,
+  // which fetch the same tiles) go to the same XCD, one after the other.
+  const int local = (int)blockIdx.x >> 3;
+  const int ordered = (((local >> 3) * 8 + ((int)blockIdx.x & 7)) << 3) |
+                      (local & 7);
+  if (ordered >= p.task_slots)
+    return; // (the grid is rounded up to whole runs)
+  const int slot = (int)p.task_order[ordered];
   const int2 task = p.task_desc[slot]; // (first query position, queries)
   if (task.y == 0)
     return; // (an unused slot; whole waves leave, no barrier below)
