@@ -1120,8 +1120,9 @@ hipError_t launch_radius_binned(const SearchInput &in, float r2,
 #define PCA_BINNED_LAUNCH(K_)                                                  \
   do {                                                                         \
     if (matrix_cores)                                                          \
-      hipLaunchKernelGGL((radius_binned_mc_kernel<K_>), dim3(waves),           \
-                         dim3(kBinMcBlock), 0, stream, p, r2, same);           \
+      hipLaunchKernelGGL((radius_binned_mc_kernel<K_>),                        \
+                         dim3((waves + 63) / 64 * 64), dim3(kBinMcBlock), 0,   \
+                         stream, p, r2, same);                                 \
     else                                                                       \
       hipLaunchKernelGGL((radius_binned_kernel<K_>), dim3(grid), dim3(kBlock), \
                          0, stream, p, r2, same);                              \

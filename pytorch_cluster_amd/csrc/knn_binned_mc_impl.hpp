@@ -339,6 +339,15 @@ __global__ __launch_bounds__(kBlock) void task_slots_clear_kernel(
   }
 }
 
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: runs
+// of 8 consecutive tasks (neighbours along the curve, which fetch the same
+// tiles) go to the same XCD, one after the other.  Maps a workgroup number to
+// its task's place in the order; grids are whole multiples of 64.
+__device__ __forceinline__ int bin_xcd_run(int workgroup) {
+  const int local = workgroup >> 3;
+  return (((local >> 3) * 8 + (workgroup & 7)) << 3) | (local & 7);
+}
+
 // Waves work on their own (no barrier): a workgroup is one wave, so that its
 // place on the SIMD frees up the moment it is done - the tasks differ a lot in
 // length.
@@ -369,12 +378,7 @@ knn_binned_mc_kernel(BinnedParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int half = lane >> 5;
   const int col = lane & 31;
-  // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2:
-  // runs of 8 consecutive tasks of the order (neighbours along the curve,
-  // which fetch the same tiles) go to the same XCD, one after the other.
-  const int local = (int)blockIdx.x >> 3;
-  const int ordered = (((local >> 3) * 8 + ((int)blockIdx.x & 7)) << 3) |
-                      (local & 7);
+  const int ordered = bin_xcd_run((int)blockIdx.x);
   if (ordered >= p.task_slots)
     return; // (the grid is rounded up to whole runs)
   const int slot = (int)p.task_order[ordered];
@@ -690,9 +694,9 @@ radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
   const int tid = lane;
   const int half = lane >> 5;
   const int col = lane & 31;
-  const int task = blockIdx.x;
+  const int task = bin_xcd_run((int)blockIdx.x);
   if (task >= p.wave_start[p.num_segments])
-    return;
+    return; // (also the padding of the grid to whole runs)
   const int seg = find_segment(p.wave_start, p.num_segments, task);
   const int x_begin = p.ptr_x ? (int)p.ptr_x[seg] : 0;
   const int x_end = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
