@@ -44,6 +44,7 @@
 #include <climits>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <type_traits>
 
 #include <rocprim/device/device_radix_sort.hpp>
@@ -702,14 +703,15 @@ __global__ __launch_bounds__(kBlock) void radius_binned_kernel(
 }
 
 struct BinnedLayout {
-  size_t seg_box, keys_a, keys_x, keys_y, vals_a, perm_x, perm_y, rows, packed,
-      box, group_box, tile_start, group_start, wave_start, half_start,
-      task_keys, sort_temp;
+  size_t seg_box, keys_a, keys_b, keys_x, keys_y, vals_a, vals_b, perm_x,
+      perm_y, rows, packed, box, group_box, tile_start, group_start,
+      wave_start, half_start, task_keys, sort_temp, side_temp;
   int tiles_bound, groups_bound;
   size_t total() const {
-    return seg_box + keys_a + keys_x + keys_y + vals_a + perm_x + perm_y +
-           rows + packed + box + group_box + tile_start + group_start +
-           wave_start + half_start + task_keys + sort_temp;
+    return seg_box + keys_a + keys_b + keys_x + keys_y + vals_a + vals_b +
+           perm_x + perm_y + rows + packed + box + group_box + tile_start +
+           group_start + wave_start + half_start + task_keys + sort_temp +
+           side_temp;
   }
 };
 
@@ -755,12 +757,15 @@ int task_slots(int blocks) {
 
 BinnedLayout binned_layout(int n, int m, int num_segments) {
   BinnedLayout w;
-  const size_t big = (size_t)std::max(n, m);
   w.seg_box = align256(sizeof(int) * 6 * (size_t)num_segments);
-  w.keys_a = align256(sizeof(uint32_t) * big);
+  // unsorted (key, row) of the rows (a) and of the queries (b): the two are
+  // sorted at the same time
+  w.keys_a = align256(sizeof(uint32_t) * (size_t)n);
+  w.keys_b = align256(sizeof(uint32_t) * (size_t)m);
   w.keys_x = align256(sizeof(uint32_t) * (size_t)n);
   w.keys_y = align256(sizeof(uint32_t) * (size_t)m);
-  w.vals_a = align256(sizeof(uint32_t) * big);
+  w.vals_a = align256(sizeof(uint32_t) * (size_t)n);
+  w.vals_b = align256(sizeof(uint32_t) * (size_t)m);
   w.perm_x = align256(sizeof(uint32_t) * (size_t)n);
   w.perm_y = align256(sizeof(uint32_t) * (size_t)m);
   // (padded: the search reads rows four at a time)
@@ -792,10 +797,10 @@ BinnedLayout binned_layout(int n, int m, int num_segments) {
       (unsigned int)task_slots(plan_upper_bound(m, num_segments, kWave / 2)),
       0u, 32u, nullptr, false);
   // (a failed size query leaves a size no workspace can meet)
-  w.sort_temp =
-      (ex == hipSuccess && ey == hipSuccess && et == hipSuccess)
-          ? align256(std::max(std::max(tx, ty), tt))
-          : ~(size_t)0 / 2;
+  const bool sized = ex == hipSuccess && ey == hipSuccess && et == hipSuccess;
+  w.sort_temp = sized ? align256(tx) : ~(size_t)0 / 2;
+  // (the queries and the task slots are sorted beside the rows' stream)
+  w.side_temp = sized ? align256(std::max(ty, tt)) : 0;
   return w;
 }
 
@@ -804,18 +809,109 @@ struct Bins {
   const int *tile_start, *group_start;
   const int *wave_start; // tasks of 64 queries
   const int *half_start; // tasks of 32 queries
-  uint32_t *task_keys;   // 6 words per task slot
-  void *sort_temp;
-  size_t sort_bytes;
   const uint32_t *keys_x, *keys_y, *perm_y;
   const float4 *rows;
   const uint4 *packed;
   const Box *box, *group_box;
+  // the tasks of 32 queries in starting order (when asked for)
+  const int2 *task_desc;
+  const uint32_t *task_order;
+  int task_slots; // slots of the order
+  int task_grid;  // workgroups that cover them
+  int code_bits;
 };
 
-// Orders rows and queries along the curve, copies the rows, builds the boxes.
-hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
-                        hipStream_t stream) {
+// A second stream of the device: the queries are ordered there while the rows
+// are ordered on the caller's stream (both chains are short kernels that
+// leave most of the device idle).  fork / join are recorded and waited for
+// within one call, under g_lane_mutex.
+struct SideLane {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+};
+constexpr int kMaxDevices = 64;
+constexpr int kSideLaneQueries = 131072; // fewer queries stay on one stream
+std::mutex g_lane_mutex;
+SideLane g_lanes[kMaxDevices];
+
+// The current device's lane, made at its first use (g_lane_mutex held).
+// PCA_BINNED_SIDE_STREAM=0 (diagnostic switch) keeps everything on the
+// caller's stream: `lane` stays null.
+hipError_t side_lane(SideLane *&lane) {
+  lane = nullptr;
+  const char *env = getenv("PCA_BINNED_SIDE_STREAM");
+  if (env != nullptr && env[0] == '0')
+    return hipSuccess;
+  int device = 0;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess)
+    return err;
+  if (device < 0 || device >= kMaxDevices)
+    return hipSuccess;
+  SideLane &mine = g_lanes[device];
+  if (mine.stream == nullptr) {
+    SideLane made;
+    if ((err = hipStreamCreateWithFlags(&made.stream, hipStreamNonBlocking)) !=
+        hipSuccess)
+      return err;
+    if ((err = hipEventCreateWithFlags(&made.fork, hipEventDisableTiming)) !=
+            hipSuccess ||
+        (err = hipEventCreateWithFlags(&made.join, hipEventDisableTiming)) !=
+            hipSuccess)
+      return err;
+    mine = made;
+  }
+  lane = &mine;
+  return hipSuccess;
+}
+
+// The tasks (blocks of 32 queries, long spans split) and their starting
+// order, from the sorted keys of the queries; results in `bins`.
+hipError_t order_tasks(const SearchInput &in, Bins &bins, uint32_t *task_keys,
+                       void *sort_temp, size_t sort_bytes, hipStream_t stream) {
+  const int blocks = plan_upper_bound(in.m, in.num_segments, kWave / 2);
+  const int slots = task_slots(blocks);
+  const int extra = slots - blocks;
+  int *extra_used = reinterpret_cast<int *>(task_keys);
+  int2 *desc = reinterpret_cast<int2 *>(task_keys + 64);
+  uint32_t *keys_in = task_keys + 64 + 2 * (size_t)slots;
+  uint32_t *vals_in = keys_in + slots;
+  uint32_t *keys_out = vals_in + slots;
+  uint32_t *vals_out = keys_out + slots;
+  // (what task_span_kernel reads)
+  BinnedParams p;
+  memset(&p, 0, sizeof(p));
+  p.ptr_y = in.ptr_y;
+  p.m = in.m;
+  p.num_segments = in.num_segments;
+  p.wave_start = bins.half_start;
+  p.keys_y = bins.keys_y;
+  p.code_bits = 3 * axis_bits(in.num_segments);
+  hipLaunchKernelGGL(task_slots_clear_kernel,
+                     dim3((extra + kBlock) / kBlock), dim3(kBlock), 0, stream,
+                     blocks, extra, extra_used, desc, keys_in, vals_in);
+  hipLaunchKernelGGL(task_span_kernel, dim3((blocks + kBlock - 1) / kBlock),
+                     dim3(kBlock), 0, stream, p, blocks, extra, extra_used,
+                     desc, keys_in, vals_in);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess)
+    return err;
+  err = rocprim::radix_sort_pairs(sort_temp, sort_bytes, keys_in, keys_out,
+                                  vals_in, vals_out, (unsigned int)slots, 0u,
+                                  32u, stream, false);
+  bins.task_desc = desc;
+  bins.task_order = vals_out;
+  bins.task_slots = slots;
+  // (the search kernels' grid: whole runs of 8 tasks on each of 8 XCDs)
+  bins.task_grid = (slots + 63) / 64 * 64;
+  bins.code_bits = p.code_bits;
+  return err;
+}
+
+// Orders rows and queries along the curve, copies the rows, builds the boxes;
+// with `with_tasks` also the tasks of 32 queries and their starting order.
+hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
+                        Bins &bins, hipStream_t stream) {
   const BinnedLayout lay = binned_layout(in.n, in.m, in.num_segments);
   char *cursor = static_cast<char *>(scratch);
   auto take = [&cursor](size_t bytes) {
@@ -825,9 +921,11 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
   };
   int *seg_box = static_cast<int *>(take(lay.seg_box));
   uint32_t *keys_a = static_cast<uint32_t *>(take(lay.keys_a));
+  uint32_t *keys_b = static_cast<uint32_t *>(take(lay.keys_b));
   uint32_t *keys_x = static_cast<uint32_t *>(take(lay.keys_x));
   uint32_t *keys_y = static_cast<uint32_t *>(take(lay.keys_y));
   uint32_t *vals_a = static_cast<uint32_t *>(take(lay.vals_a));
+  uint32_t *vals_b = static_cast<uint32_t *>(take(lay.vals_b));
   uint32_t *perm_x = static_cast<uint32_t *>(take(lay.perm_x));
   uint32_t *perm_y = static_cast<uint32_t *>(take(lay.perm_y));
   float4 *rows = static_cast<float4 *>(take(lay.rows));
@@ -840,11 +938,35 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
   int *half_start = static_cast<int *>(take(lay.half_start));
   uint32_t *task_keys = static_cast<uint32_t *>(take(lay.task_keys));
   void *sort_temp = take(lay.sort_temp);
-  size_t sort_bytes = lay.sort_temp;
+  void *side_temp = take(lay.side_temp);
 
   const float *x = static_cast<const float *>(in.x);
   const float *y = static_cast<const float *>(in.y);
   const int nseg = in.num_segments;
+  // the rows searching for themselves (the graph entry points): one order
+  // serves both sides
+  const bool self_search = in.y == in.x && in.m == in.n &&
+                           (in.ptr_y == in.ptr_x || in.ptr_x == nullptr);
+  if (self_search) {
+    keys_y = keys_x;
+    perm_y = perm_x;
+  }
+  bins.tile_start = tile_start;
+  bins.group_start = group_start;
+  bins.wave_start = wave_start;
+  bins.half_start = half_start;
+  bins.keys_x = keys_x;
+  bins.keys_y = keys_y;
+  bins.perm_y = perm_y;
+  bins.rows = rows;
+  bins.packed = packed;
+  bins.box = box;
+  bins.group_box = group_box;
+  bins.task_desc = nullptr;
+  bins.task_order = nullptr;
+  bins.task_slots = 0;
+  bins.task_grid = 0;
+  bins.code_bits = 0;
 
   hipError_t err;
   if ((err = launch_plan(in.ptr_x, in.n, nseg, kBinTile, tile_start, stream)) !=
@@ -870,32 +992,65 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
                        dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
                        seg_box);
   }
+  if ((err = hipGetLastError()) != hipSuccess)
+    return err;
+
+  // The queries' chain (keys, sort, tasks) runs beside the rows' chain: it
+  // forks off the caller's stream here and joins it again below - when it is
+  // long enough to pay for the two waits between streams (measured: 0.82 ->
+  // 0.77 ms for 1.03 M rows and 258 k queries, 0.68 -> 0.59 ms for 500 k
+  // queries among 1 M rows; a loss of 0.02 ms at 65 k queries).  When the
+  // rows' order serves the queries too, only the tasks are left to order,
+  // which follows the rows' sort on the caller's stream.
+  const bool beside = !self_search && in.m >= kSideLaneQueries;
+  std::unique_lock<std::mutex> lane_lock(g_lane_mutex, std::defer_lock);
+  SideLane *lane = nullptr;
+  hipStream_t side = stream;
+  auto fork = [&]() -> hipError_t {
+    lane_lock.lock();
+    hipError_t e = side_lane(lane);
+    if (e != hipSuccess || lane == nullptr)
+      return e;
+    if ((e = hipEventRecord(lane->fork, stream)) != hipSuccess)
+      return e;
+    side = lane->stream;
+    return hipStreamWaitEvent(side, lane->fork, 0);
+  };
+  auto queries_chain = [&]() -> hipError_t {
+    hipError_t e = hipSuccess;
+    if (!self_search) {
+      hipLaunchKernelGGL(morton_keys_kernel,
+                         dim3((in.m + kBlock - 1) / kBlock), dim3(kBlock), 0,
+                         side, y, in.ptr_y, in.m, in.d, nseg, seg_box,
+                         axis_bits(nseg), keys_b, vals_b);
+      if ((e = hipGetLastError()) != hipSuccess)
+        return e;
+      size_t bytes = lay.side_temp;
+      if ((e = sort_pairs(side_temp, bytes, keys_b, keys_y, vals_b, perm_y,
+                          in.m, nseg, side)) != hipSuccess)
+        return e;
+    }
+    if (with_tasks)
+      e = order_tasks(in, bins, task_keys, side_temp, lay.side_temp, side);
+    if (e == hipSuccess && lane != nullptr)
+      e = hipEventRecord(lane->join, side);
+    return e;
+  };
+  if (beside && (err = fork()) != hipSuccess)
+    return err;
+  if (!self_search && (err = queries_chain()) != hipSuccess)
+    return err;
   hipLaunchKernelGGL(morton_keys_kernel, dim3((in.n + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
                      seg_box, axis_bits(nseg), keys_a, vals_a);
   if ((err = hipGetLastError()) != hipSuccess)
     return err;
+  size_t sort_bytes = lay.sort_temp;
   if ((err = sort_pairs(sort_temp, sort_bytes, keys_a, keys_x, vals_a, perm_x,
                         in.n, nseg, stream)) != hipSuccess)
     return err;
-  // the rows searching for themselves (the graph entry points): one order
-  // serves both sides
-  const bool self_search = in.y == in.x && in.m == in.n &&
-                           (in.ptr_y == in.ptr_x || in.ptr_x == nullptr);
-  if (self_search) {
-    keys_y = keys_x;
-    perm_y = perm_x;
-  } else {
-    hipLaunchKernelGGL(morton_keys_kernel, dim3((in.m + kBlock - 1) / kBlock),
-                       dim3(kBlock), 0, stream, y, in.ptr_y, in.m, in.d, nseg,
-                       seg_box, axis_bits(nseg), keys_a, vals_a);
-    if ((err = hipGetLastError()) != hipSuccess)
-      return err;
-    sort_bytes = lay.sort_temp;
-    if ((err = sort_pairs(sort_temp, sort_bytes, keys_a, keys_y, vals_a,
-                          perm_y, in.m, nseg, stream)) != hipSuccess)
-      return err;
-  }
+  if (self_search && with_tasks && (err = queries_chain()) != hipSuccess)
+    return err;
   {
     const int per_block = kBlock / kBinTile;
     hipLaunchKernelGGL(gather_tiles_kernel,
@@ -913,22 +1068,9 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, Bins &bins,
   }
   if ((err = hipGetLastError()) != hipSuccess)
     return err;
-
-  bins.tile_start = tile_start;
-  bins.group_start = group_start;
-  bins.wave_start = wave_start;
-  bins.half_start = half_start;
-  bins.task_keys = task_keys;
-  bins.sort_temp = sort_temp;
-  bins.sort_bytes = lay.sort_temp;
-  bins.keys_x = keys_x;
-  bins.keys_y = keys_y;
-  bins.perm_y = perm_y;
-  bins.rows = rows;
-  bins.packed = packed;
-  bins.box = box;
-  bins.group_box = group_box;
-  return hipSuccess;
+  if (lane != nullptr)
+    err = hipStreamWaitEvent(stream, lane->join, 0);
+  return err;
 }
 
 void fill_params(BinnedParams &p, const SearchInput &in, const Bins &bins,
@@ -954,44 +1096,13 @@ void fill_params(BinnedParams &p, const SearchInput &in, const Bins &bins,
   p.out_dist = out.dist;
   p.out_count = out.count;
   p.out_nearest = nullptr;
-  p.task_order = nullptr;
-  p.task_desc = nullptr;
-  p.task_slots = 0;
-  p.code_bits = 0;
+  p.task_order = bins.task_order;
+  p.task_desc = bins.task_desc;
+  p.task_slots = bins.task_slots;
+  p.code_bits = bins.code_bits;
 }
 
 } // namespace
-
-// p.wave_start = blocks of 32 queries (`blocks`: their upper bound); leaves
-// p.task_desc and p.task_order set and returns the number of task slots.
-hipError_t order_tasks(BinnedParams &p, const Bins &bins, int blocks,
-                       int num_segments, int &slots, hipStream_t stream) {
-  slots = task_slots(blocks);
-  const int extra = slots - blocks;
-  int *extra_used = reinterpret_cast<int *>(bins.task_keys);
-  int2 *desc = reinterpret_cast<int2 *>(bins.task_keys + 64);
-  uint32_t *keys_in = bins.task_keys + 64 + 2 * (size_t)slots;
-  uint32_t *vals_in = keys_in + slots;
-  uint32_t *keys_out = vals_in + slots;
-  uint32_t *vals_out = keys_out + slots;
-  p.code_bits = 3 * axis_bits(num_segments);
-  hipLaunchKernelGGL(task_slots_clear_kernel,
-                     dim3((extra + kBlock) / kBlock), dim3(kBlock), 0, stream,
-                     blocks, extra, extra_used, desc, keys_in, vals_in);
-  hipLaunchKernelGGL(task_span_kernel, dim3((blocks + kBlock - 1) / kBlock),
-                     dim3(kBlock), 0, stream, p, blocks, extra, extra_used,
-                     desc, keys_in, vals_in);
-  size_t bytes = bins.sort_bytes;
-  const hipError_t err = rocprim::radix_sort_pairs(
-      bins.sort_temp, bytes, keys_in, keys_out, vals_in, vals_out,
-      (unsigned int)slots, 0u, 32u, stream, false);
-  p.task_desc = desc;
-  p.task_order = vals_out;
-  p.task_slots = slots;
-  // (the search kernels' grid: whole runs of 8 tasks on each of 8 XCDs)
-  slots = (slots + 63) / 64 * 64;
-  return err;
-}
 
 bool knn_binned_supported(int d, int k, bool cosine) {
   return !cosine && d >= 1 && d <= 3 && k >= 1 && k <= 64;
@@ -1006,29 +1117,22 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
                              hipEvent_t time_stop, hipStream_t stream) {
   if (time_start)
     (void)hipEventRecord(time_start, stream);
+  // (diagnostic switch: the vector-ALU scan instead of the matrix-core one)
+  // (lists of more than 32 entries exist for the matrix-core scan only)
+  const char *env = getenv("PCA_KNN_BINNED_MATRIX_CORES");
+  const bool matrix_cores = k > 32 || !(env != nullptr && env[0] == '0');
   Bins bins;
-  const hipError_t err = prepare_bins(in, scratch, bins, stream);
+  const hipError_t err = prepare_bins(in, scratch, matrix_cores, bins, stream);
   if (err != hipSuccess)
     return err;
   BinnedParams p;
   fill_params(p, in, bins, out);
   p.k = k;
-  // (diagnostic switch: the vector-ALU scan instead of the matrix-core one)
-  // (lists of more than 32 entries exist for the matrix-core scan only)
-  const char *env = getenv("PCA_KNN_BINNED_MATRIX_CORES");
-  const bool matrix_cores = k > 32 || !(env != nullptr && env[0] == '0');
-  const int per_task = matrix_cores ? kWave / 2 : kWave;
   if (matrix_cores)
     p.wave_start = bins.half_start;
-  const int waves = plan_upper_bound(in.m, in.num_segments, per_task);
+  const int waves = plan_upper_bound(in.m, in.num_segments, kWave);
   const int grid = (waves + kBlock / kWave - 1) / (kBlock / kWave);
-  int slots = 0;
-  if (matrix_cores) {
-    const hipError_t order_err =
-        order_tasks(p, bins, waves, in.num_segments, slots, stream);
-    if (order_err != hipSuccess)
-      return order_err;
-  }
+  const int slots = bins.task_grid;
 #define PCA_BINNED_LAUNCH(K_)                                                  \
   do {                                                                         \
     if (matrix_cores)                                                          \
@@ -1072,7 +1176,7 @@ hipError_t launch_nearest_binned(const SearchInput &in, void *scratch,
   if (time_start)
     (void)hipEventRecord(time_start, stream);
   Bins bins;
-  const hipError_t err = prepare_bins(in, scratch, bins, stream);
+  const hipError_t err = prepare_bins(in, scratch, true, bins, stream);
   if (err != hipSuccess)
     return err;
   BinnedParams p;
@@ -1081,13 +1185,7 @@ hipError_t launch_nearest_binned(const SearchInput &in, void *scratch,
   p.k = 1;
   p.out_nearest = out;
   p.wave_start = bins.half_start;
-  const int waves = plan_upper_bound(in.m, in.num_segments, kWave / 2);
-  int slots = 0;
-  const hipError_t order_err =
-      order_tasks(p, bins, waves, in.num_segments, slots, stream);
-  if (order_err != hipSuccess)
-    return order_err;
-  hipLaunchKernelGGL((knn_binned_mc_kernel<1, true>), dim3(slots),
+  hipLaunchKernelGGL((knn_binned_mc_kernel<1, true>), dim3(bins.task_grid),
                      dim3(kBinMcBlock), 0, stream, p);
   if (time_stop)
     (void)hipEventRecord(time_stop, stream);
@@ -1102,7 +1200,7 @@ hipError_t launch_radius_binned(const SearchInput &in, float r2,
                                 bool ignore_same_index, void *scratch,
                                 const DenseResult &out, hipStream_t stream) {
   Bins bins;
-  const hipError_t err = prepare_bins(in, scratch, bins, stream);
+  const hipError_t err = prepare_bins(in, scratch, false, bins, stream);
   if (err != hipSuccess)
     return err;
   BinnedParams p;

@@ -148,6 +148,41 @@ def test_full_size_against_the_scanning_kernels():
     assert torch.equal(da.view(torch.int32), db.view(torch.int32))
 
 
+def test_queries_ordered_beside_the_rows(monkeypatch):
+    """From 131,072 queries on, the queries are ordered on a second stream
+    while the rows are ordered on the caller's: same edges with and without
+    it, call after call, on the default stream and on another one."""
+    c = testing.lidar_scans(0)
+    x, y = c["x"].to(DEV), c["y"].to(DEV)
+    px = testing.pointers(c["batch_x"], c["batch_size"]).to(DEV)
+    py = testing.pointers(c["batch_y"], c["batch_size"]).to(DEV)
+    monkeypatch.setenv("PCA_BINNED_SIDE_STREAM", "0")
+    want, want_dist = capi.knn_edges(x, y, px, py, 16, want_dist=True,
+                                     binned=True)
+    monkeypatch.delenv("PCA_BINNED_SIDE_STREAM")
+    other = torch.cuda.Stream()
+    for stream in (torch.cuda.current_stream(), other, other):
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            # (other work of the caller's stream right before and after)
+            noise = torch.rand(1 << 20, device=DEV).sort().values
+            got, got_dist = capi.knn_edges(x, y, px, py, 16, want_dist=True,
+                                           binned=True)
+            total = got.sum() + noise.numel()
+        torch.cuda.current_stream().wait_stream(stream)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+        assert torch.equal(got_dist.view(torch.int32),
+                           want_dist.view(torch.int32))
+        assert int(total) == int(want.sum()) + (1 << 20)
+    # the nearest search: 1M searching rows
+    monkeypatch.setenv("PCA_BINNED_SIDE_STREAM", "0")
+    want = capi.nearest_rows(x, y, px, py, binned=True)
+    monkeypatch.delenv("PCA_BINNED_SIDE_STREAM")
+    for _ in range(2):
+        assert torch.equal(capi.nearest_rows(x, y, px, py, binned=True), want)
+
+
 def test_uniform_clouds_against_the_scanning_kernels():
     c = testing.uniform_batched(0)
     x = c["x"].to(DEV)
