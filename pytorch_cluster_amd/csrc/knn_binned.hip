@@ -727,22 +727,35 @@ int axis_bits(int num_segments) {
   return std::min(10, (32 - segment_bits(num_segments)) / 3);
 }
 
+// rocPRIM's radix sort with this file's choices (measured on 1.03 M pairs
+// with 30-bit keys: the library's default - merge sort up to 2^20 items, 19
+// launches - 170 us; its one-sweep radix sort as configured by default
+// 140 us; the same with workgroups of 1,024 threads x 8 items and the
+// match-based ranking 109 us, and 98 us with 10 bits per pass, which saves
+// the fourth pass).  Below 200,000 items the merge sort is quicker (54 us
+// against 68 us at 131,072).
+template <unsigned int RadixBits>
+using SortConfig = rocprim::radix_sort_config<
+    rocprim::default_config, rocprim::default_config,
+    rocprim::radix_sort_onesweep_config<
+        rocprim::kernel_config<256, 12>, rocprim::kernel_config<1024, 8>,
+        RadixBits, rocprim::block_radix_rank_algorithm::match>,
+    200000>;
+
 hipError_t sort_pairs(void *temp, size_t &temp_bytes, const uint32_t *keys_in,
                       uint32_t *keys_out, const uint32_t *vals_in,
                       uint32_t *vals_out, int count, int num_segments,
                       hipStream_t stream) {
-  const int bits = segment_bits(num_segments) + 3 * axis_bits(num_segments);
-  // (rocPRIM's default turns to merge sort up to 2^20 items - 19 launches for
-  // a million rows; measured here, its one-sweep radix sort is quicker from a
-  // few hundred thousand rows on and slower below)
-  using Config =
-      rocprim::radix_sort_config<rocprim::default_config,
-                                 rocprim::default_config,
-                                 rocprim::default_config, 300000>;
-  return rocprim::radix_sort_pairs<Config>(temp, temp_bytes, keys_in, keys_out,
-                                   vals_in, vals_out, (unsigned int)count, 0u,
-                                   (unsigned int)std::max(bits, 1), stream,
-                                   false);
+  const unsigned int bits = (unsigned int)std::max(
+      segment_bits(num_segments) + 3 * axis_bits(num_segments), 1);
+  // (10 bits per pass where that takes fewer passes than 8)
+  if ((bits + 9) / 10 < (bits + 7) / 8)
+    return rocprim::radix_sort_pairs<SortConfig<10>>(
+        temp, temp_bytes, keys_in, keys_out, vals_in, vals_out,
+        (unsigned int)count, 0u, bits, stream, false);
+  return rocprim::radix_sort_pairs<SortConfig<8>>(
+      temp, temp_bytes, keys_in, keys_out, vals_in, vals_out,
+      (unsigned int)count, 0u, bits, stream, false);
 }
 
 // Task slots for `blocks` blocks of 32 queries: one each, and half as many
