@@ -214,6 +214,48 @@ __device__ __forceinline__ int xcd_swizzle(int block, int grid) {
   return (block & 7) * (grid >> 3) + (block >> 3);
 }
 
+// Work items of ragged segments, by a single workgroup of kPlanThreads
+// threads: work_start[b] = exclusive scan of ceil(rows of segment b /
+// per_item), work_start[num_segments] = their total.  ptr == nullptr: one
+// segment of m rows.  `partial`: kPlanThreads ints of LDS.
+constexpr int kPlanThreads = 1024;
+__device__ __forceinline__ void
+plan_segments(const int64_t *__restrict__ ptr, int m, int num_segments,
+              int per_item, int *__restrict__ work_start, int *partial) {
+  const int tid = threadIdx.x;
+  // contiguous chunk of segments per thread
+  const int per_thread = (num_segments + kPlanThreads - 1) / kPlanThreads;
+  const int b0 = min(tid * per_thread, num_segments);
+  const int b1 = min(b0 + per_thread, num_segments);
+
+  int sum = 0;
+  for (int b = b0; b < b1; ++b) {
+    const int64_t lo = ptr ? ptr[b] : 0;
+    const int64_t hi = ptr ? ptr[b + 1] : m;
+    const int len = (int)max((int64_t)0, hi - lo);
+    sum += (len + per_item - 1) / per_item;
+  }
+  partial[tid] = sum;
+  __syncthreads();
+  // Hillis-Steele inclusive scan over the partial sums
+  for (int off = 1; off < kPlanThreads; off <<= 1) {
+    const int v = tid >= off ? partial[tid - off] : 0;
+    __syncthreads();
+    partial[tid] += v;
+    __syncthreads();
+  }
+  int run = partial[tid] - sum; // exclusive prefix of this thread's chunk
+  for (int b = b0; b < b1; ++b) {
+    work_start[b] = run;
+    const int64_t lo = ptr ? ptr[b] : 0;
+    const int64_t hi = ptr ? ptr[b + 1] : m;
+    const int len = (int)max((int64_t)0, hi - lo);
+    run += (len + per_item - 1) / per_item;
+  }
+  if (tid == kPlanThreads - 1)
+    work_start[num_segments] = partial[tid];
+}
+
 } // namespace pca
 
 // experiment switch: -DPCA_NO_SWIZZLE maps workgroup ids to tiles directly

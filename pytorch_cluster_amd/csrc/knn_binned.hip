@@ -81,11 +81,37 @@ __device__ __forceinline__ int find_segment64(const int64_t *__restrict__ ptr,
   return lo;
 }
 
-// seg_box: [num_segments][6] = lower corner, upper corner (ordered integers)
-__global__ void seg_box_init_kernel(int *seg_box, int count) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < count)
-    seg_box[i] = (i % 6) < 3 ? INT_MAX : INT_MIN;
+// The first launch of a binned search (a call starts with kernels so short
+// that the host's launch rate sets the pace: one launch instead of five):
+// workgroups 0-3 count the work items of the segments - tiles and groups of
+// tiles of x, tasks of 64 and of 32 queries of y -, the others empty the
+// segment boxes.  seg_box: [num_segments][6] = lower corner, upper corner
+// (ordered integers).
+struct BinsSetup {
+  const int64_t *ptr_x, *ptr_y;
+  int n, m, num_segments;
+  int *tile_start, *group_start, *wave_start, *half_start;
+  int *seg_box;
+};
+__global__ __launch_bounds__(kPlanThreads) void bins_setup_kernel(BinsSetup s) {
+  __shared__ int partial[kPlanThreads];
+  const int job = blockIdx.x; // (uniform over the workgroup)
+  if (job == 0) {
+    plan_segments(s.ptr_x, s.n, s.num_segments, kBinTile, s.tile_start,
+                  partial);
+  } else if (job == 1) {
+    plan_segments(s.ptr_x, s.n, s.num_segments, kBinTile * kBinGroup,
+                  s.group_start, partial);
+  } else if (job == 2) {
+    plan_segments(s.ptr_y, s.m, s.num_segments, kWave, s.wave_start, partial);
+  } else if (job == 3) {
+    plan_segments(s.ptr_y, s.m, s.num_segments, kWave / 2, s.half_start,
+                  partial);
+  } else {
+    const int i = (job - 4) * kPlanThreads + (int)threadIdx.x;
+    if (i < 6 * s.num_segments)
+      s.seg_box[i] = (i % 6) < 3 ? INT_MAX : INT_MIN;
+  }
 }
 
 // Bounding box of the finite coordinates of every segment; grid (parts,
@@ -982,20 +1008,22 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
   bins.code_bits = 0;
 
   hipError_t err;
-  if ((err = launch_plan(in.ptr_x, in.n, nseg, kBinTile, tile_start, stream)) !=
-      hipSuccess)
-    return err;
-  if ((err = launch_plan(in.ptr_x, in.n, nseg, kBinTile * kBinGroup,
-                         group_start, stream)) != hipSuccess)
-    return err;
-  if ((err = launch_plan(in.ptr_y, in.m, nseg, kWave, wave_start, stream)) !=
-      hipSuccess)
-    return err;
-  if ((err = launch_plan(in.ptr_y, in.m, nseg, kWave / 2, half_start,
-                         stream)) != hipSuccess)
-    return err;
-  hipLaunchKernelGGL(seg_box_init_kernel, dim3((6 * nseg + kBlock - 1) / kBlock),
-                     dim3(kBlock), 0, stream, seg_box, 6 * nseg);
+  {
+    BinsSetup setup;
+    setup.ptr_x = in.ptr_x;
+    setup.ptr_y = in.ptr_y;
+    setup.n = in.n;
+    setup.m = in.m;
+    setup.num_segments = nseg;
+    setup.tile_start = tile_start;
+    setup.group_start = group_start;
+    setup.wave_start = wave_start;
+    setup.half_start = half_start;
+    setup.seg_box = seg_box;
+    hipLaunchKernelGGL(bins_setup_kernel,
+                       dim3(4 + (6 * nseg + kPlanThreads - 1) / kPlanThreads),
+                       dim3(kPlanThreads), 0, stream, setup);
+  }
   {
     // enough workgroups per segment to fill the device when segments are few
     const int parts = std::max(
@@ -1010,9 +1038,10 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
 
   // The queries' chain (keys, sort, tasks) runs beside the rows' chain: it
   // forks off the caller's stream here and joins it again below - when it is
-  // long enough to pay for the two waits between streams (measured: 0.82 ->
-  // 0.77 ms for 1.03 M rows and 258 k queries, 0.68 -> 0.59 ms for 500 k
-  // queries among 1 M rows; a loss of 0.02 ms at 65 k queries).  When the
+  // long enough to pay for the two waits between streams (measured, with
+  // rocPRIM's default sort configuration: 0.82 -> 0.77 ms for 1.03 M rows and
+  // 258 k queries, 0.68 -> 0.59 ms for 500 k queries among 1 M rows; a loss
+  // of 0.02 ms at 65 k queries).  When the
   // rows' order serves the queries too, only the tasks are left to order,
   // which follows the rows' sort on the caller's stream.
   const bool beside = !self_search && in.m >= kSideLaneQueries;
@@ -1024,13 +1053,14 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
     hipError_t e = side_lane(lane);
     if (e != hipSuccess || lane == nullptr)
       return e;
-    if ((e = hipEventRecord(lane->fork, stream)) != hipSuccess)
-      return e;
     side = lane->stream;
-    return hipStreamWaitEvent(side, lane->fork, 0);
+    return hipEventRecord(lane->fork, stream);
   };
   auto queries_chain = [&]() -> hipError_t {
     hipError_t e = hipSuccess;
+    if (lane != nullptr &&
+        (e = hipStreamWaitEvent(side, lane->fork, 0)) != hipSuccess)
+      return e;
     if (!self_search) {
       hipLaunchKernelGGL(morton_keys_kernel,
                          dim3((in.m + kBlock - 1) / kBlock), dim3(kBlock), 0,
@@ -1049,9 +1079,12 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
       e = hipEventRecord(lane->join, side);
     return e;
   };
+  // (the fork is where the segment boxes are done; the longer of the two
+  // chains is handed to the device first)
   if (beside && (err = fork()) != hipSuccess)
     return err;
-  if (!self_search && (err = queries_chain()) != hipSuccess)
+  const bool queries_first = beside && in.m > in.n;
+  if (queries_first && (err = queries_chain()) != hipSuccess)
     return err;
   hipLaunchKernelGGL(morton_keys_kernel, dim3((in.n + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
@@ -1062,7 +1095,8 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
   if ((err = sort_pairs(sort_temp, sort_bytes, keys_a, keys_x, vals_a, perm_x,
                         in.n, nseg, stream)) != hipSuccess)
     return err;
-  if (self_search && with_tasks && (err = queries_chain()) != hipSuccess)
+  if (!queries_first && (!self_search || with_tasks) &&
+      (err = queries_chain()) != hipSuccess)
     return err;
   {
     const int per_block = kBlock / kBinTile;

@@ -19,45 +19,12 @@ namespace pca {
 
 namespace {
 
-constexpr int kPlanThreads = 1024;
-
 // Single workgroup: exclusive scan of ceil(m_b / per_item) over segments.
 __global__ __launch_bounds__(kPlanThreads) void plan_kernel(
     const int64_t *__restrict__ ptr_y, int m, int num_segments, int per_item,
     int *__restrict__ work_start) {
   __shared__ int partial[kPlanThreads];
-  const int tid = threadIdx.x;
-  // contiguous chunk of segments per thread
-  const int per_thread = (num_segments + kPlanThreads - 1) / kPlanThreads;
-  const int b0 = min(tid * per_thread, num_segments);
-  const int b1 = min(b0 + per_thread, num_segments);
-
-  int sum = 0;
-  for (int b = b0; b < b1; ++b) {
-    int64_t lo = ptr_y ? ptr_y[b] : 0;
-    int64_t hi = ptr_y ? ptr_y[b + 1] : m;
-    int len = (int)max((int64_t)0, hi - lo);
-    sum += (len + per_item - 1) / per_item;
-  }
-  partial[tid] = sum;
-  __syncthreads();
-  // Hillis-Steele inclusive scan over the 1024 partial sums
-  for (int off = 1; off < kPlanThreads; off <<= 1) {
-    int v = tid >= off ? partial[tid - off] : 0;
-    __syncthreads();
-    partial[tid] += v;
-    __syncthreads();
-  }
-  int run = partial[tid] - sum; // exclusive prefix of this thread's chunk
-  for (int b = b0; b < b1; ++b) {
-    work_start[b] = run;
-    int64_t lo = ptr_y ? ptr_y[b] : 0;
-    int64_t hi = ptr_y ? ptr_y[b + 1] : m;
-    int len = (int)max((int64_t)0, hi - lo);
-    run += (len + per_item - 1) / per_item;
-  }
-  if (tid == kPlanThreads - 1)
-    work_start[num_segments] = partial[tid];
+  plan_segments(ptr_y, m, num_segments, per_item, work_start, partial);
 }
 
 // ---- compaction -----------------------------------------------------------
