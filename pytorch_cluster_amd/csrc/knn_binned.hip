@@ -85,13 +85,18 @@ __device__ __forceinline__ int find_segment64(const int64_t *__restrict__ ptr,
 // that the host's launch rate sets the pace: one launch instead of five):
 // workgroups 0-3 count the work items of the segments - tiles and groups of
 // tiles of x, tasks of 64 and of 32 queries of y -, the others empty the
-// segment boxes.  seg_box: [num_segments][6] = lower corner, upper corner
-// (ordered integers).
+// segment boxes and the extra task slots.  seg_box: [num_segments][6] = lower
+// corner, upper corner (ordered integers).
 struct BinsSetup {
   const int64_t *ptr_x, *ptr_y;
   int n, m, num_segments;
   int *tile_start, *group_start, *wave_start, *half_start;
   int *seg_box;
+  // task slots (task_span_kernel's; task_extra == 0: no tasks wanted)
+  int task_blocks, task_extra;
+  int *extra_used;
+  int2 *task_desc;
+  uint32_t *task_keys, *task_vals;
 };
 __global__ __launch_bounds__(kPlanThreads) void bins_setup_kernel(BinsSetup s) {
   __shared__ int partial[kPlanThreads];
@@ -111,6 +116,14 @@ __global__ __launch_bounds__(kPlanThreads) void bins_setup_kernel(BinsSetup s) {
     const int i = (job - 4) * kPlanThreads + (int)threadIdx.x;
     if (i < 6 * s.num_segments)
       s.seg_box[i] = (i % 6) < 3 ? INT_MAX : INT_MIN;
+    // the extra task slots start out unused
+    if (i == 0 && s.extra_used != nullptr)
+      *s.extra_used = 0;
+    if (i < s.task_extra) {
+      s.task_desc[s.task_blocks + i] = make_int2(0, 0);
+      s.task_keys[s.task_blocks + i] = 0xffffffffu;
+      s.task_vals[s.task_blocks + i] = (uint32_t)(s.task_blocks + i);
+    }
   }
 }
 
@@ -222,6 +235,12 @@ __global__ __launch_bounds__(kBlock) void gather_tiles_kernel(
     uint4 *__restrict__ packed, Box *__restrict__ box) {
   const int gt = (blockIdx.x * kBlock + threadIdx.x) / kBinTile;
   const int r = threadIdx.x & (kBinTile - 1);
+  // behind the last row a tile of rows that never pass the filter (operand
+  // w = NaN), so that a fetch of a whole tile stays inside the copy
+  if (blockIdx.x == 0 && threadIdx.x < kBinTile) {
+    packed[(size_t)(n + r) * 2] = make_uint4(0u, 0x7fc00000u, 0u, 0u);
+    packed[(size_t)(n + r) * 2 + 1] = make_uint4(0u, 0u, 0u, 0u);
+  }
   if (gt >= tile_start[num_segments])
     return;
   const int seg = find_segment(tile_start, num_segments, gt);
@@ -266,16 +285,6 @@ __global__ __launch_bounds__(kBlock) void gather_tiles_kernel(
   if (r == 0) {
     box[gt].min_row = min_row;
     box[gt].pad = 0u;
-  }
-}
-
-// A tile of rows behind the last one that never pass the filter (operand
-// w = NaN), so that a fetch of a whole tile stays inside the copy.
-__global__ void pad_packed_kernel(uint4 *__restrict__ packed, int n) {
-  const int r = threadIdx.x;
-  if (r < kBinTile) {
-    packed[(size_t)(n + r) * 2] = make_uint4(0u, 0x7fc00000u, 0u, 0u);
-    packed[(size_t)(n + r) * 2 + 1] = make_uint4(0u, 0u, 0u, 0u);
   }
 }
 
@@ -906,17 +915,36 @@ hipError_t side_lane(SideLane *&lane) {
 
 // The tasks (blocks of 32 queries, long spans split) and their starting
 // order, from the sorted keys of the queries; results in `bins`.
+// The pieces of the task-slot buffer (6 words per slot + 64).
+struct TaskBuffers {
+  int blocks, slots;
+  int *extra_used;
+  int2 *desc;
+  uint32_t *keys_in, *vals_in, *keys_out, *vals_out;
+};
+TaskBuffers task_buffers(uint32_t *task_keys, int m, int num_segments) {
+  TaskBuffers t;
+  t.blocks = plan_upper_bound(m, num_segments, kWave / 2);
+  t.slots = task_slots(t.blocks);
+  t.extra_used = reinterpret_cast<int *>(task_keys);
+  t.desc = reinterpret_cast<int2 *>(task_keys + 64);
+  t.keys_in = task_keys + 64 + 2 * (size_t)t.slots;
+  t.vals_in = t.keys_in + t.slots;
+  t.keys_out = t.vals_in + t.slots;
+  t.vals_out = t.keys_out + t.slots;
+  return t;
+}
+
+// (the extra slots were cleared by bins_setup_kernel)
 hipError_t order_tasks(const SearchInput &in, Bins &bins, uint32_t *task_keys,
                        void *sort_temp, size_t sort_bytes, hipStream_t stream) {
-  const int blocks = plan_upper_bound(in.m, in.num_segments, kWave / 2);
-  const int slots = task_slots(blocks);
+  const TaskBuffers t = task_buffers(task_keys, in.m, in.num_segments);
+  const int blocks = t.blocks, slots = t.slots;
   const int extra = slots - blocks;
-  int *extra_used = reinterpret_cast<int *>(task_keys);
-  int2 *desc = reinterpret_cast<int2 *>(task_keys + 64);
-  uint32_t *keys_in = task_keys + 64 + 2 * (size_t)slots;
-  uint32_t *vals_in = keys_in + slots;
-  uint32_t *keys_out = vals_in + slots;
-  uint32_t *vals_out = keys_out + slots;
+  int *extra_used = t.extra_used;
+  int2 *desc = t.desc;
+  uint32_t *keys_in = t.keys_in, *vals_in = t.vals_in;
+  uint32_t *keys_out = t.keys_out, *vals_out = t.vals_out;
   // (what task_span_kernel reads)
   BinnedParams p;
   memset(&p, 0, sizeof(p));
@@ -926,9 +954,6 @@ hipError_t order_tasks(const SearchInput &in, Bins &bins, uint32_t *task_keys,
   p.wave_start = bins.half_start;
   p.keys_y = bins.keys_y;
   p.code_bits = 3 * axis_bits(in.num_segments);
-  hipLaunchKernelGGL(task_slots_clear_kernel,
-                     dim3((extra + kBlock) / kBlock), dim3(kBlock), 0, stream,
-                     blocks, extra, extra_used, desc, keys_in, vals_in);
   hipLaunchKernelGGL(task_span_kernel, dim3((blocks + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, p, blocks, extra, extra_used,
                      desc, keys_in, vals_in);
@@ -1020,8 +1045,16 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
     setup.wave_start = wave_start;
     setup.half_start = half_start;
     setup.seg_box = seg_box;
+    const TaskBuffers t = task_buffers(task_keys, in.m, nseg);
+    setup.task_blocks = t.blocks;
+    setup.task_extra = with_tasks ? t.slots - t.blocks : 0;
+    setup.extra_used = with_tasks ? t.extra_used : nullptr;
+    setup.task_desc = t.desc;
+    setup.task_keys = t.keys_in;
+    setup.task_vals = t.vals_in;
+    const int resets = std::max(6 * nseg, setup.task_extra);
     hipLaunchKernelGGL(bins_setup_kernel,
-                       dim3(4 + (6 * nseg + kPlanThreads - 1) / kPlanThreads),
+                       dim3(4 + (resets + kPlanThreads - 1) / kPlanThreads),
                        dim3(kPlanThreads), 0, stream, setup);
   }
   {
@@ -1104,8 +1137,6 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
                        dim3((lay.tiles_bound + per_block - 1) / per_block),
                        dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
                        tile_start, perm_x, rows, packed, box);
-    hipLaunchKernelGGL(pad_packed_kernel, dim3(1), dim3(kWave), 0, stream,
-                       packed, in.n);
     const int groups_per_block = kBlock / kWave;
     hipLaunchKernelGGL(
         group_boxes_kernel,

@@ -324,21 +324,6 @@ __global__ __launch_bounds__(kBlock) void task_span_kernel(
   vals[block] = (uint32_t)block;
 }
 
-// Extra slots start out unused (before task_span_kernel).
-__global__ __launch_bounds__(kBlock) void task_slots_clear_kernel(
-    int bound, int extra, int *__restrict__ extra_used,
-    int2 *__restrict__ desc, uint32_t *__restrict__ keys,
-    uint32_t *__restrict__ vals) {
-  const int i = blockIdx.x * kBlock + threadIdx.x;
-  if (i == 0)
-    *extra_used = 0;
-  if (i < extra) {
-    desc[bound + i] = make_int2(0, 0);
-    keys[bound + i] = 0xffffffffu;
-    vals[bound + i] = (uint32_t)(bound + i);
-  }
-}
-
 // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: runs
 // of 8 consecutive tasks (neighbours along the curve, which fetch the same
 // tiles) go to the same XCD, one after the other.  Maps a workgroup number to
