@@ -96,7 +96,6 @@ struct BinsSetup {
   int task_blocks, task_extra;
   int *extra_used;
   int2 *task_desc;
-  uint32_t *task_keys, *task_vals;
 };
 __global__ __launch_bounds__(kPlanThreads) void bins_setup_kernel(BinsSetup s) {
   __shared__ int partial[kPlanThreads];
@@ -119,11 +118,8 @@ __global__ __launch_bounds__(kPlanThreads) void bins_setup_kernel(BinsSetup s) {
     // the extra task slots start out unused
     if (i == 0 && s.extra_used != nullptr)
       *s.extra_used = 0;
-    if (i < s.task_extra) {
+    if (i < s.task_extra)
       s.task_desc[s.task_blocks + i] = make_int2(0, 0);
-      s.task_keys[s.task_blocks + i] = 0xffffffffu;
-      s.task_vals[s.task_blocks + i] = (uint32_t)(s.task_blocks + i);
-    }
   }
 }
 
@@ -803,6 +799,13 @@ int task_slots(int blocks) {
   return blocks <= 6144 ? blocks + (blocks / 6) * 3 : blocks;
 }
 
+// Words of the task-slot buffer (see TaskBuffers).
+size_t task_buffer_words(int m, int num_segments) {
+  const int blocks = plan_upper_bound(m, num_segments, kWave / 2);
+  const int groups = (blocks + kBlock - 1) / kBlock;
+  return 64 + 4 * (size_t)task_slots(blocks) + (size_t)kTaskClasses * groups;
+}
+
 BinnedLayout binned_layout(int n, int m, int num_segments) {
   BinnedLayout w;
   w.seg_box = align256(sizeof(int) * 6 * (size_t)num_segments);
@@ -827,28 +830,19 @@ BinnedLayout binned_layout(int n, int m, int num_segments) {
   w.group_start = align256(sizeof(int) * (size_t)(num_segments + 1));
   w.wave_start = align256(sizeof(int) * (size_t)(num_segments + 1));
   w.half_start = align256(sizeof(int) * (size_t)(num_segments + 1));
-  // per task slot: descriptor (2 words), span key and slot number, unsorted
-  // and sorted (4 words)
-  w.task_keys = align256(
-      sizeof(uint32_t) *
-      (6 * (size_t)task_slots(plan_upper_bound(m, num_segments, kWave / 2)) +
-       64));
-  size_t tx = 0, ty = 0, tt = 0;
+  // per task slot: descriptor (2 words), class, place in the starting order;
+  // a histogram of the classes per kBlock blocks
+  w.task_keys = align256(sizeof(uint32_t) * task_buffer_words(m, num_segments));
+  size_t tx = 0, ty = 0;
   const hipError_t ex = sort_pairs(nullptr, tx, nullptr, nullptr, nullptr,
                                    nullptr, n, num_segments, nullptr);
   const hipError_t ey = sort_pairs(nullptr, ty, nullptr, nullptr, nullptr,
                                    nullptr, m, num_segments, nullptr);
-  // (the task slots, sorted on all 32 bits by order_tasks)
-  const hipError_t et = rocprim::radix_sort_pairs(
-      nullptr, tt, (const uint32_t *)nullptr, (uint32_t *)nullptr,
-      (const uint32_t *)nullptr, (uint32_t *)nullptr,
-      (unsigned int)task_slots(plan_upper_bound(m, num_segments, kWave / 2)),
-      0u, 32u, nullptr, false);
   // (a failed size query leaves a size no workspace can meet)
-  const bool sized = ex == hipSuccess && ey == hipSuccess && et == hipSuccess;
+  const bool sized = ex == hipSuccess && ey == hipSuccess;
   w.sort_temp = sized ? align256(tx) : ~(size_t)0 / 2;
-  // (the queries and the task slots are sorted beside the rows' stream)
-  w.side_temp = sized ? align256(std::max(ty, tt)) : 0;
+  // (the queries are sorted beside the rows' stream)
+  w.side_temp = sized ? align256(ty) : 0;
   return w;
 }
 
@@ -915,36 +909,34 @@ hipError_t side_lane(SideLane *&lane) {
 
 // The tasks (blocks of 32 queries, long spans split) and their starting
 // order, from the sorted keys of the queries; results in `bins`.
-// The pieces of the task-slot buffer (6 words per slot + 64).
+// The pieces of the task-slot buffer.
 struct TaskBuffers {
-  int blocks, slots;
+  int blocks, slots, groups; // groups: workgroups of kBlock blocks
   int *extra_used;
   int2 *desc;
-  uint32_t *keys_in, *vals_in, *keys_out, *vals_out;
+  uint32_t *cls, *order;
+  int *hist;
 };
 TaskBuffers task_buffers(uint32_t *task_keys, int m, int num_segments) {
   TaskBuffers t;
   t.blocks = plan_upper_bound(m, num_segments, kWave / 2);
   t.slots = task_slots(t.blocks);
+  t.groups = (t.blocks + kBlock - 1) / kBlock;
   t.extra_used = reinterpret_cast<int *>(task_keys);
   t.desc = reinterpret_cast<int2 *>(task_keys + 64);
-  t.keys_in = task_keys + 64 + 2 * (size_t)t.slots;
-  t.vals_in = t.keys_in + t.slots;
-  t.keys_out = t.vals_in + t.slots;
-  t.vals_out = t.keys_out + t.slots;
+  t.cls = task_keys + 64 + 2 * (size_t)t.slots;
+  t.order = t.cls + t.slots;
+  t.hist = reinterpret_cast<int *>(t.order + t.slots);
   return t;
 }
 
-// (the extra slots were cleared by bins_setup_kernel)
+// The tasks (blocks of 32 queries, long spans split) and their starting
+// order, from the sorted keys of the queries; results in `bins`.  (The extra
+// slots were cleared by bins_setup_kernel.)
 hipError_t order_tasks(const SearchInput &in, Bins &bins, uint32_t *task_keys,
-                       void *sort_temp, size_t sort_bytes, hipStream_t stream) {
+                       hipStream_t stream) {
   const TaskBuffers t = task_buffers(task_keys, in.m, in.num_segments);
-  const int blocks = t.blocks, slots = t.slots;
-  const int extra = slots - blocks;
-  int *extra_used = t.extra_used;
-  int2 *desc = t.desc;
-  uint32_t *keys_in = t.keys_in, *vals_in = t.vals_in;
-  uint32_t *keys_out = t.keys_out, *vals_out = t.vals_out;
+  const int extra = t.slots - t.blocks;
   // (what task_span_kernel reads)
   BinnedParams p;
   memset(&p, 0, sizeof(p));
@@ -954,22 +946,18 @@ hipError_t order_tasks(const SearchInput &in, Bins &bins, uint32_t *task_keys,
   p.wave_start = bins.half_start;
   p.keys_y = bins.keys_y;
   p.code_bits = 3 * axis_bits(in.num_segments);
-  hipLaunchKernelGGL(task_span_kernel, dim3((blocks + kBlock - 1) / kBlock),
-                     dim3(kBlock), 0, stream, p, blocks, extra, extra_used,
-                     desc, keys_in, vals_in);
-  hipError_t err = hipGetLastError();
-  if (err != hipSuccess)
-    return err;
-  err = rocprim::radix_sort_pairs(sort_temp, sort_bytes, keys_in, keys_out,
-                                  vals_in, vals_out, (unsigned int)slots, 0u,
-                                  32u, stream, false);
-  bins.task_desc = desc;
-  bins.task_order = vals_out;
-  bins.task_slots = slots;
+  hipLaunchKernelGGL(task_span_kernel, dim3(t.groups), dim3(kBlock), 0, stream,
+                     p, t.blocks, extra, t.extra_used, t.desc, t.cls, t.hist);
+  hipLaunchKernelGGL(task_order_kernel, dim3(t.groups), dim3(kBlock), 0,
+                     stream, t.blocks, extra, t.extra_used, t.cls, t.hist,
+                     t.order);
+  bins.task_desc = t.desc;
+  bins.task_order = t.order;
+  bins.task_slots = t.slots;
   // (the search kernels' grid: whole runs of 8 tasks on each of 8 XCDs)
-  bins.task_grid = (slots + 63) / 64 * 64;
+  bins.task_grid = (t.slots + 63) / 64 * 64;
   bins.code_bits = p.code_bits;
-  return err;
+  return hipGetLastError();
 }
 
 // Orders rows and queries along the curve, copies the rows, builds the boxes;
@@ -1050,8 +1038,6 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
     setup.task_extra = with_tasks ? t.slots - t.blocks : 0;
     setup.extra_used = with_tasks ? t.extra_used : nullptr;
     setup.task_desc = t.desc;
-    setup.task_keys = t.keys_in;
-    setup.task_vals = t.vals_in;
     const int resets = std::max(6 * nseg, setup.task_extra);
     hipLaunchKernelGGL(bins_setup_kernel,
                        dim3(4 + (resets + kPlanThreads - 1) / kPlanThreads),
@@ -1107,7 +1093,7 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
         return e;
     }
     if (with_tasks)
-      e = order_tasks(in, bins, task_keys, side_temp, lay.side_temp, side);
+      e = order_tasks(in, bins, task_keys, side);
     if (e == hipSuccess && lane != nullptr)
       e = hipEventRecord(lane->join, side);
     return e;

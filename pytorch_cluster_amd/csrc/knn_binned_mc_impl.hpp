@@ -275,53 +275,135 @@ __device__ __forceinline__ void bin_box_of_lane(const Box &held, int src,
 // tiles as a wave in a dense region - the tail of the launch.  Such a block is
 // split into four tasks of 8 queries: its own slot and three extra slots
 // behind the blocks' ones, handed out by an atomic counter while they last
-// (`extra` slots; `*extra_used` starts at 0).  The sort key of a slot is the
-// complement of its span, so that the longest tasks start first and unused
-// extra slots come last (their waves leave at once).
-// Octave of the span first (longest first), position along the curve second:
-// tasks of about the same length keep their neighbours next to them, and
-// neighbours look at the same tiles.
-__device__ __forceinline__ uint32_t bin_task_key(uint32_t span, int block) {
-  const uint32_t octave = span != 0 ? (uint32_t)__builtin_clz(span) : 32u;
-  return (octave << 25) | min((uint32_t)block, (1u << 25) - 1u);
+// (`extra` slots; `*extra_used` starts at 0).
+//
+// Starting order: the used extra slots first (parts of the longest tasks),
+// then the blocks by the octave of their span, widest first, and inside an
+// octave in curve order: tasks of about the same length keep their neighbours
+// next to them, and neighbours look at the same tiles.  Unused slots come
+// last (their waves leave at once).  It is a counting sort in two launches:
+// task_span_kernel leaves every block's class and a histogram of the classes
+// per workgroup of kBlock blocks, task_order_kernel turns them into places.
+constexpr int kTaskClasses = 64; // octaves 0..32, 33 = unused block, rest empty
+
+__device__ __forceinline__ uint32_t bin_task_class(uint32_t span) {
+  return span != 0 ? (uint32_t)__builtin_clz(span) : 32u;
 }
 
+// cls: [bound] class per block; hist: [workgroups][kTaskClasses].
 __global__ __launch_bounds__(kBlock) void task_span_kernel(
     BinnedParams p, int bound, int extra, int *__restrict__ extra_used,
-    int2 *__restrict__ desc, uint32_t *__restrict__ keys,
-    uint32_t *__restrict__ vals) {
+    int2 *__restrict__ desc, uint32_t *__restrict__ cls,
+    int *__restrict__ hist) {
+  __shared__ int count_of[kTaskClasses];
+  if (threadIdx.x < kTaskClasses)
+    count_of[threadIdx.x] = 0;
+  __syncthreads();
   const int block = blockIdx.x * kBlock + threadIdx.x;
-  if (block >= bound)
-    return;
-  int2 mine = make_int2(0, 0);
-  uint32_t key = 0xffffffffu;
-  if (block < p.wave_start[p.num_segments]) {
-    const int seg = find_segment(p.wave_start, p.num_segments, block);
-    const int y_begin = p.ptr_y ? (int)p.ptr_y[seg] : 0;
-    const int y_end = p.ptr_y ? (int)p.ptr_y[seg + 1] : p.m;
-    const int jq0 = y_begin + (block - p.wave_start[seg]) * 32;
-    const int count = min(32, y_end - jq0);
-    const uint32_t span = p.keys_y[jq0 + count - 1] - p.keys_y[jq0];
-    const int blocks = p.wave_start[seg + 1] - p.wave_start[seg];
-    const uint64_t average = ((uint64_t)1 << p.code_bits) / (uint64_t)blocks;
-    mine = make_int2(jq0, count);
-    key = bin_task_key(span, block);
-    if (count == 32 && (uint64_t)span > 8 * average) {
-      const int at = atomicAdd(extra_used, 3);
-      if (at + 3 <= extra) {
-        mine = make_int2(jq0, 8);
-        key = bin_task_key(span / 4, block);
-        for (int i = 0; i < 3; ++i) {
-          desc[bound + at + i] = make_int2(jq0 + 8 * (i + 1), 8);
-          keys[bound + at + i] = key;
-          vals[bound + at + i] = (uint32_t)(bound + at + i);
+  if (block < bound) {
+    int2 mine = make_int2(0, 0);
+    uint32_t mine_class = 33u;
+    if (block < p.wave_start[p.num_segments]) {
+      const int seg = find_segment(p.wave_start, p.num_segments, block);
+      const int y_begin = p.ptr_y ? (int)p.ptr_y[seg] : 0;
+      const int y_end = p.ptr_y ? (int)p.ptr_y[seg + 1] : p.m;
+      const int jq0 = y_begin + (block - p.wave_start[seg]) * 32;
+      const int count = min(32, y_end - jq0);
+      const uint32_t span = p.keys_y[jq0 + count - 1] - p.keys_y[jq0];
+      const int blocks = p.wave_start[seg + 1] - p.wave_start[seg];
+      const uint64_t average = ((uint64_t)1 << p.code_bits) / (uint64_t)blocks;
+      mine = make_int2(jq0, count);
+      mine_class = bin_task_class(span);
+      if (count == 32 && (uint64_t)span > 8 * average) {
+        const int at = atomicAdd(extra_used, 3);
+        if (at + 3 <= extra) {
+          mine = make_int2(jq0, 8);
+          mine_class = bin_task_class(span / 4);
+          for (int i = 0; i < 3; ++i)
+            desc[bound + at + i] = make_int2(jq0 + 8 * (i + 1), 8);
         }
       }
     }
+    desc[block] = mine;
+    cls[block] = mine_class;
+    atomicAdd(&count_of[mine_class], 1);
   }
-  desc[block] = mine;
-  keys[block] = key;
-  vals[block] = (uint32_t)block;
+  __syncthreads();
+  if (threadIdx.x < kTaskClasses)
+    hist[blockIdx.x * kTaskClasses + threadIdx.x] = count_of[threadIdx.x];
+}
+
+// Same grid as task_span_kernel.  order: [bound + extra] slot numbers.
+__global__ __launch_bounds__(kBlock) void task_order_kernel(
+    int bound, int extra, const int *__restrict__ extra_used,
+    const uint32_t *__restrict__ cls, const int *__restrict__ hist,
+    uint32_t *__restrict__ order) {
+  constexpr int kParts = kBlock / kTaskClasses;
+  constexpr int kWaves = kBlock / kWave;
+  __shared__ int before_part[kParts][kTaskClasses];
+  __shared__ int total_part[kParts][kTaskClasses];
+  __shared__ int base[kTaskClasses];
+  __shared__ int wave_count[kWaves][kTaskClasses];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int used = min(*extra_used, extra);
+
+  // the extra slots: used ones first, the others behind everything
+  for (int i = blockIdx.x * kBlock + tid; i < extra; i += gridDim.x * kBlock)
+    order[i < used ? i : bound + i] = (uint32_t)(bound + i);
+
+  // blocks of every class in the workgroups before this one, and in all
+  {
+    const int c = tid & (kTaskClasses - 1);
+    const int part = tid / kTaskClasses;
+    int before = 0, total = 0;
+    for (int g = part; g < (int)gridDim.x; g += kParts) {
+      const int v = hist[g * kTaskClasses + c];
+      total += v;
+      before += g < (int)blockIdx.x ? v : 0;
+    }
+    before_part[part][c] = before;
+    total_part[part][c] = total;
+    wave_count[tid / kTaskClasses][c] = 0; // (kParts == kWaves)
+  }
+  static_assert(kParts == kWaves, "one zeroing pass covers wave_count");
+  __syncthreads();
+  if (tid == 0) {
+    int run = used;
+    for (int c = 0; c < kTaskClasses; ++c) {
+      int before = 0, total = 0;
+      for (int part = 0; part < kParts; ++part) {
+        before += before_part[part][c];
+        total += total_part[part][c];
+      }
+      base[c] = run + before;
+      run += total;
+    }
+  }
+  // place inside the wave among the blocks of the same class
+  const int block = blockIdx.x * kBlock + tid;
+  const bool valid = block < bound;
+  const int mine = valid ? (int)cls[block] : -1;
+  int rank = 0;
+  uint64_t todo = __ballot(valid);
+  while (todo != 0) {
+    const int leader = __builtin_ctzll(todo);
+    const int c = __shfl(mine, leader);
+    const uint64_t same = __ballot(mine == c);
+    if (mine == c)
+      rank = __builtin_popcountll(same & (((uint64_t)1 << lane) - 1));
+    if (lane == leader)
+      wave_count[wave][c] = __builtin_popcountll(same);
+    todo &= ~same;
+  }
+  __syncthreads();
+  if (valid) {
+    int at = base[mine] + rank;
+    for (int w = 0; w < wave; ++w)
+      at += wave_count[w][mine];
+    order[at] = (uint32_t)block;
+  }
 }
 
 // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: runs
