@@ -250,7 +250,9 @@ __global__ __launch_bounds__(kBlock) void gather_tiles_kernel(
   for (int c = 0; c < 3; ++c)
     v[c] = (ok && c < d) ? x[(size_t)id * d + c] : 0.0f;
   if (ok) {
-    rows[j] = make_float4(v[0], v[1], v[2], __uint_as_float(id));
+    // (the plain copy is read by the vector-ALU scans only)
+    if (rows != nullptr)
+      rows[j] = make_float4(v[0], v[1], v[2], __uint_as_float(id));
     // the operand of the matrix-core filter, then coordinates and row number
     uint4 rec[McShape<3>::REC];
     mc_pack_row<3>(v, rec);
@@ -963,7 +965,7 @@ hipError_t order_tasks(const SearchInput &in, Bins &bins, uint32_t *task_keys,
 // Orders rows and queries along the curve, copies the rows, builds the boxes;
 // with `with_tasks` also the tasks of 32 queries and their starting order.
 hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
-                        Bins &bins, hipStream_t stream) {
+                        bool plain_rows, Bins &bins, hipStream_t stream) {
   const BinnedLayout lay = binned_layout(in.n, in.m, in.num_segments);
   char *cursor = static_cast<char *>(scratch);
   auto take = [&cursor](size_t bytes) {
@@ -1046,8 +1048,8 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
   {
     // enough workgroups per segment to fill the device when segments are few
     const int parts = std::max(
-        1, std::min((in.n / nseg + 16 * kBlock - 1) / (16 * kBlock),
-                    std::max(1, 1024 / nseg)));
+        1, std::min((in.n / nseg + 4 * kBlock - 1) / (4 * kBlock),
+                    std::max(1, 4096 / nseg)));
     hipLaunchKernelGGL(seg_box_kernel, dim3(parts, std::min(nseg, 65535)),
                        dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
                        seg_box);
@@ -1122,7 +1124,8 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
     hipLaunchKernelGGL(gather_tiles_kernel,
                        dim3((lay.tiles_bound + per_block - 1) / per_block),
                        dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
-                       tile_start, perm_x, rows, packed, box);
+                       tile_start, perm_x, plain_rows ? rows : nullptr, packed,
+                       box);
     const int groups_per_block = kBlock / kWave;
     hipLaunchKernelGGL(
         group_boxes_kernel,
@@ -1186,7 +1189,8 @@ hipError_t launch_knn_binned(const SearchInput &in, int k, void *scratch,
   const char *env = getenv("PCA_KNN_BINNED_MATRIX_CORES");
   const bool matrix_cores = k > 32 || !(env != nullptr && env[0] == '0');
   Bins bins;
-  const hipError_t err = prepare_bins(in, scratch, matrix_cores, bins, stream);
+  const hipError_t err =
+      prepare_bins(in, scratch, matrix_cores, !matrix_cores, bins, stream);
   if (err != hipSuccess)
     return err;
   BinnedParams p;
@@ -1240,7 +1244,7 @@ hipError_t launch_nearest_binned(const SearchInput &in, void *scratch,
   if (time_start)
     (void)hipEventRecord(time_start, stream);
   Bins bins;
-  const hipError_t err = prepare_bins(in, scratch, true, bins, stream);
+  const hipError_t err = prepare_bins(in, scratch, true, false, bins, stream);
   if (err != hipSuccess)
     return err;
   BinnedParams p;
@@ -1263,17 +1267,18 @@ bool radius_binned_supported(int d, int slots) {
 hipError_t launch_radius_binned(const SearchInput &in, float r2,
                                 bool ignore_same_index, void *scratch,
                                 const DenseResult &out, hipStream_t stream) {
+  // (diagnostic switch: the vector-ALU scan instead of the matrix-core one)
+  const char *env = getenv("PCA_RADIUS_BINNED_MATRIX_CORES");
+  const bool matrix_cores = !(env != nullptr && env[0] == '0');
   Bins bins;
-  const hipError_t err = prepare_bins(in, scratch, false, bins, stream);
+  const hipError_t err =
+      prepare_bins(in, scratch, false, !matrix_cores, bins, stream);
   if (err != hipSuccess)
     return err;
   BinnedParams p;
   fill_params(p, in, bins, out);
   p.k = out.slots;
   const int same = ignore_same_index ? 1 : 0;
-  // (diagnostic switch: the vector-ALU scan instead of the matrix-core one)
-  const char *env = getenv("PCA_RADIUS_BINNED_MATRIX_CORES");
-  const bool matrix_cores = !(env != nullptr && env[0] == '0');
   const int per_task = matrix_cores ? kWave / 2 : kWave;
   if (matrix_cores)
     p.wave_start = bins.half_start;
