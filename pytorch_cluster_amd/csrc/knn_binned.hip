@@ -1047,9 +1047,11 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
   }
   {
     // enough workgroups per segment to fill the device when segments are few
+    // (more of them were no quicker: their atomic updates of the same few
+    // words take turns)
     const int parts = std::max(
-        1, std::min((in.n / nseg + 4 * kBlock - 1) / (4 * kBlock),
-                    std::max(1, 4096 / nseg)));
+        1, std::min((in.n / nseg + 16 * kBlock - 1) / (16 * kBlock),
+                    std::max(1, 1024 / nseg)));
     hipLaunchKernelGGL(seg_box_kernel, dim3(parts, std::min(nseg, 65535)),
                        dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
                        seg_box);
