@@ -1,5 +1,8 @@
 // Exact Euclidean kNN over spatially binned rows: fp32 points of up to three
-// dimensions, k <= 32.  Same results, bit for bit, as the reference's scan of
+// dimensions, k <= 64 (more than 32 with the matrix-core scan of
+// knn_binned_mc_impl.hpp only), and the radius and nearest searches over the
+// same bins (further down).  This comment describes the vector-ALU kNN scan,
+// the first of them, and the binning all share.  Same results, bit for bit, as the reference's scan of
 // every row of the segment (csrc/cuda/knn_cuda.cu:52-78: distances as chains
 // of direct differences and fused multiply-adds, neighbours by ascending
 // distance, ties by ascending row, strictly below 1e10), but a query looks only
