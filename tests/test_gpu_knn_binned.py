@@ -183,6 +183,29 @@ def test_queries_ordered_beside_the_rows(monkeypatch):
         assert torch.equal(capi.nearest_rows(x, y, px, py, binned=True), want)
 
 
+@pytest.mark.parametrize("m", [1, 32, 33, 8192, 8224, 131071, 131072,
+                               196608, 196640])
+def test_task_counts_at_the_edges(m):
+    """Blocks of 32 queries: one, one and a bit, a whole workgroup of the
+    ordering kernels (256 blocks) and one more, the first size ordered on a
+    second stream (131,072 queries), the last size whose long blocks are
+    split (6,144 blocks) and the first that is not.  Clustered queries (long
+    and short spans) in two segments, against the scanning kernels."""
+    g = torch.Generator().manual_seed(m)
+    x = torch.rand(40000, 3, generator=g)
+    y = torch.cat([torch.rand(m - m // 2, 3, generator=g) ** 3,
+                   torch.rand(m // 2, 3, generator=g)])
+    ptr_x = torch.tensor([0, 15000, 40000])
+    ptr_y = torch.tensor([0, m - m // 2, m])
+    x, y, ptr_x, ptr_y = (t.to(DEV) for t in (x, y, ptr_x, ptr_y))
+    a, da = capi.knn_edges(x, y, ptr_x, ptr_y, 7, want_dist=True)
+    b, db = capi.knn_edges(x, y, ptr_x, ptr_y, 7, want_dist=True, binned=True)
+    assert torch.equal(a, b)
+    assert torch.equal(da.view(torch.int32), db.view(torch.int32))
+    assert torch.equal(capi.nearest_rows(y, x, ptr_y, ptr_x),
+                       capi.nearest_rows(y, x, ptr_y, ptr_x, binned=True))
+
+
 def test_uniform_clouds_against_the_scanning_kernels():
     c = testing.uniform_batched(0)
     x = c["x"].to(DEV)
