@@ -269,7 +269,8 @@ __device__ __forceinline__ void bin_box_of_lane(const Box &held, int src,
 
 // Tasks of the matrix-core searches.  Normally a block of 32
 // curve-consecutive queries is one task (slot = block number).  A block whose
-// queries span much more of the curve than the segment's average lies where
+// queries span much more of the curve than the segment's average (4 times:
+// measured) lies where
 // the points are sparse: its queries are far apart, each with a neighbourhood
 // of its own, and one wave would look at several times as many boxes and
 // tiles as a wave in a dense region - the tail of the launch.  Such a block is
@@ -314,7 +315,7 @@ __global__ __launch_bounds__(kBlock) void task_span_kernel(
       const uint64_t average = ((uint64_t)1 << p.code_bits) / (uint64_t)blocks;
       mine = make_int2(jq0, count);
       mine_class = bin_task_class(span);
-      if (count == 32 && (uint64_t)span > 8 * average) {
+      if (count == 32 && (uint64_t)span > 4 * average) {
         const int at = atomicAdd(extra_used, 3);
         if (at + 3 <= extra) {
           mine = make_int2(jq0, 8);
