@@ -213,7 +213,7 @@ struct MfmaWalk {
 // the reference's order among equal distances: see device_utils.hpp); the
 // lists go through knn_merge_kernel like those of the kNN.
 template <int NB, int K, bool COSINE, bool NEAREST = false>
-__global__ __launch_bounds__(kBlock) void knn_mfma_kernel(KnnMfmaParams p) {
+__global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfmaParams p) {
   static_assert(!NEAREST || !COSINE, "nearest is Euclidean");
   constexpr float kLimit = SearchLimit<NEAREST>::value;
   typedef MfmaShape<NB> S;
