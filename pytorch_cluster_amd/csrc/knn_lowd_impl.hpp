@@ -160,8 +160,21 @@ __device__ __forceinline__ float filter_cut(float thresh, float ysq) {
   return f;
 }
 
+// Waves per SIMD asked of the compiler where it would otherwise stop just
+// above a register limit (512 / waves per lane): lists of 64 entries and, in
+// up to four dimensions, of 100 came out at 270-282 registers - one wave -
+// and run faster at two with a few dozen spilled words; lists of 32 entries
+// with one query per lane at 133 instead of the 128 that four waves take.
+template <int DIM, int K, int QPT>
+constexpr int knn_lowd_min_waves() {
+  return (K == 64 || (K == 100 && DIM <= 4)) ? 2
+         : (K == 32 && QPT == 1 && DIM <= 4) ? 4
+                                             : 1;
+}
+
 template <int DIM, int K, int QPT, bool COSINE>
-__global__ __launch_bounds__(kBlock) void knn_lowd_kernel(KnnLowdParams p) {
+__global__ __launch_bounds__(kBlock, (knn_lowd_min_waves<DIM, K, QPT>())) void
+knn_lowd_kernel(KnnLowdParams p) {
   constexpr int TX = kLowdTileX;
   constexpr int QCAP = kLowdQueueCap;
   constexpr int U = kLowdGroup;
