@@ -174,9 +174,12 @@ __global__ __launch_bounds__(kBlock) void mc_pack_rows_kernel(
 // the reference's order among equal distances (see device_utils.hpp) -- whose
 // result goes to p.out_nearest as a row number (0 when nothing qualified).
 // (launch bounds: 5-8 dimensions with lists of 16 came out at 136 registers,
-// three waves per SIMD; asked for four - 128 registers - it runs 5 % faster)
+// up to 3 dimensions with lists of 24 at 138-140: three waves per SIMD; asked
+// for four - 128 registers, up to 12 spilled words - they run 5 % and 10 %
+// faster on clouds that fill the device, 2 % slower on 16 x 4,096 points)
 template <int DIM, int K, bool NEAREST = false>
-__global__ __launch_bounds__(kBlock, (DIM == 8 && K == 16) ? 4 : 1) void
+__global__ __launch_bounds__(
+    kBlock, ((DIM == 8 && K == 16) || (DIM <= 3 && K == 24)) ? 4 : 1) void
 knn_lowd_mc_kernel(KnnLowdParams p) {
   static_assert(!NEAREST || K == 1, "nearest keeps one neighbour");
   constexpr float kLimit = SearchLimit<NEAREST>::value;
