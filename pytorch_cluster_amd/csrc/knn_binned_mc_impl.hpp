@@ -427,7 +427,7 @@ constexpr int kBinMcBlock = kWave;
 // equal distances (device_utils.hpp) - whose result goes to p.out_nearest as
 // a row number (0 when nothing qualified).
 template <int K, bool NEAREST = false>
-__global__ __launch_bounds__(kBinMcBlock, K <= 16 ? 4 : (K <= 32 ? 3 : 2)) void
+__global__ __launch_bounds__(kBinMcBlock, K <= 8 ? 5 : (K <= 16 ? 4 : (K <= 32 ? 3 : 2))) void
 knn_binned_mc_kernel(BinnedParams p) {
   static_assert(!NEAREST || K == 1, "nearest keeps one neighbour");
   constexpr int DIM = 3;
@@ -753,7 +753,7 @@ knn_binned_mc_kernel(BinnedParams p) {
 // largest one of a full list go into the list (row numbers as doubles).
 // p.wave_start counts tasks of 32 queries.
 template <int K>
-__global__ __launch_bounds__(kBinMcBlock, K <= 16 ? 4 : (K <= 32 ? 3 : 2)) void
+__global__ __launch_bounds__(kBinMcBlock, K <= 8 ? 5 : (K <= 16 ? 4 : (K <= 32 ? 3 : 2))) void
 radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
   __shared__ __attribute__((aligned(16))) uint4 ring[kBinRing][kBinTile];
   __shared__ uint32_t queue[kBinRing][kBinMcBlock];
