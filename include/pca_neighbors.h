@@ -187,7 +187,7 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
                size_t workspace_bytes, void *stream);
 
 /*
- * pca_radius for fp32 points of up to 3 dimensions and at most 32 neighbours
+ * pca_radius for fp32 points of up to 3 dimensions and at most 64 neighbours
  * per query (pca_radius_slots; PCA_ERR_UNSUPPORTED otherwise) over the
  * spatially binned rows of pca_knn_binned: a query scans only the tiles whose
  * box is closer than r, and of the rows found keeps the max_num_neighbors

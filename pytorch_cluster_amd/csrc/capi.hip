@@ -633,7 +633,7 @@ int pca_radius_binned(const void *x, const void *y, const int64_t *ptr_x,
   if (!pca::radius_binned_supported((int)d, (int)slots))
     return fail(PCA_ERR_UNSUPPORTED,
                 "binned search: fp32 points of up to 3 dimensions and at most "
-                "32 neighbours per query, got d=%lld slots=%lld",
+                "64 neighbours per query, got d=%lld slots=%lld",
                 (long long)d, (long long)slots);
   if (x == nullptr || y == nullptr || edges == nullptr)
     return fail(PCA_ERR_INVALID_ARGUMENT, "x, y or edges is NULL");

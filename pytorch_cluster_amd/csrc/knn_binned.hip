@@ -1266,15 +1266,17 @@ hipError_t launch_nearest_binned(const SearchInput &in, void *scratch,
 }
 
 bool radius_binned_supported(int d, int slots) {
-  return d >= 1 && d <= 3 && slots >= 1 && slots <= 32;
+  return d >= 1 && d <= 3 && slots >= 1 && slots <= 64;
 }
 
 hipError_t launch_radius_binned(const SearchInput &in, float r2,
                                 bool ignore_same_index, void *scratch,
                                 const DenseResult &out, hipStream_t stream) {
   // (diagnostic switch: the vector-ALU scan instead of the matrix-core one)
+  // (lists of more than 32 entries exist for the matrix-core scan only)
   const char *env = getenv("PCA_RADIUS_BINNED_MATRIX_CORES");
-  const bool matrix_cores = !(env != nullptr && env[0] == '0');
+  const bool matrix_cores =
+      out.slots > 32 || !(env != nullptr && env[0] == '0');
   Bins bins;
   const hipError_t err =
       prepare_bins(in, scratch, false, !matrix_cores, bins, stream);
@@ -1299,14 +1301,27 @@ hipError_t launch_radius_binned(const SearchInput &in, float r2,
       hipLaunchKernelGGL((radius_binned_kernel<K_>), dim3(grid), dim3(kBlock), \
                          0, stream, p, r2, same);                              \
   } while (0)
+#define PCA_BINNED_LAUNCH_WIDE(K_)                                             \
+  hipLaunchKernelGGL((radius_binned_mc_kernel<K_>),                            \
+                     dim3((waves + 63) / 64 * 64), dim3(kBinMcBlock), 0,       \
+                     stream, p, r2, same)
   if (out.slots <= 8)
     PCA_BINNED_LAUNCH(8);
   else if (out.slots <= 16)
     PCA_BINNED_LAUNCH(16);
   else if (out.slots <= 24)
     PCA_BINNED_LAUNCH(24);
-  else
+  else if (out.slots <= 32)
     PCA_BINNED_LAUNCH(32);
+  else if (out.slots <= 40)
+    PCA_BINNED_LAUNCH_WIDE(40);
+  else if (out.slots <= 48)
+    PCA_BINNED_LAUNCH_WIDE(48);
+  else if (out.slots <= 56)
+    PCA_BINNED_LAUNCH_WIDE(56);
+  else
+    PCA_BINNED_LAUNCH_WIDE(64);
+#undef PCA_BINNED_LAUNCH_WIDE
 #undef PCA_BINNED_LAUNCH
   return hipGetLastError();
 }

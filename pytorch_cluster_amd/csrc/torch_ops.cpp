@@ -283,7 +283,7 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
   const int dtype = dtype_code(x);
   const int64_t slots = pca_radius_slots(n, max_num_neighbors);
   const bool binned = bins_wanted(n, m, seg.count, 1e10, 2e-3) &&
-                      dtype == PCA_F32 && d <= 3 && slots <= 32;
+                      dtype == PCA_F32 && d <= 3 && slots <= 64;
   const size_t ws_bytes =
       binned ? pca_radius_binned_workspace_bytes(n, m, d, seg.count,
                                                  max_num_neighbors)

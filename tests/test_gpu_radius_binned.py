@@ -147,10 +147,32 @@ def test_strategy_switch_of_the_entry_points():
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("cap", [33, 40, 41, 50, 57, 64])
+def test_more_than_32_neighbours(oracle, cap, scan_kind):
+    """Lists of 40 to 64 entries (matrix-core scan only): dense
+    neighbourhoods, so that the cap cuts most lists, and some below it."""
+    if scan_kind == "0":
+        pytest.skip("wide lists exist for the matrix-core scan only")
+    rng = np.random.default_rng(cap)
+    x = rng.random((6000, 3)).astype(np.float32)
+    x[:800] = np.round(x[:800] * 8) / 8       # exact ties and duplicates
+    y = rng.random((500, 3)).astype(np.float32)
+    ptr_x = np.array([0, 2500, 6000], dtype=np.int64)
+    ptr_y = np.array([0, 200, 500], dtype=np.int64)
+    for r in (0.12, 0.3):
+        got = gpu_radius_binned(x, y, ptr_x, ptr_y, r, cap)
+        want = oracle.radius_op(x, y, ptr_x, ptr_y, r, cap)
+        assert np.array_equal(got, want)
+    a = capi.radius_edges(dev(x), dev(x), None, None, 0.2, cap, True)
+    b = capi.radius_edges(dev(x), dev(x), None, None, 0.2, cap, True,
+                          binned=True)
+    assert torch.equal(a, b)
+
+
 def test_unsupported_shapes_are_refused():
     x = torch.rand(100, 4, device=DEV)
     with pytest.raises(RuntimeError, match="binned search"):
         capi.radius_edges(x, x, None, None, 0.1, 8, binned=True)
     x = torch.rand(100, 3, device=DEV)
     with pytest.raises(RuntimeError, match="binned search"):
-        capi.radius_edges(x, x, None, None, 0.1, 33, binned=True)
+        capi.radius_edges(x, x, None, None, 0.1, 65, binned=True)
