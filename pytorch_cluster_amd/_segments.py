@@ -63,3 +63,16 @@ def graph_pointers(x: torch.Tensor, batch: Optional[torch.Tensor],
         return None
     assert batch is not None
     return torch.bucketize(torch.arange(b + 1, device=x.device), batch)
+
+
+def batch_pointers(rows: torch.Tensor, batch: torch.Tensor,
+                   batch_size: Optional[int]) -> torch.Tensor:
+    """CSR pointers ``[B + 1]`` of one sorted batch vector (always an array,
+    also for a single example).  Without ``batch_size`` the number of examples
+    is read from the vector's LAST entry (sorted: its largest), which is one
+    8-byte read instead of a reduction over the vector."""
+    assert rows.size(0) == batch.numel()
+    b = batch_size
+    if b is None:
+        b = int(batch[-1]) + 1 if batch.numel() > 0 else 1
+    return torch.bucketize(torch.arange(b + 1, device=rows.device), batch)
