@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define PCA_ABI_VERSION 2
+#define PCA_ABI_VERSION 3
 
 enum pca_status {
   PCA_OK = 0,
@@ -130,6 +130,30 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
             int64_t num_segments, int64_t k, int cosine, int dtype,
             int edge_flags, int64_t *edges, int64_t *num_edges, void *dist,
             void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * pca_knn without a workspace argument, for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid it).  No counterpart in the reference, whose operator allocates
+ * its temporaries through PyTorch.  Same arguments, results and errors as
+ * pca_knn; the scratch the kernels need lives in a buffer of
+ * PCA_FIXED_SCRATCH_BYTES that is part of the library's device code (one copy
+ * per GPU, held until the process ends), so the call itself allocates and
+ * frees nothing.  A search whose pca_knn_workspace_bytes() exceeds
+ * PCA_FIXED_SCRATCH_BYTES is refused with PCA_ERR_WORKSPACE before anything is
+ * launched.  All calls on one GPU share that buffer: calls that may overlap
+ * on the GPU (different streams, different host threads) race and must be
+ * ordered by the caller.  The buffer's address is looked up at the first call
+ * on a device; make that call outside of any stream capture.
+ */
+#define PCA_FIXED_SCRATCH_BYTES (32u << 20)
+
+int pca_knn_fixed_scratch(const void *x, const void *y, const int64_t *ptr_x,
+                          const int64_t *ptr_y, int64_t n, int64_t m,
+                          int64_t d, int64_t num_segments, int64_t k,
+                          int cosine, int dtype, int edge_flags,
+                          int64_t *edges, int64_t *num_edges, void *dist,
+                          void *stream);
 
 /*
  * pca_knn for fp32 points of up to 3 dimensions, Euclidean distance and

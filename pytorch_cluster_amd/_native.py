@@ -23,6 +23,7 @@ _BUILD_HINT = ("build it with `python pytorch_cluster_amd/build.py` "
 
 PCA_F32, PCA_F64, PCA_F16, PCA_BF16 = 0, 1, 2, 3
 PCA_EDGES_DROP_SELF, PCA_EDGES_X_FIRST = 1, 2
+PCA_FIXED_SCRATCH_BYTES = 32 << 20
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -39,6 +40,10 @@ C_ABI = {
                 [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                  ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp,
                  ctypes.c_size_t, _vp]),
+    "pca_knn_fixed_scratch": (ctypes.c_int,
+                              [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
+                               _i64, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                               _vp, _vp, _vp, _vp]),
     "pca_knn_binned_workspace_bytes": (ctypes.c_size_t,
                                        [_i64, _i64, _i64, _i64, _i64]),
     "pca_knn_binned": (ctypes.c_int,

@@ -55,16 +55,31 @@ def _edge_flags(drop_self: bool, x_first: bool) -> int:
 
 def knn_launch(x, y, ptr_x, ptr_y, k: int, cosine: bool = False,
                want_dist: bool = False, stream=None, drop_self: bool = False,
-               x_first: bool = False, binned: bool = False):
-    """Queues ``pca_knn`` (``binned``: ``pca_knn_binned``); returns (edges
-    buffer [2*m*k], num_edges [1] on the device, dist buffer or None,
-    workspace).  Nothing is synchronised."""
+               x_first: bool = False, binned: bool = False,
+               fixed_scratch: bool = False):
+    """Queues ``pca_knn`` (``binned``: ``pca_knn_binned``; ``fixed_scratch``:
+    ``pca_knn_fixed_scratch``, no workspace); returns (edges buffer [2*m*k],
+    num_edges [1] on the device, dist buffer or None, workspace or None).
+    Nothing is synchronised."""
     assert x.is_cuda and y.is_cuda and x.is_contiguous() and y.is_contiguous()
     assert x.dtype == y.dtype and x.dtype in _DTYPE_CODE
     dtype = _DTYPE_CODE[x.dtype]
     n, d = x.shape
     m = y.shape[0]
     ptr_x, ptr_y, nseg = _segments(ptr_x, ptr_y)
+    edges = torch.empty(max(2 * m * max(k, 0), 1), dtype=torch.long,
+                        device=x.device)
+    num_edges = torch.empty(1, dtype=torch.long, device=x.device)
+    dist = (torch.empty(max(m * max(k, 0), 1), dtype=torch.float32,
+                        device=x.device) if want_dist else None)
+    if fixed_scratch:
+        assert not binned
+        _check(capi.pca_knn_fixed_scratch(
+            _dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x), _dev_ptr(ptr_y), n, m,
+            d, nseg, k, int(cosine), dtype, _edge_flags(drop_self, x_first),
+            _dev_ptr(edges), _dev_ptr(num_edges), _dev_ptr(dist),
+            _stream_handle(stream, x.device)))
+        return edges, num_edges, dist, None
     if binned:
         assert dtype == 0 and not cosine
         ws_bytes = capi.pca_knn_binned_workspace_bytes(n, m, d, nseg, k)
@@ -74,11 +89,6 @@ def knn_launch(x, y, ptr_x, ptr_y, k: int, cosine: bool = False,
         # let the entry point produce the precise error
         ws_bytes = 256
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
-    edges = torch.empty(max(2 * m * max(k, 0), 1), dtype=torch.long,
-                        device=x.device)
-    num_edges = torch.empty(1, dtype=torch.long, device=x.device)
-    dist = (torch.empty(max(m * max(k, 0), 1), dtype=torch.float32,
-                        device=x.device) if want_dist else None)
     if binned:
         _check(capi.pca_knn_binned(_dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x),
                                    _dev_ptr(ptr_y), n, m, d, nseg, k,
@@ -98,12 +108,13 @@ def knn_launch(x, y, ptr_x, ptr_y, k: int, cosine: bool = False,
 
 def knn_edges(x, y, ptr_x=None, ptr_y=None, k: int = 1, cosine: bool = False,
               want_dist: bool = False, stream=None, drop_self: bool = False,
-              x_first: bool = False, binned: bool = False
+              x_first: bool = False, binned: bool = False,
+              fixed_scratch: bool = False
               ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """``[2, E]`` edges (and the ``[E]`` distances when asked for)."""
     edges, num_edges, dist, _ws = knn_launch(x, y, ptr_x, ptr_y, k, cosine,
                                              want_dist, stream, drop_self,
-                                             x_first, binned)
+                                             x_first, binned, fixed_scratch)
     e = int(num_edges.item())
     out = edges[:2 * e].view(2, e)
     return out, (dist[:e] if dist is not None else None)

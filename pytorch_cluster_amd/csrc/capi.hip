@@ -13,6 +13,7 @@
 #include <algorithm>
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 
 namespace {
 
@@ -197,6 +198,49 @@ int check_launch(hipError_t err, const char *what) {
   return PCA_OK;
 }
 
+int knn_call(const void *x, const void *y, const int64_t *ptr_x,
+             const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+             int64_t num_segments, int64_t k, int cosine, int dtype,
+             int edge_flags, int64_t *edges, int64_t *num_edges, void *dist,
+             void *workspace, size_t workspace_bytes, void *stream_);
+
+} // namespace
+
+// Scratch of pca_knn_fixed_scratch: device memory of the library itself, one
+// copy per GPU the library runs on, held until the process ends.  In host code
+// the array's name is only a handle for hipGetSymbolAddress; kernels and copies
+// take the per-device address kept in g_fixed_scratch.
+static __device__ __align__(256) unsigned char scratch[PCA_FIXED_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_fixed_scratch_mutex;
+void *g_fixed_scratch[kMaxDevices] = {};
+
+// The address of `scratch` on the device that is current on this thread
+// (looked up once per device; nothing is allocated).
+int fixed_scratch_of_current_device(void **out) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess || device < 0 || device >= kMaxDevices)
+    return fail(PCA_ERR_NO_DEVICE, "hipGetDevice: %s (device %d)",
+                hipGetErrorString(err), device);
+  std::lock_guard<std::mutex> lock(g_fixed_scratch_mutex);
+  if (g_fixed_scratch[device] == nullptr) {
+    void *ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || ptr == nullptr)
+      return fail(PCA_ERR_NO_DEVICE, "hipGetSymbolAddress(scratch): %s",
+                  hipGetErrorString(err));
+    if (((uintptr_t)ptr & 255) != 0)
+      return fail(PCA_ERR_WORKSPACE, "the fixed scratch is not 256-aligned");
+    g_fixed_scratch[device] = ptr;
+  }
+  *out = g_fixed_scratch[device];
+  return PCA_OK;
+}
+
 } // namespace
 
 extern "C" {
@@ -250,6 +294,49 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
             int64_t num_segments, int64_t k, int cosine, int dtype,
             int edge_flags, int64_t *edges, int64_t *num_edges, void *dist,
             void *workspace, size_t workspace_bytes, void *stream_) {
+  return knn_call(x, y, ptr_x, ptr_y, n, m, d, num_segments, k, cosine, dtype,
+                  edge_flags, edges, num_edges, dist, workspace,
+                  workspace_bytes, stream_);
+}
+
+int pca_knn_fixed_scratch(const void *x, const void *y, const int64_t *ptr_x,
+                          const int64_t *ptr_y, int64_t n, int64_t m,
+                          int64_t d, int64_t num_segments, int64_t k,
+                          int cosine, int dtype, int edge_flags,
+                          int64_t *edges, int64_t *num_edges, void *dist,
+                          void *stream_) {
+  g_last_error[0] = 0;
+  // (same normalisation as knn_call, so that the size test sees what the
+  // search will use; invalid sizes are reported by knn_call itself)
+  const int64_t segs = ptr_x == nullptr ? 1 : num_segments;
+  if (sizes_ok(n, m, d, segs) && k >= 1 && k <= PCA_KNN_MAX_K &&
+      dtype_ok(dtype) && n > 0 && m > 0) {
+    const size_t need = knn_workspace(n, m, d, segs, k, dtype);
+    if (need > PCA_FIXED_SCRATCH_BYTES)
+      return fail(PCA_ERR_WORKSPACE,
+                  "pca_knn_fixed_scratch: this search needs %zu bytes of "
+                  "scratch, the library's fixed buffer holds %zu; use pca_knn "
+                  "with a workspace of the caller",
+                  need, (size_t)PCA_FIXED_SCRATCH_BYTES);
+  }
+  void *buffer = nullptr;
+  const int rc = fixed_scratch_of_current_device(&buffer);
+  if (rc != PCA_OK)
+    return rc;
+  return knn_call(x, y, ptr_x, ptr_y, n, m, d, num_segments, k, cosine, dtype,
+                  edge_flags, edges, num_edges, dist, buffer,
+                  PCA_FIXED_SCRATCH_BYTES, stream_);
+}
+
+} // extern "C"
+
+namespace {
+
+int knn_call(const void *x, const void *y, const int64_t *ptr_x,
+             const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+             int64_t num_segments, int64_t k, int cosine, int dtype,
+             int edge_flags, int64_t *edges, int64_t *num_edges, void *dist,
+             void *workspace, size_t workspace_bytes, void *stream_) {
   g_last_error[0] = 0;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   SearchTimer timer(stream);
@@ -376,6 +463,10 @@ int pca_knn(const void *x, const void *y, const int64_t *ptr_x,
                           (edge_flags & PCA_EDGES_X_FIRST) != 0),
       "compaction kernels");
 }
+
+} // namespace
+
+extern "C" {
 
 size_t pca_knn_binned_workspace_bytes(int64_t n, int64_t m, int64_t d,
                                       int64_t num_segments, int64_t k) {

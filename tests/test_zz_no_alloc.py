@@ -1,0 +1,74 @@
+"""pca_knn_fixed_scratch: the kNN entry point that takes no workspace and
+allocates nothing (its scratch is a fixed buffer inside the library's device
+code) returns what pca_knn returns -- bit for bit, edges and distances -- on
+calls in a row that share that buffer, the second one smaller than the first.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _both(x, y, ptr_x, ptr_y, k, cosine=False, drop_self=False):
+    from gpu_common import dev
+    from pytorch_cluster_amd import capi
+    args = (dev(x), dev(y), dev(ptr_x, torch.long), dev(ptr_y, torch.long), k,
+            cosine)
+    want_e, want_d = capi.knn_edges(*args, want_dist=True,
+                                    drop_self=drop_self)
+    got_e, got_d = capi.knn_edges(*args, want_dist=True, drop_self=drop_self,
+                                  fixed_scratch=True)
+    torch.cuda.synchronize()
+    return (want_e.cpu().numpy(), want_d.cpu().numpy(),
+            got_e.cpu().numpy(), got_d.cpu().numpy())
+
+
+def test_fixed_scratch_matches_pca_knn_on_consecutive_calls(oracle):
+    from gpu_common import oracle_knn_edges
+    rng = np.random.default_rng(5)
+    # 1. three clouds of 3-D points (sliced scan: shared bounds, partial
+    # lists and the merge all live in the scratch)
+    x1 = rng.random((6000, 3), dtype=np.float32)
+    ptr1 = np.array([0, 2500, 2500, 6000], dtype=np.int64)
+    # 2. right after it a smaller search of another shape (feature space)
+    x2 = rng.standard_normal((700, 24)).astype(np.float32)
+    y2 = rng.standard_normal((90, 24)).astype(np.float32)
+    # 3. and a tiny one
+    x3 = rng.random((40, 2), dtype=np.float32)
+    cases = [(x1, x1, ptr1, ptr1, 17, False, True),
+             (x2, y2, None, None, 9, False, False),
+             (x2, y2, None, None, 9, True, False),
+             (x3, x3[:7], None, None, 50, False, False)]
+    for x, y, px, py, k, cosine, drop_self in cases:
+        want_e, want_d, got_e, got_d = _both(x, y, px, py, k, cosine,
+                                             drop_self)
+        assert got_e.shape == want_e.shape
+        assert (got_e == want_e).all()
+        assert (got_d == want_d).all()  # bit-exact, fp32
+        if not drop_self:
+            oe, od = oracle_knn_edges(oracle, x, y, px, py, k, cosine)
+            assert (got_e == oe).all() and (got_d == od).all()
+
+
+def test_fixed_scratch_refuses_what_does_not_fit():
+    from pytorch_cluster_amd import capi
+    from pytorch_cluster_amd._native import PCA_FIXED_SCRATCH_BYTES
+    from pytorch_cluster_amd._native import capi as lib
+    n = m = 1 << 20
+    assert lib.pca_knn_workspace_bytes(n, m, 3, 1, 32, 0) \
+        > PCA_FIXED_SCRATCH_BYTES
+    x = torch.zeros(n, 3, device="cuda:0")
+    with pytest.raises(capi.PcaError) as err:
+        capi.knn_launch(x, x, None, None, 32, fixed_scratch=True)
+    assert err.value.status == -3  # PCA_ERR_WORKSPACE
+    assert "fixed buffer" in str(err.value)
+    # invalid arguments are reported as by pca_knn
+    with pytest.raises(capi.PcaError) as err:
+        capi.knn_launch(x[:10], x[:10], None, None, 101, fixed_scratch=True)
+    assert err.value.status == -2
+    # and the entry point still works afterwards
+    e, _ = capi.knn_edges(x[:10], x[:10], None, None, 3, fixed_scratch=True)
+    assert e.shape == (2, 30)
