@@ -88,150 +88,282 @@ def cpu_baseline(data, ptr_x, ptr_y):
                       "OpenMP" % (stride, len(sample))}
 
 
-def other_configs(torch, pca, testing, dev):
-    """End-to-end times of the other benchmark configurations (median of a few
-    calls, inputs resident in HBM); reported beside the headline number, they
-    are parity-test cases, not the benchmark."""
-    def median_ms(fn, reps):
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 matrix peak
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+# Pairs the reference's radius kernel has to look at on configs[2] (seed 0):
+# for every query the scan position of its 32nd hit, or the segment length
+# (csrc/cuda/radius_cuda.cu:26-41).  tests/test_bench_constants.py recomputes
+# it with the CPU checker.
+C3_REQUIRED_PAIRS = 255153263
+
+
+def _median_ms(torch, fn, reps):
+    fn()
+    torch.cuda.synchronize()
+    times = []
+    out = None
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        out = fn()
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+    return statistics.median(times), out
+
+
+def _search_ms(torch, capi, events, fn, reps=3):
+    """Average duration of the search kernel of `fn` (HIP events recorded by
+    the library immediately around that kernel, on its launch stream)."""
+    total = 0.0
+    for _ in range(reps):
+        start, stop = events.create(), events.create()
+        capi.pca_time_next_search(start, stop)
         fn()
         torch.cuda.synchronize()
-        times = []
-        for _ in range(reps):
-            t0 = time.perf_counter()
-            out = fn()
-            torch.cuda.synchronize()
-            times.append((time.perf_counter() - t0) * 1e3)
-        return statistics.median(times), out
+        total += events.elapsed_ms(start, stop)
+        events.destroy(start)
+        events.destroy(stop)
+    return total / reps
 
-    report = {}
-    # (the scanning kernels unless an entry names its strategy)
-    pca.set_search_strategy("scan")
-    c2 = testing.uniform_batched(0)
-    x, b = c2["x"].to(dev), c2["batch"].to(dev)
-    ms, out = median_ms(lambda: pca.knn_graph(x, 20, b, batch_size=16), 10)
-    report["configs[1] knn_graph 16x4096 k=20"] = {
-        "ms": ms, "queries_per_s": x.shape[0] / ms * 1e3,
-        "edges": int(out.shape[1])}
-    c3 = testing.gaussian_mixture_batched(0)
-    x, b = c3["x"].to(dev), c3["batch"].to(dev)
-    ms, out = median_ms(
-        lambda: pca.radius_graph(x, 0.05, b, max_num_neighbors=32,
-                                 batch_size=8), 10)
-    report["configs[2] radius_graph 8x16384 r=0.05 max 32"] = {
-        "ms": ms, "edges_per_s": out.shape[1] / ms * 1e3,
-        "edges": int(out.shape[1])}
-    c4 = testing.feature_space(0)
-    x, y = c4["x"].to(dev), c4["y"].to(dev)
-    for cosine in (False, True):
-        ms, out = median_ms(lambda: pca.knn(x, y, 32, cosine=cosine), 3)
-        report["configs[3] knn 200000x128 / 50000x128 k=32 cosine=%s"
-               % cosine] = {
-            "ms": ms, "queries_per_s": y.shape[0] / ms * 1e3,
-            "gemm_tflops": 2 * 128 * x.shape[0] * y.shape[0] / ms / 1e9}
+
+def _roofline(kernel, kernel_ms, flop, peak_tflops, bound, detail):
+    achieved = flop / kernel_ms / 1e9
+    return {"bound": bound, "bound_detail": detail, "kernel": kernel,
+            "kernel_ms": kernel_ms, "flop_per_launch": flop,
+            "achieved": achieved, "peak": peak_tflops, "unit": "TFLOP/s",
+            "frac": achieved / peak_tflops}
+
+
+class Cases:
+    """The benchmark configurations beside the headline one, by name; each
+    returns its report (whole-call time, rate, roofline of its search
+    kernel)."""
+
+    def __init__(self, torch, pca, testing, dev):
+        from pytorch_cluster_amd._native import capi
+        self.torch, self.pca, self.testing, self.dev = torch, pca, testing, dev
+        self.capi = capi
+        self.events = HipEvents(torch)
+
+    def names(self):
+        return ["c1", "c2", "c3", "c4", "c4cos", "d256", "nearest_points",
+                "nearest_codes", "fps", "strategies"]
+
+    def run(self, name, reps=None):
+        return getattr(self, "case_" + name)(reps)
+
+    # configs[0]: the plumbing case, on the GPU here (CPU tensors take the
+    # package's CPU path: see cpu_build_baseline)
+    def case_c1(self, reps):
+        t, pca = self.torch, self.pca
+        x = self.testing.uniform_cloud(0)["x"].to(self.dev)
+        pca.set_search_strategy("scan")
+        fn = lambda: pca.knn_graph(x, 16)  # noqa: E731
+        ms, out = _median_ms(t, fn, reps or 10)
+        kms = _search_ms(t, self.capi, self.events, fn)
+        pairs = x.shape[0] * x.shape[0]
+        return {"configs[0] knn_graph 1024 k=16": {
+            "ms": ms, "queries_per_s": x.shape[0] / ms * 1e3,
+            "edges": int(out.shape[1]),
+            "roofline": _roofline(
+                "knn_lowd_mc_kernel<3,24>", kms, 9 * pairs, PEAK_FP32_TFLOPS,
+                "mfma", "algorithmic 3*D flop per pair against the fp32 "
+                "peak; 8 workgroups: a launch-latency case")}}
+
+    def case_c2(self, reps):
+        t, pca = self.torch, self.pca
+        c2 = self.testing.uniform_batched(0)
+        x, b = c2["x"].to(self.dev), c2["batch"].to(self.dev)
+        pca.set_search_strategy("scan")
+        fn = lambda: pca.knn_graph(x, 20, b, batch_size=16)  # noqa: E731
+        ms, out = _median_ms(t, fn, reps or 10)
+        kms = _search_ms(t, self.capi, self.events, fn)
+        pairs = 16 * 4096 * 4096
+        return {"configs[1] knn_graph 16x4096 k=20": {
+            "ms": ms, "queries_per_s": x.shape[0] / ms * 1e3,
+            "edges": int(out.shape[1]),
+            "roofline": _roofline(
+                "knn_lowd_mc_kernel<3,24>", kms, 9 * pairs, PEAK_FP32_TFLOPS,
+                "mfma", "algorithmic 3*D flop per pair against the fp32 peak "
+                "(vector = matrix)")}}
+
+    def case_c3(self, reps):
+        t, pca = self.torch, self.pca
+        c3 = self.testing.gaussian_mixture_batched(0)
+        x, b = c3["x"].to(self.dev), c3["batch"].to(self.dev)
+        pca.set_search_strategy("scan")
+        fn = lambda: pca.radius_graph(  # noqa: E731
+            x, 0.05, b, max_num_neighbors=32, batch_size=8)
+        ms, out = _median_ms(t, fn, reps or 10)
+        kms = _search_ms(t, self.capi, self.events, fn)
+        full = 8 * 16384 * 16384
+        detail = ("algorithmic 3*D flop per pair against the fp32 peak; the "
+                  "kernel stops a query at its 32nd hit")
+        return {"configs[2] radius_graph 8x16384 r=0.05 max 32": {
+            "ms": ms, "edges_per_s": out.shape[1] / ms * 1e3,
+            "edges": int(out.shape[1]),
+            "roofline": _roofline(
+                "radius_mc_kernel<3>", kms, 9 * C3_REQUIRED_PAIRS,
+                PEAK_FP32_TFLOPS, "mfma", detail + "; pairs = those the "
+                "reference's scan has to look at (position of the 32nd hit)"),
+            "roofline_all_pairs": _roofline(
+                "radius_mc_kernel<3>", kms, 9 * full, PEAK_FP32_TFLOPS,
+                "mfma", detail + "; pairs = all pairs of a segment")}}
+
+    def _feature_case(self, label, n, m, d, k, cosine, reps):
+        t, pca = self.torch, self.pca
+        c = self.testing.feature_space(0, n, m, d)
+        x, y = c["x"].to(self.dev), c["y"].to(self.dev)
+        fn = lambda: pca.knn(x, y, k, cosine=cosine)  # noqa: E731
+        ms, out = _median_ms(t, fn, reps or 3)
+        kms = _search_ms(t, self.capi, self.events, fn)
+        flop = 2 * d * n * m
+        return {label: {
+            "ms": ms, "queries_per_s": m / ms * 1e3,
+            "edges": int(out.shape[1]),
+            "roofline": _roofline(
+                "knn_mfma_kernel", kms, flop, PEAK_BF16_TFLOPS, "mfma",
+                "algorithmic 2*D flop per pair against the dense bf16 "
+                "matrix peak (the filter is three split-bf16 products per "
+                "pair and component; every returned distance is exact "
+                "fp32)")}}
+
+    def case_c4(self, reps):
+        return self._feature_case(
+            "configs[3] knn 200000x128 / 50000x128 k=32 cosine=False",
+            200000, 50000, 128, 32, False, reps)
+
+    def case_c4cos(self, reps):
+        return self._feature_case(
+            "configs[3] knn 200000x128 / 50000x128 k=32 cosine=True",
+            200000, 50000, 128, 32, True, reps)
+
+    def case_d256(self, reps):
+        return self._feature_case(
+            "knn 50000x256 onto themselves k=32", 50000, 50000, 256, 32,
+            False, reps)
+
     # nearest: every point of the LiDAR-like scans looks for the nearest of
     # its scan's every-8th point (the operator that follows the neighbour
     # searches in the reference's list; 3 * D flop per pair as above)
-    from pytorch_cluster_amd._native import capi
-    lidar = testing.lidar_scans(0, query_stride=8)
-    x, y = lidar["x"].to(dev), lidar["y"].to(dev)
-    bx, by = lidar["batch_x"].to(dev), lidar["batch_y"].to(dev)
-    sizes_x = torch.bincount(lidar["batch_x"])
-    sizes_y = torch.bincount(lidar["batch_y"])
-    pairs = int((sizes_x * sizes_y).sum())
-    ms, out = median_ms(lambda: pca.nearest(x, y, bx, by), 10)
-    events = HipEvents(torch)
-    start, stop = events.create(), events.create()
-    capi.pca_time_next_search(start, stop)
-    pca.nearest(x, y, bx, by)
-    torch.cuda.synchronize()
-    kernel_ms = events.elapsed_ms(start, stop)
-    events.destroy(start)
-    events.destroy(stop)
-    report["nearest: %d scan points -> their scan's every 8th point (%d)"
-           % (x.shape[0], y.shape[0])] = {
-        "ms": ms, "rows_per_s": x.shape[0] / ms * 1e3,
-        "kernel_ms": kernel_ms,
-        "kernel_tflops": 9 * pairs / kernel_ms / 1e9}
+    def case_nearest_points(self, reps):
+        t, pca = self.torch, self.pca
+        lidar = self.testing.lidar_scans(0, query_stride=8)
+        x, y = lidar["x"].to(self.dev), lidar["y"].to(self.dev)
+        bx, by = lidar["batch_x"].to(self.dev), lidar["batch_y"].to(self.dev)
+        sizes_x = t.bincount(lidar["batch_x"])
+        sizes_y = t.bincount(lidar["batch_y"])
+        pairs = int((sizes_x * sizes_y).sum())
+        pca.set_search_strategy("scan")
+        fn = lambda: pca.nearest(x, y, bx, by)  # noqa: E731
+        ms, _ = _median_ms(t, fn, reps or 10)
+        kms = _search_ms(t, self.capi, self.events, fn)
+        return {"nearest: %d scan points -> their scan's every 8th point (%d)"
+                % (x.shape[0], y.shape[0]): {
+            "ms": ms, "rows_per_s": x.shape[0] / ms * 1e3,
+            "roofline": _roofline(
+                "knn_lowd_mc_kernel<3,1,nearest>", kms, 9 * pairs,
+                PEAK_FP32_TFLOPS, "mfma",
+                "algorithmic 3*D flop per pair against the fp32 peak")}}
+
     # nearest in feature space: a code-book assignment (1M rows of 64
     # components to 4,096 code vectors, one segment; 2 * D flop per pair)
-    g = torch.Generator().manual_seed(0)
-    codes = torch.randn(4096, 64, generator=g)
-    feats = (codes[torch.randint(0, 4096, (1 << 20,), generator=g)]
-             + 0.5 * torch.randn(1 << 20, 64, generator=g)).to(dev)
-    codes = codes.to(dev)
-    ms, out = median_ms(lambda: pca.nearest(feats, codes), 5)
-    start, stop = events.create(), events.create()
-    capi.pca_time_next_search(start, stop)
-    pca.nearest(feats, codes)
-    torch.cuda.synchronize()
-    kernel_ms = events.elapsed_ms(start, stop)
-    events.destroy(start)
-    events.destroy(stop)
-    report["nearest: 1048576 x 64 features -> 4096 code vectors"] = {
-        "ms": ms, "rows_per_s": feats.shape[0] / ms * 1e3,
-        "kernel_ms": kernel_ms,
-        "kernel_tflops": 2 * 64 * feats.shape[0] * 4096 / kernel_ms / 1e9}
+    def case_nearest_codes(self, reps):
+        t, pca = self.torch, self.pca
+        g = t.Generator().manual_seed(0)
+        codes = t.randn(4096, 64, generator=g)
+        feats = (codes[t.randint(0, 4096, (1 << 20,), generator=g)]
+                 + 0.5 * t.randn(1 << 20, 64, generator=g)).to(self.dev)
+        codes = codes.to(self.dev)
+        fn = lambda: pca.nearest(feats, codes)  # noqa: E731
+        ms, _ = _median_ms(t, fn, reps or 5)
+        kms = _search_ms(t, self.capi, self.events, fn)
+        return {"nearest: 1048576 x 64 features -> 4096 code vectors": {
+            "ms": ms, "rows_per_s": feats.shape[0] / ms * 1e3,
+            "roofline": _roofline(
+                "knn_mfma_kernel<5,8,nearest>", kms,
+                2 * 64 * feats.shape[0] * 4096, PEAK_BF16_TFLOPS, "mfma",
+                "algorithmic 2*D flop per pair against the dense bf16 "
+                "matrix peak (three split-bf16 products per pair and "
+                "component)")}}
+
     # fps: the sampling step that precedes radius / knn in a set-abstraction
     # layer; a quarter of every cloud, first row as start
-    for clouds, points in ((16, 4096), (8, 16384)):
-        pts = testing.uniform_batched(0, clouds, points)["x"].to(dev)
-        ptr = (torch.arange(clouds + 1) * points).to(dev)
-        ratio = torch.tensor(0.25, device=dev)
-        ms, out = median_ms(
-            lambda: torch.ops.torch_cluster.fps(pts, ptr, ratio, False), 5)
-        report["fps %dx%d ratio 0.25" % (clouds, points)] = {
-            "ms": ms, "samples": int(out.numel()),
-            "us_per_sample_step": ms * 1e3 / (points // 4)}
-    # the headline workload and one large cloud through the binned search
-    # (rows ordered along a space-filling curve, exact pruning by tile boxes):
-    # same edges as the scan; `search_ms` covers binning and search
-    lidar = testing.lidar_scans(0)
-    x, y = lidar["x"].to(dev), lidar["y"].to(dev)
-    bx, by = lidar["batch_x"].to(dev), lidar["batch_y"].to(dev)
-    big = torch.rand(1000000, 3, generator=torch.Generator().manual_seed(1))
-    big = big.to(dev)
-    c3 = testing.gaussian_mixture_batched(0)
-    x3, b3 = c3["x"].to(dev), c3["batch"].to(dev)
-    cases = (("configs[4] ragged LiDAR-like knn k=16",
-              lambda: pca.knn(x, y, 16, bx, by, batch_size=8), y.shape[0]),
-             ("knn 1000000 uniform points onto themselves k=16",
-              lambda: pca.knn(big, big, 16), big.shape[0]),
-             ("configs[2] radius_graph 8x16384 r=0.05 max 32",
-              lambda: pca.radius_graph(x3, 0.05, b3, max_num_neighbors=32,
-                                       batch_size=8), x3.shape[0]),
-             ("radius 1000000 uniform points onto themselves r=0.01 max 32",
-              lambda: pca.radius(big, big, 0.01, max_num_neighbors=32),
-              big.shape[0]))
-    for name, fn, queries in cases:
-        for strategy in ("scan", "binned"):
-            pca.set_search_strategy(strategy)
-            try:
-                ms, out = median_ms(fn, 5)
-                start, stop = events.create(), events.create()
-                capi.pca_time_next_search(start, stop)
-                fn()
-                torch.cuda.synchronize()
-                search_ms = events.elapsed_ms(start, stop)
-                events.destroy(start)
-                events.destroy(stop)
-            finally:
-                pca.set_search_strategy("scan")
-            report["%s, strategy %s" % (name, strategy)] = {
-                "ms": ms, "queries_per_s": queries / ms * 1e3,
-                "search_ms": search_ms, "edges": int(out.shape[1])}
-    # nearest on the LiDAR-like points again, through both strategies
-    lidar8 = testing.lidar_scans(0, query_stride=8)
-    nx, ny = lidar8["x"].to(dev), lidar8["y"].to(dev)
-    nbx, nby = lidar8["batch_x"].to(dev), lidar8["batch_y"].to(dev)
-    for strategy in ("scan", "binned"):
-        pca.set_search_strategy(strategy)
-        try:
-            ms, out = median_ms(lambda: pca.nearest(nx, ny, nbx, nby), 5)
-        finally:
-            pca.set_search_strategy("scan")
-        report["nearest on the LiDAR-like points, strategy %s" % strategy] = {
-            "ms": ms, "rows_per_s": nx.shape[0] / ms * 1e3}
-    pca.set_search_strategy("auto")
+    def case_fps(self, reps):
+        t = self.torch
+        report = {}
+        for clouds, points in ((16, 4096), (8, 16384)):
+            pts = self.testing.uniform_batched(0, clouds, points)["x"]
+            pts = pts.to(self.dev)
+            ptr = (t.arange(clouds + 1) * points).to(self.dev)
+            ratio = t.tensor(0.25, device=self.dev)
+            ms, out = _median_ms(
+                t, lambda: t.ops.torch_cluster.fps(pts, ptr, ratio, False),
+                reps or 5)
+            report["fps %dx%d ratio 0.25" % (clouds, points)] = {
+                "ms": ms, "samples": int(out.numel()),
+                "us_per_sample_step": ms * 1e3 / (points // 4)}
+        return report
+
+    # the headline workload and large clouds through both search strategies
+    # (binned: rows ordered along a space-filling curve, exact pruning by tile
+    # boxes; same edges as the scan); `search_ms` covers binning and search
+    def case_strategies(self, reps):
+        t, pca = self.torch, self.pca
+        report = {}
+        lidar = self.testing.lidar_scans(0)
+        x, y = lidar["x"].to(self.dev), lidar["y"].to(self.dev)
+        bx, by = lidar["batch_x"].to(self.dev), lidar["batch_y"].to(self.dev)
+        big = t.rand(1000000, 3, generator=t.Generator().manual_seed(1))
+        big = big.to(self.dev)
+        c3 = self.testing.gaussian_mixture_batched(0)
+        x3, b3 = c3["x"].to(self.dev), c3["batch"].to(self.dev)
+        lidar8 = self.testing.lidar_scans(0, query_stride=8)
+        nx, ny = lidar8["x"].to(self.dev), lidar8["y"].to(self.dev)
+        nbx = lidar8["batch_x"].to(self.dev)
+        nby = lidar8["batch_y"].to(self.dev)
+        cases = (("configs[4] ragged LiDAR-like knn k=16",
+                  lambda: pca.knn(x, y, 16, bx, by, batch_size=8),
+                  y.shape[0]),
+                 ("knn 1000000 uniform points onto themselves k=16",
+                  lambda: pca.knn(big, big, 16), big.shape[0]),
+                 ("configs[2] radius_graph 8x16384 r=0.05 max 32",
+                  lambda: pca.radius_graph(x3, 0.05, b3, max_num_neighbors=32,
+                                           batch_size=8), x3.shape[0]),
+                 ("radius 1000000 uniform points onto themselves r=0.01 "
+                  "max 32",
+                  lambda: pca.radius(big, big, 0.01, max_num_neighbors=32),
+                  big.shape[0]),
+                 ("nearest on the LiDAR-like points",
+                  lambda: pca.nearest(nx, ny, nbx, nby), nx.shape[0]))
+        for name, fn, queries in cases:
+            for strategy in ("scan", "binned"):
+                pca.set_search_strategy(strategy)
+                try:
+                    ms, out = _median_ms(t, fn, reps or 5)
+                    search_ms = _search_ms(t, self.capi, self.events, fn, 1)
+                finally:
+                    pca.set_search_strategy("scan")
+                report["%s, strategy %s" % (name, strategy)] = {
+                    "ms": ms, "queries_per_s": queries / ms * 1e3,
+                    "search_ms": search_ms,
+                    "edges": int(out.shape[1]) if out.dim() == 2 else None}
+        return report
+
+
+def other_configs(torch, pca, testing, dev, only=None):
+    """End-to-end times and search-kernel rooflines of the other benchmark
+    configurations (median of a few calls, inputs resident in HBM); reported
+    beside the headline number, they are parity-test cases, not the
+    benchmark."""
+    cases = Cases(torch, pca, testing, dev)
+    report = {}
+    before = pca.get_search_strategy()
+    try:
+        for name in (only or cases.names()):
+            report.update(cases.run(name))
+    finally:
+        pca.set_search_strategy(before)
     return report
 
 
@@ -261,6 +393,10 @@ def main():
                     help="run only the other benchmark configurations and "
                          "print their timings (for kernel traces of those "
                          "paths)")
+    ap.add_argument("--case", action="append", default=None,
+                    help="with --extras-only: run only this configuration "
+                         "(c1, c2, c3, c4, c4cos, d256, nearest_points, "
+                         "nearest_codes, fps, strategies; repeatable)")
     ap.add_argument("--strategy", choices=("scan", "binned", "auto"),
                     default="scan",
                     help="search strategy of the timed steps: scan (default "
@@ -287,7 +423,8 @@ def main():
     dev = torch.device("cuda:0")
     if args.extras_only:
         print(json.dumps({"other_configs":
-                          other_configs(torch, pca, testing, dev)}))
+                          other_configs(torch, pca, testing, dev,
+                                        args.case)}))
         return
     data = testing.lidar_scans(0)
     B = data["batch_size"]
