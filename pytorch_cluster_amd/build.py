@@ -32,7 +32,7 @@ HIP_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument",
-]
+] + os.environ.get("PCA_EXTRA_HIP_FLAGS", "").split()
 
 
 def _run(cmd):

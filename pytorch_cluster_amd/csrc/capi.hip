@@ -95,7 +95,10 @@ KnnLayout knn_layout(int64_t n, int64_t m, int64_t d, int64_t num_segments,
     w.x_norm = align256(pca::anytype_norm_bytes((int)n));
   } else if (d > 8) {
     w.x_norm = align256(sizeof(float) * (size_t)n);
-    if (pca::knn_mfma_supported((int)d, (int)k, false))
+    if (pca::knn_feat_supported((int)d, (int)k, false))
+      w.sliced = pca::knn_feat_scratch_bytes((int)n, (int)m, (int)d,
+                                             (int)num_segments, (int)k);
+    else if (pca::knn_mfma_supported((int)d, (int)k, false))
       w.sliced = pca::knn_mfma_scratch_bytes((int)n, (int)m, (int)d,
                                              (int)num_segments, (int)k);
   } else {
@@ -405,9 +408,11 @@ int knn_call(const void *x, const void *y, const int64_t *ptr_x,
 
   pca::SearchInput in{x,      y,      ptr_x,  ptr_y,
                       (int)n, (int)m, (int)d, (int)num_segments};
-  const bool mfma =
-      f32 && !low_d && pca::knn_mfma_supported((int)d, (int)k, cosine != 0);
-  if (mfma)
+  const bool feat =
+      f32 && !low_d && pca::knn_feat_supported((int)d, (int)k, cosine != 0);
+  const bool mfma = f32 && !low_d && !feat &&
+                    pca::knn_mfma_supported((int)d, (int)k, cosine != 0);
+  if (mfma || feat)
     cfg.tile_queries = pca::kMfmaTileQueries;
   else if (!low_d)
     cfg.tile_queries = pca::kBlock; // any-dimension kernel: one query per lane
@@ -425,6 +430,12 @@ int knn_call(const void *x, const void *y, const int64_t *ptr_x,
                                            work_start, lowd_scratch, dense,
                                            timer.start, timer.stop, stream),
                       "knn_lowd_kernel");
+    timer.stop = nullptr;
+  } else if (feat) {
+    rc = check_launch(pca::launch_knn_feat(in, (int)k, cosine != 0, work_start,
+                                           lowd_scratch, dense, timer.start,
+                                           timer.stop, stream),
+                      "knn_feat_kernel");
     timer.stop = nullptr;
   } else if (mfma) {
     rc = check_launch(pca::launch_knn_mfma(in, (int)k, cosine != 0, work_start,

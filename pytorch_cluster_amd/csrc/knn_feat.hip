@@ -1,0 +1,383 @@
+// Dispatch of the feature-space kNN with the fp16 matrix-core filter (see
+// knn_feat_impl.hpp): preparation, the filter kernel, the exact second kernel
+// and the second pass for the queries that one flags.
+#include "knn_feat_impl.hpp"
+
+#include <algorithm>
+#include <cstdlib>
+
+namespace pca {
+
+#define PCA_DECLARE_FEAT_BLOCKS(NB)                                            \
+  template <>                                                                  \
+  hipError_t launch_knn_feat_blocks<NB>(const KnnFeatParams &, int, bool,      \
+                                        int, hipStream_t);                     \
+  template <>                                                                  \
+  hipError_t launch_feat_pack<NB>(const float *, const float *,                \
+                                  const float *, int, int, bool,               \
+                                  FeatGlobals *, uint4 *, hipStream_t);
+PCA_DECLARE_FEAT_BLOCKS(3)
+PCA_DECLARE_FEAT_BLOCKS(5)
+PCA_DECLARE_FEAT_BLOCKS(9)
+PCA_DECLARE_FEAT_BLOCKS(17)
+#undef PCA_DECLARE_FEAT_BLOCKS
+
+namespace {
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// list width for k neighbours: k + 16 real entries
+int feat_width(int k) {
+  static const int widths[] = {24, 32, 48, 64};
+  for (int w : widths)
+    if (k + kFeatSlack <= w)
+      return w;
+  return 0;
+}
+
+// blocks of 16 components: the coordinates and the block that carries W
+int feat_blocks(int d) {
+  if (d <= 32)
+    return 3;
+  if (d <= 64)
+    return 5;
+  if (d <= 128)
+    return 9;
+  return 17;
+}
+
+int feat_tile_rows(int d) { return feat_blocks(d) <= 9 ? 64 : 32; }
+
+size_t feat_pack_bytes(int n, int d) {
+  const size_t units = 2 * (size_t)feat_blocks(d) + 1; // FeatShape::RSU
+  return align256(sizeof(uint4) * units * ((size_t)n + feat_tile_rows(d)));
+}
+
+__global__ __launch_bounds__(kBlock) void feat_init_kernel(FeatGlobals *g,
+                                                           float *tau, int m) {
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < m)
+    tau[i] = __builtin_inff();
+  if (i == 0) {
+    g->max_bits = 0;
+    g->odd_rows = 0;
+    g->any_redo = 0;
+    g->pad = 0;
+  }
+}
+
+// slices of every segment's x rows of the second pass of the exact kernel
+constexpr int kSecondPassChunks = 16;
+
+// Squared norms of rows (16 lanes per row, coalesced reads; any summation
+// order serves the filter; NaN for a row with a non-finite component) and the
+// largest finite |component| of the matrix.
+__global__ __launch_bounds__(kBlock) void feat_rows_kernel(
+    const float *__restrict__ x, int n, int d, float *__restrict__ sq_out,
+    FeatGlobals *g) {
+  __shared__ unsigned part[kBlock / kWave];
+  const int sub = threadIdx.x & 15;
+  const int row = blockIdx.x * (kBlock / 16) + (threadIdx.x >> 4);
+  float s = 0.0f;
+  unsigned big = 0;
+  if (row < n) {
+    const float *p = x + (size_t)row * d;
+    bool finite = true;
+    auto take = [&](float v) {
+      s = __builtin_fmaf(v, v, s);
+      const unsigned u = __float_as_uint(v) & 0x7fffffffu;
+      if (u >= 0x7f800000u)
+        finite = false;
+      else if (u > big)
+        big = u;
+    };
+    if ((d & 3) == 0) {
+      const float4 *p4 = reinterpret_cast<const float4 *>(p);
+      for (int c = sub; c < d / 4; c += 16) {
+        const float4 v = p4[c];
+        take(v.x), take(v.y), take(v.z), take(v.w);
+      }
+    } else {
+      for (int c = sub; c < d; c += 16)
+        take(p[c]);
+    }
+    // a row with an infinite or NaN component is nobody's neighbour
+    // (csrc/cuda/knn_cuda.cu:48,68: its distances are infinite or NaN); it is
+    // told apart from a finite row whose squared norm overflows
+    if (!finite)
+      s = __builtin_nanf("");
+  }
+#pragma unroll
+  for (int sh = 8; sh >= 1; sh >>= 1)
+    s += __shfl_xor(s, sh);
+  if (row < n && sub == 0 && sq_out != nullptr)
+    sq_out[row] = s;
+  // rows the filter leaves out do not set the scale
+  if (!(s < __builtin_inff()))
+    big = 0;
+#pragma unroll
+  for (int sh = 32; sh >= 1; sh >>= 1) {
+    const unsigned o = (unsigned)__shfl_xor((int)big, sh);
+    big = o > big ? o : big;
+  }
+  if ((threadIdx.x & (kWave - 1)) == 0)
+    part[threadIdx.x / kWave] = big;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kBlock / kWave; ++w)
+      big = part[w] > big ? part[w] : big;
+    if (big != 0)
+      atomicMax(&g->max_bits, big);
+  }
+}
+
+template <int KP>
+void launch_feat_merge(const KnnFeatParams &p, int tiles_bound,
+                       hipStream_t stream) {
+  hipLaunchKernelGGL((feat_merge_kernel<KP>), dim3(tiles_bound), dim3(kBlock),
+                     0, stream, p);
+}
+
+struct FeatLayout {
+  size_t globals, x_norm, x_class, y_norm, tau, redo, plan256;
+  size_t pack, partial, cand; // first pass
+  size_t second;              // second pass (reuses the first pass's bytes)
+  size_t shared() const {
+    return globals + x_norm + x_class + y_norm + tau + redo + plan256;
+  }
+  size_t total() const {
+    return shared() + std::max(pack + partial + cand, second);
+  }
+};
+
+} // namespace
+
+bool knn_feat_supported(int d, int k, bool cosine) {
+  if (const char *env = std::getenv("PCA_KNN_NO_MFMA"))
+    if (env[0] == '1')
+      return false;
+  if (const char *env = std::getenv("PCA_KNN_FEAT"))
+    if (env[0] == '0')
+      return false;
+  (void)cosine;
+  return d > 8 && d <= 256 && k >= 1 && feat_width(k) != 0;
+}
+
+int knn_feat_slices(int n, int m, int d, int num_segments) {
+  const int tiles = plan_upper_bound(m, num_segments, kFeatQueries);
+  const int want = (3072 + tiles - 1) / tiles;
+  const int by_length = (n / num_segments) / (8 * feat_tile_rows(d));
+  int chunks = std::max(1, std::min(std::min(want, 32), by_length));
+  if (const char *env = std::getenv("PCA_KNN_SLICES")) {
+    const int v = std::atoi(env);
+    if (v >= 1 && v <= 64)
+      chunks = v;
+  }
+  return chunks;
+}
+
+static FeatLayout feat_layout(int n, int m, int d, int num_segments, int k) {
+  FeatLayout w;
+  const size_t tiles = plan_upper_bound(m, num_segments, kFeatQueries);
+  const int chunks = knn_feat_slices(n, m, d, num_segments);
+  const size_t kk = (size_t)k + kFeatSlack;
+  w.globals = align256(sizeof(FeatGlobals));
+  w.x_norm = align256(sizeof(float) * (size_t)n);
+  w.x_class = align256(sizeof(float) * (size_t)n);
+  w.y_norm = align256(sizeof(float) * (size_t)m);
+  w.tau = align256(sizeof(float) * (size_t)m);
+  w.redo = align256(sizeof(int) * (size_t)m);
+  w.plan256 = align256(sizeof(int) * ((size_t)num_segments + 1));
+  w.pack = feat_pack_bytes(n, d);
+  w.partial = align256(sizeof(double) * tiles * chunks * kk * kFeatQueries);
+  w.cand = align256(sizeof(double) * (size_t)m * kk);
+  w.second = d <= 128 ? knn_mfma_scratch_bytes(n, m, d, num_segments, k,
+                                               kSecondPassChunks)
+                      : 0;
+  return w;
+}
+
+size_t knn_feat_scratch_bytes(int n, int m, int d, int num_segments, int k) {
+  return feat_layout(n, m, d, num_segments, k).total();
+}
+
+hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
+                           const int *work_start, void *scratch,
+                           const DenseResult &out, hipEvent_t time_start,
+                           hipEvent_t time_stop, hipStream_t stream) {
+  const FeatLayout lay =
+      feat_layout(in.n, in.m, in.d, in.num_segments, k);
+  const int tiles_bound =
+      plan_upper_bound(in.m, in.num_segments, kFeatQueries);
+  const int chunks = knn_feat_slices(in.n, in.m, in.d, in.num_segments);
+  char *base = static_cast<char *>(scratch);
+  auto take = [&base](size_t bytes) {
+    char *piece = base;
+    base += bytes;
+    return piece;
+  };
+  FeatGlobals *globals = reinterpret_cast<FeatGlobals *>(take(lay.globals));
+  float *x_norm = reinterpret_cast<float *>(take(lay.x_norm));
+  float *x_class_buf = reinterpret_cast<float *>(take(lay.x_class));
+  float *y_norm = reinterpret_cast<float *>(take(lay.y_norm));
+  float *tau = reinterpret_cast<float *>(take(lay.tau));
+  int *redo_q = reinterpret_cast<int *>(take(lay.redo));
+  int *plan256 = reinterpret_cast<int *>(take(lay.plan256));
+  char *first_pass = base;
+  uint4 *x_pack = reinterpret_cast<uint4 *>(take(lay.pack));
+  double *partial = reinterpret_cast<double *>(take(lay.partial));
+  double *cand = reinterpret_cast<double *>(take(lay.cand));
+
+  const float *xf = static_cast<const float *>(in.x);
+  const float *yf = static_cast<const float *>(in.y);
+  const int nb = feat_blocks(in.d);
+
+  hipLaunchKernelGGL(feat_init_kernel, dim3((in.m + kBlock - 1) / kBlock),
+                     dim3(kBlock), 0, stream, globals, tau, in.m);
+  // squared norms that only classify the rows (NaN: a non-finite component);
+  // for the Euclidean distance they also enter the filter
+  float *x_class = cosine ? x_class_buf : x_norm;
+  const int rows_per_block = kBlock / 16;
+  if (cosine) {
+    // |x|, |y| as the reference's Cosine::norm computes them: they enter the
+    // exact distances
+    (void)launch_row_norms(xf, in.n, in.d, x_norm, stream);
+    (void)launch_row_norms(yf, in.m, in.d, y_norm, stream);
+    hipLaunchKernelGGL(feat_rows_kernel,
+                       dim3((in.n + rows_per_block - 1) / rows_per_block),
+                       dim3(kBlock), 0, stream, xf, in.n, in.d, x_class,
+                       globals);
+  } else {
+    hipLaunchKernelGGL(feat_rows_kernel,
+                       dim3((in.n + rows_per_block - 1) / rows_per_block),
+                       dim3(kBlock), 0, stream, xf, in.n, in.d, x_norm,
+                       globals);
+    hipLaunchKernelGGL(feat_rows_kernel,
+                       dim3((in.m + rows_per_block - 1) / rows_per_block),
+                       dim3(kBlock), 0, stream, yf, in.m, in.d,
+                       static_cast<float *>(nullptr), globals);
+  }
+  {
+    hipError_t perr;
+    switch (nb) {
+    case 3:
+      perr = launch_feat_pack<3>(xf, x_norm, x_class, in.n, in.d, cosine,
+                                 globals, x_pack, stream);
+      break;
+    case 5:
+      perr = launch_feat_pack<5>(xf, x_norm, x_class, in.n, in.d, cosine,
+                                 globals, x_pack, stream);
+      break;
+    case 9:
+      perr = launch_feat_pack<9>(xf, x_norm, x_class, in.n, in.d, cosine,
+                                 globals, x_pack, stream);
+      break;
+    default:
+      perr = launch_feat_pack<17>(xf, x_norm, x_class, in.n, in.d, cosine,
+                                  globals, x_pack, stream);
+      break;
+    }
+    if (perr != hipSuccess)
+      return perr;
+  }
+
+  KnnFeatParams p;
+  p.x = xf;
+  p.y = yf;
+  p.ptr_x = in.ptr_x;
+  p.ptr_y = in.ptr_y;
+  p.x_norm = x_norm;
+  p.y_norm = y_norm;
+  p.x_pack = x_pack;
+  p.globals = globals;
+  p.n = in.n;
+  p.m = in.m;
+  p.d = in.d;
+  p.num_segments = in.num_segments;
+  p.k = k;
+  p.work_start = work_start;
+  p.num_chunks = chunks;
+  p.round_period = kFeatRoundPeriod;
+  if (const char *env = std::getenv("PCA_FEAT_ROUND_PERIOD")) {
+    const int v = std::atoi(env);
+    if (v >= 1 && v <= 64)
+      p.round_period = v;
+  }
+  p.tau = tau;
+  p.partial = partial;
+  p.cand = cand;
+  p.redo_q = redo_q;
+  p.out_idx = out.idx;
+  p.out_dist = out.dist;
+  p.out_count = out.count;
+
+  const int kp = feat_width(k);
+  const int grid = tiles_bound * chunks;
+  if (time_start)
+    (void)hipEventRecord(time_start, stream);
+  hipError_t err;
+  switch (nb) {
+  case 3:
+    err = launch_knn_feat_blocks<3>(p, kp, cosine, grid, stream);
+    break;
+  case 5:
+    err = launch_knn_feat_blocks<5>(p, kp, cosine, grid, stream);
+    break;
+  case 9:
+    err = launch_knn_feat_blocks<9>(p, kp, cosine, grid, stream);
+    break;
+  default:
+    err = launch_knn_feat_blocks<17>(p, kp, cosine, grid, stream);
+    break;
+  }
+  if (time_stop)
+    (void)hipEventRecord(time_stop, stream);
+  if (err != hipSuccess)
+    return err;
+
+  switch (kp) {
+  case 24:
+    launch_feat_merge<24>(p, tiles_bound, stream);
+    break;
+  case 32:
+    launch_feat_merge<32>(p, tiles_bound, stream);
+    break;
+  case 48:
+    launch_feat_merge<48>(p, tiles_bound, stream);
+    break;
+  default:
+    launch_feat_merge<64>(p, tiles_bound, stream);
+    break;
+  }
+  {
+    const int waves = kBlock / kWave;
+    const int rgrid = (in.m + waves - 1) / waves;
+    if (cosine)
+      hipLaunchKernelGGL((feat_refine_kernel<true>), dim3(rgrid),
+                         dim3(kBlock), 0, stream, p);
+    else
+      hipLaunchKernelGGL((feat_refine_kernel<false>), dim3(rgrid),
+                         dim3(kBlock), 0, stream, p);
+  }
+  err = hipGetLastError();
+  if (err != hipSuccess)
+    return err;
+
+  // Second pass for the flagged queries: the kernels are queued in any case
+  // and leave at once while nothing is flagged (no host read in between).
+  const int *gate = &globals->any_redo;
+  if (in.d <= 128) {
+    MfmaSecondPass second{gate, redo_q, x_norm, y_norm, kSecondPassChunks};
+    return launch_knn_mfma(in, k, cosine, work_start, first_pass, out, nullptr,
+                           nullptr, stream, nullptr, &second);
+  }
+  err = launch_plan(in.ptr_y, in.m, in.num_segments, kBlock, plan256, stream);
+  if (err != hipSuccess)
+    return err;
+  return launch_knn_generic(
+      in, k, cosine, x_norm, plan256,
+      plan_upper_bound(in.m, in.num_segments, kBlock), out, stream, gate,
+      redo_q);
+}
+
+} // namespace pca

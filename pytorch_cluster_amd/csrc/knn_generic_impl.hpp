@@ -37,7 +37,8 @@ __global__ __launch_bounds__(kBlock) void knn_generic_kernel(
     const float *__restrict__ x_norm, int n, int m, int d, int num_segments,
     int k, const int *__restrict__ work_start, int grid,
     int *__restrict__ out_idx, float *__restrict__ out_dist,
-    int *__restrict__ out_count) {
+    int *__restrict__ out_count, const int *__restrict__ gate,
+    const int *__restrict__ redo_q) {
   constexpr int TG = kGenTile;
   constexpr int CH = kGenChunk;
   constexpr int QCAP = kGenQueueCap;
@@ -46,6 +47,10 @@ __global__ __launch_bounds__(kBlock) void knn_generic_kernel(
   __shared__ float xn[TG];
   __shared__ double queue[QCAP][kBlock];
 
+  // (second pass behind another search: only when that search flagged
+  // queries, and only the flagged ones)
+  if (gate != nullptr && *gate == 0)
+    return;
   const int tid = threadIdx.x;
   const int tile = PCA_TILE_OF_BLOCK(blockIdx.x, grid);
   if (tile >= work_start[num_segments])
@@ -56,7 +61,12 @@ __global__ __launch_bounds__(kBlock) void knn_generic_kernel(
   const int y_begin = ptr_y ? (int)ptr_y[seg] : 0;
   const int y_end = ptr_y ? (int)ptr_y[seg + 1] : m;
   const int q = y_begin + (tile - work_start[seg]) * kBlock + tid;
-  const bool valid = q < y_end;
+  bool valid = q < y_end;
+  if (redo_q != nullptr) {
+    valid = valid && redo_q[q] != 0;
+    if (!__syncthreads_or(valid))
+      return;
+  }
   const float *yrow = y + (size_t)(valid ? q : y_begin) * d;
 
   double best[K];
@@ -197,7 +207,8 @@ hipError_t launch_knn_generic_metric(const SearchInput &in, int k, int kbucket,
                                      const float *x_norm,
                                      const int *work_start, int grid_bound,
                                      const DenseResult &out,
-                                     hipStream_t stream);
+                                     hipStream_t stream, const int *gate,
+                                     const int *redo_q);
 
 #define PCA_GENERIC_CASE(KB, C)                                                \
   case KB:                                                                     \
@@ -205,7 +216,7 @@ hipError_t launch_knn_generic_metric(const SearchInput &in, int k, int kbucket,
                        0, stream, (const float *)in.x, (const float *)in.y,    \
                        in.ptr_x, in.ptr_y, x_norm, in.n, in.m, in.d,           \
                        in.num_segments, k, work_start, grid, out.idx,          \
-                       out.dist, out.count);                                   \
+                       out.dist, out.count, gate, redo_q);                     \
     break;
 
 #define PCA_GENERIC_DEFINE(C)                                                  \
@@ -213,7 +224,7 @@ hipError_t launch_knn_generic_metric(const SearchInput &in, int k, int kbucket,
   hipError_t launch_knn_generic_metric<C>(                                     \
       const SearchInput &in, int k, int kbucket, const float *x_norm,          \
       const int *work_start, int grid_bound, const DenseResult &out,           \
-      hipStream_t stream) {                                                    \
+      hipStream_t stream, const int *gate, const int *redo_q) {                \
     const int grid = (grid_bound + 7) & ~7;                                    \
     switch (kbucket) {                                                         \
       PCA_GENERIC_CASE(8, C)                                                   \

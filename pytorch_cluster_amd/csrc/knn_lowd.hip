@@ -282,14 +282,15 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
 hipError_t launch_knn_generic(const SearchInput &in, int k, bool cosine,
                               const float *x_norm, const int *work_start,
                               int grid_bound, const DenseResult &out,
-                              hipStream_t stream) {
+                              hipStream_t stream, const int *gate,
+                              const int *redo_q) {
   const int kb = k_bucket(k);
   return cosine ? launch_knn_generic_metric<true>(in, k, kb, x_norm,
                                                   work_start, grid_bound, out,
-                                                  stream)
+                                                  stream, gate, redo_q)
                 : launch_knn_generic_metric<false>(in, k, kb, x_norm,
                                                    work_start, grid_bound, out,
-                                                   stream);
+                                                   stream, gate, redo_q);
 }
 
 } // namespace pca

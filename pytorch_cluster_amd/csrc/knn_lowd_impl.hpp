@@ -72,6 +72,10 @@ struct KnnLowdParams {
   float *out_dist;
   int *out_count;
   int64_t *out_nearest;  // [m] result of the `nearest` search, else unused
+  // second pass behind another search (knn_merge_kernel): nothing runs while
+  // *gate is 0, and only queries with a non-zero redo_q entry are written
+  const int *gate = nullptr;
+  const int *redo_q = nullptr;
 };
 
 __device__ __forceinline__ float next_up_positive(float v) {
@@ -521,6 +525,8 @@ knn_lowd_kernel(KnnLowdParams p) {
 // p.num_chunks is the number of lists per query.
 template <int K, int TQ, bool NEAREST = false>
 __global__ __launch_bounds__(kBlock) void knn_merge_kernel(KnnLowdParams p) {
+  if (p.gate != nullptr && *p.gate == 0)
+    return;
   const int tid = threadIdx.x;
   const int total_tiles = p.work_start[p.num_segments];
   const int tile = blockIdx.x;
@@ -551,7 +557,7 @@ __global__ __launch_bounds__(kBlock) void knn_merge_kernel(KnnLowdParams p) {
         sorted_insert<K>(best, key);
       }
     }
-    if (q < y_end) {
+    if (q < y_end && (p.redo_q == nullptr || p.redo_q[q] != 0)) {
       if constexpr (NEAREST) // (k = 1: the one real slot is the last)
         write_nearest(best[K - 1], q, p.ptr_x ? (int)p.ptr_x[seg] : 0,
                       p.out_nearest);

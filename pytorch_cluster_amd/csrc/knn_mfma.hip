@@ -14,14 +14,15 @@ hipError_t launch_knn_mfma_blocks(const KnnMfmaParams &p, int kbucket,
 template <int NB>
 hipError_t launch_mfma_pack_rows(const float *x, const float *norms, int n,
                                  int d, bool cosine, uint4 *out,
-                                 hipStream_t stream);
+                                 hipStream_t stream, const int *gate);
 #define PCA_DECLARE_BLOCKS(NB)                                                 \
   template <>                                                                  \
   hipError_t launch_knn_mfma_blocks<NB>(const KnnMfmaParams &, int, bool,      \
                                         int, hipStream_t);                     \
   template <>                                                                  \
   hipError_t launch_mfma_pack_rows<NB>(const float *, const float *, int,      \
-                                       int, bool, uint4 *, hipStream_t);
+                                       int, bool, uint4 *, hipStream_t,        \
+                                       const int *);
 PCA_DECLARE_BLOCKS(2)
 PCA_DECLARE_BLOCKS(3)
 PCA_DECLARE_BLOCKS(5)
@@ -111,10 +112,13 @@ int knn_mfma_slices(int n, int m, int num_segments) {
   return chunks;
 }
 
-size_t knn_mfma_scratch_bytes(int n, int m, int d, int num_segments, int k) {
+size_t knn_mfma_scratch_bytes(int n, int m, int d, int num_segments, int k,
+                              int forced_chunks) {
   const size_t tiles = plan_upper_bound(m, num_segments, kMfmaQueries);
   // the largest slice count a call may choose
-  const int chunks = std::max(knn_mfma_slices(n, m, num_segments), 1);
+  const int chunks = forced_chunks > 0
+                         ? forced_chunks
+                         : std::max(knn_mfma_slices(n, m, num_segments), 1);
   return mfma_pack_bytes(n, d) + align256(sizeof(float) * (size_t)n) +
          2 * align256(sizeof(float) * (size_t)m) +
          align256(sizeof(double) * tiles * chunks * (size_t)k *
@@ -125,11 +129,13 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
                            const int *work_start, void *scratch,
                            const DenseResult &out, hipEvent_t time_start,
                            hipEvent_t time_stop, hipStream_t stream,
-                           int64_t *nearest_out) {
+                           int64_t *nearest_out, const MfmaSecondPass *second) {
   const bool nearest = nearest_out != nullptr;
   const int tiles_bound =
       plan_upper_bound(in.m, in.num_segments, kMfmaQueries);
-  const int chunks = knn_mfma_slices(in.n, in.m, in.num_segments);
+  const int chunks = second ? second->chunks
+                            : knn_mfma_slices(in.n, in.m, in.num_segments);
+  const int *gate = second ? second->gate : nullptr;
   char *base = static_cast<char *>(scratch);
   uint4 *x_pack = reinterpret_cast<uint4 *>(base);
   base += mfma_pack_bytes(in.n, in.d);
@@ -141,7 +147,11 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   base += align256(sizeof(float) * (size_t)in.m);
   double *partial = reinterpret_cast<double *>(base);
 
-  if (cosine) {
+  if (second) {
+    // the first pass has the norms already
+    x_sq = const_cast<float *>(second->x_norm);
+    y_norm = const_cast<float *>(second->y_norm);
+  } else if (cosine) {
     (void)launch_row_norms(static_cast<const float *>(in.x), in.n, in.d, x_sq,
                            stream);
     (void)launch_row_norms(static_cast<const float *>(in.y), in.m, in.d,
@@ -159,19 +169,19 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
     switch (mfma_blocks(in.d)) {
     case 2:
       perr = launch_mfma_pack_rows<2>(xf, x_sq, in.n, in.d, cosine, x_pack,
-                                      stream);
+                                      stream, gate);
       break;
     case 3:
       perr = launch_mfma_pack_rows<3>(xf, x_sq, in.n, in.d, cosine, x_pack,
-                                      stream);
+                                      stream, gate);
       break;
     case 5:
       perr = launch_mfma_pack_rows<5>(xf, x_sq, in.n, in.d, cosine, x_pack,
-                                      stream);
+                                      stream, gate);
       break;
     default:
       perr = launch_mfma_pack_rows<9>(xf, x_sq, in.n, in.d, cosine, x_pack,
-                                      stream);
+                                      stream, gate);
       break;
     }
     if (perr != hipSuccess)
@@ -195,6 +205,8 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   p.num_chunks = chunks;
   p.tau = tau;
   p.partial = partial;
+  p.gate = gate;
+  p.redo_q = second ? second->redo_q : nullptr;
 
   const int kb = nearest ? 1 : k_bucket(k);
   const int grid = tiles_bound * chunks;
@@ -238,6 +250,8 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
   mp.out_count = out.count;
   mp.out_nearest = nearest_out;
   mp.x_split = nullptr;
+  mp.gate = gate;
+  mp.redo_q = second ? second->redo_q : nullptr;
   switch (kb) {
   case 1:
     hipLaunchKernelGGL((knn_merge_kernel<8, kMfmaQueries, true>),

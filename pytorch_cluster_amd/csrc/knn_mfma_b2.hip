@@ -10,7 +10,7 @@ hipError_t launch_knn_mfma_blocks(const KnnMfmaParams &p, int kbucket,
 template <int NB>
 hipError_t launch_mfma_pack_rows(const float *x, const float *norms, int n,
                                  int d, bool cosine, uint4 *out,
-                                 hipStream_t stream);
+                                 hipStream_t stream, const int *gate);
 
 PCA_KNN_MFMA_DEFINE(2)
 

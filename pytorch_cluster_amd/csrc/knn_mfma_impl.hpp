@@ -96,6 +96,10 @@ struct KnnMfmaParams {
   int num_chunks;        // slices of every segment's x rows
   float *tau;            // [m] shared pruning bounds
   double *partial;       // [num_chunks * tiles][k][128] keys
+  // second pass behind another search: nothing runs while *gate is 0, and
+  // only tiles with a query whose redo_q entry is non-zero are searched
+  const int *gate = nullptr;
+  const int *redo_q = nullptr;
 };
 
 // Squared row norms, one FMA per component in ascending order.
@@ -138,8 +142,10 @@ __device__ __forceinline__ float mfma_filter_cut(float thresh, float ysq,
 template <int NB, bool COSINE>
 __global__ __launch_bounds__(kBlock) void mfma_pack_rows_kernel(
     const float *__restrict__ x, const float *__restrict__ norms, int n, int d,
-    uint4 *__restrict__ out) {
+    uint4 *__restrict__ out, const int *__restrict__ gate) {
   typedef MfmaShape<NB> S;
+  if (gate != nullptr && *gate == 0)
+    return;
   const size_t id = (size_t)blockIdx.x * kBlock + threadIdx.x;
   if (id >= (size_t)n * S::UNITS)
     return;
@@ -240,6 +246,8 @@ __global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfm
   __shared__ int2 pairs[kBlock / kWave][CAP];
   __shared__ double results[kBlock / kWave][CAP];
 
+  if (p.gate != nullptr && *p.gate == 0)
+    return;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
@@ -260,6 +268,9 @@ __global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfm
   const int y_end = p.ptr_y ? (int)p.ptr_y[seg + 1] : p.m;
   const int q = y_begin + (tile - p.work_start[seg]) * TQ + wave * 32 + col;
   const bool valid = q < y_end;
+  if (p.redo_q != nullptr &&
+      !__syncthreads_or(valid && p.redo_q[q] != 0))
+    return;
   const int d = p.d;
   const int k = p.k;
   const float *yrow = p.y + (size_t)(valid ? q : y_begin) * d;
@@ -780,15 +791,16 @@ __global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfm
   template <>                                                                  \
   hipError_t launch_mfma_pack_rows<NB_>(const float *x, const float *norms,    \
                                         int n, int d, bool cosine, uint4 *out, \
-                                        hipStream_t stream) {                  \
+                                        hipStream_t stream,                    \
+                                        const int *gate) {                     \
     const size_t units = (size_t)n * MfmaShape<NB_>::UNITS;                    \
     const unsigned grid = (unsigned)((units + kBlock - 1) / kBlock);           \
     if (cosine)                                                                \
       hipLaunchKernelGGL((mfma_pack_rows_kernel<NB_, true>), dim3(grid),       \
-                         dim3(kBlock), 0, stream, x, norms, n, d, out);        \
+                         dim3(kBlock), 0, stream, x, norms, n, d, out, gate);  \
     else                                                                       \
       hipLaunchKernelGGL((mfma_pack_rows_kernel<NB_, false>), dim3(grid),      \
-                         dim3(kBlock), 0, stream, x, norms, n, d, out);        \
+                         dim3(kBlock), 0, stream, x, norms, n, d, out, gate);  \
     return hipGetLastError();                                                  \
   }
 

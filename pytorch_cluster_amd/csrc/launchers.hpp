@@ -109,14 +109,41 @@ hipError_t launch_radius_binned(const SearchInput &in, float r2,
 
 constexpr int kMfmaTileQueries = 128;
 bool knn_mfma_supported(int d, int k, bool cosine);
-size_t knn_mfma_scratch_bytes(int n, int m, int d, int num_segments, int k);
+// forced_chunks > 0: for that number of slices instead of the call's own choice
+size_t knn_mfma_scratch_bytes(int n, int m, int d, int num_segments, int k,
+                              int forced_chunks = 0);
+// The search as a second pass behind another one, for the queries that one
+// flagged: nothing runs while *gate is 0; only tiles with a flagged query
+// (redo_q [m], non-zero) are searched and only flagged queries written; the
+// norms come from the first pass (x_norm: squared norms, for the cosine
+// distance norms; y_norm: cosine only).
+struct MfmaSecondPass {
+  const int *gate;
+  const int *redo_q;
+  const float *x_norm;
+  const float *y_norm;
+  int chunks; // slices of every segment's x rows
+};
 // work_start: tiles of kMfmaTileQueries queries.  nearest_out: the `nearest`
 // search (k = 1, Euclidean; `out` unused, [m] rows written there).
 hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
                            const int *work_start, void *scratch,
                            const DenseResult &out, hipEvent_t time_start,
                            hipEvent_t time_stop, hipStream_t stream,
-                           int64_t *nearest_out = nullptr);
+                           int64_t *nearest_out = nullptr,
+                           const MfmaSecondPass *second = nullptr);
+
+// --- knn_feat*.hip ---------------------------------------------------------
+
+// Feature-space kNN with the fp16 matrix-core filter and the exact second
+// kernel (knn_feat_impl.hpp): fp32, 8 < d <= 256, k <= 48.
+bool knn_feat_supported(int d, int k, bool cosine);
+size_t knn_feat_scratch_bytes(int n, int m, int d, int num_segments, int k);
+// work_start: tiles of kMfmaTileQueries queries (planned by the caller).
+hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
+                           const int *work_start, void *scratch,
+                           const DenseResult &out, hipEvent_t time_start,
+                           hipEvent_t time_stop, hipStream_t stream);
 
 // --- knn_generic_*.hip -----------------------------------------------------
 
@@ -124,11 +151,14 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
 hipError_t launch_row_norms(const float *x, int n, int d, float *norm,
                             hipStream_t stream);
 // x_norm: [n] row norms of x (cosine only, else NULL).  One query per lane:
-// work items are tiles of kBlock queries.
+// work items are tiles of kBlock queries.  As a second pass behind another
+// search: gate (device flag, nothing runs while it is 0) and redo_q ([m], only
+// queries with a non-zero entry are searched and written).
 hipError_t launch_knn_generic(const SearchInput &in, int k, bool cosine,
                               const float *x_norm, const int *work_start,
                               int grid_bound, const DenseResult &out,
-                              hipStream_t stream);
+                              hipStream_t stream, const int *gate = nullptr,
+                              const int *redo_q = nullptr);
 
 // --- anytype.hip (fp64 / fp16 / bf16; dtype codes of enum pca_dtype) -------
 

@@ -1,0 +1,162 @@
+"""CPU model of the fp16 matrix-core filter of the feature-space kNN
+(pytorch_cluster_amd/csrc/knn_feat_impl.hpp): the value l the filter derives
+for a (row, query) pair must never exceed the distance e the reference's
+scalar loop computes (csrc/cuda/knn_cuda.cu:61-64), and F(l) must never fall
+below it -- on random rows and on rows built to make the fp16 roundings add up
+(every component at a rounding midpoint, query equal to the row, mixed scales,
+values at the flush-to-zero limit).
+
+The model rounds exactly as the kernels do (numpy float16, the same flush and
+the same truncated parts of W) and sums the products in float64, i.e. without
+the matrix cores' own accumulation error; the test therefore demands that the
+roundings alone leave the share of the budget that the header of
+knn_feat_impl.hpp reserves for accumulation (0.15 x 2^-10 of |X|^2 + |Y|^2 at
+256 components) unused.
+"""
+import numpy as np
+import pytest
+
+RHO = 1.0 / 512.0
+GROW = 1.0 + 4.1 / 512.0
+
+
+def inv_sigma(max_abs):
+    if max_abs == 0:
+        return 1.0
+    bits = np.float32(max_abs).view(np.uint32)
+    e = 137 - int((bits >> 23) & 0xff)
+    return float(2.0 ** max(-100, min(100, e)))
+
+
+def h(v):
+    """fp16 nearest-even, magnitudes below 2^-14 flushed to zero."""
+    v = np.asarray(v, dtype=np.float32)
+    out = v.astype(np.float16).astype(np.float64)
+    out[np.abs(v) < 2.0 ** -14] = 0.0
+    return out
+
+
+def h_down(v):
+    """Largest flushed fp16 <= v (v >= 0)."""
+    r = np.float16(np.float32(v))
+    if float(r) > v:
+        r = np.nextafter(r, np.float16(0))
+    if v >= 65504.0:
+        r = np.float16(65504.0)
+    return 0.0 if float(r) < 2.0 ** -14 else float(r)
+
+
+def w_parts(w):
+    a1 = h_down(w / 32768.0)
+    r1 = w - a1 * 32768.0
+    a2 = h_down(r1 / 16.0)
+    r2 = r1 - a2 * 16.0
+    a3 = h_down(r2 * 128.0)
+    return a1 * 32768.0 + a2 * 16.0 + a3 / 128.0
+
+
+def reference_distances(x, y):
+    """e[j, i]: one fused multiply-add per component in ascending order, in
+    fp32 (float64 holds the exact product and sum of two fp32 numbers'
+    product and a third before the one rounding)."""
+    e = np.zeros((len(y), len(x)), dtype=np.float32)
+    for c in range(x.shape[1]):
+        diff = (x[None, :, c] - y[:, None, c]).astype(np.float32)
+        e = (diff.astype(np.float64) ** 2 + e.astype(np.float64)).astype(
+            np.float32)
+    return e.astype(np.float64)
+
+
+def check(x, y):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    d = x.shape[1]
+    inv = inv_sigma(max(np.abs(x).max(), np.abs(y).max()))
+    scale2 = inv * inv
+    c0 = d / 4096.0 + d * 2.0 ** -149 * scale2
+    xs = (x * np.float32(inv)).astype(np.float32)
+    ys = (y * np.float32(inv)).astype(np.float32)
+    hx = h(xs)
+    hy = h(-2.0 * ys.astype(np.float64))
+    xsq32 = np.zeros(len(x), dtype=np.float32)
+    for c in range(d):  # (any fp32 summation order serves)
+        xsq32 = (x[:, c].astype(np.float64) ** 2 + xsq32).astype(np.float32)
+    w = np.array([w_parts(float(v) * scale2 * (1.0 - RHO)) for v in xsq32])
+    s = w[None, :] + hy @ hx.T
+    ysq = (ys.astype(np.float64) ** 2).sum(1)
+    shift = ysq * (1.0 - RHO) - c0
+    widen = 6.0 * RHO * ysq + 2.0 * c0
+    lower = s + shift[:, None]
+    upper = (lower + widen[:, None]) * GROW
+    e = reference_distances(x, y) * scale2
+    norms = (xs.astype(np.float64) ** 2).sum(1)[None, :] + ysq[:, None]
+    room = 0.15 * 2.0 ** -10 * norms  # what accumulation may still take
+    assert (lower + room <= e + 1e-300).all(), \
+        "lower bound above the reference's distance"
+    assert (e <= upper - room).all(), "upper bound below it"
+    return float(np.max((lower - (e - RHO * norms - c0))
+                        / (RHO * norms + c0)))
+
+
+def midpoint_rows(rng, n, d, exponents, side):
+    # every component sits just below (side = -1) or just above (+1) the
+    # middle between two fp16 numbers (odd multiples of 2^-11 of its power of
+    # two), all with one sign: every rounding goes the same way by nearly the
+    # largest amount, and in a row times itself the errors add up
+    frac = 1.0 + (2 * rng.integers(0, 1024, (n, d)) + 1) * 2.0 ** -11
+    frac = frac + side * 2.0 ** -21
+    return (frac * 2.0 ** exponents).astype(np.float32)
+
+
+@pytest.mark.parametrize("d", [9, 64, 128, 256])
+def test_random_rows(d):
+    rng = np.random.default_rng(d)
+    x = rng.standard_normal((400, d))
+    y = rng.standard_normal((60, d))
+    check(x, y)
+    check(x, x[:60])  # queries that are rows: distance zero
+
+
+@pytest.mark.parametrize("d", [16, 128, 256])
+def test_rounding_midpoints_with_one_sign(d):
+    rng = np.random.default_rng(d + 1)
+    used = []
+    for side in (-1, 1):
+        x = midpoint_rows(rng, 300, d, 0, side)
+        used.append(check(x, x[:50]))
+        y = midpoint_rows(rng, 50, d, 0, side)
+        used.append(check(x, y))
+    # rounding down in a row times itself takes about half of the budget (the
+    # products are 2^-10 too small, and rho = 2 x 2^-10): the case is as hard
+    # as it is meant to be
+    assert 0.3 <= max(used) <= 0.7
+
+
+@pytest.mark.parametrize("case", ["mixed", "flush_limit", "tiny", "huge",
+                                  "outlier", "near_duplicates"])
+def test_scales(case):
+    rng = np.random.default_rng(hash(case) % 2 ** 32)
+    d = 96
+    if case == "mixed":
+        x = midpoint_rows(rng, 300, d, rng.integers(-12, 1, (300, 1)), -1)
+        y = midpoint_rows(rng, 40, d, rng.integers(-12, 1, (40, 1)), -1)
+    elif case == "flush_limit":
+        # after scaling most components lie around 2^-14, where fp16 flushes
+        x = rng.standard_normal((300, d)) * 2.0 ** -24
+        x[0] = 1.0
+        y = rng.standard_normal((40, d)) * 2.0 ** -24
+    elif case == "tiny":
+        x = rng.standard_normal((300, d)) * 1e-21
+        y = rng.standard_normal((40, d)) * 1e-21
+    elif case == "huge":
+        x = rng.standard_normal((300, d)) * 1e16
+        y = rng.standard_normal((40, d)) * 1e16
+    elif case == "outlier":
+        x = rng.standard_normal((300, d))
+        x[5] *= 1e6
+        y = rng.standard_normal((40, d))
+    else:
+        base = rng.standard_normal((10, d))
+        x = np.repeat(base, 30, 0) * (1 + 1e-6 * rng.standard_normal((300, d)))
+        y = base * (1 + 1e-6 * rng.standard_normal((10, d)))
+    check(x, y)

@@ -1,0 +1,174 @@
+"""Feature-space kNN with the fp16 matrix-core filter (knn_feat_impl.hpp):
+parity with the CPU checker where the mechanisms of that path are exercised --
+lists that overflow (near-duplicates: the flagged queries go through the
+second pass), rows and queries the filter cannot represent, 129-256
+components, every list width, scales at both ends of fp32.  Bit-exact edges
+and distances, as everywhere.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(oracle, x, y, ptr_x, ptr_y, k, cosine=False):
+    from gpu_common import gpu_knn, oracle_knn_edges
+    got, gd = gpu_knn(x, y, ptr_x, ptr_y, k, cosine=cosine)
+    want, wd = oracle_knn_edges(oracle, x, y, ptr_x, ptr_y, k, cosine=cosine)
+    assert got.shape == want.shape
+    assert (got == want).all()
+    assert (gd == wd).all()
+
+
+def _flagged_queries(x, y, k, cosine=False):
+    """Number of queries the filter kernel handed to the second pass (read
+    from the per-call block at the start of the path's scratch: the workspace
+    begins with the [n] row norms, 256-byte aligned)."""
+    from gpu_common import dev
+    from pytorch_cluster_amd import capi
+    xd, yd = dev(x), dev(y)
+    _e, _n, _d, ws = capi.knn_launch(xd, yd, None, None, k, cosine)
+    torch.cuda.synchronize()
+    off = (4 * x.shape[0] + 255) // 256 * 256
+    words = ws[off:off + 16].cpu().view(torch.int32).tolist()
+    return words[1], words[2]  # (rows the filter cannot represent, flagged)
+
+
+@pytest.mark.parametrize("d,k,cosine", [(130, 5, False), (200, 16, False),
+                                        (256, 32, False), (256, 32, True),
+                                        (129, 48, True), (24, 33, False),
+                                        (64, 40, True), (96, 48, False),
+                                        (32, 1, False), (48, 8, True)])
+def test_parity_wide_rows_and_every_list_width(oracle, d, k, cosine):
+    rng = np.random.default_rng(d * 11 + k)
+    n, m = 3000, 500
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    y = rng.standard_normal((m, d)).astype(np.float32)
+    ptr_x = np.array([0, 70, 70, 1200, 3000])
+    ptr_y = np.array([0, 100, 130, 131, 500])
+    _run(oracle, x, y, ptr_x, ptr_y, k, cosine)
+
+
+@pytest.mark.parametrize("d", [20, 128, 200])
+@pytest.mark.parametrize("cosine", [False, True])
+def test_near_duplicates_go_through_the_second_pass(oracle, d, cosine):
+    # 60 copies (equal up to the last bits) of every cluster centre: far more
+    # than 16 rows within the filter's rounding margin of the k-th distance,
+    # so the lists cannot be shown complete and the queries are searched again
+    rng = np.random.default_rng(d)
+    centres = rng.standard_normal((40, d)).astype(np.float32)
+    x = np.repeat(centres, 60, axis=0)
+    x = x * (1.0 + 1e-7 * rng.standard_normal(x.shape)).astype(np.float32)
+    x = x[rng.permutation(len(x))].astype(np.float32)
+    y = np.concatenate([centres[:25],
+                        rng.standard_normal((40, d)).astype(np.float32)])
+    odd, flagged = _flagged_queries(x, y, 8, cosine)
+    assert odd == 0 and flagged >= 25
+    _run(oracle, x, y, None, None, 8, cosine)
+    # exact duplicates: ties settled by row number
+    x2 = np.repeat(centres, 30, axis=0)
+    _run(oracle, x2, y, None, None, 20, cosine)
+
+
+def test_rows_and_queries_the_filter_cannot_represent(oracle):
+    rng = np.random.default_rng(3)
+    d = 40
+    x = rng.standard_normal((2000, d)).astype(np.float32)
+    y = rng.standard_normal((300, d)).astype(np.float32)
+    # NaN and infinite components: never neighbours, the filter skips them
+    xa = x.copy()
+    xa[5, 3] = np.nan
+    xa[700] = np.inf
+    xa[900, 0] = -np.inf
+    ya = y.copy()
+    ya[7, 1] = np.nan      # no neighbours at all
+    ya[8] = np.inf
+    odd, flagged = _flagged_queries(xa, ya, 12)
+    assert odd == 0
+    _run(oracle, xa, ya, None, None, 12)
+    _run(oracle, xa, ya, None, None, 12, cosine=True)
+    # finite rows whose squared norm overflows: everything takes the second
+    # pass (such a row can be the duplicate of an equally large query)
+    xb = x.copy()
+    xb[11] = 3e19
+    yb = y.copy()
+    yb[4] = 3e19
+    odd, flagged = _flagged_queries(xb, yb, 12)
+    assert odd == 1 and flagged == len(yb)
+    _run(oracle, xb, yb, None, None, 12)
+    _run(oracle, xb, yb, None, None, 12, cosine=True)
+    # a query of that kind alone: only its tile is searched again
+    odd, flagged = _flagged_queries(x, yb, 12)
+    assert odd == 0 and flagged == 1
+    _run(oracle, x, yb, None, None, 12)
+
+
+@pytest.mark.parametrize("case", ["tiny", "huge", "mixed", "outlier",
+                                  "zeros", "sparse"])
+def test_scales_at_both_ends(oracle, case):
+    # one power of two scales all rows into the fp16 range: rows far below the
+    # largest one lose their bits there, and the lists must notice
+    rng = np.random.default_rng(hash(case) % 2 ** 32)
+    d, n, m, k = 72, 4000, 400, 16
+    x = rng.standard_normal((n, d))
+    y = rng.standard_normal((m, d))
+    if case == "tiny":
+        x, y = 1e-30 * x, 1e-30 * y
+    elif case == "huge":
+        x, y = 1e15 * x, 1e15 * y
+        y[:40] = x[:40]
+    elif case == "mixed":
+        x = x * 10.0 ** rng.integers(-5, 6, (n, 1))
+        y = y * 10.0 ** rng.integers(-5, 6, (m, 1))
+    elif case == "outlier":
+        x[17] *= 1e9   # one row sets the scale, all others are tiny beside it
+    elif case == "zeros":
+        x[:] = 0.0
+        x[100:110] = 1.0
+        y[:5] = 0.0
+    else:
+        x = x * (rng.random((n, d)) < 0.05)
+        y = y * (rng.random((m, d)) < 0.05)
+    x = x.astype(np.float32)
+    y = y.astype(np.float32)
+    ptr_x = np.array([0, 1500, 4000])
+    ptr_y = np.array([0, 150, 400])
+    _run(oracle, x, y, ptr_x, ptr_y, k)
+    if case not in ("zeros",):
+        _run(oracle, x, y, ptr_x, ptr_y, k, cosine=True)
+
+
+def test_many_slices_share_their_bounds(oracle, monkeypatch):
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((20000, 64)).astype(np.float32)
+    y = rng.standard_normal((300, 64)).astype(np.float32)
+    for slices in ("1", "3", "16"):
+        monkeypatch.setenv("PCA_KNN_SLICES", slices)
+        _run(oracle, x, y, None, None, 24)
+        _run(oracle, x, y, None, None, 24, cosine=True)
+
+
+def test_feature_space_knn_256_full_size_properties(oracle):
+    # 50,000 rows of 256 components onto themselves, k = 32: every 400th query
+    # exactly, all of them by the properties the result must have
+    from gpu_common import dev
+    from pytorch_cluster_amd import capi
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(50000, 256, generator=g)
+    e, dist = capi.knn_edges(dev(x.numpy()), dev(x.numpy()), None, None, 32,
+                             want_dist=True)
+    torch.cuda.synchronize()
+    e, dist = e.cpu().numpy(), dist.cpu().numpy()
+    assert e.shape == (2, 50000 * 32)
+    rows = e[0].reshape(50000, 32)
+    cols = e[1].reshape(50000, 32)
+    dd = dist.reshape(50000, 32)
+    assert (rows == np.arange(50000)[:, None]).all()
+    assert (cols[:, 0] == np.arange(50000)).all() and (dd[:, 0] == 0).all()
+    assert (np.diff(dd, axis=1) >= 0).all()
+    sample = np.arange(0, 50000, 400)
+    xs = x.numpy()
+    _, col, d_ref = oracle.knn_dense(xs, xs[sample], None, None, 32)
+    assert (cols[sample] == col).all()
+    assert (dd[sample] == d_ref).all()
