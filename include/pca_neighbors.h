@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define PCA_ABI_VERSION 3
+#define PCA_ABI_VERSION 4
 
 enum pca_status {
   PCA_OK = 0,
@@ -279,6 +279,41 @@ int pca_nearest_binned(const void *x, const void *y, const int64_t *ptr_x,
                        const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
                        int64_t num_segments, int64_t *out, void *workspace,
                        size_t workspace_bytes, void *stream);
+
+/* ----------------------------------------------------- host (CPU) path -- */
+
+/*
+ * The two searches on the host, for points that are not on a GPU.  Every
+ * pointer is HOST memory here; the calls run on `num_threads` threads of their
+ * own (at least one), allocate their temporaries with the C++ allocator and
+ * return when the result is complete.  Same arguments and the same result as
+ * pca_knn / pca_radius (bit for bit, order included), no cosine distance; k
+ * may exceed PCA_KNN_MAX_K.  edges: capacity 2 * m * min(k, n) resp.
+ * 2 * m * pca_radius_slots(n, max_num_neighbors); *num_edges (host) receives E.
+ * dist (optional, fp32 / fp64 points only): capacity m * min(k, n).
+ *
+ * Stand under the CPU branch of the reference operators
+ *   csrc/knn.cpp:32-35 -> knn_cpu, csrc/cpu/knn_cpu.cpp:7-105
+ *   csrc/radius.cpp:31-34 -> radius_cpu, csrc/cpu/radius_cpu.cpp:7-117
+ * (nanoflann k-d trees), with the result contract of the GPU kernels instead
+ * of nanoflann's: neighbours by ascending (distance, row), for the radius
+ * search the first max_num_neighbors rows in row order where the reference's
+ * CPU code keeps those its tree meets first.
+ * Errors: status codes as above, text from pca_host_last_error().
+ */
+const char *pca_host_last_error(void);
+
+int pca_knn_host(const void *x, const void *y, const int64_t *ptr_x,
+                 const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+                 int64_t num_segments, int64_t k, int dtype, int edge_flags,
+                 int num_threads, int64_t *edges, int64_t *num_edges,
+                 void *dist);
+
+int pca_radius_host(const void *x, const void *y, const int64_t *ptr_x,
+                    const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+                    int64_t num_segments, double r, int64_t max_num_neighbors,
+                    int ignore_same_index, int dtype, int edge_flags,
+                    int num_threads, int64_t *edges, int64_t *num_edges);
 
 /* ------------------------------------------------------------------ fps -- */
 

@@ -74,6 +74,15 @@ C_ABI = {
     "pca_nearest_binned": (ctypes.c_int,
                            [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp,
                             _vp, ctypes.c_size_t, _vp]),
+    "pca_host_last_error": (ctypes.c_char_p, []),
+    "pca_knn_host": (ctypes.c_int,
+                     [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
+                      ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp,
+                      _vp]),
+    "pca_radius_host": (ctypes.c_int,
+                        [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
+                         ctypes.c_double, _i64, ctypes.c_int, ctypes.c_int,
+                         ctypes.c_int, ctypes.c_int, _vp, _vp]),
     "pca_fps_workspace_bytes": (ctypes.c_size_t,
                                 [_i64, _i64, _i64, _i64, ctypes.c_int]),
     "pca_fps": (ctypes.c_int,

@@ -52,13 +52,29 @@ def _compile_hip(src):
     return obj
 
 
+# The host (CPU) searches: plain C++, fused multiply-adds and 8-wide vectors
+# (checked for at run time).
+HOST_SOURCES = ["cpu_search.cpp"]
+HOST_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-mavx2", "-mfma", "-pthread",
+              "-fno-math-errno", "-Wall"]
+
+
+def _compile_host(src):
+    obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
+    _run(["g++"] + HOST_FLAGS + ["-c", src, "-o", obj])
+    return obj
+
+
 def build_capi(jobs):
     os.makedirs(OBJ_DIR, exist_ok=True)
     sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    host = [os.path.join(CSRC, name) for name in HOST_SOURCES]
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        host_objects = [pool.submit(_compile_host, src) for src in host]
         objects = list(pool.map(_compile_hip, sources))
-    _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", CAPI_LIB]
-         + objects)
+        objects += [f.result() for f in host_objects]
+    _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-pthread",
+          "-o", CAPI_LIB] + objects)
     return CAPI_LIB
 
 

@@ -9,9 +9,12 @@
 //
 // Validation and error texts follow the reference's GPU host wrappers
 // (csrc/cuda/knn_cuda.cu:91-114, csrc/cuda/radius_cuda.cu:49-73,
-// csrc/cuda/utils.cuh:5-9).  There is no CPU implementation behind these
-// operators: tensors that are not on an AMD GPU are rejected.
+// csrc/cuda/utils.cuh:5-9).  Tensors that are not on a GPU take the host
+// searches (pca_knn_host / pca_radius_host), as the reference's dispatchers
+// send them to knn_cpu / radius_cpu (csrc/knn.cpp:26-36,
+// csrc/radius.cpp:27-35); `nearest` and `fps` are GPU-only here.
 #include <ATen/ATen.h>
+#include <ATen/Parallel.h>
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
 #include <hip/hip_version.h>
@@ -118,7 +121,128 @@ at::Tensor finish(const at::Tensor &edges, const at::Tensor &num_edges) {
   // the only host synchronisation of the operator: the edge count sizes the
   // result (the reference synchronises in its masked_selects)
   const int64_t E = num_edges.item<int64_t>();
-  return edges.narrow(0, 0, 2 * E).view({2, E});
+  at::Tensor out = edges.narrow(0, 0, 2 * E).view({2, E});
+  // (a view keeps the whole slot buffer alive: a result that fills less than
+  // half of it gets storage of its own, like the reference's [2, E])
+  if (4 * E < edges.numel())
+    out = out.clone();
+  return out;
+}
+
+// ---- tensors that are not on a GPU ---------------------------------------
+
+#define PCA_CHECK_CPU(x)                                                       \
+  TORCH_CHECK((x).device().is_cpu(), #x " must be CPU tensor")
+
+struct HostPoints {
+  at::Tensor x, y, ptr_x, ptr_y;
+  const int64_t *px = nullptr, *py = nullptr;
+  int64_t segments = 1;
+  int dtype = PCA_F32;
+};
+
+// Checks of csrc/cpu/knn_cpu.cpp:12-24 / radius_cpu.cpp:13-25; integer points
+// are searched as doubles (their squared distances are exact there).
+HostPoints host_points(at::Tensor x, at::Tensor y,
+                       std::optional<at::Tensor> ptr_x,
+                       std::optional<at::Tensor> ptr_y) {
+  PCA_CHECK_CPU(x);
+  PCA_CHECK_INPUT(x.dim() == 2);
+  PCA_CHECK_CPU(y);
+  PCA_CHECK_INPUT(y.dim() == 2);
+  PCA_CHECK_INPUT(x.size(1) == y.size(1));
+  PCA_CHECK_INPUT(x.scalar_type() == y.scalar_type());
+  HostPoints h;
+  if (ptr_x.has_value()) {
+    PCA_CHECK_CPU(ptr_x.value());
+    PCA_CHECK_INPUT(ptr_x.value().dim() == 1);
+  }
+  if (ptr_y.has_value()) {
+    PCA_CHECK_CPU(ptr_y.value());
+    PCA_CHECK_INPUT(ptr_y.value().dim() == 1);
+  }
+  if (!at::isFloatingType(x.scalar_type())) {
+    x = x.to(at::kDouble);
+    y = y.to(at::kDouble);
+  }
+  h.x = x.contiguous();
+  h.y = y.contiguous();
+  h.dtype = dtype_code(h.x);
+  if (ptr_x.has_value() || ptr_y.has_value()) {
+    if (!ptr_x.has_value())
+      ptr_x = at::arange(0, x.size(0) + 1, x.size(0), at::kLong);
+    if (!ptr_y.has_value())
+      ptr_y = at::arange(0, y.size(0) + 1, y.size(0), at::kLong);
+    PCA_CHECK_INPUT(ptr_x.value().numel() == ptr_y.value().numel());
+    PCA_CHECK_INPUT(ptr_x.value().numel() >= 2);
+    h.ptr_x = ptr_x.value().to(at::kLong).contiguous();
+    h.ptr_y = ptr_y.value().to(at::kLong).contiguous();
+    h.px = h.ptr_x.data_ptr<int64_t>();
+    h.py = h.ptr_y.data_ptr<int64_t>();
+    h.segments = h.ptr_x.numel() - 1;
+  }
+  return h;
+}
+
+int host_threads(int64_t num_workers) {
+  return (int)std::max<int64_t>(std::max<int64_t>(num_workers, 1),
+                                at::get_num_threads());
+}
+
+void check_host_status(int status) {
+  if (status == PCA_OK)
+    return;
+  const char *detail = pca_host_last_error();
+  TORCH_CHECK(false, (detail && detail[0]) ? detail
+                                           : pca_status_string(status));
+}
+
+at::Tensor host_result(const at::Tensor &edges, int64_t E) {
+  at::Tensor out = edges.narrow(0, 0, 2 * E).view({2, E});
+  return 4 * E < edges.numel() ? out.clone() : out;
+}
+
+at::Tensor knn_host(at::Tensor x, at::Tensor y,
+                    std::optional<at::Tensor> ptr_x,
+                    std::optional<at::Tensor> ptr_y, int64_t k, bool cosine,
+                    int flags, int64_t num_workers) {
+  // csrc/knn.cpp:33-34
+  TORCH_CHECK(!cosine, "`cosine` argument not supported on CPU");
+  TORCH_CHECK(k >= 1, "`k` needs to be positive");
+  HostPoints h = host_points(x, y, ptr_x, ptr_y);
+  const int64_t n = h.x.size(0), m = h.y.size(0), d = h.x.size(1);
+  auto long_opts = at::TensorOptions().dtype(at::kLong);
+  if (n == 0 || m == 0)
+    return at::empty({2, 0}, long_opts);
+  auto edges = at::empty({2 * m * std::min(k, n)}, long_opts);
+  int64_t E = 0;
+  check_host_status(pca_knn_host(
+      h.x.data_ptr(), h.y.data_ptr(), h.px, h.py, n, m, d, h.segments, k,
+      h.dtype, flags, host_threads(num_workers), edges.data_ptr<int64_t>(),
+      &E, nullptr));
+  return host_result(edges, E);
+}
+
+at::Tensor radius_host(at::Tensor x, at::Tensor y,
+                       std::optional<at::Tensor> ptr_x,
+                       std::optional<at::Tensor> ptr_y, double r,
+                       int64_t max_num_neighbors, bool ignore_same_index,
+                       int flags, int64_t num_workers) {
+  TORCH_CHECK(max_num_neighbors >= 1,
+              "`max_num_neighbors` needs to be positive");
+  HostPoints h = host_points(x, y, ptr_x, ptr_y);
+  const int64_t n = h.x.size(0), m = h.y.size(0), d = h.x.size(1);
+  auto long_opts = at::TensorOptions().dtype(at::kLong);
+  if (n == 0 || m == 0)
+    return at::empty({2, 0}, long_opts);
+  auto edges =
+      at::empty({2 * m * pca_radius_slots(n, max_num_neighbors)}, long_opts);
+  int64_t E = 0;
+  check_host_status(pca_radius_host(
+      h.x.data_ptr(), h.y.data_ptr(), h.px, h.py, n, m, d, h.segments, r,
+      max_num_neighbors, ignore_same_index ? 1 : 0, h.dtype, flags,
+      host_threads(num_workers), edges.data_ptr<int64_t>(), &E));
+  return host_result(edges, E);
 }
 
 int edge_flags(bool drop_self, bool x_first) {
@@ -189,7 +313,10 @@ bool bins_wanted(int64_t searched, int64_t searching, int64_t num_segments,
 at::Tensor knn_search(at::Tensor x, at::Tensor y,
                       std::optional<at::Tensor> ptr_x,
                       std::optional<at::Tensor> ptr_y, int64_t k, bool cosine,
-                      int flags) {
+                      int flags, int64_t num_workers = 1) {
+  // the device branch of csrc/knn.cpp:26-36
+  if (!x.device().is_cuda())
+    return knn_host(x, y, ptr_x, ptr_y, k, cosine, flags, num_workers);
   PCA_CHECK_GPU(x);
   PCA_CHECK_CONTIGUOUS(x);
   PCA_CHECK_INPUT(x.dim() == 2);
@@ -241,8 +368,9 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
 at::Tensor knn(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
                std::optional<at::Tensor> ptr_y, int64_t k, bool cosine,
                int64_t num_workers) {
-  (void)num_workers; // unused by the reference as well (csrc/cpu/knn_cpu.cpp)
-  return knn_search(x, y, ptr_x, ptr_y, k, cosine, 0);
+  // (num_workers: unused by the reference, csrc/cpu/knn_cpu.cpp; here the
+  // host search runs on at least that many threads)
+  return knn_search(x, y, ptr_x, ptr_y, k, cosine, 0, num_workers);
 }
 
 // The search of knn_graph with its epilogue (torch_cluster/knn.py:135-144)
@@ -260,7 +388,11 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
                          std::optional<at::Tensor> ptr_x,
                          std::optional<at::Tensor> ptr_y, double r,
                          int64_t max_num_neighbors, bool ignore_same_index,
-                         int flags) {
+                         int flags, int64_t num_workers = 1) {
+  // the device branch of csrc/radius.cpp:27-35
+  if (!x.device().is_cuda())
+    return radius_host(x, y, ptr_x, ptr_y, r, max_num_neighbors,
+                       ignore_same_index, flags, num_workers);
   PCA_CHECK_GPU(x);
   PCA_CHECK_CONTIGUOUS(x);
   PCA_CHECK_INPUT(x.dim() == 2);
@@ -317,9 +449,8 @@ at::Tensor radius(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
                   std::optional<at::Tensor> ptr_y, double r,
                   int64_t max_num_neighbors, int64_t num_workers,
                   bool ignore_same_index) {
-  (void)num_workers;
   return radius_search(x, y, ptr_x, ptr_y, r, max_num_neighbors,
-                       ignore_same_index, 0);
+                       ignore_same_index, 0, num_workers);
 }
 
 // The search of radius_graph with the flow flip of

@@ -26,7 +26,7 @@ def test_header_symbols_are_exported():
     for name in sorted(declared):
         assert hasattr(lib, name), "missing export: " + name
     assert declared == set(_native.C_ABI), "ctypes table out of date"
-    assert lib.pca_abi_version() == 3
+    assert lib.pca_abi_version() == 4
 
 
 def test_capi_validation_needs_no_gpu():
@@ -69,16 +69,11 @@ def test_operators_are_registered_and_scriptable():
     assert "float r" in schema and "bool ignore_same_index" in schema
 
 
-def test_cpu_tensors_fail_loudly():
+def test_gpu_only_operators_refuse_cpu_tensors():
     x = torch.rand(8, 3)
-    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
-        pca.knn(x, x, 2)
-    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
-        pca.radius_graph(x, 0.5)
-    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
-        pca.knn_graph(x, 2)
-    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
-        torch.ops.torch_cluster.knn(x, x, None, None, 2, False, 1)
+    with pytest.raises(RuntimeError, match="No CPU version supported"):
+        torch.ops.torch_cluster.nearest(x, x, torch.tensor([0, 8]),
+                                        torch.tensor([0, 8]))
 
 
 def test_empty_inputs_short_circuit():
