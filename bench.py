@@ -51,6 +51,27 @@ class HipEvents:
         self.hip.hipEventDestroy(ev)
 
 
+def cpu_build_baseline(pca, data):
+    """This package's own CPU path (the operators called with CPU tensors:
+    k-d trees searched on all host threads) on the full workload."""
+    import torch
+    x, y = data["x"], data["y"]
+    bx, by = data["batch_x"], data["batch_y"]
+    times = []
+    for _ in range(4):
+        t0 = time.perf_counter()
+        e = pca.knn(x, y, K, bx, by, batch_size=data["batch_size"])
+        times.append(time.perf_counter() - t0)
+    assert e.shape[1] == y.shape[0] * K
+    return {"value": y.shape[0] / statistics.median(times[1:]),
+            "unit": "queries/s", "cores": torch.get_num_threads(),
+            "kind": "build",
+            "sample": "full workload (%d queries over %d points), median of "
+                      "3 calls after one untimed; pytorch_cluster_amd.knn on "
+                      "CPU tensors (k-d tree per scan, queries spread over "
+                      "the host threads)" % (y.shape[0], x.shape[0])}
+
+
 def cpu_baseline(data, ptr_x, ptr_y):
     """The reference's CPU operator (nanoflann KD-tree; single-threaded by
     construction, `num_workers` is never read) on the same inputs, or the
@@ -132,6 +153,28 @@ def _roofline(kernel, kernel_ms, flop, peak_tflops, bound, detail):
             "kernel_ms": kernel_ms, "flop_per_launch": flop,
             "achieved": achieved, "peak": peak_tflops, "unit": "TFLOP/s",
             "frac": achieved / peak_tflops}
+
+
+def _hbm_roofline(kernel, kernel_ms, nbytes, detail):
+    achieved = nbytes / kernel_ms / 1e6
+    return {"bound": "hbm", "bound_detail": detail, "kernel": kernel,
+            "kernel_ms": kernel_ms, "bytes_per_launch": nbytes,
+            "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": achieved / PEAK_HBM_GBS}
+
+
+def _search_bytes(n, m, d, slots, elem=4):
+    """Bytes a neighbour search has to move: every point and query once, and
+    the [2, m * slots] int64 edge list."""
+    return (n + m) * d * elem + m * slots * 16
+
+
+def _feat_shape(d, k):
+    """(16-component blocks per row incl. the one that carries |x|^2, list
+    width) of the feature-space kernel that serves (d, k)."""
+    blocks = next(b for b in (3, 5, 9, 17) if 16 * (b - 1) >= d)
+    width = next(w for w in (24, 32, 48, 64) if w >= k + 16)
+    return blocks, width
 
 
 class Cases:
@@ -218,15 +261,32 @@ class Cases:
         ms, out = _median_ms(t, fn, reps or 3)
         kms = _search_ms(t, self.capi, self.events, fn)
         flop = 2 * d * n * m
+        if k > 48:
+            kernel = "knn_mfma_kernel" if d <= 128 else "knn_generic_kernel"
+            issued = None
+        else:
+            blocks, width = _feat_shape(d, k)
+            kernel = "knn_feat_kernel<%d,%d,%s>" % (
+                blocks, width, "true" if cosine else "false")
+            # one v_mfma_f32_32x32x16_f16 (32,768 flop) per block and 32 x 32
+            # pairs; rows in tiles of 64 (32 from 144 components on), queries
+            # in tiles of 128
+            tile = 64 if blocks <= 9 else 32
+            issued = (-(-n // tile) * tile) * (-(-m // 128) * 128) // 1024 \
+                * blocks * 32768
+        roof = _roofline(
+            kernel, kms, flop, PEAK_BF16_TFLOPS, "mfma",
+            "algorithmic 2*D flop per pair against the dense fp16 / bf16 "
+            "matrix peak; the kernel forms one fp16 product per pair and "
+            "component on the matrix cores (a proven lower bound of the "
+            "distance), keeps k + 16 rows per query, and a second kernel "
+            "evaluates those exactly in fp32")
+        if issued is not None:
+            roof["issued_flop_per_launch"] = issued
+            roof["issued_frac"] = issued / kms / 1e9 / PEAK_BF16_TFLOPS
         return {label: {
             "ms": ms, "queries_per_s": m / ms * 1e3,
-            "edges": int(out.shape[1]),
-            "roofline": _roofline(
-                "knn_mfma_kernel", kms, flop, PEAK_BF16_TFLOPS, "mfma",
-                "algorithmic 2*D flop per pair against the dense bf16 "
-                "matrix peak (the filter is three split-bf16 products per "
-                "pair and component; every returned distance is exact "
-                "fp32)")}}
+            "edges": int(out.shape[1]), "roofline": roof}}
 
     def case_c4(self, reps):
         return self._feature_case(
@@ -239,9 +299,13 @@ class Cases:
             200000, 50000, 128, 32, True, reps)
 
     def case_d256(self, reps):
-        return self._feature_case(
+        report = self._feature_case(
             "knn 50000x256 onto themselves k=32", 50000, 50000, 256, 32,
             False, reps)
+        report.update(self._feature_case(
+            "knn 50000x256 onto themselves k=64", 50000, 50000, 256, 64,
+            False, reps))
+        return report
 
     # nearest: every point of the LiDAR-like scans looks for the nearest of
     # its scan's every-8th point (the operator that follows the neighbour
@@ -284,8 +348,8 @@ class Cases:
                 "knn_mfma_kernel<5,8,nearest>", kms,
                 2 * 64 * feats.shape[0] * 4096, PEAK_BF16_TFLOPS, "mfma",
                 "algorithmic 2*D flop per pair against the dense bf16 "
-                "matrix peak (three split-bf16 products per pair and "
-                "component)")}}
+                "matrix peak (this kernel forms three split-bf16 products "
+                "per pair and component)")}}
 
     # fps: the sampling step that precedes radius / knn in a set-abstraction
     # layer; a quarter of every cloud, first row as start
@@ -322,21 +386,24 @@ class Cases:
         nx, ny = lidar8["x"].to(self.dev), lidar8["y"].to(self.dev)
         nbx = lidar8["batch_x"].to(self.dev)
         nby = lidar8["batch_y"].to(self.dev)
+        N, M = x.shape[0], y.shape[0]
         cases = (("configs[4] ragged LiDAR-like knn k=16",
                   lambda: pca.knn(x, y, 16, bx, by, batch_size=8),
-                  y.shape[0]),
+                  M, _search_bytes(N, M, 3, 16)),
                  ("knn 1000000 uniform points onto themselves k=16",
-                  lambda: pca.knn(big, big, 16), big.shape[0]),
+                  lambda: pca.knn(big, big, 16), big.shape[0],
+                  _search_bytes(big.shape[0], big.shape[0], 3, 16)),
                  ("configs[2] radius_graph 8x16384 r=0.05 max 32",
                   lambda: pca.radius_graph(x3, 0.05, b3, max_num_neighbors=32,
-                                           batch_size=8), x3.shape[0]),
+                                           batch_size=8), x3.shape[0], None),
                  ("radius 1000000 uniform points onto themselves r=0.01 "
                   "max 32",
                   lambda: pca.radius(big, big, 0.01, max_num_neighbors=32),
-                  big.shape[0]),
+                  big.shape[0], None),
                  ("nearest on the LiDAR-like points",
-                  lambda: pca.nearest(nx, ny, nbx, nby), nx.shape[0]))
-        for name, fn, queries in cases:
+                  lambda: pca.nearest(nx, ny, nbx, nby), nx.shape[0],
+                  (nx.shape[0] + ny.shape[0]) * 12 + nx.shape[0] * 8))
+        for name, fn, queries, nbytes in cases:
             for strategy in ("scan", "binned"):
                 pca.set_search_strategy(strategy)
                 try:
@@ -344,10 +411,21 @@ class Cases:
                     search_ms = _search_ms(t, self.capi, self.events, fn, 1)
                 finally:
                     pca.set_search_strategy("scan")
-                report["%s, strategy %s" % (name, strategy)] = {
+                entry = {
                     "ms": ms, "queries_per_s": queries / ms * 1e3,
                     "search_ms": search_ms,
                     "edges": int(out.shape[1]) if out.dim() == 2 else None}
+                if nbytes is None and strategy == "binned":
+                    # radius: the edge list actually written
+                    nbytes = (2 * queries * 12 + int(out.shape[1]) * 16)
+                if strategy == "binned":
+                    entry["roofline"] = _hbm_roofline(
+                        "binning passes + binned search kernel", search_ms,
+                        nbytes, "bytes a search has to move (points and "
+                        "queries once, the int64 edge list once) over the "
+                        "time from the first binning pass to the end of the "
+                        "search kernel, against the HBM peak")
+                report["%s, strategy %s" % (name, strategy)] = entry
         return report
 
 
@@ -534,6 +612,7 @@ def main():
         torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(data, ptr_x, ptr_y)
+        result["cpu_baseline"]["build"] = cpu_build_baseline(pca, data)
     print(json.dumps(result))
 
 

@@ -48,21 +48,27 @@ int feat_blocks(int d) {
 
 int feat_tile_rows(int d) { return feat_blocks(d) <= 9 ? 64 : 32; }
 
+// flagged queries the threshold scan can take
+int feat_redo_cap(int m) { return std::min(m, kFeatRedoCap); }
+
 size_t feat_pack_bytes(int n, int d) {
   const size_t units = 2 * (size_t)feat_blocks(d) + 1; // FeatShape::RSU
   return align256(sizeof(uint4) * units * ((size_t)n + feat_tile_rows(d)));
 }
 
-__global__ __launch_bounds__(kBlock) void feat_init_kernel(FeatGlobals *g,
-                                                           float *tau, int m) {
+__global__ __launch_bounds__(kBlock) void feat_init_kernel(
+    FeatGlobals *g, float *tau, int m, int *hit_count, int redo_cap) {
   const int i = blockIdx.x * kBlock + threadIdx.x;
   if (i < m)
     tau[i] = __builtin_inff();
+  if (i < redo_cap)
+    hit_count[i] = 0;
   if (i == 0) {
     g->max_bits = 0;
     g->odd_rows = 0;
     g->any_redo = 0;
-    g->pad = 0;
+    g->unresolved = 0;
+    g->queued = 0;
   }
 }
 
@@ -131,6 +137,63 @@ __global__ __launch_bounds__(kBlock) void feat_rows_kernel(
   }
 }
 
+// The k smallest keys of a queued query's hit list (one wave per query); a
+// list that overflowed sends its query to the full second pass.
+__global__ __launch_bounds__(kBlock) void feat_redo_select_kernel(
+    KnnFeatParams p) {
+  constexpr int WAVES = kBlock / kWave;
+  constexpr int PER = kFeatHitCap / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int j = blockIdx.x * WAVES + threadIdx.x / kWave;
+  const int queued = min(p.globals->queued, p.redo_cap);
+  if (j >= queued)
+    return;
+  const int q = p.redo_list[j];
+  const int found = p.hit_count[j];
+  if (found > kFeatHitCap) {
+    if (lane == 0) {
+      p.redo_q[q] = 1;
+      atomicAdd(&p.globals->unresolved, 1);
+    }
+    return;
+  }
+  double keys[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int e = i * kWave + lane;
+    keys[i] = e < found ? p.hits[(size_t)j * kFeatHitCap + e] : empty_key();
+  }
+  const int k = p.k;
+  const size_t slot0 = (size_t)q * k;
+  int taken = 0;
+  for (; taken < k; ++taken) {
+    double mine = keys[0];
+#pragma unroll
+    for (int i = 1; i < PER; ++i)
+      mine = keys[i] < mine ? keys[i] : mine;
+    double least = mine;
+#pragma unroll
+    for (int sh = 32; sh >= 1; sh >>= 1) {
+      const double o = __shfl_xor(least, sh);
+      least = o < least ? o : least;
+    }
+    if (!(least < empty_key()))
+      break;
+    // (keys differ: rows differ)
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if (keys[i] == least)
+        keys[i] = empty_key();
+    if (lane == 0) {
+      p.out_idx[slot0 + taken] = key_row(least);
+      if (p.out_dist)
+        p.out_dist[slot0 + taken] = key_dist(least);
+    }
+  }
+  if (lane == 0)
+    p.out_count[q] = taken;
+}
+
 template <int KP>
 void launch_feat_merge(const KnnFeatParams &p, int tiles_bound,
                        hipStream_t stream) {
@@ -140,10 +203,12 @@ void launch_feat_merge(const KnnFeatParams &p, int tiles_bound,
 
 struct FeatLayout {
   size_t globals, x_norm, x_class, y_norm, tau, redo, plan256;
+  size_t redo_list, redo_tau, hit_count, hits; // threshold scan
   size_t pack, partial, cand; // first pass
   size_t second;              // second pass (reuses the first pass's bytes)
   size_t shared() const {
-    return globals + x_norm + x_class + y_norm + tau + redo + plan256;
+    return globals + x_norm + x_class + y_norm + tau + redo + plan256 +
+           redo_list + redo_tau + hit_count + hits;
   }
   size_t total() const {
     return shared() + std::max(pack + partial + cand, second);
@@ -188,6 +253,11 @@ static FeatLayout feat_layout(int n, int m, int d, int num_segments, int k) {
   w.tau = align256(sizeof(float) * (size_t)m);
   w.redo = align256(sizeof(int) * (size_t)m);
   w.plan256 = align256(sizeof(int) * ((size_t)num_segments + 1));
+  const size_t cap = (size_t)feat_redo_cap(m);
+  w.redo_list = align256(sizeof(int) * cap);
+  w.redo_tau = align256(sizeof(float) * cap);
+  w.hit_count = align256(sizeof(int) * cap);
+  w.hits = align256(sizeof(double) * cap * kFeatHitCap);
   w.pack = feat_pack_bytes(n, d);
   w.partial = align256(sizeof(double) * tiles * chunks * kk * kFeatQueries);
   w.cand = align256(sizeof(double) * (size_t)m * kk);
@@ -223,6 +293,11 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   float *tau = reinterpret_cast<float *>(take(lay.tau));
   int *redo_q = reinterpret_cast<int *>(take(lay.redo));
   int *plan256 = reinterpret_cast<int *>(take(lay.plan256));
+  int *redo_list = reinterpret_cast<int *>(take(lay.redo_list));
+  float *redo_tau = reinterpret_cast<float *>(take(lay.redo_tau));
+  int *hit_count = reinterpret_cast<int *>(take(lay.hit_count));
+  double *hits = reinterpret_cast<double *>(take(lay.hits));
+  const int redo_cap = feat_redo_cap(in.m);
   char *first_pass = base;
   uint4 *x_pack = reinterpret_cast<uint4 *>(take(lay.pack));
   double *partial = reinterpret_cast<double *>(take(lay.partial));
@@ -233,7 +308,8 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   const int nb = feat_blocks(in.d);
 
   hipLaunchKernelGGL(feat_init_kernel, dim3((in.m + kBlock - 1) / kBlock),
-                     dim3(kBlock), 0, stream, globals, tau, in.m);
+                     dim3(kBlock), 0, stream, globals, tau, in.m, hit_count,
+                     redo_cap);
   // squared norms that only classify the rows (NaN: a non-finite component);
   // for the Euclidean distance they also enter the filter
   float *x_class = cosine ? x_class_buf : x_norm;
@@ -307,6 +383,11 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   p.partial = partial;
   p.cand = cand;
   p.redo_q = redo_q;
+  p.redo_list = redo_list;
+  p.redo_tau = redo_tau;
+  p.hit_count = hit_count;
+  p.hits = hits;
+  p.redo_cap = redo_cap;
   p.out_idx = out.idx;
   p.out_dist = out.dist;
   p.out_count = out.count;
@@ -363,9 +444,27 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   if (err != hipSuccess)
     return err;
 
-  // Second pass for the flagged queries: the kernels are queued in any case
-  // and leave at once while nothing is flagged (no host read in between).
-  const int *gate = &globals->any_redo;
+  // The flagged queries: the kernels are queued in any case and leave at once
+  // while nothing is flagged (no host read in between).  First the scan that
+  // collects the rows at or below a query's k-th listed distance, then --
+  // only for what that scan could not take -- the full second pass.
+  {
+    const int waves = kBlock / kWave;
+    const int sgrid = redo_cap * (kFeatRedoSlices / waves);
+    if (cosine)
+      hipLaunchKernelGGL((feat_redo_scan_kernel<true>), dim3(sgrid),
+                         dim3(kBlock), 0, stream, p);
+    else
+      hipLaunchKernelGGL((feat_redo_scan_kernel<false>), dim3(sgrid),
+                         dim3(kBlock), 0, stream, p);
+    hipLaunchKernelGGL(feat_redo_select_kernel,
+                       dim3((redo_cap + waves - 1) / waves), dim3(kBlock), 0,
+                       stream, p);
+    err = hipGetLastError();
+    if (err != hipSuccess)
+      return err;
+  }
+  const int *gate = &globals->unresolved;
   if (in.d <= 128) {
     MfmaSecondPass second{gate, redo_q, x_norm, y_norm, kSecondPassChunks};
     return launch_knn_mfma(in, k, cosine, work_start, first_pass, out, nullptr,

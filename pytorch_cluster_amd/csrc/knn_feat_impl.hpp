@@ -73,6 +73,9 @@ constexpr int kFeatQueue = 8;     // parked rows per lane
 constexpr int kFeatSlack = 16;    // list entries beyond k
 constexpr int kFeatDrainEvery = 64;
 constexpr int kFeatRoundPeriod = 8; // tiles between scheduled rounds
+constexpr int kFeatRedoCap = 1024;  // flagged queries the threshold scan takes
+constexpr int kFeatHitCap = 256;    // rows it can hold per query
+constexpr int kFeatRedoSlices = 32; // waves that share a flagged query's rows
 
 typedef _Float16 feat_f16x8_t __attribute__((ext_vector_type(8)));
 typedef float feat_acc_t __attribute__((ext_vector_type(16)));
@@ -81,8 +84,10 @@ typedef float feat_acc_t __attribute__((ext_vector_type(16)));
 struct FeatGlobals {
   unsigned max_bits; // largest finite |component| of x and y (float bits)
   int odd_rows;      // rows of x the filter cannot represent
-  int any_redo;      // queries that must be searched again
-  int pad;
+  int any_redo;      // queries whose list could not be shown complete
+  int unresolved;    // ... of them, those left to the full second pass
+  int queued;        // ... and those queued for the threshold scan
+  int pad[3];
   // event counts of the filter kernel, written only by builds with
   // -DPCA_FEAT_STATS (steps, flagged steps, parked singles, lane-by-lane
   // values, drains, list rounds, direct steps, direct rounds)
@@ -226,7 +231,13 @@ struct KnnFeatParams {
   float *tau;            // [m] shared bounds U (scaled units, float bits)
   double *partial;       // [num_chunks * tiles][k + 16][128] keys
   double *cand;          // [m][k + 16] merged keys
-  int *redo_q;           // [m] 1: search this query again
+  int *redo_q;           // [m] 1: search this query again (full second pass)
+  // threshold scan of the flagged queries (feat_redo_scan_kernel)
+  int *redo_list;        // [redo_cap] queued queries
+  float *redo_tau;       // [redo_cap] their k-th distance among the listed rows
+  int *hit_count;        // [redo_cap] rows found at or below it
+  double *hits;          // [redo_cap][kFeatHitCap] their (distance, row) keys
+  int redo_cap;
   int *out_idx;
   float *out_dist;
   int *out_count;
@@ -955,11 +966,15 @@ __global__ __launch_bounds__(kBlock) void feat_refine_kernel(KnnFeatParams p) {
   const int kk = k + kFeatSlack;
   const int d = p.d;
   const size_t slot0 = (size_t)q * k;
+  // a query the filter cannot serve at all: left to the full second pass
+  auto unresolved = [&]() {
+    p.redo_q[q] = 1;
+    atomicAdd(&p.globals->any_redo, 1);
+    atomicAdd(&p.globals->unresolved, 1);
+  };
   if (p.globals->odd_rows != 0) {
-    if (lane == 0) {
-      p.redo_q[q] = 1;
-      atomicAdd(&p.globals->any_redo, 1);
-    }
+    if (lane == 0)
+      unresolved();
     return;
   }
   const float *yrow = p.y + (size_t)q * d;
@@ -970,9 +985,9 @@ __global__ __launch_bounds__(kBlock) void feat_refine_kernel(KnnFeatParams p) {
   if (fq.dead || fq.odd) {
     if (lane == 0) {
       p.out_count[q] = 0;
-      p.redo_q[q] = fq.odd ? 1 : 0;
+      p.redo_q[q] = 0;
       if (fq.odd)
-        atomicAdd(&p.globals->any_redo, 1);
+        unresolved();
     }
     return;
   }
@@ -1075,10 +1090,13 @@ __global__ __launch_bounds__(kBlock) void feat_refine_kernel(KnnFeatParams p) {
   }
   // is the list provably complete?  k-th exact distance found, scaled
   double kth = __builtin_inf();
+  float kth_plain = __builtin_inff();
   {
     const uint64_t who = __ballot(good && rank == k - 1);
-    if (who != 0)
-      kth = (double)__shfl(dist, __builtin_ctzll(who)) * scale2;
+    if (who != 0) {
+      kth_plain = __shfl(dist, __builtin_ctzll(who));
+      kth = (double)kth_plain * scale2;
+    }
   }
   // lower bound of every row outside the list: that of the list's last entry
   const double last_lower = __shfl(lower, kk - 1);
@@ -1087,9 +1105,152 @@ __global__ __launch_bounds__(kBlock) void feat_refine_kernel(KnnFeatParams p) {
   const bool complete = !full || last_lower > kth;
   if (lane == 0) {
     p.out_count[q] = good_count < k ? good_count : k;
-    p.redo_q[q] = complete ? 0 : 1;
-    if (!complete)
-      atomicAdd(&p.globals->any_redo, 1);
+    p.redo_q[q] = 0;
+    if (!complete) {
+      // The k nearest rows all lie at or below the k-th distance found among
+      // the listed ones: queue the query for the scan that collects exactly
+      // those rows; the full second pass takes what the queue cannot hold.
+      const int slot = kth_plain < kKnnSentinel
+                           ? atomicAdd(&p.globals->queued, 1)
+                           : p.redo_cap;
+      if (slot < p.redo_cap) {
+        p.redo_list[slot] = q;
+        p.redo_tau[slot] = kth_plain;
+        atomicAdd(&p.globals->any_redo, 1);
+      } else {
+        unresolved();
+      }
+    }
+  }
+}
+
+// Segment of query q: the last b with ptr[b] <= q (segments may be empty).
+__device__ __forceinline__ int feat_segment_of(const int64_t *__restrict__ ptr,
+                                               int num_segments, int q) {
+  int lo = 0, hi = num_segments;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (ptr[mid] <= (int64_t)q)
+      lo = mid;
+    else
+      hi = mid;
+  }
+  return lo;
+}
+
+// Threshold scan of the queued queries: one wave per (query, slice of its
+// segment's rows); a lane evaluates the exact distance of one row per step --
+// the reference's chain, one fused multiply-add per component in ascending
+// order (csrc/cuda/knn_cuda.cu:55-66) -- and rows at or below the query's
+// threshold are appended to its hit list.  Rows reach the lanes through LDS:
+// 64 rows x 32 components per step, read from global memory in full 128-byte
+// pieces; missing rows and components are zeros, which leave a chain as it is.
+template <bool COSINE>
+__global__ __launch_bounds__(kBlock) void feat_redo_scan_kernel(
+    KnnFeatParams p) {
+  constexpr int WAVES = kBlock / kWave;
+  constexpr int SLAB = 32;   // components per step
+  constexpr int STRIDE = 36; // floats per staged row: 16-byte reads of
+                             // neighbouring rows fall on distinct banks
+  __shared__ __attribute__((aligned(16))) float tile[WAVES][kWave][STRIDE];
+  __shared__ __attribute__((aligned(16))) float ys[WAVES][256];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  constexpr int GROUPS = kFeatRedoSlices / WAVES;
+  const int j = blockIdx.x / GROUPS;
+  const int slice = (blockIdx.x - j * GROUPS) * WAVES + wave;
+  const int queued = min(p.globals->queued, p.redo_cap);
+  if (j >= queued)
+    return;
+  const int q = p.redo_list[j];
+  const float tau = p.redo_tau[j];
+  const int d = p.d;
+  const int seg = p.ptr_y ? feat_segment_of(p.ptr_y, p.num_segments, q) : 0;
+  const int x_begin = p.ptr_x ? (int)p.ptr_x[seg] : 0;
+  const int x_end = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
+  const int seg_len = x_end - x_begin;
+  const int per_slice =
+      ((seg_len + kFeatRedoSlices - 1) / kFeatRedoSlices + kWave - 1) / kWave *
+      kWave;
+  const int r0 = min(x_end, x_begin + slice * per_slice);
+  const int r1 = min(x_end, r0 + per_slice);
+  if (r0 >= r1)
+    return;
+
+  const float *yrow = p.y + (size_t)q * d;
+  const int d_pad = (d + SLAB - 1) / SLAB * SLAB;
+  for (int c = lane; c < d_pad; c += kWave)
+    ys[wave][c] = c < d ? yrow[c] : 0.0f;
+  const float ynorm = COSINE ? p.y_norm[q] : 1.0f;
+  const bool vector_rows = (d & 3) == 0;
+
+  for (int base = r0; base < r1; base += kWave) {
+    float acc = 0.0f;
+    for (int c0 = 0; c0 < d; c0 += SLAB) {
+      // (the lanes of this wave alone use tile[wave])
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      if (vector_rows) {
+        const int part = (lane & 7) * 4;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int r = i * 8 + (lane >> 3);
+          float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+          if (base + r < r1 && c0 + part < d)
+            v = *reinterpret_cast<const float4 *>(
+                p.x + (size_t)(base + r) * d + c0 + part);
+          *reinterpret_cast<float4 *>(&tile[wave][r][part]) = v;
+        }
+      } else {
+        const int c = lane & 31;
+#pragma unroll 8
+        for (int i = 0; i < 32; ++i) {
+          const int r = i * 2 + (lane >> 5);
+          float v = 0.0f;
+          if (base + r < r1 && c0 + c < d)
+            v = p.x[(size_t)(base + r) * d + c0 + c];
+          tile[wave][r][c] = v;
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int g = 0; g < SLAB / 4; ++g) {
+        const float4 a = *reinterpret_cast<const float4 *>(&tile[wave][lane][4 * g]);
+        const float4 b = *reinterpret_cast<const float4 *>(&ys[wave][c0 + 4 * g]);
+        if (COSINE) {
+          acc = __builtin_fmaf(a.x, b.x, acc);
+          acc = __builtin_fmaf(a.y, b.y, acc);
+          acc = __builtin_fmaf(a.z, b.z, acc);
+          acc = __builtin_fmaf(a.w, b.w, acc);
+        } else {
+          const float d0 = a.x - b.x, d1 = a.y - b.y;
+          const float d2 = a.z - b.z, d3 = a.w - b.w;
+          acc = __builtin_fmaf(d0, d0, acc);
+          acc = __builtin_fmaf(d1, d1, acc);
+          acc = __builtin_fmaf(d2, d2, acc);
+          acc = __builtin_fmaf(d3, d3, acc);
+        }
+      }
+    }
+    const int row = base + lane;
+    if (COSINE) {
+      acc = acc / (p.x_norm[row < r1 ? row : r0] * ynorm);
+      acc = 1.0f - acc;
+    }
+    const bool hit = row < r1 && acc <= tau; // (false for NaN)
+    const uint64_t hits = __ballot(hit);
+    if (hits == 0)
+      continue;
+    int first = 0;
+    if (lane == 0)
+      first = atomicAdd(&p.hit_count[j], __builtin_popcountll(hits));
+    first = __shfl(first, 0);
+    const int at =
+        first + __builtin_popcountll(hits & ((1ull << lane) - 1ull));
+    if (hit && at < kFeatHitCap)
+      p.hits[(size_t)j * kFeatHitCap + at] = make_key(acc, (uint32_t)row);
   }
 }
 

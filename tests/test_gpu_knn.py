@@ -404,8 +404,11 @@ def test_operator_errors():
     with pytest.raises(RuntimeError, match="Input mismatch"):
         op(x, x, torch.tensor([0, 10], device=DEV),
            torch.tensor([0, 5, 10], device=DEV), 2, False, 1)
-    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
+    # x decides the branch (csrc/knn.cpp:26); the other tensors must follow it
+    with pytest.raises(RuntimeError, match="y must be CPU tensor"):
         op(x.cpu(), x, None, None, 2, False, 1)
+    with pytest.raises(RuntimeError, match="y must be CUDA tensor"):
+        op(x, x.cpu(), None, None, 2, False, 1)
 
 
 def test_runs_on_the_current_stream(oracle):

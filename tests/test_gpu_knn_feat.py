@@ -71,6 +71,44 @@ def test_near_duplicates_go_through_the_second_pass(oracle, d, cosine):
     _run(oracle, x2, y, None, None, 20, cosine)
 
 
+def _unresolved_queries(x, y, k, cosine=False):
+    """Flagged queries that the threshold scan could not settle (fourth word
+    of the per-call block, see _flagged_queries)."""
+    from gpu_common import dev
+    from pytorch_cluster_amd import capi
+    _e, _n, _d, ws = capi.knn_launch(dev(x), dev(y), None, None, k, cosine)
+    torch.cuda.synchronize()
+    off = (4 * x.shape[0] + 255) // 256 * 256
+    return ws[off:off + 16].cpu().view(torch.int32).tolist()[3]
+
+
+@pytest.mark.parametrize("d", [40, 160])
+def test_flagged_queries_beyond_what_the_threshold_scan_holds(oracle, d):
+    rng = np.random.default_rng(d + 5)
+    # (a) 400 exact copies of one row: more rows at the k-th distance than a
+    # hit list holds, the query goes on to the full second pass
+    centres = rng.standard_normal((6, d)).astype(np.float32)
+    x = np.concatenate([np.repeat(centres[:1], 400, axis=0),
+                        np.repeat(centres[1:], 40, axis=0),
+                        rng.standard_normal((500, d)).astype(np.float32)])
+    x = x[rng.permutation(len(x))]
+    y = np.concatenate([centres, rng.standard_normal((30, d)).astype(np.float32)])
+    assert _unresolved_queries(x, y, 8) >= 1
+    _run(oracle, x, y, None, None, 8)
+    _run(oracle, x, y, None, None, 8, cosine=True)
+    # (b) more flagged queries than the scan's queue takes (1,024)
+    centres = rng.standard_normal((30, d)).astype(np.float32)
+    x = np.repeat(centres, 40, axis=0)
+    x = x * (1.0 + 1e-7 * rng.standard_normal(x.shape)).astype(np.float32)
+    x = x.astype(np.float32)
+    y = np.repeat(centres, 50, axis=0)
+    odd, flagged = _flagged_queries(x, y, 6)
+    assert flagged > 1024 and _unresolved_queries(x, y, 6) >= flagged - 1024
+    ptr_x = np.array([0, 600, 1200])
+    ptr_y = np.array([0, 700, 1500])
+    _run(oracle, x, y, ptr_x, ptr_y, 6)
+
+
 def test_rows_and_queries_the_filter_cannot_represent(oracle):
     rng = np.random.default_rng(3)
     d = 40
