@@ -172,8 +172,8 @@ def _search_bytes(n, m, d, slots, elem=4):
 def _feat_shape(d, k):
     """(16-component blocks per row incl. the one that carries |x|^2, list
     width) of the feature-space kernel that serves (d, k)."""
-    blocks = next(b for b in (3, 5, 9, 17) if 16 * (b - 1) >= d)
-    width = next(w for w in (24, 32, 48, 64) if w >= k + 16)
+    blocks = next(b for b in (3, 5, 9, 17, 33) if 16 * (b - 1) >= d)
+    width = next(w for w in (24, 32, 48, 64, 80, 116) if w >= k + 16)
     return blocks, width
 
 
@@ -261,8 +261,8 @@ class Cases:
         ms, out = _median_ms(t, fn, reps or 3)
         kms = _search_ms(t, self.capi, self.events, fn)
         flop = 2 * d * n * m
-        if k > 48:
-            kernel = "knn_mfma_kernel" if d <= 128 else "knn_generic_kernel"
+        if d > 512:
+            kernel = "knn_generic_kernel"
             issued = None
         else:
             blocks, width = _feat_shape(d, k)

@@ -20,6 +20,7 @@ PCA_DECLARE_FEAT_BLOCKS(3)
 PCA_DECLARE_FEAT_BLOCKS(5)
 PCA_DECLARE_FEAT_BLOCKS(9)
 PCA_DECLARE_FEAT_BLOCKS(17)
+PCA_DECLARE_FEAT_BLOCKS(33)
 #undef PCA_DECLARE_FEAT_BLOCKS
 
 namespace {
@@ -28,7 +29,7 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 // list width for k neighbours: k + 16 real entries
 int feat_width(int k) {
-  static const int widths[] = {24, 32, 48, 64};
+  static const int widths[] = {24, 32, 48, 64, 80, 116};
   for (int w : widths)
     if (k + kFeatSlack <= w)
       return w;
@@ -43,13 +44,21 @@ int feat_blocks(int d) {
     return 5;
   if (d <= 128)
     return 9;
-  return 17;
+  if (d <= 256)
+    return 17;
+  return 33;
 }
 
 int feat_tile_rows(int d) { return feat_blocks(d) <= 9 ? 64 : 32; }
 
 // flagged queries the threshold scan can take
-int feat_redo_cap(int m) { return std::min(m, kFeatRedoCap); }
+int feat_redo_cap(int m) { return std::min(m, std::max(8192, m / 4)); }
+
+// rows the threshold scan holds per query: the k it looks for and the ones a
+// loose bound let through beside them
+int feat_hit_cap(int k) {
+  return std::min(kFeatMaxHits, (k + 60 + kWave - 1) / kWave * kWave);
+}
 
 size_t feat_pack_bytes(int n, int d) {
   const size_t units = 2 * (size_t)feat_blocks(d) + 1; // FeatShape::RSU
@@ -142,7 +151,7 @@ __global__ __launch_bounds__(kBlock) void feat_rows_kernel(
 __global__ __launch_bounds__(kBlock) void feat_redo_select_kernel(
     KnnFeatParams p) {
   constexpr int WAVES = kBlock / kWave;
-  constexpr int PER = kFeatHitCap / kWave;
+  constexpr int PER = kFeatMaxHits / kWave;
   const int lane = threadIdx.x & (kWave - 1);
   const int j = blockIdx.x * WAVES + threadIdx.x / kWave;
   const int queued = min(p.globals->queued, p.redo_cap);
@@ -150,7 +159,7 @@ __global__ __launch_bounds__(kBlock) void feat_redo_select_kernel(
     return;
   const int q = p.redo_list[j];
   const int found = p.hit_count[j];
-  if (found > kFeatHitCap) {
+  if (found > p.hit_cap) {
     if (lane == 0) {
       p.redo_q[q] = 1;
       atomicAdd(&p.globals->unresolved, 1);
@@ -161,7 +170,7 @@ __global__ __launch_bounds__(kBlock) void feat_redo_select_kernel(
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int e = i * kWave + lane;
-    keys[i] = e < found ? p.hits[(size_t)j * kFeatHitCap + e] : empty_key();
+    keys[i] = e < found ? p.hits[(size_t)j * p.hit_cap + e] : empty_key();
   }
   const int k = p.k;
   const size_t slot0 = (size_t)q * k;
@@ -225,7 +234,7 @@ bool knn_feat_supported(int d, int k, bool cosine) {
     if (env[0] == '0')
       return false;
   (void)cosine;
-  return d > 8 && d <= 256 && k >= 1 && feat_width(k) != 0;
+  return d > 8 && d <= kFeatMaxDim && k >= 1 && feat_width(k) != 0;
 }
 
 int knn_feat_slices(int n, int m, int d, int num_segments) {
@@ -239,6 +248,12 @@ int knn_feat_slices(int n, int m, int d, int num_segments) {
       chunks = v;
   }
   return chunks;
+}
+
+// the full second pass: the exact matrix-core kernel where it applies, else
+// the any-dimension kernel
+static bool second_pass_on_matrix_cores(int d, int k) {
+  return d <= 128 && k <= 64;
 }
 
 static FeatLayout feat_layout(int n, int m, int d, int num_segments, int k) {
@@ -257,11 +272,12 @@ static FeatLayout feat_layout(int n, int m, int d, int num_segments, int k) {
   w.redo_list = align256(sizeof(int) * cap);
   w.redo_tau = align256(sizeof(float) * cap);
   w.hit_count = align256(sizeof(int) * cap);
-  w.hits = align256(sizeof(double) * cap * kFeatHitCap);
+  w.hits = align256(sizeof(double) * cap * feat_hit_cap(k));
   w.pack = feat_pack_bytes(n, d);
   w.partial = align256(sizeof(double) * tiles * chunks * kk * kFeatQueries);
   w.cand = align256(sizeof(double) * (size_t)m * kk);
-  w.second = d <= 128 ? knn_mfma_scratch_bytes(n, m, d, num_segments, k,
+  w.second = second_pass_on_matrix_cores(d, k)
+                 ? knn_mfma_scratch_bytes(n, m, d, num_segments, k,
                                                kSecondPassChunks)
                       : 0;
   return w;
@@ -348,8 +364,12 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
       perr = launch_feat_pack<9>(xf, x_norm, x_class, in.n, in.d, cosine,
                                  globals, x_pack, stream);
       break;
-    default:
+    case 17:
       perr = launch_feat_pack<17>(xf, x_norm, x_class, in.n, in.d, cosine,
+                                  globals, x_pack, stream);
+      break;
+    default:
+      perr = launch_feat_pack<33>(xf, x_norm, x_class, in.n, in.d, cosine,
                                   globals, x_pack, stream);
       break;
     }
@@ -388,6 +408,7 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   p.hit_count = hit_count;
   p.hits = hits;
   p.redo_cap = redo_cap;
+  p.hit_cap = feat_hit_cap(k);
   p.out_idx = out.idx;
   p.out_dist = out.dist;
   p.out_count = out.count;
@@ -407,8 +428,11 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   case 9:
     err = launch_knn_feat_blocks<9>(p, kp, cosine, grid, stream);
     break;
-  default:
+  case 17:
     err = launch_knn_feat_blocks<17>(p, kp, cosine, grid, stream);
+    break;
+  default:
+    err = launch_knn_feat_blocks<33>(p, kp, cosine, grid, stream);
     break;
   }
   if (time_stop)
@@ -426,8 +450,14 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   case 48:
     launch_feat_merge<48>(p, tiles_bound, stream);
     break;
-  default:
+  case 64:
     launch_feat_merge<64>(p, tiles_bound, stream);
+    break;
+  case 80:
+    launch_feat_merge<80>(p, tiles_bound, stream);
+    break;
+  default:
+    launch_feat_merge<116>(p, tiles_bound, stream);
     break;
   }
   {
@@ -450,7 +480,8 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   // only for what that scan could not take -- the full second pass.
   {
     const int waves = kBlock / kWave;
-    const int sgrid = redo_cap * (kFeatRedoSlices / waves);
+    const int sgrid =
+        (redo_cap + kFeatRedoGroup - 1) / kFeatRedoGroup * kFeatRedoSlices;
     if (cosine)
       hipLaunchKernelGGL((feat_redo_scan_kernel<true>), dim3(sgrid),
                          dim3(kBlock), 0, stream, p);
@@ -465,7 +496,7 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
       return err;
   }
   const int *gate = &globals->unresolved;
-  if (in.d <= 128) {
+  if (second_pass_on_matrix_cores(in.d, k)) {
     MfmaSecondPass second{gate, redo_q, x_norm, y_norm, kSecondPassChunks};
     return launch_knn_mfma(in, k, cosine, work_start, first_pass, out, nullptr,
                            nullptr, stream, nullptr, &second);

@@ -73,9 +73,10 @@ constexpr int kFeatQueue = 8;     // parked rows per lane
 constexpr int kFeatSlack = 16;    // list entries beyond k
 constexpr int kFeatDrainEvery = 64;
 constexpr int kFeatRoundPeriod = 8; // tiles between scheduled rounds
-constexpr int kFeatRedoCap = 1024;  // flagged queries the threshold scan takes
-constexpr int kFeatHitCap = 256;    // rows it can hold per query
-constexpr int kFeatRedoSlices = 32; // waves that share a flagged query's rows
+constexpr int kFeatMaxDim = 512;    // components this path takes
+constexpr int kFeatRedoGroup = 32;  // queued queries per workgroup of the scan
+constexpr int kFeatMaxHits = 256;   // most rows the scan holds per query
+constexpr int kFeatRedoSlices = 32; // workgroups that share a group's rows
 
 typedef _Float16 feat_f16x8_t __attribute__((ext_vector_type(8)));
 typedef float feat_acc_t __attribute__((ext_vector_type(16)));
@@ -95,10 +96,19 @@ struct FeatGlobals {
 };
 
 // ---- constants of the error analysis (see the header) ----------------------
-constexpr double kFeatRho = 1.0 / 512.0;
-constexpr double kFeatGrow = 1.0 + 4.1 / 512.0;
+// rho: 2^-9 up to 256 components, 2^-8 beyond (the accumulation error of the
+// longer chains no longer fits under 2^-9)
+__host__ __device__ __forceinline__ double feat_rho(int d) {
+  return d <= 256 ? 1.0 / 512.0 : 1.0 / 256.0;
+}
+__host__ __device__ __forceinline__ double feat_grow(int d) {
+  return 1.0 + 4.1 * feat_rho(d);
+}
 constexpr double kFeatCosScale = 1048576.0; // 2^20
-constexpr double kFeatCosErr = 2048.0;      // 2^-9 x 2^20
+// Ec = rho x 2^20
+__host__ __device__ __forceinline__ double feat_cos_err(int d) {
+  return feat_rho(d) * kFeatCosScale;
+}
 constexpr float kFeatCosTiny = 1e-18f;      // smallest norm the cosine filter takes
 
 __host__ __device__ __forceinline__ double feat_c0(int d) {
@@ -185,8 +195,8 @@ __device__ __forceinline__ FeatQuery feat_query(const float *yrow, int d,
     // for the margin Ec)
     fq.odd = !fq.dead &&
              !(norm_in < __builtin_inff() && norm_in >= kFeatCosTiny);
-    fq.shift = -kFeatCosErr;
-    fq.widen = 2.0 * kFeatCosErr;
+    fq.shift = -feat_cos_err(d);
+    fq.widen = 2.0 * feat_cos_err(d);
     fq.grow = 1.0;
     return fq;
   }
@@ -204,9 +214,9 @@ __device__ __forceinline__ FeatQuery feat_query(const float *yrow, int d,
   const double c0 =
       feat_c0(d) + (double)d * 1.4012984643248171e-45 * (double)inv_sigma *
                        (double)inv_sigma;
-  fq.shift = ysq * (1.0 - kFeatRho) - c0;
-  fq.widen = 6.0 * kFeatRho * ysq + 2.0 * c0;
-  fq.grow = kFeatGrow;
+  fq.shift = ysq * (1.0 - feat_rho(d)) - c0;
+  fq.widen = 6.0 * feat_rho(d) * ysq + 2.0 * c0;
+  fq.grow = feat_grow(d);
   return fq;
 }
 
@@ -236,8 +246,9 @@ struct KnnFeatParams {
   int *redo_list;        // [redo_cap] queued queries
   float *redo_tau;       // [redo_cap] their k-th distance among the listed rows
   int *hit_count;        // [redo_cap] rows found at or below it
-  double *hits;          // [redo_cap][kFeatHitCap] their (distance, row) keys
+  double *hits;          // [redo_cap][hit_cap] their (distance, row) keys
   int redo_cap;
+  int hit_cap;
   int *out_idx;
   float *out_dist;
   int *out_count;
@@ -251,7 +262,16 @@ template <int NB> struct FeatShape {
   static constexpr int RSU = UNITS + 1;
   static constexpr int MAX_D = 16 * (NB - 1);
   static constexpr int TILE = NB <= 9 ? 64 : 32; // rows per LDS tile
+  // LDS buffers the tiles rotate through (160 KB per CU)
+  static constexpr int RING = 3;
 };
+
+// Workgroups per CU the filter kernel is compiled for: two (256 registers per
+// lane) while the query operands (4 NB registers) and the list (KP registers)
+// leave room for the rest, one (512 registers) beyond.
+constexpr int feat_resident_groups(int nb, int kp) {
+  return (nb > 17 || kp > 64) ? 1 : 2;
+}
 
 // ---- preparation ------------------------------------------------------------
 
@@ -311,7 +331,7 @@ __global__ __launch_bounds__(kBlock) void feat_pack_kernel(
           w = kFeatCosScale;
         } else {
           const double inv = (double)scale;
-          w = (double)nv * inv * inv * (1.0 - kFeatRho);
+          w = (double)nv * inv * inv * (1.0 - feat_rho(d));
         }
         const uint32_t a1 = feat_h_down(w * (1.0 / 32768.0));
         const double r1 = w - feat_h_value(a1) * 32768.0;
@@ -370,7 +390,8 @@ __device__ __forceinline__ float feat_pick(const feat_acc_t (&a)[SUBS], int v) {
 // own key), so the upper half may lag by one key -- its entries are then too
 // large, never too small, which keeps every bound read from it valid.
 template <int NB, int KP, bool COSINE>
-__global__ __launch_bounds__(kBlock, 2) void knn_feat_kernel(KnnFeatParams p) {
+__global__ __launch_bounds__(kBlock, feat_resident_groups(NB, KP)) void
+knn_feat_kernel(KnnFeatParams p) {
   typedef FeatShape<NB> S;
   constexpr int RSU = S::RSU;
   constexpr int TILE = S::TILE;
@@ -378,7 +399,7 @@ __global__ __launch_bounds__(kBlock, 2) void knn_feat_kernel(KnnFeatParams p) {
   constexpr int TILE_UNITS = TILE * RSU;
   constexpr int PIECES = (TILE_UNITS + kWave - 1) / kWave;
   constexpr int MAX_PIECES_PER_WAVE = (PIECES + 3) / 4;
-  constexpr int RING = 3;
+  constexpr int RING = S::RING;
   constexpr int QCAP = kFeatQueue;
   static_assert((QCAP & (QCAP - 1)) == 0, "the queue is a ring");
   constexpr int TQ = kFeatQueries;
@@ -576,15 +597,12 @@ __global__ __launch_bounds__(kBlock, 2) void knn_feat_kernel(KnnFeatParams p) {
     request_tile(0);
   if (num_tiles > 1)
     request_tile(1);
-  if (num_tiles > 2)
+  if (RING > 2 && num_tiles > 2)
     request_tile(2);
   update_bound(false); // what other slices already know
   if (num_tiles > 0) {
     await_tile(num_tiles > 1); // (tiles 1 and 2 count as one newer tile here:
                                // at worst the wait is longer than needed)
-    if (num_tiles > 2)
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * MAX_PIECES_PER_WAVE - 1)
-                   : "memory");
   }
 
   // One pass per tile, software-pipelined: pass t issues the chains of matrix
@@ -617,8 +635,8 @@ __global__ __launch_bounds__(kBlock, 2) void knn_feat_kernel(KnnFeatParams p) {
       // previous pass); after the barrier so have everybody's, and everybody
       // is done with tile t - 1
       __syncthreads();
-      if (t >= 1 && t + 2 < num_tiles)
-        request_tile(t + 2); // into the buffer of tile t - 1
+      if (t >= 1 && t + RING - 1 < num_tiles)
+        request_tile(t + RING - 1); // into the buffer of tile t - 1
       // the tile's SUBS * NB operands, read AHEAD operands before they are
       // used (LDS latency is several matrix instructions long); pass
       // num_tiles has no tile: it computes on what the buffer holds and
@@ -686,7 +704,7 @@ __global__ __launch_bounds__(kBlock, 2) void knn_feat_kernel(KnnFeatParams p) {
       // the next tile's pieces of this wave, so that the next pass starts with
       // the barrier
       if (t + 1 < num_tiles)
-        await_tile(t + 2 < num_tiles);
+        await_tile(RING > 2 && t + 2 < num_tiles);
       // (consumed inside the branch, so that the wait for it stays there)
       if ((t & 63) == 63) {
         const float now = __hip_atomic_load(&p.tau[valid ? q : y_begin],
@@ -956,7 +974,7 @@ __global__ __launch_bounds__(kBlock) void feat_merge_kernel(KnnFeatParams p) {
 template <bool COSINE>
 __global__ __launch_bounds__(kBlock) void feat_refine_kernel(KnnFeatParams p) {
   constexpr int WAVES = kBlock / kWave;
-  __shared__ __attribute__((aligned(16))) float ys[WAVES][256];
+  __shared__ __attribute__((aligned(16))) float ys[WAVES][kFeatMaxDim];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int q = blockIdx.x * WAVES + wave;
@@ -999,12 +1017,22 @@ __global__ __launch_bounds__(kBlock) void feat_refine_kernel(KnnFeatParams p) {
 
   const double scale2 =
       COSINE ? kFeatCosScale : (double)inv_sigma * (double)inv_sigma;
-  const double key = lane < kk ? p.cand[(size_t)q * kk + lane]
-                               : feat_empty_key();
-  const bool listed = key < feat_empty_key();
-  const int row = key_row(key);
-  const double lower = (double)key_dist(key) + fq.shift; // l of the row
-  const int listed_count = __builtin_popcountll(__ballot(listed));
+  // a lane looks after the list entries lane and lane + 64 (lists of up to
+  // 116 entries)
+  constexpr int PER = 2;
+  double key[PER], lower[PER];
+  bool listed[PER];
+  int row[PER];
+  int listed_count = 0;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int c = lane + kWave * i;
+    key[i] = c < kk ? p.cand[(size_t)q * kk + c] : feat_empty_key();
+    listed[i] = key[i] < feat_empty_key();
+    row[i] = key_row(key[i]);
+    lower[i] = (double)key_dist(key[i]) + fq.shift; // l of the row
+    listed_count += __builtin_popcountll(__ballot(listed[i]));
+  }
 
   auto exact = [&](int g) {
     const float *xr = p.x + (size_t)g * d;
@@ -1049,19 +1077,30 @@ __global__ __launch_bounds__(kBlock) void feat_refine_kernel(KnnFeatParams p) {
 
   // the first k listed rows, then those whose lower bound does not exceed
   // the largest distance found among them
-  float dist = __builtin_nanf("");
-  bool done = false;
-  if (listed && lane < k) {
-    dist = exact(row);
-    done = true;
-  }
+  float dist[PER];
+  bool done[PER];
   auto usable = [&](float v) { return v < kKnnSentinel; }; // (false for NaN)
+  int first_good = 0;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    dist[i] = __builtin_nanf("");
+    done[i] = false;
+    if (listed[i] && lane + kWave * i < k) {
+      dist[i] = exact(row[i]);
+      done[i] = true;
+    }
+    first_good += __builtin_popcountll(__ballot(done[i] && usable(dist[i])));
+  }
   {
-    const uint64_t good = __ballot(done && usable(dist));
     double reach = __builtin_inf(); // scaled distance rows must stay below
-    if (__builtin_popcountll(good) >= k) {
+    if (first_good >= k) {
       // the k-th smallest of k values is their largest
-      double mine = done ? (double)dist * scale2 : 0.0;
+      double mine = 0.0;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const double v = done[i] ? (double)dist[i] * scale2 : 0.0;
+        mine = v > mine ? v : mine;
+      }
 #pragma unroll
       for (int sh = 32; sh >= 1; sh >>= 1) {
         const double o = __shfl_xor(mine, sh);
@@ -1069,37 +1108,53 @@ __global__ __launch_bounds__(kBlock) void feat_refine_kernel(KnnFeatParams p) {
       }
       reach = mine;
     }
-    if (listed && !done && lower <= reach) {
-      dist = exact(row);
-      done = true;
-    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if (listed[i] && !done[i] && lower[i] <= reach) {
+        dist[i] = exact(row[i]);
+        done[i] = true;
+      }
   }
-  const bool good = done && usable(dist);
-  const double ekey = good ? make_key(dist, (uint32_t)row) : empty_key();
+  bool good[PER];
+  double ekey[PER];
+  int good_count = 0;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    good[i] = done[i] && usable(dist[i]);
+    ekey[i] = good[i] ? make_key(dist[i], (uint32_t)row[i]) : empty_key();
+    good_count += __builtin_popcountll(__ballot(good[i]));
+  }
   // rank among the evaluated rows (keys differ: rows differ)
-  int rank = 0;
+  int rank[PER] = {0, 0};
+  const bool second_half = kk > kWave; // (uniform)
   for (int j = 0; j < kWave; ++j) {
-    const double other = __shfl(ekey, j);
-    rank += other < ekey ? 1 : 0;
-  }
-  const int good_count = __builtin_popcountll(__ballot(good));
-  if (good && rank < k) {
-    p.out_idx[slot0 + rank] = row;
-    if (p.out_dist)
-      p.out_dist[slot0 + rank] = dist;
+    const double o0 = __shfl(ekey[0], j);
+    rank[0] += o0 < ekey[0] ? 1 : 0;
+    if (second_half) {
+      const double o1 = __shfl(ekey[1], j);
+      rank[0] += o1 < ekey[0] ? 1 : 0;
+      rank[1] += (o0 < ekey[1] ? 1 : 0) + (o1 < ekey[1] ? 1 : 0);
+    }
   }
   // is the list provably complete?  k-th exact distance found, scaled
   double kth = __builtin_inf();
   float kth_plain = __builtin_inff();
-  {
-    const uint64_t who = __ballot(good && rank == k - 1);
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    if (good[i] && rank[i] < k) {
+      p.out_idx[slot0 + rank[i]] = row[i];
+      if (p.out_dist)
+        p.out_dist[slot0 + rank[i]] = dist[i];
+    }
+    const uint64_t who = __ballot(good[i] && rank[i] == k - 1);
     if (who != 0) {
-      kth_plain = __shfl(dist, __builtin_ctzll(who));
+      kth_plain = __shfl(dist[i], __builtin_ctzll(who));
       kth = (double)kth_plain * scale2;
     }
   }
   // lower bound of every row outside the list: that of the list's last entry
-  const double last_lower = __shfl(lower, kk - 1);
+  const double last_lower = kk > kWave ? __shfl(lower[1], kk - 1 - kWave)
+                                       : __shfl(lower[0], kk - 1);
   const bool full = listed_count == kk;
   // rows that were listed but not evaluated have lower > reach >= kth
   const bool complete = !full || last_lower > kth;
@@ -1138,119 +1193,182 @@ __device__ __forceinline__ int feat_segment_of(const int64_t *__restrict__ ptr,
   return lo;
 }
 
-// Threshold scan of the queued queries: one wave per (query, slice of its
-// segment's rows); a lane evaluates the exact distance of one row per step --
-// the reference's chain, one fused multiply-add per component in ascending
-// order (csrc/cuda/knn_cuda.cu:55-66) -- and rows at or below the query's
-// threshold are appended to its hit list.  Rows reach the lanes through LDS:
-// 64 rows x 32 components per step, read from global memory in full 128-byte
-// pieces; missing rows and components are zeros, which leave a chain as it is.
+// Threshold scan of the queued queries.  A workgroup takes 32 of them (8 per
+// wave) and one slice of their segment's rows; a lane evaluates the exact
+// distance of one row per step against each of its wave's queries -- the
+// reference's chain, one fused multiply-add per component in ascending order
+// (csrc/cuda/knn_cuda.cu:55-66) -- and rows at or below a query's threshold
+// are appended to that query's hit list.  Rows and query components reach the
+// lanes through LDS, 64 rows x 32 components per step, read from global
+// memory in full 128-byte pieces; missing rows and components are zeros,
+// which leave a chain as it is.  Queries of different segments in one group
+// are served one segment after the other.
 template <bool COSINE>
 __global__ __launch_bounds__(kBlock) void feat_redo_scan_kernel(
     KnnFeatParams p) {
-  constexpr int WAVES = kBlock / kWave;
   constexpr int SLAB = 32;   // components per step
   constexpr int STRIDE = 36; // floats per staged row: 16-byte reads of
                              // neighbouring rows fall on distinct banks
-  __shared__ __attribute__((aligned(16))) float tile[WAVES][kWave][STRIDE];
-  __shared__ __attribute__((aligned(16))) float ys[WAVES][256];
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
-  constexpr int GROUPS = kFeatRedoSlices / WAVES;
-  const int j = blockIdx.x / GROUPS;
-  const int slice = (blockIdx.x - j * GROUPS) * WAVES + wave;
+  constexpr int G = kFeatRedoGroup;
+  constexpr int Q = G / (kBlock / kWave);
+  __shared__ __attribute__((aligned(16))) float tile[kWave][STRIDE];
+  __shared__ __attribute__((aligned(16))) float ysl[G][SLAB];
+  __shared__ int s_q[G], s_xb[G], s_xe[G];
+  __shared__ float s_tau[G], s_yn[G];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int group = blockIdx.x / kFeatRedoSlices;
+  const int slice = blockIdx.x - group * kFeatRedoSlices;
   const int queued = min(p.globals->queued, p.redo_cap);
-  if (j >= queued)
+  if (group * G >= queued)
     return;
-  const int q = p.redo_list[j];
-  const float tau = p.redo_tau[j];
   const int d = p.d;
-  const int seg = p.ptr_y ? feat_segment_of(p.ptr_y, p.num_segments, q) : 0;
-  const int x_begin = p.ptr_x ? (int)p.ptr_x[seg] : 0;
-  const int x_end = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
-  const int seg_len = x_end - x_begin;
-  const int per_slice =
-      ((seg_len + kFeatRedoSlices - 1) / kFeatRedoSlices + kWave - 1) / kWave *
-      kWave;
-  const int r0 = min(x_end, x_begin + slice * per_slice);
-  const int r1 = min(x_end, r0 + per_slice);
-  if (r0 >= r1)
-    return;
-
-  const float *yrow = p.y + (size_t)q * d;
-  const int d_pad = (d + SLAB - 1) / SLAB * SLAB;
-  for (int c = lane; c < d_pad; c += kWave)
-    ys[wave][c] = c < d ? yrow[c] : 0.0f;
-  const float ynorm = COSINE ? p.y_norm[q] : 1.0f;
+  if (tid < G) {
+    const int j = group * G + tid;
+    int q = -1, xb = 0, xe = 0;
+    float tau = -__builtin_inff(), yn = 1.0f;
+    if (j < queued) {
+      q = p.redo_list[j];
+      tau = p.redo_tau[j];
+      const int seg = p.ptr_y ? feat_segment_of(p.ptr_y, p.num_segments, q) : 0;
+      xb = p.ptr_x ? (int)p.ptr_x[seg] : 0;
+      xe = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
+      if (COSINE)
+        yn = p.y_norm[q];
+    }
+    s_q[tid] = q;
+    s_xb[tid] = xb;
+    s_xe[tid] = xe;
+    s_tau[tid] = tau;
+    s_yn[tid] = yn;
+  }
+  __syncthreads();
   const bool vector_rows = (d & 3) == 0;
 
-  for (int base = r0; base < r1; base += kWave) {
-    float acc = 0.0f;
-    for (int c0 = 0; c0 < d; c0 += SLAB) {
-      // (the lanes of this wave alone use tile[wave])
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      if (vector_rows) {
-        const int part = (lane & 7) * 4;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int r = i * 8 + (lane >> 3);
-          float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-          if (base + r < r1 && c0 + part < d)
-            v = *reinterpret_cast<const float4 *>(
-                p.x + (size_t)(base + r) * d + c0 + part);
-          *reinterpret_cast<float4 *>(&tile[wave][r][part]) = v;
-        }
-      } else {
-        const int c = lane & 31;
-#pragma unroll 8
-        for (int i = 0; i < 32; ++i) {
-          const int r = i * 2 + (lane >> 5);
-          float v = 0.0f;
-          if (base + r < r1 && c0 + c < d)
-            v = p.x[(size_t)(base + r) * d + c0 + c];
-          tile[wave][r][c] = v;
-        }
-      }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-      for (int g = 0; g < SLAB / 4; ++g) {
-        const float4 a = *reinterpret_cast<const float4 *>(&tile[wave][lane][4 * g]);
-        const float4 b = *reinterpret_cast<const float4 *>(&ys[wave][c0 + 4 * g]);
-        if (COSINE) {
-          acc = __builtin_fmaf(a.x, b.x, acc);
-          acc = __builtin_fmaf(a.y, b.y, acc);
-          acc = __builtin_fmaf(a.z, b.z, acc);
-          acc = __builtin_fmaf(a.w, b.w, acc);
-        } else {
-          const float d0 = a.x - b.x, d1 = a.y - b.y;
-          const float d2 = a.z - b.z, d3 = a.w - b.w;
-          acc = __builtin_fmaf(d0, d0, acc);
-          acc = __builtin_fmaf(d1, d1, acc);
-          acc = __builtin_fmaf(d2, d2, acc);
-          acc = __builtin_fmaf(d3, d3, acc);
-        }
-      }
-    }
-    const int row = base + lane;
-    if (COSINE) {
-      acc = acc / (p.x_norm[row < r1 ? row : r0] * ynorm);
-      acc = 1.0f - acc;
-    }
-    const bool hit = row < r1 && acc <= tau; // (false for NaN)
-    const uint64_t hits = __ballot(hit);
-    if (hits == 0)
+  // (everything that decides about a barrier below is the same in all lanes
+  // of the workgroup)
+  for (int lead = 0; lead < G; ++lead) {
+    if (s_q[lead] < 0)
       continue;
-    int first = 0;
-    if (lane == 0)
-      first = atomicAdd(&p.hit_count[j], __builtin_popcountll(hits));
-    first = __shfl(first, 0);
-    const int at =
-        first + __builtin_popcountll(hits & ((1ull << lane) - 1ull));
-    if (hit && at < kFeatHitCap)
-      p.hits[(size_t)j * kFeatHitCap + at] = make_key(acc, (uint32_t)row);
+    const int xb = s_xb[lead], xe = s_xe[lead];
+    bool seen = false;
+    for (int e = 0; e < lead; ++e)
+      seen |= s_q[e] >= 0 && s_xb[e] == xb && s_xe[e] == xe;
+    if (seen)
+      continue; // served together with an earlier query of the segment
+    const int per_slice =
+        ((xe - xb + kFeatRedoSlices - 1) / kFeatRedoSlices + kWave - 1) /
+        kWave * kWave;
+    const int r0 = min(xe, xb + slice * per_slice);
+    const int r1 = min(xe, r0 + per_slice);
+    if (r0 >= r1)
+      continue;
+    bool act[Q];
+#pragma unroll
+    for (int i = 0; i < Q; ++i) {
+      const int e = wave * Q + i;
+      act[i] = s_q[e] >= 0 && s_xb[e] == xb && s_xe[e] == xe;
+    }
+
+    for (int base = r0; base < r1; base += kWave) {
+      float acc[Q];
+#pragma unroll
+      for (int i = 0; i < Q; ++i)
+        acc[i] = 0.0f;
+      for (int c0 = 0; c0 < d; c0 += SLAB) {
+        __syncthreads(); // the previous step's tile has been read
+        if (vector_rows) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const int idx = tid + kBlock * i;
+            const int r = idx >> 3, part = (idx & 7) * 4;
+            float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (base + r < r1 && c0 + part < d)
+              v = *reinterpret_cast<const float4 *>(
+                  p.x + (size_t)(base + r) * d + c0 + part);
+            *reinterpret_cast<float4 *>(&tile[r][part]) = v;
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const int idx = tid + kBlock * i;
+            const int r = idx >> 5, c = idx & 31;
+            float v = 0.0f;
+            if (base + r < r1 && c0 + c < d)
+              v = p.x[(size_t)(base + r) * d + c0 + c];
+            tile[r][c] = v;
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < G * SLAB / kBlock; ++i) {
+          const int idx = tid + kBlock * i;
+          const int e = idx >> 5, c = idx & 31;
+          const int q = s_q[e];
+          float v = 0.0f;
+          if (q >= 0 && c0 + c < d)
+            v = p.y[(size_t)q * d + c0 + c];
+          ysl[e][c] = v;
+        }
+        __syncthreads();
+        float4 xr[SLAB / 4];
+#pragma unroll
+        for (int g = 0; g < SLAB / 4; ++g)
+          xr[g] = *reinterpret_cast<const float4 *>(&tile[lane][4 * g]);
+#pragma unroll
+        for (int i = 0; i < Q; ++i) {
+          if (!act[i])
+            continue;
+#pragma unroll
+          for (int g = 0; g < SLAB / 4; ++g) {
+            const float4 a = xr[g];
+            const float4 b =
+                *reinterpret_cast<const float4 *>(&ysl[wave * Q + i][4 * g]);
+            float v = acc[i];
+            if (COSINE) {
+              v = __builtin_fmaf(a.x, b.x, v);
+              v = __builtin_fmaf(a.y, b.y, v);
+              v = __builtin_fmaf(a.z, b.z, v);
+              v = __builtin_fmaf(a.w, b.w, v);
+            } else {
+              const float d0 = a.x - b.x, d1 = a.y - b.y;
+              const float d2 = a.z - b.z, d3 = a.w - b.w;
+              v = __builtin_fmaf(d0, d0, v);
+              v = __builtin_fmaf(d1, d1, v);
+              v = __builtin_fmaf(d2, d2, v);
+              v = __builtin_fmaf(d3, d3, v);
+            }
+            acc[i] = v;
+          }
+        }
+      }
+      const int row = base + lane;
+      const float xn = COSINE ? p.x_norm[row < r1 ? row : r0] : 1.0f;
+#pragma unroll
+      for (int i = 0; i < Q; ++i) {
+        if (!act[i])
+          continue;
+        const int e = wave * Q + i;
+        float dist = acc[i];
+        if (COSINE) {
+          dist = dist / (xn * s_yn[e]);
+          dist = 1.0f - dist;
+        }
+        const bool hit = row < r1 && dist <= s_tau[e]; // (false for NaN)
+        const uint64_t hits = __ballot(hit);
+        if (hits == 0)
+          continue;
+        const int j = group * G + e;
+        int first = 0;
+        if (lane == 0)
+          first = atomicAdd(&p.hit_count[j], __builtin_popcountll(hits));
+        first = __shfl(first, 0);
+        const int at =
+            first + __builtin_popcountll(hits & ((1ull << lane) - 1ull));
+        if (hit && at < p.hit_cap)
+          p.hits[(size_t)j * p.hit_cap + at] = make_key(dist, (uint32_t)row);
+      }
+    }
   }
 }
 
@@ -1291,6 +1409,12 @@ hipError_t launch_feat_pack(const float *x, const float *norms,
       break;                                                                   \
     case 64:                                                                   \
       launch_feat_one_##NB_<64>(p, cosine, grid, stream);                      \
+      break;                                                                   \
+    case 80:                                                                   \
+      launch_feat_one_##NB_<80>(p, cosine, grid, stream);                      \
+      break;                                                                   \
+    case 116:                                                                  \
+      launch_feat_one_##NB_<116>(p, cosine, grid, stream);                     \
       break;                                                                   \
     default:                                                                   \
       return hipErrorInvalidValue;                                             \

@@ -10,14 +10,15 @@ The model rounds exactly as the kernels do (numpy float16, the same flush and
 the same truncated parts of W) and sums the products in float64, i.e. without
 the matrix cores' own accumulation error; the test therefore demands that the
 roundings alone leave the share of the budget that the header of
-knn_feat_impl.hpp reserves for accumulation (0.15 x 2^-10 of |X|^2 + |Y|^2 at
-256 components) unused.
+knn_feat_impl.hpp reserves for accumulation (2^-22 x 2.01 of |X|^2 + |Y|^2 per
+term of the chain: 0.13 x 2^-10 at 256 components, 0.26 x 2^-10 at 512) unused.
 """
 import numpy as np
 import pytest
 
-RHO = 1.0 / 512.0
-GROW = 1.0 + 4.1 / 512.0
+def rho_of(d):
+    """2^-9 up to 256 components, 2^-8 beyond (feat_rho)."""
+    return 1.0 / 512.0 if d <= 256 else 1.0 / 256.0
 
 
 def inv_sigma(max_abs):
@@ -71,6 +72,8 @@ def check(x, y):
     x = np.ascontiguousarray(x, dtype=np.float32)
     y = np.ascontiguousarray(y, dtype=np.float32)
     d = x.shape[1]
+    RHO = rho_of(d)
+    GROW = 1.0 + 4.1 * RHO
     inv = inv_sigma(max(np.abs(x).max(), np.abs(y).max()))
     scale2 = inv * inv
     c0 = d / 4096.0 + d * 2.0 ** -149 * scale2
@@ -90,7 +93,8 @@ def check(x, y):
     upper = (lower + widen[:, None]) * GROW
     e = reference_distances(x, y) * scale2
     norms = (xs.astype(np.float64) ** 2).sum(1)[None, :] + ysq[:, None]
-    room = 0.15 * 2.0 ** -10 * norms  # what accumulation may still take
+    # what accumulation may still take (2^-22 x 2.01 per term of the chain)
+    room = max(0.15, (d + 16) * 2.01 / 4096.0) * 2.0 ** -10 * norms
     assert (lower + room <= e + 1e-300).all(), \
         "lower bound above the reference's distance"
     assert (e <= upper - room).all(), "upper bound below it"
@@ -108,7 +112,7 @@ def midpoint_rows(rng, n, d, exponents, side):
     return (frac * 2.0 ** exponents).astype(np.float32)
 
 
-@pytest.mark.parametrize("d", [9, 64, 128, 256])
+@pytest.mark.parametrize("d", [9, 64, 128, 256, 300, 512])
 def test_random_rows(d):
     rng = np.random.default_rng(d)
     x = rng.standard_normal((400, d))
@@ -117,7 +121,7 @@ def test_random_rows(d):
     check(x, x[:60])  # queries that are rows: distance zero
 
 
-@pytest.mark.parametrize("d", [16, 128, 256])
+@pytest.mark.parametrize("d", [16, 128, 256, 512])
 def test_rounding_midpoints_with_one_sign(d):
     rng = np.random.default_rng(d + 1)
     used = []
@@ -129,7 +133,8 @@ def test_rounding_midpoints_with_one_sign(d):
     # rounding down in a row times itself takes about half of the budget (the
     # products are 2^-10 too small, and rho = 2 x 2^-10): the case is as hard
     # as it is meant to be
-    assert 0.3 <= max(used) <= 0.7
+    # (a quarter where rho is 2^-8)
+    assert 0.3 <= max(used) * (rho_of(d) * 512.0) <= 0.7
 
 
 @pytest.mark.parametrize("case", ["mixed", "flush_limit", "tiny", "huge",

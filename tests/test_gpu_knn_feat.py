@@ -1,8 +1,8 @@
 """Feature-space kNN with the fp16 matrix-core filter (knn_feat_impl.hpp):
 parity with the CPU checker where the mechanisms of that path are exercised --
 lists that overflow (near-duplicates: the flagged queries go through the
-second pass), rows and queries the filter cannot represent, 129-256
-components, every list width, scales at both ends of fp32.  Bit-exact edges
+second pass), rows and queries the filter cannot represent, 129-512
+components, every list width (k up to 100), scales at both ends of fp32.  Bit-exact edges
 and distances, as everywhere.
 """
 import numpy as np
@@ -71,6 +71,25 @@ def test_near_duplicates_go_through_the_second_pass(oracle, d, cosine):
     _run(oracle, x2, y, None, None, 20, cosine)
 
 
+@pytest.mark.parametrize("d,k,cosine", [(300, 7, False), (512, 3, True),
+                                        (128, 65, False), (100, 100, False),
+                                        (257, 49, True), (400, 100, False),
+                                        (512, 64, True), (20, 80, False),
+                                        (9, 100, True), (384, 33, False)])
+def test_parity_up_to_512_components_and_100_neighbours(oracle, d, k, cosine):
+    rng = np.random.default_rng(d * 13 + k)
+    n, m = 2500, 300
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    y = rng.standard_normal((m, d)).astype(np.float32)
+    y[:20] = x[:20]
+    ptr_x = np.array([0, 90, 90, 1100, 2500])   # (k > rows of the first segment)
+    ptr_y = np.array([0, 60, 80, 81, 300])
+    _run(oracle, x, y, ptr_x, ptr_y, k, cosine)
+    # the filter kernel served the call: its per-call block was written
+    odd, flagged = _flagged_queries(x, y, k, cosine)
+    assert odd == 0 and 0 <= flagged <= m
+
+
 def _unresolved_queries(x, y, k, cosine=False):
     """Flagged queries that the threshold scan could not settle (fourth word
     of the per-call block, see _flagged_queries)."""
@@ -96,16 +115,16 @@ def test_flagged_queries_beyond_what_the_threshold_scan_holds(oracle, d):
     assert _unresolved_queries(x, y, 8) >= 1
     _run(oracle, x, y, None, None, 8)
     _run(oracle, x, y, None, None, 8, cosine=True)
-    # (b) more flagged queries than the scan's queue takes (1,024)
+    # (b) more flagged queries than the scan's queue takes (8,192 here)
     centres = rng.standard_normal((30, d)).astype(np.float32)
     x = np.repeat(centres, 40, axis=0)
     x = x * (1.0 + 1e-7 * rng.standard_normal(x.shape)).astype(np.float32)
     x = x.astype(np.float32)
-    y = np.repeat(centres, 50, axis=0)
+    y = np.repeat(centres, 300, axis=0)
     odd, flagged = _flagged_queries(x, y, 6)
-    assert flagged > 1024 and _unresolved_queries(x, y, 6) >= flagged - 1024
+    assert flagged > 8192 and _unresolved_queries(x, y, 6) == flagged - 8192
     ptr_x = np.array([0, 600, 1200])
-    ptr_y = np.array([0, 700, 1500])
+    ptr_y = np.array([0, 4200, 9000])
     _run(oracle, x, y, ptr_x, ptr_y, 6)
 
 
