@@ -17,6 +17,9 @@
 //               that are representable in the 16-bit type, which lets the
 //               16-bit types reuse the 64-bit (float distance, row) keys.
 #include "device_utils.hpp"
+
+#include <algorithm>
+#include <cstdlib>
 #include "launchers.hpp"
 
 #include <hip/hip_fp16.h>
@@ -185,6 +188,9 @@ template <int K> struct KeyList {
     sorted_insert<K>(b, key);
   }
   __device__ __forceinline__ int row_at(int j) const { return key_row(b[j]); }
+  __device__ __forceinline__ double dist_at(int j) const {
+    return (double)key_dist(b[j]);
+  }
 };
 
 // double distances: separate distance / row arrays, branch-free insertion
@@ -214,6 +220,7 @@ template <int K> struct PairList {
     dist[0] = here ? dd : dist[0];
   }
   __device__ __forceinline__ int row_at(int j) const { return row[j]; }
+  __device__ __forceinline__ double dist_at(int j) const { return dist[j]; }
 };
 
 template <typename Tr, int K> struct ListFor {
@@ -254,15 +261,21 @@ __global__ __launch_bounds__(kBlock) void knn_any_kernel(
     const int64_t *__restrict__ ptr_x, const int64_t *__restrict__ ptr_y,
     const typename Tr::calc_t *__restrict__ x_norm, int n, int m, int d,
     int num_segments, int k, const int *__restrict__ work_start,
-    int *__restrict__ out_idx, int *__restrict__ out_count) {
+    int *__restrict__ out_idx, int *__restrict__ out_count, int num_chunks,
+    double *__restrict__ part_dist, int *__restrict__ part_row) {
   typedef typename Tr::calc_t calc_t;
   constexpr int TG = kAnyTile;
   __shared__ calc_t xs[TG][kAnySlab];
   __shared__ calc_t xn[TG];
 
   const int tid = threadIdx.x;
-  const int tile = blockIdx.x;
-  if (tile >= work_start[num_segments])
+  // work item = (slice of the segment's x rows, tile of queries)
+  const int total_tiles = work_start[num_segments];
+  if (total_tiles == 0)
+    return;
+  const int chunk = blockIdx.x / total_tiles;
+  const int tile = blockIdx.x - chunk * total_tiles;
+  if (chunk >= num_chunks)
     return;
   const int seg = find_segment(work_start, num_segments, tile);
   const int x_begin = ptr_x ? (int)ptr_x[seg] : 0;
@@ -272,6 +285,11 @@ __global__ __launch_bounds__(kBlock) void knn_any_kernel(
   const int q = y_begin + (tile - work_start[seg]) * kBlock + tid;
   const bool valid = q < y_end;
   const typename Tr::store_t *yrow = y + (size_t)(valid ? q : y_begin) * d;
+  const int seg_len = x_end - x_begin;
+  const int chunk_len =
+      ((seg_len + num_chunks - 1) / num_chunks + TG - 1) / TG * TG;
+  const int c_begin = min(x_end, x_begin + chunk * chunk_len);
+  const int c_end = min(x_end, c_begin + chunk_len);
 
   typename ListFor<Tr, K>::type list;
   list.init(k, Tr::sentinel());
@@ -286,8 +304,8 @@ __global__ __launch_bounds__(kBlock) void knn_any_kernel(
     y_norm = Tr::norm(s);
   }
 
-  for (int base = x_begin; base < x_end; base += TG) {
-    const int rows = min(TG, x_end - base);
+  for (int base = c_begin; base < c_end; base += TG) {
+    const int rows = min(TG, c_end - base);
     calc_t acc[TG];
 #pragma unroll
     for (int j = 0; j < TG; ++j)
@@ -341,7 +359,70 @@ __global__ __launch_bounds__(kBlock) void knn_any_kernel(
     }
   }
 
+  if (num_chunks > 1) {
+    // this slice's list, [item][slot][query of the tile]: knn_any_merge_kernel
+    // unites the slices
+    const size_t at = (size_t)(chunk * total_tiles + tile) * k * kBlock + tid;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      const int e = j - (K - k);
+      if (e >= 0) {
+        part_dist[at + (size_t)e * kBlock] = list.dist_at(j);
+        part_row[at + (size_t)e * kBlock] = list.row_at(j);
+      }
+    }
+    return;
+  }
   if (valid) {
+    int found = 0;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      const int e = j - (K - k);
+      const int r = list.row_at(j);
+      if (e >= 0 && r >= 0) {
+        out_idx[(size_t)q * k + e] = r;
+        ++found;
+      }
+    }
+    out_count[q] = found;
+  }
+}
+
+// Unites the lists of a query's slices (ascending slices = ascending rows, so
+// an entry of equal distance from a later slice stays behind the earlier
+// ones, as in one scan over all rows).
+template <typename Tr, int K>
+__global__ __launch_bounds__(kBlock) void knn_any_merge_kernel(
+    const int64_t *__restrict__ ptr_y, int m, int num_segments, int k,
+    const int *__restrict__ work_start, int num_chunks,
+    const double *__restrict__ part_dist, const int *__restrict__ part_row,
+    int *__restrict__ out_idx, int *__restrict__ out_count) {
+  typedef typename Tr::calc_t calc_t;
+  const int tid = threadIdx.x;
+  const int total_tiles = work_start[num_segments];
+  const int tile = blockIdx.x;
+  if (tile >= total_tiles)
+    return;
+  const int seg = find_segment(work_start, num_segments, tile);
+  const int y_begin = ptr_y ? (int)ptr_y[seg] : 0;
+  const int y_end = ptr_y ? (int)ptr_y[seg + 1] : m;
+  const int q = y_begin + (tile - work_start[seg]) * kBlock + tid;
+  typename ListFor<Tr, K>::type list;
+  list.init(k, Tr::sentinel());
+  for (int c = 0; c < num_chunks; ++c) {
+    const size_t at = (size_t)(c * total_tiles + tile) * k * kBlock + tid;
+    for (int e = 0; e < k; ++e) {
+      const int row = part_row[at + (size_t)e * kBlock];
+      const calc_t dist = (calc_t)part_dist[at + (size_t)e * kBlock];
+      // (lists are ascending: behind an entry that does not get in, or an
+      // empty slot, nothing of this slice does)
+      const bool take = row >= 0 && dist < list.worst();
+      if (!__any(take))
+        break;
+      list.insert(take, dist, row);
+    }
+  }
+  if (q < y_end) {
     int found = 0;
 #pragma unroll
     for (int j = 0; j < K; ++j) {
@@ -535,44 +616,66 @@ __global__ __launch_bounds__(kBlock) void radius_any_kernel(
 
 // ---- launch helpers --------------------------------------------------------
 
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// bytes of the slices' distances (then their rows follow)
+size_t part_dist_bytes(int m, int num_segments, int k, int chunks) {
+  const size_t tiles = plan_upper_bound(m, num_segments, kBlock);
+  return align256(sizeof(double) * tiles * chunks * (size_t)k * kBlock);
+}
+
 template <typename Tr, int K>
 void launch_knn_any_k(const SearchInput &in, int k, bool cosine, void *x_norm,
                       const int *work_start, int grid, const DenseResult &out,
-                      hipStream_t stream) {
+                      hipStream_t stream, int chunks, void *scratch) {
   typedef typename Tr::store_t store_t;
   typedef typename Tr::calc_t calc_t;
   const store_t *x = static_cast<const store_t *>(in.x);
   const store_t *y = static_cast<const store_t *>(in.y);
   calc_t *norms = static_cast<calc_t *>(x_norm);
+  double *part_dist = static_cast<double *>(scratch);
+  int *part_row =
+      chunks > 1 ? reinterpret_cast<int *>(
+                       static_cast<char *>(scratch) +
+                       part_dist_bytes(in.m, in.num_segments, k, chunks))
+                 : nullptr;
   if (cosine) {
     hipLaunchKernelGGL((row_norm_any_kernel<Tr>),
                        dim3((in.n + kBlock - 1) / kBlock), dim3(kBlock), 0,
                        stream, x, in.n, in.d, norms);
-    hipLaunchKernelGGL((knn_any_kernel<Tr, K, true>), dim3(grid), dim3(kBlock),
-                       0, stream, x, y, in.ptr_x, in.ptr_y, norms, in.n, in.m,
-                       in.d, in.num_segments, k, work_start, out.idx,
-                       out.count);
-  } else {
-    hipLaunchKernelGGL((knn_any_kernel<Tr, K, false>), dim3(grid),
+    hipLaunchKernelGGL((knn_any_kernel<Tr, K, true>), dim3(grid * chunks),
                        dim3(kBlock), 0, stream, x, y, in.ptr_x, in.ptr_y,
                        norms, in.n, in.m, in.d, in.num_segments, k, work_start,
-                       out.idx, out.count);
+                       out.idx, out.count, chunks, part_dist, part_row);
+  } else {
+    hipLaunchKernelGGL((knn_any_kernel<Tr, K, false>), dim3(grid * chunks),
+                       dim3(kBlock), 0, stream, x, y, in.ptr_x, in.ptr_y,
+                       norms, in.n, in.m, in.d, in.num_segments, k, work_start,
+                       out.idx, out.count, chunks, part_dist, part_row);
   }
+  if (chunks > 1)
+    hipLaunchKernelGGL((knn_any_merge_kernel<Tr, K>), dim3(grid), dim3(kBlock),
+                       0, stream, in.ptr_y, in.m, in.num_segments, k,
+                       work_start, chunks, part_dist, part_row, out.idx,
+                       out.count);
 }
 
 template <typename Tr>
 hipError_t launch_knn_any_t(const SearchInput &in, int k, bool cosine,
                             void *x_norm, const int *work_start, int grid,
-                            const DenseResult &out, hipStream_t stream) {
+                            const DenseResult &out, hipStream_t stream,
+                            void *scratch) {
+  const int chunks =
+      scratch ? knn_anytype_slices(in.n, in.m, in.num_segments) : 1;
   if (k <= 16)
     launch_knn_any_k<Tr, 16>(in, k, cosine, x_norm, work_start, grid, out,
-                             stream);
+                             stream, chunks, scratch);
   else if (k <= 48)
     launch_knn_any_k<Tr, 48>(in, k, cosine, x_norm, work_start, grid, out,
-                             stream);
+                             stream, chunks, scratch);
   else
     launch_knn_any_k<Tr, 100>(in, k, cosine, x_norm, work_start, grid, out,
-                              stream);
+                              stream, chunks, scratch);
   return hipGetLastError();
 }
 
@@ -629,22 +732,47 @@ hipError_t launch_nearest_any(int dtype, const SearchInput &in,
 
 size_t anytype_norm_bytes(int n) { return sizeof(double) * (size_t)n; }
 
+int knn_anytype_slices(int n, int m, int num_segments) {
+  // enough work items for four workgroups per CU, slices of at least 32 LDS
+  // tiles on average
+  const int tiles = plan_upper_bound(m, num_segments, kBlock);
+  const int want = (1024 + tiles - 1) / tiles;
+  const int by_length = (n / num_segments) / (32 * kAnyTile);
+  int chunks = std::max(1, std::min(std::min(want, 64), by_length));
+  if (const char *env = std::getenv("PCA_KNN_SLICES")) {
+    const int v = std::atoi(env);
+    if (v >= 1 && v <= 64)
+      chunks = v;
+  }
+  return chunks;
+}
+
+size_t knn_anytype_scratch_bytes(int n, int m, int num_segments, int k) {
+  const int chunks = knn_anytype_slices(n, m, num_segments);
+  if (chunks <= 1)
+    return 0;
+  const size_t tiles = plan_upper_bound(m, num_segments, kBlock);
+  return part_dist_bytes(m, num_segments, k, chunks) +
+         align256(sizeof(int) * tiles * chunks * (size_t)k * kBlock);
+}
+
 hipError_t launch_knn_anytype(int dtype, const SearchInput &in, int k,
                               bool cosine, void *x_norm,
                               const int *work_start, int grid_bound,
-                              const DenseResult &out, hipStream_t stream) {
+                              const DenseResult &out, hipStream_t stream,
+                              void *scratch) {
   switch (dtype) {
   case 1:
     return launch_knn_any_t<F64Traits>(in, k, cosine, x_norm, work_start,
-                                       grid_bound, out, stream);
+                                       grid_bound, out, stream, scratch);
   case 2:
     return launch_knn_any_t<R16Traits<false>>(in, k, cosine, x_norm,
                                               work_start, grid_bound, out,
-                                              stream);
+                                              stream, scratch);
   case 3:
     return launch_knn_any_t<R16Traits<true>>(in, k, cosine, x_norm,
                                              work_start, grid_bound, out,
-                                             stream);
+                                             stream, scratch);
   default:
     return hipErrorInvalidValue;
   }

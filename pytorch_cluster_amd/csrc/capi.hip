@@ -93,6 +93,8 @@ KnnLayout knn_layout(int64_t n, int64_t m, int64_t d, int64_t num_segments,
   KnnLayout w;
   if (dtype != PCA_F32) {
     w.x_norm = align256(pca::anytype_norm_bytes((int)n));
+    w.sliced = pca::knn_anytype_scratch_bytes((int)n, (int)m,
+                                              (int)num_segments, (int)k);
   } else if (d > 8) {
     w.x_norm = align256(sizeof(float) * (size_t)n);
     if (pca::knn_feat_supported((int)d, (int)k, false))
@@ -101,6 +103,9 @@ KnnLayout knn_layout(int64_t n, int64_t m, int64_t d, int64_t num_segments,
     else if (pca::knn_mfma_supported((int)d, (int)k, false))
       w.sliced = pca::knn_mfma_scratch_bytes((int)n, (int)m, (int)d,
                                              (int)num_segments, (int)k);
+    else
+      w.sliced = pca::knn_generic_scratch_bytes((int)n, (int)m,
+                                                (int)num_segments, (int)k);
   } else {
     // the larger of the two metrics' needs, so one size query serves both
     for (int cosine = 0; cosine < 2; ++cosine) {
@@ -447,7 +452,9 @@ int knn_call(const void *x, const void *y, const int64_t *ptr_x,
     timer.begin();
     rc = check_launch(pca::launch_knn_anytype(dtype, in, (int)k, cosine != 0,
                                               x_norm, work_start, bound,
-                                              dense, stream),
+                                              dense, stream,
+                                              lay.sliced ? lowd_scratch
+                                                         : nullptr),
                       "knn_any_kernel");
     timer.done();
   } else {
@@ -459,9 +466,9 @@ int knn_call(const void *x, const void *y, const int64_t *ptr_x,
         return rc;
     }
     timer.begin();
-    rc = check_launch(pca::launch_knn_generic(in, (int)k, cosine != 0, x_norm,
-                                              work_start, bound, dense,
-                                              stream),
+    rc = check_launch(pca::launch_knn_generic(
+                          in, (int)k, cosine != 0, x_norm, work_start, bound,
+                          dense, stream, lay.sliced ? lowd_scratch : nullptr),
                       "knn_generic_kernel");
     timer.done();
   }

@@ -278,8 +278,8 @@ static FeatLayout feat_layout(int n, int m, int d, int num_segments, int k) {
   w.cand = align256(sizeof(double) * (size_t)m * kk);
   w.second = second_pass_on_matrix_cores(d, k)
                  ? knn_mfma_scratch_bytes(n, m, d, num_segments, k,
-                                               kSecondPassChunks)
-                      : 0;
+                                          kSecondPassChunks)
+                 : knn_generic_scratch_bytes(n, m, num_segments, k);
   return w;
 }
 
@@ -506,8 +506,8 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
     return err;
   return launch_knn_generic(
       in, k, cosine, x_norm, plan256,
-      plan_upper_bound(in.m, in.num_segments, kBlock), out, stream, gate,
-      redo_q);
+      plan_upper_bound(in.m, in.num_segments, kBlock), out, stream,
+      lay.second ? first_pass : nullptr, gate, redo_q);
 }
 
 } // namespace pca

@@ -38,7 +38,8 @@ __global__ __launch_bounds__(kBlock) void knn_generic_kernel(
     int k, const int *__restrict__ work_start, int grid,
     int *__restrict__ out_idx, float *__restrict__ out_dist,
     int *__restrict__ out_count, const int *__restrict__ gate,
-    const int *__restrict__ redo_q) {
+    const int *__restrict__ redo_q, int num_chunks,
+    double *__restrict__ partial) {
   constexpr int TG = kGenTile;
   constexpr int CH = kGenChunk;
   constexpr int QCAP = kGenQueueCap;
@@ -52,8 +53,14 @@ __global__ __launch_bounds__(kBlock) void knn_generic_kernel(
   if (gate != nullptr && *gate == 0)
     return;
   const int tid = threadIdx.x;
-  const int tile = PCA_TILE_OF_BLOCK(blockIdx.x, grid);
-  if (tile >= work_start[num_segments])
+  // work item = (slice of the segment's x rows, tile of queries)
+  const int item = PCA_TILE_OF_BLOCK(blockIdx.x, grid);
+  const int total_tiles = work_start[num_segments];
+  if (total_tiles == 0)
+    return;
+  const int chunk = item / total_tiles;
+  const int tile = item - chunk * total_tiles;
+  if (chunk >= num_chunks)
     return;
   const int seg = find_segment(work_start, num_segments, tile);
   const int x_begin = ptr_x ? (int)ptr_x[seg] : 0;
@@ -68,6 +75,11 @@ __global__ __launch_bounds__(kBlock) void knn_generic_kernel(
       return;
   }
   const float *yrow = y + (size_t)(valid ? q : y_begin) * d;
+  const int seg_len = x_end - x_begin;
+  const int chunk_len =
+      ((seg_len + num_chunks - 1) / num_chunks + TG - 1) / TG * TG;
+  const int c_begin = min(x_end, x_begin + chunk * chunk_len);
+  const int c_end = min(x_end, c_begin + chunk_len);
 
   double best[K];
 #pragma unroll
@@ -100,8 +112,8 @@ __global__ __launch_bounds__(kBlock) void knn_generic_kernel(
     qcount = 0;
   };
 
-  for (int base = x_begin; base < x_end; base += TG) {
-    const int rows = min(TG, x_end - base);
+  for (int base = c_begin; base < c_end; base += TG) {
+    const int rows = min(TG, c_end - base);
     float acc[TG];
 #pragma unroll
     for (int j = 0; j < TG; ++j)
@@ -185,6 +197,18 @@ __global__ __launch_bounds__(kBlock) void knn_generic_kernel(
   }
   flush();
 
+  if (num_chunks > 1) {
+    // sorted keys of this slice, [item][slot][query of the tile]; the merge
+    // (knn_merge_kernel) unites the slices
+    double *dst = partial + (size_t)(chunk * total_tiles + tile) * k * kBlock + tid;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      const int e = j - (K - k);
+      if (e >= 0)
+        dst[(size_t)e * kBlock] = best[j];
+    }
+    return;
+  }
   if (valid) {
     const size_t row = (size_t)q * k;
     int found = 0;
@@ -208,7 +232,8 @@ hipError_t launch_knn_generic_metric(const SearchInput &in, int k, int kbucket,
                                      const int *work_start, int grid_bound,
                                      const DenseResult &out,
                                      hipStream_t stream, const int *gate,
-                                     const int *redo_q);
+                                     const int *redo_q, int num_chunks,
+                                     double *partial);
 
 #define PCA_GENERIC_CASE(KB, C)                                                \
   case KB:                                                                     \
@@ -216,7 +241,8 @@ hipError_t launch_knn_generic_metric(const SearchInput &in, int k, int kbucket,
                        0, stream, (const float *)in.x, (const float *)in.y,    \
                        in.ptr_x, in.ptr_y, x_norm, in.n, in.m, in.d,           \
                        in.num_segments, k, work_start, grid, out.idx,          \
-                       out.dist, out.count, gate, redo_q);                     \
+                       out.dist, out.count, gate, redo_q, num_chunks,          \
+                       partial);                                               \
     break;
 
 #define PCA_GENERIC_DEFINE(C)                                                  \
@@ -224,8 +250,9 @@ hipError_t launch_knn_generic_metric(const SearchInput &in, int k, int kbucket,
   hipError_t launch_knn_generic_metric<C>(                                     \
       const SearchInput &in, int k, int kbucket, const float *x_norm,          \
       const int *work_start, int grid_bound, const DenseResult &out,           \
-      hipStream_t stream, const int *gate, const int *redo_q) {                \
-    const int grid = (grid_bound + 7) & ~7;                                    \
+      hipStream_t stream, const int *gate, const int *redo_q,                  \
+      int num_chunks, double *partial) {                                       \
+    const int grid = (grid_bound * num_chunks + 7) & ~7;                       \
     switch (kbucket) {                                                         \
       PCA_GENERIC_CASE(8, C)                                                   \
       PCA_GENERIC_CASE(16, C)                                                  \

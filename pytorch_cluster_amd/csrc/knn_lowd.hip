@@ -4,6 +4,7 @@
 #include "knn_lowd_impl.hpp"
 #include "knn_lowd_mc_impl.hpp"
 
+#include <algorithm>
 #include <cstdlib>
 
 namespace pca {
@@ -279,18 +280,93 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
   return hipGetLastError();
 }
 
+int knn_generic_slices(int n, int m, int num_segments) {
+  // enough work items for four workgroups per CU, slices of at least 16 LDS
+  // tiles on average
+  const int tiles = plan_upper_bound(m, num_segments, kBlock);
+  const int want = (1024 + tiles - 1) / tiles;
+  const int by_length = (n / num_segments) / (16 * kGenTile);
+  int chunks = std::max(1, std::min(std::min(want, 64), by_length));
+  const int forced = env_int("PCA_KNN_SLICES", 0);
+  if (forced >= 1 && forced <= 64)
+    chunks = forced;
+  return chunks;
+}
+
+size_t knn_generic_scratch_bytes(int n, int m, int num_segments, int k) {
+  const int chunks = knn_generic_slices(n, m, num_segments);
+  if (chunks <= 1)
+    return 0;
+  const size_t tiles = plan_upper_bound(m, num_segments, kBlock);
+  return align256(sizeof(double) * tiles * chunks * (size_t)k * kBlock);
+}
+
 hipError_t launch_knn_generic(const SearchInput &in, int k, bool cosine,
                               const float *x_norm, const int *work_start,
                               int grid_bound, const DenseResult &out,
-                              hipStream_t stream, const int *gate,
-                              const int *redo_q) {
+                              hipStream_t stream, void *scratch,
+                              const int *gate, const int *redo_q) {
   const int kb = k_bucket(k);
-  return cosine ? launch_knn_generic_metric<true>(in, k, kb, x_norm,
-                                                  work_start, grid_bound, out,
-                                                  stream, gate, redo_q)
-                : launch_knn_generic_metric<false>(in, k, kb, x_norm,
-                                                   work_start, grid_bound, out,
-                                                   stream, gate, redo_q);
+  const int chunks =
+      scratch ? knn_generic_slices(in.n, in.m, in.num_segments) : 1;
+  double *partial = static_cast<double *>(scratch);
+  const hipError_t err =
+      cosine ? launch_knn_generic_metric<true>(in, k, kb, x_norm, work_start,
+                                               grid_bound, out, stream, gate,
+                                               redo_q, chunks, partial)
+             : launch_knn_generic_metric<false>(in, k, kb, x_norm, work_start,
+                                                grid_bound, out, stream, gate,
+                                                redo_q, chunks, partial);
+  if (err != hipSuccess || chunks <= 1)
+    return err;
+  // the slices' lists -> dense results
+  KnnLowdParams p;
+  p.x = static_cast<const float *>(in.x);
+  p.y = static_cast<const float *>(in.y);
+  p.ptr_x = in.ptr_x;
+  p.ptr_y = in.ptr_y;
+  p.n = in.n;
+  p.m = in.m;
+  p.d_in = in.d;
+  p.num_segments = in.num_segments;
+  p.k = k;
+  p.work_start = work_start;
+  p.num_chunks = chunks;
+  p.tau = nullptr;
+  p.partial = partial;
+  p.out_idx = out.idx;
+  p.out_dist = out.dist;
+  p.out_count = out.count;
+  p.out_nearest = nullptr;
+  p.x_split = nullptr;
+  p.gate = gate;
+  p.redo_q = redo_q;
+  switch (kb) {
+  case 8:
+    launch_merge<8>(p, kBlock, grid_bound, stream);
+    break;
+  case 16:
+    launch_merge<16>(p, kBlock, grid_bound, stream);
+    break;
+  case 24:
+    launch_merge<24>(p, kBlock, grid_bound, stream);
+    break;
+  case 32:
+    launch_merge<32>(p, kBlock, grid_bound, stream);
+    break;
+  case 48:
+    launch_merge<48>(p, kBlock, grid_bound, stream);
+    break;
+  case 64:
+    launch_merge<64>(p, kBlock, grid_bound, stream);
+    break;
+  case 100:
+    launch_merge<100>(p, kBlock, grid_bound, stream);
+    break;
+  default:
+    return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
 }
 
 } // namespace pca

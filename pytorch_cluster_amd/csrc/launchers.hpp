@@ -150,14 +150,21 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
 // |x_i| for the cosine distance of the any-dimension kernel.
 hipError_t launch_row_norms(const float *x, int n, int d, float *norm,
                             hipStream_t stream);
+// Slices of every segment's x rows the any-dimension kernel works in, and
+// the bytes of their partial lists (0: one slice, no scratch needed).
+int knn_generic_slices(int n, int m, int num_segments);
+size_t knn_generic_scratch_bytes(int n, int m, int num_segments, int k);
 // x_norm: [n] row norms of x (cosine only, else NULL).  One query per lane:
-// work items are tiles of kBlock queries.  As a second pass behind another
-// search: gate (device flag, nothing runs while it is 0) and redo_q ([m], only
-// queries with a non-zero entry are searched and written).
+// work items are tiles of kBlock queries times the slices.  scratch:
+// knn_generic_scratch_bytes bytes, or NULL to search every segment in one
+// slice.  As a second pass behind another search: gate (device flag, nothing
+// runs while it is 0) and redo_q ([m], only queries with a non-zero entry are
+// searched and written).
 hipError_t launch_knn_generic(const SearchInput &in, int k, bool cosine,
                               const float *x_norm, const int *work_start,
                               int grid_bound, const DenseResult &out,
-                              hipStream_t stream, const int *gate = nullptr,
+                              hipStream_t stream, void *scratch,
+                              const int *gate = nullptr,
                               const int *redo_q = nullptr);
 
 // --- anytype.hip (fp64 / fp16 / bf16; dtype codes of enum pca_dtype) -------
@@ -165,10 +172,15 @@ hipError_t launch_knn_generic(const SearchInput &in, int k, bool cosine,
 size_t anytype_norm_bytes(int n);
 // work_start: tiles of kBlock queries (kNN), wave tasks of
 // kRadiusQueriesPerWave queries (radius).
+// scratch: knn_anytype_scratch_bytes bytes for the slices' lists, or NULL to
+// search every segment in one slice.
+int knn_anytype_slices(int n, int m, int num_segments);
+size_t knn_anytype_scratch_bytes(int n, int m, int num_segments, int k);
 hipError_t launch_knn_anytype(int dtype, const SearchInput &in, int k,
                               bool cosine, void *x_norm,
                               const int *work_start, int grid_bound,
-                              const DenseResult &out, hipStream_t stream);
+                              const DenseResult &out, hipStream_t stream,
+                              void *scratch);
 hipError_t launch_radius_anytype(int dtype, const SearchInput &in, double r,
                                  bool ignore_same_index,
                                  const int *work_start, int task_bound,

@@ -65,7 +65,10 @@ def test_reference_fixtures_all_dtypes(dtype):
 @pytest.mark.parametrize("d,k", [(3, 7), (2, 16), (5, 40), (40, 9),
                                  (200, 3)])
 @pytest.mark.parametrize("cosine", [False, True])
-def test_knn_fp64_parity(oracle, d, k, cosine):
+@pytest.mark.parametrize("slices", [1, 6])
+def test_knn_fp64_parity(oracle, monkeypatch, d, k, cosine, slices):
+    # (slices of every segment's rows, whose lists a second kernel unites)
+    monkeypatch.setenv("PCA_KNN_SLICES", str(slices))
     rng = np.random.default_rng(d * 31 + k)
     n, m = 1300, 400
     x = rng.standard_normal((n, d))
@@ -83,7 +86,10 @@ def test_knn_fp64_parity(oracle, d, k, cosine):
                                         (torch.bfloat16, 1)])
 @pytest.mark.parametrize("d,k", [(3, 7), (2, 16), (6, 40), (40, 9)])
 @pytest.mark.parametrize("cosine", [False, True])
-def test_knn_16bit_parity(oracle, dtype, kind, d, k, cosine):
+@pytest.mark.parametrize("slices", [1, 5])
+def test_knn_16bit_parity(oracle, monkeypatch, dtype, kind, d, k, cosine,
+                          slices):
+    monkeypatch.setenv("PCA_KNN_SLICES", str(slices))
     rng = np.random.default_rng(d * 17 + k + kind)
     n, m = 1100, 300
     # 16-bit arithmetic produces many exactly equal distances: the order by
@@ -95,6 +101,18 @@ def test_knn_16bit_parity(oracle, dtype, kind, d, k, cosine):
     got = gpu_knn_t(x, y, ptr_x, ptr_y, k, cosine)
     want, _ = oracle.knn_op16(bits(x), bits(y), ptr_x, ptr_y, k, cosine, kind)
     assert got.shape == want.shape
+    assert (got == want).all()
+
+
+def test_knn_fp64_large_cloud_default_slices(oracle):
+    # enough rows that the library slices on its own; duplicated rows, so that
+    # equal distances meet across slice borders
+    rng = np.random.default_rng(77)
+    base = rng.standard_normal((6000, 3))
+    x = np.concatenate([base, base[:3000], base[:1500]])
+    y = base[::40] + 0.0
+    got = gpu_knn_t(torch.from_numpy(x), torch.from_numpy(y), None, None, 12)
+    want = oracle.knn_op(x, y, None, None, 12, False, fma_mode=1)
     assert (got == want).all()
 
 

@@ -192,7 +192,19 @@ def test_cosine_parity(oracle, d, k):
                                         (100, 50, False), (64, 64, True),
                                         (128, 64, False), (128, 65, False),
                                         (300, 7, False), (515, 3, True)])
-def test_parity_high_dimension(oracle, d, k, cosine):
+@pytest.mark.parametrize("path", ["default", "exact_mfma", "any_dimension",
+                                  "any_dimension_sliced"])
+def test_parity_high_dimension(oracle, monkeypatch, d, k, cosine, path):
+    # default: the fp16 matrix-core filter (up to 512 components); the other
+    # kernels of these shapes -- the exact split-bf16 kernel (d <= 128,
+    # k <= 64) and the any-dimension kernel, in one slice and in several --
+    # serve as its last resort and beyond 512 components
+    if path == "exact_mfma":
+        monkeypatch.setenv("PCA_KNN_FEAT", "0")
+    elif path != "default":
+        monkeypatch.setenv("PCA_KNN_NO_MFMA", "1")
+        monkeypatch.setenv("PCA_KNN_SLICES",
+                           "1" if path == "any_dimension" else "5")
     rng = np.random.default_rng(d * 7 + k)
     n, m = 1500, 300
     x = rng.standard_normal((n, d)).astype(np.float32)
