@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define PCA_ABI_VERSION 4
+#define PCA_ABI_VERSION 5
 
 enum pca_status {
   PCA_OK = 0,
@@ -76,9 +76,20 @@ enum pca_dtype {
  *                        ignore_same_index)
  *   PCA_EDGES_X_FIRST    edges[0 .. E) are the x rows, edges[E .. 2E) the
  *                        query rows (flow "source_to_target")
+ * and the prologue of all four entry points (torch_cluster/knn.py:62-79,
+ * torch_cluster/radius.py:66-84) into the launch that prepares the search:
+ *   PCA_SEGMENTS_BY_ID   ptr_x / ptr_y are not pointers but the SORTED example
+ *                        ids of the rows ([n] and [m] int64, values in
+ *                        [0, num_segments)); the pointers -- ptr[b] = number
+ *                        of rows with an id below b, what the reference's
+ *                        wrappers get from two bucketize calls -- are derived
+ *                        on the device.  pca_knn, pca_knn_fixed_scratch and
+ *                        pca_radius take it; for the other entry points call
+ *                        pca_segment_pointers first.
  */
 #define PCA_EDGES_DROP_SELF 1
 #define PCA_EDGES_X_FIRST 2
+#define PCA_SEGMENTS_BY_ID 4
 
 /* ABI version of the loaded library (== PCA_ABI_VERSION it was built with). */
 int pca_abi_version(void);
@@ -99,6 +110,16 @@ const char *pca_last_error(void);
  * to cancel it.  No counterpart in the reference.
  */
 int pca_time_next_search(void *start_event, void *stop_event);
+
+/*
+ * ptr_x[b] / ptr_y[b] = number of rows of x / y whose example id is below b,
+ * b = 0 .. num_segments: the segment pointers of sorted example-id vectors
+ * (torch_cluster/knn.py:75-79: two torch.bucketize calls).  One small launch;
+ * ptr_x and ptr_y: num_segments + 1 entries each, device memory.
+ */
+int pca_segment_pointers(const int64_t *ids_x, int64_t n, const int64_t *ids_y,
+                         int64_t m, int64_t num_segments, int64_t *ptr_x,
+                         int64_t *ptr_y, void *stream);
 
 /* ------------------------------------------------------------------ kNN -- */
 

@@ -22,7 +22,7 @@ _BUILD_HINT = ("build it with `python pytorch_cluster_amd/build.py` "
                "(or `python -c 'import __graft_entry__ as g; g.build()'`)")
 
 PCA_F32, PCA_F64, PCA_F16, PCA_BF16 = 0, 1, 2, 3
-PCA_EDGES_DROP_SELF, PCA_EDGES_X_FIRST = 1, 2
+PCA_EDGES_DROP_SELF, PCA_EDGES_X_FIRST, PCA_SEGMENTS_BY_ID = 1, 2, 4
 PCA_FIXED_SCRATCH_BYTES = 32 << 20
 
 _vp = ctypes.c_void_p
@@ -40,6 +40,8 @@ C_ABI = {
                 [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                  ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp,
                  ctypes.c_size_t, _vp]),
+    "pca_segment_pointers": (ctypes.c_int,
+                             [_vp, _i64, _vp, _i64, _i64, _vp, _vp, _vp]),
     "pca_knn_fixed_scratch": (ctypes.c_int,
                               [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                                _i64, ctypes.c_int, ctypes.c_int, ctypes.c_int,

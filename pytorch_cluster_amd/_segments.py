@@ -18,6 +18,14 @@ def as_points(t: torch.Tensor) -> torch.Tensor:
     return t.contiguous()
 
 
+def check_ids(x: torch.Tensor, y: torch.Tensor, batch_x: torch.Tensor,
+              batch_y: torch.Tensor) -> None:
+    """The size checks of the reference's wrappers
+    (``torch_cluster/knn.py:66,71``)."""
+    assert x.size(0) == batch_x.numel()
+    assert y.size(0) == batch_y.numel()
+
+
 def num_examples(x: torch.Tensor, y: torch.Tensor,
                  batch_x: Optional[torch.Tensor],
                  batch_y: Optional[torch.Tensor],

@@ -10,6 +10,7 @@ from typing import Optional, Tuple
 import torch
 
 from ._native import (PCA_BF16, PCA_EDGES_DROP_SELF, PCA_EDGES_X_FIRST, PCA_F16,
+                      PCA_SEGMENTS_BY_ID,
                       PCA_F32, PCA_F64, capi)
 
 _DTYPE_CODE = {torch.float32: PCA_F32, torch.float64: PCA_F64,
@@ -38,35 +39,58 @@ def _stream_handle(stream: Optional[torch.cuda.Stream], device):
     return ctypes.c_void_p(s.cuda_stream)
 
 
-def _segments(ptr_x, ptr_y):
+def _segments(ptr_x, ptr_y, ids_examples: int = 0):
+    """(ptr_x, ptr_y, number of segments); with ``ids_examples`` > 0 the two
+    tensors are the rows' sorted example ids (``PCA_SEGMENTS_BY_ID``)."""
     if ptr_x is None and ptr_y is None:
         return None, None, 1
     assert ptr_x is not None and ptr_y is not None
     assert ptr_x.dtype == torch.long and ptr_y.dtype == torch.long
     assert ptr_x.is_contiguous() and ptr_y.is_contiguous()
+    if ids_examples > 0:
+        return ptr_x, ptr_y, ids_examples
     assert ptr_x.numel() == ptr_y.numel()
     return ptr_x, ptr_y, ptr_x.numel() - 1
 
 
-def _edge_flags(drop_self: bool, x_first: bool) -> int:
+def _edge_flags(drop_self: bool, x_first: bool, by_id: bool = False) -> int:
     return ((PCA_EDGES_DROP_SELF if drop_self else 0)
-            | (PCA_EDGES_X_FIRST if x_first else 0))
+            | (PCA_EDGES_X_FIRST if x_first else 0)
+            | (PCA_SEGMENTS_BY_ID if by_id else 0))
+
+
+def segment_pointers(ids_x, ids_y, num_segments: int, stream=None):
+    """``pca_segment_pointers``: (ptr_x, ptr_y), ``num_segments + 1`` entries
+    each, of two sorted example-id vectors."""
+    assert ids_x.is_cuda and ids_x.dtype == torch.long
+    assert ids_y.is_cuda and ids_y.dtype == torch.long
+    ptr_x = torch.empty(num_segments + 1, dtype=torch.long,
+                        device=ids_x.device)
+    ptr_y = torch.empty_like(ptr_x)
+    _check(capi.pca_segment_pointers(
+        _dev_ptr(ids_x), ids_x.numel(), _dev_ptr(ids_y), ids_y.numel(),
+        num_segments, _dev_ptr(ptr_x), _dev_ptr(ptr_y),
+        _stream_handle(stream, ids_x.device)))
+    return ptr_x, ptr_y
 
 
 def knn_launch(x, y, ptr_x, ptr_y, k: int, cosine: bool = False,
                want_dist: bool = False, stream=None, drop_self: bool = False,
                x_first: bool = False, binned: bool = False,
-               fixed_scratch: bool = False):
+               fixed_scratch: bool = False, ids_examples: int = 0):
     """Queues ``pca_knn`` (``binned``: ``pca_knn_binned``; ``fixed_scratch``:
     ``pca_knn_fixed_scratch``, no workspace); returns (edges buffer [2*m*k],
     num_edges [1] on the device, dist buffer or None, workspace or None).
-    Nothing is synchronised."""
+    ``ids_examples`` > 0: ``ptr_x`` / ``ptr_y`` are the rows' sorted example
+    ids, that many examples.  Nothing is synchronised."""
     assert x.is_cuda and y.is_cuda and x.is_contiguous() and y.is_contiguous()
     assert x.dtype == y.dtype and x.dtype in _DTYPE_CODE
     dtype = _DTYPE_CODE[x.dtype]
     n, d = x.shape
     m = y.shape[0]
-    ptr_x, ptr_y, nseg = _segments(ptr_x, ptr_y)
+    ptr_x, ptr_y, nseg = _segments(ptr_x, ptr_y, ids_examples)
+    by_id = ids_examples > 0
+    assert not (by_id and binned)
     edges = torch.empty(max(2 * m * max(k, 0), 1), dtype=torch.long,
                         device=x.device)
     num_edges = torch.empty(1, dtype=torch.long, device=x.device)
@@ -76,7 +100,8 @@ def knn_launch(x, y, ptr_x, ptr_y, k: int, cosine: bool = False,
         assert not binned
         _check(capi.pca_knn_fixed_scratch(
             _dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x), _dev_ptr(ptr_y), n, m,
-            d, nseg, k, int(cosine), dtype, _edge_flags(drop_self, x_first),
+            d, nseg, k, int(cosine), dtype,
+            _edge_flags(drop_self, x_first, by_id),
             _dev_ptr(edges), _dev_ptr(num_edges), _dev_ptr(dist),
             _stream_handle(stream, x.device)))
         return edges, num_edges, dist, None
@@ -99,7 +124,7 @@ def knn_launch(x, y, ptr_x, ptr_y, k: int, cosine: bool = False,
         return edges, num_edges, dist, ws
     _check(capi.pca_knn(_dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x),
                         _dev_ptr(ptr_y), n, m, d, nseg, k, int(cosine),
-                        dtype, _edge_flags(drop_self, x_first),
+                        dtype, _edge_flags(drop_self, x_first, by_id),
                         _dev_ptr(edges), _dev_ptr(num_edges),
                         _dev_ptr(dist), _dev_ptr(ws), ws_bytes,
                         _stream_handle(stream, x.device)))
@@ -109,12 +134,13 @@ def knn_launch(x, y, ptr_x, ptr_y, k: int, cosine: bool = False,
 def knn_edges(x, y, ptr_x=None, ptr_y=None, k: int = 1, cosine: bool = False,
               want_dist: bool = False, stream=None, drop_self: bool = False,
               x_first: bool = False, binned: bool = False,
-              fixed_scratch: bool = False
+              fixed_scratch: bool = False, ids_examples: int = 0
               ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """``[2, E]`` edges (and the ``[E]`` distances when asked for)."""
     edges, num_edges, dist, _ws = knn_launch(x, y, ptr_x, ptr_y, k, cosine,
                                              want_dist, stream, drop_self,
-                                             x_first, binned, fixed_scratch)
+                                             x_first, binned, fixed_scratch,
+                                             ids_examples)
     e = int(num_edges.item())
     out = edges[:2 * e].view(2, e)
     return out, (dist[:e] if dist is not None else None)
@@ -122,13 +148,16 @@ def knn_edges(x, y, ptr_x=None, ptr_y=None, k: int = 1, cosine: bool = False,
 
 def radius_launch(x, y, ptr_x, ptr_y, r: float, max_num_neighbors: int,
                   ignore_same_index: bool = False, stream=None,
-                  x_first: bool = False, binned: bool = False):
+                  x_first: bool = False, binned: bool = False,
+                  ids_examples: int = 0):
     assert x.is_cuda and y.is_cuda and x.is_contiguous() and y.is_contiguous()
     assert x.dtype == y.dtype and x.dtype in _DTYPE_CODE
     dtype = _DTYPE_CODE[x.dtype]
     n, d = x.shape
     m = y.shape[0]
-    ptr_x, ptr_y, nseg = _segments(ptr_x, ptr_y)
+    ptr_x, ptr_y, nseg = _segments(ptr_x, ptr_y, ids_examples)
+    by_id = ids_examples > 0
+    assert not (by_id and binned)
     if binned:
         assert dtype == 0
         ws_bytes = capi.pca_radius_binned_workspace_bytes(
@@ -153,7 +182,7 @@ def radius_launch(x, y, ptr_x, ptr_y, r: float, max_num_neighbors: int,
     _check(capi.pca_radius(_dev_ptr(x), _dev_ptr(y), _dev_ptr(ptr_x),
                            _dev_ptr(ptr_y), n, m, d, nseg, float(r),
                            max_num_neighbors, int(ignore_same_index), dtype,
-                           _edge_flags(False, x_first),
+                           _edge_flags(False, x_first, by_id),
                            _dev_ptr(edges), _dev_ptr(num_edges), _dev_ptr(ws),
                            ws_bytes, _stream_handle(stream, x.device)))
     return edges, num_edges, ws
@@ -162,11 +191,11 @@ def radius_launch(x, y, ptr_x, ptr_y, r: float, max_num_neighbors: int,
 def radius_edges(x, y, ptr_x=None, ptr_y=None, r: float = 1.0,
                  max_num_neighbors: int = 32, ignore_same_index: bool = False,
                  stream=None, x_first: bool = False,
-                 binned: bool = False) -> torch.Tensor:
+                 binned: bool = False, ids_examples: int = 0) -> torch.Tensor:
     edges, num_edges, _ws = radius_launch(x, y, ptr_x, ptr_y, r,
                                           max_num_neighbors,
                                           ignore_same_index, stream, x_first,
-                                          binned)
+                                          binned, ids_examples)
     e = int(num_edges.item())
     return edges[:2 * e].view(2, e)
 

@@ -78,13 +78,40 @@ bool sizes_ok(int64_t n, int64_t m, int64_t d, int64_t num_segments) {
          d <= (1 << 20) && num_segments >= 1 && num_segments <= kMaxRows;
 }
 
+// two arrays of num_segments + 1 pointers (PCA_SEGMENTS_BY_ID)
+size_t segment_pointer_bytes(int64_t num_segments) {
+  return 2 * align256(sizeof(int64_t) * (size_t)(num_segments + 1));
+}
+
+// With PCA_SEGMENTS_BY_ID the caller's ptr_x / ptr_y are sorted example ids;
+// the pointers the kernels read live in `area` (segment_pointer_bytes) and are
+// written by the launch that plans the work.  Returns the source description
+// for that launch and redirects ptr_x / ptr_y.
+pca::SegmentSource segments_by_id(const int64_t *&ptr_x, const int64_t *&ptr_y,
+                                  int64_t n, int64_t m, int64_t num_segments,
+                                  void *area) {
+  pca::SegmentSource src;
+  src.ids_x = ptr_x;
+  src.ids_y = ptr_y;
+  src.n = (int)n;
+  src.m = (int)m;
+  src.ptr_x = static_cast<int64_t *>(area);
+  src.ptr_y = reinterpret_cast<int64_t *>(
+      static_cast<char *>(area) +
+      align256(sizeof(int64_t) * (size_t)(num_segments + 1)));
+  ptr_x = src.ptr_x;
+  ptr_y = src.ptr_y;
+  return src;
+}
+
 // Sizes of the pieces pca_knn carves out of the workspace, in carving order.
 struct KnnLayout {
   size_t x_norm = 0;  // |x| (any-dimension kernel, cosine)
   size_t sliced = 0;  // shared bounds + partial key lists of sliced segments
   size_t work_start, idx, dist, count, compact;
+  size_t ptrs = 0;    // segment pointers derived from example ids, both sides
   size_t total() const {
-    return x_norm + sliced + work_start + idx + dist + count + compact;
+    return x_norm + sliced + work_start + idx + dist + count + compact + ptrs;
   }
 };
 
@@ -123,6 +150,7 @@ KnnLayout knn_layout(int64_t n, int64_t m, int64_t d, int64_t num_segments,
   w.dist = align256(sizeof(float) * (size_t)m * (size_t)k);
   w.count = align256(sizeof(int) * (size_t)m);
   w.compact = pca::compact_workspace_bytes((int)m);
+  w.ptrs = segment_pointer_bytes(num_segments);
   return w;
 }
 
@@ -165,11 +193,15 @@ size_t radius_workspace(int64_t n, int64_t m, int64_t d, int64_t num_segments,
   bytes += align256(sizeof(int) * (size_t)m * (size_t)slots);
   bytes += align256(sizeof(int) * (size_t)m);
   bytes += pca::compact_workspace_bytes((int)m);
+  bytes += segment_pointer_bytes(num_segments);
   return bytes;
 }
 
-bool edge_flags_ok(int flags) {
-  return (flags & ~(PCA_EDGES_DROP_SELF | PCA_EDGES_X_FIRST)) == 0;
+// by_id: the entry point takes example ids in place of pointers
+bool edge_flags_ok(int flags, bool by_id = false) {
+  const int known = PCA_EDGES_DROP_SELF | PCA_EDGES_X_FIRST |
+                    (by_id ? PCA_SEGMENTS_BY_ID : 0);
+  return (flags & ~known) == 0;
 }
 
 bool nearest_dtype_ok(int dtype) {
@@ -287,6 +319,31 @@ int pca_time_next_search(void *start_event, void *stop_event) {
   return PCA_OK;
 }
 
+int pca_segment_pointers(const int64_t *ids_x, int64_t n, const int64_t *ids_y,
+                         int64_t m, int64_t num_segments, int64_t *ptr_x,
+                         int64_t *ptr_y, void *stream_) {
+  g_last_error[0] = 0;
+  if (n < 0 || m < 0 || n > kMaxRows || m > kMaxRows || num_segments < 1 ||
+      num_segments > kMaxRows)
+    return fail(PCA_ERR_INVALID_ARGUMENT,
+                "bad sizes n=%lld m=%lld num_segments=%lld", (long long)n,
+                (long long)m, (long long)num_segments);
+  if (ptr_x == nullptr || ptr_y == nullptr || (n > 0 && ids_x == nullptr) ||
+      (m > 0 && ids_y == nullptr))
+    return fail(PCA_ERR_INVALID_ARGUMENT, "ids or pointers are NULL");
+  pca::SegmentSource src;
+  src.ids_x = ids_x;
+  src.ids_y = ids_y;
+  src.n = (int)n;
+  src.m = (int)m;
+  src.ptr_x = ptr_x;
+  src.ptr_y = ptr_y;
+  return check_launch(
+      pca::launch_segment_pointers(src, (int)num_segments,
+                                   static_cast<hipStream_t>(stream_)),
+      "segment_pointers_kernel");
+}
+
 size_t pca_knn_workspace_bytes(int64_t n, int64_t m, int64_t d,
                                int64_t num_segments, int64_t k, int dtype) {
   if (num_segments < 1)
@@ -371,7 +428,7 @@ int knn_call(const void *x, const void *y, const int64_t *ptr_x,
   if (dtype != PCA_F32 && dist != nullptr)
     return fail(PCA_ERR_UNSUPPORTED,
                 "per-edge distances are returned for fp32 points only");
-  if (!edge_flags_ok(edge_flags))
+  if (!edge_flags_ok(edge_flags, true))
     return fail(PCA_ERR_INVALID_ARGUMENT, "unknown edge flags %d", edge_flags);
 
   if (n == 0 || m == 0) {
@@ -408,6 +465,10 @@ int knn_call(const void *x, const void *y, const int64_t *ptr_x,
   void *compact_ws = take(lay.compact);
   if (dist == nullptr)
     dense.dist = nullptr;
+  pca::SegmentSource src;
+  const bool by_id = (edge_flags & PCA_SEGMENTS_BY_ID) != 0 && ptr_x != nullptr;
+  if (by_id)
+    src = segments_by_id(ptr_x, ptr_y, n, m, num_segments, take(lay.ptrs));
   pca::KnnLowdConfig cfg = pca::knn_lowd_config(
       (int)d, (int)k, (int)n, (int)m, (int)num_segments, cosine != 0);
 
@@ -421,19 +482,24 @@ int knn_call(const void *x, const void *y, const int64_t *ptr_x,
     cfg.tile_queries = pca::kMfmaTileQueries;
   else if (!low_d)
     cfg.tile_queries = pca::kBlock; // any-dimension kernel: one query per lane
-  int rc = check_launch(pca::launch_plan(ptr_y, (int)m, (int)num_segments,
-                                         cfg.tile_queries, work_start, stream),
-                        "plan_kernel");
+  int rc = PCA_OK;
+  // (the low-dimensional path plans its work inside its own first launch)
+  if (!low_d)
+    rc = check_launch(pca::launch_plan(ptr_y, (int)m, (int)num_segments,
+                                       cfg.tile_queries, work_start, stream,
+                                       by_id ? &src : nullptr),
+                      "plan_kernel");
   if (rc != PCA_OK)
     return rc;
   const int bound =
       pca::plan_upper_bound((int)m, (int)num_segments, cfg.tile_queries);
   if (low_d) {
-    // the events bracket the search kernel itself, not the bound fill and
+    // the events bracket the search kernel itself, not the preparation and
     // the merge around it
     rc = check_launch(pca::launch_knn_lowd(in, (int)k, cosine != 0, cfg,
                                            work_start, lowd_scratch, dense,
-                                           timer.start, timer.stop, stream),
+                                           timer.start, timer.stop, stream,
+                                           nullptr, by_id ? &src : nullptr),
                       "knn_lowd_kernel");
     timer.stop = nullptr;
   } else if (feat) {
@@ -611,7 +677,7 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
     return fail(PCA_ERR_INVALID_ARGUMENT,
                 "max_num_neighbors must be >= 1, got %lld",
                 (long long)max_num_neighbors);
-  if (!edge_flags_ok(edge_flags))
+  if (!edge_flags_ok(edge_flags, true))
     return fail(PCA_ERR_INVALID_ARGUMENT, "unknown edge flags %d", edge_flags);
   // (the search itself skips the row; it must not count towards the limit)
   if (edge_flags & PCA_EDGES_DROP_SELF)
@@ -650,6 +716,11 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
   dense.count = ws.take<int>((size_t)m);
   dense.slots = (int)slots;
   void *compact_ws = ws.take<char>(pca::compact_workspace_bytes((int)m));
+  pca::SegmentSource src;
+  const bool by_id = (edge_flags & PCA_SEGMENTS_BY_ID) != 0 && ptr_x != nullptr;
+  if (by_id)
+    src = segments_by_id(ptr_x, ptr_y, n, m, num_segments,
+                         ws.take<char>(segment_pointer_bytes(num_segments)));
 
   // r * r in double, narrowed to the element type at the launch
   // (csrc/cuda/radius_cuda.cu:90)
@@ -659,18 +730,24 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
                       (int)n, (int)m, (int)d, (int)num_segments};
   const int per_item = matrix_cores ? pca::kRadiusMcTileQueries
                                     : pca::kRadiusQueriesPerWave;
-  int rc = check_launch(pca::launch_plan(ptr_y, (int)m, (int)num_segments,
-                                         per_item, work_start, stream),
-                        "plan_kernel");
+  int rc = PCA_OK;
+  // (the matrix-core path plans its work in the launch that packs the rows)
+  if (!matrix_cores)
+    rc = check_launch(pca::launch_plan(ptr_y, (int)m, (int)num_segments,
+                                       per_item, work_start, stream,
+                                       by_id ? &src : nullptr),
+                      "plan_kernel");
   if (rc != PCA_OK)
     return rc;
   const int bound =
       pca::plan_upper_bound((int)m, (int)num_segments, per_item);
-  timer.begin();
+  if (!matrix_cores)
+    timer.begin();
   if (matrix_cores)
     rc = check_launch(pca::launch_radius_mc(in, r2, ignore_same_index != 0,
                                             work_start, bound, packed_rows,
-                                            dense, stream),
+                                            dense, timer.start, stream,
+                                            by_id ? &src : nullptr),
                       "radius_mc_kernel");
   else if (dtype == PCA_F32)
     rc = check_launch(pca::launch_radius(in, r2, ignore_same_index != 0,
@@ -844,9 +921,11 @@ int pca_nearest(const void *x, const void *y, const int64_t *ptr_x,
     cfg = pca::nearest_lowd_config((int)d, (int)m, (int)n, (int)num_segments);
     per_item = cfg.tile_queries;
   }
-  int rc = check_launch(pca::launch_plan(ptr_x, (int)n, (int)num_segments,
-                                         per_item, work_start, stream),
-                        "plan_kernel");
+  int rc = PCA_OK;
+  if (!low_d)
+    rc = check_launch(pca::launch_plan(ptr_x, (int)n, (int)num_segments,
+                                       per_item, work_start, stream),
+                      "plan_kernel");
   if (rc != PCA_OK)
     return rc;
   if (low_d) {

@@ -256,6 +256,29 @@ plan_segments(const int64_t *__restrict__ ptr, int m, int num_segments,
     work_start[num_segments] = partial[tid];
 }
 
+// Pointers of both sides from sorted example ids, by all threads of one
+// workgroup: ptr[b] = number of rows whose id is below b.  Src is
+// launchers.hpp's SegmentSource.
+template <typename Src>
+__device__ __forceinline__ void pointers_from_ids(const Src &src,
+                                                  int num_segments) {
+  for (int b = threadIdx.x; b <= num_segments; b += blockDim.x) {
+    for (int side = 0; side < 2; ++side) {
+      const int64_t *ids = side ? src.ids_y : src.ids_x;
+      const int count = side ? src.m : src.n;
+      int lo = 0, hi = count; // first index with ids[i] >= b
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (ids[mid] < (int64_t)b)
+          lo = mid + 1;
+        else
+          hi = mid;
+      }
+      (side ? src.ptr_y : src.ptr_x)[b] = lo;
+    }
+  }
+}
+
 } // namespace pca
 
 // experiment switch: -DPCA_NO_SWIZZLE maps workgroup ids to tiles directly

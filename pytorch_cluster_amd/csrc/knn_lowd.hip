@@ -179,10 +179,11 @@ hipError_t launch_lowd_pass(const KnnLowdParams &p, const KnnLowdConfig &cfg,
 }
 
 hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
-                           const KnnLowdConfig &cfg, const int *work_start,
+                           const KnnLowdConfig &cfg, int *work_start,
                            void *scratch, const DenseResult &out,
                            hipEvent_t time_start, hipEvent_t time_stop,
-                           hipStream_t stream, int64_t *nearest_out) {
+                           hipStream_t stream, int64_t *nearest_out,
+                           const SegmentSource *src) {
   const int tiles_bound =
       plan_upper_bound(in.m, in.num_segments, cfg.tile_queries);
   KnnLowdParams p;
@@ -207,34 +208,56 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
   char *base = static_cast<char *>(scratch);
   const size_t tau_bytes = align256(sizeof(float) * (size_t)in.m);
   const size_t split_bytes = mc_split_bytes(cfg, in.n, in.d);
+  if (cfg.num_chunks > 1) {
+    p.tau = reinterpret_cast<float *>(base);
+    p.partial = reinterpret_cast<double *>(base + tau_bytes + split_bytes);
+  }
+  const float tau_start = cfg.nearest ? kNearestLimit : kKnnSentinel;
   if (cfg.matrix_cores) {
+    // one launch: pointers (when the caller passed example ids), plan, packed
+    // rows, start value of the shared bounds
     uint4 *split = reinterpret_cast<uint4 *>(base + tau_bytes);
     p.x_split = split;
+    McSetup a;
+    a.x = p.x;
+    a.n = in.n;
+    a.d_in = in.d;
+    a.out = split;
+    a.tau = p.tau;
+    a.m = in.m;
+    a.tau_value = tau_start;
+    a.ptr_y = in.ptr_y;
+    a.num_segments = in.num_segments;
+    a.per_item = cfg.tile_queries;
+    a.work_start = work_start;
+    if (src)
+      a.src = *src;
     hipError_t perr = hipErrorInvalidValue;
     switch (padded_dim(in.d)) {
     case 2:
-      perr = launch_mc_pack_rows<2>(p.x, in.n, in.d, split, stream);
+      perr = launch_mc_setup<2>(a, stream);
       break;
     case 3:
-      perr = launch_mc_pack_rows<3>(p.x, in.n, in.d, split, stream);
+      perr = launch_mc_setup<3>(a, stream);
       break;
     case 4:
-      perr = launch_mc_pack_rows<4>(p.x, in.n, in.d, split, stream);
+      perr = launch_mc_setup<4>(a, stream);
       break;
     case 8:
-      perr = launch_mc_pack_rows<8>(p.x, in.n, in.d, split, stream);
+      perr = launch_mc_setup<8>(a, stream);
       break;
     }
     if (perr != hipSuccess)
       return perr;
-  }
-  if (cfg.num_chunks > 1) {
-    float *tau = reinterpret_cast<float *>(base);
-    p.partial = reinterpret_cast<double *>(base + tau_bytes + split_bytes);
-    p.tau = tau;
-    hipLaunchKernelGGL(fill_f32_kernel, dim3((in.m + kBlock - 1) / kBlock),
-                       dim3(kBlock), 0, stream, tau, in.m,
-                       cfg.nearest ? kNearestLimit : kKnnSentinel);
+  } else {
+    const hipError_t perr =
+        launch_plan(in.ptr_y, in.m, in.num_segments, cfg.tile_queries,
+                    work_start, stream, src);
+    if (perr != hipSuccess)
+      return perr;
+    if (cfg.num_chunks > 1)
+      hipLaunchKernelGGL(fill_f32_kernel, dim3((in.m + kBlock - 1) / kBlock),
+                         dim3(kBlock), 0, stream, p.tau, in.m, tau_start);
   }
 
   if (time_start)

@@ -150,13 +150,45 @@ __device__ __forceinline__ void mc_pack_row(const float (&x)[DIM],
   }
 }
 
-// Packs every x row once per call; the search kernel's workgroups, each of
-// which streams its whole segment through LDS, then just copy.
+// Everything the search kernel needs prepared, in one launch (workgroups of
+// kPlanThreads threads over max(n, m) rows):
+//   * every x row packed once per call; the search kernel's workgroups, each
+//     of which streams its whole segment through LDS, then just copy;
+//   * the shared bounds of sliced segments set to their start value (tau);
+//   * by the first workgroup: the segment pointers when the caller passed
+//     example ids (src), and the first work item of every segment (the plan,
+//     when work_start is given).
+struct McSetup {
+  const float *x;
+  int n, d_in;
+  uint4 *out;
+  float *tau; // [m] or NULL
+  int m;
+  float tau_value;
+  const int64_t *ptr_y; // plan input (src.ptr_y when src is used)
+  int num_segments, per_item;
+  int *work_start; // NULL: no plan
+  SegmentSource src;
+};
+
 template <int DIM>
-__global__ __launch_bounds__(kBlock) void mc_pack_rows_kernel(
-    const float *__restrict__ x, int n, int d_in, uint4 *__restrict__ out) {
+__global__ __launch_bounds__(kPlanThreads) void mc_setup_kernel(McSetup a) {
   constexpr int REC = McShape<DIM>::REC;
-  const int row = blockIdx.x * kBlock + threadIdx.x;
+  __shared__ int partial[kPlanThreads];
+  if (blockIdx.x == 0 && a.work_start != nullptr) {
+    if (a.src.ids_x != nullptr) {
+      pointers_from_ids(a.src, a.num_segments);
+      __syncthreads();
+    }
+    plan_segments(a.ptr_y, a.m, a.num_segments, a.per_item, a.work_start,
+                  partial);
+  }
+  const int row = blockIdx.x * kPlanThreads + threadIdx.x;
+  if (a.tau != nullptr && row < a.m)
+    a.tau[row] = a.tau_value;
+  const float *__restrict__ x = a.x;
+  uint4 *__restrict__ out = a.out;
+  const int n = a.n, d_in = a.d_in;
   if (row >= n)
     return;
   float v[DIM];
@@ -584,18 +616,17 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
 template <int DIM>
 hipError_t launch_knn_lowd_mc_dim(const KnnLowdParams &p, int kbucket,
                                   int grid, hipStream_t stream);
-// Fills `out` (n * McShape<DIM>::REC entries) with the packed rows.
+// Fills a.out (n * McShape<DIM>::REC entries) with the packed rows, and the
+// rest of McSetup.
 template <int DIM>
-hipError_t launch_mc_pack_rows(const float *x, int n, int d_in, uint4 *out,
-                               hipStream_t stream);
-
+hipError_t launch_mc_setup(const McSetup &a, hipStream_t stream);
 #define PCA_LOWD_MC_DEFINE(DIM_)                                               \
   template <>                                                                  \
-  hipError_t launch_mc_pack_rows<DIM_>(const float *x, int n, int d_in,        \
-                                       uint4 *out, hipStream_t stream) {       \
-    hipLaunchKernelGGL((mc_pack_rows_kernel<DIM_>),                            \
-                       dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0,       \
-                       stream, x, n, d_in, out);                               \
+  hipError_t launch_mc_setup<DIM_>(const McSetup &a, hipStream_t stream) {     \
+    const int rows = a.n > a.m ? a.n : a.m;                                    \
+    hipLaunchKernelGGL((mc_setup_kernel<DIM_>),                                \
+                       dim3((rows + kPlanThreads - 1) / kPlanThreads),         \
+                       dim3(kPlanThreads), 0, stream, a);                      \
     return hipGetLastError();                                                  \
   }                                                                            \
   template <>                                                                  \

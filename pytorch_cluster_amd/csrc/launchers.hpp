@@ -30,11 +30,28 @@ struct SearchInput {
 
 // --- segments.hip ----------------------------------------------------------
 
+// Segments given as sorted example ids (one int64 per row) instead of
+// pointers: the kernel that plans the work derives the pointers first,
+// ptr[b] = first row whose id is >= b, as the reference's wrappers do with two
+// bucketize calls (torch_cluster/knn.py:75-79).
+struct SegmentSource {
+  const int64_t *ids_x = nullptr; // [n]; NULL: the caller passed pointers
+  const int64_t *ids_y = nullptr; // [m]
+  int n = 0, m = 0;
+  int64_t *ptr_x = nullptr;       // [num_segments + 1], written
+  int64_t *ptr_y = nullptr;
+};
+
 // work_start[b] = sum over b' < b of ceil(m_b' / per_item): the first work item
 // (query tile / wave task) of each segment; work_start has num_segments + 1
-// entries.
+// entries.  src: derive the pointers of both sides first (ptr_y must then be
+// src->ptr_y).
 hipError_t launch_plan(const int64_t *ptr_y, int m, int num_segments,
-                       int per_item, int *work_start, hipStream_t stream);
+                       int per_item, int *work_start, hipStream_t stream,
+                       const SegmentSource *src = nullptr);
+// The pointers alone (for the paths that plan their work elsewhere).
+hipError_t launch_segment_pointers(const SegmentSource &src, int num_segments,
+                                   hipStream_t stream);
 
 // Upper bound of work_start[num_segments] that needs no device data.
 inline int plan_upper_bound(int m, int num_segments, int per_item) {
@@ -72,13 +89,17 @@ KnnLowdConfig nearest_lowd_config(int d, int n, int m, int num_segments);
 // key lists of sliced segments).
 size_t knn_lowd_scratch_bytes(const KnnLowdConfig &cfg, int n, int m, int d,
                               int num_segments, int k);
-// cfg.nearest: `out` is unused and nearest_out [m] receives the rows.
+// Plans the work itself (work_start: num_segments + 1 entries, written; with
+// src the segment pointers in.ptr_x / in.ptr_y = src->ptr_x / ptr_y are
+// derived first) -- for the matrix-core kernel in the same launch that packs
+// the rows.  cfg.nearest: `out` is unused and nearest_out [m] receives the
+// rows.
 hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
-                           const KnnLowdConfig &cfg, const int *work_start,
+                           const KnnLowdConfig &cfg, int *work_start,
                            void *scratch, const DenseResult &out,
                            hipEvent_t time_start, hipEvent_t time_stop,
-                           hipStream_t stream,
-                           int64_t *nearest_out = nullptr);
+                           hipStream_t stream, int64_t *nearest_out = nullptr,
+                           const SegmentSource *src = nullptr);
 
 // --- knn_binned.hip --------------------------------------------------------
 
@@ -213,11 +234,16 @@ constexpr int kRadiusMcTileQueries = 128;
 bool radius_mc_supported(int d, int n, int m, int num_segments);
 // packed rows of x
 size_t radius_mc_scratch_bytes(int n, int d);
-// work_start: tiles of kRadiusMcTileQueries queries.
+// Plans the work itself, in the launch that packs the rows (work_start:
+// num_segments + 1 entries, written: tiles of kRadiusMcTileQueries queries;
+// src as for launch_knn_lowd).  time_start: recorded right before the search
+// kernel.
 hipError_t launch_radius_mc(const SearchInput &in, float r2,
-                            bool ignore_same_index, const int *work_start,
+                            bool ignore_same_index, int *work_start,
                             int tiles_bound, void *scratch,
-                            const DenseResult &out, hipStream_t stream);
+                            const DenseResult &out, hipEvent_t time_start,
+                            hipStream_t stream,
+                            const SegmentSource *src = nullptr);
 
 // --- radius.hip ------------------------------------------------------------
 

@@ -17,12 +17,17 @@ int padded_dim(int d) {
   return 8;
 }
 
+// Two launches: the preparation (segment pointers from example ids when src
+// is used, the plan, the packed rows) and the search.
 template <int DIM>
-hipError_t launch_dim(RadiusMcParams p, const float *x, uint4 *packed,
-                      int grid, hipStream_t stream) {
-  hipLaunchKernelGGL((mc_pack_rows_kernel<DIM>),
-                     dim3((p.n + kBlock - 1) / kBlock), dim3(kBlock), 0,
-                     stream, x, p.n, p.d_in, packed);
+hipError_t launch_dim(RadiusMcParams p, const McSetup &setup, int grid,
+                      hipEvent_t time_start, hipStream_t stream) {
+  const int rows = setup.n > setup.m ? setup.n : setup.m;
+  hipLaunchKernelGGL((mc_setup_kernel<DIM>),
+                     dim3((rows + kPlanThreads - 1) / kPlanThreads),
+                     dim3(kPlanThreads), 0, stream, setup);
+  if (time_start)
+    (void)hipEventRecord(time_start, stream);
   hipLaunchKernelGGL((radius_mc_kernel<DIM>), dim3(grid), dim3(kBlock), 0,
                      stream, p);
   return hipGetLastError();
@@ -55,9 +60,10 @@ size_t radius_mc_scratch_bytes(int n, int d) {
 }
 
 hipError_t launch_radius_mc(const SearchInput &in, float r2,
-                            bool ignore_same_index, const int *work_start,
+                            bool ignore_same_index, int *work_start,
                             int tiles_bound, void *scratch,
-                            const DenseResult &out, hipStream_t stream) {
+                            const DenseResult &out, hipEvent_t time_start,
+                            hipStream_t stream, const SegmentSource *src) {
   if (tiles_bound <= 0)
     return hipSuccess;
   RadiusMcParams p;
@@ -75,17 +81,29 @@ hipError_t launch_radius_mc(const SearchInput &in, float r2,
   p.work_start = work_start;
   p.out_idx = out.idx;
   p.out_count = out.count;
-  const float *x = static_cast<const float *>(in.x);
-  uint4 *packed = static_cast<uint4 *>(scratch);
+  McSetup a;
+  a.x = static_cast<const float *>(in.x);
+  a.n = in.n;
+  a.d_in = in.d;
+  a.out = static_cast<uint4 *>(scratch);
+  a.tau = nullptr;
+  a.m = in.m;
+  a.tau_value = 0.0f;
+  a.ptr_y = in.ptr_y;
+  a.num_segments = in.num_segments;
+  a.per_item = kRadiusMcTileQueries;
+  a.work_start = work_start;
+  if (src)
+    a.src = *src;
   switch (padded_dim(in.d)) {
   case 2:
-    return launch_dim<2>(p, x, packed, tiles_bound, stream);
+    return launch_dim<2>(p, a, tiles_bound, time_start, stream);
   case 3:
-    return launch_dim<3>(p, x, packed, tiles_bound, stream);
+    return launch_dim<3>(p, a, tiles_bound, time_start, stream);
   case 4:
-    return launch_dim<4>(p, x, packed, tiles_bound, stream);
+    return launch_dim<4>(p, a, tiles_bound, time_start, stream);
   case 8:
-    return launch_dim<8>(p, x, packed, tiles_bound, stream);
+    return launch_dim<8>(p, a, tiles_bound, time_start, stream);
   }
   return hipErrorInvalidValue;
 }

@@ -19,12 +19,23 @@ namespace pca {
 
 namespace {
 
-// Single workgroup: exclusive scan of ceil(m_b / per_item) over segments.
+// Single workgroup: exclusive scan of ceil(m_b / per_item) over segments;
+// before that, when the caller passed sorted example ids instead of pointers,
+// the pointers of both sides (ptr_y is then src.ptr_y).
 __global__ __launch_bounds__(kPlanThreads) void plan_kernel(
     const int64_t *__restrict__ ptr_y, int m, int num_segments, int per_item,
-    int *__restrict__ work_start) {
+    int *__restrict__ work_start, SegmentSource src) {
   __shared__ int partial[kPlanThreads];
+  if (src.ids_x != nullptr) {
+    pointers_from_ids(src, num_segments);
+    __syncthreads();
+  }
   plan_segments(ptr_y, m, num_segments, per_item, work_start, partial);
+}
+
+__global__ __launch_bounds__(kPlanThreads) void segment_pointers_kernel(
+    SegmentSource src, int num_segments) {
+  pointers_from_ids(src, num_segments);
 }
 
 // ---- compaction -----------------------------------------------------------
@@ -123,15 +134,62 @@ __global__ __launch_bounds__(kBlock) void find_self_kernel(
   }
 }
 
+// The two kernels of the short path (up to kInlineScanBlocks blocks of
+// queries): count_block_kernel = find_self_kernel + block_sum_kernel in one
+// pass (self_pos == nullptr: nothing is left out, only the sums), and a
+// scatter that adds up the sums of the blocks before it on its own.
+constexpr int kInlineScanBlocks = 2048;
+
+__global__ __launch_bounds__(kBlock) void count_block_kernel(
+    const int *__restrict__ idx, const int *__restrict__ count, int m,
+    int slots, int *__restrict__ self_pos, int *__restrict__ kept,
+    int64_t *__restrict__ block_sums) {
+  __shared__ int s_self[kCompactQueries];
+  __shared__ int s_count[kCompactQueries];
+  __shared__ int lds[kBlock];
+  const int tid = threadIdx.x;
+  const int q0 = blockIdx.x * kCompactQueries;
+  const int nq = min(kCompactQueries, m - q0);
+  int c = tid < nq ? count[q0 + tid] : 0;
+  if (self_pos != nullptr) {
+    s_self[tid] = -1;
+    s_count[tid] = c;
+    __syncthreads();
+    const int *rows = idx + (size_t)q0 * slots;
+    const int total = nq * slots;
+#pragma unroll 4
+    for (int e = tid; e < total; e += kBlock) {
+      const int ql = e / slots;
+      const int sl = e - ql * slots;
+      const int v = rows[e];
+      if (sl < s_count[ql] && v == q0 + ql)
+        s_self[ql] = sl;
+    }
+    __syncthreads();
+    if (tid < nq) {
+      c -= s_self[tid] >= 0 ? 1 : 0;
+      self_pos[q0 + tid] = s_self[tid];
+      kept[q0 + tid] = c;
+    }
+  }
+  int total;
+  block_exclusive_scan(c, lds, &total);
+  if (tid == 0)
+    block_sums[blockIdx.x] = total;
+}
+
 // count: slots to write per query (without the self slot when self_pos is
 // given).  x_first: the x row goes to the first half of `edges`.
+// inline_scan: block_offsets holds the blocks' SUMS; this block adds up the
+// ones before it and all of them (block 0 also stores the total).
 __global__ __launch_bounds__(kBlock) void scatter_kernel(
     const int *__restrict__ idx, const float *__restrict__ dist,
     const int *__restrict__ count, const int *__restrict__ self_pos, int m,
     int slots, int x_first, const int64_t *__restrict__ block_offsets,
-    const int64_t *__restrict__ num_edges, int64_t *__restrict__ edges,
-    float *__restrict__ dist_out) {
+    int64_t *__restrict__ num_edges, int64_t *__restrict__ edges,
+    float *__restrict__ dist_out, int inline_scan) {
   __shared__ int lds[kBlock];
+  __shared__ int64_t s_before[kBlock], s_all[kBlock];
   __shared__ int s_count[kCompactQueries];
   __shared__ int s_offset[kCompactQueries];
   __shared__ int s_self[kCompactQueries];
@@ -146,11 +204,35 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
   // (a position no slot has when nothing is left out)
   s_self[tid] = (self_pos && q < m && self_pos[q] >= 0) ? self_pos[q] : slots;
   __syncthreads();
+  int64_t E, base;
+  if (inline_scan) {
+    int64_t before = 0, all = 0;
+    for (int b = tid; b < (int)gridDim.x; b += kBlock) {
+      const int64_t v = block_offsets[b];
+      all += v;
+      before += b < (int)blockIdx.x ? v : 0;
+    }
+    s_before[tid] = before;
+    s_all[tid] = all;
+    __syncthreads();
+    for (int off = kBlock / 2; off >= 1; off >>= 1) {
+      if (tid < off) {
+        s_before[tid] += s_before[tid + off];
+        s_all[tid] += s_all[tid + off];
+      }
+      __syncthreads();
+    }
+    E = s_all[0];
+    base = s_before[0];
+    if (blockIdx.x == 0 && tid == 0)
+      *num_edges = E;
+  } else {
+    E = *num_edges;
+    base = block_offsets[blockIdx.x];
+  }
   if (total == 0)
     return;
 
-  const int64_t E = *num_edges;
-  const int64_t base = block_offsets[blockIdx.x];
   const int nq = min(kCompactQueries, m - q0);
   int64_t *first = x_first ? edges + E : edges;  // receives the query rows
   int64_t *second = x_first ? edges : edges + E; // receives the x rows
@@ -179,9 +261,18 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 } // namespace
 
 hipError_t launch_plan(const int64_t *ptr_y, int m, int num_segments,
-                       int per_item, int *work_start, hipStream_t stream) {
+                       int per_item, int *work_start, hipStream_t stream,
+                       const SegmentSource *src) {
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(kPlanThreads), 0, stream, ptr_y,
-                     m, num_segments, per_item, work_start);
+                     m, num_segments, per_item, work_start,
+                     src ? *src : SegmentSource{});
+  return hipGetLastError();
+}
+
+hipError_t launch_segment_pointers(const SegmentSource &src, int num_segments,
+                                   hipStream_t stream) {
+  hipLaunchKernelGGL(segment_pointers_kernel, dim3(1), dim3(kPlanThreads), 0,
+                     stream, src, num_segments);
   return hipGetLastError();
 }
 
@@ -202,6 +293,18 @@ hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
   int *self_pos = reinterpret_cast<int *>(ws);
   int *kept = reinterpret_cast<int *>(ws + align256(sizeof(int) * (size_t)m));
   const int *count = dense.count;
+  if (blocks <= kInlineScanBlocks) {
+    hipLaunchKernelGGL(count_block_kernel, dim3(blocks), dim3(kBlock), 0,
+                       stream, dense.idx, dense.count, m, dense.slots,
+                       drop_self ? self_pos : (int *)nullptr, kept,
+                       block_sums);
+    hipLaunchKernelGGL(scatter_kernel, dim3(blocks), dim3(kBlock), 0, stream,
+                       dense.idx, dense.dist, drop_self ? kept : count,
+                       drop_self ? self_pos : (const int *)nullptr, m,
+                       dense.slots, x_first ? 1 : 0, block_sums, num_edges,
+                       edges, dist_out, 1);
+    return hipGetLastError();
+  }
   if (drop_self) {
     hipLaunchKernelGGL(find_self_kernel, dim3(blocks), dim3(kBlock), 0, stream,
                        dense.idx, dense.count, m, dense.slots, self_pos, kept);
@@ -215,7 +318,7 @@ hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
                      dense.idx, dense.dist, count,
                      drop_self ? self_pos : (const int *)nullptr, m,
                      dense.slots, x_first ? 1 : 0, block_sums, num_edges,
-                     edges, dist_out);
+                     edges, dist_out, 0);
   return hipGetLastError();
 }
 

@@ -117,6 +117,42 @@ Segments resolve_segments(const at::Tensor &x, const at::Tensor &y,
   return s;
 }
 
+// Segments given as the sorted example ids of the rows (what the Python entry
+// points receive as batch_x / batch_y) with the number of examples: the
+// pointers are derived on the device, in the launch that prepares the search
+// (PCA_SEGMENTS_BY_ID), instead of by two bucketize calls before it
+// (torch_cluster/knn.py:75-79).
+Segments segments_by_id(const at::Tensor &x, const at::Tensor &y,
+                        const at::Tensor &batch_x, const at::Tensor &batch_y,
+                        int64_t batch_size) {
+  PCA_CHECK_GPU(batch_x);
+  PCA_CHECK_GPU(batch_y);
+  PCA_CHECK_INPUT(batch_x.dim() == 1 && batch_x.numel() == x.size(0));
+  PCA_CHECK_INPUT(batch_y.dim() == 1 && batch_y.numel() == y.size(0));
+  TORCH_CHECK(batch_size >= 1, "`batch_size` needs to be positive");
+  Segments s;
+  s.keep_x = batch_x.to(at::kLong).contiguous();
+  s.keep_y = batch_y.to(at::kLong).contiguous();
+  s.ptr_x = s.keep_x.data_ptr<int64_t>();
+  s.ptr_y = s.keep_y.data_ptr<int64_t>();
+  s.count = batch_size;
+  return s;
+}
+
+// For the entry points that take pointers only: the pointers of `ids` in a
+// tensor of their own (one small launch).
+void pointers_for(Segments &s, int64_t n, int64_t m, hipStream_t stream) {
+  auto both = at::empty({2, s.count + 1}, s.keep_x.options());
+  int64_t *px = both.data_ptr<int64_t>();
+  int64_t *py = px + (s.count + 1);
+  check_status(
+      pca_segment_pointers(s.ptr_x, n, s.ptr_y, m, s.count, px, py, stream));
+  s.keep_x = both;
+  s.keep_y = both;
+  s.ptr_x = px;
+  s.ptr_y = py;
+}
+
 at::Tensor finish(const at::Tensor &edges, const at::Tensor &num_edges) {
   // the only host synchronisation of the operator: the edge count sizes the
   // result (the reference synchronises in its masked_selects)
@@ -313,10 +349,15 @@ bool bins_wanted(int64_t searched, int64_t searching, int64_t num_segments,
 at::Tensor knn_search(at::Tensor x, at::Tensor y,
                       std::optional<at::Tensor> ptr_x,
                       std::optional<at::Tensor> ptr_y, int64_t k, bool cosine,
-                      int flags, int64_t num_workers = 1) {
+                      int flags, int64_t num_workers = 1,
+                      int64_t ids_examples = 0) {
+  // ids_examples > 0: ptr_x / ptr_y hold the rows' example ids, that many
+  // examples (GPU tensors only)
   // the device branch of csrc/knn.cpp:26-36
-  if (!x.device().is_cuda())
+  if (!x.device().is_cuda()) {
+    TORCH_CHECK(ids_examples == 0, "example ids are taken for GPU tensors");
     return knn_host(x, y, ptr_x, ptr_y, k, cosine, flags, num_workers);
+  }
   PCA_CHECK_GPU(x);
   PCA_CHECK_CONTIGUOUS(x);
   PCA_CHECK_INPUT(x.dim() == 2);
@@ -329,7 +370,10 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
   TORCH_CHECK(k <= PCA_KNN_MAX_K, "`k` needs to smaller than or equal to 100");
   TORCH_CHECK(k >= 1, "`k` needs to be positive");
 
-  Segments seg = resolve_segments(x, y, ptr_x, ptr_y);
+  Segments seg = ids_examples > 0
+                     ? segments_by_id(x, y, ptr_x.value(), ptr_y.value(),
+                                      ids_examples)
+                     : resolve_segments(x, y, ptr_x, ptr_y);
   DeviceScope scope(x.get_device());
   auto long_opts = x.options().dtype(at::kLong);
   const int64_t n = x.size(0), m = y.size(0), d = x.size(1);
@@ -349,6 +393,12 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
   auto num_edges = at::empty({1}, long_opts);
 
   hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
+  if (ids_examples > 0) {
+    if (binned)
+      pointers_for(seg, n, m, stream);
+    else
+      flags |= PCA_SEGMENTS_BY_ID;
+  }
   if (binned) {
     check_status(pca_knn_binned(x.data_ptr(), y.data_ptr(), seg.ptr_x,
                                 seg.ptr_y, n, m, d, seg.count, k, flags,
@@ -384,15 +434,29 @@ at::Tensor knn_edges(at::Tensor x, at::Tensor y,
                     edge_flags(drop_self, x_first));
 }
 
+// knn_edges with the segments given as the rows' sorted example ids and the
+// number of examples (the prologue of torch_cluster/knn.py:62-79 folded into
+// the launch that prepares the search).
+at::Tensor knn_batched(at::Tensor x, at::Tensor y, at::Tensor batch_x,
+                       at::Tensor batch_y, int64_t batch_size, int64_t k,
+                       bool cosine, bool drop_self, bool x_first) {
+  return knn_search(x, y, batch_x, batch_y, k, cosine,
+                    edge_flags(drop_self, x_first), 1, batch_size);
+}
+
 at::Tensor radius_search(at::Tensor x, at::Tensor y,
                          std::optional<at::Tensor> ptr_x,
                          std::optional<at::Tensor> ptr_y, double r,
                          int64_t max_num_neighbors, bool ignore_same_index,
-                         int flags, int64_t num_workers = 1) {
+                         int flags, int64_t num_workers = 1,
+                         int64_t ids_examples = 0) {
+  // (ids_examples: as for knn_search)
   // the device branch of csrc/radius.cpp:27-35
-  if (!x.device().is_cuda())
+  if (!x.device().is_cuda()) {
+    TORCH_CHECK(ids_examples == 0, "example ids are taken for GPU tensors");
     return radius_host(x, y, ptr_x, ptr_y, r, max_num_neighbors,
                        ignore_same_index, flags, num_workers);
+  }
   PCA_CHECK_GPU(x);
   PCA_CHECK_CONTIGUOUS(x);
   PCA_CHECK_INPUT(x.dim() == 2);
@@ -405,7 +469,10 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
   TORCH_CHECK(max_num_neighbors >= 1,
               "`max_num_neighbors` needs to be positive");
 
-  Segments seg = resolve_segments(x, y, ptr_x, ptr_y);
+  Segments seg = ids_examples > 0
+                     ? segments_by_id(x, y, ptr_x.value(), ptr_y.value(),
+                                      ids_examples)
+                     : resolve_segments(x, y, ptr_x, ptr_y);
   DeviceScope scope(x.get_device());
   auto long_opts = x.options().dtype(at::kLong);
   const int64_t n = x.size(0), m = y.size(0), d = x.size(1);
@@ -428,6 +495,12 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
   auto num_edges = at::empty({1}, long_opts);
 
   hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
+  if (ids_examples > 0) {
+    if (binned)
+      pointers_for(seg, n, m, stream);
+    else
+      flags |= PCA_SEGMENTS_BY_ID;
+  }
   if (binned) {
     check_status(pca_radius_binned(
         x.data_ptr(), y.data_ptr(), seg.ptr_x, seg.ptr_y, n, m, d, seg.count,
@@ -462,6 +535,16 @@ at::Tensor radius_edges(at::Tensor x, at::Tensor y,
                         bool x_first) {
   return radius_search(x, y, ptr_x, ptr_y, r, max_num_neighbors,
                        ignore_same_index, edge_flags(false, x_first));
+}
+
+// radius_edges with the segments given as example ids (see knn_batched).
+at::Tensor radius_batched(at::Tensor x, at::Tensor y, at::Tensor batch_x,
+                          at::Tensor batch_y, int64_t batch_size, double r,
+                          int64_t max_num_neighbors, bool ignore_same_index,
+                          bool x_first) {
+  return radius_search(x, y, batch_x, batch_y, r, max_num_neighbors,
+                       ignore_same_index, edge_flags(false, x_first), 1,
+                       batch_size);
 }
 
 // csrc/nearest.cpp:22-36 -> nearest_cuda (csrc/cuda/nearest_cuda.cu:68-94):
@@ -606,6 +689,14 @@ TORCH_LIBRARY(pytorch_cluster_amd, m) {
         "float r, int max_num_neighbors, bool ignore_same_index, "
         "bool x_first) -> Tensor",
         &radius_edges);
+  m.def("knn_batched(Tensor x, Tensor y, Tensor batch_x, Tensor batch_y, "
+        "int batch_size, int k, bool cosine, bool drop_self, bool x_first) "
+        "-> Tensor",
+        &knn_batched);
+  m.def("radius_batched(Tensor x, Tensor y, Tensor batch_x, Tensor batch_y, "
+        "int batch_size, float r, int max_num_neighbors, "
+        "bool ignore_same_index, bool x_first) -> Tensor",
+        &radius_batched);
   m.def("set_search_strategy(str name) -> ()", &set_search_strategy);
   m.def("get_search_strategy() -> str", &get_search_strategy);
 }

@@ -26,7 +26,7 @@ def test_header_symbols_are_exported():
     for name in sorted(declared):
         assert hasattr(lib, name), "missing export: " + name
     assert declared == set(_native.C_ABI), "ctypes table out of date"
-    assert lib.pca_abi_version() == 4
+    assert lib.pca_abi_version() == 5
 
 
 def test_capi_validation_needs_no_gpu():
