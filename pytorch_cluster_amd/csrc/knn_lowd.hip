@@ -133,9 +133,14 @@ size_t mc_split_bytes(const KnnLowdConfig &cfg, int n, int d) {
   return align256(sizeof(uint4) * (size_t)n * per_row);
 }
 
+// shared bounds [m], then the 8 counters of the work items taken per XCD
+size_t lowd_bounds_bytes(int m) {
+  return align256(sizeof(float) * (size_t)m) + 256;
+}
+
 size_t knn_lowd_scratch_bytes(const KnnLowdConfig &cfg, int n, int m, int d,
                               int num_segments, int k) {
-  size_t bytes = align256(sizeof(float) * (size_t)m); // shared bounds
+  size_t bytes = lowd_bounds_bytes(m);
   bytes += mc_split_bytes(cfg, n, d);
   if (cfg.num_chunks > 1) {
     const size_t tiles = plan_upper_bound(m, num_segments, cfg.tile_queries);
@@ -206,7 +211,14 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
   p.out_nearest = nearest_out;
   p.x_split = nullptr;
   char *base = static_cast<char *>(scratch);
-  const size_t tau_bytes = align256(sizeof(float) * (size_t)in.m);
+  const size_t tau_bytes = lowd_bounds_bytes(in.m);
+  p.claim = nullptr;
+  // tiles between two exchanges of bounds among the slices of a query
+  // (a power of two; PCA_KNN_SYNC_PERIOD overrides)
+  int period = env_int("PCA_KNN_SYNC_PERIOD", 4);
+  if (period < 1 || period > 64 || (period & (period - 1)) != 0)
+    period = 4;
+  p.sync_mask = period - 1;
   const size_t split_bytes = mc_split_bytes(cfg, in.n, in.d);
   if (cfg.num_chunks > 1) {
     p.tau = reinterpret_cast<float *>(base);
@@ -218,7 +230,15 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
     // rows, start value of the shared bounds
     uint4 *split = reinterpret_cast<uint4 *>(base + tau_bytes);
     p.x_split = split;
+    // PCA_KNN_XCD_CLAIM=1: work items are handed out XCD by XCD instead of by
+    // workgroup number.  On 8 scans of 60,000-200,000 points that cut the
+    // kernel's HBM reads from 373 MB to 112 MB per launch and made it 25 %
+    // slower, so it stays an option.
+    if (env_int("PCA_KNN_XCD_CLAIM", 0) != 0)
+      p.claim = reinterpret_cast<int *>(
+          base + align256(sizeof(float) * (size_t)in.m));
     McSetup a;
+    a.claim = p.claim;
     a.x = p.x;
     a.n = in.n;
     a.d_in = in.d;

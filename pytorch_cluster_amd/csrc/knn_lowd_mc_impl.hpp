@@ -163,6 +163,7 @@ struct McSetup {
   int n, d_in;
   uint4 *out;
   float *tau; // [m] or NULL
+  int *claim; // 8 counters to clear, or NULL
   int m;
   float tau_value;
   const int64_t *ptr_y; // plan input (src.ptr_y when src is used)
@@ -175,6 +176,8 @@ template <int DIM>
 __global__ __launch_bounds__(kPlanThreads) void mc_setup_kernel(McSetup a) {
   constexpr int REC = McShape<DIM>::REC;
   __shared__ int partial[kPlanThreads];
+  if (blockIdx.x == 0 && a.claim != nullptr && threadIdx.x < 8)
+    a.claim[threadIdx.x] = 0;
   if (blockIdx.x == 0 && a.work_start != nullptr) {
     if (a.src.ids_x != nullptr) {
       pointers_from_ids(a.src, a.num_segments);
@@ -234,13 +237,36 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
   const int half = lane >> 5;
   const int col = lane & 31;
 
+  // this workgroup's work item = (slice, tile of queries): from its own
+  // number, or taken next to those of the other workgroups on this XCD (the
+  // queue's first words pass it from thread 0 to the others: the kernel's LDS
+  // is exactly a quarter of a CU's)
   const int total_tiles = p.work_start[p.num_segments];
   if (total_tiles == 0)
     return;
-  const int chunk = blockIdx.x / total_tiles;
-  const int tile = blockIdx.x - chunk * total_tiles;
-  if (chunk >= p.num_chunks)
-    return;
+  int chunk, tile;
+  if (p.claim != nullptr) {
+    int *pass = reinterpret_cast<int *>(&queue[0][0]);
+    if (tid == 0) {
+      int c = 0;
+      pass[0] = claim_item_on_xcd(p.claim, (int)gridDim.x / p.num_chunks,
+                                  p.num_chunks, &c);
+      pass[1] = c;
+    }
+    __syncthreads();
+    // (the same in every lane: kept in scalar registers like blockIdx.x)
+    tile = __builtin_amdgcn_readfirstlane(pass[0]);
+    chunk = __builtin_amdgcn_readfirstlane(pass[1]);
+    __syncthreads(); // before the queue is used as a queue
+    if (tile < 0 || tile >= total_tiles)
+      return;
+  } else {
+    chunk = blockIdx.x / total_tiles;
+    tile = blockIdx.x - chunk * total_tiles;
+    if (chunk >= p.num_chunks)
+      return;
+  }
+  const int item = chunk * total_tiles + tile;
   const int seg = find_segment(p.work_start, p.num_segments, tile);
   const int x_begin = p.ptr_x ? (int)p.ptr_x[seg] : 0;
   const int x_end = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
@@ -526,7 +552,10 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
     __syncthreads();
     if (t + 1 < num_tiles)
       load_tile(t + 1);
-    if (p.tau)
+    // (early in a scan the bounds move fastest: tiles 0, 1, 3, 7, then every
+    // sync_mask + 1 tiles)
+    if (p.tau && (t < 8 ? (t & (t + 1)) == 0
+                        : (t & p.sync_mask) == p.sync_mask))
       sync_bounds();
     const int g_base = c_begin + t * TX;
     const int rows = min(TX, c_count - t * TX);
@@ -600,7 +629,7 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
       }
     } else {
       // sorted keys of this slice, [item][slot][query of the tile]
-      double *dst = p.partial + (size_t)blockIdx.x * k * TQ + wave * 32 + col;
+      double *dst = p.partial + (size_t)item * k * TQ + wave * 32 + col;
 #pragma unroll
       for (int j = 0; j < K; ++j) {
         const int e = j - (K - k);
