@@ -18,7 +18,7 @@ __version__ = "0.1.0"
 
 def set_search_strategy(name: str) -> None:
     """How ``knn`` / ``knn_graph`` (Euclidean, k <= 64) and ``radius`` /
-    ``radius_graph`` (at most 32 neighbours per query) search fp32 points of
+    ``radius_graph`` (at most 64 neighbours per query) search fp32 points of
     up to 3 dimensions: ``"scan"`` looks at every row of the example,
     ``"binned"`` orders the rows along a space-filling curve first and looks
     only at rows near the query, ``"auto"`` (the default) bins when its

@@ -289,7 +289,7 @@ int edge_flags(bool drop_self, bool x_first) {
 // How a search over fp32 points of up to 3 dimensions goes about it: "scan"
 // looks at every row of the segment (pca_knn, pca_radius), "binned" at the
 // rows near the query (pca_knn_binned: Euclidean, k <= 64; pca_radius_binned:
-// at most 32 neighbours per query - anything else is scanned).  Same edges
+// at most 64 neighbours per query - anything else is scanned).  Same edges
 // either way.  "auto" - the default - bins when that is expected to pay off
 // (bins_wanted).  Process-wide; the environment variable PCA_SEARCH_STRATEGY
 // sets the initial value.
@@ -346,6 +346,31 @@ bool bins_wanted(int64_t searched, int64_t searching, int64_t num_segments,
   return scan_ms > binned_ms;
 }
 
+// The two estimates of bins_wanted per operator: (scan_rate, query_us).
+struct SearchCost {
+  double scan_rate, query_us;
+};
+constexpr SearchCost kKnnCost{3e9, 2e-3};
+constexpr SearchCost kRadiusCost{1e10, 2e-3};
+constexpr SearchCost kNearestCost{1e10, 0.5e-3};
+
+// What the current strategy picks for an operator ("knn", "radius",
+// "nearest") and these sizes, when the points qualify for binning at all
+// (fp32, up to 3 dimensions, Euclidean): "scan" or "binned".
+std::string strategy_for(std::string op, int64_t searched, int64_t searching,
+                         int64_t num_segments) {
+  const SearchCost *cost = op == "knn"       ? &kKnnCost
+                           : op == "radius"  ? &kRadiusCost
+                           : op == "nearest" ? &kNearestCost
+                                             : nullptr;
+  TORCH_CHECK(cost != nullptr, "operator is 'knn', 'radius' or 'nearest', got '",
+              op, "'");
+  return bins_wanted(searched, searching, num_segments, cost->scan_rate,
+                     cost->query_us)
+             ? "binned"
+             : "scan";
+}
+
 at::Tensor knn_search(at::Tensor x, at::Tensor y,
                       std::optional<at::Tensor> ptr_x,
                       std::optional<at::Tensor> ptr_y, int64_t k, bool cosine,
@@ -381,7 +406,8 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
     return at::empty({2, 0}, long_opts);
 
   const int dtype = dtype_code(x);
-  const bool binned = bins_wanted(n, m, seg.count, 3e9, 2e-3) &&
+  const bool binned = bins_wanted(n, m, seg.count, kKnnCost.scan_rate,
+                                  kKnnCost.query_us) &&
                       dtype == PCA_F32 && !cosine && d <= 3 && k <= 64;
   const size_t ws_bytes =
       binned ? pca_knn_binned_workspace_bytes(n, m, d, seg.count, k)
@@ -481,7 +507,8 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
 
   const int dtype = dtype_code(x);
   const int64_t slots = pca_radius_slots(n, max_num_neighbors);
-  const bool binned = bins_wanted(n, m, seg.count, 1e10, 2e-3) &&
+  const bool binned = bins_wanted(n, m, seg.count, kRadiusCost.scan_rate,
+                                  kRadiusCost.query_us) &&
                       dtype == PCA_F32 && d <= 3 && slots <= 64;
   const size_t ws_bytes =
       binned ? pca_radius_binned_workspace_bytes(n, m, d, seg.count,
@@ -579,7 +606,9 @@ at::Tensor nearest(at::Tensor x, at::Tensor y, at::Tensor ptr_x,
               "nearest is not implemented for 'BFloat16'");
   // (the searched rows, y, are the ones a binned search orders)
   const bool binned =
-      bins_wanted(m, n, segments, 1e10, 0.5e-3) && dtype == PCA_F32 &&
+      bins_wanted(m, n, segments, kNearestCost.scan_rate,
+                  kNearestCost.query_us) &&
+      dtype == PCA_F32 &&
       d <= 3 && m > 0;
   const size_t ws_bytes =
       binned ? pca_nearest_binned_workspace_bytes(n, m, d, segments)
@@ -699,4 +728,7 @@ TORCH_LIBRARY(pytorch_cluster_amd, m) {
         &radius_batched);
   m.def("set_search_strategy(str name) -> ()", &set_search_strategy);
   m.def("get_search_strategy() -> str", &get_search_strategy);
+  m.def("strategy_for(str op, int searched, int searching, int num_segments) "
+        "-> str",
+        &strategy_for);
 }

@@ -48,3 +48,19 @@ def ragged_ptrs(rng, total, segments, allow_empty=True):
     if allow_empty and segments > 2:
         cuts[1] = cuts[0]  # force one empty segment
     return np.concatenate([[0], cuts, [total]]).astype(np.int64)
+
+
+def use_strategy(name):
+    """Context manager: the package's search strategy for the block."""
+    import contextlib
+    import pytorch_cluster_amd as pca
+
+    @contextlib.contextmanager
+    def scope():
+        before = pca.get_search_strategy()
+        pca.set_search_strategy(name)
+        try:
+            yield
+        finally:
+            pca.set_search_strategy(before)
+    return scope()

@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 
 import pytorch_cluster_amd as pca  # noqa: E402
 from pytorch_cluster_amd import capi, testing  # noqa: E402
-from gpu_common import (DEV, dev, gpu_knn, oracle_knn_edges,  # noqa: E402
+from gpu_common import (use_strategy, DEV, dev, gpu_knn, oracle_knn_edges,  # noqa: E402
                         ragged_ptrs)
 from helpers import (brute_force_knn_f64, check_knn_against_exact,  # noqa
                      to_set)
@@ -438,20 +438,32 @@ def test_runs_on_the_current_stream(oracle):
 
 # ---- the benchmark configurations -----------------------------------------------
 
-def test_config1_knn_graph_1024(oracle):
+# (every configuration under "scan" and under "auto", the library's default,
+# which bins the large ones)
+STRATEGIES = ["scan", "auto"]
+
+
+@pytest.mark.parametrize("strategy", STRATEGIES)
+def test_config1_knn_graph_1024(oracle, strategy):
     data = testing.uniform_cloud(0)
     x = data["x"]
-    e = pca.knn_graph(x.to(DEV), k=16, loop=False, flow='source_to_target')
+    with use_strategy(strategy):
+        e = pca.knn_graph(x.to(DEV), k=16, loop=False,
+                          flow='source_to_target')
     want = oracle.knn_graph(x.numpy(), 16, loop=False,
                             flow='source_to_target')
     assert e.shape == (2, 16384)
     assert (e.cpu().numpy() == want).all()
 
 
-def test_config2_batched_knn_graph(oracle):
+@pytest.mark.parametrize("strategy", STRATEGIES)
+@pytest.mark.parametrize("batch_size", [None, 16])
+def test_config2_batched_knn_graph(oracle, strategy, batch_size):
     data = testing.uniform_batched(0)
     x, batch = data["x"], data["batch"]
-    e = pca.knn_graph(x.to(DEV), k=20, batch=batch.to(DEV), loop=False)
+    with use_strategy(strategy):
+        e = pca.knn_graph(x.to(DEV), k=20, batch=batch.to(DEV), loop=False,
+                          batch_size=batch_size)
     want = oracle.knn_graph(x.numpy(), 20, batch.numpy(), loop=False)
     assert e.shape == (2, 16 * 4096 * 20)
     assert (e.cpu().numpy() == want).all()
@@ -501,12 +513,17 @@ def test_config4_feature_space_full_size(oracle, cosine):
     assert (cols[sample] == want[1].reshape(len(sample), 32)).all()
 
 
-def test_config5_ragged_lidar_full_size(oracle):
+@pytest.mark.parametrize("strategy", STRATEGIES)
+def test_config5_ragged_lidar_full_size(oracle, strategy):
     data = testing.lidar_scans(0)
     x, y = data["x"], data["y"]
     bx, by, B = data["batch_x"], data["batch_y"], data["batch_size"]
-    e = pca.knn(x.to(DEV), y.to(DEV), 16, bx.to(DEV), by.to(DEV),
-                batch_size=B).cpu().numpy()
+    with use_strategy(strategy):
+        if strategy == "auto":
+            assert torch.ops.pytorch_cluster_amd.strategy_for(
+                "knn", x.shape[0], y.shape[0], B) == "binned"
+        e = pca.knn(x.to(DEV), y.to(DEV), 16, bx.to(DEV), by.to(DEV),
+                    batch_size=B).cpu().numpy()
     m = y.shape[0]
     # size-independent properties at full size
     assert e.shape == (2, 16 * m)

@@ -340,3 +340,62 @@ def test_rows_searching_for_themselves_share_one_order(oracle):
     r = capi.radius_edges(xt, xt, pt, pt, 1.5, 12, True, binned=True)
     want_r = oracle.radius_op(x, x, ptr, ptr, 1.5, 12, 1, True)
     assert (r.cpu().numpy() == want_r).all()
+
+
+def test_auto_strategy_crossover():
+    """Where "auto" changes its mind: the decisions at the benchmark sizes,
+    that more rows per example never turn a binned search back into a scan,
+    and -- at sizes on both sides of every switch -- the same edges from
+    either strategy."""
+    import pytorch_cluster_amd as pca
+    pick = torch.ops.pytorch_cluster_amd.strategy_for
+    before = pca.get_search_strategy()
+    pca.set_search_strategy("auto")
+    try:
+        # small clouds are scanned, large ones binned
+        assert pick("knn", 1024, 1024, 1) == "scan"
+        assert pick("knn", 16 * 4096, 16 * 4096, 16) == "scan"
+        assert pick("radius", 8 * 16384, 8 * 16384, 8) == "scan"
+        assert pick("knn", 1033867, 258468, 8) == "binned"
+        assert pick("knn", 1000000, 1000000, 1) == "binned"
+        assert pick("radius", 1000000, 1000000, 1) == "binned"
+        assert pick("nearest", 129236, 1033867, 8) == "binned"
+        # a handful of queries against many rows: binning the rows costs more
+        # than looking at them
+        assert pick("knn", 1000000, 50, 1) == "scan"
+        for op in ("knn", "radius", "nearest"):
+            for segments in (1, 8):
+                sizes = [2 ** e for e in range(8, 24)]
+                picks = [pick(op, n * segments, n * segments, segments)
+                         for n in sizes]
+                first = picks.index("binned")
+                assert all(p == "binned" for p in picks[first:]), (op, picks)
+                assert 2 ** 12 <= sizes[first] <= 2 ** 17, (op, sizes[first])
+                # same edges just below and just above the switch
+                g = torch.Generator().manual_seed(first)
+                for n in (sizes[first - 1], sizes[first]):
+                    x = torch.rand(n * segments, 3, generator=g).to(DEV)
+                    b = (torch.arange(n * segments) // n).to(DEV)
+                    results = []
+                    for strategy in ("scan", "binned", "auto"):
+                        pca.set_search_strategy(strategy)
+                        if op == "knn":
+                            results.append(pca.knn(x, x, 5, b, b,
+                                                   batch_size=segments))
+                        elif op == "radius":
+                            results.append(pca.radius(
+                                x, x, 0.6 * n ** (-1 / 3), b, b,
+                                max_num_neighbors=10, batch_size=segments))
+                        else:
+                            results.append(pca.nearest(x, x[::3].contiguous(),
+                                                       b, b[::3].contiguous()))
+                    pca.set_search_strategy("auto")
+                    assert torch.equal(results[0], results[1])
+                    assert torch.equal(results[0], results[2])
+        # the forced strategies answer for themselves
+        pca.set_search_strategy("scan")
+        assert pick("knn", 10 ** 7, 10 ** 7, 1) == "scan"
+        pca.set_search_strategy("binned")
+        assert pick("knn", 10, 10, 1) == "binned"
+    finally:
+        pca.set_search_strategy(before)

@@ -8,7 +8,7 @@ pytestmark = pytest.mark.gpu
 
 import pytorch_cluster_amd as pca  # noqa: E402
 from pytorch_cluster_amd import testing  # noqa: E402
-from gpu_common import DEV, dev, gpu_radius, ragged_ptrs  # noqa: E402
+from gpu_common import DEV, dev, gpu_radius, ragged_ptrs, use_strategy  # noqa: E402
 from helpers import to_set  # noqa: E402
 
 
@@ -188,12 +188,14 @@ def test_operator_errors():
 
 # ---- benchmark configuration 3 -------------------------------------------------
 
-def test_config3_gaussian_mixture_radius_graph(oracle):
+@pytest.mark.parametrize("strategy", ["scan", "auto", "binned"])
+def test_config3_gaussian_mixture_radius_graph(oracle, strategy):
     data = testing.gaussian_mixture_batched(0)
     x, batch = data["x"], data["batch"]
-    e = pca.radius_graph(x.to(DEV), r=0.05, batch=batch.to(DEV),
-                         max_num_neighbors=32, loop=False,
-                         batch_size=data["batch_size"])
+    with use_strategy(strategy):
+        e = pca.radius_graph(x.to(DEV), r=0.05, batch=batch.to(DEV),
+                             max_num_neighbors=32, loop=False,
+                             batch_size=data["batch_size"])
     want = oracle.radius_graph(x.numpy(), 0.05, batch.numpy(), loop=False,
                                max_num_neighbors=32)
     assert e.shape == want.shape
