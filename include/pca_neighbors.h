@@ -1,13 +1,28 @@
 /*
  * pca_neighbors.h -- C ABI of the MI355X (gfx950) neighbour-search library.
  *
- * Plain pointers and sizes only: every pointer is DEVICE memory of the GPU
- * that is current on the calling thread unless a parameter says otherwise.
- * All entry points are asynchronous on `stream` (a hipStream_t passed as
- * void*; NULL = the default stream) and return a status code; they never
- * allocate, free or synchronise.  The library keeps no state between calls
- * (pca_last_error's text and the one-shot pca_time_next_search request are
- * per calling thread).
+ * Plain pointers and sizes only.  In the device entry points every pointer is
+ * DEVICE memory of the GPU that is current on the calling thread unless a
+ * parameter says otherwise; they are asynchronous on `stream` (a hipStream_t
+ * passed as void*; NULL = the default stream), return a status code, and
+ * never allocate or free device memory or synchronise with the host.  The
+ * *_host entry points at the end take HOST memory and return when done.
+ *
+ * What the library keeps between calls:
+ *   - per calling thread: pca_last_error's text, the one-shot
+ *     pca_time_next_search request, the last size query of the binned
+ *     searches' sort;
+ *   - per device, from the first call that needs them until the process ends:
+ *     the address of the fixed scratch of pca_knn_fixed_scratch, and -- for
+ *     the *_binned entry points with 131,072 queries or more -- one extra
+ *     stream and two events: the queries are ordered on that stream beside
+ *     the rows on the caller's (forked and joined with events inside the
+ *     call).  Calls on one device queue that part of their work under a mutex,
+ *     one after the other; PCA_BINNED_SIDE_STREAM=0 in the environment keeps
+ *     everything on the caller's stream.
+ * Stream capture: the *_binned entry points refuse a stream that is being
+ * captured into a graph (PCA_ERR_UNSUPPORTED: their sorts clear buffers with
+ * memset nodes); all other device entry points record kernels only.
  *
  * The reference (rusty1s/pytorch_cluster 1.6.3) has no C ABI: its boundary is
  * the TorchScript operator registry.  Each entry point below names the

@@ -232,6 +232,25 @@ size_t nearest_workspace(int64_t n, int64_t m, int64_t d,
   return bytes;
 }
 
+// The binned entry points sort with rocPRIM, whose clears of histograms are
+// memset nodes in a captured graph: they are refused while `stream` is being
+// captured (the scanning entry points can be captured).
+bool being_captured(hipStream_t stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+
+int refuse_capture(const char *entry) {
+  return fail(PCA_ERR_UNSUPPORTED,
+              "%s cannot be captured into a graph (its sorts clear their "
+              "buffers with memset nodes); use the scanning entry point",
+              entry);
+}
+
 int check_launch(hipError_t err, const char *what) {
   if (err != hipSuccess)
     return fail(PCA_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(err));
@@ -569,6 +588,8 @@ int pca_knn_binned(const void *x, const void *y, const int64_t *ptr_x,
                    void *workspace, size_t workspace_bytes, void *stream_) {
   g_last_error[0] = 0;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (being_captured(stream))
+    return refuse_capture("pca_knn_binned");
   SearchTimer timer(stream);
   if ((ptr_x == nullptr) != (ptr_y == nullptr))
     return fail(PCA_ERR_INVALID_ARGUMENT,
@@ -789,6 +810,8 @@ int pca_radius_binned(const void *x, const void *y, const int64_t *ptr_x,
                       void *workspace, size_t workspace_bytes, void *stream_) {
   g_last_error[0] = 0;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (being_captured(stream))
+    return refuse_capture("pca_radius_binned");
   SearchTimer timer(stream);
   if ((ptr_x == nullptr) != (ptr_y == nullptr))
     return fail(PCA_ERR_INVALID_ARGUMENT,
@@ -977,6 +1000,8 @@ int pca_nearest_binned(const void *x, const void *y, const int64_t *ptr_x,
                        size_t workspace_bytes, void *stream_) {
   g_last_error[0] = 0;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (being_captured(stream))
+    return refuse_capture("pca_nearest_binned");
   SearchTimer timer(stream);
   if ((ptr_x == nullptr) != (ptr_y == nullptr))
     return fail(PCA_ERR_INVALID_ARGUMENT,

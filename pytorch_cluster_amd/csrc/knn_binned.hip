@@ -838,13 +838,31 @@ BinnedLayout binned_layout(int n, int m, int num_segments) {
   // per task slot: descriptor (2 words), class, place in the starting order;
   // a histogram of the classes per kBlock blocks
   w.task_keys = align256(sizeof(uint32_t) * task_buffer_words(m, num_segments));
-  size_t tx = 0, ty = 0;
-  const hipError_t ex = sort_pairs(nullptr, tx, nullptr, nullptr, nullptr,
-                                   nullptr, n, num_segments, nullptr);
-  const hipError_t ey = sort_pairs(nullptr, ty, nullptr, nullptr, nullptr,
-                                   nullptr, m, num_segments, nullptr);
+  // (the sort's size queries are kept per thread for the sizes asked last:
+  // a call asks for the same layout three times -- workspace query, argument
+  // check, carving)
+  struct SortSizes {
+    int n = -1, m = -1, num_segments = -1;
+    size_t tx = 0, ty = 0;
+    bool sized = false;
+  };
+  thread_local SortSizes last;
+  if (last.n != n || last.m != m || last.num_segments != num_segments) {
+    last.n = n;
+    last.m = m;
+    last.num_segments = num_segments;
+    last.tx = last.ty = 0;
+    const hipError_t ex =
+        sort_pairs(nullptr, last.tx, nullptr, nullptr, nullptr, nullptr, n,
+                   num_segments, nullptr);
+    const hipError_t ey =
+        sort_pairs(nullptr, last.ty, nullptr, nullptr, nullptr, nullptr, m,
+                   num_segments, nullptr);
+    last.sized = ex == hipSuccess && ey == hipSuccess;
+  }
+  const size_t tx = last.tx, ty = last.ty;
   // (a failed size query leaves a size no workspace can meet)
-  const bool sized = ex == hipSuccess && ey == hipSuccess;
+  const bool sized = last.sized;
   w.sort_temp = sized ? align256(tx) : ~(size_t)0 / 2;
   // (the queries are sorted beside the rows' stream)
   w.side_temp = sized ? align256(ty) : 0;
@@ -870,8 +888,10 @@ struct Bins {
 
 // A second stream of the device: the queries are ordered there while the rows
 // are ordered on the caller's stream (both chains are short kernels that
-// leave most of the device idle).  fork / join are recorded and waited for
-// within one call, under g_lane_mutex.
+// leave most of the device idle).  The library keeps one such stream and two
+// events per device, made at the first call that needs them and held until
+// the process ends; fork / join are recorded and waited for within one call,
+// under g_lane_mutex (held only while that call queues its work).
 struct SideLane {
   hipStream_t stream = nullptr;
   hipEvent_t fork = nullptr, join = nullptr;
@@ -904,8 +924,13 @@ hipError_t side_lane(SideLane *&lane) {
     if ((err = hipEventCreateWithFlags(&made.fork, hipEventDisableTiming)) !=
             hipSuccess ||
         (err = hipEventCreateWithFlags(&made.join, hipEventDisableTiming)) !=
-            hipSuccess)
+            hipSuccess) {
+      // nothing half-made is kept
+      if (made.fork != nullptr)
+        (void)hipEventDestroy(made.fork);
+      (void)hipStreamDestroy(made.stream);
       return err;
+    }
     mine = made;
   }
   lane = &mine;
@@ -1074,19 +1099,38 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
   std::unique_lock<std::mutex> lane_lock(g_lane_mutex, std::defer_lock);
   SideLane *lane = nullptr;
   hipStream_t side = stream;
+  // Once the side stream has work of this call, the caller's stream waits for
+  // it on EVERY way out of this function -- also the failing ones: the
+  // workspace may be reused as soon as the caller's stream gets there.
+  struct Rejoin {
+    SideLane *&lane;
+    hipStream_t stream;
+    bool forked = false, joined = false;
+    hipError_t join() {
+      if (!forked || joined || lane == nullptr)
+        return hipSuccess;
+      joined = true;
+      hipError_t e = hipEventRecord(lane->join, lane->stream);
+      if (e == hipSuccess)
+        e = hipStreamWaitEvent(stream, lane->join, 0);
+      return e;
+    }
+    ~Rejoin() { (void)join(); }
+  } rejoin{lane, stream};
   auto fork = [&]() -> hipError_t {
     lane_lock.lock();
     hipError_t e = side_lane(lane);
     if (e != hipSuccess || lane == nullptr)
       return e;
     side = lane->stream;
-    return hipEventRecord(lane->fork, stream);
+    e = hipEventRecord(lane->fork, stream);
+    if (e == hipSuccess)
+      e = hipStreamWaitEvent(side, lane->fork, 0);
+    rejoin.forked = e == hipSuccess;
+    return e;
   };
   auto queries_chain = [&]() -> hipError_t {
     hipError_t e = hipSuccess;
-    if (lane != nullptr &&
-        (e = hipStreamWaitEvent(side, lane->fork, 0)) != hipSuccess)
-      return e;
     if (!self_search) {
       hipLaunchKernelGGL(morton_keys_kernel,
                          dim3((in.m + kBlock - 1) / kBlock), dim3(kBlock), 0,
@@ -1101,8 +1145,6 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
     }
     if (with_tasks)
       e = order_tasks(in, bins, task_keys, side);
-    if (e == hipSuccess && lane != nullptr)
-      e = hipEventRecord(lane->join, side);
     return e;
   };
   // (the fork is where the segment boxes are done; the longer of the two
@@ -1140,9 +1182,7 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
   }
   if ((err = hipGetLastError()) != hipSuccess)
     return err;
-  if (lane != nullptr)
-    err = hipStreamWaitEvent(stream, lane->join, 0);
-  return err;
+  return rejoin.join();
 }
 
 void fill_params(BinnedParams &p, const SearchInput &in, const Bins &bins,

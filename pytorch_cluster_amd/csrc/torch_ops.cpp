@@ -346,6 +346,17 @@ bool bins_wanted(int64_t searched, int64_t searching, int64_t num_segments,
   return scan_ms > binned_ms;
 }
 
+// A stream that is being captured into a graph takes the scanning kernels:
+// the binned entry points refuse capture.
+bool being_captured(hipStream_t stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+
 // The two estimates of bins_wanted per operator: (scan_rate, query_us).
 struct SearchCost {
   double scan_rate, query_us;
@@ -408,7 +419,10 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
   const int dtype = dtype_code(x);
   const bool binned = bins_wanted(n, m, seg.count, kKnnCost.scan_rate,
                                   kKnnCost.query_us) &&
-                      dtype == PCA_F32 && !cosine && d <= 3 && k <= 64;
+                      dtype == PCA_F32 && !cosine && d <= 3 && k <= 64 &&
+                      !being_captured(c10::hip::getCurrentHIPStream(
+                                          x.get_device())
+                                          .stream());
   const size_t ws_bytes =
       binned ? pca_knn_binned_workspace_bytes(n, m, d, seg.count, k)
              : pca_knn_workspace_bytes(n, m, d, seg.count, k, dtype);
@@ -509,7 +523,10 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
   const int64_t slots = pca_radius_slots(n, max_num_neighbors);
   const bool binned = bins_wanted(n, m, seg.count, kRadiusCost.scan_rate,
                                   kRadiusCost.query_us) &&
-                      dtype == PCA_F32 && d <= 3 && slots <= 64;
+                      dtype == PCA_F32 && d <= 3 && slots <= 64 &&
+                      !being_captured(c10::hip::getCurrentHIPStream(
+                                          x.get_device())
+                                          .stream());
   const size_t ws_bytes =
       binned ? pca_radius_binned_workspace_bytes(n, m, d, seg.count,
                                                  max_num_neighbors)
@@ -608,8 +625,9 @@ at::Tensor nearest(at::Tensor x, at::Tensor y, at::Tensor ptr_x,
   const bool binned =
       bins_wanted(m, n, segments, kNearestCost.scan_rate,
                   kNearestCost.query_us) &&
-      dtype == PCA_F32 &&
-      d <= 3 && m > 0;
+      dtype == PCA_F32 && d <= 3 && m > 0 &&
+      !being_captured(
+          c10::hip::getCurrentHIPStream(x.get_device()).stream());
   const size_t ws_bytes =
       binned ? pca_nearest_binned_workspace_bytes(n, m, d, segments)
              : pca_nearest_workspace_bytes(n, m, d, segments, dtype);

@@ -103,3 +103,49 @@ def test_more_than_three_dimensions_are_refused():
     x = torch.rand(100, 4, device=DEV)
     with pytest.raises(RuntimeError, match="binned search"):
         capi.nearest_rows(x, x, None, None, binned=True)
+
+
+def test_graph_capture_takes_the_scanning_kernel():
+    """A stream that is being captured never gets the binned search (its
+    sorts would record memset nodes): the operator scans instead, the C entry
+    point says so.  Replays give the eager result every time."""
+    import pytorch_cluster_amd as pca
+    from pytorch_cluster_amd import capi
+    from pytorch_cluster_amd._native import capi as lib
+    g = torch.Generator().manual_seed(3)
+    n, m = 150000, 90000
+    x = torch.rand(n, 3, generator=g).to(DEV)
+    y = torch.rand(m, 3, generator=g).to(DEV)
+    ptr_x = torch.tensor([0, 70000, n], device=DEV)
+    ptr_y = torch.tensor([0, 40000, m], device=DEV)
+    before = pca.get_search_strategy()
+    pca.set_search_strategy("binned")
+    try:
+        op = torch.ops.torch_cluster.nearest
+        want = op(x, y, ptr_x, ptr_y)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = op(x, y, ptr_x, ptr_y)
+            # the C entry point on the capturing stream: refused, nothing
+            # recorded
+            edges, num_edges, _d, _ws = None, None, None, None
+            ws = torch.empty(lib.pca_nearest_binned_workspace_bytes(n, m, 3, 2),
+                             dtype=torch.uint8, device=DEV)
+            res = torch.empty(n, dtype=torch.long, device=DEV)
+            rc = lib.pca_nearest_binned(
+                capi._dev_ptr(x), capi._dev_ptr(y), capi._dev_ptr(ptr_x),
+                capi._dev_ptr(ptr_y), n, m, 3, 2, capi._dev_ptr(res),
+                capi._dev_ptr(ws), ws.numel(),
+                capi._stream_handle(None, x.device))
+            assert rc == -5 and b"captured" in lib.pca_last_error()
+        for _ in range(3):
+            out.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, want)
+            # (eager work between the replays)
+            assert torch.equal(op(x, y, ptr_x, ptr_y), want)
+    finally:
+        pca.set_search_strategy(before)
