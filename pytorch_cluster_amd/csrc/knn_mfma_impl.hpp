@@ -8,7 +8,8 @@
 //     t = w - 2 x.y,      w = fl(|x|^2) (1 - eps),
 // the dot product of the augmented rows (x, w) and (-2 y, 1).  Every fp32
 // operand v is split into two bf16 numbers, v = hi + lo + r with
-// |r| <= 2^-18 |v| (bf16 keeps the exponent range of fp32), and the products
+// |lo| <= 2^-8 |v| and |r| <= 2^-17 |v| (the worst cases over all 2^23
+// mantissas; bf16 keeps the exponent range of fp32), and the products
 // hi*hi + hi*lo + lo*hi of 16 components at a time are one
 // v_mfma_f32_32x32x16_bf16 each (exact products, fp32 accumulation): 32
 // candidates x 32 queries x 16 components in 8 passes, where the fp32 matrix
@@ -17,10 +18,15 @@
 //     cut = thresh (1 + eps) - fl(|y|^2) (1 - eps)   (rounded up),
 // so the SIGN of a result says whether the candidate can still have an exact
 // distance below thresh.  Error budget, relative to |x|^2 + |y|^2 + thresh:
-// the dropped lo*lo products and the split residuals 2^-16.4; accumulating
+// a product x_c y_c misses lo*lo (2^-16 |x_c y_c|) and the residuals
+// (2 x 2^-17), all of one sign when y is close to x: 2^-15 |x_c y_c| each,
+// 2^-15 (|x|^2 + |y|^2) for -2 x.y, and 2^-17 |x|^2 for w; accumulating
 // 3 d + 4 terms, each step within 2^-23 of the running magnitude (which stays
 // below 2 (|x|^2 + |y|^2) + thresh), (3 d + 4) 2^-22; norms and the exact
-// chain (d + 2) 2^-24 each.  eps = 2^-15 + (3 d + 8) 2^-21 covers twice that.
+// chain (d + 2) 2^-24 each: 2^-15 + 2^-17 + (3 d + 4) 2^-22 + (d + 2) 2^-23.
+// eps = 2^-14 + (3 d + 8) 2^-21 is 1.6 times that or more for every d
+// (tests/test_filter_bounds.py holds the inequality against rows whose
+// mantissas maximise the split's error, y equal to x).
 // Rows whose squared norm is not a moderate finite number enter with zero
 // coordinates and w = -1e38 (always looked at; an infinity would meet a zero
 // part of another operand and turn into NaN), padding rows with a huge
@@ -119,7 +125,7 @@ template <int NB> struct MfmaShape {
 };
 
 __host__ __device__ __forceinline__ double mfma_filter_eps(int d) {
-  return 1.0 / 32768.0 + (double)(3 * d + 8) * (1.0 / 2097152.0);
+  return 1.0 / 16384.0 + (double)(3 * d + 8) * (1.0 / 2097152.0);
 }
 
 __device__ __forceinline__ float mfma_filter_cut(float thresh, float ysq,

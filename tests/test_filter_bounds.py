@@ -165,3 +165,75 @@ def test_scales(case):
         x = np.repeat(base, 30, 0) * (1 + 1e-6 * rng.standard_normal((300, d)))
         y = base * (1 + 1e-6 * rng.standard_normal((10, d)))
     check(x, y)
+
+
+# ---- the split-bf16 filter of the exact matrix-core kernel --------------------
+# (pytorch_cluster_amd/csrc/knn_mfma_impl.hpp): t = w - 2 x.y from the
+# products hi*hi + hi*lo + lo*hi of operands split into two bf16 numbers,
+# w = fl(|x|^2) (1 - eps), cut = thresh (1 + eps) - fl(|y|^2) (1 - eps).  A pair
+# whose exact distance is below thresh must come out with t < cut.
+
+def bf16(v):
+    """fp32 -> bf16, nearest-even, as fp32 values."""
+    u = np.asarray(v, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7fff + ((u >> 16) & 1)) >> 16) << 16
+    return r.astype(np.uint32).view(np.float32)
+
+
+def split(v):
+    hi = bf16(v)
+    lo = bf16((np.asarray(v, dtype=np.float32) - hi).astype(np.float32))
+    return hi.astype(np.float64), lo.astype(np.float64)
+
+
+def mfma_eps(d):
+    return 2.0 ** -14 + (3 * d + 8) * 2.0 ** -21
+
+
+def worst_split_mantissas(count):
+    """fp32 numbers in [1, 2) whose split loses the most in a product with
+    themselves: v^2 - (hi^2 + 2 hi lo) largest."""
+    m = np.arange(0, 1 << 23, 7, dtype=np.uint32)
+    v = (m | np.uint32(0x3f800000)).view(np.float32)
+    hi, lo = split(v)
+    loss = v.astype(np.float64) ** 2 - (hi * hi + 2.0 * hi * lo)
+    return v[np.argsort(loss / v.astype(np.float64) ** 2)[-count:]]
+
+
+@pytest.mark.parametrize("d", [9, 16, 40, 128])
+def test_split_bf16_filter_keeps_near_duplicates(d):
+    rng = np.random.default_rng(d)
+    worst = worst_split_mantissas(4096)
+    n = 200
+    x = rng.choice(worst, (n, d)) * 2.0 ** rng.integers(-3, 4, (n, 1))
+    x = x.astype(np.float32)
+    # queries: the rows themselves, and rows a few ulps away
+    y = np.concatenate([x[:50], np.nextafter(x[50:100], np.float32(4.0))])
+    eps = mfma_eps(d)
+    e = reference_distances(x, y)                         # [m, n]
+    xsq = np.zeros(n, dtype=np.float32)
+    for c in range(d):
+        xsq = (x[:, c].astype(np.float64) ** 2 + xsq).astype(np.float32)
+    ysq = np.zeros(len(y), dtype=np.float32)
+    for c in range(d):
+        ysq = (y[:, c].astype(np.float64) ** 2 + ysq).astype(np.float32)
+    w = (xsq * np.float32(1.0 - eps)).astype(np.float32)
+    wh, wl = split(w)
+    xh, xl = split(x)
+    yh, yl = split((-2.0 * y).astype(np.float32))
+    # exact sums of the products the matrix cores form (no accumulation error)
+    t = (wh + wl)[None, :] + yh @ xh.T + yh @ xl.T + yl @ xh.T
+    # thresh just above the exact distance: the pair must be looked at
+    thresh = np.nextafter(e.astype(np.float32), np.float32(np.inf)).astype(
+        np.float64)
+    cut = thresh * (1.0 + eps) - ysq.astype(np.float64)[:, None] * (1.0 - eps)
+    scale = xsq.astype(np.float64)[None, :] + ysq.astype(np.float64)[:, None] \
+        + thresh
+    # what fp32 accumulation of the 3 d + 4 terms may still add
+    room = (3 * d + 4) * 2.0 ** -22 * scale
+    assert (t + room < cut).all()
+    # and the case is as hard as meant: for y = x the split alone takes more
+    # than half of the 2^-15 (|x|^2 + |y|^2) its analysis allows
+    used = (t - (e - ysq.astype(np.float64)[:, None]
+                 - eps * xsq.astype(np.float64)[None, :])) / (2.0 ** -15 * scale)
+    assert 0.5 < used[:50, :50].diagonal().max() <= 1.0
