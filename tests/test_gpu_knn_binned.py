@@ -183,6 +183,34 @@ def test_queries_ordered_beside_the_rows(monkeypatch):
         assert torch.equal(capi.nearest_rows(x, y, px, py, binned=True), want)
 
 
+def test_crowded_cells_and_many_segments():
+    """What the ordering of the rows has to cope with: most rows in a handful of
+    cells (duplicates, a dense clump beside a sparse cloud), more segments
+    than rows per segment, a single row."""
+    rng = np.random.default_rng(21)
+    clump = np.repeat(rng.random((5, 3)), 3000, axis=0)
+    clump += 1e-6 * rng.standard_normal(clump.shape)
+    x = np.concatenate([clump, rng.random((5000, 3)) * 50.0,
+                        np.repeat(rng.random((1, 3)), 4000, axis=0)])
+    x = x[rng.permutation(len(x))].astype(np.float32)
+    y = x[::3].copy()
+    a, da = capi.knn_edges(dev(x), dev(y), None, None, 9, want_dist=True)
+    b, db = capi.knn_edges(dev(x), dev(y), None, None, 9, want_dist=True,
+                           binned=True)
+    assert torch.equal(a, b) and torch.equal(da.view(torch.int32),
+                                             db.view(torch.int32))
+    # 700 segments of ~30 rows, some empty
+    n = 21000
+    x = rng.random((n, 3)).astype(np.float32)
+    ptr = ragged_ptrs(rng, n, 700)
+    a, _ = capi.knn_edges(dev(x), dev(x), dev(ptr), dev(ptr), 4)
+    b, _ = capi.knn_edges(dev(x), dev(x), dev(ptr), dev(ptr), 4, binned=True)
+    assert torch.equal(a, b)
+    one = dev(x[:1])
+    b, _ = capi.knn_edges(one, one, None, None, 3, binned=True)
+    assert b.cpu().tolist() == [[0], [0]]
+
+
 @pytest.mark.parametrize("m", [1, 32, 33, 8192, 8224, 131071, 131072,
                                196608, 196640])
 def test_task_counts_at_the_edges(m):
