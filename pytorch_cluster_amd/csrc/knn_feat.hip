@@ -141,7 +141,9 @@ __global__ __launch_bounds__(kBlock) void feat_rows_kernel(
   if (threadIdx.x == 0) {
     for (int w = 1; w < kBlock / kWave; ++w)
       big = part[w] > big ? part[w] : big;
-    if (big != 0)
+    // (one word for the whole call: only workgroups that raise it go there)
+    if (big != 0 && big > __hip_atomic_load(&g->max_bits, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT))
       atomicMax(&g->max_bits, big);
   }
 }

@@ -96,8 +96,11 @@ KnnLowdConfig knn_lowd_config(int /*d*/, int k, int n, int m,
   // ragged segments, but slices of at least ~4 LDS tiles on average -- every
   // slice pays the start-up phase of its candidate lists again.
   const int tiles = plan_upper_bound(m, num_segments, cfg.tile_queries);
-  // (about 6,000 items measure best for the matrix-core kernel, whose
-  // workgroups hold half as many queries)
+  // (about 6,000 items for the matrix-core kernel, whose workgroups hold
+  // half as many queries.  On 8 scans of 60,000-200,000 points 2, 3 and 4
+  // slices run equally fast -- 2.77 / 2.76 / 2.77 ms; 2.83 / 2.87 / 2.94 ms with
+  // 5 / 6 / 8 --, but with 2 the slices outgrow the L2s: 443 MB read + 119 MB
+  // written per launch against 312 + 175 MB with 4)
   const int target = cfg.matrix_cores ? 6144 : 8192;
   const int want = (target + tiles - 1) / tiles;
   const int by_length = (n / num_segments) / (4 * kLowdTileX);
