@@ -42,7 +42,9 @@
  *              contiguous [2, E] matrix at its start: edges[0 .. E) are the
  *              query (y) rows, edges[E .. 2E) the matching x rows, global row
  *              numbers, grouped by ascending query row.
- *   num_edges  one int64 on the device that receives E.
+ *   num_edges  one int64 that receives E: device memory, or pinned host
+ *              memory (the library only ever writes it, from a kernel; a
+ *              caller that waits for the stream then reads E without a copy).
  *   workspace  scratch of at least the size the matching *_workspace_bytes()
  *              call returns, 256-byte aligned.
  *   n, m < 2^31 - 1.

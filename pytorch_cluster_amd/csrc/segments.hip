@@ -95,8 +95,12 @@ __global__ __launch_bounds__(kPlanThreads) void scan_block_sums_kernel(
     block_sums[i] = run;
     run += v;
   }
-  if (tid == kPlanThreads - 1)
+  // (the total also behind the offsets: the scatter reads it from there, so
+  // that num_edges is only ever written -- it may be host memory)
+  if (tid == kPlanThreads - 1) {
     *num_edges = partial[tid];
+    block_sums[num_blocks] = partial[tid];
+  }
 }
 
 // Both kernels below walk the slot rows of a block of queries as ONE flat
@@ -227,7 +231,7 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
     if (blockIdx.x == 0 && tid == 0)
       *num_edges = E;
   } else {
-    E = *num_edges;
+    E = block_offsets[gridDim.x];
     base = block_offsets[blockIdx.x];
   }
   if (total == 0)

@@ -153,10 +153,21 @@ void pointers_for(Segments &s, int64_t n, int64_t m, hipStream_t stream) {
   s.ptr_y = py;
 }
 
-at::Tensor finish(const at::Tensor &edges, const at::Tensor &num_edges) {
+// The edge count in pinned host memory (PyTorch keeps such blocks for reuse):
+// the kernel that knows E writes it there, and the operator waits for the
+// stream instead of queueing a copy behind it.
+at::Tensor edge_count_slot() {
+  return at::empty({1}, at::TensorOptions().dtype(at::kLong).pinned_memory(
+                            true));
+}
+
+at::Tensor finish(const at::Tensor &edges, const at::Tensor &num_edges,
+                  hipStream_t stream) {
   // the only host synchronisation of the operator: the edge count sizes the
   // result (the reference synchronises in its masked_selects)
-  const int64_t E = num_edges.item<int64_t>();
+  TORCH_CHECK(hipStreamSynchronize(stream) == hipSuccess,
+              "hipStreamSynchronize failed");
+  const int64_t E = *num_edges.data_ptr<int64_t>();
   at::Tensor out = edges.narrow(0, 0, 2 * E).view({2, E});
   // (a view keeps the whole slot buffer alive: a result that fills less than
   // half of it gets storage of its own, like the reference's [2, E])
@@ -430,7 +441,7 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
   auto workspace =
       at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
   auto edges = at::empty({2 * m * k}, long_opts);
-  auto num_edges = at::empty({1}, long_opts);
+  auto num_edges = edge_count_slot();
 
   hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
   if (ids_examples > 0) {
@@ -445,14 +456,14 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
                                 edges.data_ptr<int64_t>(),
                                 num_edges.data_ptr<int64_t>(), nullptr,
                                 workspace.data_ptr(), ws_bytes, stream));
-    return finish(edges, num_edges);
+    return finish(edges, num_edges, stream);
   }
   check_status(pca_knn(x.data_ptr(), y.data_ptr(), seg.ptr_x, seg.ptr_y, n, m,
                        d, seg.count, k, cosine ? 1 : 0, dtype, flags,
                        edges.data_ptr<int64_t>(),
                        num_edges.data_ptr<int64_t>(), nullptr,
                        workspace.data_ptr(), ws_bytes, stream));
-  return finish(edges, num_edges);
+  return finish(edges, num_edges, stream);
 }
 
 at::Tensor knn(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
@@ -536,7 +547,7 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
   auto workspace =
       at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
   auto edges = at::empty({2 * m * slots}, long_opts);
-  auto num_edges = at::empty({1}, long_opts);
+  auto num_edges = edge_count_slot();
 
   hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
   if (ids_examples > 0) {
@@ -551,7 +562,7 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
         r, max_num_neighbors, ignore_same_index ? 1 : 0, flags,
         edges.data_ptr<int64_t>(), num_edges.data_ptr<int64_t>(),
         workspace.data_ptr(), ws_bytes, stream));
-    return finish(edges, num_edges);
+    return finish(edges, num_edges, stream);
   }
   check_status(pca_radius(x.data_ptr(), y.data_ptr(), seg.ptr_x, seg.ptr_y, n,
                           m, d, seg.count, r, max_num_neighbors,
@@ -559,7 +570,7 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
                           edges.data_ptr<int64_t>(),
                           num_edges.data_ptr<int64_t>(), workspace.data_ptr(),
                           ws_bytes, stream));
-  return finish(edges, num_edges);
+  return finish(edges, num_edges, stream);
 }
 
 at::Tensor radius(at::Tensor x, at::Tensor y, std::optional<at::Tensor> ptr_x,
