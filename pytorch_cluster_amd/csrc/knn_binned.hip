@@ -794,6 +794,33 @@ hipError_t sort_pairs(void *temp, size_t &temp_bytes, const uint32_t *keys_in,
       (unsigned int)count, 0u, bits, stream, false);
 }
 
+// Tasks in a row that one XCD takes, as a power of two: long runs keep what a
+// task fetches in the L2 its neighbours fill (256 in a row: 258 MB fetched by
+// the search kernel of the 1 M-point workload, 8 in a row: 594 MB, at the
+// same speed), but every XCD needs a few runs for its share of the long tasks
+// at the front of the order.  PCA_BINNED_XCD_RUN_LOG2 overrides.
+int xcd_run_log2(int tasks) {
+  static const int fixed = [] {
+    const char *text = std::getenv("PCA_BINNED_XCD_RUN_LOG2");
+    if (!text)
+      return -1;
+    const int v = std::atoi(text);
+    return v < 0 ? 0 : (v > 12 ? 12 : v);
+  }();
+  if (fixed >= 0)
+    return fixed;
+  int log2 = 3;
+  while (log2 < 8 && (size_t)(8 << (log2 + 1)) * 3 <= (size_t)tasks)
+    ++log2;
+  return log2;
+}
+
+// Workgroups of a search on matrix cores: whole runs on each of the 8 XCDs.
+int xcd_run_grid(int tasks) {
+  const int unit = 8 << xcd_run_log2(tasks);
+  return (tasks + unit - 1) / unit * unit;
+}
+
 // Task slots for `blocks` blocks of 32 queries: one each, and half as many
 // again for the parts of split blocks - while the blocks are not many more
 // than the waves the device holds at once (256 CUs x 4 SIMDs x 4 waves).  With
@@ -882,7 +909,8 @@ struct Bins {
   const int2 *task_desc;
   const uint32_t *task_order;
   int task_slots; // slots of the order
-  int task_grid;  // workgroups that cover them
+  int task_grid;  // workgroups that cover them: whole runs of
+                  // 2^xcd_run_log2(task_slots) tasks on each of 8 XCDs
   int code_bits;
 };
 
@@ -984,8 +1012,7 @@ hipError_t order_tasks(const SearchInput &in, Bins &bins, uint32_t *task_keys,
   bins.task_desc = t.desc;
   bins.task_order = t.order;
   bins.task_slots = t.slots;
-  // (the search kernels' grid: whole runs of 8 tasks on each of 8 XCDs)
-  bins.task_grid = (t.slots + 63) / 64 * 64;
+  bins.task_grid = xcd_run_grid(t.slots);
   bins.code_bits = p.code_bits;
   return hipGetLastError();
 }
@@ -1211,6 +1238,7 @@ void fill_params(BinnedParams &p, const SearchInput &in, const Bins &bins,
   p.task_order = bins.task_order;
   p.task_desc = bins.task_desc;
   p.task_slots = bins.task_slots;
+  p.xcd_run_log2 = xcd_run_log2(bins.task_slots);
   p.code_bits = bins.code_bits;
 }
 
@@ -1331,11 +1359,12 @@ hipError_t launch_radius_binned(const SearchInput &in, float r2,
     p.wave_start = bins.half_start;
   const int waves = plan_upper_bound(in.m, in.num_segments, per_task);
   const int grid = (waves + kBlock / kWave - 1) / (kBlock / kWave);
+  p.xcd_run_log2 = xcd_run_log2(waves); // (tasks in curve order, no slots)
 #define PCA_BINNED_LAUNCH(K_)                                                  \
   do {                                                                         \
     if (matrix_cores)                                                          \
       hipLaunchKernelGGL((radius_binned_mc_kernel<K_>),                        \
-                         dim3((waves + 63) / 64 * 64), dim3(kBinMcBlock), 0,   \
+                         dim3(xcd_run_grid(waves)), dim3(kBinMcBlock), 0,   \
                          stream, p, r2, same);                                 \
     else                                                                       \
       hipLaunchKernelGGL((radius_binned_kernel<K_>), dim3(grid), dim3(kBlock), \
@@ -1343,7 +1372,7 @@ hipError_t launch_radius_binned(const SearchInput &in, float r2,
   } while (0)
 #define PCA_BINNED_LAUNCH_WIDE(K_)                                             \
   hipLaunchKernelGGL((radius_binned_mc_kernel<K_>),                            \
-                     dim3((waves + 63) / 64 * 64), dim3(kBinMcBlock), 0,       \
+                     dim3(xcd_run_grid(waves)), dim3(kBinMcBlock), 0,       \
                      stream, p, r2, same)
   if (out.slots <= 8)
     PCA_BINNED_LAUNCH(8);

@@ -51,6 +51,7 @@ struct BinnedParams {
   const uint32_t *task_order; // task slots, the longest tasks first
   const int2 *task_desc;      // per slot: first query position, queries
   int task_slots;             // entries of task_order
+  int xcd_run_log2;           // log2 of the tasks in a row that one XCD takes
   int code_bits;              // bits of the curve code inside a key
   const Box *box;           // of every tile
   const int *group_start;   // first group of tiles of every segment
@@ -279,16 +280,21 @@ __device__ __forceinline__ void bin_box_of_lane(const Box &held, int src,
 // (`extra` slots; `*extra_used` starts at 0).
 //
 // Starting order: the used extra slots first (parts of the longest tasks),
-// then the blocks by the octave of their span, widest first, and inside an
-// octave in curve order: tasks of about the same length keep their neighbours
-// next to them, and neighbours look at the same tiles.  Unused slots come
-// last (their waves leave at once).  It is a counting sort in two launches:
-// task_span_kernel leaves every block's class and a histogram of the classes
-// per workgroup of kBlock blocks, task_order_kernel turns them into places.
-constexpr int kTaskClasses = 64; // octaves 0..32, 33 = unused block, rest empty
+// then the blocks by the class of their span - three octaves to a class,
+// widest first - and inside a class in curve order: the long tasks start
+// early, and tasks keep their neighbours next to them, which look at the same
+// tiles.  (One octave to a class orders the lengths more finely and ends no
+// sooner, but neighbours along the curve then alternate between two or three
+// classes, every class sweeps the whole cloud, and the search kernel of the
+// 1 M-point LiDAR-like workload fetched 594 MB instead of 258 MB.)  Unused
+// slots come last (their waves leave at once).  It is a counting sort in two
+// launches: task_span_kernel leaves every block's class and a histogram of
+// the classes per workgroup of kBlock blocks, task_order_kernel turns them
+// into places.
+constexpr int kTaskClasses = 64; // classes 0..11, 33 = unused block, rest empty
 
 __device__ __forceinline__ uint32_t bin_task_class(uint32_t span) {
-  return span != 0 ? (uint32_t)__builtin_clz(span) : 32u;
+  return span != 0 ? (uint32_t)__builtin_clz(span) / 3u : 11u;
 }
 
 // cls: [bound] class per block; hist: [workgroups][kTaskClasses].
@@ -408,12 +414,14 @@ __global__ __launch_bounds__(kBlock) void task_order_kernel(
 }
 
 // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: runs
-// of 8 consecutive tasks (neighbours along the curve, which fetch the same
-// tiles) go to the same XCD, one after the other.  Maps a workgroup number to
-// its task's place in the order; grids are whole multiples of 64.
-__device__ __forceinline__ int bin_xcd_run(int workgroup) {
+// of 2^run_log2 consecutive tasks (neighbours along the curve, which fetch the
+// same tiles) go to the same XCD, one after the other.  Maps a workgroup
+// number to its task's place in the order; grids are whole multiples of
+// 8 << run_log2.
+__device__ __forceinline__ int bin_xcd_run(int workgroup, int run_log2) {
   const int local = workgroup >> 3;
-  return (((local >> 3) * 8 + (workgroup & 7)) << 3) | (local & 7);
+  return ((((local >> run_log2) << 3) + (workgroup & 7)) << run_log2) |
+         (local & ((1 << run_log2) - 1));
 }
 
 // Waves work on their own (no barrier): a workgroup is one wave, so that its
@@ -446,7 +454,7 @@ knn_binned_mc_kernel(BinnedParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int half = lane >> 5;
   const int col = lane & 31;
-  const int ordered = bin_xcd_run((int)blockIdx.x);
+  const int ordered = bin_xcd_run((int)blockIdx.x, p.xcd_run_log2);
   if (ordered >= p.task_slots)
     return; // (the grid is rounded up to whole runs)
   const int slot = (int)p.task_order[ordered];
@@ -506,20 +514,27 @@ knn_binned_mc_kernel(BinnedParams p) {
 
   // What the two lanes of a query tell each other about its final k-th
   // distance (see knn_lowd_mc_impl.hpp; equality admitted).
-  auto partner_bounds = [&]() __attribute__((always_inline)) {
-    const float own = key_dist(best[K - 1]);
-    const auto both = __builtin_amdgcn_permlane32_swap(
-        __float_as_uint(own), __float_as_uint(own), false, false);
-    float partner = __uint_as_float(half ? both[0] : both[1]);
+  // this lane's ceil(k/2)-th smallest distance so far (kLimit for k = 1)
+  auto own_mid = [&]() __attribute__((always_inline)) {
+    float mid = kLimit;
     if (K >= 2) {
       const int c = k >> 1;
-      float mid = kLimit;
 #pragma unroll
       for (int cc = (K >= 8 ? K / 2 - 4 : 0); cc <= K / 2; ++cc)
         if (cc >= 1 && cc == c) {
           asm volatile(""); // (keeps this a branch)
           mid = key_dist(best[K - 1 - cc]);
         }
+    }
+    return mid;
+  };
+  auto partner_bounds = [&]() __attribute__((always_inline)) {
+    const float own = key_dist(best[K - 1]);
+    const auto both = __builtin_amdgcn_permlane32_swap(
+        __float_as_uint(own), __float_as_uint(own), false, false);
+    float partner = __uint_as_float(half ? both[0] : both[1]);
+    if (K >= 2) {
+      const float mid = own_mid();
       const auto mids = __builtin_amdgcn_permlane32_swap(
           __float_as_uint(mid), __float_as_uint(mid), false, false);
       const float partner_mid = __uint_as_float(half ? mids[0] : mids[1]);
@@ -607,7 +622,13 @@ knn_binned_mc_kernel(BinnedParams p) {
       ++qn;
     }
     ++scanned;
-    if (scanned % kBinRing == 0)
+    // every kBinRing tiles, and after the first, second and fourth tile of
+    // the task: until the lists are full every row passes the filter, and
+    // with a first bound after 32 rows instead of 256 the filter passes half
+    // as many rows of the seed tiles (the insertions, which dominate, stay:
+    // the same time on LiDAR-like clouds, 3 % less on uniform ones)
+    if (scanned % kBinRing == 0 ||
+        (scanned < kBinRing && (scanned & (scanned - 1)) == 0))
       drain();
   };
 
@@ -762,7 +783,7 @@ radius_binned_mc_kernel(BinnedParams p, float r2, int ignore_same_index) {
   const int tid = lane;
   const int half = lane >> 5;
   const int col = lane & 31;
-  const int task = bin_xcd_run((int)blockIdx.x);
+  const int task = bin_xcd_run((int)blockIdx.x, p.xcd_run_log2);
   if (task >= p.wave_start[p.num_segments])
     return; // (also the padding of the grid to whole runs)
   const int seg = find_segment(p.wave_start, p.num_segments, task);
