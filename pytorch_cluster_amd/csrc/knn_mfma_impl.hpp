@@ -82,6 +82,7 @@
 namespace pca {
 
 constexpr int kMfmaQueries = 128;   // queries per workgroup
+constexpr int kMfmaEarlySteps = 128; // drains after steps 0, 1, 3, 7, ... below this
 constexpr int kMfmaRows = 32;       // candidates per step
 constexpr int kMfmaDrainSteps = 8;  // queue entries (parked steps) per lane
 constexpr int kMfmaMaxBatch = 128;  // steps between drains at most
@@ -689,9 +690,58 @@ __global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfm
     if (t + 2 < num_steps)
       request_tile(t + 2);
 
+    const uint4 *arow = &xs[buf][col * RSU + half];
+    if (NEAREST && t == 0) {
+      // `nearest` starts without a bound, and without one every row of the
+      // first step would pass the filter (32 exact distances per query, when
+      // the whole slice needs about ten).  First bound: the filter values of
+      // this step with a cut of zero are |x|^2 - 2 x.y, which orders a
+      // query's rows like their distances; every lane takes its smallest one
+      // and that row's exact distance, the smaller of a pair's two is the
+      // query's bound.  The row itself passes the filter again below and
+      // enters the list there.
+      mfma_acc_t probe = {0};
+#pragma unroll
+      for (int i = 0; i < NB; ++i) {
+        const mc_bf16x8_t ah = __builtin_bit_cast(mc_bf16x8_t, arow[2 * i]);
+        if (i < NB - 1) {
+          const mc_bf16x8_t al =
+              __builtin_bit_cast(mc_bf16x8_t, arow[S::HI + 2 * i]);
+          probe = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, yh[i], probe, 0, 0, 0);
+          probe = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              ah, yl[i < NB - 1 ? i : 0], probe, 0, 0, 0);
+          probe = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, yh[i], probe, 0, 0, 0);
+        } else {
+          uint4 b = __builtin_bit_cast(uint4, yh[i]);
+          b.w = 0;
+          probe = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              ah, __builtin_bit_cast(mc_bf16x8_t, b), probe, 0, 0, 0);
+        }
+      }
+      float least = __builtin_inff();
+      int least_row = -1;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = 8 * (v / 4) + 4 * half + (v % 4);
+        if (row < c_count && probe[v] < least) {
+          least = probe[v];
+          least_row = row;
+        }
+      }
+      float first = __builtin_inff();
+      if (active && least_row >= 0)
+        first = exact_distance(q, c_begin + least_row);
+      const auto both = __builtin_amdgcn_permlane32_swap(
+          __float_as_uint(first), __float_as_uint(first), false, false);
+      // (fminf drops a NaN; what is left may be +inf: no bound yet)
+      first = __builtin_fminf(__uint_as_float(both[0]),
+                              __uint_as_float(both[1]));
+      if (first < thresh)
+        set_thresh(first);
+    }
+
     // ---- 32 x 32 filter values on the matrix cores ----------------------
     mfma_acc_t acc = {0};
-    const uint4 *arow = &xs[buf][col * RSU + half];
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
       const mc_bf16x8_t ah = __builtin_bit_cast(mc_bf16x8_t, arow[2 * i]);
@@ -729,7 +779,8 @@ __global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfm
     // few steps; later, when hits are rare, a drain (four memory round trips
     // whether it holds 1 pair or 64) comes only every kMfmaMaxBatch steps.
     if (__any(qn == QCAP) || drain_ordered ||
-        t - batch_t0 == kMfmaMaxBatch - 1 || !more || t <= 1 || t == 3) {
+        t - batch_t0 == kMfmaMaxBatch - 1 || !more ||
+        (t < kMfmaEarlySteps && (t & (t + 1)) == 0)) {
       drain(batch_t0 * TR);
       batch_t0 = t + 1;
     }

@@ -144,6 +144,82 @@ def test_codebook_assignment_in_feature_space(oracle):
     assert (got == oracle.nearest_op(x, y, [0, len(x)], [0, len(y)])).all()
 
 
+def _filter_cases():
+    """Inputs for the feature-space search: random rows, exact ties beyond
+    1,024 candidates, the limits, far-apart clusters, a code book with exact
+    duplicates, segments without rows on either side."""
+    for d in (9, 16, 33, 64, 128):
+        for segments in (1, 5):
+            rng = np.random.default_rng(1000 * d + segments)
+            n, m = 3000, 2600
+            x = rng.standard_normal((n, d)).astype(np.float32)
+            y = rng.standard_normal((m, d)).astype(np.float32)
+            ptr_x, ptr_y = matched_ptrs(rng, n, m, segments)
+            yield "random d=%d segments=%d" % (d, segments), x, y, ptr_x, ptr_y
+    for d in (12, 40, 128):
+        rng = np.random.default_rng(7 + d)
+        ptr_y = np.array([0, 2500, 2500, 3530, 8530], dtype=np.int64)
+        ptr_x = np.array([0, 700, 700, 764, 1664], dtype=np.int64)
+        pool = rng.integers(0, 3, (48, d)).astype(np.float32)
+        y = pool[rng.integers(0, 48, ptr_y[-1])]
+        x = pool[rng.integers(0, 48, ptr_x[-1])]
+        yield "ties d=%d" % d, x, y, ptr_x, ptr_y
+    y = np.zeros((6, 9), dtype=np.float32)
+    y[0, 0], y[1, 0], y[2, 0], y[3, 0] = 3e19, np.inf, np.nan, 9e18
+    y[4, 0], y[5, 0] = -2.5e19, 1e30
+    x = np.zeros((4, 9), dtype=np.float32)
+    x[0, 0], x[2, 0], x[3, 0] = -3e19, np.nan, 2e19
+    yield ("limits", x, y, np.array([0, 4, 4], dtype=np.int64),
+           np.array([0, 6, 6], dtype=np.int64))
+    rng = np.random.default_rng(3)
+    y = (rng.standard_normal((4000, 32)) * 10 + 5e6).astype(np.float32)
+    x = (rng.standard_normal((2500, 32)) * 10).astype(np.float32)
+    yield "far apart", x, y, None, None
+    # one far cluster among near ones: distances on both sides of 1e10
+    y = np.concatenate([y[:100], (rng.standard_normal((300, 32))).astype(
+        np.float32)])
+    x = np.concatenate([x[:200], (rng.standard_normal((200, 32)) * 10
+                                  + 5e6).astype(np.float32)])
+    yield "near and far", x, y, None, None
+    rng = np.random.default_rng(12)
+    y = rng.standard_normal((4096 * 5, 64)).astype(np.float32)
+    y[1::7] = y[0::7][:len(y[1::7])]  # exact duplicates in the code book
+    x = (y[rng.integers(0, len(y), 20000)]
+         + 0.3 * rng.standard_normal((20000, 64))).astype(np.float32)
+    x[::3] = y[rng.integers(0, len(y), len(x[::3]))]  # rows that ARE codes
+    yield "code book", x, y, None, None
+    # a query segment without candidates, and the other way round
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((700, 24)).astype(np.float32)
+    y = rng.standard_normal((900, 24)).astype(np.float32)
+    yield ("empty segments", x, y, np.array([0, 300, 300, 700], dtype=np.int64),
+           np.array([0, 0, 500, 900], dtype=np.int64))
+
+
+def test_feature_space_cases_agree_with_the_oracle(oracle):
+    """The matrix-core search of fp32 rows, 8 < d <= 128, on inputs that
+    stress its first bound (taken from one row per lane of the first step),
+    its filter near ties and the limits."""
+    for name, x, y, ptr_x, ptr_y in _filter_cases():
+        got = gpu_nearest(x, y, ptr_x, ptr_y)
+        px = ptr_x if ptr_x is not None else [0, len(x)]
+        py = ptr_y if ptr_y is not None else [0, len(y)]
+        want = oracle.nearest_op(x, y, px, py)
+        bad = np.flatnonzero(got != want)
+        assert bad.size == 0, (name, bad[:5], got[bad[:5]], want[bad[:5]])
+
+
+def test_first_step_shorter_than_a_tile(oracle):
+    """Fewer candidates than the 32 rows of a step, down to one: the first
+    bound only looks at rows that exist."""
+    rng = np.random.default_rng(77)
+    for m in (1, 2, 5, 31, 33):
+        y = rng.integers(0, 3, (m, 20)).astype(np.float32)
+        x = rng.integers(0, 3, (500, 20)).astype(np.float32)
+        got = gpu_nearest(x, y, None, None)
+        assert (got == oracle.nearest_op(x, y, [0, 500], [0, m])).all(), m
+
+
 def test_unsupported_and_invalid():
     x = torch.rand(8, 3, device=DEV).to(torch.bfloat16)
     with pytest.raises(capi.PcaError):
