@@ -86,7 +86,10 @@ constexpr int kMfmaEarlySteps = 128; // drains after steps 0, 1, 3, 7, ... below
 constexpr int kMfmaRows = 32;       // candidates per step
 constexpr int kMfmaDrainSteps = 8;  // queue entries (parked steps) per lane
 constexpr int kMfmaMaxBatch = 128;  // steps between drains at most
-constexpr int kMfmaPassPairs = 256; // pairs a wave evaluates per pass
+// pairs a wave evaluates per pass (248, not 256: with five blocks of
+// components the workgroup then needs 53,256 bytes of LDS, and three fit the
+// CU's 160 KB, which is handed out in pieces of 1,280 bytes)
+constexpr int kMfmaPassPairs = 248;
 
 typedef float mfma_acc_t __attribute__((ext_vector_type(16)));
 
@@ -247,8 +250,9 @@ __global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfm
   __shared__ uint32_t queue[QCAP][kBlock];
   // the step after which every wave of the workgroup drains: written by
   // lanes that are about to run out of queue entries (waves that drain
-  // together also wait for memory together)
-  __shared__ int drain_at;
+  // together also wait for memory together).  Entry t & 1 is read during
+  // step t and written (for step t + 2) during step t + 1, a barrier later.
+  __shared__ int drain_at[2];
   // dense re-rank, per wave: (query, row) pairs and their keys
   __shared__ int2 pairs[kBlock / kWave][CAP];
   __shared__ double results[kBlock / kWave][CAP];
@@ -671,7 +675,7 @@ __global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfm
   if (num_steps > 1)
     request_tile(1);
   if (tid == 0)
-    drain_at = -1;
+    drain_at[0] = drain_at[1] = -1;
   sync_bounds(); // what other slices already know
 
   // steps [batch_t0, t] are parked and not yet resolved; the first drains
@@ -686,7 +690,6 @@ __global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfm
     // t + 2 may now overwrite
     await_tile(more);
     __syncthreads();
-    const bool drain_ordered = drain_at == t;
     if (t + 2 < num_steps)
       request_tile(t + 2);
 
@@ -771,13 +774,15 @@ __global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfm
       ++qn;
       // one entry left: everybody drains after the next step
       if (qn == QCAP - 1)
-        drain_at = t + 1;
+        drain_at[(t + 1) & 1] = t + 1;
     }
     // Parked steps are resolved when a lane of this wave has no entry left,
     // when some lane of the workgroup announced it one step ago, after
     // kMfmaMaxBatch steps, and at the end.  While lists fill, that is every
     // few steps; later, when hits are rare, a drain (four memory round trips
     // whether it holds 1 pair or 64) comes only every kMfmaMaxBatch steps.
+    // (read here, behind the operand reads, not straight after the barrier)
+    const bool drain_ordered = drain_at[t & 1] == t;
     if (__any(qn == QCAP) || drain_ordered ||
         t - batch_t0 == kMfmaMaxBatch - 1 || !more ||
         (t < kMfmaEarlySteps && (t & (t + 1)) == 0)) {
