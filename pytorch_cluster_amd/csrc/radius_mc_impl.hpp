@@ -58,8 +58,10 @@ __global__ __launch_bounds__(kBlock) void radius_mc_kernel(RadiusMcParams p) {
 
   __shared__ __attribute__((aligned(16))) uint4 rows_lds[TX][REC];
   // parked steps: (step << 16) | mask of the lane's 16 rows that passed
+  // (also carries, between the two barriers at the top of a tile, the four
+  // waves' "all my queries are full" flags: one more variable would take the
+  // workgroup past 40,960 bytes, the most that lets four of them share a CU)
   __shared__ uint32_t queue[QCAP][kBlock];
-  __shared__ int waves_done;
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -83,9 +85,6 @@ __global__ __launch_bounds__(kBlock) void radius_mc_kernel(RadiusMcParams p) {
   const float r2 = p.r2;
   const int c_count = x_end - x_begin;
   const int num_tiles = (c_count + TX - 1) / TX;
-
-  if (tid == 0)
-    waves_done = 0;
 
   // ---- per-lane query state ---------------------------------------------
   float yq[DIM];
@@ -279,8 +278,15 @@ __global__ __launch_bounds__(kBlock) void radius_mc_kernel(RadiusMcParams p) {
   for (int t = 0; t < num_tiles; ++t) {
     // one LDS buffer: the next tile waits in registers while this one is
     // scanned
+    // (no lane has anything parked here)
+    if (lane == 0)
+      queue[0][wave * kWave] = wave_done ? 1u : 0u;
     __syncthreads();
-    if (waves_done == kBlock / kWave)
+    bool all_done = true;
+#pragma unroll
+    for (int w = 0; w < kBlock / kWave; ++w)
+      all_done = all_done && queue[0][w * kWave] != 0;
+    if (all_done)
       break; // (read between two barriers: the same for every thread)
     store_tile();
     __syncthreads();
@@ -337,11 +343,8 @@ __global__ __launch_bounds__(kBlock) void radius_mc_kernel(RadiusMcParams p) {
       }
     }
     drain(g_base, rows);
-    if (!__any(!done)) {
+    if (!__any(!done))
       wave_done = true;
-      if (lane == 0)
-        atomicAdd(&waves_done, 1);
-    }
   }
 
   if (valid && half == 0)
