@@ -679,8 +679,8 @@ __global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfm
   sync_bounds(); // what other slices already know
 
   // steps [batch_t0, t] are parked and not yet resolved; the first drains
-  // come early (after steps 0, 1 and 3), while the lists are still empty and
-  // every row passes
+  // come early (after steps 0, 1, 3, 7, ... of the slice), while the lists
+  // are empty or their bounds still loose and many rows pass
   int batch_t0 = 0;
   for (int t = 0; t < num_steps; ++t) {
     const int buf = t % RING;
