@@ -604,10 +604,11 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
               ((uint32_t)rt << 16) | mask;
           qnext += QROW;
         }
-        // (the first drains of a scan come early -- after steps 0, 1 and 3
-        // -- while the lists are empty and every row passes)
+        // (the first drains of a scan come early -- after steps 0, 1, 3, 7,
+        // 15 and 31 of its first tile -- while the lists are empty or their
+        // bounds still loose and many rows pass)
         if (__any(qnext >= qfirst + QCAP * QROW) ||
-            (t == 0 && (rt <= 1 || rt == 3)))
+            (t == 0 && (rt & (rt + 1)) == 0))
           drain(g_base, rows);
       }
     }
