@@ -584,12 +584,15 @@ knn_binned_mc_kernel(BinnedParams p) {
       // (a row of EQUAL distance and smaller number can still get in)
       if (own_bound < kLimit)
         own_bound = next_up_positive(own_bound);
-      set_thresh(__builtin_fminf(own_bound, shared));
+      // (the filter's cut follows once, after the last round)
+      if (searching)
+        thresh = __builtin_fminf(own_bound, shared);
       changed = true;
     }
     qn = 0;
     if (!changed)
       return;
+    set_thresh(thresh);
     partner_bounds();
     refresh_cut();
   };

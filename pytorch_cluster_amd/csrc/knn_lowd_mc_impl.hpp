@@ -531,12 +531,15 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
       // (`nearest`: a later row of EQUAL distance can still win the tie)
       if (NEAREST && own_bound < kLimit)
         own_bound = next_up_positive(own_bound);
-      set_thresh(__builtin_fminf(own_bound, shared));
+      // (the filter's cut follows once, after the last round)
+      if (valid)
+        thresh = __builtin_fminf(own_bound, shared);
       changed = true;
     }
     qnext = qfirst;
     if (!changed)
       return;
+    set_thresh(thresh);
     partner_bounds();
     refresh_cut();
   };
