@@ -357,26 +357,8 @@ __device__ __forceinline__ float feat_pick(const feat_acc_t (&a)[SUBS], int v) {
   float r = 0.0f;
 #pragma unroll
   for (int sub = 0; sub < SUBS; ++sub) {
-    if ((v >> 4) == sub) {
-      switch (v & 15) {
-      case 0: r = a[sub][0]; break;
-      case 1: r = a[sub][1]; break;
-      case 2: r = a[sub][2]; break;
-      case 3: r = a[sub][3]; break;
-      case 4: r = a[sub][4]; break;
-      case 5: r = a[sub][5]; break;
-      case 6: r = a[sub][6]; break;
-      case 7: r = a[sub][7]; break;
-      case 8: r = a[sub][8]; break;
-      case 9: r = a[sub][9]; break;
-      case 10: r = a[sub][10]; break;
-      case 11: r = a[sub][11]; break;
-      case 12: r = a[sub][12]; break;
-      case 13: r = a[sub][13]; break;
-      case 14: r = a[sub][14]; break;
-      default: r = a[sub][15]; break;
-      }
-    }
+    if ((v >> 4) == sub)
+      r = a[sub][v & 15]; // (a uniform index: register-relative read)
   }
   return r;
 }
