@@ -103,6 +103,21 @@ __global__ __launch_bounds__(kPlanThreads) void scan_block_sums_kernel(
   }
 }
 
+// e / slots without a division, for the entries e < kCompactQueries * slots
+// of a block: with magic = ceil(2^32 / slots) the product's high word is the
+// quotient as long as e (slots - 1) < 2^32, which holds up to 4,000 slots; 0
+// (one slot, or more than that) stands for "divide".
+inline uint32_t slots_magic(int slots) {
+  if (slots < 2 || slots > 4000)
+    return 0;
+  return (uint32_t)((((uint64_t)1 << 32) + (uint64_t)slots - 1) /
+                    (uint64_t)slots);
+}
+__device__ __forceinline__ int quotient_by_slots(int e, int slots,
+                                                 uint32_t magic) {
+  return magic != 0 ? (int)__umulhi((uint32_t)e, magic) : e / slots;
+}
+
 // Both kernels below walk the slot rows of a block of queries as ONE flat
 // range (element e = slot e % slots of query e / slots): reads are contiguous
 // and independent of each other, so many are in flight per thread.
@@ -112,7 +127,8 @@ __global__ __launch_bounds__(kPlanThreads) void scan_block_sums_kernel(
 // number of slots without it.
 __global__ __launch_bounds__(kBlock) void find_self_kernel(
     const int *__restrict__ idx, const int *__restrict__ count, int m,
-    int slots, int *__restrict__ self_pos, int *__restrict__ kept) {
+    int slots, uint32_t magic, int *__restrict__ self_pos,
+    int *__restrict__ kept) {
   __shared__ int s_self[kCompactQueries];
   __shared__ int s_count[kCompactQueries];
   const int tid = threadIdx.x;
@@ -125,7 +141,7 @@ __global__ __launch_bounds__(kBlock) void find_self_kernel(
   const int total = nq * slots;
 #pragma unroll 4
   for (int e = tid; e < total; e += kBlock) {
-    const int ql = e / slots;
+    const int ql = quotient_by_slots(e, slots, magic);
     const int sl = e - ql * slots;
     const int v = rows[e];
     if (sl < s_count[ql] && v == q0 + ql)
@@ -146,8 +162,8 @@ constexpr int kInlineScanBlocks = 2048;
 
 __global__ __launch_bounds__(kBlock) void count_block_kernel(
     const int *__restrict__ idx, const int *__restrict__ count, int m,
-    int slots, int *__restrict__ self_pos, int *__restrict__ kept,
-    int64_t *__restrict__ block_sums) {
+    int slots, uint32_t magic, int *__restrict__ self_pos,
+    int *__restrict__ kept, int64_t *__restrict__ block_sums) {
   __shared__ int s_self[kCompactQueries];
   __shared__ int s_count[kCompactQueries];
   __shared__ int lds[kBlock];
@@ -163,7 +179,7 @@ __global__ __launch_bounds__(kBlock) void count_block_kernel(
     const int total = nq * slots;
 #pragma unroll 4
     for (int e = tid; e < total; e += kBlock) {
-      const int ql = e / slots;
+      const int ql = quotient_by_slots(e, slots, magic);
       const int sl = e - ql * slots;
       const int v = rows[e];
       if (sl < s_count[ql] && v == q0 + ql)
@@ -189,7 +205,8 @@ __global__ __launch_bounds__(kBlock) void count_block_kernel(
 __global__ __launch_bounds__(kBlock) void scatter_kernel(
     const int *__restrict__ idx, const float *__restrict__ dist,
     const int *__restrict__ count, const int *__restrict__ self_pos, int m,
-    int slots, int x_first, const int64_t *__restrict__ block_offsets,
+    int slots, uint32_t magic, int x_first,
+    const int64_t *__restrict__ block_offsets,
     int64_t *__restrict__ num_edges, int64_t *__restrict__ edges,
     float *__restrict__ dist_out, int inline_scan) {
   __shared__ int lds[kBlock];
@@ -245,7 +262,7 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
   const int span = nq * slots;
 #pragma unroll 4
   for (int e = tid; e < span; e += kBlock) {
-    const int ql = e / slots;
+    const int ql = quotient_by_slots(e, slots, magic);
     const int sl = e - ql * slots;
     const int skip = s_self[ql];
     // slot sl goes to position sl, or sl - 1 behind the left-out slot
@@ -297,21 +314,23 @@ hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
   int *self_pos = reinterpret_cast<int *>(ws);
   int *kept = reinterpret_cast<int *>(ws + align256(sizeof(int) * (size_t)m));
   const int *count = dense.count;
+  const uint32_t magic = slots_magic(dense.slots);
   if (blocks <= kInlineScanBlocks) {
     hipLaunchKernelGGL(count_block_kernel, dim3(blocks), dim3(kBlock), 0,
-                       stream, dense.idx, dense.count, m, dense.slots,
+                       stream, dense.idx, dense.count, m, dense.slots, magic,
                        drop_self ? self_pos : (int *)nullptr, kept,
                        block_sums);
     hipLaunchKernelGGL(scatter_kernel, dim3(blocks), dim3(kBlock), 0, stream,
                        dense.idx, dense.dist, drop_self ? kept : count,
                        drop_self ? self_pos : (const int *)nullptr, m,
-                       dense.slots, x_first ? 1 : 0, block_sums, num_edges,
-                       edges, dist_out, 1);
+                       dense.slots, magic, x_first ? 1 : 0, block_sums,
+                       num_edges, edges, dist_out, 1);
     return hipGetLastError();
   }
   if (drop_self) {
     hipLaunchKernelGGL(find_self_kernel, dim3(blocks), dim3(kBlock), 0, stream,
-                       dense.idx, dense.count, m, dense.slots, self_pos, kept);
+                       dense.idx, dense.count, m, dense.slots, magic, self_pos,
+                       kept);
     count = kept;
   }
   hipLaunchKernelGGL(block_sum_kernel, dim3(blocks), dim3(kBlock), 0, stream,
@@ -321,7 +340,7 @@ hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
   hipLaunchKernelGGL(scatter_kernel, dim3(blocks), dim3(kBlock), 0, stream,
                      dense.idx, dense.dist, count,
                      drop_self ? self_pos : (const int *)nullptr, m,
-                     dense.slots, x_first ? 1 : 0, block_sums, num_edges,
+                     dense.slots, magic, x_first ? 1 : 0, block_sums, num_edges,
                      edges, dist_out, 0);
   return hipGetLastError();
 }
