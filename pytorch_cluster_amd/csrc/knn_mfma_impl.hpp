@@ -87,7 +87,7 @@ constexpr int kMfmaRows = 32;       // candidates per step
 constexpr int kMfmaDrainSteps = 8;  // queue entries (parked steps) per lane
 constexpr int kMfmaMaxBatch = 128;  // steps between drains at most
 // pairs a wave evaluates per pass (248, not 256: with five blocks of
-// components the workgroup then needs 53,256 bytes of LDS, and three fit the
+// components the workgroup then needs 53,512 bytes of LDS, and three fit the
 // CU's 160 KB, which is handed out in pieces of 1,280 bytes)
 constexpr int kMfmaPassPairs = 248;
 
