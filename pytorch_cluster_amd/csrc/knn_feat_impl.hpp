@@ -1,4 +1,4 @@
-// Feature-space kNN (8 < d <= 256, k <= 48, Euclidean or cosine) on the gfx950
+// Feature-space kNN (8 < d <= 512, k <= 100, Euclidean or cosine) on the gfx950
 // matrix cores: ONE fp16 product per pair and component picks a short list of
 // candidates per query, a second kernel evaluates those exactly.  Results are
 // bit-identical to the reference's scalar loop (csrc/cuda/knn_cuda.cu:52-78).
@@ -11,7 +11,8 @@
 //     s = W + sum_c h(X_c) h(-2 Y_c),      W <= |X|^2 (1 - rho),
 // is one chain of v_mfma_f32_32x32x16_f16 over the blocks of 16 components
 // plus one block that carries W (three fp16 parts times 2^15, 2^4, 2^-7).
-// With rho = 2^-9 and C0 = 2^-12 d the value
+// With rho = 2^-9 (2^-8 beyond 256 components, feat_rho) and C0 = 2^-12 d
+// the value
 //     l = s + |Y|^2 (1 - rho) - C0
 // is a LOWER bound of the distance e' = e / sigma^2 the reference computes,
 // and e' <= F(l) = (l + 6 rho |Y|^2 + 2 C0) (1 + 4.1 rho):

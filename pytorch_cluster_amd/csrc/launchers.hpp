@@ -157,7 +157,7 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
 // --- knn_feat*.hip ---------------------------------------------------------
 
 // Feature-space kNN with the fp16 matrix-core filter and the exact second
-// kernel (knn_feat_impl.hpp): fp32, 8 < d <= 256, k <= 48.
+// kernel (knn_feat_impl.hpp): fp32, 8 < d <= 512, k <= 100.
 bool knn_feat_supported(int d, int k, bool cosine);
 size_t knn_feat_scratch_bytes(int n, int m, int d, int num_segments, int k);
 // work_start: tiles of kMfmaTileQueries queries (planned by the caller).
