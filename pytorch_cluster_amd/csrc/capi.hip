@@ -490,6 +490,10 @@ int knn_call(const void *x, const void *y, const int64_t *ptr_x,
     src = segments_by_id(ptr_x, ptr_y, n, m, num_segments, take(lay.ptrs));
   pca::KnnLowdConfig cfg = pca::knn_lowd_config(
       (int)d, (int)k, (int)n, (int)m, (int)num_segments, cosine != 0);
+  // (the matrix-core kernels count the edges while they write their lists)
+  if (low_d && cfg.matrix_cores)
+    pca::compact_hints(dense, (int)m, compact_ws,
+                       (edge_flags & PCA_EDGES_DROP_SELF) != 0);
 
   pca::SearchInput in{x,      y,      ptr_x,  ptr_y,
                       (int)n, (int)m, (int)d, (int)num_segments};
@@ -764,6 +768,8 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
       pca::plan_upper_bound((int)m, (int)num_segments, per_item);
   if (!matrix_cores)
     timer.begin();
+  if (matrix_cores)
+    pca::compact_hints(dense, (int)m, compact_ws, false);
   if (matrix_cores)
     rc = check_launch(pca::launch_radius_mc(in, r2, ignore_same_index != 0,
                                             work_start, bound, packed_rows,

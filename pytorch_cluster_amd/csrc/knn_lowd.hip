@@ -240,8 +240,16 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
     if (env_int("PCA_KNN_XCD_CLAIM", 0) != 0)
       p.claim = reinterpret_cast<int *>(
           base + align256(sizeof(float) * (size_t)in.m));
+    // (only this set-up clears the compaction's block sums: the other path
+    // leaves the counting to the compaction)
+    p.edge_sums = nearest_out ? nullptr : out.edge_sums;
+    p.self_pos = out.self_pos;
+    p.kept = out.kept;
     McSetup a;
     a.claim = p.claim;
+    a.edge_sums = p.edge_sums;
+    a.edge_blocks =
+        (in.m + kCompactBlockQueries - 1) / kCompactBlockQueries + 1;
     a.x = p.x;
     a.n = in.n;
     a.d_in = in.d;

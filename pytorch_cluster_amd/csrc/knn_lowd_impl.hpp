@@ -75,6 +75,12 @@ struct KnnLowdParams {
   float *out_dist;
   int *out_count;
   int64_t *out_nearest;  // [m] result of the `nearest` search, else unused
+  // for the compaction (DenseResult; NULL: not asked for): slots it will
+  // write per kCompactBlockQueries queries, the slot of the query's own row
+  // and the count without it
+  unsigned long long *edge_sums = nullptr;
+  int *self_pos = nullptr;
+  int *kept = nullptr;
   // second pass behind another search (knn_merge_kernel): nothing runs while
   // *gate is 0, and only queries with a non-zero redo_q entry are written
   const int *gate = nullptr;
@@ -87,9 +93,9 @@ __device__ __forceinline__ float next_up_positive(float v) {
 
 // Writes the real slots of a sorted key list as dense results.
 template <int K>
-__device__ __forceinline__ void write_dense(const double (&best)[K], int k,
-                                            int q, int *out_idx,
-                                            float *out_dist, int *out_count) {
+__device__ __forceinline__ int write_dense(const double (&best)[K], int k,
+                                           int q, int *out_idx,
+                                           float *out_dist, int *out_count) {
   const size_t row = (size_t)q * k;
   int found = 0;
 #pragma unroll
@@ -103,6 +109,58 @@ __device__ __forceinline__ void write_dense(const double (&best)[K], int k,
     }
   }
   out_count[q] = found;
+  return found;
+}
+
+// sums[block] += value for every lane that gets here (any subset of a wave;
+// 0 <= value < 128), with one atomic per distinct block among them: the lanes
+// of a wave hold neighbouring queries, and atomics on one address take turns
+// in the L2 (65,536 single ones on 256 addresses cost 45 us).
+__device__ __forceinline__ void add_to_block_sum(unsigned long long *sums,
+                                                 int block, int value) {
+  const int lane = (int)(threadIdx.x & (kWave - 1));
+  bool done = false;
+  for (;;) {
+    const uint64_t waiting = __ballot(!done);
+    if (waiting == 0)
+      break;
+    const int leader = (int)__builtin_ctzll(waiting);
+    const int lead_block = __shfl(block, leader);
+    const bool mine = !done && block == lead_block;
+    int total = 0;
+#pragma unroll
+    for (int b = 0; b < 7; ++b)
+      total += __builtin_popcountll(__ballot(mine && ((value >> b) & 1))) << b;
+    if (lane == leader)
+      atomicAdd(&sums[lead_block], (unsigned long long)total);
+    done = done || mine;
+  }
+}
+
+// What the compaction wants to know about the list just written (see
+// DenseResult): adds the query's slots to its block's sum and, for graph
+// results (self_pos given), notes where the query's own row sits.
+template <int K>
+__device__ __forceinline__ void note_edges(const double (&best)[K], int k,
+                                           int q, int found,
+                                           unsigned long long *edge_sums,
+                                           int *self_pos, int *kept) {
+  if (edge_sums == nullptr)
+    return;
+  int keep = found;
+  if (self_pos != nullptr) {
+    int self = -1;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      const int e = j - (K - k);
+      if (e >= 0 && best[j] < empty_key() && key_row(best[j]) == q)
+        self = e;
+    }
+    keep -= self >= 0 ? 1 : 0;
+    self_pos[q] = self;
+    kept[q] = keep;
+  }
+  add_to_block_sum(edge_sums, q / kCompactBlockQueries, keep);
 }
 
 // Result of a `nearest` search: the row behind the smallest key, or 0 when no
@@ -565,7 +623,10 @@ __global__ __launch_bounds__(kBlock) void knn_merge_kernel(KnnLowdParams p) {
         write_nearest(best[K - 1], q, p.ptr_x ? (int)p.ptr_x[seg] : 0,
                       p.out_nearest);
       else
-        write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+        note_edges<K>(best, k, q,
+                      write_dense<K>(best, k, q, p.out_idx, p.out_dist,
+                                     p.out_count),
+                      p.edge_sums, p.self_pos, p.kept);
     }
   }
 }

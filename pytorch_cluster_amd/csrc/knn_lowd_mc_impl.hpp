@@ -164,6 +164,9 @@ struct McSetup {
   uint4 *out;
   float *tau; // [m] or NULL
   int *claim; // 8 counters to clear, or NULL
+  // the compaction's block sums to clear (DenseResult::edge_sums), or NULL
+  unsigned long long *edge_sums = nullptr;
+  int edge_blocks = 0;
   int m;
   float tau_value;
   const int64_t *ptr_y; // plan input (src.ptr_y when src is used)
@@ -178,6 +181,10 @@ __global__ __launch_bounds__(kPlanThreads) void mc_setup_kernel(McSetup a) {
   __shared__ int partial[kPlanThreads];
   if (blockIdx.x == 0 && a.claim != nullptr && threadIdx.x < 8)
     a.claim[threadIdx.x] = 0;
+  if (a.edge_sums != nullptr)
+    for (int b = blockIdx.x * kPlanThreads + threadIdx.x; b < a.edge_blocks;
+         b += gridDim.x * kPlanThreads)
+      a.edge_sums[b] = 0ull;
   if (blockIdx.x == 0 && a.work_start != nullptr) {
     if (a.src.ids_x != nullptr) {
       pointers_from_ids(a.src, a.num_segments);
@@ -629,7 +636,10 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
         if constexpr (NEAREST)
           write_nearest(best[0], q, x_begin, p.out_nearest);
         else
-          write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+          note_edges<K>(best, k, q,
+                        write_dense<K>(best, k, q, p.out_idx, p.out_dist,
+                                       p.out_count),
+                        p.edge_sums, p.self_pos, p.kept);
       }
     } else {
       // sorted keys of this slice, [item][slot][query of the tile]

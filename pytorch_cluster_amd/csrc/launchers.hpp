@@ -17,6 +17,15 @@ struct DenseResult {
   float *dist;
   int *count;
   int slots;
+  // What the compaction otherwise finds out in a pass of its own, from a
+  // search that leaves it behind (compact_hints; NULL: it does not): per
+  // block of queries the number of slots the compaction will write (added up
+  // with atomics; zeroed by the search's set-up launch), and for graph
+  // results the slot of the query's own row (-1: none) and the count without
+  // it.
+  unsigned long long *edge_sums = nullptr;
+  int *self_pos = nullptr;
+  int *kept = nullptr;
 };
 
 struct SearchInput {
@@ -67,6 +76,14 @@ hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
                           int64_t *num_edges, float *dist_out, void *workspace,
                           hipStream_t stream, bool drop_self = false,
                           bool x_first = false);
+// Points dense.edge_sums (and, with drop_self, self_pos / kept) into the
+// compaction's workspace when the call is small enough for the compaction
+// that adds up the block sums on its own; launch_compact then skips its
+// counting pass.  Only for searches that fill them (the low-dimensional
+// matrix-core kernels).
+void compact_hints(DenseResult &dense, int m, void *workspace, bool drop_self);
+// Queries per block sum.
+constexpr int kCompactBlockQueries = 256;
 
 // --- knn_lowd_*.hip --------------------------------------------------------
 

@@ -81,7 +81,10 @@ hipError_t launch_radius_mc(const SearchInput &in, float r2,
   p.work_start = work_start;
   p.out_idx = out.idx;
   p.out_count = out.count;
+  p.edge_sums = out.edge_sums;
   McSetup a;
+  a.edge_sums = out.edge_sums;
+  a.edge_blocks = (in.m + kCompactBlockQueries - 1) / kCompactBlockQueries + 1;
   a.x = static_cast<const float *>(in.x);
   a.n = in.n;
   a.d_in = in.d;

@@ -44,6 +44,9 @@ struct RadiusMcParams {
   const int *work_start; // [num_segments + 1] first 128-query tile per segment
   int *out_idx;          // [m, slots]
   int *out_count;        // [m]
+  // for the compaction (DenseResult::edge_sums; NULL: not asked for):
+  // neighbours found per kCompactBlockQueries queries
+  unsigned long long *edge_sums = nullptr;
 };
 
 template <int DIM>
@@ -347,8 +350,15 @@ __global__ __launch_bounds__(kBlock) void radius_mc_kernel(RadiusMcParams p) {
       wave_done = true;
   }
 
-  if (valid && half == 0)
+  if (valid && half == 0) {
     p.out_count[q] = count;
+    if (p.edge_sums != nullptr) // (count <= slots; wide lists: one by one)
+      if (p.slots < 128)
+        add_to_block_sum(p.edge_sums, q / kCompactBlockQueries, count);
+      else
+        atomicAdd(&p.edge_sums[q / kCompactBlockQueries],
+                  (unsigned long long)count);
+  }
 }
 
 } // namespace pca

@@ -304,6 +304,20 @@ size_t compact_workspace_bytes(int m) {
          2 * align256(sizeof(int) * (size_t)m);
 }
 
+void compact_hints(DenseResult &dense, int m, void *workspace, bool drop_self) {
+  static_assert(kCompactBlockQueries == kCompactQueries, "one block, one sum");
+  const int blocks = (m + kCompactQueries - 1) / kCompactQueries;
+  if (blocks > kInlineScanBlocks)
+    return;
+  char *ws = static_cast<char *>(workspace);
+  dense.edge_sums = reinterpret_cast<unsigned long long *>(ws);
+  ws += align256(sizeof(int64_t) * (size_t)(blocks + 1));
+  if (drop_self) {
+    dense.self_pos = reinterpret_cast<int *>(ws);
+    dense.kept = reinterpret_cast<int *>(ws + align256(sizeof(int) * (size_t)m));
+  }
+}
+
 hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
                           int64_t *num_edges, float *dist_out, void *workspace,
                           hipStream_t stream, bool drop_self, bool x_first) {
@@ -315,6 +329,17 @@ hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
   int *kept = reinterpret_cast<int *>(ws + align256(sizeof(int) * (size_t)m));
   const int *count = dense.count;
   const uint32_t magic = slots_magic(dense.slots);
+  if (dense.edge_sums != nullptr && blocks <= kInlineScanBlocks &&
+      (!drop_self || dense.self_pos != nullptr)) {
+    // the search left the block sums (and the self slots) behind
+    hipLaunchKernelGGL(scatter_kernel, dim3(blocks), dim3(kBlock), 0, stream,
+                       dense.idx, dense.dist, drop_self ? dense.kept : count,
+                       drop_self ? dense.self_pos : (const int *)nullptr, m,
+                       dense.slots, magic, x_first ? 1 : 0,
+                       reinterpret_cast<const int64_t *>(dense.edge_sums),
+                       num_edges, edges, dist_out, 1);
+    return hipGetLastError();
+  }
   if (blocks <= kInlineScanBlocks) {
     hipLaunchKernelGGL(count_block_kernel, dim3(blocks), dim3(kBlock), 0,
                        stream, dense.idx, dense.count, m, dense.slots, magic,
