@@ -1,7 +1,7 @@
 // Dispatch of the feature-space kNN with the fp16 matrix-core filter (see
 // knn_feat_impl.hpp): preparation, the filter kernel, the exact second kernel
 // and the second pass for the queries that one flags.
-#include "knn_feat_impl.hpp"
+#include "knn_feat_wide_impl.hpp"
 
 #include <algorithm>
 #include <cstdlib>
@@ -22,6 +22,15 @@ PCA_DECLARE_FEAT_BLOCKS(9)
 PCA_DECLARE_FEAT_BLOCKS(17)
 PCA_DECLARE_FEAT_BLOCKS(33)
 #undef PCA_DECLARE_FEAT_BLOCKS
+
+#define PCA_DECLARE_FEAT_WIDE_BLOCKS(NB)                                       \
+  template <>                                                                  \
+  hipError_t launch_knn_feat_wide_blocks<NB>(const KnnFeatWideParams &, int,   \
+                                             bool, int, hipStream_t);
+PCA_DECLARE_FEAT_WIDE_BLOCKS(3)
+PCA_DECLARE_FEAT_WIDE_BLOCKS(5)
+PCA_DECLARE_FEAT_WIDE_BLOCKS(9)
+#undef PCA_DECLARE_FEAT_WIDE_BLOCKS
 
 namespace {
 
@@ -66,10 +75,14 @@ size_t feat_pack_bytes(int n, int d) {
 }
 
 __global__ __launch_bounds__(kBlock) void feat_init_kernel(
-    FeatGlobals *g, float *tau, int m, int *hit_count, int redo_cap) {
+    FeatGlobals *g, float *tau, int m, int *hit_count, int redo_cap,
+    int *overflow) {
   const int i = blockIdx.x * kBlock + threadIdx.x;
-  if (i < m)
+  if (i < m) {
     tau[i] = __builtin_inff();
+    if (overflow != nullptr)
+      overflow[i] = 0;
+  }
   if (i < redo_cap)
     hit_count[i] = 0;
   if (i == 0) {
@@ -212,13 +225,141 @@ void launch_feat_merge(const KnnFeatParams &p, int tiles_bound,
                      0, stream, p);
 }
 
+// Single workgroup: per segment the first 512-query tile and the first
+// (tile, unit) pair -- exclusive sums of tiles_s and of tiles_s * units_s.
+__global__ __launch_bounds__(kPlanThreads) void feat_wide_plan_kernel(
+    const int64_t *__restrict__ ptr_x, const int64_t *__restrict__ ptr_y,
+    int n, int m, int num_segments, int *__restrict__ tile_start,
+    long long *__restrict__ unit_start) {
+  __shared__ long long part_u[kPlanThreads];
+  __shared__ int part_t[kPlanThreads];
+  const int tid = threadIdx.x;
+  const int per_thread = (num_segments + kPlanThreads - 1) / kPlanThreads;
+  const int b0 = min(tid * per_thread, num_segments);
+  const int b1 = min(b0 + per_thread, num_segments);
+  auto counts = [&](int b, int &tiles, long long &pairs) {
+    const int64_t xl = ptr_x ? ptr_x[b] : 0, xh = ptr_x ? ptr_x[b + 1] : n;
+    const int64_t yl = ptr_y ? ptr_y[b] : 0, yh = ptr_y ? ptr_y[b + 1] : m;
+    const int rows = (int)max((int64_t)0, xh - xl);
+    const int queries = (int)max((int64_t)0, yh - yl);
+    tiles = (queries + kWideQueries - 1) / kWideQueries;
+    pairs = (long long)tiles * ((rows + kWideTileRows - 1) / kWideTileRows);
+  };
+  int st = 0;
+  long long su = 0;
+  for (int b = b0; b < b1; ++b) {
+    int t;
+    long long u;
+    counts(b, t, u);
+    st += t;
+    su += u;
+  }
+  part_t[tid] = st;
+  part_u[tid] = su;
+  __syncthreads();
+  for (int off = 1; off < kPlanThreads; off <<= 1) {
+    const int vt = tid >= off ? part_t[tid - off] : 0;
+    const long long vu = tid >= off ? part_u[tid - off] : 0;
+    __syncthreads();
+    part_t[tid] += vt;
+    part_u[tid] += vu;
+    __syncthreads();
+  }
+  int rt = part_t[tid] - st;
+  long long ru = part_u[tid] - su;
+  for (int b = b0; b < b1; ++b) {
+    tile_start[b] = rt;
+    unit_start[b] = ru;
+    int t;
+    long long u;
+    counts(b, t, u);
+    rt += t;
+    ru += u;
+  }
+  if (tid == kPlanThreads - 1) {
+    tile_start[num_segments] = part_t[tid];
+    unit_start[num_segments] = part_u[tid];
+  }
+}
+
+// list width of the eight-wave first stage: the k smallest values
+int feat_wide_width(int k) {
+  static const int widths[] = {16, 32, 64, 100};
+  for (int w : widths)
+    if (k <= w)
+      return w;
+  return 0;
+}
+
+int device_cu_count() {
+  static int cached = 0;
+  if (cached == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount,
+                              dev) != hipSuccess ||
+        cus <= 0)
+      cus = 256;
+    cached = cus;
+  }
+  return cached;
+}
+
+// The eight-wave first stage (knn_feat_wide_impl.hpp) takes calls with enough
+// queries per segment to fill its tiles of 512.
+bool feat_wide_applies(int m, int d, int num_segments, int k) {
+  const bool fits = d <= kWideMaxDim && feat_wide_width(k) != 0;
+  // PCA_KNN_FEAT_WIDE: 0 never, 1 whenever the shape fits (the tests)
+  if (const char *env = std::getenv("PCA_KNN_FEAT_WIDE")) {
+    if (env[0] == '0')
+      return false;
+    if (env[0] == '1')
+      return fits;
+  }
+  return fits && m >= 4096 && (long long)num_segments * 1024 <= (long long)m;
+}
+
+struct FeatWidePlan {
+  int grid;      // workgroups of the first stage
+  int tiles;     // upper bound of the 512-query tiles
+  int cap;       // buffer entries per (piece, query)
+  size_t pieces; // upper bound of the pieces
+};
+
+FeatWidePlan feat_wide_plan(int n, int m, int num_segments, int k) {
+  FeatWidePlan w;
+  w.tiles = plan_upper_bound(m, num_segments, kWideQueries);
+  // (tile, unit) pairs, roughly: every tile of a segment meets the segment's
+  // units
+  const long long units_per_segment =
+      ((long long)n / num_segments + kWideTileRows - 1) / kWideTileRows + 1;
+  const long long pairs = (long long)w.tiles * units_per_segment;
+  w.grid = (int)std::max(1LL, std::min((long long)device_cu_count(),
+                                       pairs / 4));
+  if (const char *env = std::getenv("PCA_FEAT_WIDE_GRID")) {
+    const int v = std::atoi(env);
+    if (v >= 1 && v <= 4096)
+      w.grid = v;
+  }
+  w.cap = (256 + 4 * (k + kFeatSlack) + 63) / 64 * 64;
+  if (const char *env = std::getenv("PCA_FEAT_WIDE_CAP")) {
+    const int v = std::atoi(env);
+    if (v >= 256 && v <= 8192)
+      w.cap = v / 64 * 64;
+  }
+  w.pieces = (size_t)w.grid + (size_t)w.tiles;
+  return w;
+}
+
 struct FeatLayout {
-  size_t globals, x_norm, x_class, y_norm, tau, redo, plan256;
+  size_t globals, x_norm, x_class, y_norm, tau, redo, over, plan256;
   size_t redo_list, redo_tau, hit_count, hits; // threshold scan
   size_t pack, partial, cand; // first pass
+  // eight-wave first stage: `partial` is then these four
+  size_t wide_plan = 0, wide_buf = 0, wide_count = 0, wide_lists = 0;
   size_t second;              // second pass (reuses the first pass's bytes)
   size_t shared() const {
-    return globals + x_norm + x_class + y_norm + tau + redo + plan256 +
+    return globals + x_norm + x_class + y_norm + tau + redo + over + plan256 +
            redo_list + redo_tau + hit_count + hits;
   }
   size_t total() const {
@@ -269,6 +410,7 @@ static FeatLayout feat_layout(int n, int m, int d, int num_segments, int k) {
   w.y_norm = align256(sizeof(float) * (size_t)m);
   w.tau = align256(sizeof(float) * (size_t)m);
   w.redo = align256(sizeof(int) * (size_t)m);
+  w.over = align256(sizeof(int) * (size_t)m);
   w.plan256 = align256(sizeof(int) * ((size_t)num_segments + 1));
   const size_t cap = (size_t)feat_redo_cap(m);
   w.redo_list = align256(sizeof(int) * cap);
@@ -276,7 +418,18 @@ static FeatLayout feat_layout(int n, int m, int d, int num_segments, int k) {
   w.hit_count = align256(sizeof(int) * cap);
   w.hits = align256(sizeof(double) * cap * feat_hit_cap(k));
   w.pack = feat_pack_bytes(n, d);
-  w.partial = align256(sizeof(double) * tiles * chunks * kk * kFeatQueries);
+  if (feat_wide_applies(m, d, num_segments, k)) {
+    const FeatWidePlan wp = feat_wide_plan(n, m, num_segments, k);
+    w.wide_plan = align256(sizeof(int) * ((size_t)num_segments + 1)) +
+                  align256(sizeof(long long) * ((size_t)num_segments + 1));
+    w.wide_buf = align256(sizeof(uint2) * wp.pieces * kWideQueries * wp.cap);
+    w.wide_count = align256(sizeof(int) * wp.pieces * kWideQueries);
+    w.wide_lists = align256(sizeof(float) * (size_t)wp.grid *
+                            feat_wide_width(k) * kWideQueries);
+    w.partial = w.wide_plan + w.wide_buf + w.wide_count + w.wide_lists;
+  } else {
+    w.partial = align256(sizeof(double) * tiles * chunks * kk * kFeatQueries);
+  }
   w.cand = align256(sizeof(double) * (size_t)m * kk);
   w.second = second_pass_on_matrix_cores(d, k)
                  ? knn_mfma_scratch_bytes(n, m, d, num_segments, k,
@@ -310,6 +463,7 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   float *y_norm = reinterpret_cast<float *>(take(lay.y_norm));
   float *tau = reinterpret_cast<float *>(take(lay.tau));
   int *redo_q = reinterpret_cast<int *>(take(lay.redo));
+  int *overflow = reinterpret_cast<int *>(take(lay.over));
   int *plan256 = reinterpret_cast<int *>(take(lay.plan256));
   int *redo_list = reinterpret_cast<int *>(take(lay.redo_list));
   float *redo_tau = reinterpret_cast<float *>(take(lay.redo_tau));
@@ -327,7 +481,7 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
 
   hipLaunchKernelGGL(feat_init_kernel, dim3((in.m + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, globals, tau, in.m, hit_count,
-                     redo_cap);
+                     redo_cap, overflow);
   // squared norms that only classify the rows (NaN: a non-finite component);
   // for the Euclidean distance they also enter the filter
   float *x_class = cosine ? x_class_buf : x_norm;
@@ -414,15 +568,85 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   p.hits = hits;
   p.redo_cap = redo_cap;
   p.hit_cap = feat_hit_cap(k);
+  p.overflow = nullptr;
   p.out_idx = out.idx;
   p.out_dist = out.dist;
   p.out_count = out.count;
 
   const int kp = feat_width(k);
+  hipError_t err;
+  if (lay.wide_buf != 0) {
+    // eight-wave first stage: plan, filter, gather
+    const FeatWidePlan wp = feat_wide_plan(in.n, in.m, in.num_segments, k);
+    char *wb = reinterpret_cast<char *>(partial);
+    KnnFeatWideParams wpar;
+    p.overflow = overflow;
+    wpar.base = p;
+    int *tile_start = reinterpret_cast<int *>(wb);
+    long long *unit_start = reinterpret_cast<long long *>(
+        wb + align256(sizeof(int) * ((size_t)in.num_segments + 1)));
+    wb += lay.wide_plan;
+    wpar.tile_start = tile_start;
+    wpar.unit_start = unit_start;
+    wpar.cap = wp.cap;
+    wpar.buf = reinterpret_cast<uint2 *>(wb);
+    wb += lay.wide_buf;
+    wpar.buf_count = reinterpret_cast<int *>(wb);
+    wb += lay.wide_count;
+    wpar.lists = reinterpret_cast<float *>(wb);
+    wpar.overflow = overflow;
+    hipLaunchKernelGGL(feat_wide_plan_kernel, dim3(1), dim3(kPlanThreads), 0,
+                       stream, in.ptr_x, in.ptr_y, in.n, in.m,
+                       in.num_segments, tile_start, unit_start);
+    if (time_start)
+      (void)hipEventRecord(time_start, stream);
+    const int kw = feat_wide_width(k);
+    switch (nb) {
+    case 3:
+      err = launch_knn_feat_wide_blocks<3>(wpar, kw, cosine, wp.grid, stream);
+      break;
+    case 5:
+      err = launch_knn_feat_wide_blocks<5>(wpar, kw, cosine, wp.grid, stream);
+      break;
+    default:
+      err = launch_knn_feat_wide_blocks<9>(wpar, kw, cosine, wp.grid, stream);
+      break;
+    }
+    if (time_stop)
+      (void)hipEventRecord(time_stop, stream);
+    if (err != hipSuccess)
+      return err;
+    const int ggrid = wp.tiles * (kWideQueries / kBlock);
+    switch (kp) {
+    case 24:
+      hipLaunchKernelGGL((feat_wide_gather_kernel<24>), dim3(ggrid),
+                         dim3(kBlock), 0, stream, wpar, wp.grid);
+      break;
+    case 32:
+      hipLaunchKernelGGL((feat_wide_gather_kernel<32>), dim3(ggrid),
+                         dim3(kBlock), 0, stream, wpar, wp.grid);
+      break;
+    case 48:
+      hipLaunchKernelGGL((feat_wide_gather_kernel<48>), dim3(ggrid),
+                         dim3(kBlock), 0, stream, wpar, wp.grid);
+      break;
+    case 64:
+      hipLaunchKernelGGL((feat_wide_gather_kernel<64>), dim3(ggrid),
+                         dim3(kBlock), 0, stream, wpar, wp.grid);
+      break;
+    case 80:
+      hipLaunchKernelGGL((feat_wide_gather_kernel<80>), dim3(ggrid),
+                         dim3(kBlock), 0, stream, wpar, wp.grid);
+      break;
+    default:
+      hipLaunchKernelGGL((feat_wide_gather_kernel<116>), dim3(ggrid),
+                         dim3(kBlock), 0, stream, wpar, wp.grid);
+      break;
+    }
+  } else {
   const int grid = tiles_bound * chunks;
   if (time_start)
     (void)hipEventRecord(time_start, stream);
-  hipError_t err;
   switch (nb) {
   case 3:
     err = launch_knn_feat_blocks<3>(p, kp, cosine, grid, stream);
@@ -464,6 +688,7 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   default:
     launch_feat_merge<116>(p, tiles_bound, stream);
     break;
+  }
   }
   {
     const int waves = kBlock / kWave;

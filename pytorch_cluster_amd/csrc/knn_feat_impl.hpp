@@ -250,6 +250,7 @@ struct KnnFeatParams {
   double *hits;          // [redo_cap][hit_cap] their (distance, row) keys
   int redo_cap;
   int hit_cap;
+  const int *overflow;   // [m] or null: 1 = the first stage lost candidates
   int *out_idx;
   float *out_dist;
   int *out_count;
@@ -343,6 +344,15 @@ __global__ __launch_bounds__(kBlock) void feat_pack_kernel(
         part[1] = a2;
         part[2] = a3;
       }
+      // powers of two for a cut carried by the query's operand
+      // (knn_feat_wide_impl.hpp; queries without one hold zeros there)
+      part[3] = 0x7800u; // 2^15
+      part[4] = 0x5000u; // 2^5
+      part[5] = 0x2800u; // 2^-5
+    } else {
+      part[0] = 0x7800u;
+      part[1] = 0x5000u;
+      part[2] = 0x2800u;
     }
   }
   out[id] = make_uint4(part[0] | (part[1] << 16), part[2] | (part[3] << 16),
@@ -989,6 +999,14 @@ __global__ __launch_bounds__(kBlock) void feat_refine_kernel(KnnFeatParams p) {
       p.redo_q[q] = 0;
       if (fq.odd)
         unresolved();
+    }
+    return;
+  }
+  // a candidate buffer of the query overflowed: its list may lack rows
+  if (p.overflow != nullptr && p.overflow[q] != 0) {
+    if (lane == 0) {
+      p.out_count[q] = 0;
+      unresolved();
     }
     return;
   }
