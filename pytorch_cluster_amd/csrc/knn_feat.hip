@@ -341,10 +341,12 @@ FeatWidePlan feat_wide_plan(int n, int m, int num_segments, int k) {
     if (v >= 1 && v <= 4096)
       w.grid = v;
   }
-  w.cap = (256 + 4 * (k + kFeatSlack) + 63) / 64 * 64;
+  // (per query, piece and half of the wave; a checkpoint tidies a buffer
+  // that is half full, and one that comes within two tiles of its end)
+  w.cap = (96 + 2 * (k + kFeatSlack) + 63) / 64 * 64;
   if (const char *env = std::getenv("PCA_FEAT_WIDE_CAP")) {
     const int v = std::atoi(env);
-    if (v >= 256 && v <= 8192)
+    if (v >= 192 && v <= 8192)
       w.cap = v / 64 * 64;
   }
   w.pieces = (size_t)w.grid + (size_t)w.tiles;
@@ -356,7 +358,8 @@ struct FeatLayout {
   size_t redo_list, redo_tau, hit_count, hits; // threshold scan
   size_t pack, partial, cand; // first pass
   // eight-wave first stage: `partial` is then these four
-  size_t wide_plan = 0, wide_buf = 0, wide_count = 0, wide_lists = 0;
+  size_t wide_plan = 0, wide_buf = 0, wide_count = 0, wide_lists = 0,
+         wide_owners = 0;
   size_t second;              // second pass (reuses the first pass's bytes)
   size_t shared() const {
     return globals + x_norm + x_class + y_norm + tau + redo + over + plan256 +
@@ -422,11 +425,15 @@ static FeatLayout feat_layout(int n, int m, int d, int num_segments, int k) {
     const FeatWidePlan wp = feat_wide_plan(n, m, num_segments, k);
     w.wide_plan = align256(sizeof(int) * ((size_t)num_segments + 1)) +
                   align256(sizeof(long long) * ((size_t)num_segments + 1));
-    w.wide_buf = align256(sizeof(uint2) * wp.pieces * kWideQueries * wp.cap);
-    w.wide_count = align256(sizeof(int) * wp.pieces * kWideQueries);
+    w.wide_buf =
+        align256(sizeof(uint2) * wp.pieces * kWideQueries * 2 * wp.cap);
+    w.wide_count = align256(sizeof(int) * wp.pieces * 2 * kWideQueries);
+    w.wide_owners =
+        align256(sizeof(WideOwner) * (size_t)wp.grid * kWideQueries);
     w.wide_lists = align256(sizeof(float) * (size_t)wp.grid *
                             feat_wide_width(k) * kWideQueries);
-    w.partial = w.wide_plan + w.wide_buf + w.wide_count + w.wide_lists;
+    w.partial = w.wide_plan + w.wide_buf + w.wide_count + w.wide_lists +
+                w.wide_owners;
   } else {
     w.partial = align256(sizeof(double) * tiles * chunks * kk * kFeatQueries);
   }
@@ -594,6 +601,8 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
     wpar.buf_count = reinterpret_cast<int *>(wb);
     wb += lay.wide_count;
     wpar.lists = reinterpret_cast<float *>(wb);
+    wb += lay.wide_lists;
+    wpar.owners = reinterpret_cast<WideOwner *>(wb);
     wpar.overflow = overflow;
     hipLaunchKernelGGL(feat_wide_plan_kernel, dim3(1), dim3(kPlanThreads), 0,
                        stream, in.ptr_x, in.ptr_y, in.n, in.m,

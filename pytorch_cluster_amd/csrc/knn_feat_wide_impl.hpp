@@ -14,8 +14,11 @@
 //     one block each);
 //   * the sorted lists of the other kernel cost registers (one workgroup of
 //     four waves had to hold 128 lists) and issue slots in the loop.  Here a
-//     lane that finds a value below the cut appends (value, row) to the
-//     query's candidate buffer in global memory, and only at checkpoints --
+//     lane that finds a value below the cut parks (value, row) in a small
+//     LDS queue of its own; the queues are written to the queries' candidate
+//     buffers in global memory one tile later (stores that have just been
+//     issued would be waited for together with the tile loads: one counter
+//     covers both); and only at checkpoints --
 //     after 64, 128, 256, ... rows of the piece, or when a buffer fills up --
 //     the lane that owns a query runs the new candidates through a sorted
 //     list of the k smallest VALUES (fp32, one v_med3_f32 per slot and
@@ -56,6 +59,10 @@
 
 #include "knn_feat_impl.hpp"
 
+#ifndef PCA_WIDE_EXP
+#define PCA_WIDE_EXP 0 // (timing experiments: parts of the loop switched off)
+#endif
+
 namespace pca {
 
 constexpr int kWideWaves = 8;
@@ -64,6 +71,7 @@ constexpr int kWideQueries = kWideThreads;       // one owned query per lane
 constexpr int kWideTileRows = 64;                // rows per staged tile (unit)
 constexpr int kWideRing = 4;                     // LDS buffers of the tile ring
 constexpr int kWideMaxDim = 128;
+constexpr int kWideQueue = 8;                    // parked values per lane
 
 // the cut's three fp16 parts are multiplied by these (fp16 bit patterns)
 constexpr uint32_t kWideScale0 = 0x7800u; // 2^15
@@ -74,11 +82,38 @@ struct KnnFeatWideParams {
   KnnFeatParams base;
   const int *tile_start;        // [num_segments + 1] first 512-query tile
   const long long *unit_start;  // [num_segments + 1] first (tile, unit) pair
-  int cap;                      // buffer entries per (piece, query)
-  uint2 *buf;                   // [pieces][8 waves][cap][64] (value bits, row)
-  int *buf_count;               // [pieces][512] entries left at the piece's end
+  int cap;                      // buffer entries per (piece, query, half)
+  // candidate buffers: one per query and half of the wave that found the
+  // values (the two lanes that share a query's values write their own)
+  uint2 *buf;                   // [pieces][8 waves][2][cap][64] (value, row)
+  int *buf_count;               // [pieces][2][512] entries at the piece's end
   float *lists;                 // [grid][K][512] the owners' sorted values
+  struct WideOwner *owners;     // [grid][512] the owners' state
   int *overflow;                // [m] 1: a buffer of the query overflowed
+};
+
+// State of the lane that owns a query, kept in global memory between
+// checkpoints (the loop itself has no use for it, and registers are what the
+// loop is short of).
+struct WideOwner {
+  double bound;    // U: upper bound of the query's final k-th distance
+  double fold_err; // largest D of the piece's cuts so far
+  double shift;    // l = value + shift
+  double widen;    // F(l) = (l + widen) * grow
+  float posted;    // what this piece has published to `tau`
+  float tau_seen;  // what the query's other pieces have
+  int seen[2];     // buffer entries the list has taken, per half
+  int flags;       // 1: the list exists, 2: a buffer overflowed
+  int pad;
+};
+
+// What a checkpoint hands back to the loop.
+struct WideCut {
+  uint32_t part01, part2; // the three fp16 parts of -c_rep
+  float recon;            // what is added to a flagged value
+  int fill;               // no cut: every row counts
+  int kept[2];            // entries left in the two buffers
+  int rounds;             // insertions the wave ran (statistics)
 };
 
 // D(c) of the header.
@@ -154,6 +189,193 @@ __device__ __forceinline__ long long wide_stretch(long long total, int grid) {
   return (total + grid - 1) / grid;
 }
 
+// A checkpoint of the lane that owns a query (all lanes of a wave together).
+// The entries the query's two buffers have got since the last checkpoint go
+// through the sorted list of the k smallest values (`list`, [K] floats 512
+// apart); the list's k-th value and what the query's other pieces have
+// published give the bound U; entries above the new cut leave the buffers
+// when one is half full (always at the piece's end, where the counts are
+// written to count_out[0] and count_out[512]).  col_buf: the query's column
+// of the first buffer (entries 64 apart; the second buffer cap entries on).
+template <int K, bool COSINE>
+__device__ __attribute__((noinline)) WideCut wide_checkpoint(
+    WideOwner *o_mem, uint2 *col_buf, float *list, int cap, int count0,
+    int count1, int d, int k, float *tau_q, bool own_active, bool last,
+    int *count_out, int *overflow_q) {
+  // this wave's appends have reached the L2 (the loads below are device-scope
+  // atomics: they see them there; no cache is written back or invalidated)
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  WideOwner o = *o_mem;
+  double bound = o.bound, fold_err = o.fold_err;
+  float posted = o.posted, tau_seen = o.tau_seen;
+  const bool have_list = (o.flags & 1) != 0;
+  bool over = (o.flags & 2) != 0;
+  WideCut out;
+  out.rounds = 0;
+  int n[2] = {count0, count1};
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+    if (n[h] > cap) {
+      over = true;
+      n[h] = cap;
+    }
+  float best[K];
+  if (have_list) {
+#pragma unroll
+    for (int j = 0; j < K; ++j)
+      best[j] = list[(unsigned)(j * kWideQueries)];
+  } else {
+#pragma unroll
+    for (int j = 0; j < K; ++j)
+      best[j] = j < K - k ? -__builtin_inff() : __builtin_inff();
+  }
+  int most[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    uint2 *src = col_buf + (size_t)h * cap * kWave;
+    most[h] = n[h];
+#pragma unroll
+    for (int sh = 32; sh >= 1; sh >>= 1)
+      most[h] = max(most[h], __shfl_xor(most[h], sh));
+    const int first = o.seen[h];
+    int least = first;
+#pragma unroll
+    for (int sh = 32; sh >= 1; sh >>= 1)
+      least = min(least, __shfl_xor(least, sh));
+#pragma unroll 1
+    for (int e = least; e < most[h]; ++e) {
+      float key = __builtin_inff();
+      if (e >= first && e < n[h]) {
+        const unsigned long long w = __hip_atomic_load(
+            reinterpret_cast<const unsigned long long *>(src +
+                                                         (size_t)e * kWave),
+            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        key = __uint_as_float((uint32_t)w);
+      }
+      if (!__any(key < best[K - 1]))
+        continue;
+      ++out.rounds;
+#pragma unroll
+      for (int j = K - 1; j >= 1; --j)
+        best[j] = __builtin_amdgcn_fmed3f(best[j - 1], best[j], key);
+      best[0] = __builtin_fminf(best[0], key);
+    }
+    o.seen[h] = n[h];
+  }
+#pragma unroll
+  for (int j = 0; j < K; ++j)
+    list[(unsigned)(j * kWideQueries)] = best[j];
+
+  // the bound: from the list's k-th value and from the query's other pieces
+  const float kth = best[K - 1];
+  float cut_plain = __builtin_inff(); // s < cut_plain: the row can matter
+  if (own_active) {
+    if (kth < __builtin_inff()) {
+      const double l = (double)kth + o.shift;
+      const double u = (l + o.widen + 2.0 * fold_err) *
+                       (COSINE ? 1.0 : feat_grow(d));
+      bound = u < bound ? u : bound;
+    }
+    float own = bound < 3.0e38 ? feat_float_above(bound) : __builtin_inff();
+    own = __builtin_fmaxf(own, 0.0f);
+    const float now = __hip_atomic_load(tau_q, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+    tau_seen = __builtin_fminf(tau_seen, now);
+    if (own < tau_seen && (own < posted * 0.999f || (last && own < posted))) {
+      __hip_atomic_fetch_min(reinterpret_cast<int *>(tau_q),
+                             (int)__float_as_uint(own), __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+      posted = own;
+    } else if (tau_seen < posted) {
+      posted = tau_seen;
+      bound = (double)tau_seen < bound ? (double)tau_seen : bound;
+    }
+    if (bound < __builtin_inf())
+      cut_plain = feat_float_above(bound - o.shift);
+  } else {
+    cut_plain = -__builtin_inff();
+  }
+
+  // entries above the new cut leave the buffers
+  const bool tidy = __any(n[0] > cap / 2 || n[1] > cap / 2) || last;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    if (tidy) {
+      uint2 *src = col_buf + (size_t)h * cap * kWave;
+      int kept = 0;
+#pragma unroll 1
+      for (int e = 0; e < most[h]; ++e) {
+        if (e < n[h]) {
+          const unsigned long long w = __hip_atomic_load(
+              reinterpret_cast<const unsigned long long *>(src +
+                                                           (size_t)e * kWave),
+              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (__uint_as_float((uint32_t)w) < cut_plain) {
+            __hip_atomic_store(reinterpret_cast<unsigned long long *>(
+                                   src + (size_t)kept * kWave),
+                               w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            ++kept;
+          }
+        }
+      }
+      n[h] = kept;
+      o.seen[h] = kept;
+    }
+    out.kept[h] = n[h];
+  }
+  o.bound = bound;
+  o.posted = posted;
+  o.tau_seen = tau_seen;
+  o.flags = 1 | (over ? 2 : 0);
+  out.part01 = 0;
+  out.part2 = 0;
+  out.recon = 0.0f;
+  out.fill = 0;
+  if (last) {
+    count_out[0] = n[0];
+    count_out[kWideQueries] = n[1];
+    if (over && overflow_q != nullptr)
+      *overflow_q = 1;
+    return out;
+  }
+
+  // the cut for the query's operand
+  uint32_t part[3] = {0, 0, 0};
+  float my_recon = 0.0f;
+  bool my_fill = own_active;
+  if (own_active && cut_plain < __builtin_inff()) {
+    const double c0 = (double)cut_plain;
+    const double want = c0 + wide_fold_err(d, c0) * 1.002 + 1e-30;
+    double rep = 0.0;
+    if (wide_cut_parts(want, part, rep)) {
+      const double err = wide_fold_err(d, rep);
+      // (rep >= want covers D(rep) as long as rep is within 0.2 % of c0;
+      // checked, not assumed)
+      if (rep >= c0 + err) {
+        // (the operand carries -c_rep)
+#pragma unroll
+        for (int i = 0; i < 3; ++i)
+          part[i] = part[i] ? part[i] ^ 0x8000u : 0u;
+        my_fill = false;
+        my_recon = wide_float_below(rep - err);
+        // (the list may hold values of every cut so far)
+        fold_err = err > fold_err ? err : fold_err;
+      } else {
+        part[0] = part[1] = part[2] = 0;
+      }
+    } else {
+      part[0] = part[1] = part[2] = 0;
+    }
+  }
+  o.fold_err = fold_err;
+  *o_mem = o;
+  out.part01 = part[0] | (part[1] << 16);
+  out.part2 = part[2];
+  out.recon = my_recon;
+  out.fill = my_fill ? 1 : 0;
+  return out;
+}
+
 // K: width of the owners' lists (>= k; the first K - k slots hold -inf).
 template <int NB, int K, bool COSINE>
 __global__ __launch_bounds__(kWideThreads, 1) void knn_feat_wide_kernel(
@@ -172,7 +394,8 @@ __global__ __launch_bounds__(kWideThreads, 1) void knn_feat_wide_kernel(
 
   __shared__ __attribute__((aligned(16))) uint4 xs[RING][TILE_UNITS];
   __shared__ __attribute__((aligned(16))) uint4 dump[kWideThreads][4];
-  __shared__ int cnt[kWideQueries];
+  // parked (value, row | block << 31) pairs of every lane: a ring of QCAP
+  __shared__ uint2 queue[kWideQueue][kWideThreads];
 
   if (p.globals->odd_rows != 0)
     return; // everything is searched by the other kernel
@@ -290,30 +513,43 @@ __global__ __launch_bounds__(kWideThreads, 1) void knn_feat_wide_kernel(
     }
 
     // ---- owner state -------------------------------------------------------
-    double bound = __builtin_inf(); // U of the owned query
-    float posted = __builtin_inff();
-    float tau_seen = own_valid
-                         ? __hip_atomic_load(&p.tau[q_own], __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT)
-                         : __builtin_inff();
-    double fold_err = 0.0; // largest D of the piece's cuts so far
-    int seen = 0;          // buffer entries the list has taken
-    bool have_list = false;
-    bool over = false;
+    WideOwner *const my_owner =
+        P.owners + (size_t)blockIdx.x * kWideQueries + tid;
+    {
+      WideOwner o;
+      o.bound = __builtin_inf();
+      o.fold_err = 0.0;
+      o.shift = fq.shift;
+      o.widen = fq.widen;
+      o.posted = __builtin_inff();
+      o.tau_seen = own_valid
+                       ? __hip_atomic_load(&p.tau[q_own], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT)
+                       : __builtin_inff();
+      o.seen[0] = o.seen[1] = 0;
+      o.flags = 0;
+      o.pad = 0;
+      *my_owner = o;
+    }
     // per block, for the values this lane sees: what is added to a flagged
-    // value, and whether the block's query has no cut yet (every row counts)
+    // value, whether the block's query has no cut yet (every row counts), and
+    // the entries this lane has written to the query's buffer of its half
     float recon[RB] = {0.0f, 0.0f};
     bool fill[RB];
+    int written[RB] = {0, 0};
 #pragma unroll
     for (int b = 0; b < RB; ++b)
       fill[b] = b == half ? own_active : other_active;
     bool need_ckpt = false;
+    bool fresh_stores = false; // stores issued since the last tile request
+    int qh = 0, qt = 0;        // the lane's queue: entries qh .. qt - 1
 
-    cnt[tid] = 0;
+    // (wave-uniform: a scalar base for the stores and loads below)
     uint2 *const my_buf =
-        P.buf + ((size_t)piece * kWideWaves + wave) * P.cap * kWave;
+        P.buf + ((size_t)piece * kWideWaves + wave_u) * 2 * P.cap * kWave;
 
     // ---- tile staging ------------------------------------------------------
+    // (scalar base, one 32-bit lane offset: no per-lane pointers to keep)
     auto request_tile = [&](int t) __attribute__((always_inline)) {
       const uint4 *src = p.x_pack + ((size_t)c_begin + (size_t)t * TILE) * RSU;
       const uint32_t dst = (uint32_t)(uintptr_t)&xs[t % RING][0];
@@ -322,36 +558,60 @@ __global__ __launch_bounds__(kWideThreads, 1) void knn_feat_wide_kernel(
         const int pc = wave_u + kWideWaves * e;
         const int u = pc * kWave + lane;
         if (pc < PIECES && (TILE_UNITS % kWave == 0 || u < TILE_UNITS)) {
-          const uint4 *g = src + u;
+          const uint4 *g = src + pc * kWave; // (uniform)
           const uint32_t base = dst + (uint32_t)pc * (kWave * 16);
-          asm volatile("s_mov_b32 m0, %1\n\t"
+          asm volatile("s_mov_b32 m0, %2\n\t"
                        "s_nop 0\n\t"
-                       "global_load_lds_dwordx4 %0, off"
+                       "global_load_lds_dwordx4 %0, %1"
                        :
-                       : "v"(g), "s"(base)
+                       : "v"(lane * 16), "s"(g), "s"(base)
                        : "memory");
         }
       }
     };
-    __syncthreads(); // cnt is clear; everybody has left the previous piece
+    __syncthreads(); // everybody has left the previous piece
 #pragma unroll
     for (int r = 0; r < RING - 1; ++r)
       if (r < num_tiles)
         request_tile(r);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    // ---- appending a flagged value ------------------------------------------
-    auto append = [&](int b, float value, int row, bool on)
-                      __attribute__((always_inline)) {
+    // ---- parked values -------------------------------------------------------
+    // The queues go to the buffers: entry (value, row) of block b to slot
+    // written[b] of the buffer of (query, this lane's half).
+    auto flush = [&]() __attribute__((always_inline)) {
+#pragma unroll 1
+      while (__any(qh != qt)) {
+        if (qh != qt) {
+          const uint2 e = queue[qh & (kWideQueue - 1)][tid];
+          ++qh;
+          const int b = (int)(e.y >> 31);
+          const int at = b ? written[1] : written[0];
+          written[0] += b ? 0 : 1;
+          written[1] += b ? 1 : 0;
+          int slot = lane;
+          asm volatile("" : "+v"(slot));
+          slot = (slot & 31) + b * 32 + (slot >> 5) * P.cap * kWave;
+          if (at < P.cap)
+            *reinterpret_cast<uint2 *>(reinterpret_cast<char *>(my_buf) +
+                                       (unsigned)((at * kWave + slot) * 8)) =
+                make_uint2(e.x, e.y & 0x7fffffffu);
+          if (at >= P.cap - TILE)
+            need_ckpt = true;
+        }
+      }
+    };
+    // parks a flagged value (the queue is flushed first when a lane's is full)
+    auto park = [&](int b, float value, int row, bool on)
+                    __attribute__((always_inline)) {
+      if (__any(on && qt - qh >= kWideQueue)) {
+        flush();
+        fresh_stores = true;
+      }
       if (on) {
-        const int at = __hip_atomic_fetch_add(
-            &cnt[wave * kWave + b * 32 + col], 1, __ATOMIC_RELAXED,
-            __HIP_MEMORY_SCOPE_WORKGROUP);
-        if (at < P.cap)
-          my_buf[(size_t)at * kWave + b * 32 + col] =
-              make_uint2(__float_as_uint(value), (uint32_t)row);
-        if (at >= P.cap - 3 * TILE)
-          need_ckpt = true;
+        queue[qt & (kWideQueue - 1)][tid] = make_uint2(
+            __float_as_uint(value), (uint32_t)row | ((uint32_t)b << 31));
+        ++qt;
       }
     };
 
@@ -404,13 +664,13 @@ __global__ __launch_bounds__(kWideThreads, 1) void knn_feat_wide_kernel(
         return;
       PCA_WSTAT(1, 1);
       const int row0 = c_begin + pos0 + 4 * half;
-      if (!tail && !__any(several)) {
+      if ((PCA_WIDE_EXP & 2) || (!tail && !__any(several))) {
         // at most one flagged value per lane and block: it is the minimum
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
           const int v = __builtin_clz(mask[b] | 1u) - 16;
-          append(b, lo[b] + rec[b], row0 + 8 * (v >> 2) + (v & 3),
-                 mask[b] != 0);
+          park(b, lo[b] + rec[b], row0 + 8 * (v >> 2) + (v & 3),
+               mask[b] != 0);
         }
         return;
       }
@@ -437,178 +697,61 @@ __global__ __launch_bounds__(kWideThreads, 1) void knn_feat_wide_kernel(
           const bool on = bits != 0;
           bits &= ~(0x8000u >> v);
           const float s = on ? mine[v] : 0.0f;
-          append(b, s + rec[b], row0 + 8 * (v >> 2) + (v & 3), on);
+          park(b, s + rec[b], row0 + 8 * (v >> 2) + (v & 3), on);
           PCA_WSTAT(3, 1);
         }
       }
     };
 
     // ---- checkpoint: the owners take their new candidates in ----------------
+    // (a call, not inlined: the rare path's registers stay out of the loop's)
     auto checkpoint = [&](bool last) __attribute__((always_inline)) {
       PCA_WSTAT(4, 1);
-      // this wave's appends have reached memory
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "agent");
-      int n = cnt[tid];
-      if (n > P.cap) {
-        over = true;
-        n = P.cap;
-      }
-      float best[K];
-      if (have_list) {
-#pragma unroll
-        for (int j = 0; j < K; ++j)
-          best[j] = my_list[(size_t)j * kWideQueries];
-      } else {
-#pragma unroll
-        for (int j = 0; j < K; ++j)
-          best[j] = j < K - p.k ? -__builtin_inff() : __builtin_inff();
-      }
-      const uint2 *col_buf = my_buf + lane;
-      int most = n;
-#pragma unroll
-      for (int sh = 32; sh >= 1; sh >>= 1)
-        most = max(most, __shfl_xor(most, sh));
-      const int first = seen;
-      int least = first;
-#pragma unroll
-      for (int sh = 32; sh >= 1; sh >>= 1)
-        least = min(least, __shfl_xor(least, sh));
-#pragma unroll 1
-      for (int e = least; e < most; ++e) {
-        float key = __builtin_inff();
-        if (e >= first && e < n) {
-          const unsigned long long w = __hip_atomic_load(
-              reinterpret_cast<const unsigned long long *>(col_buf +
-                                                           (size_t)e * kWave),
-              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          key = __uint_as_float((uint32_t)w);
-        }
-        if (!__any(key < best[K - 1]))
-          continue;
-        PCA_WSTAT(5, 1);
-#pragma unroll
-        for (int j = K - 1; j >= 1; --j)
-          best[j] = __builtin_amdgcn_fmed3f(best[j - 1], best[j], key);
-        best[0] = __builtin_fminf(best[0], key);
-      }
-      seen = n;
-#pragma unroll
-      for (int j = 0; j < K; ++j)
-        my_list[(size_t)j * kWideQueries] = best[j];
-      have_list = true;
-
-      // the bound: from the list's k-th value and from the query's other
-      // pieces
-      const float kth = best[K - 1];
-      float cut_plain = __builtin_inff(); // s < cut_plain: the row can matter
-      if (own_active) {
-        if (kth < __builtin_inff()) {
-          const double l = (double)kth + fq.shift;
-          const double u = (l + fq.widen + 2.0 * fold_err) * fq.grow;
-          bound = u < bound ? u : bound;
-        }
-        float own = bound < 3.0e38 ? feat_float_above(bound) : __builtin_inff();
-        own = __builtin_fmaxf(own, 0.0f);
-        if (q_own < y_end) {
-          const float now = __hip_atomic_load(&p.tau[q_own], __ATOMIC_RELAXED,
-                                              __HIP_MEMORY_SCOPE_AGENT);
-          tau_seen = __builtin_fminf(tau_seen, now);
-        }
-        if (own < tau_seen && (own < posted * 0.999f || (last && own < posted))) {
-          __hip_atomic_fetch_min(reinterpret_cast<int *>(&p.tau[q_own]),
-                                 (int)__float_as_uint(own), __ATOMIC_RELAXED,
-                                 __HIP_MEMORY_SCOPE_AGENT);
-          posted = own;
-        } else if (tau_seen < posted) {
-          posted = tau_seen;
-          bound = (double)tau_seen < bound ? (double)tau_seen : bound;
-        }
-        if (bound < __builtin_inf())
-          cut_plain = feat_float_above(bound - fq.shift);
-      } else {
-        cut_plain = -__builtin_inff();
-      }
-
-      // entries above the new cut leave the buffer (always at the end; before
-      // that when the buffer is half full)
-      if (__any(n > P.cap / 2) || last) {
-        int kept = 0;
-#pragma unroll 1
-        for (int e = 0; e < most; ++e) {
-          if (e < n) {
-            uint2 *src = const_cast<uint2 *>(col_buf) + (size_t)e * kWave;
-            const unsigned long long w = __hip_atomic_load(
-                reinterpret_cast<const unsigned long long *>(src),
-                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (__uint_as_float((uint32_t)w) < cut_plain) {
-              __hip_atomic_store(
-                  reinterpret_cast<unsigned long long *>(
-                      const_cast<uint2 *>(col_buf) + (size_t)kept * kWave),
-                  w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-              ++kept;
-            }
-          }
-        }
-        n = kept;
-        seen = kept;
-        cnt[tid] = kept;
-      }
-      if (last) {
-        P.buf_count[(size_t)piece * kWideQueries + tid] = n;
-        if (over && own_valid)
-          P.overflow[q_own] = 1;
+      flush();
+      // the entries of the owned query: this lane's, and the other half's
+      const int mine = half ? written[1] : written[0];
+      const int theirs = (int)partner((uint32_t)(half ? written[0] : written[1]));
+      const WideCut cut = wide_checkpoint<K, COSINE>(
+          my_owner, my_buf + lane, my_list, P.cap, half ? theirs : mine,
+          half ? mine : theirs, d, p.k, own_valid ? &p.tau[q_own] : nullptr,
+          own_active, last,
+          &P.buf_count[(size_t)piece * 2 * kWideQueries + tid],
+          own_valid ? &P.overflow[q_own] : nullptr);
+      PCA_WSTAT(5, cut.rounds);
+      fresh_stores = true;
+      if (last)
         return;
-      }
-
-      // the cut goes into the query's operand
-      uint32_t part[3] = {0, 0, 0};
-      float my_recon = 0.0f;
-      bool my_fill = own_active;
-      if (own_active && cut_plain < __builtin_inff()) {
-        const double c0 = (double)cut_plain;
-        double want = c0 + wide_fold_err(d, c0) * 1.002 + 1e-30;
-        double rep = 0.0;
-        if (wide_cut_parts(want, part, rep)) {
-          const double err = wide_fold_err(d, rep);
-          // (rep >= want >= c0 + D(c0) 1.002 covers D(rep) as long as rep is
-          // within 0.2 % of c0; checked, not assumed)
-          if (rep >= c0 + err) {
-            // (the operand carries -c_rep)
-#pragma unroll
-            for (int i = 0; i < 3; ++i)
-              part[i] = part[i] ? part[i] ^ 0x8000u : 0u;
-            my_fill = false;
-            my_recon = wide_float_below(rep - err);
-            // (the list may hold values of every cut so far)
-            fold_err = err > fold_err ? err : fold_err;
-          } else {
-            part[0] = part[1] = part[2] = 0;
-          }
-        }
-      }
-      if (!own_active) {
-        my_fill = false;
-      }
+      // what is left in the buffers: the own half's count, and the other
+      // half's back to the lane that writes there
       {
-        // components 3..5 of the lower lanes' registers (block 0's queries),
-        // 0..2 of the upper lanes' (block 1's): k = 3..5 and 8..10
+        const int kept_mine = half ? cut.kept[1] : cut.kept[0];
+        const int kept_theirs = half ? cut.kept[0] : cut.kept[1];
+        const int back = (int)partner((uint32_t)kept_theirs);
+        written[0] = half ? back : kept_mine;
+        written[1] = half ? kept_mine : back;
+      }
+      // the cut goes into the query's operand: components 3..5 of the lower
+      // lanes' registers (block 0's queries), 0..2 of the upper lanes'
+      // (block 1's): k = 3..5 and 8..10
+      {
         uint4 w0 = __builtin_bit_cast(uint4, yh[0][NB - 1]);
         uint4 w1 = __builtin_bit_cast(uint4, yh[1][NB - 1]);
         if (half == 0) {
-          w0.y = (w0.y & 0xffffu) | (part[0] << 16);
-          w0.z = part[1] | (part[2] << 16);
+          w0.y = (w0.y & 0xffffu) | (cut.part01 << 16);
+          w0.z = (cut.part01 >> 16) | (cut.part2 << 16);
         } else {
-          w1.x = part[0] | (part[1] << 16);
-          w1.y = part[2];
+          w1.x = cut.part01;
+          w1.y = cut.part2;
         }
         yh[0][NB - 1] = __builtin_bit_cast(feat_f16x8_t, w0);
         yh[1][NB - 1] = __builtin_bit_cast(feat_f16x8_t, w1);
       }
-      const float other_recon = __uint_as_float(partner(__float_as_uint(my_recon)));
+      const float other_recon =
+          __uint_as_float(partner(__float_as_uint(cut.recon)));
+      const bool my_fill = cut.fill != 0;
       const bool other_fill = partner(my_fill ? 1u : 0u) != 0;
-      recon[0] = half ? other_recon : my_recon;
-      recon[1] = half ? my_recon : other_recon;
+      recon[0] = half ? other_recon : cut.recon;
+      recon[1] = half ? cut.recon : other_recon;
       fill[0] = half ? other_fill : my_fill;
       fill[1] = half ? my_fill : other_fill;
       need_ckpt = false;
@@ -624,7 +767,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void knn_feat_wide_kernel(
                     __attribute__((always_inline)) {
       const uint4 *arow =
           &xs[t % RING][(sub * kFeatStep + col) * RSU + half];
-      constexpr int AHEAD = 4;
+      constexpr int AHEAD = 3;
       uint4 window[AHEAD];
 #pragma unroll
       for (int o = 0; o < AHEAD && o < NB; ++o)
@@ -656,7 +799,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void knn_feat_wide_kernel(
       for (int b = 0; b < RB; ++b)
         asm volatile("" : "+v"(mask[b]), "+v"(lo[b]));
       __builtin_amdgcn_sched_barrier(0);
-      if (old_valid)
+      if (old_valid && !(PCA_WIDE_EXP & 1))
         events(old, mask, lo, old_pos0, rec_old, all_old);
     };
 
@@ -672,6 +815,10 @@ __global__ __launch_bounds__(kWideThreads, 1) void knn_feat_wide_kernel(
       int next_ckpt = 1;
 #pragma unroll 1
       for (int t = 0; t <= num_tiles; ++t) {
+        // what the last tile's steps parked goes to the buffers now: by the
+        // time this tile's end waits for the next one's loads, these stores
+        // are a tile old
+        flush();
         // this wave's pieces of tile t have arrived (awaited below); after
         // the barrier so have everybody's, and everybody is done with tile
         // t - 1
@@ -689,7 +836,8 @@ __global__ __launch_bounds__(kWideThreads, 1) void knn_feat_wide_kernel(
              all_b);
         // (one call site: at the piece's end the same code writes the counts)
         const bool last = t == num_tiles;
-        if (last || t == next_ckpt || __any(need_ckpt)) {
+        if (last || (!(PCA_WIDE_EXP & 16) &&
+                     (t == next_ckpt || __any(need_ckpt)))) {
           checkpoint(last);
           if (t == next_ckpt)
             next_ckpt *= 2;
@@ -706,13 +854,16 @@ __global__ __launch_bounds__(kWideThreads, 1) void knn_feat_wide_kernel(
         if (t + 1 < num_tiles) {
           // requests in flight beyond tile t + 1: tiles t + 2 .. t + RING - 1
           const int newer = min(num_tiles - (t + 2), RING - 2);
-          if (newer >= 2)
+          // (stores issued after the last request would be counted as the
+          // newest requests: then everything is waited for)
+          if (newer >= 2 && !fresh_stores)
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (MAXP - 1))
                          : "memory");
-          else if (newer == 1)
+          else if (newer == 1 && !fresh_stores)
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(MAXP - 1) : "memory");
           else
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          fresh_stores = false;
         }
       }
     }
@@ -761,22 +912,28 @@ __global__ __launch_bounds__(kBlock) void feat_wide_gather_kernel(
     const int wave = local / kWave, lane = local % kWave;
     for (int w = w_lo; w <= w_hi; ++w) {
       const int piece = w + tile;
-      int n = P.buf_count[(size_t)piece * kWideQueries + local];
-      int most = n;
+#pragma unroll 1
+      for (int h = 0; h < 2; ++h) {
+        const int n =
+            P.buf_count[((size_t)piece * 2 + h) * kWideQueries + local];
+        int most = n;
 #pragma unroll
-      for (int sh = 32; sh >= 1; sh >>= 1)
-        most = max(most, __shfl_xor(most, sh));
-      const uint2 *src =
-          P.buf + ((size_t)piece * kWideWaves + wave) * P.cap * kWave + lane;
-      for (int e = 0; e < most; ++e) {
-        double key = feat_empty_key();
-        if (e < n) {
-          const uint2 w2 = src[(size_t)e * kWave];
-          key = make_key(__uint_as_float(w2.x), w2.y);
+        for (int sh = 32; sh >= 1; sh >>= 1)
+          most = max(most, __shfl_xor(most, sh));
+        const uint2 *src = P.buf +
+                           (((size_t)piece * kWideWaves + wave) * 2 + h) *
+                               P.cap * kWave +
+                           lane;
+        for (int e = 0; e < most; ++e) {
+          double key = feat_empty_key();
+          if (e < n) {
+            const uint2 w2 = src[(size_t)e * kWave];
+            key = make_key(__uint_as_float(w2.x), w2.y);
+          }
+          if (!__any(key < best[KP - 1]))
+            continue;
+          sorted_insert<KP>(best, key);
         }
-        if (!__any(key < best[KP - 1]))
-          continue;
-        sorted_insert<KP>(best, key);
       }
     }
   }
