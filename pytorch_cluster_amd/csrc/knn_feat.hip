@@ -596,6 +596,12 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
     wpar.tile_start = tile_start;
     wpar.unit_start = unit_start;
     wpar.cap = wp.cap;
+    wpar.ckpt_growth = 32;
+    if (const char *env = std::getenv("PCA_FEAT_WIDE_CKPT")) {
+      const int v = std::atoi(env);
+      if (v >= 17 && v <= 64)
+        wpar.ckpt_growth = v;
+    }
     wpar.buf = reinterpret_cast<uint2 *>(wb);
     wb += lay.wide_buf;
     wpar.buf_count = reinterpret_cast<int *>(wb);

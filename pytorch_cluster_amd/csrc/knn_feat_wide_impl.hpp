@@ -83,6 +83,7 @@ struct KnnFeatWideParams {
   const int *tile_start;        // [num_segments + 1] first 512-query tile
   const long long *unit_start;  // [num_segments + 1] first (tile, unit) pair
   int cap;                      // buffer entries per (piece, query, half)
+  int ckpt_growth;              // next checkpoint at tile t * this / 16 (> 16)
   // candidate buffers: one per query and half of the wave that found the
   // values (the two lanes that share a query's values write their own)
   uint2 *buf;                   // [pieces][8 waves][2][cap][64] (value, row)
@@ -242,23 +243,32 @@ __device__ __attribute__((noinline)) WideCut wide_checkpoint(
 #pragma unroll
     for (int sh = 32; sh >= 1; sh >>= 1)
       least = min(least, __shfl_xor(least, sh));
+    // (CHUNK loads in flight at a time: one after the other, each would
+    // wait a full trip to the L2)
+    constexpr int CHUNK = 16;
 #pragma unroll 1
-    for (int e = least; e < most[h]; ++e) {
-      float key = __builtin_inff();
-      if (e >= first && e < n[h]) {
-        const unsigned long long w = __hip_atomic_load(
-            reinterpret_cast<const unsigned long long *>(src +
-                                                         (size_t)e * kWave),
-            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        key = __uint_as_float((uint32_t)w);
-      }
-      if (!__any(key < best[K - 1]))
-        continue;
-      ++out.rounds;
+    for (int e0 = least; e0 < most[h]; e0 += CHUNK) {
+      float keys[CHUNK];
 #pragma unroll
-      for (int j = K - 1; j >= 1; --j)
-        best[j] = __builtin_amdgcn_fmed3f(best[j - 1], best[j], key);
-      best[0] = __builtin_fminf(best[0], key);
+      for (int i = 0; i < CHUNK; ++i) {
+        const int e = e0 + i;
+        keys[i] = __builtin_inff();
+        if (e >= first && e < n[h])
+          keys[i] = __uint_as_float(__hip_atomic_load(
+              reinterpret_cast<const uint32_t *>(src + (size_t)e * kWave),
+              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      }
+#pragma unroll
+      for (int i = 0; i < CHUNK; ++i) {
+        const float key = keys[i];
+        if (!__any(key < best[K - 1]))
+          continue;
+        ++out.rounds;
+#pragma unroll
+        for (int j = K - 1; j >= 1; --j)
+          best[j] = __builtin_amdgcn_fmed3f(best[j - 1], best[j], key);
+        best[0] = __builtin_fminf(best[0], key);
+      }
     }
     o.seen[h] = n[h];
   }
@@ -303,17 +313,28 @@ __device__ __attribute__((noinline)) WideCut wide_checkpoint(
     if (tidy) {
       uint2 *src = col_buf + (size_t)h * cap * kWave;
       int kept = 0;
+      constexpr int CHUNK = 8;
 #pragma unroll 1
-      for (int e = 0; e < most[h]; ++e) {
-        if (e < n[h]) {
-          const unsigned long long w = __hip_atomic_load(
-              reinterpret_cast<const unsigned long long *>(src +
-                                                           (size_t)e * kWave),
-              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          if (__uint_as_float((uint32_t)w) < cut_plain) {
+      for (int e0 = 0; e0 < most[h]; e0 += CHUNK) {
+        unsigned long long w[CHUNK];
+#pragma unroll
+        for (int i = 0; i < CHUNK; ++i) {
+          w[i] = 0;
+          if (e0 + i < n[h])
+            w[i] = __hip_atomic_load(
+                reinterpret_cast<const unsigned long long *>(
+                    src + (size_t)(e0 + i) * kWave),
+                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // (kept <= e0 + i: a store never reaches an entry not yet loaded)
+#pragma unroll
+        for (int i = 0; i < CHUNK; ++i) {
+          if (e0 + i < n[h] &&
+              __uint_as_float((uint32_t)w[i]) < cut_plain) {
             __hip_atomic_store(reinterpret_cast<unsigned long long *>(
                                    src + (size_t)kept * kWave),
-                               w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                               w[i], __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
             ++kept;
           }
         }
@@ -840,7 +861,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void knn_feat_wide_kernel(
                      (t == next_ckpt || __any(need_ckpt)))) {
           checkpoint(last);
           if (t == next_ckpt)
-            next_ckpt *= 2;
+            next_ckpt = max(t + 1, (int)((long long)t * P.ckpt_growth >> 4));
         }
         if (last)
           break;
@@ -924,15 +945,24 @@ __global__ __launch_bounds__(kBlock) void feat_wide_gather_kernel(
                            (((size_t)piece * kWideWaves + wave) * 2 + h) *
                                P.cap * kWave +
                            lane;
-        for (int e = 0; e < most; ++e) {
-          double key = feat_empty_key();
-          if (e < n) {
-            const uint2 w2 = src[(size_t)e * kWave];
-            key = make_key(__uint_as_float(w2.x), w2.y);
+        constexpr int CHUNK = 8; // loads in flight at a time
+        for (int e0 = 0; e0 < most; e0 += CHUNK) {
+          uint2 w2[CHUNK];
+#pragma unroll
+          for (int i = 0; i < CHUNK; ++i) {
+            w2[i] = make_uint2(0u, 0u);
+            if (e0 + i < n)
+              w2[i] = src[(size_t)(e0 + i) * kWave];
           }
-          if (!__any(key < best[KP - 1]))
-            continue;
-          sorted_insert<KP>(best, key);
+#pragma unroll
+          for (int i = 0; i < CHUNK; ++i) {
+            const double key = e0 + i < n
+                                   ? make_key(__uint_as_float(w2[i].x), w2[i].y)
+                                   : feat_empty_key();
+            if (!__any(key < best[KP - 1]))
+              continue;
+            sorted_insert<KP>(best, key);
+          }
         }
       }
     }
