@@ -16,6 +16,8 @@ term of the chain: 0.13 x 2^-10 at 256 components, 0.26 x 2^-10 at 512) unused.
 import numpy as np
 import pytest
 
+from helpers import stable_seed
+
 def rho_of(d):
     """2^-9 up to 256 components, 2^-8 beyond (feat_rho)."""
     return 1.0 / 512.0 if d <= 256 else 1.0 / 256.0
@@ -140,7 +142,7 @@ def test_rounding_midpoints_with_one_sign(d):
 @pytest.mark.parametrize("case", ["mixed", "flush_limit", "tiny", "huge",
                                   "outlier", "near_duplicates"])
 def test_scales(case):
-    rng = np.random.default_rng(hash(case) % 2 ** 32)
+    rng = np.random.default_rng(stable_seed(case))
     d = 96
     if case == "mixed":
         x = midpoint_rows(rng, 300, d, rng.integers(-12, 1, (300, 1)), -1)
@@ -165,6 +167,128 @@ def test_scales(case):
         x = np.repeat(base, 30, 0) * (1 + 1e-6 * rng.standard_normal((300, d)))
         y = base * (1 + 1e-6 * rng.standard_normal((10, d)))
     check(x, y)
+
+
+# ---- the cut inside the matrix product (knn_feat_wide_impl.hpp) --------------
+# The eight-wave first stage lets the chain of matrix instructions subtract the
+# cut: the query's operand carries -c_rep as three fp16 numbers, the packed
+# rows the powers of two 2^15, 2^5, 2^-5.  Checked here, with the chain
+# modelled as fp32 additions in several orders: c_rep is what its parts say
+# and lies above the cut by the rounding the three extra terms can add, D(c);
+# every pair the plain test `s < cut` must flag comes out negative; and the
+# value kept for a flagged pair, acc + float_below(c_rep - D), stays within
+# [S - room - 2 D, S + room] of the exact sum S.
+
+def h_down_any(v):
+    """h_down() for the kernel's feat_h_down (v >= 0)."""
+    return h_down(v)
+
+
+def cut_parts(c):
+    """wide_cut_parts: (p0, p1, p2) as fp16 values with sign, and rep."""
+    neg = c < 0.0
+    a = -c if neg else c
+    if not a < 2.0e9:
+        return None
+    a0 = h_down_any(a / 32768.0)
+    r0 = a - a0 * 32768.0
+    a1 = h_down_any(r0 / 32.0)
+    r1 = r0 - a1 * 32.0
+    a2 = h_down_any(r1 * 32.0)
+    r2 = r1 - a2 / 32.0
+    if not neg and r2 > 0.0:
+        a2 = 2.0 ** -14 if a2 == 0.0 else float(
+            np.nextafter(np.float16(a2), np.float16(np.inf)))
+        if a2 > 65504.0:
+            return None
+        r2 = r1 - a2 / 32.0
+    mag = a - r2
+    sign = -1.0 if neg else 1.0
+    return (sign * a0, sign * a1, sign * a2), sign * mag
+
+
+def fold_err(d, c):
+    return (d + 23) * 2.0 ** -22 * abs(c)
+
+
+def float_below(v):
+    f = np.float32(v)
+    if float(f) > v:
+        f = np.nextafter(f, np.float32(-np.inf))
+    return f
+
+
+def chain(terms, order):
+    acc = np.float32(0.0)
+    for i in order:
+        acc = np.float32(acc + np.float32(terms[i]))  # (terms are fp32-exact)
+    return acc
+
+
+@pytest.mark.parametrize("d", [16, 64, 128])
+def test_cut_inside_the_product(d):
+    rng = np.random.default_rng(stable_seed("fold", d))
+    RHO = rho_of(d)
+    x = rng.standard_normal((40, d)).astype(np.float32)
+    x[:8] *= 10.0 ** rng.integers(-4, 1, (8, 1))
+    y = (x[:6] + 0.05 * rng.standard_normal((6, d))).astype(np.float32)
+    inv = inv_sigma(max(np.abs(x).max(), np.abs(y).max()))
+    scale2 = inv * inv
+    xs = (x * np.float32(inv)).astype(np.float32)
+    ys = (y * np.float32(inv)).astype(np.float32)
+    hx = h(xs)
+    hy = h(-2.0 * ys.astype(np.float64))
+    xsq = (x.astype(np.float64) ** 2).sum(1)
+    ysq = (ys.astype(np.float64) ** 2).sum(1)
+    checked = 0
+    for j in range(len(y)):
+        for i in range(len(x)):
+            w = float(xsq[i]) * scale2 * (1.0 - RHO)
+            a1 = h_down(w / 32768.0)
+            r1 = w - a1 * 32768.0
+            a2 = h_down(r1 / 16.0)
+            r2 = r1 - a2 * 16.0
+            a3 = h_down(r2 * 128.0)
+            base = [a1 * 32768.0, a2 * 16.0, a3 / 128.0] + list(hx[i] * hy[j])
+            total = float(np.sum(np.array(base, dtype=np.float64)))
+            norms = float((xs[i].astype(np.float64) ** 2).sum() + ysq[j])
+            room = max(0.15, (d + 16) * 2.01 / 4096.0) * 2.0 ** -10 * norms
+            # cuts around the pair's own value, far above, below, negative
+            for c0 in (total + room * 1.0001 + 1e-6, total * 1.5 + 3.0,
+                       total - abs(total) * 0.01 - 1.0, abs(total) * 40.0 + 7.0,
+                       -abs(total) * 0.3 - 0.125, 2.0 ** -20):
+                c0 = float(np.float32(c0))
+                got = cut_parts(c0 + fold_err(d, c0) * 1.002 + 1e-30)
+                if got is None:
+                    # beyond the parts' range: the kernel works without a cut
+                    assert abs(c0) > 1.9e9
+                    checked += 1
+                    continue
+                (p0, p1, p2), rep = got
+                for part in (p0, p1, p2):
+                    assert float(np.float16(part)) == part
+                    assert part == 0.0 or abs(part) >= 2.0 ** -14
+                assert rep == p0 * 32768.0 + p1 * 32.0 + p2 / 32.0
+                err = fold_err(d, rep)
+                assert rep >= c0 + err
+                recon = float_below(rep - err)
+                terms = base + [-p0 * 32768.0, -p1 * 32.0, -p2 / 32.0]
+                n = len(terms)
+                orders = [list(range(n)), list(range(n))[::-1],
+                          list(rng.permutation(n)),
+                          # the cut first, then the rest
+                          [n - 3, n - 2, n - 1] + list(range(n - 3))]
+                for order in orders:
+                    acc = chain(terms, order)
+                    bound = (d + 22) * 2.0 ** -22 * (2.01 * norms + abs(rep))
+                    assert abs(float(acc) - (total - rep)) <= bound
+                    if total + room <= c0:
+                        assert acc < 0.0, "a pair the plain test flags got away"
+                    key = float(np.float32(acc + recon))
+                    assert key <= total + room
+                    assert key >= total - room - 2.0 * err - 1e-30
+                checked += 1
+    assert checked == 40 * 6 * 6
 
 
 # ---- the split-bf16 filter of the exact matrix-core kernel --------------------

@@ -17,7 +17,7 @@ from pytorch_cluster_amd import capi, testing  # noqa: E402
 from gpu_common import (use_strategy, DEV, dev, gpu_knn, oracle_knn_edges,  # noqa: E402
                         ragged_ptrs)
 from helpers import (brute_force_knn_f64, check_knn_against_exact,  # noqa
-                     to_set)
+                     stable_seed, to_set)
 
 
 def tensor(v, dtype=torch.float32):
@@ -226,7 +226,7 @@ def test_prefilter_never_drops_a_neighbour(oracle, lowd_path, d, k, case):
     # the expanded-form pre-filter must stay conservative where it is least
     # accurate: tight clusters far from the origin, coordinates near the
     # overflow / underflow ends of fp32, wildly mixed scales
-    rng = np.random.default_rng(hash((d, k, case)) % (2 ** 32))
+    rng = np.random.default_rng(stable_seed((d, k, case)))
     n, m = 5000, 600
     if case == "offset":
         x = 1000.0 + 1e-2 * rng.standard_normal((n, d))
@@ -267,7 +267,7 @@ def test_split_bf16_filter_edge_cases(oracle, d, k, case):
     # values that round up across a power of two, rows around the norm above
     # which the filter is switched off, non-finite rows and queries mixed in,
     # and segments much shorter than a 32-row step
-    rng = np.random.default_rng(hash((d, k, case, "bf16")) % (2 ** 32))
+    rng = np.random.default_rng(stable_seed((d, k, case, "bf16")))
     n, m = 6000, 700
     ptr_x = np.array([0, 2500, 6000])
     ptr_y = np.array([0, 300, 700])
@@ -317,7 +317,7 @@ def test_split_bf16_filter_edge_cases(oracle, d, k, case):
 @pytest.mark.parametrize("case", ["parallel", "random", "scaled_copies",
                                   "zero_rows"])
 def test_cosine_prefilter_never_drops_a_neighbour(oracle, d, k, case):
-    rng = np.random.default_rng(hash((d, k, case, "cos")) % (2 ** 32))
+    rng = np.random.default_rng(stable_seed((d, k, case, "cos")))
     n, m = 4000, 500
     if case == "parallel":
         # all rows within a narrow cone: cosine distances ~1e-6, many

@@ -1,4 +1,6 @@
-"""Feature-space kNN with the fp16 matrix-core filter (knn_feat_impl.hpp):
+"""Feature-space kNN with the fp16 matrix-core filter (knn_feat_impl.hpp and,
+for up to 128 components, the eight-wave first stage of
+knn_feat_wide_impl.hpp; every test runs with either):
 parity with the CPU checker where the mechanisms of that path are exercised --
 lists that overflow (near-duplicates: the flagged queries go through the
 second pass), rows and queries the filter cannot represent, 129-512
@@ -9,7 +11,30 @@ import numpy as np
 import pytest
 import torch
 
+import zlib
+
 pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True, params=["four_waves", "eight_waves"])
+def first_stage(request, monkeypatch):
+    """Which first stage serves the calls of a test: the four-wave kernel
+    with its register lists, or (where the shape fits: up to 128 components)
+    the eight-wave kernel with candidate buffers.  Left to itself the library
+    takes the second one from 4,096 queries on."""
+    monkeypatch.setenv("PCA_KNN_FEAT_WIDE",
+                       "1" if request.param == "eight_waves" else "0")
+    return request.param
+
+
+def _only_once_beyond_128(first_stage, d):
+    if d > 128 and first_stage == "eight_waves":
+        pytest.skip("more than 128 components: the four-wave kernel either way")
+
+
+def _seed(*parts):
+    """The same seed in every process (str hashes are salted per run)."""
+    return zlib.crc32(repr(parts).encode())
 
 
 def _run(oracle, x, y, ptr_x, ptr_y, k, cosine=False):
@@ -40,7 +65,9 @@ def _flagged_queries(x, y, k, cosine=False):
                                         (129, 48, True), (24, 33, False),
                                         (64, 40, True), (96, 48, False),
                                         (32, 1, False), (48, 8, True)])
-def test_parity_wide_rows_and_every_list_width(oracle, d, k, cosine):
+def test_parity_wide_rows_and_every_list_width(oracle, first_stage, d, k,
+                                                cosine):
+    _only_once_beyond_128(first_stage, d)
     rng = np.random.default_rng(d * 11 + k)
     n, m = 3000, 500
     x = rng.standard_normal((n, d)).astype(np.float32)
@@ -52,7 +79,9 @@ def test_parity_wide_rows_and_every_list_width(oracle, d, k, cosine):
 
 @pytest.mark.parametrize("d", [20, 128, 200])
 @pytest.mark.parametrize("cosine", [False, True])
-def test_near_duplicates_go_through_the_second_pass(oracle, d, cosine):
+def test_near_duplicates_go_through_the_second_pass(oracle, first_stage, d,
+                                                    cosine):
+    _only_once_beyond_128(first_stage, d)
     # 60 copies (equal up to the last bits) of every cluster centre: far more
     # than 16 rows within the filter's rounding margin of the k-th distance,
     # so the lists cannot be shown complete and the queries are searched again
@@ -76,7 +105,9 @@ def test_near_duplicates_go_through_the_second_pass(oracle, d, cosine):
                                         (257, 49, True), (400, 100, False),
                                         (512, 64, True), (20, 80, False),
                                         (9, 100, True), (384, 33, False)])
-def test_parity_up_to_512_components_and_100_neighbours(oracle, d, k, cosine):
+def test_parity_up_to_512_components_and_100_neighbours(oracle, first_stage,
+                                                        d, k, cosine):
+    _only_once_beyond_128(first_stage, d)
     rng = np.random.default_rng(d * 13 + k)
     n, m = 2500, 300
     x = rng.standard_normal((n, d)).astype(np.float32)
@@ -102,7 +133,9 @@ def _unresolved_queries(x, y, k, cosine=False):
 
 
 @pytest.mark.parametrize("d", [40, 160])
-def test_flagged_queries_beyond_what_the_threshold_scan_holds(oracle, d):
+def test_flagged_queries_beyond_what_the_threshold_scan_holds(oracle,
+                                                              first_stage, d):
+    _only_once_beyond_128(first_stage, d)
     rng = np.random.default_rng(d + 5)
     # (a) 400 exact copies of one row: more rows at the k-th distance than a
     # hit list holds, the query goes on to the full second pass
@@ -166,7 +199,7 @@ def test_rows_and_queries_the_filter_cannot_represent(oracle):
 def test_scales_at_both_ends(oracle, case):
     # one power of two scales all rows into the fp16 range: rows far below the
     # largest one lose their bits there, and the lists must notice
-    rng = np.random.default_rng(hash(case) % 2 ** 32)
+    rng = np.random.default_rng(_seed("scales", case))
     d, n, m, k = 72, 4000, 400, 16
     x = rng.standard_normal((n, d))
     y = rng.standard_normal((m, d))
@@ -206,7 +239,48 @@ def test_many_slices_share_their_bounds(oracle, monkeypatch):
         _run(oracle, x, y, None, None, 24, cosine=True)
 
 
-def test_feature_space_knn_256_full_size_properties(oracle):
+def test_pieces_of_the_eight_wave_stage(oracle, monkeypatch):
+    # the eight-wave stage cuts the (tile of 512 queries, 64 rows) pairs of a
+    # call into as many stretches as it has workgroups: one workgroup that
+    # walks through every tile, pieces of a few rows, several pieces per tile,
+    # and the buffers at their smallest (a checkpoint tidies them more often)
+    monkeypatch.setenv("PCA_KNN_FEAT_WIDE", "1")
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((9000, 48)).astype(np.float32)
+    y = rng.standard_normal((1500, 48)).astype(np.float32)
+    ptr_x = np.array([0, 3000, 3000, 3100, 9000])
+    ptr_y = np.array([0, 700, 800, 900, 1500])
+    for grid, cap in (("1", "192"), ("7", "8192"), ("64", "192"),
+                      ("200", "256")):
+        monkeypatch.setenv("PCA_FEAT_WIDE_GRID", grid)
+        monkeypatch.setenv("PCA_FEAT_WIDE_CAP", cap)
+        _run(oracle, x, y, ptr_x, ptr_y, 20)
+        _run(oracle, x, y, None, None, 70, cosine=True)
+    # rows that arrive ever closer to the queries: every row passes the cut of
+    # its time, the buffers fill up between the scheduled checkpoints
+    monkeypatch.setenv("PCA_FEAT_WIDE_GRID", "2")
+    monkeypatch.setenv("PCA_FEAT_WIDE_CAP", "192")
+    centre = rng.standard_normal(48)
+    radius = np.linspace(30.0, 0.5, 6000)[:, None]
+    xs = (centre + radius * rng.standard_normal((6000, 48))
+          / np.sqrt(48)).astype(np.float32)
+    ys = (centre + 0.01 * rng.standard_normal((600, 48))).astype(np.float32)
+    _run(oracle, xs, ys, None, None, 16)
+
+
+def test_queries_enough_for_the_eight_wave_stage_by_default(oracle,
+                                                            monkeypatch):
+    # from 4,096 queries on the library takes the eight-wave stage by itself
+    monkeypatch.delenv("PCA_KNN_FEAT_WIDE", raising=False)
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((12000, 96)).astype(np.float32)
+    y = rng.standard_normal((5000, 96)).astype(np.float32)
+    _run(oracle, x, y, np.array([0, 5000, 12000]), np.array([0, 2100, 5000]),
+         20)
+
+
+def test_feature_space_knn_256_full_size_properties(oracle, first_stage):
+    _only_once_beyond_128(first_stage, 256)
     # 50,000 rows of 256 components onto themselves, k = 32: every 400th query
     # exactly, all of them by the properties the result must have
     from gpu_common import dev

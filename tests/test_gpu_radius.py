@@ -9,7 +9,7 @@ pytestmark = pytest.mark.gpu
 import pytorch_cluster_amd as pca  # noqa: E402
 from pytorch_cluster_amd import testing  # noqa: E402
 from gpu_common import DEV, dev, gpu_radius, ragged_ptrs, use_strategy  # noqa: E402
-from helpers import to_set  # noqa: E402
+from helpers import stable_seed, to_set  # noqa: E402
 
 
 def tensor(v, dtype=torch.float32):
@@ -139,7 +139,7 @@ def test_strict_inequality_at_the_radius(oracle, radius_path):
 def test_filter_never_drops_a_neighbour(oracle, radius_path, d, case):
     # where the split-bf16 pre-filter is least accurate or switched off, and
     # where queries fill up early and whole waves leave the scan
-    rng = np.random.default_rng(hash((d, case, "radius")) % (2 ** 32))
+    rng = np.random.default_rng(stable_seed((d, case, "radius")))
     n, m, cap, r = 7000, 900, 16, 0.05
     ptr_x = np.array([0, 3000, 7000])
     ptr_y = np.array([0, 500, 900])
