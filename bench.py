@@ -266,21 +266,30 @@ class Cases:
             issued = None
         else:
             blocks, width = _feat_shape(d, k)
-            kernel = "knn_feat_kernel<%d,%d,%s>" % (
-                blocks, width, "true" if cosine else "false")
+            # up to 128 components and from 4,096 queries on: the eight-wave
+            # first stage (queries in tiles of 512, lists of the k smallest
+            # values); else the four-wave one (tiles of 128, lists of k + 16)
+            wide = d <= 128 and m >= 4096
+            if wide:
+                kernel = "knn_feat_wide_kernel<%d,%d,%s>" % (
+                    blocks, next(w for w in (16, 32, 64, 100) if w >= k),
+                    "true" if cosine else "false")
+            else:
+                kernel = "knn_feat_kernel<%d,%d,%s>" % (
+                    blocks, width, "true" if cosine else "false")
             # one v_mfma_f32_32x32x16_f16 (32,768 flop) per block and 32 x 32
-            # pairs; rows in tiles of 64 (32 from 144 components on), queries
-            # in tiles of 128
+            # pairs; rows in tiles of 64 (32 from 144 components on)
             tile = 64 if blocks <= 9 else 32
-            issued = (-(-n // tile) * tile) * (-(-m // 128) * 128) // 1024 \
-                * blocks * 32768
+            qtile = 512 if wide else 128
+            issued = (-(-n // tile) * tile) * (-(-m // qtile) * qtile) \
+                // 1024 * blocks * 32768
         roof = _roofline(
             kernel, kms, flop, PEAK_BF16_TFLOPS, "mfma",
             "algorithmic 2*D flop per pair against the dense fp16 / bf16 "
             "matrix peak; the kernel forms one fp16 product per pair and "
             "component on the matrix cores (a proven lower bound of the "
-            "distance), keeps k + 16 rows per query, and a second kernel "
-            "evaluates those exactly in fp32")
+            "distance), keeps the k + 16 rows per query with the smallest "
+            "bounds, and a second kernel evaluates those exactly in fp32")
         if issued is not None:
             roof["issued_flop_per_launch"] = issued
             roof["issued_frac"] = issued / kms / 1e9 / PEAK_BF16_TFLOPS
