@@ -138,6 +138,25 @@ int pca_segment_pointers(const int64_t *ids_x, int64_t n, const int64_t *ids_y,
                          int64_t m, int64_t num_segments, int64_t *ptr_x,
                          int64_t *ptr_y, void *stream);
 
+/*
+ * For a caller that does not know the number of examples (the reference's
+ * wrappers read it from the device, torch_cluster/knn.py:62-72: two
+ * batch.max() reductions with a host wait each): the next call of the calling
+ * thread that derives pointers from example ids -- pca_knn / pca_radius /
+ * pca_knn_fixed_scratch with PCA_SEGMENTS_BY_ID, or pca_segment_pointers --
+ * stores the largest id it was given + 1 to *examples_in_use (memory the
+ * device can write: device memory or pinned host memory) from the launch
+ * that derives the pointers.  Such a caller passes its best guess as
+ * num_segments, reads the number together with the edge count after the one
+ * wait it needs anyway, and calls again only if the guess was too small.  (A
+ * guess that is too large gives the same edges: examples without rows.  One
+ * that is too small is harmless -- queries of the examples beyond it are
+ * searched in the last example, their rows of x not at all, as the
+ * reference's lookup does, csrc/cuda/utils.cuh:11-19 -- but not what the
+ * caller wants.)  NULL cancels the request.
+ */
+int pca_report_examples(int64_t *examples_in_use);
+
 /* ------------------------------------------------------------------ kNN -- */
 
 /*

@@ -34,6 +34,7 @@ C_ABI = {
     "pca_status_string": (ctypes.c_char_p, [ctypes.c_int]),
     "pca_last_error": (ctypes.c_char_p, []),
     "pca_time_next_search": (ctypes.c_int, [_vp, _vp]),
+    "pca_report_examples": (ctypes.c_int, [_vp]),
     "pca_knn_workspace_bytes": (ctypes.c_size_t,
                                 [_i64, _i64, _i64, _i64, _i64, ctypes.c_int]),
     "pca_knn": (ctypes.c_int,

@@ -26,14 +26,25 @@ def check_ids(x: torch.Tensor, y: torch.Tensor, batch_x: torch.Tensor,
     assert y.size(0) == batch_y.numel()
 
 
+def examples_or_unknown(batch_size: Optional[int]) -> int:
+    """``batch_size`` for the operators that take example ids: -1 stands for
+    "not known" (the operator then starts with the number of examples of the
+    previous call and checks it against the ids on the device)."""
+    if batch_size is None:
+        return -1
+    return batch_size
+
+
 def num_examples(x: torch.Tensor, y: torch.Tensor,
                  batch_x: Optional[torch.Tensor],
                  batch_y: Optional[torch.Tensor],
                  batch_size: Optional[int]) -> int:
-    """Number of examples B.  Without ``batch_size`` it is read from the
-    device: the LAST entry of each batch vector (they are sorted, so that is
-    the largest) -- one 8-byte read each instead of the reference's
-    ``batch.max()`` reductions (``torch_cluster/knn.py:62-72``)."""
+    """Number of examples B (CPU tensors, and GPU calls that go through
+    pointers).  Without ``batch_size`` it is read from the LAST entry of each
+    batch vector: the vectors must be sorted (as the reference requires,
+    ``torch_cluster/knn.py:27-29``), so that is the largest -- one 8-byte read
+    each instead of the reference's ``batch.max()`` reductions
+    (``torch_cluster/knn.py:62-72``).  An unsorted vector is not detected."""
     if batch_size is not None:
         assert batch_size > 0
         return batch_size

@@ -28,6 +28,9 @@ int fail(int status, const char *fmt, ...) {
 }
 
 // one-shot request of pca_time_next_search
+// pca_report_examples: where the next call that derives pointers from ids
+// leaves the number of examples those ids speak of
+thread_local int64_t *g_examples_out = nullptr;
 thread_local hipEvent_t g_time_start = nullptr;
 thread_local hipEvent_t g_time_stop = nullptr;
 
@@ -73,6 +76,11 @@ __global__ void fill_i64_kernel(int64_t *p, int64_t count, int64_t v) {
 
 constexpr int64_t kMaxRows = 2147483646; // n, m < 2^31 - 1
 
+// Segments a call works with: one when no pointers are given.
+int64_t segments_in_use(const int64_t *ptr_x, int64_t num_segments) {
+  return ptr_x == nullptr ? 1 : num_segments;
+}
+
 bool sizes_ok(int64_t n, int64_t m, int64_t d, int64_t num_segments) {
   return n >= 0 && m >= 0 && n <= kMaxRows && m <= kMaxRows && d >= 1 &&
          d <= (1 << 20) && num_segments >= 1 && num_segments <= kMaxRows;
@@ -101,6 +109,8 @@ pca::SegmentSource segments_by_id(const int64_t *&ptr_x, const int64_t *&ptr_y,
       align256(sizeof(int64_t) * (size_t)(num_segments + 1)));
   ptr_x = src.ptr_x;
   ptr_y = src.ptr_y;
+  src.examples_out = g_examples_out;
+  g_examples_out = nullptr;
   return src;
 }
 
@@ -338,6 +348,11 @@ int pca_time_next_search(void *start_event, void *stop_event) {
   return PCA_OK;
 }
 
+int pca_report_examples(int64_t *examples_in_use) {
+  g_examples_out = examples_in_use;
+  return PCA_OK;
+}
+
 int pca_segment_pointers(const int64_t *ids_x, int64_t n, const int64_t *ids_y,
                          int64_t m, int64_t num_segments, int64_t *ptr_x,
                          int64_t *ptr_y, void *stream_) {
@@ -357,6 +372,8 @@ int pca_segment_pointers(const int64_t *ids_x, int64_t n, const int64_t *ids_y,
   src.m = (int)m;
   src.ptr_x = ptr_x;
   src.ptr_y = ptr_y;
+  src.examples_out = g_examples_out;
+  g_examples_out = nullptr;
   return check_launch(
       pca::launch_segment_pointers(src, (int)num_segments,
                                    static_cast<hipStream_t>(stream_)),
@@ -390,9 +407,10 @@ int pca_knn_fixed_scratch(const void *x, const void *y, const int64_t *ptr_x,
                           int64_t *edges, int64_t *num_edges, void *dist,
                           void *stream_) {
   g_last_error[0] = 0;
-  // (same normalisation as knn_call, so that the size test sees what the
-  // search will use; invalid sizes are reported by knn_call itself)
-  const int64_t segs = ptr_x == nullptr ? 1 : num_segments;
+  // (the size test sees what the search will use: knn_call sizes its
+  // workspace by the same two functions; invalid sizes are reported by
+  // knn_call itself)
+  const int64_t segs = segments_in_use(ptr_x, num_segments);
   if (sizes_ok(n, m, d, segs) && k >= 1 && k <= PCA_KNN_MAX_K &&
       dtype_ok(dtype) && n > 0 && m > 0) {
     const size_t need = knn_workspace(n, m, d, segs, k, dtype);
@@ -427,8 +445,7 @@ int knn_call(const void *x, const void *y, const int64_t *ptr_x,
   if ((ptr_x == nullptr) != (ptr_y == nullptr))
     return fail(PCA_ERR_INVALID_ARGUMENT,
                 "ptr_x and ptr_y must both be given or both be NULL");
-  if (ptr_x == nullptr)
-    num_segments = 1;
+  num_segments = segments_in_use(ptr_x, num_segments);
   if (!sizes_ok(n, m, d, num_segments))
     return fail(PCA_ERR_INVALID_ARGUMENT,
                 "bad sizes n=%lld m=%lld d=%lld num_segments=%lld",

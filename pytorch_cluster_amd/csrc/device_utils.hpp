@@ -302,6 +302,16 @@ __device__ __forceinline__ void pointers_from_ids(const Src &src,
   const int wave = threadIdx.x >> 6;
   const int waves = blockDim.x >> 6;
   const int searches = 2 * (num_segments + 1);
+  // for a caller that guessed num_segments: the examples the ids speak of
+  // (sorted ids: the last ones are the largest)
+  if (src.examples_out != nullptr && threadIdx.x == 0) {
+    int64_t last = -1;
+    if (src.n > 0)
+      last = src.ids_x[src.n - 1];
+    if (src.m > 0 && src.ids_y[src.m - 1] > last)
+      last = src.ids_y[src.m - 1];
+    *src.examples_out = last + 1;
+  }
   for (int s = wave; s < searches; s += waves) {
     const int side = s & 1;
     const int b = s >> 1;
@@ -325,7 +335,13 @@ __device__ __forceinline__ void pointers_from_ids(const Src &src,
       hi = new_hi;
     }
     const bool is_below = lo + lane < hi && ids[lo + lane] < (int64_t)b;
-    const int result = lo + __builtin_popcountll(__ballot(is_below));
+    int result = lo + __builtin_popcountll(__ballot(is_below));
+    // Rows whose id is num_segments or more (a caller's batch_size below the
+    // largest id + 1): the reference's lookup hands such a query to the LAST
+    // example (csrc/cuda/utils.cuh:11-19 returns num_examples - 1 when no
+    // pointer lies above the row), and never searches such a row of x.
+    if (side == 1 && b == num_segments)
+      result = count;
     if (lane == 0)
       (side ? src.ptr_y : src.ptr_x)[b] = result;
   }

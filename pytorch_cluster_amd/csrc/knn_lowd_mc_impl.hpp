@@ -233,8 +233,11 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
   constexpr int PT = TX / kBlock; // rows staged per thread
 
   constexpr int REC = McShape<DIM>::REC;
-  // packed rows as mc_pack_row leaves them
-  __shared__ __attribute__((aligned(16))) uint4 rows_lds[TX][REC];
+  // the tile's packed rows, every 16-byte unit of a row in a plane of its
+  // own: the lanes of a wave read the same unit of 32 consecutive rows, and
+  // with the units of one row side by side (32 bytes from row to row in three
+  // dimensions) two lanes met in every bank
+  __shared__ __attribute__((aligned(16))) uint4 rows_lds[REC][TX];
   // parked steps: (step << 16) | mask of the lane's 16 rows that passed
   __shared__ uint32_t queue[QCAP][kBlock];
 
@@ -421,7 +424,7 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
     for (int r = 0; r < PT; ++r)
 #pragma unroll
       for (int i = 0; i < REC; ++i)
-        rows_lds[r * kBlock + tid][i] = stage[r][i];
+        rows_lds[i][r * kBlock + tid] = stage[r][i];
   };
 
   auto sync_bounds = [&]() {
@@ -510,7 +513,7 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
       float row[XF];
 #pragma unroll
       for (int e = 0; e < XF; e += 4) {
-        const uint4 q4 = rows_lds[j][NI + e / 4];
+        const uint4 q4 = rows_lds[NI + e / 4][j];
         row[e] = __uint_as_float(q4.x);
         row[e + 1] = __uint_as_float(q4.y);
         row[e + 2] = __uint_as_float(q4.z);
@@ -574,7 +577,7 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
     uint4 a_next[NI];
 #pragma unroll
     for (int i = 0; i < NI; ++i)
-      a_next[i] = rows_lds[col][i];
+      a_next[i] = rows_lds[i][col];
     for (int rt = 0; rt < steps32; ++rt) {
       mfma_acc_t acc = {0};
 #pragma unroll
@@ -597,7 +600,7 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
       // (the last read stays inside the tile)
 #pragma unroll
       for (int i = 0; i < NI; ++i)
-        a_next[i] = rows_lds[min(rt + 1, TX / 32 - 1) * 32 + col][i];
+        a_next[i] = rows_lds[i][min(rt + 1, TX / 32 - 1) * 32 + col];
 
       // accumulator v = t - cut of row 8 (v / 4) + 4 half + v % 4: its sign
       // bit says "look at this row".  One funnel shift per accumulator

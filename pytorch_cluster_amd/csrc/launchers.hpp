@@ -49,6 +49,8 @@ struct SegmentSource {
   int n = 0, m = 0;
   int64_t *ptr_x = nullptr;       // [num_segments + 1], written
   int64_t *ptr_y = nullptr;
+  // where the largest id met + 1 goes (device-accessible memory), or NULL
+  int64_t *examples_out = nullptr;
 };
 
 // work_start[b] = sum over b' < b of ceil(m_b' / per_item): the first work item

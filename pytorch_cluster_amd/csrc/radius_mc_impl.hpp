@@ -59,7 +59,9 @@ __global__ __launch_bounds__(kBlock) void radius_mc_kernel(RadiusMcParams p) {
   constexpr int QCAP = kMcQueueCap;
   constexpr int PT = TX / kBlock; // rows staged per thread
 
-  __shared__ __attribute__((aligned(16))) uint4 rows_lds[TX][REC];
+  // (every 16-byte unit of a row in a plane of its own, as in
+  // knn_lowd_mc_impl.hpp: conflict-free reads)
+  __shared__ __attribute__((aligned(16))) uint4 rows_lds[REC][TX];
   // parked steps: (step << 16) | mask of the lane's 16 rows that passed
   // (also carries, between the two barriers at the top of a tile, the four
   // waves' "all my queries are full" flags: one more variable would take the
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(kBlock) void radius_mc_kernel(RadiusMcParams p) {
     for (int r = 0; r < PT; ++r)
 #pragma unroll
       for (int i = 0; i < REC; ++i)
-        rows_lds[r * kBlock + tid][i] = stage[r][i];
+        rows_lds[i][r * kBlock + tid] = stage[r][i];
   };
 
   // One lane's walk over parked rows (see knn_lowd_mc_kernel): peek returns
@@ -244,7 +246,7 @@ __global__ __launch_bounds__(kBlock) void radius_mc_kernel(RadiusMcParams p) {
         float row[XF];
 #pragma unroll
         for (int e = 0; e < XF; e += 4) {
-          const uint4 q4 = rows_lds[j][NI + e / 4];
+          const uint4 q4 = rows_lds[NI + e / 4][j];
           row[e] = __uint_as_float(q4.x);
           row[e + 1] = __uint_as_float(q4.y);
           row[e + 2] = __uint_as_float(q4.z);
@@ -304,7 +306,7 @@ __global__ __launch_bounds__(kBlock) void radius_mc_kernel(RadiusMcParams p) {
     uint4 a_next[NI];
 #pragma unroll
     for (int i = 0; i < NI; ++i)
-      a_next[i] = rows_lds[col][i];
+      a_next[i] = rows_lds[i][col];
     for (int rt = 0; rt < steps32; ++rt) {
       mfma_acc_t acc = {0};
 #pragma unroll
@@ -325,7 +327,7 @@ __global__ __launch_bounds__(kBlock) void radius_mc_kernel(RadiusMcParams p) {
       }
 #pragma unroll
       for (int i = 0; i < NI; ++i)
-        a_next[i] = rows_lds[min(rt + 1, TX / 32 - 1) * 32 + col][i];
+        a_next[i] = rows_lds[i][min(rt + 1, TX / 32 - 1) * 32 + col];
 
       uint32_t mask = 0;
 #pragma unroll

@@ -161,12 +161,48 @@ at::Tensor edge_count_slot() {
                             true));
 }
 
+// Waits of the host for the device that the operators of this library have
+// made (for tests and profiles: the default calls are meant to make one).
+std::atomic<int64_t> g_host_waits{0};
+int64_t host_waits() { return g_host_waits.load(); }
+
+// Until an operator has waited for its stream the kernels it queued may still
+// write the edge count: on every way out before that wait -- an exception
+// after some kernels were queued -- the stream is waited for here, so that
+// the pinned slot is not handed to a later call while a kernel of this one
+// can still write it.
+struct SlotGuard {
+  hipStream_t stream;
+  bool armed = true;
+  explicit SlotGuard(hipStream_t s) : stream(s) {}
+  ~SlotGuard() {
+    if (armed)
+      (void)hipStreamSynchronize(stream);
+  }
+};
+
+// The size of an edge list depends on the data: the operators read it from
+// the device before they return, which a stream that is being captured into
+// a graph cannot do.
+void refuse_capture(hipStream_t stream, const char *op) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return;
+  }
+  TORCH_CHECK(status == hipStreamCaptureStatusNone, op,
+              " cannot be captured into a graph: the size of its result "
+              "depends on the data (call pca_knn / pca_radius of the C ABI "
+              "with buffers of the largest size instead)");
+}
+
 at::Tensor finish(const at::Tensor &edges, const at::Tensor &num_edges,
                   hipStream_t stream) {
   // the only host synchronisation of the operator: the edge count sizes the
   // result (the reference synchronises in its masked_selects)
   TORCH_CHECK(hipStreamSynchronize(stream) == hipSuccess,
               "hipStreamSynchronize failed");
+  g_host_waits += 1;
   const int64_t E = *num_edges.data_ptr<int64_t>();
   at::Tensor out = edges.narrow(0, 0, 2 * E).view({2, E});
   // (a view keeps the whole slot buffer alive: a result that fills less than
@@ -397,9 +433,11 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
                       std::optional<at::Tensor> ptr_x,
                       std::optional<at::Tensor> ptr_y, int64_t k, bool cosine,
                       int flags, int64_t num_workers = 1,
-                      int64_t ids_examples = 0) {
+                      int64_t ids_examples = 0,
+                      int64_t *examples_report = nullptr) {
   // ids_examples > 0: ptr_x / ptr_y hold the rows' example ids, that many
-  // examples (GPU tensors only)
+  // examples (GPU tensors only); examples_report: where the launch that
+  // derives the pointers leaves the largest id + 1 (pinned host memory)
   // the device branch of csrc/knn.cpp:26-36
   if (!x.device().is_cuda()) {
     TORCH_CHECK(ids_examples == 0, "example ids are taken for GPU tensors");
@@ -427,13 +465,12 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
   if (n == 0 || m == 0)
     return at::empty({2, 0}, long_opts);
 
+  refuse_capture(c10::hip::getCurrentHIPStream(x.get_device()).stream(),
+                 "knn");
   const int dtype = dtype_code(x);
   const bool binned = bins_wanted(n, m, seg.count, kKnnCost.scan_rate,
                                   kKnnCost.query_us) &&
-                      dtype == PCA_F32 && !cosine && d <= 3 && k <= 64 &&
-                      !being_captured(c10::hip::getCurrentHIPStream(
-                                          x.get_device())
-                                          .stream());
+                      dtype == PCA_F32 && !cosine && d <= 3 && k <= 64;
   const size_t ws_bytes =
       binned ? pca_knn_binned_workspace_bytes(n, m, d, seg.count, k)
              : pca_knn_workspace_bytes(n, m, d, seg.count, k, dtype);
@@ -444,7 +481,9 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
   auto num_edges = edge_count_slot();
 
   hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
+  SlotGuard guard(stream);
   if (ids_examples > 0) {
+    (void)pca_report_examples(examples_report);
     if (binned)
       pointers_for(seg, n, m, stream);
     else
@@ -456,6 +495,7 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
                                 edges.data_ptr<int64_t>(),
                                 num_edges.data_ptr<int64_t>(), nullptr,
                                 workspace.data_ptr(), ws_bytes, stream));
+    guard.armed = false; // (finish waits for the stream itself)
     return finish(edges, num_edges, stream);
   }
   check_status(pca_knn(x.data_ptr(), y.data_ptr(), seg.ptr_x, seg.ptr_y, n, m,
@@ -463,6 +503,7 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
                        edges.data_ptr<int64_t>(),
                        num_edges.data_ptr<int64_t>(), nullptr,
                        workspace.data_ptr(), ws_bytes, stream));
+  guard.armed = false;
   return finish(edges, num_edges, stream);
 }
 
@@ -485,14 +526,61 @@ at::Tensor knn_edges(at::Tensor x, at::Tensor y,
                     edge_flags(drop_self, x_first));
 }
 
+// The number of examples of a call that was not told (batch_size < 1): the
+// reference's wrappers read it from the device before they can start
+// (torch_cluster/knn.py:62-72, two reductions with a host wait each).  Here
+// the search starts with the number the previous call of the process met, the
+// launch that derives the pointers reports the number the ids really speak
+// of into pinned host memory, and the operator looks at it after the one wait
+// it has anyway (for the edge count): equal or smaller, the edges are right
+// (examples without rows); larger, the search runs once more with the right
+// number.  Only the first call of a process reads the ids' last entries up
+// front.
+std::atomic<int64_t> g_examples_hint{0};
+
+template <typename Run>
+at::Tensor with_examples(const at::Tensor &batch_x, const at::Tensor &batch_y,
+                         int64_t batch_size, Run run) {
+  if (batch_size >= 1)
+    return run(batch_size, nullptr);
+  int64_t guess = g_examples_hint.load();
+  if (guess < 1) {
+    // (sorted ids: the last ones are the largest)
+    int64_t last = -1;
+    if (batch_x.numel() > 0)
+      last = std::max(last, batch_x[-1].item<int64_t>());
+    if (batch_y.numel() > 0 && !batch_y.is_same(batch_x))
+      last = std::max(last, batch_y[-1].item<int64_t>());
+    g_host_waits += 1;
+    guess = std::max<int64_t>(last + 1, 1);
+    g_examples_hint.store(guess);
+    return run(guess, nullptr);
+  }
+  auto slot = at::empty({1}, at::TensorOptions().dtype(at::kLong).pinned_memory(
+                                 true));
+  int64_t *in_use = slot.data_ptr<int64_t>();
+  *in_use = 0;
+  at::Tensor out = run(guess, in_use);
+  // (run has waited for the stream: the number is there)
+  const int64_t met = std::max<int64_t>(*in_use, 1);
+  g_examples_hint.store(met);
+  if (met > guess)
+    out = run(met, nullptr);
+  return out;
+}
+
 // knn_edges with the segments given as the rows' sorted example ids and the
 // number of examples (the prologue of torch_cluster/knn.py:62-79 folded into
-// the launch that prepares the search).
+// the launch that prepares the search); batch_size < 1: not known, see
+// with_examples.
 at::Tensor knn_batched(at::Tensor x, at::Tensor y, at::Tensor batch_x,
                        at::Tensor batch_y, int64_t batch_size, int64_t k,
                        bool cosine, bool drop_self, bool x_first) {
-  return knn_search(x, y, batch_x, batch_y, k, cosine,
-                    edge_flags(drop_self, x_first), 1, batch_size);
+  return with_examples(
+      batch_x, batch_y, batch_size, [&](int64_t examples, int64_t *report) {
+        return knn_search(x, y, batch_x, batch_y, k, cosine,
+                          edge_flags(drop_self, x_first), 1, examples, report);
+      });
 }
 
 at::Tensor radius_search(at::Tensor x, at::Tensor y,
@@ -500,8 +588,9 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
                          std::optional<at::Tensor> ptr_y, double r,
                          int64_t max_num_neighbors, bool ignore_same_index,
                          int flags, int64_t num_workers = 1,
-                         int64_t ids_examples = 0) {
-  // (ids_examples: as for knn_search)
+                         int64_t ids_examples = 0,
+                         int64_t *examples_report = nullptr) {
+  // (ids_examples, examples_report: as for knn_search)
   // the device branch of csrc/radius.cpp:27-35
   if (!x.device().is_cuda()) {
     TORCH_CHECK(ids_examples == 0, "example ids are taken for GPU tensors");
@@ -530,14 +619,13 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
   if (n == 0 || m == 0)
     return at::empty({2, 0}, long_opts);
 
+  refuse_capture(c10::hip::getCurrentHIPStream(x.get_device()).stream(),
+                 "radius");
   const int dtype = dtype_code(x);
   const int64_t slots = pca_radius_slots(n, max_num_neighbors);
   const bool binned = bins_wanted(n, m, seg.count, kRadiusCost.scan_rate,
                                   kRadiusCost.query_us) &&
-                      dtype == PCA_F32 && d <= 3 && slots <= 64 &&
-                      !being_captured(c10::hip::getCurrentHIPStream(
-                                          x.get_device())
-                                          .stream());
+                      dtype == PCA_F32 && d <= 3 && slots <= 64;
   const size_t ws_bytes =
       binned ? pca_radius_binned_workspace_bytes(n, m, d, seg.count,
                                                  max_num_neighbors)
@@ -550,7 +638,9 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
   auto num_edges = edge_count_slot();
 
   hipStream_t stream = c10::hip::getCurrentHIPStream(x.get_device()).stream();
+  SlotGuard guard(stream);
   if (ids_examples > 0) {
+    (void)pca_report_examples(examples_report);
     if (binned)
       pointers_for(seg, n, m, stream);
     else
@@ -562,6 +652,7 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
         r, max_num_neighbors, ignore_same_index ? 1 : 0, flags,
         edges.data_ptr<int64_t>(), num_edges.data_ptr<int64_t>(),
         workspace.data_ptr(), ws_bytes, stream));
+    guard.armed = false; // (finish waits for the stream itself)
     return finish(edges, num_edges, stream);
   }
   check_status(pca_radius(x.data_ptr(), y.data_ptr(), seg.ptr_x, seg.ptr_y, n,
@@ -570,6 +661,7 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
                           edges.data_ptr<int64_t>(),
                           num_edges.data_ptr<int64_t>(), workspace.data_ptr(),
                           ws_bytes, stream));
+  guard.armed = false;
   return finish(edges, num_edges, stream);
 }
 
@@ -597,9 +689,12 @@ at::Tensor radius_batched(at::Tensor x, at::Tensor y, at::Tensor batch_x,
                           at::Tensor batch_y, int64_t batch_size, double r,
                           int64_t max_num_neighbors, bool ignore_same_index,
                           bool x_first) {
-  return radius_search(x, y, batch_x, batch_y, r, max_num_neighbors,
-                       ignore_same_index, edge_flags(false, x_first), 1,
-                       batch_size);
+  return with_examples(
+      batch_x, batch_y, batch_size, [&](int64_t examples, int64_t *report) {
+        return radius_search(x, y, batch_x, batch_y, r, max_num_neighbors,
+                             ignore_same_index, edge_flags(false, x_first), 1,
+                             examples, report);
+      });
 }
 
 // csrc/nearest.cpp:22-36 -> nearest_cuda (csrc/cuda/nearest_cuda.cu:68-94):
@@ -755,6 +850,7 @@ TORCH_LIBRARY(pytorch_cluster_amd, m) {
         "int batch_size, float r, int max_num_neighbors, "
         "bool ignore_same_index, bool x_first) -> Tensor",
         &radius_batched);
+  m.def("host_waits() -> int", &host_waits);
   m.def("set_search_strategy(str name) -> ()", &set_search_strategy);
   m.def("get_search_strategy() -> str", &get_search_strategy);
   m.def("strategy_for(str op, int searched, int searching, int num_segments) "

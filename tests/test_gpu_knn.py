@@ -568,3 +568,20 @@ def test_graph_epilogue_in_the_output_pass(oracle, flow, loop):
     keep = full[0] != full[1]
     assert e.tolist() == full[::-1][:, keep].tolist()
     assert (d == dfull[keep]).all()
+
+
+def test_operators_refuse_graph_capture():
+    # the size of an edge list depends on the data: knn / radius read it from
+    # the device before they return, which a capturing stream cannot do --
+    # they say so instead of breaking the capture halfway
+    x = torch.rand(500, 3, device=DEV)
+    pca.knn(x, x, 3)  # (everything lazy is done before the capture)
+    graph = torch.cuda.CUDAGraph()
+    for call in (lambda: pca.knn(x, x, 3),
+                 lambda: pca.radius(x, x, 0.1)):
+        with pytest.raises(RuntimeError, match="cannot be captured"):
+            with torch.cuda.graph(graph):
+                call()
+        torch.cuda.synchronize()
+    # and work as before afterwards
+    assert pca.knn(x, x, 3).shape == (2, 1500)

@@ -147,3 +147,104 @@ def test_scripted_wrappers_take_the_id_path():
     assert (f(x, 4, batch, batch_size=3) == pca.knn_graph(x, 4, batch)).all()
     assert (g(x, 0.1, batch, batch_size=3)
             == pca.radius_graph(x, 0.1, batch)).all()
+
+
+@pytest.mark.parametrize("strategy", ["scan", "binned"])
+def test_batch_size_below_the_ids_in_use(oracle, strategy):
+    # a batch_size smaller than the largest id + 1: the reference's lookup
+    # (csrc/cuda/utils.cuh:11-19) hands the queries of the examples beyond it
+    # to the last example it knows, and the rows of those examples are never
+    # searched; the id path does the same, for every kernel that plans its
+    # work differently
+    rng = np.random.default_rng(31)
+    before = pca.get_search_strategy()
+    pca.set_search_strategy(strategy)
+    try:
+        for d, k in ((3, 7), (40, 5), (3, 40)):
+            n = 12000
+            x = rng.random((n, d)).astype(np.float32)
+            ptr = ragged_ptrs(rng, n, 6)
+            batch = _ids(ptr)
+            y, by = x[::5].copy(), batch[::5].copy()
+            xd, yd = dev(x), dev(y)
+            bd, byd = dev(batch), dev(by)
+            for size in (4, 2):
+                got = pca.knn(xd, yd, k, bd, byd, batch_size=size)
+                want = oracle.knn(x, y, k, batch, by, batch_size=size)
+                assert got.shape == want.shape
+                assert (got.cpu().numpy() == want).all()
+                got = pca.knn_graph(xd, k, bd, batch_size=size)
+                want = oracle.knn_graph(x, k, batch, batch_size=size)
+                assert got.shape == want.shape
+                assert (got.cpu().numpy() == want).all()
+            if d == 3:
+                got = pca.radius(xd, yd, 0.05, bd, byd, max_num_neighbors=9,
+                                 batch_size=3)
+                want = oracle.radius(x, y, 0.05, batch, by,
+                                     max_num_neighbors=9, batch_size=3)
+                assert got.shape == want.shape
+                assert (got.cpu().numpy() == want).all()
+    finally:
+        pca.set_search_strategy(before)
+
+
+def test_default_calls_wait_for_the_device_once(oracle):
+    # without batch_size the reference reads the number of examples from the
+    # device before it starts (two reductions, two waits).  Here the search
+    # starts with the number the previous call met and the launch that
+    # derives the pointers reports the real one: a call waits for the device
+    # once (for its edge count) -- twice when the number grew, and only the
+    # first call of a process reads the ids' last entries up front
+    waits = torch.ops.pytorch_cluster_amd.host_waits
+    rng = np.random.default_rng(41)
+    n = 9000
+    x = rng.random((n, 3)).astype(np.float32)
+
+    def clouds(count):
+        ptr = ragged_ptrs(rng, n, count)
+        return _ids(ptr)
+
+    xd = dev(x)
+    first = clouds(5)
+    pca.knn_graph(xd, 4, dev(first))          # (whatever the process did before)
+    for count, expected in ((5, 1), (5, 1), (3, 1), (3, 1), (9, 2), (9, 1),
+                            (1, 1), (2, 2)):
+        batch = clouds(count)
+        bd = dev(batch)
+        before = waits()
+        got = pca.knn_graph(xd, 6, bd)
+        assert waits() - before == expected, (count, waits() - before)
+        want = oracle.knn_graph(x, 6, batch)
+        assert got.shape == want.shape and (got.cpu().numpy() == want).all()
+    # radius_graph, knn and radius share the number
+    batch = clouds(4)
+    bd = dev(batch)
+    pca.knn_graph(xd, 3, bd)
+    y, by = x[::3].copy(), batch[::3].copy()
+    for call, ref in (
+            (lambda: pca.radius_graph(xd, 0.05, bd, max_num_neighbors=7),
+             lambda: oracle.radius_graph(x, 0.05, batch, max_num_neighbors=7)),
+            (lambda: pca.knn(xd, dev(y), 5, bd, dev(by)),
+             lambda: oracle.knn(x, y, 5, batch, by)),
+            (lambda: pca.radius(xd, dev(y), 0.04, bd, dev(by),
+                                max_num_neighbors=6),
+             lambda: oracle.radius(x, y, 0.04, batch, by,
+                                   max_num_neighbors=6))):
+        before = waits()
+        got = call()
+        assert waits() - before == 1
+        want = ref()
+        assert got.shape == want.shape and (got.cpu().numpy() == want).all()
+    # the binned searches take the same road
+    before_strategy = pca.get_search_strategy()
+    pca.set_search_strategy("binned")
+    try:
+        for count, expected in ((4, 1), (7, 2), (7, 1)):
+            batch = clouds(count)
+            before = waits()
+            got = pca.knn_graph(xd, 6, dev(batch))
+            assert waits() - before == expected
+            want = oracle.knn_graph(x, 6, batch)
+            assert (got.cpu().numpy() == want).all()
+    finally:
+        pca.set_search_strategy(before_strategy)

@@ -53,6 +53,53 @@ def test_fixed_scratch_matches_pca_knn_on_consecutive_calls(oracle):
             assert (got_e == oe).all() and (got_d == od).all()
 
 
+def test_fixed_scratch_call_allocates_nothing():
+    # the entry point's defining property: with the outputs allocated by the
+    # caller, a direct call through the C ABI leaves the device's free memory
+    # as it was (the driver's own figure, not the caching allocator's) -- on
+    # the first calls of three kernel families and on repeated ones
+    from gpu_common import dev
+    from pytorch_cluster_amd._native import capi as lib
+    rng = np.random.default_rng(6)
+    cases = [(rng.random((5000, 3), dtype=np.float32), 12, 0),
+             (rng.standard_normal((900, 40)).astype(np.float32), 7, 1),
+             (rng.random((300, 2)).astype(np.float64), 5, 0)]
+    # everything the calls touch exists before the first reading
+    prepared = []
+    for x, k, cosine in cases:
+        xd = dev(x)
+        m = x.shape[0]
+        edges = torch.empty(2 * m * k, dtype=torch.long, device="cuda:0")
+        count = torch.empty(1, dtype=torch.long, device="cuda:0")
+        dist = torch.empty(m * k, dtype=xd.dtype, device="cuda:0")
+        prepared.append((xd, k, cosine, edges, count, dist))
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.cuda.synchronize()
+
+    def call(xd, k, cosine, edges, count, dist):
+        dtype = 1 if xd.dtype == torch.float64 else 0
+        rc = lib.pca_knn_fixed_scratch(
+            xd.data_ptr(), xd.data_ptr(), None, None, xd.shape[0],
+            xd.shape[0], xd.shape[1], 1, k, cosine, dtype, 0,
+            edges.data_ptr(), count.data_ptr(), dist.data_ptr(), stream)
+        assert rc == 0, lib.pca_last_error()
+
+    # (one round first: the runtime loads a library's kernels into device
+    # memory at the first launch in a process, whoever launches)
+    for item in prepared:
+        call(*item)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for rounds in range(3):
+        for item in prepared:
+            call(*item)
+    torch.cuda.synchronize()
+    free_after = torch.cuda.mem_get_info()[0]
+    assert free_after == free_before, (free_before, free_after)
+    for xd, k, cosine, edges, count, dist in prepared:
+        assert int(count.item()) == xd.shape[0] * k
+
+
 def test_fixed_scratch_refuses_what_does_not_fit():
     from pytorch_cluster_amd import capi
     from pytorch_cluster_amd._native import PCA_FIXED_SCRATCH_BYTES
