@@ -201,10 +201,18 @@ __global__ __launch_bounds__(kBlock) void morton_keys_kernel(
     const float *__restrict__ pts, const int64_t *__restrict__ ptr, int count,
     int d, int num_segments, const int *__restrict__ seg_box,
     int axis_bits, uint32_t *__restrict__ keys,
-    uint32_t *__restrict__ vals) {
+    uint32_t *__restrict__ vals, bool searched_side) {
   const int i = blockIdx.x * kBlock + threadIdx.x;
   if (i >= count)
     return;
+  // rows of x behind the last pointer belong to no segment (a caller's
+  // batch_size below the ids in use: the reference never searches them,
+  // csrc/cuda/utils.cuh:11-19): they sort behind every segment's rows
+  if (searched_side && ptr != nullptr && (int64_t)i >= ptr[num_segments]) {
+    keys[i] = 0xffffffffu;
+    vals[i] = (uint32_t)i;
+    return;
+  }
   const int seg = find_segment64(ptr, num_segments, i);
   uint32_t code = 0;
 #pragma unroll
@@ -1162,7 +1170,7 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
       hipLaunchKernelGGL(morton_keys_kernel,
                          dim3((in.m + kBlock - 1) / kBlock), dim3(kBlock), 0,
                          side, y, in.ptr_y, in.m, in.d, nseg, seg_box,
-                         axis_bits(nseg), keys_b, vals_b);
+                         axis_bits(nseg), keys_b, vals_b, false);
       if ((e = hipGetLastError()) != hipSuccess)
         return e;
       size_t bytes = lay.side_temp;
@@ -1183,7 +1191,7 @@ hipError_t prepare_bins(const SearchInput &in, void *scratch, bool with_tasks,
     return err;
   hipLaunchKernelGGL(morton_keys_kernel, dim3((in.n + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, x, in.ptr_x, in.n, in.d, nseg,
-                     seg_box, axis_bits(nseg), keys_a, vals_a);
+                     seg_box, axis_bits(nseg), keys_a, vals_a, true);
   if ((err = hipGetLastError()) != hipSuccess)
     return err;
   size_t sort_bytes = lay.sort_temp;

@@ -576,9 +576,9 @@ def test_operators_refuse_graph_capture():
     # they say so instead of breaking the capture halfway
     x = torch.rand(500, 3, device=DEV)
     pca.knn(x, x, 3)  # (everything lazy is done before the capture)
-    graph = torch.cuda.CUDAGraph()
     for call in (lambda: pca.knn(x, x, 3),
                  lambda: pca.radius(x, x, 0.1)):
+        graph = torch.cuda.CUDAGraph()
         with pytest.raises(RuntimeError, match="cannot be captured"):
             with torch.cuda.graph(graph):
                 call()

@@ -71,7 +71,9 @@ def test_fixed_scratch_call_allocates_nothing():
         m = x.shape[0]
         edges = torch.empty(2 * m * k, dtype=torch.long, device="cuda:0")
         count = torch.empty(1, dtype=torch.long, device="cuda:0")
-        dist = torch.empty(m * k, dtype=xd.dtype, device="cuda:0")
+        # (distances come with fp32 points only)
+        dist = (torch.empty(m * k, dtype=torch.float32, device="cuda:0")
+                if xd.dtype == torch.float32 else None)
         prepared.append((xd, k, cosine, edges, count, dist))
     stream = torch.cuda.current_stream().cuda_stream
     torch.cuda.synchronize()
@@ -81,7 +83,8 @@ def test_fixed_scratch_call_allocates_nothing():
         rc = lib.pca_knn_fixed_scratch(
             xd.data_ptr(), xd.data_ptr(), None, None, xd.shape[0],
             xd.shape[0], xd.shape[1], 1, k, cosine, dtype, 0,
-            edges.data_ptr(), count.data_ptr(), dist.data_ptr(), stream)
+            edges.data_ptr(), count.data_ptr(),
+            dist.data_ptr() if dist is not None else None, stream)
         assert rc == 0, lib.pca_last_error()
 
     # (one round first: the runtime loads a library's kernels into device
