@@ -372,6 +372,30 @@ int pca_radius_host(const void *x, const void *y, const int64_t *ptr_x,
                     int ignore_same_index, int dtype, int edge_flags,
                     int num_threads, int64_t *edges, int64_t *num_edges);
 
+/*
+ * `fps` and `nearest` on the host (fp32 / fp64 points; all pointers HOST
+ * memory, `num_threads` threads over the examples resp. over blocks of rows).
+ * Arguments as for pca_fps / pca_nearest, and the same rows as those return:
+ * the tie rules and limits of the reference's CUDA kernels
+ * (csrc/cuda/fps_cuda.cu:10-66, csrc/cuda/nearest_cuda.cu:10-66), distances
+ * by one fused multiply-add per component.  They stand under
+ *   csrc/fps.cpp:31-33 -> fps_cpu, csrc/cpu/fps_cpu.cpp:11-64 (no 5e4 cap, the
+ *   first row among equal values: the same samples wherever distances stay
+ *   below 5e4 and do not tie)
+ *   torch_cluster/nearest.py:93-124 (scipy.cluster.vq.vq per example: the
+ *   lowest row among equal distances)
+ * Errors: status codes as above, text from pca_host_last_error().
+ */
+int pca_fps_host(const void *src, const int64_t *ptr, const int64_t *out_ptr,
+                 const int64_t *start, int64_t n, int64_t d,
+                 int64_t num_segments, int dtype, int num_threads,
+                 int64_t *out);
+
+int pca_nearest_host(const void *x, const void *y, const int64_t *ptr_x,
+                     const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+                     int64_t num_segments, int dtype, int num_threads,
+                     int64_t *out);
+
 /* ------------------------------------------------------------------ fps -- */
 
 /*

@@ -86,6 +86,12 @@ C_ABI = {
                         [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                          ctypes.c_double, _i64, ctypes.c_int, ctypes.c_int,
                          ctypes.c_int, ctypes.c_int, _vp, _vp]),
+    "pca_fps_host": (ctypes.c_int,
+                     [_vp, _vp, _vp, _vp, _i64, _i64, _i64, ctypes.c_int,
+                      ctypes.c_int, _vp]),
+    "pca_nearest_host": (ctypes.c_int,
+                         [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
+                          ctypes.c_int, ctypes.c_int, _vp]),
     "pca_fps_workspace_bytes": (ctypes.c_size_t,
                                 [_i64, _i64, _i64, _i64, ctypes.c_int]),
     "pca_fps": (ctypes.c_int,

@@ -699,6 +699,86 @@ bool host_sizes_ok(int64_t n, int64_t m, int64_t d, int64_t num_segments) {
   return n >= 0 && m >= 0 && d >= 1 && num_segments >= 1;
 }
 
+// ---- fps and nearest on the host ---------------------------------------------
+// Both follow the result contract of the GPU operators (which is the one of
+// the reference's CUDA kernels), so that CPU and GPU tensors give the same
+// rows.
+
+// Farthest point sampling of one example (csrc/cuda/fps_cuda.cu:10-66 is the
+// contract: running minima that start at 5e4, the next sample is the row with
+// the largest one, among equal ones the smallest (row - start) % 256, then the
+// smallest row; global row 0 when no row has a value).
+template <typename T>
+void fps_example(const T *src, int64_t d, int64_t begin, int64_t end,
+                 int64_t first, int64_t out_begin, int64_t out_end,
+                 int64_t *out) {
+  if (out_begin >= out_end)
+    return;
+  const int64_t rows = end - begin;
+  std::vector<T> nearest_sample((size_t)std::max<int64_t>(rows, 1), (T)5e4);
+  int64_t current = begin + first;
+  out[out_begin] = current;
+  for (int64_t s = out_begin + 1; s < out_end; ++s) {
+    const T *centre = src + current * d;
+    T best = (T)-1;
+    int64_t best_row = 0, best_slot = 0;
+    bool found = false;
+    for (int64_t i = 0; i < rows; ++i) {
+      const T *row = src + (begin + i) * d;
+      T acc = 0;
+      for (int64_t c = 0; c < d; ++c) {
+        const T diff = row[c] - centre[c];
+        acc = std::fma(diff, diff, acc);
+      }
+      // (a NaN distance leaves the minimum as it is)
+      T v = nearest_sample[(size_t)i];
+      v = acc < v ? acc : v;
+      nearest_sample[(size_t)i] = v;
+      const int64_t slot = i & 255;
+      // larger value; equal value: the smaller slot, then the smaller row
+      // (rows are visited in ascending order)
+      if (v > best || (found && v == best && slot < best_slot)) {
+        best = v;
+        best_row = begin + i;
+        best_slot = slot;
+        found = true;
+      }
+    }
+    current = found ? best_row : 0;
+    out[s] = current;
+  }
+}
+
+// The nearest row of y for one row of x (csrc/cuda/nearest_cuda.cu:10-66 is
+// the contract: strictly below 1e38, among equal distances the smallest
+// (row - start) % 1024, then the smallest row; 0 when nothing qualifies).
+template <typename T>
+int64_t nearest_row(const T *xrow, const T *y, int64_t d, int64_t begin,
+                    int64_t end) {
+  const T limit = (T)1e38f;
+  T best = limit;
+  int64_t best_row = 0, best_slot = 0;
+  bool found = false;
+  for (int64_t j = begin; j < end; ++j) {
+    const T *row = y + j * d;
+    T acc = 0;
+    for (int64_t c = 0; c < d; ++c) {
+      const T diff = xrow[c] - row[c];
+      acc = std::fma(diff, diff, acc);
+    }
+    const int64_t slot = (j - begin) & 1023;
+    if (acc < best || (found && acc == best && slot < best_slot)) {
+      if (!(acc < limit))
+        continue;
+      best = acc;
+      best_row = j;
+      best_slot = slot;
+      found = true;
+    }
+  }
+  return found ? best_row : 0;
+}
+
 bool host_cpu_ok() {
   return __builtin_cpu_supports("fma") && __builtin_cpu_supports("avx2");
 }
@@ -779,6 +859,79 @@ int pca_radius_host(const void *x, const void *y, const int64_t *ptr_x,
   p.ignore_same_index = ignore_same_index != 0;
   p.dist = nullptr;
   return run(p, edge_flags, num_threads, edges, num_edges, nullptr);
+}
+
+int pca_fps_host(const void *src, const int64_t *ptr, const int64_t *out_ptr,
+                 const int64_t *start, int64_t n, int64_t d,
+                 int64_t num_segments, int dtype, int num_threads,
+                 int64_t *out) {
+  g_host_error[0] = 0;
+  if (n < 0 || d < 1 || num_segments < 1 || ptr == nullptr ||
+      out_ptr == nullptr)
+    return host_fail(PCA_ERR_INVALID_ARGUMENT, "bad sizes or NULL pointers");
+  if (dtype != PCA_F32 && dtype != PCA_F64)
+    return host_fail(PCA_ERR_UNSUPPORTED,
+                     "fps on the host takes fp32 and fp64 points");
+  if (n == 0)
+    return PCA_OK;
+  if (src == nullptr || out == nullptr)
+    return host_fail(PCA_ERR_INVALID_ARGUMENT, "src or out is NULL");
+  parallel_blocks(num_segments, std::max(num_threads, 1), [&](int64_t b) {
+    const int64_t first = start ? start[b] : 0;
+    if (dtype == PCA_F32)
+      fps_example(static_cast<const float *>(src), d, ptr[b], ptr[b + 1],
+                  first, out_ptr[b], out_ptr[b + 1], out);
+    else
+      fps_example(static_cast<const double *>(src), d, ptr[b], ptr[b + 1],
+                  first, out_ptr[b], out_ptr[b + 1], out);
+  });
+  return PCA_OK;
+}
+
+int pca_nearest_host(const void *x, const void *y, const int64_t *ptr_x,
+                     const int64_t *ptr_y, int64_t n, int64_t m, int64_t d,
+                     int64_t num_segments, int dtype, int num_threads,
+                     int64_t *out) {
+  g_host_error[0] = 0;
+  if (n < 0 || m < 0 || d < 1 || num_segments < 1 || ptr_x == nullptr ||
+      ptr_y == nullptr)
+    return host_fail(PCA_ERR_INVALID_ARGUMENT, "bad sizes or NULL pointers");
+  if (dtype != PCA_F32 && dtype != PCA_F64)
+    return host_fail(PCA_ERR_UNSUPPORTED,
+                     "nearest on the host takes fp32 and fp64 points");
+  if (n == 0)
+    return PCA_OK;
+  if (x == nullptr || out == nullptr || (m > 0 && y == nullptr))
+    return host_fail(PCA_ERR_INVALID_ARGUMENT, "x, y or out is NULL");
+  // blocks of 256 searching rows, each inside one segment
+  struct Piece {
+    int64_t seg, begin, end;
+  };
+  std::vector<Piece> pieces;
+  for (int64_t b = 0; b < num_segments; ++b)
+    for (int64_t r = ptr_x[b]; r < ptr_x[b + 1]; r += 256)
+      pieces.push_back({b, r, std::min(r + 256, ptr_x[b + 1])});
+  // (rows behind the last pointer: the reference's lookup gives them the
+  // last example, csrc/cuda/utils.cuh:11-19)
+  for (int64_t r = ptr_x[num_segments]; r < n; r += 256)
+    pieces.push_back({num_segments - 1, r, std::min(r + 256, n)});
+  parallel_blocks((int64_t)pieces.size(), std::max(num_threads, 1),
+                  [&](int64_t i) {
+                    const Piece &pc = pieces[(size_t)i];
+                    for (int64_t r = pc.begin; r < pc.end; ++r) {
+                      if (dtype == PCA_F32)
+                        out[r] = nearest_row(
+                            static_cast<const float *>(x) + r * d,
+                            static_cast<const float *>(y), d, ptr_y[pc.seg],
+                            ptr_y[pc.seg + 1]);
+                      else
+                        out[r] = nearest_row(
+                            static_cast<const double *>(x) + r * d,
+                            static_cast<const double *>(y), d, ptr_y[pc.seg],
+                            ptr_y[pc.seg + 1]);
+                    }
+                  });
+  return PCA_OK;
 }
 
 } // extern "C"

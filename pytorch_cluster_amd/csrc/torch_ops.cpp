@@ -699,9 +699,44 @@ at::Tensor radius_batched(at::Tensor x, at::Tensor y, at::Tensor batch_x,
 
 // csrc/nearest.cpp:22-36 -> nearest_cuda (csrc/cuda/nearest_cuda.cu:68-94):
 // both pointer tensors are required, x and y are flattened to [N, -1].
+// Points that are not on a GPU: the package's own host search (the reference
+// has no operator for them: its Python entry point goes through
+// scipy.cluster.vq.vq, torch_cluster/nearest.py:93-124).
+at::Tensor nearest_host(at::Tensor x, at::Tensor y, at::Tensor ptr_x,
+                        at::Tensor ptr_y) {
+  PCA_CHECK_CPU(x);
+  PCA_CHECK_CPU(y);
+  PCA_CHECK_CPU(ptr_x);
+  PCA_CHECK_CPU(ptr_y);
+  PCA_CHECK_INPUT(x.dim() >= 1 && y.dim() >= 1);
+  x = x.view({x.size(0), -1});
+  y = y.view({y.size(0), -1});
+  PCA_CHECK_INPUT(x.size(1) == y.size(1));
+  PCA_CHECK_INPUT(ptr_x.dim() == 1 && ptr_y.dim() == 1);
+  PCA_CHECK_INPUT(ptr_x.numel() == ptr_y.numel() && ptr_x.numel() >= 2);
+  // (half and bfloat16 points are searched as float, integers as double)
+  const auto type = x.scalar_type() == at::kDouble || !x.is_floating_point()
+                        ? at::kDouble
+                        : at::kFloat;
+  x = x.to(type).contiguous();
+  y = y.to(type).contiguous();
+  ptr_x = ptr_x.to(at::kLong).contiguous();
+  ptr_y = ptr_y.to(at::kLong).contiguous();
+  auto out = at::empty({x.size(0)}, ptr_x.options());
+  const int rc = pca_nearest_host(
+      x.data_ptr(), y.size(0) > 0 ? y.data_ptr() : nullptr,
+      ptr_x.data_ptr<int64_t>(), ptr_y.data_ptr<int64_t>(), x.size(0),
+      y.size(0), x.size(1), ptr_x.numel() - 1,
+      type == at::kDouble ? PCA_F64 : PCA_F32, at::get_num_threads(),
+      out.data_ptr<int64_t>());
+  TORCH_CHECK(rc == PCA_OK, pca_host_last_error());
+  return out;
+}
+
 at::Tensor nearest(at::Tensor x, at::Tensor y, at::Tensor ptr_x,
                    at::Tensor ptr_y) {
-  TORCH_CHECK(x.device().is_cuda(), "No CPU version supported");
+  if (!x.device().is_cuda())
+    return nearest_host(x, y, ptr_x, ptr_y);
   PCA_CHECK_GPU(x);
   PCA_CHECK_GPU(y);
   PCA_CHECK_GPU(ptr_x);
@@ -759,8 +794,51 @@ at::Tensor nearest(at::Tensor x, at::Tensor y, at::Tensor ptr_x,
 // example = ceil(deg * ratio) in the ratio's element type, random start rows
 // from the device generator, one host read for the output size (here the
 // largest example comes with it and selects the kernel).
+// csrc/fps.cpp:31-33 -> fps_cpu (csrc/cpu/fps_cpu.cpp:11-64): the same
+// arithmetic for the numbers of samples (in float, as there: :25-27), a random
+// first row from the host generator, the sampling itself by the package's
+// host code.
+at::Tensor fps_host(at::Tensor src, at::Tensor ptr, at::Tensor ratio,
+                    bool random_start) {
+  PCA_CHECK_CPU(src);
+  PCA_CHECK_CPU(ptr);
+  PCA_CHECK_CPU(ratio);
+  PCA_CHECK_INPUT(ptr.dim() == 1);
+  PCA_CHECK_INPUT(ptr.numel() >= 2);
+  PCA_CHECK_INPUT(src.dim() >= 1);
+  src = src.view({src.size(0), -1});
+  const auto type =
+      src.scalar_type() == at::kDouble || !src.is_floating_point()
+          ? at::kDouble
+          : at::kFloat;
+  src = src.to(type).contiguous();
+  ptr = ptr.to(at::kLong).contiguous();
+  const int64_t batch_size = ptr.numel() - 1;
+  auto deg = ptr.narrow(0, 1, batch_size) - ptr.narrow(0, 0, batch_size);
+  auto out_ptr = deg.toType(at::kFloat) * ratio;
+  out_ptr = out_ptr.ceil().toType(at::kLong).cumsum(0);
+  out_ptr = at::cat({at::zeros({1}, ptr.options()), out_ptr}, 0).contiguous();
+  at::Tensor start;
+  if (random_start) {
+    start = (at::rand({batch_size}, at::kDouble) * deg.toType(at::kDouble))
+                .toType(at::kLong)
+                .contiguous();
+  }
+  auto out = at::empty({out_ptr[-1].item<int64_t>()}, ptr.options());
+  const int rc = pca_fps_host(
+      src.size(0) > 0 ? src.data_ptr() : nullptr, ptr.data_ptr<int64_t>(),
+      out_ptr.data_ptr<int64_t>(),
+      random_start ? start.data_ptr<int64_t>() : nullptr, src.size(0),
+      src.size(1), batch_size, type == at::kDouble ? PCA_F64 : PCA_F32,
+      at::get_num_threads(), out.data_ptr<int64_t>());
+  TORCH_CHECK(rc == PCA_OK, pca_host_last_error());
+  return out;
+}
+
 at::Tensor fps(at::Tensor src, at::Tensor ptr, at::Tensor ratio,
                bool random_start) {
+  if (!src.device().is_cuda())
+    return fps_host(src, ptr, ratio, random_start);
   PCA_CHECK_GPU(src);
   PCA_CHECK_GPU(ptr);
   PCA_CHECK_GPU(ratio);

@@ -1,11 +1,13 @@
-"""``nearest``: drop-in for ``torch_cluster.nearest`` on GPU tensors
+"""``nearest``: drop-in for ``torch_cluster.nearest``
 (reference: ``torch_cluster/nearest.py:7-91``, the ``x.is_cuda`` branch).
 
 Same signature, argument checks and errors.  The search itself is
 ``torch.ops.torch_cluster.nearest``, registered by this package's native
-library; the reference's route for CPU tensors (scipy's ``vq``,
-``torch_cluster/nearest.py:93-124``) has no counterpart here: the operator
-rejects them ("No CPU version supported", as ``csrc/nearest.cpp:33``).
+library.  CPU tensors take the same checks and the same operator, which
+searches them on host threads with the result contract of the GPU kernel
+(the reference normalises them per example and calls scipy's ``vq``,
+``torch_cluster/nearest.py:93-124``; its operator rejects CPU tensors,
+``csrc/nearest.cpp:33``).
 
 The reference reads from the device five times before it calls the operator
 (two sortedness tests, two ``batch.max()``, one comparison of the non-empty

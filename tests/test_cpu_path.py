@@ -184,3 +184,124 @@ def test_radius_graph_and_threads(oracle):
             assert got.shape == want.shape and (got.numpy() == want).all()
     finally:
         torch.set_num_threads(before)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("d", [1, 3, 7, 40])
+def test_fps_on_the_cpu_matches_the_checker(oracle, dtype, d):
+    rng = np.random.default_rng(d)
+    x = rng.standard_normal((3000, d)).astype(dtype)
+    ptr = np.array([0, 700, 700, 1001, 3000])
+    for ratio in (0.25, [0.5, 1.0, 0.01, 0.1]):
+        # the CPU operator sizes the samples in float, whatever the points'
+        # type (csrc/cpu/fps_cpu.cpp:25-27)
+        out_ptr = oracle.fps_out_ptr(ptr, ratio, np.float32)
+        share = torch.tensor(ratio, dtype=torch.float32)
+        got = torch.ops.torch_cluster.fps(torch.from_numpy(x),
+                                          torch.from_numpy(ptr), share, False)
+        want = oracle.fps_op(x, ptr, ratio)
+        if dtype == np.float32:
+            assert (got.numpy() == want).all()
+        else:
+            # (the checker sizes in the points' type: compare per example)
+            mine = oracle.fps_out_ptr(ptr, ratio, np.float64)
+            for b in range(4):
+                n = min(out_ptr[b + 1] - out_ptr[b], mine[b + 1] - mine[b])
+                assert (got.numpy()[out_ptr[b]:out_ptr[b] + n]
+                        == want[mine[b]:mine[b] + n]).all()
+        assert got.numel() == out_ptr[-1]
+
+
+def test_fps_entry_point_on_the_cpu(oracle, ref):
+    # the reference's fixture (test/test_fps.py:16-65) on CPU tensors
+    x = torch.tensor([[-1.0, -1.0], [-1.0, 1.0], [1.0, 1.0], [1.0, -1.0],
+                      [-2.0, -2.0], [-2.0, 2.0], [2.0, 2.0], [2.0, -2.0]])
+    batch = torch.tensor([0, 0, 0, 0, 1, 1, 1, 1])
+    assert pca.fps(x, batch, random_start=False).tolist() == [0, 2, 4, 6]
+    assert pca.fps(x, batch, ratio=0.5,
+                   random_start=False).tolist() == [0, 2, 4, 6]
+    assert pca.fps(x, batch, ratio=torch.tensor([0.5, 0.5]),
+                   random_start=False).tolist() == [0, 2, 4, 6]
+    assert pca.fps(x, ptr=[0, 4, 8], ratio=0.5,
+                   random_start=False).tolist() == [0, 2, 4, 6]
+    assert pca.fps(x, random_start=False).sort()[0].tolist() == [0, 5, 6, 7]
+
+    @torch.jit.script
+    def fps2(x: torch.Tensor, ratio: torch.Tensor) -> torch.Tensor:
+        return pca.fps(x, None, ratio, False)
+    assert fps2(x, torch.tensor([0.5])).sort()[0].tolist() == [0, 5, 6, 7]
+    # integer grid: exact ties, by the kernels' rule (slot of 256, then row)
+    rng = np.random.default_rng(11)
+    g = rng.integers(0, 5, (1500, 3)).astype(np.float32)
+    ptr = np.array([0, 600, 1500])
+    got = pca.fps(torch.from_numpy(g), ptr=torch.from_numpy(ptr), ratio=0.05,
+                  random_start=False)
+    assert (got.numpy() == oracle.fps_op(g, ptr, 0.05)).all()
+    # a random start is a row of the example, and the rest follows from it
+    torch.manual_seed(4)
+    pts = rng.standard_normal((900, 3)).astype(np.float32)
+    ptr = np.array([0, 300, 900])
+    got = pca.fps(torch.from_numpy(pts), ptr=torch.from_numpy(ptr),
+                  ratio=0.1).numpy()
+    assert 0 <= got[0] < 300 and 300 <= got[30] < 900
+    want = oracle.fps_op(pts, ptr, 0.1, start=[got[0], got[30] - 300])
+    assert (got == want).all()
+    # and the reference's compiled CPU operator, where no near-tie decides
+    # (it sums the squares in another order)
+    big = rng.standard_normal((4000, 3)).astype(np.float32)
+    ptr = np.array([0, 1500, 4000])
+    got = pca.fps(torch.from_numpy(big), ptr=torch.from_numpy(ptr),
+                  ratio=0.05, random_start=False).numpy()
+    want = ref.ref_fps(big, ptr, 0.05)
+    assert got.shape == want.shape
+    first_diff = np.flatnonzero(got != want)
+    assert first_diff.size == 0 or first_diff[0] > 50
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("d", [1, 2, 3, 16, 100])
+def test_nearest_on_the_cpu_matches_the_checker(oracle, dtype, d):
+    rng = np.random.default_rng(d + 100)
+    x = rng.standard_normal((5000, d)).astype(dtype)
+    y = rng.standard_normal((1300, d)).astype(dtype)
+    ptr_x = np.array([0, 1200, 1200, 5000])
+    ptr_y = np.array([0, 300, 300, 1300])
+    got = torch.ops.torch_cluster.nearest(
+        torch.from_numpy(x), torch.from_numpy(y), torch.from_numpy(ptr_x),
+        torch.from_numpy(ptr_y))
+    assert (got.numpy() == oracle.nearest_op(x, y, ptr_x, ptr_y)).all()
+    # brute force in float64 where no near-tie decides
+    if dtype == np.float64:
+        for b in (0, 2):
+            xs = x[ptr_x[b]:ptr_x[b + 1]][:200]
+            ys = y[ptr_y[b]:ptr_y[b + 1]]
+            dd = ((xs[:, None, :] - ys[None, :, :]) ** 2).sum(-1)
+            assert (got.numpy()[ptr_x[b]:ptr_x[b] + 200]
+                    == dd.argmin(1) + ptr_y[b]).all()
+
+
+def test_nearest_entry_point_on_the_cpu(oracle):
+    # the reference's fixture (test/test_nearest.py:11-64) on CPU tensors
+    x = torch.tensor([[-1.0, -1.0], [-1.0, 1.0], [1.0, 1.0], [1.0, -1.0],
+                      [-2.0, -2.0], [-2.0, 2.0], [2.0, 2.0], [2.0, -2.0]])
+    y = torch.tensor([[-1.0, 0.0], [1.0, 0.0], [-2.0, 0.0], [2.0, 0.0]])
+    batch_x = torch.tensor([0, 0, 0, 0, 1, 1, 1, 1])
+    batch_y = torch.tensor([0, 0, 1, 1])
+    assert pca.nearest(x, y, batch_x, batch_y).tolist() \
+        == [0, 0, 1, 1, 2, 2, 3, 3]
+    assert pca.nearest(x, y).tolist() == [0, 0, 1, 1, 2, 2, 3, 3]
+    with pytest.raises(ValueError, match="'batch_x' is not sorted"):
+        pca.nearest(x, y, torch.tensor([0, 0, 1, 0, 1, 1, 1, 1]), batch_y)
+    with pytest.raises(ValueError, match="do not occur in 'batch_y'"):
+        pca.nearest(x, y, batch_x, torch.tensor([0, 0, 0, 0]))
+    # ties (integer grid), NaN rows and rows beyond the 1e38 limit
+    rng = np.random.default_rng(2)
+    gx = rng.integers(0, 4, (3000, 2)).astype(np.float32)
+    gy = rng.integers(0, 4, (2500, 2)).astype(np.float32)
+    gy[5] = np.nan
+    gy[9] = 3e19
+    gx[17] = np.nan
+    got = pca.nearest(torch.from_numpy(gx), torch.from_numpy(gy))
+    assert (got.numpy() == oracle.nearest_op(gx, gy, [0, 3000],
+                                             [0, 2500])).all()
+    assert got[17] == 0  # nothing qualifies for a NaN row

@@ -69,11 +69,18 @@ def test_operators_are_registered_and_scriptable():
     assert "float r" in schema and "bool ignore_same_index" in schema
 
 
-def test_gpu_only_operators_refuse_cpu_tensors():
+def test_operators_refuse_tensors_of_mixed_devices():
+    # (every operator takes CPU tensors; what it refuses is a mix)
     x = torch.rand(8, 3)
-    with pytest.raises(RuntimeError, match="No CPU version supported"):
-        torch.ops.torch_cluster.nearest(x, x, torch.tensor([0, 8]),
+    meta = torch.empty(8, 3, device="meta")
+    with pytest.raises(RuntimeError):
+        torch.ops.torch_cluster.nearest(x, meta, torch.tensor([0, 8]),
                                         torch.tensor([0, 8]))
+    # half-precision points are searched in float on the host
+    got = torch.ops.torch_cluster.nearest(x.half(), x.half(),
+                                          torch.tensor([0, 8]),
+                                          torch.tensor([0, 8]))
+    assert got.tolist() == list(range(8))
 
 
 def test_empty_inputs_short_circuit():

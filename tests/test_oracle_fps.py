@@ -205,15 +205,14 @@ def test_wrapper_fixture(oracle_fps_op):
                    random_start=False).tolist() == [0, 2, 4, 6]
 
 
-def test_entry_point_is_scriptable_and_rejects_cpu():
+def test_entry_point_is_scriptable_and_takes_cpu_tensors():
     @torch.jit.script
     def fps2(x: Tensor, ratio: Tensor) -> Tensor:
         return pca.fps(x, None, ratio, False)
 
     x = torch.rand(16, 3)
-    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
-        fps2(x, torch.tensor([0.5]))
-    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
-        pca.fps(x, random_start=False)
+    assert torch.equal(fps2(x, torch.tensor([0.5])),
+                       pca.fps(x, random_start=False))
+    assert pca.fps(x, random_start=False).numel() == 8
     schema = str(torch.ops.torch_cluster.fps.default._schema)
     assert "Tensor ratio, bool random_start" in schema
