@@ -373,9 +373,27 @@ class Cases:
             ms, out = _median_ms(
                 t, lambda: t.ops.torch_cluster.fps(pts, ptr, ratio, False),
                 reps or 5)
+            # A sample step depends on the one before it, and a cloud is
+            # one workgroup's (its running minima stay in that compute
+            # unit's registers), so the floor is latency, not bandwidth:
+            # per step and row 3 subtractions, 3 multiply-adds, the minimum
+            # and two compare/selects for the running maximum = 9 vector
+            # instructions, 4 cycles each per wave of 64 on one of the
+            # unit's 4 SIMDs at 2.4 GHz; the two reductions across the
+            # workgroup come on top.
+            step_us = ms * 1e3 / (points // 4)
+            floor_us = points / 64.0 * 9 * 4 / 4 / 2400.0
             report["fps %dx%d ratio 0.25" % (clouds, points)] = {
                 "ms": ms, "samples": int(out.numel()),
-                "us_per_sample_step": ms * 1e3 / (points // 4)}
+                "us_per_sample_step": step_us,
+                "roofline": {
+                    "bound": "valu-latency", "unit": "us/step",
+                    "floor": floor_us, "achieved": step_us,
+                    "frac": floor_us / step_us,
+                    "note": "vector-ALU time of one compute unit per "
+                            "sample step (9 instructions per row); "
+                            "clouds run side by side, %d of the chip's "
+                            "256 units busy" % clouds}}
         return report
 
     # the headline workload and large clouds through both search strategies
@@ -467,6 +485,22 @@ def measured_traffic():
         return None
 
 
+def probe_feat_loop(reps):
+    """pytorch_cluster_amd/csrc/probes/feat_loop_probe.hip: the loop of the
+    feature-space filter with everything but the matrix-core chain taken
+    away, then put back piece by piece (best of `reps` launches each)."""
+    import ctypes
+    here = os.path.dirname(os.path.abspath(__file__))
+    lib = ctypes.CDLL(os.path.join(here, "pytorch_cluster_amd",
+                                   "libpca_probe.so"))
+    text = ctypes.create_string_buffer(1 << 16)
+    count = lib.pca_probe_feat_loop(ctypes.c_int(reps), text,
+                                    ctypes.c_int(len(text)))
+    if count < 0:
+        sys.exit("bench.py: the probe failed (a HIP call returned an error)")
+    sys.stdout.write(text.value.decode())
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -495,7 +529,14 @@ def main():
                     help="also run a plain 1 GiB device copy three times, so "
                          "that a counter profile of this command can scale "
                          "FETCH_SIZE / WRITE_SIZE by a kernel of known traffic")
+    ap.add_argument("--probe", choices=("feat_loop",), default=None,
+                    help="run a measurement aid instead of the benchmark: "
+                         "feat_loop = the stripped matrix-core loop of the "
+                         "feature-space filter, variant by variant (one JSON "
+                         "line each)")
     args = ap.parse_args()
+    if args.probe == "feat_loop":
+        return probe_feat_loop(max(args.steps // 4, 3))
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not "
                  "supported (the path would shard by segment, without "

@@ -7,6 +7,8 @@
 Outputs (next to this file, git-ignored):
   libpca_neighbors.so   HIP kernels + the C ABI of include/pca_neighbors.h
   _torch_ops.so         TorchScript operator binding (links the above)
+  libpca_probe.so       csrc/probes/: measurement aids (`bench.py --probe`),
+                        no part of the searches
 """
 import argparse
 import concurrent.futures
@@ -20,6 +22,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "_build")
 CAPI_LIB = os.path.join(HERE, "libpca_neighbors.so")
 TORCH_OPS_LIB = os.path.join(HERE, "_torch_ops.so")
+PROBE_LIB = os.path.join(HERE, "libpca_probe.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
@@ -78,6 +81,12 @@ def build_capi(jobs):
     return CAPI_LIB
 
 
+def build_probes():
+    sources = sorted(glob.glob(os.path.join(CSRC, "probes", "*.hip")))
+    _run([HIPCC] + HIP_FLAGS + ["-shared"] + sources + ["-o", PROBE_LIB])
+    return PROBE_LIB
+
+
 def build_torch_ops():
     import torch
     from torch.utils import cpp_extension
@@ -106,6 +115,7 @@ def build_torch_ops():
 def build_all(jobs=None, torch_ops=True):
     jobs = jobs or min(8, os.cpu_count() or 1)
     build_capi(jobs)
+    build_probes()
     if torch_ops:
         build_torch_ops()
 
