@@ -58,13 +58,44 @@
 // are resolved by all lanes together, exactly, when a queue fills up or the
 // tile ends -- as in knn_lowd_impl.hpp.  Slices, shared bounds (`tau`) and the merge of partial
 // lists are those of knn_lowd_impl.hpp with tiles of 128 queries.
+//
+// Start of a scan.  With empty lists every row passes, and until the bounds
+// have come down most rows do: three quarters of all insertions of a scan
+// over 4,096 rows fall into its first 1,024.  So before the first tile is
+// scanned, its filter values are formed once without a cut: of the 16 values
+// a lane receives per step it takes the smallest, evaluates that row exactly,
+// and keeps the ceil(k / 2) smallest of these distances (one row per step:
+// all different, and different from the partner lane's).  The larger of the
+// two lanes' ceil(k / 2)-th distances bounds the query's k-th distance (at
+// least k rows lie at or below it), and it is a bound of the quality "the
+// k-th of 64 minima of 16": about k + k / 4 rows of the first tile pass
+// it instead of k (1 + ln(1024 / k)).  The lists then fill from rows that
+// pass this bound, in the scan proper.
 #pragma once
 
 #include "knn_mfma_impl.hpp"
 
 namespace pca {
 
+#ifdef PCA_MC_STATS
+// (instrumented builds only) 0 drain rounds, 1 rounds with an insertion,
+// 2 lane-rounds with a row, 3 lane-rounds with an insertion, 4 steps,
+// 5 steps with a parked mask, 6 drains, 7 parked lane-steps
+__device__ unsigned long long g_mc_stats[8];
+#define PCA_MC_COUNT(i, v) atomicAdd(&g_mc_stats[i], (unsigned long long)(v))
+#else
+#define PCA_MC_COUNT(i, v) ((void)0)
+#endif
+
 constexpr int kMcQueries = 128; // queries per workgroup
+// unsliced scans of up to this many LDS tiles start with a bound from sampled
+// rows (measured on 64 x 2,048 / 32 x 4,096 points: 12-30 % less time in the
+// kernel for k = 7 .. 31; slices of longer scans pay the sampling once each
+// and already share their bounds: 2-8 % more time on 8 x 16,384 points)
+#ifndef PCA_MC_SEED_TILES
+#define PCA_MC_SEED_TILES 8
+#endif
+constexpr int kMcSeedTiles = PCA_MC_SEED_TILES;
 constexpr int kMcQueueCap = 8; // parked steps per lane
 
 template <int DIM> struct McShape {
@@ -490,6 +521,7 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
   // tile in LDS together.
   auto drain = [&](int g_base, int rows) {
     bool changed = false; // wave-uniform
+    PCA_MC_COUNT(6, lane == 0);
     const int qcount = (qnext - qfirst) / QROW;
     int taken = 0;         // parked steps this lane has started on
     uint32_t pending = 0;  // rows of the current step still to look at
@@ -504,6 +536,8 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
       const bool has = pending != 0;
       if (!__any(has))
         break;
+      PCA_MC_COUNT(0, lane == 0);
+      PCA_MC_COUNT(2, has);
       // bit 15 - v of the mask stands for accumulator v = row
       // 8 (v / 4) + v % 4 of the lane's rows: highest bit first
       const int bit = 31 - __builtin_clz(has ? pending : 1u);
@@ -531,6 +565,8 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
       const bool ok = has && j < rows && d < thresh;
       if (!__any(ok))
         continue;
+      PCA_MC_COUNT(1, lane == 0);
+      PCA_MC_COUNT(3, ok);
       const uint32_t row_id = NEAREST
                                   ? nearest_tie((uint32_t)(g_base + j - x_begin))
                                   : (uint32_t)(g_base + j);
@@ -574,6 +610,93 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
     const int rows = min(TX, c_count - t * TX);
     const int steps32 = (rows + 31) / 32;
 
+    // a bound before the first row is looked at (see "Start of a scan")
+    constexpr int SEEDS = K / 2;
+    const bool seeded = !NEAREST && K >= 8 && t == 0 &&
+                        steps32 >= 2 * SEEDS && num_tiles <= kMcSeedTiles &&
+                        p.num_chunks == 1;
+    if (!NEAREST && K >= 8 && seeded) {
+      float seed[SEEDS > 0 ? SEEDS : 1];
+#pragma unroll
+      for (int j = 0; j < SEEDS; ++j)
+        seed[j] = __builtin_inff();
+      // no cut in the product: the slots that carry it multiply by zero
+      yb[WI] = __builtin_bit_cast(mc_bf16x8_t, yb_plain);
+      uint4 a_seed[NI];
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        a_seed[i] = rows_lds[i][col];
+      for (int rt = 0; rt < steps32; ++rt) {
+        mfma_acc_t acc = {0};
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              __builtin_bit_cast(mc_bf16x8_t, a_seed[i]), yb[i], acc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+          a_seed[i] = rows_lds[i][min(rt + 1, TX / 32 - 1) * 32 + col];
+        // the smallest of the 16 values, its accumulator number in the four
+        // lowest bits (which of two nearly equal rows is taken does not
+        // matter; a NaN -- padding -- loses against any number)
+        float tagged[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          tagged[v] = __uint_as_float((__float_as_uint(acc[v]) & ~15u) |
+                                      (uint32_t)v);
+        float m0 = min3f(tagged[0], tagged[1], tagged[2]);
+        float m1 = min3f(tagged[3], tagged[4], tagged[5]);
+        float m2 = min3f(tagged[6], tagged[7], tagged[8]);
+        float m3 = min3f(tagged[9], tagged[10], tagged[11]);
+        float m4 = min3f(tagged[12], tagged[13], tagged[14]);
+        m0 = min3f(m0, m1, m2);
+        m3 = min3f(m3, m4, tagged[15]);
+        const int v = (int)(__float_as_uint(__builtin_fminf(m0, m3)) & 15u);
+        const int j = rt * 32 + 4 * half + 2 * (v & 12) + (v & 3);
+        float row[XF];
+#pragma unroll
+        for (int e = 0; e < XF; e += 4) {
+          const uint4 q4 = rows_lds[NI + e / 4][j];
+          row[e] = __uint_as_float(q4.x);
+          row[e + 1] = __uint_as_float(q4.y);
+          row[e + 2] = __uint_as_float(q4.z);
+          row[e + 3] = __uint_as_float(q4.w);
+        }
+        const float d0 = row[0] - yq[0];
+        float d = d0 * d0;
+#pragma unroll
+        for (int c = 1; c < DIM; ++c) {
+          const float dc = row[c] - yq[c];
+          d = __builtin_fmaf(dc, dc, d);
+        }
+        // (a padding row, a NaN or a distance beyond the limit is no sample)
+        const float sample = (j < rows && d < kLimit) ? d : __builtin_inff();
+#pragma unroll
+        for (int e = SEEDS - 1; e >= 1; --e)
+          seed[e] = __builtin_amdgcn_fmed3f(seed[e - 1], seed[e], sample);
+        seed[0] = __builtin_fminf(seed[0], sample);
+      }
+      // the ceil(k / 2)-th smallest sample of this lane and of its partner
+      const int mine = (k + 1) / 2 - 1;
+      float own = __builtin_inff();
+#pragma unroll
+      for (int e = 0; e < SEEDS; ++e)
+        if (e == mine) {
+          asm volatile(""); // (keeps this a branch)
+          own = seed[e];
+        }
+      const auto both = __builtin_amdgcn_permlane32_swap(
+          __float_as_uint(own), __float_as_uint(own), false, false);
+      const float partner = __uint_as_float(half ? both[0] : both[1]);
+      const float bound = __builtin_fmaxf(own, partner);
+      if (valid && bound < kLimit) {
+        // (equality must pass: the rows at the bound are among the k nearest)
+        shared = __builtin_fminf(shared, next_up_positive(bound));
+        if (shared < thresh)
+          set_thresh(shared);
+      }
+      refresh_cut();
+    }
+
     uint4 a_next[NI];
 #pragma unroll
     for (int i = 0; i < NI; ++i)
@@ -610,7 +733,10 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v)
         mask = __builtin_amdgcn_alignbit(mask, __float_as_uint(acc[v]), 31);
+      PCA_MC_COUNT(4, lane == 0);
       if (__any(mask != 0)) {
+        PCA_MC_COUNT(5, lane == 0);
+        PCA_MC_COUNT(7, mask != 0);
         if (mask != 0) {
           *reinterpret_cast<uint32_t *>(
               reinterpret_cast<char *>(&queue[0][0]) + qnext) =
@@ -621,7 +747,7 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
         // 15 and 31 of its first tile -- while the lists are empty or their
         // bounds still loose and many rows pass)
         if (__any(qnext >= qfirst + QCAP * QROW) ||
-            (t == 0 && (rt & (rt + 1)) == 0))
+            (t == 0 && !seeded && (rt & (rt + 1)) == 0))
           drain(g_base, rows);
       }
     }

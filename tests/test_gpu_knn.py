@@ -147,6 +147,46 @@ def test_exact_ties_keep_lowest_rows(oracle, lowd_path):
         assert (gd.reshape(500, k) == d2).all()
 
 
+@pytest.mark.parametrize("d", [2, 3, 4])
+@pytest.mark.parametrize("k", [4, 7, 8, 15, 16, 21, 24, 31, 32])
+@pytest.mark.parametrize("case", ["uniform", "grid_ties", "duplicates",
+                                  "bad_rows"])
+def test_scans_that_start_from_sampled_rows(oracle, d, k, case):
+    # unsliced scans over 1-8 LDS tiles of 1,024 rows take their first bound
+    # from one exactly evaluated row per 16 (the row the matrix cores rate
+    # nearest): whatever the sample, the edges are the checker's
+    rng = np.random.default_rng(stable_seed("seeded", d, k, case))
+    sizes = [1024, 1500, 4096, 333, 2049]  # (333: too short to sample)
+    ptr_x = np.concatenate([[0], np.cumsum(sizes)])
+    n = int(ptr_x[-1])
+    if case == "uniform":
+        x = rng.random((n, d), dtype=np.float32)
+    elif case == "grid_ties":
+        x = rng.integers(0, 6, (n, d)).astype(np.float32)
+    elif case == "duplicates":
+        x = rng.random((n, d), dtype=np.float32)
+        x[::3] = x[1::3][:len(x[::3])]
+        x[ptr_x[2]:ptr_x[2] + 2000] = 0.25
+    else:
+        x = rng.standard_normal((n, d)).astype(np.float32)
+        bad = rng.choice(n, 400, replace=False)
+        x[bad[:100], 0] = np.nan
+        x[bad[100:200], d - 1] = np.inf
+        x[bad[200:300]] = 3e5          # squared distance beyond the limit
+        x[bad[300:]] *= 1e19           # norm that is not moderate
+    m_sizes = [200, 130, 257, 40, 128]
+    ptr_y = np.concatenate([[0], np.cumsum(m_sizes)])
+    y = np.concatenate([x[ptr_x[b]:ptr_x[b + 1]][rng.choice(sizes[b], ms)]
+                        for b, ms in enumerate(m_sizes)])
+    if case == "uniform":
+        y = y + rng.random(y.shape, dtype=np.float32) * 0.01
+    got, gd = gpu_knn(x, y, ptr_x, ptr_y, k)
+    want, wd = oracle_knn_edges(oracle, x, y, ptr_x, ptr_y, k)
+    assert got.shape == want.shape
+    assert (got == want).all()
+    assert (gd == wd).all()
+
+
 def test_duplicate_points(oracle):
     x = np.zeros((700, 3), dtype=np.float32)
     got, gd = gpu_knn(x, x[:300], None, None, 9)
