@@ -256,40 +256,6 @@ plan_segments(const int64_t *__restrict__ ptr, int m, int num_segments,
     work_start[num_segments] = partial[tid];
 }
 
-// The XCD (0..7: the eight dies of the device, each with an L2 of its own) the
-// calling wave runs on.
-__device__ __forceinline__ int xcd_of_wave() {
-  return __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7; // HW_REG_XCC_ID[3:0]
-}
-
-// Hands every workgroup of a launch of tiles x chunks workgroups one work item
-// (tile of queries, slice of the rows), each item exactly once, such that the
-// workgroups that run on one XCD take neighbouring items: XCD x starts with
-// the x-th eighth of the tiles -- slice 0 of all of them, then slice 1, ... --
-// and goes on to the following eighths when its own is used up.  Neighbouring
-// tiles read the same rows, which then stay in that XCD's L2, and a tile's
-// slices are still taken in ascending order (a later slice starts with the
-// bounds the earlier ones have published).
-// counters: 8 ints, zero before the launch.  Called by thread 0 only; returns
-// the tile and stores the slice, or -1.
-__device__ __forceinline__ int claim_item_on_xcd(int *counters, int tiles,
-                                                 int chunks, int *chunk_out) {
-  const int x = xcd_of_wave();
-  for (int t = 0; t < 8; ++t) {
-    const int xx = (x + t) & 7;
-    const int lo = (int)((long long)tiles * xx / 8);
-    const int width = (int)((long long)tiles * (xx + 1) / 8) - lo;
-    if (width <= 0)
-      continue;
-    const int j = atomicAdd(&counters[xx], 1);
-    if (j < width * chunks) {
-      *chunk_out = j / width;
-      return lo + j % width;
-    }
-  }
-  return -1; // (not reached: there are as many items as workgroups)
-}
-
 // Pointers of both sides from sorted example ids, by all waves of one
 // workgroup: ptr[b] = number of rows whose id is below b.  A wave takes one
 // (side, b) at a time and narrows the range 65-fold per step -- its 64 lanes

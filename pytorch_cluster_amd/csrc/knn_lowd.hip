@@ -136,9 +136,9 @@ size_t mc_split_bytes(const KnnLowdConfig &cfg, int n, int d) {
   return align256(sizeof(uint4) * (size_t)n * per_row);
 }
 
-// shared bounds [m], then the 8 counters of the work items taken per XCD
+// shared bounds [m]
 size_t lowd_bounds_bytes(int m) {
-  return align256(sizeof(float) * (size_t)m) + 256;
+  return align256(sizeof(float) * (size_t)m);
 }
 
 size_t knn_lowd_scratch_bytes(const KnnLowdConfig &cfg, int n, int m, int d,
@@ -215,7 +215,6 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
   p.x_split = nullptr;
   char *base = static_cast<char *>(scratch);
   const size_t tau_bytes = lowd_bounds_bytes(in.m);
-  p.claim = nullptr;
   // tiles between two exchanges of bounds among the slices of a query
   // (a power of two; PCA_KNN_SYNC_PERIOD overrides)
   int period = env_int("PCA_KNN_SYNC_PERIOD", 4);
@@ -233,20 +232,12 @@ hipError_t launch_knn_lowd(const SearchInput &in, int k, bool cosine,
     // rows, start value of the shared bounds
     uint4 *split = reinterpret_cast<uint4 *>(base + tau_bytes);
     p.x_split = split;
-    // PCA_KNN_XCD_CLAIM=1: work items are handed out XCD by XCD instead of by
-    // workgroup number.  On 8 scans of 60,000-200,000 points that cut the
-    // kernel's HBM reads from 373 MB to 112 MB per launch and made it 25 %
-    // slower, so it stays an option.
-    if (env_int("PCA_KNN_XCD_CLAIM", 0) != 0)
-      p.claim = reinterpret_cast<int *>(
-          base + align256(sizeof(float) * (size_t)in.m));
     // (only this set-up clears the compaction's block sums: the other path
     // leaves the counting to the compaction)
     p.edge_sums = nearest_out ? nullptr : out.edge_sums;
     p.self_pos = out.self_pos;
     p.kept = out.kept;
     McSetup a;
-    a.claim = p.claim;
     a.edge_sums = p.edge_sums;
     a.edge_blocks =
         (in.m + kCompactBlockQueries - 1) / kCompactBlockQueries + 1;

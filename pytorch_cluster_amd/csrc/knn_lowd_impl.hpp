@@ -67,8 +67,6 @@ struct KnnLowdParams {
   int num_chunks;        // S: slices of every segment's x rows
   const uint4 *x_split;  // matrix-core kernel: packed rows of x
   float *tau;            // [m] shared pruning bounds or NULL
-  int *claim = nullptr;  // matrix-core kernel: 8 zeroed counters of the work
-                         // items taken per XCD, or NULL (item = workgroup id)
   int sync_mask = 3;     // ... bounds are exchanged when (tile & mask) == mask
   double *partial;       // [S * tiles][k][tile queries] keys (S > 1) or NULL
   int *out_idx;          // dense results (written here only when S == 1)

@@ -194,7 +194,6 @@ struct McSetup {
   int n, d_in;
   uint4 *out;
   float *tau; // [m] or NULL
-  int *claim; // 8 counters to clear, or NULL
   // the compaction's block sums to clear (DenseResult::edge_sums), or NULL
   unsigned long long *edge_sums = nullptr;
   int edge_blocks = 0;
@@ -210,8 +209,6 @@ template <int DIM>
 __global__ __launch_bounds__(kPlanThreads) void mc_setup_kernel(McSetup a) {
   constexpr int REC = McShape<DIM>::REC;
   __shared__ int partial[kPlanThreads];
-  if (blockIdx.x == 0 && a.claim != nullptr && threadIdx.x < 8)
-    a.claim[threadIdx.x] = 0;
   if (a.edge_sums != nullptr)
     for (int b = blockIdx.x * kPlanThreads + threadIdx.x; b < a.edge_blocks;
          b += gridDim.x * kPlanThreads)
@@ -278,35 +275,18 @@ knn_lowd_mc_kernel(KnnLowdParams p) {
   const int half = lane >> 5;
   const int col = lane & 31;
 
-  // this workgroup's work item = (slice, tile of queries): from its own
-  // number, or taken next to those of the other workgroups on this XCD (the
-  // queue's first words pass it from thread 0 to the others: the kernel's LDS
-  // is exactly a quarter of a CU's)
+  // this workgroup's work item = (slice, tile of queries), from its number
+  // (handing the items out XCD by XCD, so that neighbours share an L2, was
+  // tried: a third of the HBM reads and 25 % more time on 8 scans of
+  // 60,000-200,000 points -- at 2 % of the HBM roof the reads cost nothing,
+  // the hand-out through atomics does)
   const int total_tiles = p.work_start[p.num_segments];
   if (total_tiles == 0)
     return;
-  int chunk, tile;
-  if (p.claim != nullptr) {
-    int *pass = reinterpret_cast<int *>(&queue[0][0]);
-    if (tid == 0) {
-      int c = 0;
-      pass[0] = claim_item_on_xcd(p.claim, (int)gridDim.x / p.num_chunks,
-                                  p.num_chunks, &c);
-      pass[1] = c;
-    }
-    __syncthreads();
-    // (the same in every lane: kept in scalar registers like blockIdx.x)
-    tile = __builtin_amdgcn_readfirstlane(pass[0]);
-    chunk = __builtin_amdgcn_readfirstlane(pass[1]);
-    __syncthreads(); // before the queue is used as a queue
-    if (tile < 0 || tile >= total_tiles)
-      return;
-  } else {
-    chunk = blockIdx.x / total_tiles;
-    tile = blockIdx.x - chunk * total_tiles;
-    if (chunk >= p.num_chunks)
-      return;
-  }
+  const int chunk = blockIdx.x / total_tiles;
+  const int tile = blockIdx.x - chunk * total_tiles;
+  if (chunk >= p.num_chunks)
+    return;
   const int item = chunk * total_tiles + tile;
   const int seg = find_segment(p.work_start, p.num_segments, tile);
   const int x_begin = p.ptr_x ? (int)p.ptr_x[seg] : 0;

@@ -90,7 +90,6 @@ hipError_t launch_radius_mc(const SearchInput &in, float r2,
   a.d_in = in.d;
   a.out = static_cast<uint4 *>(scratch);
   a.tau = nullptr;
-  a.claim = nullptr;
   a.m = in.m;
   a.tau_value = 0.0f;
   a.ptr_y = in.ptr_y;
