@@ -474,13 +474,28 @@ def other_configs(torch, pca, testing, dev, only=None):
 
 def measured_traffic():
     """HBM bytes per launch of the dominant kernel from the committed rocprof
-    counter summary, if there is one."""
+    counter summary, and the commit that summary was measured at, if there is
+    one: (bytes, commit)."""
     import re
     path = os.path.join(ROOT, "profiles", "knn_lowd_lidar_traffic.md")
     try:
         with open(path) as f:
-            found = re.search(r"hbm_bytes_per_launch:\s*(\d+)", f.read())
-        return int(found.group(1)) if found else None
+            text = f.read()
+    except OSError:
+        return None, None
+    found = re.search(r"hbm_bytes_per_launch:\s*(\d+)", text)
+    commit = re.search(r"[Mm]easured at commit\s+([0-9a-f]{7,40})", text)
+    return (int(found.group(1)) if found else None,
+            commit.group(1) if commit else None)
+
+
+def built_commit():
+    """The commit the native libraries were built from (written by
+    pytorch_cluster_amd/build.py; "+" marks a tree with local changes)."""
+    path = os.path.join(ROOT, "pytorch_cluster_amd", "build_commit.txt")
+    try:
+        with open(path) as f:
+            return f.read().strip() or None
     except OSError:
         return None
 
@@ -629,8 +644,10 @@ def main():
             "frac": achieved / PEAK_FP32_TFLOPS,
             "kernel_ms": kernel_s * 1e3,
             "flop_per_launch": flops,
-            "traffic": measured_traffic(),
+            "traffic": measured_traffic()[0],
+            "traffic_commit": measured_traffic()[1],
         },
+        "commit": built_commit(),
     }
     if binned:
         # the events bracket binning + search here, and the work is not the

@@ -112,8 +112,26 @@ def build_torch_ops():
     return TORCH_OPS_LIB
 
 
+def note_commit():
+    """Writes the commit the libraries are built from next to them (for the
+    benchmark line; the GPU box gets the tree without its history)."""
+    repo = os.path.dirname(HERE)
+    try:
+        head = subprocess.run(["git", "-C", repo, "rev-parse", "--short",
+                               "HEAD"], capture_output=True, text=True,
+                              check=True).stdout.strip()
+        dirty = subprocess.run(["git", "-C", repo, "status", "--porcelain",
+                                "--untracked-files=no"], capture_output=True,
+                               text=True, check=True).stdout.strip()
+    except (OSError, subprocess.CalledProcessError):
+        return
+    with open(os.path.join(HERE, "build_commit.txt"), "w") as f:
+        f.write(head + ("+" if dirty else "") + "\n")
+
+
 def build_all(jobs=None, torch_ops=True):
     jobs = jobs or min(8, os.cpu_count() or 1)
+    note_commit()
     build_capi(jobs)
     build_probes()
     if torch_ops:
