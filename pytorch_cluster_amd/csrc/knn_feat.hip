@@ -14,8 +14,8 @@ namespace pca {
                                         int, hipStream_t);                     \
   template <>                                                                  \
   hipError_t launch_feat_pack<NB>(const float *, const float *,                \
-                                  const float *, int, int, bool,               \
-                                  FeatGlobals *, uint4 *, hipStream_t);
+                                  const float *, const unsigned *, int, int,   \
+                                  bool, FeatGlobals *, uint4 *, hipStream_t);
 PCA_DECLARE_FEAT_BLOCKS(3)
 PCA_DECLARE_FEAT_BLOCKS(5)
 PCA_DECLARE_FEAT_BLOCKS(9)
@@ -85,12 +85,18 @@ __global__ __launch_bounds__(kBlock) void feat_init_kernel(
   }
   if (i < redo_cap)
     hit_count[i] = 0;
+  if (i < 256) {
+    g->hist_x[i] = 0;
+    g->hist_y[i] = 0;
+  }
   if (i == 0) {
     g->max_bits = 0;
     g->odd_rows = 0;
     g->any_redo = 0;
     g->unresolved = 0;
     g->queued = 0;
+    g->out_limit = 0xffffffffu;
+    g->n_out = 0;
   }
 }
 
@@ -100,10 +106,17 @@ constexpr int kSecondPassChunks = 16;
 // Squared norms of rows (16 lanes per row, coalesced reads; any summation
 // order serves the filter; NaN for a row with a non-finite component) and the
 // largest finite |component| of the matrix.
+// big_out (or null): per row, the float bits of that largest |component|;
+// hist (or null): rows per binary exponent of it.
 __global__ __launch_bounds__(kBlock) void feat_rows_kernel(
     const float *__restrict__ x, int n, int d, float *__restrict__ sq_out,
-    FeatGlobals *g) {
+    FeatGlobals *g, unsigned *__restrict__ big_out,
+    unsigned *__restrict__ hist) {
   __shared__ unsigned part[kBlock / kWave];
+  __shared__ unsigned local_hist[256];
+  static_assert(kBlock == 256, "one thread per exponent");
+  local_hist[threadIdx.x] = 0;
+  __syncthreads();
   const int sub = threadIdx.x & 15;
   const int row = blockIdx.x * (kBlock / 16) + (threadIdx.x >> 4);
   float s = 0.0f;
@@ -143,8 +156,20 @@ __global__ __launch_bounds__(kBlock) void feat_rows_kernel(
   // rows the filter leaves out do not set the scale
   if (!(s < __builtin_inff()))
     big = 0;
+  // the row's own largest component (its 16 lanes)
 #pragma unroll
-  for (int sh = 32; sh >= 1; sh >>= 1) {
+  for (int sh = 8; sh >= 1; sh >>= 1) {
+    const unsigned o = (unsigned)__shfl_xor((int)big, sh);
+    big = o > big ? o : big;
+  }
+  if (row < n && sub == 0) {
+    if (big_out != nullptr)
+      big_out[row] = big;
+    if (hist != nullptr && big != 0)
+      atomicAdd(&local_hist[big >> 23], 1u);
+  }
+#pragma unroll
+  for (int sh = 32; sh >= 16; sh >>= 1) {
     const unsigned o = (unsigned)__shfl_xor((int)big, sh);
     big = o > big ? o : big;
   }
@@ -158,6 +183,51 @@ __global__ __launch_bounds__(kBlock) void feat_rows_kernel(
     if (big != 0 && big > __hip_atomic_load(&g->max_bits, __ATOMIC_RELAXED,
                                             __HIP_MEMORY_SCOPE_AGENT))
       atomicMax(&g->max_bits, big);
+  }
+  if (hist != nullptr && local_hist[threadIdx.x] != 0)
+    atomicAdd(&hist[threadIdx.x], local_hist[threadIdx.x]);
+}
+
+// The scale of the Euclidean filter: made for the largest component of all
+// rows, unless a few rows (up to kFeatMaxOutliers of x and as many of y, and
+// never more than one in 64) are at least four times larger than all others --
+// then for the others, which keep their bits in fp16; the few are handled
+// exactly (see FeatGlobals).  One workgroup of 256 threads.
+__global__ __launch_bounds__(256) void feat_scale_kernel(FeatGlobals *g, int n,
+                                                         int m) {
+  __shared__ unsigned hx[256], hy[256];
+  __shared__ int need_x, need_y, top;
+  const int t = threadIdx.x;
+  hx[t] = g->hist_x[t];
+  hy[t] = g->hist_y[t];
+  if (t == 0) {
+    need_x = 255;
+    need_y = 255;
+    top = 0;
+  }
+  __syncthreads();
+  unsigned above_x = 0, above_y = 0; // rows with a larger exponent than t
+  for (int b = t + 1; b < 256; ++b) {
+    above_x += hx[b];
+    above_y += hy[b];
+  }
+  const unsigned allow_x = (unsigned)min(kFeatMaxOutliers, n / 64);
+  const unsigned allow_y = (unsigned)min(kFeatMaxOutliers, m / 64);
+  // the smallest exponent that leaves at most that many rows above it (not
+  // below the smallest one in use: rows, not bins, are what is left out)
+  if (above_x <= allow_x && (hx[t] != 0 || above_x == 0))
+    atomicMin(&need_x, t);
+  if (above_y <= allow_y && (hy[t] != 0 || above_y == 0))
+    atomicMin(&need_y, t);
+  if (hx[t] != 0 || hy[t] != 0)
+    atomicMax(&top, t);
+  __syncthreads();
+  if (t == 0) {
+    const int need = max(need_x, need_y);
+    if (top - need >= 2) {
+      g->max_bits = ((unsigned)(need + 1) << 23) - 1u;
+      g->out_limit = g->max_bits;
+    }
   }
 }
 
@@ -492,6 +562,7 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   // squared norms that only classify the rows (NaN: a non-finite component);
   // for the Euclidean distance they also enter the filter
   float *x_class = cosine ? x_class_buf : x_norm;
+  unsigned *x_big = nullptr;
   const int rows_per_block = kBlock / 16;
   if (cosine) {
     // |x|, |y| as the reference's Cosine::norm computes them: they enter the
@@ -501,39 +572,46 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
     hipLaunchKernelGGL(feat_rows_kernel,
                        dim3((in.n + rows_per_block - 1) / rows_per_block),
                        dim3(kBlock), 0, stream, xf, in.n, in.d, x_class,
-                       globals);
+                       globals, static_cast<unsigned *>(nullptr),
+                       static_cast<unsigned *>(nullptr));
   } else {
+    // (the classification buffer is free here: it holds every row's largest
+    // component)
+    x_big = reinterpret_cast<unsigned *>(x_class_buf);
     hipLaunchKernelGGL(feat_rows_kernel,
                        dim3((in.n + rows_per_block - 1) / rows_per_block),
                        dim3(kBlock), 0, stream, xf, in.n, in.d, x_norm,
-                       globals);
+                       globals, x_big, globals->hist_x);
     hipLaunchKernelGGL(feat_rows_kernel,
                        dim3((in.m + rows_per_block - 1) / rows_per_block),
                        dim3(kBlock), 0, stream, yf, in.m, in.d,
-                       static_cast<float *>(nullptr), globals);
+                       static_cast<float *>(nullptr), globals,
+                       static_cast<unsigned *>(nullptr), globals->hist_y);
+    hipLaunchKernelGGL(feat_scale_kernel, dim3(1), dim3(256), 0, stream,
+                       globals, in.n, in.m);
   }
   {
     hipError_t perr;
     switch (nb) {
     case 3:
-      perr = launch_feat_pack<3>(xf, x_norm, x_class, in.n, in.d, cosine,
-                                 globals, x_pack, stream);
+      perr = launch_feat_pack<3>(xf, x_norm, x_class, x_big, in.n, in.d,
+                                 cosine, globals, x_pack, stream);
       break;
     case 5:
-      perr = launch_feat_pack<5>(xf, x_norm, x_class, in.n, in.d, cosine,
-                                 globals, x_pack, stream);
+      perr = launch_feat_pack<5>(xf, x_norm, x_class, x_big, in.n, in.d,
+                                 cosine, globals, x_pack, stream);
       break;
     case 9:
-      perr = launch_feat_pack<9>(xf, x_norm, x_class, in.n, in.d, cosine,
-                                 globals, x_pack, stream);
+      perr = launch_feat_pack<9>(xf, x_norm, x_class, x_big, in.n, in.d,
+                                 cosine, globals, x_pack, stream);
       break;
     case 17:
-      perr = launch_feat_pack<17>(xf, x_norm, x_class, in.n, in.d, cosine,
-                                  globals, x_pack, stream);
+      perr = launch_feat_pack<17>(xf, x_norm, x_class, x_big, in.n, in.d,
+                                  cosine, globals, x_pack, stream);
       break;
     default:
-      perr = launch_feat_pack<33>(xf, x_norm, x_class, in.n, in.d, cosine,
-                                  globals, x_pack, stream);
+      perr = launch_feat_pack<33>(xf, x_norm, x_class, x_big, in.n, in.d,
+                                  cosine, globals, x_pack, stream);
       break;
     }
     if (perr != hipSuccess)

@@ -94,7 +94,19 @@ struct FeatGlobals {
   // -DPCA_FEAT_STATS (steps, flagged steps, parked singles, lane-by-lane
   // values, drains, list rounds, direct steps, direct rounds)
   unsigned long long stats[8];
+  // Rows far larger than the rest do not set the scale.  hist_x / hist_y: rows
+  // per binary exponent of their largest finite |component|; out_limit: float
+  // bits of the largest |component| the scale was made for (rows of x beyond
+  // it, at most kFeatMaxOutliers, stay out of the filter and are evaluated
+  // exactly for every query: out_rows; queries beyond it take the second
+  // pass)
+  unsigned out_limit;
+  int n_out;
+  int out_rows[8];
+  unsigned hist_x[256];
+  unsigned hist_y[256];
 };
+constexpr int kFeatMaxOutliers = 8;
 
 // ---- constants of the error analysis (see the header) ----------------------
 // rho: 2^-9 up to 256 components, 2^-8 beyond (the accumulation error of the
@@ -203,14 +215,19 @@ __device__ __forceinline__ FeatQuery feat_query(const float *yrow, int d,
   }
   float chain = 0.0f; // classification as the old kernel does it
   double ysq = 0.0;
+  float top = 0.0f;
   for (int c = 0; c < d; ++c) {
     const float v = yrow[c];
     chain = __builtin_fmaf(v, v, chain);
-    const double s = (double)(v * inv_sigma);
+    const float scaled = v * inv_sigma;
+    top = __builtin_fmaxf(top, __builtin_fabsf(scaled));
+    const double s = (double)scaled;
     ysq += s * s;
   }
   fq.dead = chain != chain;
-  fq.odd = !fq.dead && !(chain < __builtin_inff());
+  // (a component beyond the range the scale was made for -- a query far
+  // larger than the other rows -- would overflow the fp16 operand)
+  fq.odd = !fq.dead && !(chain < __builtin_inff() && top < 2048.0f);
   // (the reference's squares lose up to 2^-149 each where they underflow)
   const double c0 =
       feat_c0(d) + (double)d * 1.4012984643248171e-45 * (double)inv_sigma *
@@ -282,8 +299,8 @@ constexpr int feat_resident_groups(int nb, int kp) {
 template <int NB, bool COSINE>
 __global__ __launch_bounds__(kBlock) void feat_pack_kernel(
     const float *__restrict__ x, const float *__restrict__ norms,
-    const float *__restrict__ cls, int n, int d, int spare, FeatGlobals *g,
-    uint4 *__restrict__ out) {
+    const float *__restrict__ cls, const unsigned *__restrict__ big, int n,
+    int d, int spare, FeatGlobals *g, uint4 *__restrict__ out) {
   typedef FeatShape<NB> S;
   const size_t id = (size_t)blockIdx.x * kBlock + threadIdx.x;
   if (id >= (size_t)(n + spare) * S::RSU)
@@ -308,6 +325,16 @@ __global__ __launch_bounds__(kBlock) void feat_pack_kernel(
     } else {
       usable = nv < __builtin_inff(); // (false for NaN too)
       scale = feat_inv_sigma(g->max_bits);
+      // a row far larger than the others: left out here (the scale was made
+      // without it), listed for the exact stage
+      if (usable && big != nullptr && big[row] > g->out_limit) {
+        usable = false;
+        if (unit == 0) {
+          const int slot = atomicAdd(&g->n_out, 1);
+          if (slot < kFeatMaxOutliers)
+            g->out_rows[slot] = row;
+        }
+      }
     }
     if (unit == 0 &&
         (cv == __builtin_inff() || (cv == cv && nv == __builtin_inff()) ||
@@ -961,6 +988,20 @@ __global__ __launch_bounds__(kBlock) void feat_merge_kernel(KnnFeatParams p) {
   }
 }
 
+// Segment of query q: the last b with ptr[b] <= q (segments may be empty).
+__device__ __forceinline__ int feat_segment_of(const int64_t *__restrict__ ptr,
+                                               int num_segments, int q) {
+  int lo = 0, hi = num_segments;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (ptr[mid] <= (int64_t)q)
+      lo = mid;
+    else
+      hi = mid;
+  }
+  return lo;
+}
+
 // One wave per query: exact distances of the listed rows that can matter,
 // sorted; flags the query when the list cannot be shown to hold its k nearest
 // rows.
@@ -1157,8 +1198,27 @@ __global__ __launch_bounds__(kBlock) void feat_refine_kernel(KnnFeatParams p) {
   const double last_lower = kk > kWave ? __shfl(lower[1], kk - 1 - kWave)
                                        : __shfl(lower[0], kk - 1);
   const bool full = listed_count == kk;
+  // rows of x that were left out of the filter (far larger than the rest):
+  // one lane each evaluates them; one that belongs among the k nearest sends
+  // the query to the scans that look at every row
+  bool outlier_in_reach = false;
+  if (!COSINE && p.globals->n_out > 0) {
+    const int n_out = min(p.globals->n_out, kFeatMaxOutliers);
+    const int seg = p.ptr_y ? feat_segment_of(p.ptr_y, p.num_segments, q) : 0;
+    const int xb = p.ptr_x ? (int)p.ptr_x[seg] : 0;
+    const int xe = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
+    bool mine = false;
+    if (lane < n_out) {
+      const int g = p.globals->out_rows[lane];
+      if (g >= xb && g < xe) {
+        const float e = exact(g);
+        mine = usable(e) && (good_count < k || !(e > kth_plain));
+      }
+    }
+    outlier_in_reach = __any(mine);
+  }
   // rows that were listed but not evaluated have lower > reach >= kth
-  const bool complete = !full || last_lower > kth;
+  const bool complete = (!full || last_lower > kth) && !outlier_in_reach;
   if (lane == 0) {
     p.out_count[q] = good_count < k ? good_count : k;
     p.redo_q[q] = 0;
@@ -1178,20 +1238,6 @@ __global__ __launch_bounds__(kBlock) void feat_refine_kernel(KnnFeatParams p) {
       }
     }
   }
-}
-
-// Segment of query q: the last b with ptr[b] <= q (segments may be empty).
-__device__ __forceinline__ int feat_segment_of(const int64_t *__restrict__ ptr,
-                                               int num_segments, int q) {
-  int lo = 0, hi = num_segments;
-  while (hi - lo > 1) {
-    const int mid = (lo + hi) >> 1;
-    if (ptr[mid] <= (int64_t)q)
-      lo = mid;
-    else
-      hi = mid;
-  }
-  return lo;
 }
 
 // Threshold scan of the queued queries.  A workgroup takes 32 of them (8 per
@@ -1380,8 +1426,9 @@ hipError_t launch_knn_feat_blocks(const KnnFeatParams &p, int kp, bool cosine,
                                   int grid, hipStream_t stream);
 template <int NB>
 hipError_t launch_feat_pack(const float *x, const float *norms,
-                            const float *cls, int n, int d, bool cosine,
-                            FeatGlobals *g, uint4 *out, hipStream_t stream);
+                            const float *cls, const unsigned *big, int n,
+                            int d, bool cosine, FeatGlobals *g, uint4 *out,
+                            hipStream_t stream);
 
 #define PCA_KNN_FEAT_DEFINE(NB_)                                               \
   template <int KP>                                                            \
@@ -1424,20 +1471,20 @@ hipError_t launch_feat_pack(const float *x, const float *norms,
   }                                                                            \
   template <>                                                                  \
   hipError_t launch_feat_pack<NB_>(const float *x, const float *norms,         \
-                                   const float *cls, int n, int d,             \
-                                   bool cosine, FeatGlobals *g, uint4 *out,    \
-                                   hipStream_t stream) {                       \
+                                   const float *cls, const unsigned *big,      \
+                                   int n, int d, bool cosine, FeatGlobals *g,  \
+                                   uint4 *out, hipStream_t stream) {           \
     const int spare = FeatShape<NB_>::TILE;                                    \
     const size_t units = (size_t)(n + spare) * FeatShape<NB_>::RSU;            \
     const unsigned grid = (unsigned)((units + kBlock - 1) / kBlock);           \
     if (cosine)                                                                \
       hipLaunchKernelGGL((feat_pack_kernel<NB_, true>), dim3(grid),            \
-                         dim3(kBlock), 0, stream, x, norms, cls, n, d, spare,  \
-                         g, out);                                              \
+                         dim3(kBlock), 0, stream, x, norms, cls, nullptr, n,   \
+                         d, spare, g, out);                                    \
     else                                                                       \
       hipLaunchKernelGGL((feat_pack_kernel<NB_, false>), dim3(grid),           \
-                         dim3(kBlock), 0, stream, x, norms, cls, n, d, spare,  \
-                         g, out);                                              \
+                         dim3(kBlock), 0, stream, x, norms, cls, big, n, d,    \
+                         spare, g, out);                                       \
     return hipGetLastError();                                                  \
   }
 

@@ -229,6 +229,52 @@ def test_scales_at_both_ends(oracle, case):
         _run(oracle, x, y, ptr_x, ptr_y, k, cosine=True)
 
 
+@pytest.mark.parametrize("case", ["one_row", "eight_rows", "nine_rows",
+                                  "queries_too", "only_four_times",
+                                  "neighbour_of_a_query", "small_segment"])
+def test_rows_far_larger_than_the_rest(oracle, case):
+    # up to 8 rows of x (and 8 of y) at least four times larger than all
+    # others do not set the fp16 scale: they stay out of the filter, every
+    # query evaluates them exactly, and the other rows keep their bits --
+    # same edges, and (almost) no query is handed to the second pass
+    rng = np.random.default_rng(_seed("outliers", case))
+    d, n, m, k = 72, 6000, 500, 16
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    y = rng.standard_normal((m, d)).astype(np.float32)
+    ptr_x = np.array([0, 2500, 6000])
+    ptr_y = np.array([0, 200, 500])
+    few_flagged = True
+    if case == "one_row":
+        x[17] *= 1e6
+    elif case == "eight_rows":
+        x[rng.choice(n, 8, replace=False)] *= 3e4
+    elif case == "nine_rows":
+        # one too many: the scale is made for them, as before
+        x[rng.choice(n, 9, replace=False)] *= 3e4
+        few_flagged = False
+    elif case == "queries_too":
+        x[4000] *= 1e5
+        y[[3, 250, 499]] *= 1e7
+    elif case == "only_four_times":
+        x[100] *= 40.0   # (largest components 4 x 40 / 4: three binades up)
+    elif case == "neighbour_of_a_query":
+        x[[10, 3000]] *= 1e5
+        y[0] = x[10]            # the large row is this query's nearest row
+        y[1] = x[10] * (1 + 1e-3)
+        y[300] = x[3000]
+    else:
+        # a segment of 40 rows: the large row is one of many in the call
+        ptr_x = np.array([0, 40, 6000])
+        x[5] *= 1e6
+    odd, flagged = _flagged_queries(x, y, k)
+    assert odd == 0
+    if few_flagged:
+        assert flagged <= 8, flagged
+    _run(oracle, x, y, ptr_x, ptr_y, k)
+    _run(oracle, x, y, ptr_x, ptr_y, k, cosine=True)
+    _run(oracle, x, y, None, None, 40)
+
+
 def test_many_slices_share_their_bounds(oracle, monkeypatch):
     rng = np.random.default_rng(9)
     x = rng.standard_normal((20000, 64)).astype(np.float32)
