@@ -396,6 +396,53 @@ class Cases:
                             "256 units busy" % clouds}}
         return report
 
+    # "auto" against the clock: whole calls of knn / radius / nearest on
+    # uniform clouds of growing size under both strategies, with what the
+    # cost model of "auto" picks for that size (`--case crossover`; not part
+    # of the default line).  `auto_is_faster_or_within` is the time auto's
+    # pick loses against the better strategy, as a fraction of that one.
+    def case_crossover(self, reps):
+        t, pca = self.torch, self.pca
+        pick = t.ops.pytorch_cluster_amd.strategy_for
+        report = {}
+        before = pca.get_search_strategy()
+        try:
+            for segments in (1, 8):
+                for n in (2048, 4096, 8192, 16384, 32768, 65536, 131072,
+                          262144):
+                    g = t.Generator().manual_seed(n + segments)
+                    x = t.rand(n * segments, 3, generator=g).to(self.dev)
+                    b = (t.arange(n * segments) // n).to(self.dev)
+                    xq, bq = x[::3].contiguous(), b[::3].contiguous()
+                    r = 0.6 * n ** (-1.0 / 3.0)
+                    calls = {
+                        "knn": lambda: pca.knn(x, x, 16, b, b,
+                                               batch_size=segments),
+                        "radius": lambda: pca.radius(
+                            x, x, r, b, b, max_num_neighbors=32,
+                            batch_size=segments),
+                        "nearest": lambda: pca.nearest(x, xq, b, bq)}
+                    for op, call in calls.items():
+                        ms = {}
+                        for strategy in ("scan", "binned"):
+                            pca.set_search_strategy(strategy)
+                            ms[strategy], _ = _median_ms(t, call, reps or 5)
+                        pca.set_search_strategy("auto")
+                        if op == "nearest":
+                            picked = pick(op, xq.shape[0], x.shape[0],
+                                          segments)
+                        else:
+                            picked = pick(op, x.shape[0], x.shape[0],
+                                          segments)
+                        best = min(ms.values())
+                        report["%s %d x %d" % (op, segments, n)] = {
+                            "scan_ms": ms["scan"], "binned_ms": ms["binned"],
+                            "auto_picks": picked,
+                            "auto_loses": ms[picked] / best - 1.0}
+        finally:
+            pca.set_search_strategy(before)
+        return report
+
     # the headline workload and large clouds through both search strategies
     # (binned: rows ordered along a space-filling curve, exact pruning by tile
     # boxes; same edges as the scan); `search_ms` covers binning and search
@@ -532,7 +579,8 @@ def main():
     ap.add_argument("--case", action="append", default=None,
                     help="with --extras-only: run only this configuration "
                          "(c1, c2, c3, c4, c4cos, d256, nearest_points, "
-                         "nearest_codes, fps, strategies; repeatable)")
+                         "nearest_codes, fps, strategies, crossover; "
+                         "repeatable)")
     ap.add_argument("--strategy", choices=("scan", "binned", "auto"),
                     default="scan",
                     help="search strategy of the timed steps: scan (default "

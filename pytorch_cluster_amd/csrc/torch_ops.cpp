@@ -370,26 +370,40 @@ std::string get_search_strategy() {
   return code == kBinned ? "binned" : code == kAuto ? "auto" : "scan";
 }
 
+// The estimates of "auto" per operator, fitted to whole calls on an MI355X
+// (`python bench.py --extras-only --case crossover` measures both strategies
+// over uniform clouds of 2,048 - 262,144 points in 1 and 8 examples and
+// reports where the pick loses).
+struct SearchCost {
+  double scan_rate;   // pairs per ms the scan looks at
+  double query_us;    // binned search: us per searching row
+  double binned_base; // binned search: ms before the first row counts
+};
+// kNN ~3 G pairs/ms (between its small-cloud and large-cloud rates); radius and
+// nearest ~10 G (the radius scan stops at max_num_neighbors, nearest keeps one
+// neighbour); a binned radius call starts sooner than a binned kNN call (no
+// tasks to order).
+constexpr SearchCost kKnnCost{3e9, 2e-3, 0.2};
+constexpr SearchCost kRadiusCost{1e10, 0.5e-3, 0.13};
+constexpr SearchCost kNearestCost{1e10, 0.5e-3, 0.2};
+
 // searched: rows that get binned (x of knn / radius, y of nearest);
 // searching: the rows that look for neighbours.  "auto" compares two rough
-// estimates fitted to measurements on an MI355X, in ms: the scan looks at
-// every pair of a segment (segments taken as equal) at scan_rate pairs per
-// ms - kNN ~3 G (between its small-cloud and large-cloud rates), radius and
-// nearest ~10 G (the radius scan stops at max_num_neighbors, nearest keeps
-// one neighbour) -, binning costs a sort of both sides and a search that
-// grows with their sizes (query_us per searching row).  It picks the scan for
-// clouds of a few thousand points and for a handful of queries against many
-// rows, bins from some ten thousand rows per segment on.
+// estimates in ms: the scan looks at every pair of a segment (segments taken
+// as equal) at scan_rate pairs per ms, binning costs a sort of both sides and
+// a search that grows with their sizes.  It picks the scan for clouds of a few
+// thousand points and for a handful of queries against many rows, bins from
+// some ten thousand rows per segment on.
 bool bins_wanted(int64_t searched, int64_t searching, int64_t num_segments,
-                 double scan_rate, double query_us) {
+                 const SearchCost &cost) {
   const int code = g_strategy.load();
   if (code != kAuto)
     return code == kBinned;
   const double pairs = (double)searched * (double)searching /
                        (double)std::max<int64_t>(num_segments, 1);
-  const double scan_ms = 0.1 + pairs / scan_rate;
-  const double binned_ms =
-      0.2 + 1e-6 * (double)searched + 1e-3 * query_us * (double)searching;
+  const double scan_ms = 0.1 + pairs / cost.scan_rate;
+  const double binned_ms = cost.binned_base + 1e-6 * (double)searched +
+                           1e-3 * cost.query_us * (double)searching;
   return scan_ms > binned_ms;
 }
 
@@ -404,14 +418,6 @@ bool being_captured(hipStream_t stream) {
   return status != hipStreamCaptureStatusNone;
 }
 
-// The two estimates of bins_wanted per operator: (scan_rate, query_us).
-struct SearchCost {
-  double scan_rate, query_us;
-};
-constexpr SearchCost kKnnCost{3e9, 2e-3};
-constexpr SearchCost kRadiusCost{1e10, 2e-3};
-constexpr SearchCost kNearestCost{1e10, 0.5e-3};
-
 // What the current strategy picks for an operator ("knn", "radius",
 // "nearest") and these sizes, when the points qualify for binning at all
 // (fp32, up to 3 dimensions, Euclidean): "scan" or "binned".
@@ -423,8 +429,7 @@ std::string strategy_for(std::string op, int64_t searched, int64_t searching,
                                              : nullptr;
   TORCH_CHECK(cost != nullptr, "operator is 'knn', 'radius' or 'nearest', got '",
               op, "'");
-  return bins_wanted(searched, searching, num_segments, cost->scan_rate,
-                     cost->query_us)
+  return bins_wanted(searched, searching, num_segments, *cost)
              ? "binned"
              : "scan";
 }
@@ -468,8 +473,7 @@ at::Tensor knn_search(at::Tensor x, at::Tensor y,
   refuse_capture(c10::hip::getCurrentHIPStream(x.get_device()).stream(),
                  "knn");
   const int dtype = dtype_code(x);
-  const bool binned = bins_wanted(n, m, seg.count, kKnnCost.scan_rate,
-                                  kKnnCost.query_us) &&
+  const bool binned = bins_wanted(n, m, seg.count, kKnnCost) &&
                       dtype == PCA_F32 && !cosine && d <= 3 && k <= 64;
   const size_t ws_bytes =
       binned ? pca_knn_binned_workspace_bytes(n, m, d, seg.count, k)
@@ -623,8 +627,7 @@ at::Tensor radius_search(at::Tensor x, at::Tensor y,
                  "radius");
   const int dtype = dtype_code(x);
   const int64_t slots = pca_radius_slots(n, max_num_neighbors);
-  const bool binned = bins_wanted(n, m, seg.count, kRadiusCost.scan_rate,
-                                  kRadiusCost.query_us) &&
+  const bool binned = bins_wanted(n, m, seg.count, kRadiusCost) &&
                       dtype == PCA_F32 && d <= 3 && slots <= 64;
   const size_t ws_bytes =
       binned ? pca_radius_binned_workspace_bytes(n, m, d, seg.count,
@@ -764,8 +767,7 @@ at::Tensor nearest(at::Tensor x, at::Tensor y, at::Tensor ptr_x,
               "nearest is not implemented for 'BFloat16'");
   // (the searched rows, y, are the ones a binned search orders)
   const bool binned =
-      bins_wanted(m, n, segments, kNearestCost.scan_rate,
-                  kNearestCost.query_us) &&
+      bins_wanted(m, n, segments, kNearestCost) &&
       dtype == PCA_F32 && d <= 3 && m > 0 &&
       !being_captured(
           c10::hip::getCurrentHIPStream(x.get_device()).stream());
