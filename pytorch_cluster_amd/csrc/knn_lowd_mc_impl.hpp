@@ -96,6 +96,9 @@ constexpr int kMcQueries = 128; // queries per workgroup
 #define PCA_MC_SEED_TILES 8
 #endif
 constexpr int kMcSeedTiles = PCA_MC_SEED_TILES;
+// launches of up to this many workgroups (three per CU of a 256-CU device)
+// take the kernel variants compiled without a register limit
+constexpr int kMcRoomyGrid = 768;
 constexpr int kMcQueueCap = 8; // parked steps per lane
 
 template <int DIM> struct McShape {
@@ -246,10 +249,13 @@ __global__ __launch_bounds__(kPlanThreads) void mc_setup_kernel(McSetup a) {
 // (launch bounds: 5-8 dimensions with lists of 16 came out at 136 registers,
 // up to 3 dimensions with lists of 24 at 138-140: three waves per SIMD; asked
 // for four - 128 registers, up to 12 spilled words - they run 5 % and 10 %
-// faster on clouds that fill the device, 2 % slower on 16 x 4,096 points)
-template <int DIM, int K, bool NEAREST = false>
+// faster on clouds that fill the device, 2 % slower on 16 x 4,096 points;
+// ROOMY: the same kernel without that limit, for launches of at most three
+// workgroups per CU, which gain nothing from a fourth and lose to the spills)
+template <int DIM, int K, bool NEAREST = false, bool ROOMY = false>
 __global__ __launch_bounds__(
-    kBlock, ((DIM == 8 && K == 16) || (DIM <= 3 && K == 24)) ? 4 : 1) void
+    kBlock,
+    (!ROOMY && ((DIM == 8 && K == 16) || (DIM <= 3 && K == 24))) ? 4 : 1) void
 knn_lowd_mc_kernel(KnnLowdParams p) {
   static_assert(!NEAREST || K == 1, "nearest keeps one neighbour");
   constexpr float kLimit = SearchLimit<NEAREST>::value;
@@ -794,8 +800,12 @@ hipError_t launch_mc_setup(const McSetup &a, hipStream_t stream);
                          dim3(kBlock), 0, stream, p);                          \
       break;                                                                   \
     case 24:                                                                   \
-      hipLaunchKernelGGL((knn_lowd_mc_kernel<DIM_, 24>), dim3(grid),           \
-                         dim3(kBlock), 0, stream, p);                          \
+      if (DIM_ <= 3 && grid <= kMcRoomyGrid)                                   \
+        hipLaunchKernelGGL((knn_lowd_mc_kernel<DIM_, 24, false, true>),        \
+                           dim3(grid), dim3(kBlock), 0, stream, p);            \
+      else                                                                     \
+        hipLaunchKernelGGL((knn_lowd_mc_kernel<DIM_, 24>), dim3(grid),         \
+                           dim3(kBlock), 0, stream, p);                        \
       break;                                                                   \
     case 32:                                                                   \
       hipLaunchKernelGGL((knn_lowd_mc_kernel<DIM_, 32>), dim3(grid),           \
