@@ -85,9 +85,9 @@ __global__ __launch_bounds__(kBlock) void feat_init_kernel(
   }
   if (i < redo_cap)
     hit_count[i] = 0;
-  if (i < 256) {
-    g->hist_x[i] = 0;
-    g->hist_y[i] = 0;
+  for (int j = i; j < kFeatHistCopies * 256; j += gridDim.x * kBlock) {
+    g->hist_x[j] = 0;
+    g->hist_y[j] = 0;
   }
   if (i == 0) {
     g->max_bits = 0;
@@ -185,7 +185,8 @@ __global__ __launch_bounds__(kBlock) void feat_rows_kernel(
       atomicMax(&g->max_bits, big);
   }
   if (hist != nullptr && local_hist[threadIdx.x] != 0)
-    atomicAdd(&hist[threadIdx.x], local_hist[threadIdx.x]);
+    atomicAdd(&hist[(blockIdx.x % kFeatHistCopies) * 256 + threadIdx.x],
+              local_hist[threadIdx.x]);
 }
 
 // The scale of the Euclidean filter: made for the largest component of all
@@ -198,19 +199,52 @@ __global__ __launch_bounds__(256) void feat_scale_kernel(FeatGlobals *g, int n,
   __shared__ unsigned hx[256], hy[256];
   __shared__ int need_x, need_y, top;
   const int t = threadIdx.x;
-  hx[t] = g->hist_x[t];
-  hy[t] = g->hist_y[t];
+  unsigned sum_x = 0, sum_y = 0;
+  for (int c = 0; c < kFeatHistCopies; ++c) {
+    sum_x += g->hist_x[c * 256 + t];
+    sum_y += g->hist_y[c * 256 + t];
+  }
+  hx[t] = sum_x;
+  hy[t] = sum_y;
   if (t == 0) {
     need_x = 255;
     need_y = 255;
     top = 0;
   }
   __syncthreads();
-  unsigned above_x = 0, above_y = 0; // rows with a larger exponent than t
-  for (int b = t + 1; b < 256; ++b) {
-    above_x += hx[b];
-    above_y += hy[b];
+  // rows with a larger exponent than t: one wave, four bins per lane, a
+  // suffix sum over the lanes
+  __shared__ unsigned ax[256], ay[256];
+  if (t < kWave) {
+    unsigned vx[4], vy[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      vx[i] = hx[4 * t + i];
+      vy[i] = hy[4 * t + i];
+    }
+    const unsigned own_x = vx[0] + vx[1] + vx[2] + vx[3];
+    const unsigned own_y = vy[0] + vy[1] + vy[2] + vy[3];
+    unsigned sx = own_x, sy = own_y; // this lane's bins and all behind them
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1) {
+      const unsigned ox = __shfl_down(sx, sh);
+      const unsigned oy = __shfl_down(sy, sh);
+      if (t + sh < kWave) {
+        sx += ox;
+        sy += oy;
+      }
+    }
+    unsigned behind_x = sx - own_x, behind_y = sy - own_y;
+#pragma unroll
+    for (int i = 3; i >= 0; --i) {
+      ax[4 * t + i] = behind_x;
+      ay[4 * t + i] = behind_y;
+      behind_x += vx[i];
+      behind_y += vy[i];
+    }
   }
+  __syncthreads();
+  const unsigned above_x = ax[t], above_y = ay[t];
   const unsigned allow_x = (unsigned)min(kFeatMaxOutliers, n / 64);
   const unsigned allow_y = (unsigned)min(kFeatMaxOutliers, m / 64);
   // the smallest exponent that leaves at most that many rows above it (not

@@ -95,7 +95,9 @@ struct FeatGlobals {
   // values, drains, list rounds, direct steps, direct rounds)
   unsigned long long stats[8];
   // Rows far larger than the rest do not set the scale.  hist_x / hist_y: rows
-  // per binary exponent of their largest finite |component|; out_limit: float
+  // per binary exponent of their largest finite |component| (kFeatHistCopies
+  // copies that the workgroups spread their counts over: thousands of adds to
+  // one word take turns in the L2, 10 ns each); out_limit: float
   // bits of the largest |component| the scale was made for (rows of x beyond
   // it, at most kFeatMaxOutliers, stay out of the filter and are evaluated
   // exactly for every query: out_rows; queries beyond it take the second
@@ -103,10 +105,11 @@ struct FeatGlobals {
   unsigned out_limit;
   int n_out;
   int out_rows[8];
-  unsigned hist_x[256];
-  unsigned hist_y[256];
+  unsigned hist_x[32 * 256];
+  unsigned hist_y[32 * 256];
 };
 constexpr int kFeatMaxOutliers = 8;
+constexpr int kFeatHistCopies = 32;
 
 // ---- constants of the error analysis (see the header) ----------------------
 // rho: 2^-9 up to 256 components, 2^-8 beyond (the accumulation error of the
