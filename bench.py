@@ -189,8 +189,8 @@ class Cases:
         self.events = HipEvents(torch)
 
     def names(self):
-        return ["c1", "c2", "c3", "c4", "c4cos", "d256", "nearest_points",
-                "nearest_codes", "fps", "strategies"]
+        return ["c1", "c2", "c3", "c4", "c4cos", "d256", "clouds64",
+                "nearest_points", "nearest_codes", "fps", "strategies"]
 
     def run(self, name, reps=None):
         return getattr(self, "case_" + name)(reps)
@@ -315,6 +315,30 @@ class Cases:
             "knn 50000x256 onto themselves k=64", 50000, 50000, 256, 64,
             False, reps))
         return report
+
+    # the shape of a dynamic-graph layer of a point-cloud network: many small
+    # clouds searched in themselves in feature space (one kernel that needs
+    # no second stage: examples of up to 8,192 rows, d <= 128, k <= 32)
+    def case_clouds64(self, reps):
+        t, pca = self.torch, self.pca
+        clouds, points, d, k = 32, 1024, 64, 20
+        x = self.testing.feature_space(0, clouds * points, 1, d)["x"].to(
+            self.dev)
+        b = t.arange(clouds, device=self.dev).repeat_interleave(points)
+        fn = lambda: pca.knn_graph(x, k, b, batch_size=clouds)  # noqa: E731
+        ms, out = _median_ms(t, fn, reps or 10)
+        kms = _search_ms(t, self.capi, self.events, fn)
+        blocks = _feat_shape(d, k)[0]
+        return {"knn_graph 32x1024 points x 64 features k=20": {
+            "ms": ms, "queries_per_s": x.shape[0] / ms * 1e3,
+            "edges": int(out.shape[1]),
+            "roofline": _roofline(
+                "knn_feat_small_kernel<%d,24>" % blocks, kms,
+                2 * d * clouds * points * points, PEAK_BF16_TFLOPS, "mfma",
+                "algorithmic 2*D flop per pair against the dense fp16 matrix "
+                "peak; one workgroup per 128 queries goes over its cloud "
+                "twice with one wave per SIMD: a latency case, 4 GFLOP per "
+                "call")}}
 
     # nearest: every point of the LiDAR-like scans looks for the nearest of
     # its scan's every-8th point (the operator that follows the neighbour
@@ -578,8 +602,9 @@ def main():
                          "paths)")
     ap.add_argument("--case", action="append", default=None,
                     help="with --extras-only: run only this configuration "
-                         "(c1, c2, c3, c4, c4cos, d256, nearest_points, "
-                         "nearest_codes, fps, strategies, crossover; "
+                         "(c1, c2, c3, c4, c4cos, d256, clouds64, "
+                         "nearest_points, nearest_codes, fps, strategies, "
+                         "crossover; "
                          "repeatable)")
     ap.add_argument("--strategy", choices=("scan", "binned", "auto"),
                     default="scan",

@@ -1,6 +1,7 @@
 // Dispatch of the feature-space kNN with the fp16 matrix-core filter (see
 // knn_feat_impl.hpp): preparation, the filter kernel, the exact second kernel
 // and the second pass for the queries that one flags.
+#include "knn_feat_small_impl.hpp"
 #include "knn_feat_wide_impl.hpp"
 
 #include <algorithm>
@@ -32,9 +33,39 @@ PCA_DECLARE_FEAT_WIDE_BLOCKS(5)
 PCA_DECLARE_FEAT_WIDE_BLOCKS(9)
 #undef PCA_DECLARE_FEAT_WIDE_BLOCKS
 
+#define PCA_DECLARE_FEAT_SMALL_BLOCKS(NB)                                      \
+  template <>                                                                  \
+  hipError_t launch_knn_feat_small_blocks<NB>(const KnnFeatParams &, int, int, \
+                                              hipStream_t);
+PCA_DECLARE_FEAT_SMALL_BLOCKS(3)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(5)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(9)
+#undef PCA_DECLARE_FEAT_SMALL_BLOCKS
+
 namespace {
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// The one-kernel search (knn_feat_small_impl.hpp): Euclidean, up to 128
+// components, k <= 32, and examples of at most 8,192 rows on average.  Measured
+// on clouds searched in themselves, k = 20, against the better of the two
+// staged searches: 32 x 1,024 x 64 0.25 / 0.51 ms, 16 x 2,048 x 128
+// 0.47 / 0.77, 4 x 8,192 x 64 0.54 / 0.81, 2 x 16,384 x 64 0.80 / 0.93,
+// 4 x 16,384 x 128 2.33 / 1.67, 1 x 32,768 x 64 1.25 / 1.14, 1 x 65,536 x 64
+// 3.9 / 2.3: a workgroup of this kernel goes over its whole example, twice,
+// with one wave per SIMD, and longer scans are worth the staged searches'
+// sharing of an example among workgroups.  PCA_KNN_FEAT_SMALL: 0 never, 1
+// whenever the shape fits.
+bool feat_small_applies(int n, int d, int num_segments, int k, bool cosine) {
+  const bool fits = !cosine && d <= 128 && k <= 32;
+  if (const char *env = std::getenv("PCA_KNN_FEAT_SMALL")) {
+    if (env[0] == '0')
+      return false;
+    if (env[0] == '1')
+      return fits;
+  }
+  return fits && (long long)n <= 8192LL * num_segments;
+}
 
 // list width for k neighbours: k + 16 real entries
 int feat_width(int k) {
@@ -694,7 +725,29 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
 
   const int kp = feat_width(k);
   hipError_t err;
-  if (lay.wide_buf != 0) {
+  const bool small =
+      feat_small_applies(in.n, in.d, in.num_segments, k, cosine);
+  if (small) {
+    // one exact kernel: nothing is listed, merged or refined
+    const int kbucket = k <= 8 ? 8 : (k <= 16 ? 16 : (k <= 24 ? 24 : 32));
+    if (time_start)
+      (void)hipEventRecord(time_start, stream);
+    switch (nb) {
+    case 3:
+      err = launch_knn_feat_small_blocks<3>(p, kbucket, tiles_bound, stream);
+      break;
+    case 5:
+      err = launch_knn_feat_small_blocks<5>(p, kbucket, tiles_bound, stream);
+      break;
+    default:
+      err = launch_knn_feat_small_blocks<9>(p, kbucket, tiles_bound, stream);
+      break;
+    }
+    if (time_stop)
+      (void)hipEventRecord(time_stop, stream);
+    if (err != hipSuccess)
+      return err;
+  } else if (lay.wide_buf != 0) {
     // eight-wave first stage: plan, filter, gather
     const FeatWidePlan wp = feat_wide_plan(in.n, in.m, in.num_segments, k);
     char *wb = reinterpret_cast<char *>(partial);
@@ -817,7 +870,7 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
     break;
   }
   }
-  {
+  if (!small) {
     const int waves = kBlock / kWave;
     const int rgrid = (in.m + waves - 1) / waves;
     if (cosine)
@@ -835,7 +888,7 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   // while nothing is flagged (no host read in between).  First the scan that
   // collects the rows at or below a query's k-th listed distance, then --
   // only for what that scan could not take -- the full second pass.
-  {
+  if (!small) { // (the one-kernel search queues nothing for the scan)
     const int waves = kBlock / kWave;
     const int sgrid =
         (redo_cap + kFeatRedoGroup - 1) / kFeatRedoGroup * kFeatRedoSlices;

@@ -1,11 +1,13 @@
-"""Feature-space kNN with the fp16 matrix-core filter (knn_feat_impl.hpp and,
-for up to 128 components, the eight-wave first stage of
-knn_feat_wide_impl.hpp; every test runs with either):
-parity with the CPU checker where the mechanisms of that path are exercised --
-lists that overflow (near-duplicates: the flagged queries go through the
-second pass), rows and queries the filter cannot represent, 129-512
-components, every list width (k up to 100), scales at both ends of fp32.  Bit-exact edges
-and distances, as everywhere.
+"""Feature-space kNN with the fp16 matrix-core filter.  Every test runs with
+each of the three searches behind it: the four-wave first stage
+(knn_feat_impl.hpp), the eight-wave first stage (knn_feat_wide_impl.hpp, up to
+128 components), and the one-kernel search for examples of moderate size
+(knn_feat_small_impl.hpp: Euclidean, up to 128 components, k <= 32; other
+calls fall through to the stages).  Parity with the CPU checker where the
+mechanisms of that path are exercised -- lists that overflow (near-duplicates:
+the flagged queries go through the second pass), rows and queries the filter
+cannot represent, 129-512 components, every list width (k up to 100), scales
+at both ends of fp32.  Bit-exact edges and distances, as everywhere.
 """
 import numpy as np
 import pytest
@@ -16,20 +18,34 @@ import zlib
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["four_waves", "eight_waves"])
+@pytest.fixture(autouse=True,
+                params=["four_waves", "eight_waves", "one_kernel"])
 def first_stage(request, monkeypatch):
-    """Which first stage serves the calls of a test: the four-wave kernel
-    with its register lists, or (where the shape fits: up to 128 components)
-    the eight-wave kernel with candidate buffers.  Left to itself the library
-    takes the second one from 4,096 queries on."""
-    monkeypatch.setenv("PCA_KNN_FEAT_WIDE",
-                       "1" if request.param == "eight_waves" else "0")
+    """Which search serves the calls of a test: the four-wave kernel with its
+    register lists, (where the shape fits: up to 128 components) the
+    eight-wave kernel with candidate buffers, or (Euclidean, up to 128
+    components, k <= 32) the one kernel that needs no second stage.  Left to
+    itself the library takes the last one for examples of up to 8,192 rows on
+    average, else the eight-wave stage from 4,096 queries on."""
+    if request.param == "one_kernel":
+        monkeypatch.setenv("PCA_KNN_FEAT_SMALL", "1")
+        monkeypatch.delenv("PCA_KNN_FEAT_WIDE", raising=False)
+    else:
+        monkeypatch.setenv("PCA_KNN_FEAT_SMALL", "0")
+        monkeypatch.setenv("PCA_KNN_FEAT_WIDE",
+                           "1" if request.param == "eight_waves" else "0")
     return request.param
 
 
 def _only_once_beyond_128(first_stage, d):
-    if d > 128 and first_stage == "eight_waves":
+    if d > 128 and first_stage != "four_waves":
         pytest.skip("more than 128 components: the four-wave kernel either way")
+
+
+def _one_kernel(first_stage, d, k, cosine=False):
+    """Whether the one-kernel search serves such a call: it keeps no
+    candidate lists, so nothing is ever handed to a second pass."""
+    return first_stage == "one_kernel" and not cosine and d <= 128 and k <= 32
 
 
 def _seed(*parts):
@@ -93,7 +109,10 @@ def test_near_duplicates_go_through_the_second_pass(oracle, first_stage, d,
     y = np.concatenate([centres[:25],
                         rng.standard_normal((40, d)).astype(np.float32)])
     odd, flagged = _flagged_queries(x, y, 8, cosine)
-    assert odd == 0 and flagged >= 25
+    if _one_kernel(first_stage, d, 8, cosine):
+        assert odd == 0 and flagged == 0
+    else:
+        assert odd == 0 and flagged >= 25
     _run(oracle, x, y, None, None, 8, cosine)
     # exact duplicates: ties settled by row number
     x2 = np.repeat(centres, 30, axis=0)
@@ -145,7 +164,9 @@ def test_flagged_queries_beyond_what_the_threshold_scan_holds(oracle,
                         rng.standard_normal((500, d)).astype(np.float32)])
     x = x[rng.permutation(len(x))]
     y = np.concatenate([centres, rng.standard_normal((30, d)).astype(np.float32)])
-    assert _unresolved_queries(x, y, 8) >= 1
+    lists = not _one_kernel(first_stage, d, 8)
+    if lists:
+        assert _unresolved_queries(x, y, 8) >= 1
     _run(oracle, x, y, None, None, 8)
     _run(oracle, x, y, None, None, 8, cosine=True)
     # (b) more flagged queries than the scan's queue takes (8,192 here)
@@ -155,7 +176,10 @@ def test_flagged_queries_beyond_what_the_threshold_scan_holds(oracle,
     x = x.astype(np.float32)
     y = np.repeat(centres, 300, axis=0)
     odd, flagged = _flagged_queries(x, y, 6)
-    assert flagged > 8192 and _unresolved_queries(x, y, 6) == flagged - 8192
+    if lists:
+        assert flagged > 8192 and _unresolved_queries(x, y, 6) == flagged - 8192
+    else:
+        assert flagged == 0
     ptr_x = np.array([0, 600, 1200])
     ptr_y = np.array([0, 4200, 9000])
     _run(oracle, x, y, ptr_x, ptr_y, 6)
@@ -275,6 +299,48 @@ def test_rows_far_larger_than_the_rest(oracle, case):
     _run(oracle, x, y, None, None, 40)
 
 
+@pytest.mark.parametrize("d", [9, 12, 17, 32, 63, 64, 65, 100, 127, 128])
+def test_one_kernel_search_shapes(oracle, first_stage, d):
+    if first_stage != "one_kernel":
+        pytest.skip("the one-kernel search only")
+    # examples of 0, 1, 31, 32, 33 rows, of more rows than the bound samples
+    # (64 steps of 32), of exactly a number of steps, with no queries, with
+    # fewer rows than k; queries that do not fill a workgroup; every list
+    # width; components that are and are not a multiple of four
+    rng = np.random.default_rng(_seed("one_kernel", d))
+    sizes_x = [0, 1, 31, 32, 33, 2500, 512, 40, 1024, 7]
+    sizes_y = [3, 5, 130, 0, 129, 300, 128, 1, 257, 20]
+    ptr_x = np.concatenate([[0], np.cumsum(sizes_x)])
+    ptr_y = np.concatenate([[0], np.cumsum(sizes_y)])
+    x = rng.standard_normal((ptr_x[-1], d)).astype(np.float32)
+    y = rng.standard_normal((ptr_y[-1], d)).astype(np.float32)
+    y[:200] = x[rng.integers(0, len(x), 200)]      # distance zero, ties
+    x[3000:3040] = x[2990]                         # equal rows: row numbers
+    for k in (1, 7, 8, 9, 16, 20, 24, 25, 32):
+        _run(oracle, x, y, ptr_x, ptr_y, k)
+    # rows far larger than the rest, one in an example too short for a bound
+    # (every row of it is evaluated; the large one must not be listed twice)
+    x[[1000, 3120]] *= 1e5
+    for k in (5, 20, 32):
+        _run(oracle, x, y, ptr_x, ptr_y, k)
+
+
+def test_one_kernel_search_is_the_default_for_small_examples(oracle,
+                                                             first_stage,
+                                                             monkeypatch):
+    if first_stage != "one_kernel":
+        pytest.skip("once is enough")
+    monkeypatch.delenv("PCA_KNN_FEAT_SMALL", raising=False)
+    # 24 examples of 700 rows searched in themselves, as a dynamic graph
+    # layer does; no query is handed on, the per-call block says so
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((24 * 700, 64)).astype(np.float32)
+    ptr = np.arange(25) * 700
+    _run(oracle, x, x, ptr, ptr, 21)
+    odd, flagged = _flagged_queries(x, x, 21)
+    assert odd == 0 and flagged == 0
+
+
 def test_many_slices_share_their_bounds(oracle, monkeypatch):
     rng = np.random.default_rng(9)
     x = rng.standard_normal((20000, 64)).astype(np.float32)
@@ -291,6 +357,7 @@ def test_pieces_of_the_eight_wave_stage(oracle, monkeypatch):
     # walks through every tile, pieces of a few rows, several pieces per tile,
     # and the buffers at their smallest (a checkpoint tidies them more often)
     monkeypatch.setenv("PCA_KNN_FEAT_WIDE", "1")
+    monkeypatch.setenv("PCA_KNN_FEAT_SMALL", "0")
     rng = np.random.default_rng(21)
     x = rng.standard_normal((9000, 48)).astype(np.float32)
     y = rng.standard_normal((1500, 48)).astype(np.float32)
@@ -318,6 +385,7 @@ def test_queries_enough_for_the_eight_wave_stage_by_default(oracle,
                                                             monkeypatch):
     # from 4,096 queries on the library takes the eight-wave stage by itself
     monkeypatch.delenv("PCA_KNN_FEAT_WIDE", raising=False)
+    monkeypatch.setenv("PCA_KNN_FEAT_SMALL", "0")
     rng = np.random.default_rng(22)
     x = rng.standard_normal((12000, 96)).astype(np.float32)
     y = rng.standard_normal((5000, 96)).astype(np.float32)
