@@ -107,14 +107,7 @@ template <bool BF16> struct R16Traits {
   typedef uint16_t store_t;
   typedef float calc_t;
   static __device__ __forceinline__ float round16(float v) {
-    if (BF16) {
-      uint32_t x = __float_as_uint(v);
-      if ((x & 0x7fffffffu) > 0x7f800000u)
-        return __uint_as_float(0x7fc00000u);
-      x += 0x7fffu + ((x >> 16) & 1u);
-      return __uint_as_float(x & 0xffff0000u);
-    }
-    return __half2float(__float2half_rn(v));
+    return round_to_16<BF16>(v);
   }
   static __device__ __forceinline__ calc_t load(store_t v) {
     if (BF16)

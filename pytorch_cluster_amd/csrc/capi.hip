@@ -132,6 +132,15 @@ KnnLayout knn_layout(int64_t n, int64_t m, int64_t d, int64_t num_segments,
     w.x_norm = align256(pca::anytype_norm_bytes((int)n));
     w.sliced = pca::knn_anytype_scratch_bytes((int)n, (int)m,
                                               (int)num_segments, (int)k);
+    // (16-bit rows through the matrix-core filter: the Euclidean metric only,
+    // but one size query serves both)
+    if ((dtype == PCA_F16 || dtype == PCA_BF16) &&
+        pca::knn_feat16_supported((int)n, (int)d, (int)num_segments, (int)k,
+                                  false, dtype == PCA_BF16))
+      w.sliced = std::max(w.sliced,
+                          pca::knn_feat16_scratch_bytes((int)n, (int)m, (int)d,
+                                                        (int)num_segments,
+                                                        (int)k));
   } else if (d > 8) {
     w.x_norm = align256(sizeof(float) * (size_t)n);
     if (pca::knn_feat_supported((int)d, (int)k, false))
@@ -518,7 +527,11 @@ int knn_call(const void *x, const void *y, const int64_t *ptr_x,
       f32 && !low_d && pca::knn_feat_supported((int)d, (int)k, cosine != 0);
   const bool mfma = f32 && !low_d && !feat &&
                     pca::knn_mfma_supported((int)d, (int)k, cosine != 0);
-  if (mfma || feat)
+  const int r16 = dtype == PCA_F16 ? 1 : (dtype == PCA_BF16 ? 2 : 0);
+  const bool feat16 =
+      r16 != 0 && pca::knn_feat16_supported((int)n, (int)d, (int)num_segments,
+                                            (int)k, cosine != 0, r16 == 2);
+  if (mfma || feat || feat16)
     cfg.tile_queries = pca::kMfmaTileQueries;
   else if (!low_d)
     cfg.tile_queries = pca::kBlock; // any-dimension kernel: one query per lane
@@ -547,6 +560,12 @@ int knn_call(const void *x, const void *y, const int64_t *ptr_x,
                                            lowd_scratch, dense, timer.start,
                                            timer.stop, stream),
                       "knn_feat_kernel");
+    timer.stop = nullptr;
+  } else if (feat16) {
+    rc = check_launch(pca::launch_knn_feat(in, (int)k, false, work_start,
+                                           lowd_scratch, dense, timer.start,
+                                           timer.stop, stream, r16),
+                      "knn_feat_small_kernel");
     timer.stop = nullptr;
   } else if (mfma) {
     rc = check_launch(pca::launch_knn_mfma(in, (int)k, cosine != 0, work_start,

@@ -9,6 +9,20 @@ namespace pca {
 constexpr int kWave = 64;
 constexpr int kBlock = 256; // 4 waves: one per SIMD of a CU
 
+// v rounded to the nearest fp16 (BF16: bfloat16) number, ties to even, as a
+// float: what c10::Half / c10::BFloat16 arithmetic does after every operation
+// (torch/headeronly/util/Half.h:501-560, BFloat16.h).
+template <bool BF16> __device__ __forceinline__ float round_to_16(float v) {
+  if (BF16) {
+    uint32_t x = __float_as_uint(v);
+    if ((x & 0x7fffffffu) > 0x7f800000u)
+      return __uint_as_float(0x7fc00000u);
+    x += 0x7fffu + ((x >> 16) & 1u);
+    return __uint_as_float(x & 0xffff0000u);
+  }
+  return (float)(_Float16)v;
+}
+
 // Distance every kNN slot starts from; a candidate must be strictly below it
 // to be returned (csrc/cuda/knn_cuda.cu:48,68 in the reference).
 constexpr float kKnnSentinel = 1e10f;

@@ -33,13 +33,19 @@ PCA_DECLARE_FEAT_WIDE_BLOCKS(5)
 PCA_DECLARE_FEAT_WIDE_BLOCKS(9)
 #undef PCA_DECLARE_FEAT_WIDE_BLOCKS
 
-#define PCA_DECLARE_FEAT_SMALL_BLOCKS(NB)                                      \
+#define PCA_DECLARE_FEAT_SMALL_BLOCKS(NB, R16)                                 \
   template <>                                                                  \
-  hipError_t launch_knn_feat_small_blocks<NB>(const KnnFeatParams &, int, int, \
-                                              hipStream_t);
-PCA_DECLARE_FEAT_SMALL_BLOCKS(3)
-PCA_DECLARE_FEAT_SMALL_BLOCKS(5)
-PCA_DECLARE_FEAT_SMALL_BLOCKS(9)
+  hipError_t launch_knn_feat_small_blocks<NB, R16>(const KnnFeatParams &, int, \
+                                                   int, hipStream_t);
+PCA_DECLARE_FEAT_SMALL_BLOCKS(3, 0)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(5, 0)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(9, 0)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(3, 1)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(5, 1)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(9, 1)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(3, 2)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(5, 2)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(9, 2)
 #undef PCA_DECLARE_FEAT_SMALL_BLOCKS
 
 namespace {
@@ -584,10 +590,73 @@ size_t knn_feat_scratch_bytes(int n, int m, int d, int num_segments, int k) {
   return feat_layout(n, m, d, num_segments, k).total();
 }
 
-hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
+namespace {
+
+// fp16 / bf16 rows as fp32 (exact)
+template <bool BF16>
+__global__ __launch_bounds__(kBlock) void widen16_kernel(
+    const uint16_t *__restrict__ src, size_t count, float *__restrict__ dst) {
+  const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= count)
+    return;
+  const uint16_t v = src[i];
+  dst[i] = BF16 ? __uint_as_float((uint32_t)v << 16)
+                : (float)__builtin_bit_cast(_Float16, v);
+}
+
+void launch_widen16(const void *src, size_t count, bool bf16, float *dst,
+                    hipStream_t stream) {
+  const unsigned grid = (unsigned)((count + kBlock - 1) / kBlock);
+  if (bf16)
+    hipLaunchKernelGGL(widen16_kernel<true>, dim3(grid), dim3(kBlock), 0,
+                       stream, static_cast<const uint16_t *>(src), count, dst);
+  else
+    hipLaunchKernelGGL(widen16_kernel<false>, dim3(grid), dim3(kBlock), 0,
+                       stream, static_cast<const uint16_t *>(src), count, dst);
+}
+
+} // namespace
+
+bool knn_feat16_supported(int n, int d, int num_segments, int k, bool cosine,
+                          bool bf16) {
+  if (const char *env = std::getenv("PCA_KNN_FEAT_16BIT"))
+    if (env[0] == '0')
+      return false;
+  // (what 16-bit sums can lose grows with their length: at 128 components of
+  // bf16 the cut would pass rows at twice the bound)
+  return !cosine && d > 8 && d <= (bf16 ? 64 : 128) && k <= 32 && n >= 1 &&
+         num_segments >= 1;
+}
+
+size_t knn_feat16_scratch_bytes(int n, int m, int d, int num_segments,
+                                int k) {
+  return align256(sizeof(float) * (size_t)n * d) +
+         align256(sizeof(float) * (size_t)m * d) +
+         knn_feat_scratch_bytes(n, m, d, num_segments, k);
+}
+
+hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
                            const int *work_start, void *scratch,
                            const DenseResult &out, hipEvent_t time_start,
-                           hipEvent_t time_stop, hipStream_t stream) {
+                           hipEvent_t time_stop, hipStream_t stream,
+                           int r16) {
+  SearchInput in = in_given;
+  if (r16 != 0) {
+    // 16-bit rows: searched as fp32 rows (the widening is exact) by the one
+    // kernel that can compute the exact distances in the 16-bit arithmetic
+    if (cosine || in.d > 128 || k > 32)
+      return hipErrorInvalidValue;
+    char *at = static_cast<char *>(scratch);
+    float *x32 = reinterpret_cast<float *>(at);
+    at += align256(sizeof(float) * (size_t)in.n * in.d);
+    float *y32 = reinterpret_cast<float *>(at);
+    at += align256(sizeof(float) * (size_t)in.m * in.d);
+    scratch = at;
+    launch_widen16(in.x, (size_t)in.n * in.d, r16 == 2, x32, stream);
+    launch_widen16(in.y, (size_t)in.m * in.d, r16 == 2, y32, stream);
+    in.x = x32;
+    in.y = y32;
+  }
   const FeatLayout lay =
       feat_layout(in.n, in.m, in.d, in.num_segments, k);
   const int tiles_bound =
@@ -726,27 +795,34 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   const int kp = feat_width(k);
   hipError_t err;
   const bool small =
-      feat_small_applies(in.n, in.d, in.num_segments, k, cosine);
+      r16 != 0 || feat_small_applies(in.n, in.d, in.num_segments, k, cosine);
   if (small) {
-    // one exact kernel: nothing is listed, merged or refined
+    // one exact kernel: nothing is listed, merged, refined or searched again
     const int kbucket = k <= 8 ? 8 : (k <= 16 ? 16 : (k <= 24 ? 24 : 32));
     if (time_start)
       (void)hipEventRecord(time_start, stream);
+#define PCA_SMALL_CASE(NB)                                                     \
+  err = r16 == 0   ? launch_knn_feat_small_blocks<NB, 0>(p, kbucket,           \
+                                                         tiles_bound, stream)  \
+        : r16 == 1 ? launch_knn_feat_small_blocks<NB, 1>(p, kbucket,           \
+                                                         tiles_bound, stream)  \
+                   : launch_knn_feat_small_blocks<NB, 2>(p, kbucket,           \
+                                                         tiles_bound, stream)
     switch (nb) {
     case 3:
-      err = launch_knn_feat_small_blocks<3>(p, kbucket, tiles_bound, stream);
+      PCA_SMALL_CASE(3);
       break;
     case 5:
-      err = launch_knn_feat_small_blocks<5>(p, kbucket, tiles_bound, stream);
+      PCA_SMALL_CASE(5);
       break;
     default:
-      err = launch_knn_feat_small_blocks<9>(p, kbucket, tiles_bound, stream);
+      PCA_SMALL_CASE(9);
       break;
     }
+#undef PCA_SMALL_CASE
     if (time_stop)
       (void)hipEventRecord(time_stop, stream);
-    if (err != hipSuccess)
-      return err;
+    return err;
   } else if (lay.wide_buf != 0) {
     // eight-wave first stage: plan, filter, gather
     const FeatWidePlan wp = feat_wide_plan(in.n, in.m, in.num_segments, k);
@@ -870,7 +946,7 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
     break;
   }
   }
-  if (!small) {
+  {
     const int waves = kBlock / kWave;
     const int rgrid = (in.m + waves - 1) / waves;
     if (cosine)
@@ -888,7 +964,7 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
   // while nothing is flagged (no host read in between).  First the scan that
   // collects the rows at or below a query's k-th listed distance, then --
   // only for what that scan could not take -- the full second pass.
-  if (!small) { // (the one-kernel search queues nothing for the scan)
+  {
     const int waves = kBlock / kWave;
     const int sgrid =
         (redo_cap + kFeatRedoGroup - 1) / kFeatRedoGroup * kFeatRedoSlices;

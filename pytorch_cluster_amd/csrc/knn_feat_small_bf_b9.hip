@@ -1,0 +1,7 @@
+// Feature-space kNN of moderate examples in one exact kernel: 9 blocks of 16 components (up to 128 features),
+// bf16 rows.
+#include "knn_feat_small_impl.hpp"
+
+namespace pca {
+PCA_KNN_FEAT_SMALL_DEFINE(9, 2)
+} // namespace pca

@@ -50,8 +50,14 @@
 // neighbours (packed as padding); rows far larger than the rest (left out of
 // the scale, FeatGlobals::out_rows) are evaluated exactly for every query at
 // the end; if a row's squared norm overflows (FeatGlobals::odd_rows), or for a
-// query the filter cannot take (FeatQuery::odd), the queries are marked for
-// the full second pass exactly as feat_refine_kernel marks them.
+// query the filter cannot take (FeatQuery::odd), the lanes concerned park
+// every row instead of the rows under a cut: slow, and the same result.
+//
+// fp16 and bf16 rows (knn_kernel<c10::Half>, <c10::BFloat16>): the same
+// kernel on the rows widened to fp32, with the reference's 16-bit arithmetic
+// in the exact distances (SmallChain) and a cut widened by what that
+// arithmetic can lose against the distance in real numbers -- 3 % at 64
+// components of fp16, 6 % at 128; 23 % at 64 components of bf16.
 #pragma once
 
 #include <type_traits>
@@ -82,9 +88,60 @@ __device__ __forceinline__ void static_for(F &&f) {
   static_for_each(f, std::make_integer_sequence<int, N>());
 }
 
-template <int NB, int K>
+// The arithmetic of the exact distances.  R16 = 0: fp32 rows, one fused
+// multiply-add per component (csrc/cuda/knn_cuda.cu:61-64 as a GPU compiler
+// builds it).  R16 = 1 / 2: the rows were fp16 / bf16 (widened to fp32 for
+// this kernel, which is exact) and the reference computes in c10::Half /
+// c10::BFloat16: every difference, square and sum is formed in fp32 and
+// rounded to 16 bits (torch/headeronly/util/Half.h:501-560); the sentinel
+// 1e10 is +inf in fp16.
+template <int R16> struct SmallChain {
+  static __device__ __forceinline__ float step(float x, float y, float acc) {
+    // (the compiler turns "widen, operate, round" into 16-bit operations,
+    // which is exact, and would then fuse the square into the sum, which is
+    // one rounding fewer than the reference makes)
+#pragma clang fp contract(off)
+    if (R16 == 0) {
+      const float dc = x - y;
+      return __builtin_fmaf(dc, dc, acc);
+    }
+    const float dc = round_to_16<R16 == 2>(x - y);
+    const float sq = round_to_16<R16 == 2>(dc * dc);
+    return round_to_16<R16 == 2>(acc + sq);
+  }
+  static __device__ __forceinline__ float sentinel() {
+    return R16 == 0 ? kKnnSentinel : round_to_16<R16 == 2>(1e10f);
+  }
+  // A 16-bit chain value H and the distance D in real numbers: with
+  // u = 2^-11 (2^-8) + 2^-23 per rounded operation (the fp32 operation, then
+  // the rounding to 16 bits), three operations on a term and at most d sums
+  // behind it, H >= D (1 - u)^(d + 3) - d t, t what a square can lose below
+  // the normal range (differences and sums there are exact: multiples of the
+  // smallest number of the format).  Hence H < h only if
+  // D < (h + slack()) * widen(d); the factor also carries (1 + (d + 2) 2^-24)
+  // for the fp32 chain the filter's bound was proven against.
+  static __device__ __forceinline__ double widen(int d) {
+    if (R16 == 0)
+      return 1.0;
+    const double u = (R16 == 2 ? 1.0 / 256.0 : 1.0 / 2048.0) + 1.0 / 8388608.0;
+    double keep = 1.0;
+    for (int i = 0; i < d + 3; ++i)
+      keep *= 1.0 - u;
+    return (1.0 + (double)(d + 2) * (1.0 / 16777216.0)) / keep * (1.0 + 1e-9);
+  }
+  static __device__ __forceinline__ double slack(int d) {
+    if (R16 == 0)
+      return 0.0;
+    // fp16: squares below 2^-14 round to multiples of 2^-24; bf16: squares
+    // below 2^-126 may be flushed altogether
+    return (double)d * (R16 == 2 ? 1.1754943508222875e-38 : 1.0 / 16777216.0);
+  }
+};
+
+template <int NB, int K, int R16 = 0>
 __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
     KnnFeatParams p) {
+  typedef SmallChain<R16> Chain;
   typedef FeatShape<NB> S;
   constexpr int RSU = S::RSU;
   constexpr int TILE = kSmallStep;
@@ -128,19 +185,6 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   const int q = y_begin + (tile - p.work_start[seg]) * TQ + wave * 32 + col;
   const bool valid = q < y_end;
 
-  // a query the filter cannot serve at all: left to the full second pass
-  auto unresolved = [&]() {
-    p.out_count[q] = 0;
-    p.redo_q[q] = 1;
-    atomicAdd(&p.globals->any_redo, 1);
-    atomicAdd(&p.globals->unresolved, 1);
-  };
-  if (p.globals->odd_rows != 0) {
-    if (valid && half == 0)
-      unresolved();
-    return;
-  }
-
   const int d = p.d;
   const int k = p.k;
   const bool vec4 = (d & 3) == 0;
@@ -171,7 +215,13 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
 
   const float inv_sigma = feat_inv_sigma(p.globals->max_bits);
   const FeatQuery fq = feat_query<false>(my_y, d, inv_sigma, 1.0f);
-  const bool active = valid && !fq.dead && !fq.odd;
+  // active: the query searches (a NaN component: no neighbours).  filtered:
+  // it does so with the fp16 lower bound; if the filter cannot take the query
+  // (a component beyond the range the scale was made for) or some row of x
+  // (a squared norm that overflows), every row is evaluated instead.
+  const bool active = valid && !fq.dead;
+  const bool filtered = active && !fq.odd && p.globals->odd_rows == 0;
+  const float sentinel = Chain::sentinel();
   const double scale2 = (double)inv_sigma * (double)inv_sigma;
   const float y_scale = -2.0f * inv_sigma;
   const int seg_len = x_end - x_begin;
@@ -187,10 +237,10 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       const int cb = 16 * i + 8 * half;
 #pragma unroll
       for (int e = 0; e < 8; ++e)
-        hb[e] = (active && cb + e < d)
+        hb[e] = (filtered && cb + e < d)
                     ? feat_h(my_y[min(cb + e, d - 1)] * y_scale)
                     : 0u;
-    } else if (half == 0 && active) {
+    } else if (half == 0 && filtered) {
       hb[0] = 0x7800u; // 2^15
       hb[1] = 0x4c00u; // 2^4
       hb[2] = 0x2000u; // 2^-7
@@ -298,17 +348,14 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       for (int c = 0; c < (d >> 2); ++c) {
         const float4 a = x4[c];
         const float4 b = y4[c];
-        const float d0 = a.x - b.x, d1 = a.y - b.y;
-        const float d2 = a.z - b.z, d3 = a.w - b.w;
-        acc = __builtin_fmaf(d0, d0, acc);
-        acc = __builtin_fmaf(d1, d1, acc);
-        acc = __builtin_fmaf(d2, d2, acc);
-        acc = __builtin_fmaf(d3, d3, acc);
+        acc = Chain::step(a.x, b.x, acc);
+        acc = Chain::step(a.y, b.y, acc);
+        acc = Chain::step(a.z, b.z, acc);
+        acc = Chain::step(a.w, b.w, acc);
       }
     } else {
       for (int c = 0; c < d; ++c) {
-        const float dc = xr[c] - my_y[c];
-        acc = __builtin_fmaf(dc, dc, acc);
+        acc = Chain::step(xr[c], my_y[c], acc);
       }
     }
     return acc;
@@ -358,8 +405,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   // exact distances must be strictly below thresh; `shared`: what the sampled
   // rows and the partner lane say about the query's final k-th distance
   // (equality admitted: the rows at the bound are found again by the search)
-  float thresh = active ? kKnnSentinel : -__builtin_inff();
-  float shared = kKnnSentinel;
+  float thresh = active ? sentinel : -__builtin_inff();
+  float shared = sentinel;
   {
     float seed[SEEDS];
 #pragma unroll
@@ -391,7 +438,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       const float e = exact(buf, j);
       // (a padding row, a NaN or a distance beyond the limit is no sample)
       const float sample =
-          (active && j < rows && least < __builtin_inff() && e < kKnnSentinel)
+          (active && j < rows && least < __builtin_inff() && e < sentinel)
               ? e
               : __builtin_inff();
 #pragma unroll
@@ -419,7 +466,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
         __float_as_uint(own), __float_as_uint(own), false, false);
     const float partner = __uint_as_float(half ? both[0] : both[1]);
     const float bound = __builtin_fmaxf(own, partner);
-    if (active && bound < kKnnSentinel) {
+    if (active && bound < sentinel) {
       shared = next_up_positive(bound);
       thresh = __builtin_fminf(thresh, shared);
     }
@@ -430,9 +477,11 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   // against feat_float_above(c) admits everything up to c = thresh / sigma^2
   // - shift)
   float cut = -__builtin_inff();
+  const double widen = Chain::widen(d) * scale2;
+  const double slack = Chain::slack(d);
   auto set_cut = [&]() {
-    if (active)
-      cut = feat_float_above((double)thresh * scale2 - fq.shift);
+    if (filtered)
+      cut = feat_float_above(((double)thresh + slack) * widen - fq.shift);
   };
   set_cut();
   // What the two lanes of a query tell each other (knn_lowd_mc_impl.hpp).
@@ -442,7 +491,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
         __float_as_uint(own), __float_as_uint(own), false, false);
     float partner = __uint_as_float(half ? both[0] : both[1]);
     const int c = k >> 1;
-    float mid = kKnnSentinel;
+    float mid = sentinel;
 #pragma unroll
     for (int cc = (K >= 8 ? K / 2 - 4 : 0); cc <= K / 2; ++cc)
       if (cc >= 1 && cc == c) {
@@ -453,7 +502,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
         __float_as_uint(mid), __float_as_uint(mid), false, false);
     const float partner_mid = __uint_as_float(half ? mids[0] : mids[1]);
     partner = __builtin_fminf(partner, __builtin_fmaxf(mid, partner_mid));
-    if (active && partner < kKnnSentinel) {
+    if (active && partner < sentinel) {
       shared = __builtin_fminf(shared, next_up_positive(partner));
       thresh = __builtin_fminf(thresh, shared);
     }
@@ -498,12 +547,10 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
           if (f0 + 4 * c + e < quads) {
             const small_v4f xv = gathered[wave][lane][e];
             const small_v4f b = y4[f0 + 4 * c + e];
-            const float d0 = xv.x - b.x, d1 = xv.y - b.y;
-            const float d2 = xv.z - b.z, d3 = xv.w - b.w;
-            acc = __builtin_fmaf(d0, d0, acc);
-            acc = __builtin_fmaf(d1, d1, acc);
-            acc = __builtin_fmaf(d2, d2, acc);
-            acc = __builtin_fmaf(d3, d3, acc);
+            acc = Chain::step(xv.x, b.x, acc);
+            acc = Chain::step(xv.y, b.y, acc);
+            acc = Chain::step(xv.z, b.z, acc);
+            acc = Chain::step(xv.w, b.w, acc);
           }
         }
       }
@@ -515,8 +562,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
     const float *xr = p.x + (size_t)g * d;
     float acc = 0.0f;
     for (int c = 0; c < d; ++c) {
-      const float dc = xr[c] - my_y[c];
-      acc = __builtin_fmaf(dc, dc, acc);
+      acc = Chain::step(xr[c], my_y[c], acc);
     }
     return acc;
   };
@@ -627,12 +673,13 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
     m0 = min3f(m0, m1, m2);
     m3 = min3f(m3, m4, a[15]);
     const float least = __builtin_fminf(m0, m3);
-    if (__any(least < cut)) {
+    const bool all_rows = active && !filtered;
+    if (__any(least < cut || all_rows)) {
       // the lane's rows under the cut: bit 15 - v for accumulator v
       uint32_t mask = 0;
 #pragma unroll
       for (int v = 0; v < 16; ++v)
-        if (a[v] < cut && row_of(v) < rows)
+        if ((a[v] < cut || all_rows) && row_of(v) < rows)
           mask |= 0x8000u >> v;
       if (mask != 0) {
         queue[qn][tid] = ((uint32_t)t << 16) | mask;
@@ -652,8 +699,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       float e = 0.0f;
       const float *xr = p.x + (size_t)g * d;
       for (int c = 0; c < d; ++c) {
-        const float dc = xr[c] - my_y[c];
-        e = __builtin_fmaf(dc, dc, e);
+        e = Chain::step(xr[c], my_y[c], e);
       }
       // (a query without a bound -- fewer sampled rows than it takes -- cuts
       // nowhere and has met the row among its parked ones already: the same
@@ -666,22 +712,18 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       const auto both = __builtin_amdgcn_permlane32_swap(
           (unsigned)listed, (unsigned)listed, false, false);
       listed = listed || (half ? both[0] : both[1]) != 0u;
-      const bool ok = active && half == 0 && e < kKnnSentinel && !listed;
+      const bool ok = active && half == 0 && e < sentinel && !listed;
       sorted_insert<K>(best, ok ? key : empty_key());
     }
   }
 
   unite_halves<K>(best, k, half);
   if (half == 0 && valid) {
-    if (fq.odd) {
-      unresolved();
-    } else {
-      if (active)
-        write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
-      else
-        p.out_count[q] = 0;
-      p.redo_q[q] = 0;
-    }
+    if (active)
+      write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+    else
+      p.out_count[q] = 0;
+    p.redo_q[q] = 0;
   }
 #ifdef PCA_FEAT_STATS
   // (one addition per wave and counter: additions to one word take turns)
@@ -698,29 +740,29 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
 
 // Everything for one number of blocks (instantiated in its own translation
 // unit so that the sizes build in parallel).
-template <int NB>
+template <int NB, int R16>
 hipError_t launch_knn_feat_small_blocks(const KnnFeatParams &p, int kbucket,
                                         int grid, hipStream_t stream);
 
-#define PCA_KNN_FEAT_SMALL_DEFINE(NB_)                                         \
+#define PCA_KNN_FEAT_SMALL_DEFINE(NB_, R16_)                                   \
   template <>                                                                  \
-  hipError_t launch_knn_feat_small_blocks<NB_>(                                \
+  hipError_t launch_knn_feat_small_blocks<NB_, R16_>(                          \
       const KnnFeatParams &p, int kbucket, int grid, hipStream_t stream) {     \
     switch (kbucket) {                                                         \
     case 8:                                                                    \
-      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 8>), dim3(grid),          \
+      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 8, R16_>), dim3(grid),    \
                          dim3(kBlock), 0, stream, p);                          \
       break;                                                                   \
     case 16:                                                                   \
-      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 16>), dim3(grid),         \
+      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 16, R16_>), dim3(grid),   \
                          dim3(kBlock), 0, stream, p);                          \
       break;                                                                   \
     case 24:                                                                   \
-      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 24>), dim3(grid),         \
+      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 24, R16_>), dim3(grid),   \
                          dim3(kBlock), 0, stream, p);                          \
       break;                                                                   \
     case 32:                                                                   \
-      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 32>), dim3(grid),         \
+      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 32, R16_>), dim3(grid),   \
                          dim3(kBlock), 0, stream, p);                          \
       break;                                                                   \
     default:                                                                   \

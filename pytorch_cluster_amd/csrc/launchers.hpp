@@ -180,10 +180,19 @@ hipError_t launch_knn_mfma(const SearchInput &in, int k, bool cosine,
 bool knn_feat_supported(int d, int k, bool cosine);
 size_t knn_feat_scratch_bytes(int n, int m, int d, int num_segments, int k);
 // work_start: tiles of kMfmaTileQueries queries (planned by the caller).
+// r16 = 1 / 2: x and y hold fp16 / bf16 rows (knn_feat16_supported shapes
+// only; scratch: knn_feat16_scratch_bytes); the results are those of the
+// reference's kernel for that element type.
 hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
                            const int *work_start, void *scratch,
                            const DenseResult &out, hipEvent_t time_start,
-                           hipEvent_t time_stop, hipStream_t stream);
+                           hipEvent_t time_stop, hipStream_t stream,
+                           int r16 = 0);
+// fp16 / bf16 rows through the matrix-core filter (knn_feat_small_impl.hpp):
+// Euclidean, 8 < d <= 128 (bf16: 64), k <= 32; PCA_KNN_FEAT_16BIT=0: never.
+bool knn_feat16_supported(int n, int d, int num_segments, int k, bool cosine,
+                          bool bf16);
+size_t knn_feat16_scratch_bytes(int n, int m, int d, int num_segments, int k);
 
 // --- knn_generic_*.hip -----------------------------------------------------
 

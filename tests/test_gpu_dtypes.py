@@ -104,6 +104,76 @@ def test_knn_16bit_parity(oracle, monkeypatch, dtype, kind, d, k, cosine,
     assert (got == want).all()
 
 
+def _knn16_case(rng, kind, n, m, d, dtype):
+    x = rng.standard_normal((n, d))
+    y = rng.standard_normal((m, d))
+    if kind == "rows_as_queries":
+        y[: m // 2] = x[rng.integers(0, n, m // 2)]
+    elif kind == "duplicates":
+        x = x[rng.integers(0, 40, n)]
+        y = x[rng.integers(0, n, m)] + 0.0
+    elif kind == "one_large_component":
+        # sums that stop growing: the first term is worth hundreds of the rest
+        x[:, 0] *= 60.0
+        y[:, 0] *= 60.0
+    elif kind == "overflow":
+        # squared distances around and beyond the largest fp16 number
+        x *= 25.0
+        y *= 25.0
+    elif kind == "tiny":
+        x *= 2e-4
+        y *= 2e-4
+    elif kind == "large_rows_and_queries":
+        x[rng.integers(0, n, 5)] *= 300.0
+        y[[0, m - 1]] *= 500.0
+    elif kind == "not_finite":
+        x[3, 1] = np.nan
+        x[n // 2] = np.inf
+        y[5, 0] = np.nan
+        y[6, 2] = -np.inf
+    elif kind == "grid":
+        x = np.round(x)
+        y = np.round(y)
+    return (torch.from_numpy(x).to(dtype), torch.from_numpy(y).to(dtype))
+
+
+@pytest.mark.parametrize("dtype,kind16", [(torch.float16, 0),
+                                          (torch.bfloat16, 1)])
+@pytest.mark.parametrize("kind", ["plain", "rows_as_queries", "duplicates",
+                                  "one_large_component", "overflow", "tiny",
+                                  "large_rows_and_queries", "not_finite",
+                                  "grid"])
+def test_knn_16bit_feature_space_parity(oracle, dtype, kind16, kind):
+    # 16-bit rows of 9 to 128 components (bf16: 64): the matrix-core filter in
+    # front of the exact 16-bit chain (knn_feat_small_impl.hpp), against the
+    # checker's chain; the 16-bit sums produce many equal distances
+    rng = np.random.default_rng(len(kind) * 7 + kind16)
+    dims = (9, 20, 64, 100, 128) if kind16 == 0 else (9, 20, 33, 64)
+    for d in dims:
+        n, m = 2600, 420
+        x, y = _knn16_case(rng, kind, n, m, d, dtype)
+        ptr_x = np.array([0, 40, 40, 1500, n])
+        ptr_y = np.array([0, 30, 50, 300, m])
+        for k in ((1, 20) if d % 2 else (8, 32)):
+            got = gpu_knn_t(x, y, ptr_x, ptr_y, k)
+            want, _ = oracle.knn_op16(bits(x), bits(y), ptr_x, ptr_y, k, False,
+                                      kind16)
+            assert got.shape == want.shape, (d, k)
+            assert (got == want).all(), (d, k)
+
+
+def test_knn_16bit_feature_space_same_edges_without_the_filter(monkeypatch):
+    # one larger call against the exhaustive 16-bit scan of the library itself
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(24 * 900, 64, generator=g).to(torch.float16)
+    ptr = np.arange(25) * 900
+    with_filter = gpu_knn_t(x, x, ptr, ptr, 21)
+    monkeypatch.setenv("PCA_KNN_FEAT_16BIT", "0")
+    without = gpu_knn_t(x, x, ptr, ptr, 21)
+    assert with_filter.shape == without.shape == (2, 24 * 900 * 21)
+    assert (with_filter == without).all()
+
+
 def test_knn_fp64_large_cloud_default_slices(oracle):
     # enough rows that the library slices on its own; duplicated rows, so that
     # equal distances meet across slice borders
