@@ -361,3 +361,68 @@ def test_split_bf16_filter_keeps_near_duplicates(d):
     used = (t - (e - ysq.astype(np.float64)[:, None]
                  - eps * xsq.astype(np.float64)[None, :])) / (2.0 ** -15 * scale)
     assert 0.5 < used[:50, :50].diagonal().max() <= 1.0
+
+
+# ---- 16-bit rows: what the reference's chain can lose (knn_feat_small_impl.hpp)
+
+def _round16(v, bf16):
+    """float32 array -> nearest fp16 / bf16 number (ties to even) as float32."""
+    v = np.asarray(v, dtype=np.float32)
+    if not bf16:
+        return v.astype(np.float16).astype(np.float32)
+    bits = v.view(np.uint32).astype(np.uint64)
+    bits = (bits + 0x7fff + ((bits >> 16) & 1)) & 0xffff0000
+    return bits.astype(np.uint32).view(np.float32)
+
+
+def _chain16(x, y, bf16):
+    """The reference's scalar loop in c10::Half / c10::BFloat16 arithmetic
+    (csrc/cuda/knn_cuda.cu:61-64): every operator works in fp32 and rounds to
+    16 bits.  x: [rows, d], y: [d]."""
+    acc = np.zeros(len(x), dtype=np.float32)
+    for c in range(x.shape[1]):
+        diff = _round16(x[:, c] - y[c], bf16)
+        sq = _round16(diff * diff, bf16)
+        acc = _round16(acc + sq, bf16)
+    return acc
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("kind", ["normal", "first_term_large", "tiny",
+                                  "mixed_scales", "grid", "decreasing"])
+def test_16bit_chain_against_the_real_distance(bf16, kind):
+    # the cut of the one-kernel search admits a row whenever its distance in
+    # real numbers D satisfies D < (h + d t) (1 - u)^-(d + 3): every row whose
+    # chain value H is below h must do so, i.e. H >= D (1 - u)^(d + 3) - d t
+    rng = np.random.default_rng(stable_seed("chain16", bf16, kind))
+    u = (2.0 ** -8 if bf16 else 2.0 ** -11) + 2.0 ** -23
+    t = 2.0 ** -126 if bf16 else 2.0 ** -24
+    for d in (9, 33, 64) + (() if bf16 else (128,)):
+        x = rng.standard_normal((4000, d))
+        y = rng.standard_normal(d)
+        if kind == "first_term_large":
+            x[:, 0] *= 40.0
+            y[0] *= -40.0
+        elif kind == "tiny":
+            x *= 3e-4
+            y *= 3e-4
+        elif kind == "mixed_scales":
+            x *= 10.0 ** rng.integers(-4, 2, (4000, 1))
+        elif kind == "grid":
+            x, y = np.round(2 * x) / 2, np.round(2 * y) / 2
+        elif kind == "decreasing":
+            # the sum stops growing: later terms fall below half a unit of it
+            scale = 30.0 * 0.8 ** np.arange(d)
+            x *= scale
+            y *= scale
+        x16 = _round16(x, bf16)
+        y16 = _round16(y, bf16)
+        H = _chain16(x16, y16, bf16).astype(np.float64)
+        D = ((x16.astype(np.float64) - y16.astype(np.float64)) ** 2).sum(1)
+        finite = np.isfinite(H)
+        assert finite.any()
+        lower = D * (1.0 - u) ** (d + 3) - d * t
+        assert (H[finite] >= lower[finite]).all(), (d, kind)
+        # and the bound is not vacuous: the chain does lose something
+        if kind in ("normal", "decreasing"):
+            assert (H[finite] < D[finite]).any()
