@@ -113,8 +113,11 @@ size_t feat_pack_bytes(int n, int d) {
 
 __global__ __launch_bounds__(kBlock) void feat_init_kernel(
     FeatGlobals *g, float *tau, int m, int *hit_count, int redo_cap,
-    int *overflow) {
+    int *overflow, unsigned long long *edge_sums, int edge_blocks) {
   const int i = blockIdx.x * kBlock + threadIdx.x;
+  // (the compaction's block sums, when the search counts the edges)
+  if (edge_sums != nullptr && i < edge_blocks)
+    edge_sums[i] = 0ull;
   if (i < m) {
     tau[i] = __builtin_inff();
     if (overflow != nullptr)
@@ -213,7 +216,10 @@ __global__ __launch_bounds__(kBlock) void feat_rows_kernel(
   if ((threadIdx.x & (kWave - 1)) == 0)
     part[threadIdx.x / kWave] = big;
   __syncthreads();
-  if (threadIdx.x == 0) {
+  // (with a histogram the scale is made from it, feat_scale_kernel: the
+  // first couple of thousand workgroups of a launch all find this word at
+  // zero, and their maxima on one word took 20 us)
+  if (threadIdx.x == 0 && hist == nullptr) {
     for (int w = 1; w < kBlock / kWave; ++w)
       big = part[w] > big ? part[w] : big;
     // (one word for the whole call: only workgroups that raise it go there)
@@ -231,8 +237,9 @@ __global__ __launch_bounds__(kBlock) void feat_rows_kernel(
 // never more than one in 64) are at least four times larger than all others --
 // then for the others, which keep their bits in fp16; the few are handled
 // exactly (see FeatGlobals).  One workgroup of 256 threads.
+// (y_is_x: the queries are the rows of x, whose histogram stands for both)
 __global__ __launch_bounds__(256) void feat_scale_kernel(FeatGlobals *g, int n,
-                                                         int m) {
+                                                         int m, bool y_is_x) {
   __shared__ unsigned hx[256], hy[256];
   __shared__ int need_x, need_y, top;
   const int t = threadIdx.x;
@@ -241,12 +248,14 @@ __global__ __launch_bounds__(256) void feat_scale_kernel(FeatGlobals *g, int n,
     sum_x += g->hist_x[c * 256 + t];
     sum_y += g->hist_y[c * 256 + t];
   }
+  if (y_is_x)
+    sum_y = sum_x;
   hx[t] = sum_x;
   hy[t] = sum_y;
   if (t == 0) {
     need_x = 255;
     need_y = 255;
-    top = 0;
+    top = -1;
   }
   __syncthreads();
   // rows with a larger exponent than t: one wave, four bins per lane, a
@@ -294,10 +303,14 @@ __global__ __launch_bounds__(256) void feat_scale_kernel(FeatGlobals *g, int n,
     atomicMax(&top, t);
   __syncthreads();
   if (t == 0) {
+    // (only the exponent of max_bits is used: the largest number of the
+    // binade stands for the largest component)
     const int need = max(need_x, need_y);
     if (top - need >= 2) {
       g->max_bits = ((unsigned)(need + 1) << 23) - 1u;
       g->out_limit = g->max_bits;
+    } else {
+      g->max_bits = top < 0 ? 0u : ((unsigned)(top + 1) << 23) - 1u;
     }
   }
 }
@@ -617,6 +630,11 @@ void launch_widen16(const void *src, size_t count, bool bf16, float *dst,
 
 } // namespace
 
+bool knn_feat_one_kernel(int n, int d, int num_segments, int k, bool cosine) {
+  return knn_feat_supported(d, k, cosine) &&
+         feat_small_applies(n, d, num_segments, k, cosine);
+}
+
 bool knn_feat16_supported(int n, int d, int num_segments, int k, bool cosine,
                           bool bf16) {
   if (const char *env = std::getenv("PCA_KNN_FEAT_16BIT"))
@@ -652,10 +670,12 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
     float *y32 = reinterpret_cast<float *>(at);
     at += align256(sizeof(float) * (size_t)in.m * in.d);
     scratch = at;
+    const bool y_is_x = in.y == in.x && in.m == in.n;
     launch_widen16(in.x, (size_t)in.n * in.d, r16 == 2, x32, stream);
-    launch_widen16(in.y, (size_t)in.m * in.d, r16 == 2, y32, stream);
+    if (!y_is_x)
+      launch_widen16(in.y, (size_t)in.m * in.d, r16 == 2, y32, stream);
     in.x = x32;
-    in.y = y32;
+    in.y = y_is_x ? x32 : y32;
   }
   const FeatLayout lay =
       feat_layout(in.n, in.m, in.d, in.num_segments, k);
@@ -690,9 +710,13 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
   const float *yf = static_cast<const float *>(in.y);
   const int nb = feat_blocks(in.d);
 
+  const bool small =
+      r16 != 0 || feat_small_applies(in.n, in.d, in.num_segments, k, cosine);
   hipLaunchKernelGGL(feat_init_kernel, dim3((in.m + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, globals, tau, in.m, hit_count,
-                     redo_cap, overflow);
+                     redo_cap, overflow, small ? out.edge_sums : nullptr,
+                     (in.m + kCompactBlockQueries - 1) / kCompactBlockQueries +
+                         1);
   // squared norms that only classify the rows (NaN: a non-finite component);
   // for the Euclidean distance they also enter the filter
   float *x_class = cosine ? x_class_buf : x_norm;
@@ -716,13 +740,16 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
                        dim3((in.n + rows_per_block - 1) / rows_per_block),
                        dim3(kBlock), 0, stream, xf, in.n, in.d, x_norm,
                        globals, x_big, globals->hist_x);
-    hipLaunchKernelGGL(feat_rows_kernel,
-                       dim3((in.m + rows_per_block - 1) / rows_per_block),
-                       dim3(kBlock), 0, stream, yf, in.m, in.d,
-                       static_cast<float *>(nullptr), globals,
-                       static_cast<unsigned *>(nullptr), globals->hist_y);
+    // (a cloud searched in itself: one pass over the rows serves both)
+    const bool y_is_x = yf == xf && in.m == in.n;
+    if (!y_is_x)
+      hipLaunchKernelGGL(feat_rows_kernel,
+                         dim3((in.m + rows_per_block - 1) / rows_per_block),
+                         dim3(kBlock), 0, stream, yf, in.m, in.d,
+                         static_cast<float *>(nullptr), globals,
+                         static_cast<unsigned *>(nullptr), globals->hist_y);
     hipLaunchKernelGGL(feat_scale_kernel, dim3(1), dim3(256), 0, stream,
-                       globals, in.n, in.m);
+                       globals, in.n, in.m, y_is_x);
   }
   {
     hipError_t perr;
@@ -794,9 +821,10 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
 
   const int kp = feat_width(k);
   hipError_t err;
-  const bool small =
-      r16 != 0 || feat_small_applies(in.n, in.d, in.num_segments, k, cosine);
   if (small) {
+    p.edge_sums = out.edge_sums;
+    p.self_pos = out.self_pos;
+    p.kept = out.kept;
     // one exact kernel: nothing is listed, merged, refined or searched again
     const int kbucket = k <= 8 ? 8 : (k <= 16 ? 16 : (k <= 24 ? 24 : 32));
     if (time_start)

@@ -274,6 +274,11 @@ struct KnnFeatParams {
   int *out_idx;
   float *out_dist;
   int *out_count;
+  // the compaction's block sums and self slots (DenseResult; the one-kernel
+  // search fills them, NULL otherwise)
+  unsigned long long *edge_sums = nullptr;
+  int *self_pos = nullptr;
+  int *kept = nullptr;
 };
 
 // Packed row: 2 units of 16 bytes (8 fp16) per block of 16 components, NB

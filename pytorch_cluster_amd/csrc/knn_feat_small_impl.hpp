@@ -719,11 +719,14 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
 
   unite_halves<K>(best, k, half);
   if (half == 0 && valid) {
+    int found = 0;
     if (active)
-      write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
+      found = write_dense<K>(best, k, q, p.out_idx, p.out_dist, p.out_count);
     else
       p.out_count[q] = 0;
     p.redo_q[q] = 0;
+    // (edges counted here: the compaction starts from the block sums)
+    note_edges<K>(best, k, q, found, p.edge_sums, p.self_pos, p.kept);
   }
 #ifdef PCA_FEAT_STATS
   // (one addition per wave and counter: additions to one word take turns)

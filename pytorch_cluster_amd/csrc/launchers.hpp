@@ -82,7 +82,7 @@ hipError_t launch_compact(const DenseResult &dense, int m, int64_t *edges,
 // compaction's workspace when the call is small enough for the compaction
 // that adds up the block sums on its own; launch_compact then skips its
 // counting pass.  Only for searches that fill them (the low-dimensional
-// matrix-core kernels).
+// matrix-core kernels, the one-kernel feature-space search).
 void compact_hints(DenseResult &dense, int m, void *workspace, bool drop_self);
 // Queries per block sum.
 constexpr int kCompactBlockQueries = 256;
@@ -188,6 +188,9 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
                            const DenseResult &out, hipEvent_t time_start,
                            hipEvent_t time_stop, hipStream_t stream,
                            int r16 = 0);
+// Whether launch_knn_feat serves such a call (fp32 rows) with its one-kernel
+// search, which counts the edges itself (compact_hints applies).
+bool knn_feat_one_kernel(int n, int d, int num_segments, int k, bool cosine);
 // fp16 / bf16 rows through the matrix-core filter (knn_feat_small_impl.hpp):
 // Euclidean, 8 < d <= 128 (bf16: 64), k <= 32; PCA_KNN_FEAT_16BIT=0: never.
 bool knn_feat16_supported(int n, int d, int num_segments, int k, bool cosine,

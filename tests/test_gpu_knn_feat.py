@@ -342,6 +342,16 @@ def test_one_kernel_search_is_the_default_for_small_examples(oracle,
     _run(oracle, x, x, ptr, ptr, 21)
     odd, flagged = _flagged_queries(x, x, 21)
     assert odd == 0 and flagged == 0
+    # the same tensor on both sides (a graph of the cloud in itself): the
+    # preparation goes over the rows once
+    from gpu_common import dev
+    from pytorch_cluster_amd import capi
+    xd, pd = dev(x), dev(ptr)
+    for t in (xd, xd.half(), xd[:, :40].contiguous().bfloat16()):
+        one, _ = capi.knn_edges(t, t, pd, pd, 21)
+        two, _ = capi.knn_edges(t, t.clone(), pd, pd, 21)
+        assert one.shape == two.shape == (2, 24 * 700 * 21)
+        assert bool((one == two).all())
 
 
 def test_many_slices_share_their_bounds(oracle, monkeypatch):
