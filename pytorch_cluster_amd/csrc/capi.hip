@@ -208,6 +208,11 @@ size_t radius_workspace(int64_t n, int64_t m, int64_t d, int64_t num_segments,
   if (dtype == PCA_F32 &&
       pca::radius_mc_supported((int)d, (int)n, (int)m, (int)num_segments))
     bytes += pca::radius_mc_scratch_bytes((int)n, (int)d);
+  else if (dtype == PCA_F32 &&
+           pca::radius_feat_supported((int)n, (int)m, (int)d,
+                                      (int)num_segments, (int)slots))
+    bytes += pca::knn_feat_scratch_bytes((int)n, (int)m, (int)d,
+                                         (int)num_segments, (int)slots);
   bytes += align256(sizeof(int) * (size_t)(num_segments + 1));
   bytes += align256(sizeof(int) * (size_t)m * (size_t)slots);
   bytes += align256(sizeof(int) * (size_t)m);
@@ -771,11 +776,18 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
   const bool matrix_cores =
       dtype == PCA_F32 &&
       pca::radius_mc_supported((int)d, (int)n, (int)m, (int)num_segments);
+  const bool feature_space = !matrix_cores && dtype == PCA_F32 &&
+                             pca::radius_feat_supported(
+                                 (int)n, (int)m, (int)d, (int)num_segments,
+                                 (int)slots);
   Carver ws(workspace);
   void *packed_rows = nullptr;
   if (matrix_cores)
     packed_rows =
         ws.take<char>(pca::radius_mc_scratch_bytes((int)n, (int)d));
+  else if (feature_space)
+    packed_rows = ws.take<char>(pca::knn_feat_scratch_bytes(
+        (int)n, (int)m, (int)d, (int)num_segments, (int)slots));
   int *work_start = ws.take<int>((size_t)num_segments + 1);
   pca::DenseResult dense;
   dense.idx = ws.take<int>((size_t)m * slots);
@@ -795,8 +807,9 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
 
   pca::SearchInput in{x,      y,      ptr_x,  ptr_y,
                       (int)n, (int)m, (int)d, (int)num_segments};
-  const int per_item = matrix_cores ? pca::kRadiusMcTileQueries
-                                    : pca::kRadiusQueriesPerWave;
+  const int per_item = matrix_cores    ? pca::kRadiusMcTileQueries
+                       : feature_space ? pca::kMfmaTileQueries
+                                       : pca::kRadiusQueriesPerWave;
   int rc = PCA_OK;
   // (the matrix-core path plans its work in the launch that packs the rows)
   if (!matrix_cores)
@@ -808,11 +821,18 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
     return rc;
   const int bound =
       pca::plan_upper_bound((int)m, (int)num_segments, per_item);
-  if (!matrix_cores)
+  if (!matrix_cores && !feature_space)
     timer.begin();
-  if (matrix_cores)
+  if (matrix_cores || feature_space)
     pca::compact_hints(dense, (int)m, compact_ws, false);
-  if (matrix_cores)
+  if (feature_space) {
+    const pca::FeatRadius radius{r2, ignore_same_index != 0};
+    rc = check_launch(pca::launch_knn_feat(in, (int)slots, false, work_start,
+                                           packed_rows, dense, timer.start,
+                                           timer.stop, stream, 0, &radius),
+                      "knn_feat_small_kernel (radius)");
+    timer.stop = nullptr;
+  } else if (matrix_cores)
     rc = check_launch(pca::launch_radius_mc(in, r2, ignore_same_index != 0,
                                             work_start, bound, packed_rows,
                                             dense, timer.start, stream,

@@ -48,6 +48,15 @@ PCA_DECLARE_FEAT_SMALL_BLOCKS(5, 2)
 PCA_DECLARE_FEAT_SMALL_BLOCKS(9, 2)
 #undef PCA_DECLARE_FEAT_SMALL_BLOCKS
 
+#define PCA_DECLARE_RADIUS_FEAT_BLOCKS(NB, R16)                                \
+  template <>                                                                  \
+  hipError_t launch_radius_feat_blocks<NB, R16>(const KnnFeatParams &, int,    \
+                                                int, hipStream_t);
+PCA_DECLARE_RADIUS_FEAT_BLOCKS(3, 0)
+PCA_DECLARE_RADIUS_FEAT_BLOCKS(5, 0)
+PCA_DECLARE_RADIUS_FEAT_BLOCKS(9, 0)
+#undef PCA_DECLARE_RADIUS_FEAT_BLOCKS
+
 namespace {
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -635,6 +644,21 @@ bool knn_feat_one_kernel(int n, int d, int num_segments, int k, bool cosine) {
          feat_small_applies(n, d, num_segments, k, cosine);
 }
 
+bool radius_feat_supported(int n, int m, int d, int num_segments, int slots) {
+  const bool fits = d > 8 && d <= 128 && slots >= 1 && slots <= 32;
+  if (const char *env = std::getenv("PCA_RADIUS_FEAT")) {
+    if (env[0] == '0')
+      return false;
+    if (env[0] == '1')
+      return fits;
+  }
+  // (the preparation is half a dozen launches: small searches are quicker
+  // with the plain scan)
+  const double work = (double)n / (num_segments > 0 ? num_segments : 1) *
+                      (double)m * (double)d;
+  return fits && work >= 16.0e6;
+}
+
 bool knn_feat16_supported(int n, int d, int num_segments, int k, bool cosine,
                           bool bf16) {
   if (const char *env = std::getenv("PCA_KNN_FEAT_16BIT"))
@@ -657,8 +681,10 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
                            const int *work_start, void *scratch,
                            const DenseResult &out, hipEvent_t time_start,
                            hipEvent_t time_stop, hipStream_t stream,
-                           int r16) {
+                           int r16, const FeatRadius *radius) {
   SearchInput in = in_given;
+  if (radius != nullptr && (r16 != 0 || cosine))
+    return hipErrorInvalidValue;
   if (r16 != 0) {
     // 16-bit rows: searched as fp32 rows (the widening is exact) by the one
     // kernel that can compute the exact distances in the 16-bit arithmetic
@@ -710,8 +736,8 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
   const float *yf = static_cast<const float *>(in.y);
   const int nb = feat_blocks(in.d);
 
-  const bool small =
-      r16 != 0 || feat_small_applies(in.n, in.d, in.num_segments, k, cosine);
+  const bool small = r16 != 0 || radius != nullptr ||
+                     feat_small_applies(in.n, in.d, in.num_segments, k, cosine);
   hipLaunchKernelGGL(feat_init_kernel, dim3((in.m + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, globals, tau, in.m, hit_count,
                      redo_cap, overflow, small ? out.edge_sums : nullptr,
@@ -827,10 +853,16 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
     p.kept = out.kept;
     // one exact kernel: nothing is listed, merged, refined or searched again
     const int kbucket = k <= 8 ? 8 : (k <= 16 ? 16 : (k <= 24 ? 24 : 32));
+    if (radius != nullptr) {
+      p.r2 = radius->r2;
+      p.ignore_same = radius->ignore_same ? 1 : 0;
+    }
     if (time_start)
       (void)hipEventRecord(time_start, stream);
 #define PCA_SMALL_CASE(NB)                                                     \
-  err = r16 == 0   ? launch_knn_feat_small_blocks<NB, 0>(p, kbucket,           \
+  err = radius     ? launch_radius_feat_blocks<NB, 0>(p, kbucket, tiles_bound, \
+                                                      stream)                  \
+        : r16 == 0 ? launch_knn_feat_small_blocks<NB, 0>(p, kbucket,           \
                                                          tiles_bound, stream)  \
         : r16 == 1 ? launch_knn_feat_small_blocks<NB, 1>(p, kbucket,           \
                                                          tiles_bound, stream)  \

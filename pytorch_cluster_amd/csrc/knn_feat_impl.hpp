@@ -279,6 +279,9 @@ struct KnnFeatParams {
   unsigned long long *edge_sums = nullptr;
   int *self_pos = nullptr;
   int *kept = nullptr;
+  // the radius search of the one-kernel search (k: max_num_neighbors)
+  float r2 = 0.0f;
+  int ignore_same = 0;
 };
 
 // Packed row: 2 units of 16 bytes (8 fp16) per block of 16 components, NB

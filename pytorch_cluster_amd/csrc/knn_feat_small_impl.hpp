@@ -138,7 +138,7 @@ template <int R16> struct SmallChain {
   }
 };
 
-template <int NB, int K, int R16 = 0>
+template <int NB, int K, int R16 = 0, bool RADIUS = false>
 __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
     KnnFeatParams p) {
   typedef SmallChain<R16> Chain;
@@ -166,6 +166,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   // per wave: 16 components of 64 gathered rows (five 16-byte units from row
   // to row: neighbouring rows fall on distinct banks)
   __shared__ __attribute__((aligned(16))) small_v4f gathered[kBlock / kWave][kWave][5];
+  __shared__ int wave_full[kBlock / kWave];
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -364,7 +365,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   auto row_of = [&](int v) { return 8 * (v >> 2) + 4 * half + (v & 3); };
 
   // One pass over the example's tiles; body(t, buf, rows) with the tile in
-  // LDS, every(t) after each kSmallQueue tiles and after the last one.  (One
+  // LDS, every() after each kSmallQueue tiles and after the last one (true:
+  // the pass ends there).  (One
   // barrier per tile: a buffer is overwritten a whole tile after its last
   // reader passed the barrier before.)  Slot t % DEPTH of the registers
   // holds tile t + 1 until it is stored, then tile t + 1 + DEPTH.
@@ -393,7 +395,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
         }
       });
       if (((t0 + DEPTH) & (kSmallQueue - 1)) == 0 || t0 + DEPTH >= count)
-        every();
+        if (every())
+          break; // (uniform)
     }
   };
 
@@ -405,9 +408,13 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   // exact distances must be strictly below thresh; `shared`: what the sampled
   // rows and the partner lane say about the query's final k-th distance
   // (equality admitted: the rows at the bound are found again by the search)
-  float thresh = active ? sentinel : -__builtin_inff();
+  float thresh = active ? (RADIUS ? p.r2 : sentinel) : -__builtin_inff();
   float shared = sentinel;
-  {
+  // (the radius search: hits so far, and "no later row of this lane can be
+  // among the query's first k hits")
+  int hits = 0;
+  bool full = !active;
+  if constexpr (!RADIUS) {
     float seed[SEEDS];
 #pragma unroll
     for (int j = 0; j < SEEDS; ++j)
@@ -449,10 +456,10 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
     const int sampled = min(num_tiles, kSmallSampleSteps);
     if (vec4)
       for_tiles(sampled, std::true_type(), std::true_type(), sample_step,
-                [] {});
+                [] { return false; });
     else
       for_tiles(sampled, std::true_type(), std::false_type(), sample_step,
-                [] {});
+                [] { return false; });
     // the ceil(k / 2)-th smallest sample of this lane and of its partner
     const int mine = (k + 1) / 2 - 1;
     float own = __builtin_inff();
@@ -599,15 +606,26 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       g = min(x_begin + (on ? step_row + row_of(v) : 0), p.n - 1);
     };
     auto take = [&](float e, int g, bool on) {
-      const bool ok = on && e < thresh;
+      bool ok = on && e < thresh;
+      if (RADIUS)
+        ok = ok && !full && !(p.ignore_same != 0 && g == q);
       PCA_SSTAT(0, lane == 0);
       PCA_SSTAT(1, on);
       if (!__any(ok))
         return;
       PCA_SSTAT(2, ok);
-      sorted_insert<K>(best, ok ? make_key(e, (uint32_t)g) : empty_key());
-      if (active)
+      // (radius search: the key is the row number alone, the list keeps the
+      // k smallest rows among the hits; a lane's rows arrive in ascending
+      // order, so once it holds k nothing more of it can count)
+      const double key = RADIUS ? make_key(0.0f, (uint32_t)g)
+                                : make_key(e, (uint32_t)g);
+      sorted_insert<K>(best, ok ? key : empty_key());
+      if (RADIUS) {
+        hits += ok ? 1 : 0;
+        full = full || hits >= k;
+      } else if (active) {
         thresh = __builtin_fminf(key_dist(best[K - 1]), shared);
+      }
       changed = true;
     };
     int g;
@@ -657,7 +675,13 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       }
     }
     qn = 0;
-    if (changed) {
+    if (RADIUS) {
+      // both lanes of the query have looked at every row so far: k hits
+      // between them settle the query
+      const auto both = __builtin_amdgcn_permlane32_swap(
+          (unsigned)hits, (unsigned)hits, false, false);
+      full = full || hits + (int)(half ? both[0] : both[1]) >= k;
+    } else if (changed) {
       partner_bounds();
       set_cut();
     }
@@ -674,19 +698,34 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
     m3 = min3f(m3, m4, a[15]);
     const float least = __builtin_fminf(m0, m3);
     const bool all_rows = active && !filtered;
-    if (__any(least < cut || all_rows)) {
+    const bool looking = !RADIUS || !full;
+    if (__any((least < cut || all_rows) && looking)) {
       // the lane's rows under the cut: bit 15 - v for accumulator v
       uint32_t mask = 0;
 #pragma unroll
       for (int v = 0; v < 16; ++v)
-        if ((a[v] < cut || all_rows) && row_of(v) < rows)
+        if ((a[v] < cut || all_rows) && looking && row_of(v) < rows)
           mask |= 0x8000u >> v;
       if (mask != 0) {
         queue[qn][tid] = ((uint32_t)t << 16) | mask;
         ++qn;
       }
     }
-  }, [&] { drain(); });
+  }, [&] {
+    drain();
+    if constexpr (RADIUS) {
+      // a workgroup whose queries all have their k hits leaves the scan
+      const int all_full = __any(!full) ? 0 : 1;
+      if (lane == 0)
+        wave_full[wave] = all_full;
+      __syncthreads();
+      const bool stop = (wave_full[0] & wave_full[1] & wave_full[2] &
+                         wave_full[3]) != 0;
+      __syncthreads();
+      return stop;
+    }
+    return false;
+  });
 
   // rows that were left out of the scale: every query looks at them exactly
   // (the lower lane of a pair; a handful of rows at most)
@@ -704,7 +743,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       // (a query without a bound -- fewer sampled rows than it takes -- cuts
       // nowhere and has met the row among its parked ones already: the same
       // key in its list or in the partner's)
-      const double key = make_key(e, (uint32_t)g);
+      const double key = RADIUS ? make_key(0.0f, (uint32_t)g)
+                                : make_key(e, (uint32_t)g);
       bool listed = false;
 #pragma unroll
       for (int j = 0; j < K; ++j)
@@ -712,7 +752,9 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       const auto both = __builtin_amdgcn_permlane32_swap(
           (unsigned)listed, (unsigned)listed, false, false);
       listed = listed || (half ? both[0] : both[1]) != 0u;
-      const bool ok = active && half == 0 && e < sentinel && !listed;
+      const bool ok = active && half == 0 && !listed &&
+                      (RADIUS ? e < p.r2 && !(p.ignore_same != 0 && g == q)
+                              : e < sentinel);
       sorted_insert<K>(best, ok ? key : empty_key());
     }
   }
@@ -767,6 +809,42 @@ hipError_t launch_knn_feat_small_blocks(const KnnFeatParams &p, int kbucket,
     case 32:                                                                   \
       hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 32, R16_>), dim3(grid),   \
                          dim3(kBlock), 0, stream, p);                          \
+      break;                                                                   \
+    default:                                                                   \
+      return hipErrorInvalidValue;                                             \
+    }                                                                          \
+    return hipGetLastError();                                                  \
+  }
+
+// The radius search with the same kernel (RADIUS): no bound pass, a fixed cut
+// from r^2, lists of the k smallest ROW NUMBERS among the rows within the
+// radius -- what radius_kernel of the reference returns
+// (csrc/cuda/radius_cuda.cu:9-42: the first max_num_neighbors rows in
+// ascending order).
+template <int NB, int R16>
+hipError_t launch_radius_feat_blocks(const KnnFeatParams &p, int kbucket,
+                                     int grid, hipStream_t stream);
+
+#define PCA_RADIUS_FEAT_DEFINE(NB_, R16_)                                      \
+  template <>                                                                  \
+  hipError_t launch_radius_feat_blocks<NB_, R16_>(                             \
+      const KnnFeatParams &p, int kbucket, int grid, hipStream_t stream) {     \
+    switch (kbucket) {                                                         \
+    case 8:                                                                    \
+      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 8, R16_, true>),          \
+                         dim3(grid), dim3(kBlock), 0, stream, p);              \
+      break;                                                                   \
+    case 16:                                                                   \
+      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 16, R16_, true>),         \
+                         dim3(grid), dim3(kBlock), 0, stream, p);              \
+      break;                                                                   \
+    case 24:                                                                   \
+      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 24, R16_, true>),         \
+                         dim3(grid), dim3(kBlock), 0, stream, p);              \
+      break;                                                                   \
+    case 32:                                                                   \
+      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 32, R16_, true>),         \
+                         dim3(grid), dim3(kBlock), 0, stream, p);              \
       break;                                                                   \
     default:                                                                   \
       return hipErrorInvalidValue;                                             \

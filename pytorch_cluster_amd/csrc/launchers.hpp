@@ -183,11 +183,22 @@ size_t knn_feat_scratch_bytes(int n, int m, int d, int num_segments, int k);
 // r16 = 1 / 2: x and y hold fp16 / bf16 rows (knn_feat16_supported shapes
 // only; scratch: knn_feat16_scratch_bytes); the results are those of the
 // reference's kernel for that element type.
+// radius: the radius search instead (fp32 rows, radius_feat_supported shapes;
+// k = max_num_neighbors, out.dist NULL; scratch as for kNN with that k).
+struct FeatRadius {
+  float r2;
+  bool ignore_same;
+};
 hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
                            const int *work_start, void *scratch,
                            const DenseResult &out, hipEvent_t time_start,
                            hipEvent_t time_stop, hipStream_t stream,
-                           int r16 = 0);
+                           int r16 = 0, const FeatRadius *radius = nullptr);
+// Feature-space radius search through the matrix-core filter
+// (knn_feat_small_impl.hpp): fp32, 8 < d <= 128, at most 32 neighbours per
+// query, and enough pairs to pay for the preparation; PCA_RADIUS_FEAT=0:
+// never, 1: whenever the shape fits.
+bool radius_feat_supported(int n, int m, int d, int num_segments, int slots);
 // Whether launch_knn_feat serves such a call (fp32 rows) with its one-kernel
 // search, which counts the edges itself (compact_hints applies).
 bool knn_feat_one_kernel(int n, int d, int num_segments, int k, bool cosine);

@@ -1,0 +1,7 @@
+// Feature-space radius search in one kernel: 5 blocks of 16 components (up to 64 features),
+// fp32 rows.
+#include "knn_feat_small_impl.hpp"
+
+namespace pca {
+PCA_RADIUS_FEAT_DEFINE(5, 0)
+} // namespace pca

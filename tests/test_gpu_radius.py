@@ -216,3 +216,65 @@ def test_graph_orientation_in_the_output_pass(oracle, radius_path, flow, loop):
     got = pca.radius_graph(dev(x), 0.12, dev(batch), loop=loop, flow=flow,
                            max_num_neighbors=9)
     assert got.cpu().numpy().tolist() == want.tolist()
+
+
+# ---- feature space: the matrix-core filter in front of the exact distances
+# (knn_feat_small_impl.hpp, RADIUS) against the plain scan and the checker
+
+def _feature_case(rng, kind, n, m, d):
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    y = rng.standard_normal((m, d)).astype(np.float32)
+    if kind == "rows_as_queries":
+        y[: m // 2] = x[rng.integers(0, n, m // 2)]
+    elif kind == "clusters":
+        c = rng.standard_normal((30, d)).astype(np.float32)
+        x = (c[rng.integers(0, 30, n)] +
+             0.3 * rng.standard_normal((n, d))).astype(np.float32)
+        y = (c[rng.integers(0, 30, m)] +
+             0.3 * rng.standard_normal((m, d))).astype(np.float32)
+    elif kind == "duplicates":
+        x = x[rng.integers(0, 50, n)]
+        y = x[rng.integers(0, n, m)].copy()
+    elif kind == "large_rows":
+        x[rng.integers(0, n, 4)] *= 1e4
+        y[[1, m - 1]] *= 1e5
+    elif kind == "not_finite":
+        x[7, 2] = np.nan
+        x[n // 3] = np.inf
+        y[3, 0] = np.nan
+    return x, y
+
+
+@pytest.mark.parametrize("kind", ["plain", "rows_as_queries", "clusters",
+                                  "duplicates", "large_rows", "not_finite"])
+@pytest.mark.parametrize("d", [9, 24, 64, 100, 128])
+def test_feature_space_parity(oracle, monkeypatch, kind, d):
+    monkeypatch.setenv("PCA_RADIUS_FEAT", "1")
+    rng = np.random.default_rng(d * 13 + len(kind))
+    n, m = 2600, 420
+    x, y = _feature_case(rng, kind, n, m, d)
+    ptr_x = np.array([0, 40, 40, 1500, n])
+    ptr_y = np.array([0, 30, 50, 300, m])
+    # radii from "a handful of neighbours" to "more than the limit"
+    base = float(np.sqrt(2.0 * d)) if kind not in ("clusters", "duplicates") \
+        else 0.45 * float(np.sqrt(d))
+    for r, cap, ignore in ((0.8 * base, 32, False), (0.9 * base, 5, False),
+                           (1.1 * base, 32, False), (0.7 * base, 17, True),
+                           (1e-3, 8, False)):
+        got = gpu_radius(x, y, ptr_x, ptr_y, r, cap, ignore)
+        want = oracle.radius_op(x, y, ptr_x, ptr_y, r, cap, 1, ignore)
+        assert got.shape == want.shape, (r, cap)
+        assert (got == want).all(), (r, cap)
+
+
+def test_feature_space_graph_is_the_plain_scan_s(monkeypatch):
+    # 20 clouds of 900 points with 64 features, as a graph layer asks for
+    # them: the default path against the plain scan of the library
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(20 * 900, 64, generator=g).to(DEV)
+    batch = torch.arange(20, device=DEV).repeat_interleave(900)
+    a = pca.radius_graph(x, 9.2, batch, max_num_neighbors=32, batch_size=20)
+    monkeypatch.setenv("PCA_RADIUS_FEAT", "0")
+    b = pca.radius_graph(x, 9.2, batch, max_num_neighbors=32, batch_size=20)
+    assert a.shape == b.shape and a.shape[1] > 20 * 900
+    assert bool((a == b).all())
