@@ -771,6 +771,10 @@ hipError_t launch_knn_anytype(int dtype, const SearchInput &in, int k,
   }
 }
 
+float narrow_r2_16bit(double r2, bool bf16) {
+  return bf16 ? R16Traits<true>::narrow_r2(r2) : R16Traits<false>::narrow_r2(r2);
+}
+
 hipError_t launch_radius_anytype(int dtype, const SearchInput &in, double r,
                                  bool ignore_same_index,
                                  const int *work_start, int task_bound,

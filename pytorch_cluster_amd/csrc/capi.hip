@@ -213,6 +213,12 @@ size_t radius_workspace(int64_t n, int64_t m, int64_t d, int64_t num_segments,
                                       (int)num_segments, (int)slots))
     bytes += pca::knn_feat_scratch_bytes((int)n, (int)m, (int)d,
                                          (int)num_segments, (int)slots);
+  else if ((dtype == PCA_F16 || dtype == PCA_BF16) &&
+           pca::radius_feat_supported((int)n, (int)m, (int)d,
+                                      (int)num_segments, (int)slots,
+                                      dtype == PCA_F16 ? 1 : 2))
+    bytes += pca::knn_feat16_scratch_bytes((int)n, (int)m, (int)d,
+                                           (int)num_segments, (int)slots);
   bytes += align256(sizeof(int) * (size_t)(num_segments + 1));
   bytes += align256(sizeof(int) * (size_t)m * (size_t)slots);
   bytes += align256(sizeof(int) * (size_t)m);
@@ -776,18 +782,22 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
   const bool matrix_cores =
       dtype == PCA_F32 &&
       pca::radius_mc_supported((int)d, (int)n, (int)m, (int)num_segments);
-  const bool feature_space = !matrix_cores && dtype == PCA_F32 &&
-                             pca::radius_feat_supported(
-                                 (int)n, (int)m, (int)d, (int)num_segments,
-                                 (int)slots);
+  const int r16 = dtype == PCA_F16 ? 1 : (dtype == PCA_BF16 ? 2 : 0);
+  const bool feature_space =
+      !matrix_cores && (dtype == PCA_F32 || r16 != 0) &&
+      pca::radius_feat_supported((int)n, (int)m, (int)d, (int)num_segments,
+                                 (int)slots, r16);
   Carver ws(workspace);
   void *packed_rows = nullptr;
   if (matrix_cores)
     packed_rows =
         ws.take<char>(pca::radius_mc_scratch_bytes((int)n, (int)d));
   else if (feature_space)
-    packed_rows = ws.take<char>(pca::knn_feat_scratch_bytes(
-        (int)n, (int)m, (int)d, (int)num_segments, (int)slots));
+    packed_rows = ws.take<char>(
+        r16 != 0 ? pca::knn_feat16_scratch_bytes((int)n, (int)m, (int)d,
+                                                 (int)num_segments, (int)slots)
+                 : pca::knn_feat_scratch_bytes((int)n, (int)m, (int)d,
+                                               (int)num_segments, (int)slots));
   int *work_start = ws.take<int>((size_t)num_segments + 1);
   pca::DenseResult dense;
   dense.idx = ws.take<int>((size_t)m * slots);
@@ -826,10 +836,12 @@ int pca_radius(const void *x, const void *y, const int64_t *ptr_x,
   if (matrix_cores || feature_space)
     pca::compact_hints(dense, (int)m, compact_ws, false);
   if (feature_space) {
-    const pca::FeatRadius radius{r2, ignore_same_index != 0};
+    const pca::FeatRadius radius{
+        r16 != 0 ? pca::narrow_r2_16bit(r * r, r16 == 2) : r2,
+        ignore_same_index != 0};
     rc = check_launch(pca::launch_knn_feat(in, (int)slots, false, work_start,
                                            packed_rows, dense, timer.start,
-                                           timer.stop, stream, 0, &radius),
+                                           timer.stop, stream, r16, &radius),
                       "knn_feat_small_kernel (radius)");
     timer.stop = nullptr;
   } else if (matrix_cores)

@@ -55,6 +55,12 @@ PCA_DECLARE_FEAT_SMALL_BLOCKS(9, 2)
 PCA_DECLARE_RADIUS_FEAT_BLOCKS(3, 0)
 PCA_DECLARE_RADIUS_FEAT_BLOCKS(5, 0)
 PCA_DECLARE_RADIUS_FEAT_BLOCKS(9, 0)
+PCA_DECLARE_RADIUS_FEAT_BLOCKS(3, 1)
+PCA_DECLARE_RADIUS_FEAT_BLOCKS(5, 1)
+PCA_DECLARE_RADIUS_FEAT_BLOCKS(9, 1)
+PCA_DECLARE_RADIUS_FEAT_BLOCKS(3, 2)
+PCA_DECLARE_RADIUS_FEAT_BLOCKS(5, 2)
+PCA_DECLARE_RADIUS_FEAT_BLOCKS(9, 2)
 #undef PCA_DECLARE_RADIUS_FEAT_BLOCKS
 
 namespace {
@@ -644,8 +650,10 @@ bool knn_feat_one_kernel(int n, int d, int num_segments, int k, bool cosine) {
          feat_small_applies(n, d, num_segments, k, cosine);
 }
 
-bool radius_feat_supported(int n, int m, int d, int num_segments, int slots) {
-  const bool fits = d > 8 && d <= 128 && slots >= 1 && slots <= 32;
+bool radius_feat_supported(int n, int m, int d, int num_segments, int slots,
+                           int r16) {
+  const bool fits =
+      d > 8 && d <= (r16 == 2 ? 64 : 128) && slots >= 1 && slots <= 32;
   if (const char *env = std::getenv("PCA_RADIUS_FEAT")) {
     if (env[0] == '0')
       return false;
@@ -683,7 +691,7 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
                            hipEvent_t time_stop, hipStream_t stream,
                            int r16, const FeatRadius *radius) {
   SearchInput in = in_given;
-  if (radius != nullptr && (r16 != 0 || cosine))
+  if (radius != nullptr && cosine)
     return hipErrorInvalidValue;
   if (r16 != 0) {
     // 16-bit rows: searched as fp32 rows (the widening is exact) by the one
@@ -860,8 +868,13 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
     if (time_start)
       (void)hipEventRecord(time_start, stream);
 #define PCA_SMALL_CASE(NB)                                                     \
-  err = radius     ? launch_radius_feat_blocks<NB, 0>(p, kbucket, tiles_bound, \
-                                                      stream)                  \
+  err = radius                                                                 \
+            ? (r16 == 0   ? launch_radius_feat_blocks<NB, 0>(                  \
+                                p, kbucket, tiles_bound, stream)               \
+               : r16 == 1 ? launch_radius_feat_blocks<NB, 1>(                  \
+                                p, kbucket, tiles_bound, stream)               \
+                          : launch_radius_feat_blocks<NB, 2>(                  \
+                                p, kbucket, tiles_bound, stream))              \
         : r16 == 0 ? launch_knn_feat_small_blocks<NB, 0>(p, kbucket,           \
                                                          tiles_bound, stream)  \
         : r16 == 1 ? launch_knn_feat_small_blocks<NB, 1>(p, kbucket,           \

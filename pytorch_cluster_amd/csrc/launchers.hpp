@@ -183,8 +183,9 @@ size_t knn_feat_scratch_bytes(int n, int m, int d, int num_segments, int k);
 // r16 = 1 / 2: x and y hold fp16 / bf16 rows (knn_feat16_supported shapes
 // only; scratch: knn_feat16_scratch_bytes); the results are those of the
 // reference's kernel for that element type.
-// radius: the radius search instead (fp32 rows, radius_feat_supported shapes;
-// k = max_num_neighbors, out.dist NULL; scratch as for kNN with that k).
+// radius: the radius search instead (radius_feat_supported shapes;
+// k = max_num_neighbors, out.dist NULL; scratch as for kNN with that k; r2
+// narrowed to the element type by the caller).
 struct FeatRadius {
   float r2;
   bool ignore_same;
@@ -195,10 +196,12 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
                            hipEvent_t time_stop, hipStream_t stream,
                            int r16 = 0, const FeatRadius *radius = nullptr);
 // Feature-space radius search through the matrix-core filter
-// (knn_feat_small_impl.hpp): fp32, 8 < d <= 128, at most 32 neighbours per
-// query, and enough pairs to pay for the preparation; PCA_RADIUS_FEAT=0:
-// never, 1: whenever the shape fits.
-bool radius_feat_supported(int n, int m, int d, int num_segments, int slots);
+// (knn_feat_small_impl.hpp): fp32 and fp16 rows of 8 < d <= 128 components,
+// bf16 rows of up to 64, at most 32 neighbours per query, and enough pairs to
+// pay for the preparation; PCA_RADIUS_FEAT=0: never, 1: whenever the shape
+// fits.  r16: 0 fp32, 1 fp16, 2 bf16.
+bool radius_feat_supported(int n, int m, int d, int num_segments, int slots,
+                           int r16 = 0);
 // Whether launch_knn_feat serves such a call (fp32 rows) with its one-kernel
 // search, which counts the edges itself (compact_hints applies).
 bool knn_feat_one_kernel(int n, int d, int num_segments, int k, bool cosine);
@@ -244,6 +247,9 @@ hipError_t launch_knn_anytype(int dtype, const SearchInput &in, int k,
                               const int *work_start, int grid_bound,
                               const DenseResult &out, hipStream_t stream,
                               void *scratch);
+// (scalar_t)(r * r) of the reference for fp16 / bf16 points
+// (csrc/cuda/radius_cuda.cu:90), as a float.
+float narrow_r2_16bit(double r2, bool bf16);
 hipError_t launch_radius_anytype(int dtype, const SearchInput &in, double r,
                                  bool ignore_same_index,
                                  const int *work_start, int task_bound,

@@ -217,6 +217,40 @@ def test_radius_other_dtypes_parity(oracle, dtype, d, cap, ignore):
     assert (got == want).all()
 
 
+@pytest.mark.parametrize("dtype,kind16", [(torch.float16, 0),
+                                          (torch.bfloat16, 1)])
+@pytest.mark.parametrize("kind", ["plain", "rows_as_queries", "duplicates",
+                                  "one_large_component", "overflow", "tiny",
+                                  "large_rows_and_queries", "not_finite",
+                                  "grid"])
+def test_radius_16bit_feature_space_parity(oracle, monkeypatch, dtype, kind16,
+                                           kind):
+    # the radius search on 16-bit rows of 9 to 128 components (bf16: 64)
+    # through the matrix-core filter, against the checker's 16-bit chain:
+    # radii around the typical distance, so that both "fewer than the limit"
+    # and "the first 32 in row order" occur
+    monkeypatch.setenv("PCA_RADIUS_FEAT", "1")
+    rng = np.random.default_rng(len(kind) * 5 + kind16)
+    dims = (9, 20, 64, 100, 128) if kind16 == 0 else (9, 20, 33, 64)
+    for d in dims:
+        n, m = 2600, 420
+        x, y = _knn16_case(rng, kind, n, m, d, dtype)
+        ptr_x = np.array([0, 40, 40, 1500, n])
+        ptr_y = np.array([0, 30, 50, 300, m])
+        scale = {"one_large_component": 60.0, "overflow": 25.0,
+                 "tiny": 2e-4}.get(kind, 1.0)
+        base = scale * float(np.sqrt(2.0 * d))
+        if kind == "one_large_component":
+            base = scale * 1.0
+        for r, cap, ignore in ((0.8 * base, 32, False), (1.05 * base, 9, True),
+                               (0.9 * base, 1, False)):
+            got = gpu_radius_t(x, y, ptr_x, ptr_y, r, cap, ignore)
+            want = oracle.radius_op16(bits(x), bits(y), ptr_x, ptr_y, r, cap,
+                                      ignore, kind16)
+            assert got.shape == want.shape, (d, r, cap)
+            assert (got == want).all(), (d, r, cap)
+
+
 def test_distances_only_for_fp32():
     x = torch.rand(10, 3, dtype=torch.float64, device=DEV)
     with pytest.raises(capi.PcaError, match="fp32 points only"):
