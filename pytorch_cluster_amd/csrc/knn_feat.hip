@@ -68,7 +68,7 @@ namespace {
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 // The one-kernel search (knn_feat_small_impl.hpp): Euclidean, up to 128
-// components, k <= 32, and examples of at most 8,192 rows on average.  Measured
+// components, k <= 48, and examples of at most 8,192 rows on average.  Measured
 // on clouds searched in themselves, k = 20, against the better of the two
 // staged searches: 32 x 1,024 x 64 0.25 / 0.51 ms, 16 x 2,048 x 128
 // 0.47 / 0.77, 4 x 8,192 x 64 0.54 / 0.81, 2 x 16,384 x 64 0.80 / 0.93,
@@ -77,8 +77,10 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 // with one wave per SIMD, and longer scans are worth the staged searches'
 // sharing of an example among workgroups.  PCA_KNN_FEAT_SMALL: 0 never, 1
 // whenever the shape fits.
+constexpr int kFeatSmallMaxK = 48; // widest list of the one-kernel search
+
 bool feat_small_applies(int n, int d, int num_segments, int k, bool cosine) {
-  const bool fits = !cosine && d <= 128 && k <= 32;
+  const bool fits = !cosine && d <= 128 && k <= kFeatSmallMaxK;
   if (const char *env = std::getenv("PCA_KNN_FEAT_SMALL")) {
     if (env[0] == '0')
       return false;
@@ -674,7 +676,8 @@ bool knn_feat16_supported(int n, int d, int num_segments, int k, bool cosine,
       return false;
   // (what 16-bit sums can lose grows with their length: at 128 components of
   // bf16 the cut would pass rows at twice the bound)
-  return !cosine && d > 8 && d <= (bf16 ? 64 : 128) && k <= 32 && n >= 1 &&
+  return !cosine && d > 8 && d <= (bf16 ? 64 : 128) && k <= kFeatSmallMaxK &&
+         n >= 1 &&
          num_segments >= 1;
 }
 
@@ -696,7 +699,7 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
   if (r16 != 0) {
     // 16-bit rows: searched as fp32 rows (the widening is exact) by the one
     // kernel that can compute the exact distances in the 16-bit arithmetic
-    if (cosine || in.d > 128 || k > 32)
+    if (cosine || in.d > 128 || k > kFeatSmallMaxK)
       return hipErrorInvalidValue;
     char *at = static_cast<char *>(scratch);
     float *x32 = reinterpret_cast<float *>(at);
@@ -860,7 +863,8 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
     p.self_pos = out.self_pos;
     p.kept = out.kept;
     // one exact kernel: nothing is listed, merged, refined or searched again
-    const int kbucket = k <= 8 ? 8 : (k <= 16 ? 16 : (k <= 24 ? 24 : 32));
+    // (in steps of 8: the lists' padding in front is at most 7 entries)
+    const int kbucket = (k + 7) / 8 * 8;
     if (radius != nullptr) {
       p.r2 = radius->r2;
       p.ignore_same = radius->ignore_same ? 1 : 0;

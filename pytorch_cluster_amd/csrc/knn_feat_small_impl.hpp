@@ -1,5 +1,5 @@
 // Feature-space kNN for examples of up to some ten thousand rows (8 < d <= 128,
-// k <= 32, Euclidean): ONE kernel, exact in itself.  It computes what
+// k <= 48, Euclidean): ONE kernel, exact in itself.  It computes what
 // knn_kernel of the reference computes (csrc/cuda/knn_cuda.cu:30-84), bit for
 // bit, with the fp16 lower bound of knn_feat_impl.hpp as its filter.
 //
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   constexpr int SEEDS = K / 2;
   constexpr int DEPTH = 4; // tiles in flight
   static_assert(kSmallQueue % DEPTH == 0, "drains fall between groups of tiles");
-  static_assert(K % 8 == 0 && K <= 32, "list widths 8, 16, 24, 32");
+  static_assert(K % 8 == 0 && K <= 48, "list widths in steps of 8, up to 48");
   static_assert(kBlock == 256 && TQ == 128, "four waves of 32 queries");
 
   __shared__ __attribute__((aligned(16))) uint4 xs[2][TILE_UNITS];
@@ -808,6 +808,14 @@ hipError_t launch_knn_feat_small_blocks(const KnnFeatParams &p, int kbucket,
       break;                                                                   \
     case 32:                                                                   \
       hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 32, R16_>), dim3(grid),   \
+                         dim3(kBlock), 0, stream, p);                          \
+      break;                                                                   \
+    case 40:                                                                   \
+      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 40, R16_>), dim3(grid),   \
+                         dim3(kBlock), 0, stream, p);                          \
+      break;                                                                   \
+    case 48:                                                                   \
+      hipLaunchKernelGGL((knn_feat_small_kernel<NB_, 48, R16_>), dim3(grid),   \
                          dim3(kBlock), 0, stream, p);                          \
       break;                                                                   \
     default:                                                                   \

@@ -154,7 +154,7 @@ def test_knn_16bit_feature_space_parity(oracle, dtype, kind16, kind):
         x, y = _knn16_case(rng, kind, n, m, d, dtype)
         ptr_x = np.array([0, 40, 40, 1500, n])
         ptr_y = np.array([0, 30, 50, 300, m])
-        for k in ((1, 20) if d % 2 else (8, 32)):
+        for k in ((1, 20, 41) if d % 2 else (8, 32, 48)):
             got = gpu_knn_t(x, y, ptr_x, ptr_y, k)
             want, _ = oracle.knn_op16(bits(x), bits(y), ptr_x, ptr_y, k, False,
                                       kind16)

@@ -2,7 +2,7 @@
 each of the three searches behind it: the four-wave first stage
 (knn_feat_impl.hpp), the eight-wave first stage (knn_feat_wide_impl.hpp, up to
 128 components), and the one-kernel search for examples of moderate size
-(knn_feat_small_impl.hpp: Euclidean, up to 128 components, k <= 32; other
+(knn_feat_small_impl.hpp: Euclidean, up to 128 components, k <= 48; other
 calls fall through to the stages).  Parity with the CPU checker where the
 mechanisms of that path are exercised -- lists that overflow (near-duplicates:
 the flagged queries go through the second pass), rows and queries the filter
@@ -24,7 +24,7 @@ def first_stage(request, monkeypatch):
     """Which search serves the calls of a test: the four-wave kernel with its
     register lists, (where the shape fits: up to 128 components) the
     eight-wave kernel with candidate buffers, or (Euclidean, up to 128
-    components, k <= 32) the one kernel that needs no second stage.  Left to
+    components, k <= 48) the one kernel that needs no second stage.  Left to
     itself the library takes the last one for examples of up to 8,192 rows on
     average, else the eight-wave stage from 4,096 queries on."""
     if request.param == "one_kernel":
@@ -45,7 +45,7 @@ def _only_once_beyond_128(first_stage, d):
 def _one_kernel(first_stage, d, k, cosine=False):
     """Whether the one-kernel search serves such a call: it keeps no
     candidate lists, so nothing is ever handed to a second pass."""
-    return first_stage == "one_kernel" and not cosine and d <= 128 and k <= 32
+    return first_stage == "one_kernel" and not cosine and d <= 128 and k <= 48
 
 
 def _seed(*parts):
@@ -319,12 +319,12 @@ def test_one_kernel_search_shapes(oracle, first_stage, d):
     y = rng.standard_normal((ptr_y[-1], d)).astype(np.float32)
     y[:200] = x[rng.integers(0, len(x), 200)]      # distance zero, ties
     x[3000:3040] = x[2990]                         # equal rows: row numbers
-    for k in (1, 7, 8, 9, 16, 20, 24, 25, 32):
+    for k in (1, 7, 8, 9, 16, 20, 24, 25, 32, 33, 41, 48):
         _run(oracle, x, y, ptr_x, ptr_y, k)
     # rows far larger than the rest, one in an example too short for a bound
     # (every row of it is evaluated; the large one must not be listed twice)
     x[[1000, 3120]] *= 1e5
-    for k in (5, 20, 32):
+    for k in (5, 20, 32, 47):
         _run(oracle, x, y, ptr_x, ptr_y, k)
 
 
