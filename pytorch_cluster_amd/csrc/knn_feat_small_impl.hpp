@@ -600,7 +600,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
         pending = word & 0xffffu;
         step_row = (int)(word >> 16) * TILE;
       }
-      on = pending != 0;
+      // (radius search: a lane that holds its k hits looks no further)
+      on = pending != 0 && !(RADIUS && full);
       const int v = __builtin_clz(pending | 1u) - 16;
       pending &= ~(0x8000u >> v);
       g = min(x_begin + (on ? step_row + row_of(v) : 0), p.n - 1);
