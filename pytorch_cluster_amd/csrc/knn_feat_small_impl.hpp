@@ -27,8 +27,8 @@
 //      lower bound of the scaled distance e / sigma^2 the reference computes
 //      (knn_feat_impl.hpp), so every row with e below a bound has s <= bound /
 //      sigma^2 - shift =: cut.  A lane parks the rows under its cut (one word
-//      per step: step and 16-bit mask); every 16 steps all waves turn to
-//      their parked rows: in rounds of one row per lane the rows are fetched
+//      per step: step and 16-bit mask); when a queue is about to fill up,
+//      and at the end, all waves turn to their parked rows: in rounds of one row per lane the rows are fetched
 //      from global memory (four lanes per 64-byte line, handed to the owner
 //      through LDS), evaluated exactly, and enter the lane's sorted list of
 //      (distance, row) keys; the list's k-th distance and the partner's
@@ -154,7 +154,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   constexpr int TQ = kFeatQueries;
   constexpr int SEEDS = K / 2;
   constexpr int DEPTH = 4; // tiles in flight
-  static_assert(kSmallQueue % DEPTH == 0, "drains fall between groups of tiles");
+  static_assert(kSmallQueue % DEPTH == 0 && kSmallQueue >= 3 * DEPTH,
+                "a queue outlasts two looks");
   static_assert(K % 8 == 0 && K <= 48, "list widths in steps of 8, up to 48");
   static_assert(kBlock == 256 && TQ == 128, "four waves of 32 queries");
 
@@ -167,6 +168,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   // to row: neighbouring rows fall on distinct banks)
   __shared__ __attribute__((aligned(16))) small_v4f gathered[kBlock / kWave][kWave][5];
   __shared__ int wave_full[kBlock / kWave];
+  // what the waves said at the last two looks at their queues (see the search)
+  __shared__ int wave_says[2][kBlock / kWave];
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -178,6 +181,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   const int tile = blockIdx.x;
   if (tile >= total_tiles)
     return;
+  if (tid < 2 * (kBlock / kWave))
+    (&wave_says[0][0])[tid] = 0; // (a barrier follows before the first look)
   const int seg = find_segment(p.work_start, p.num_segments, tile);
   const int x_begin = p.ptr_x ? (int)p.ptr_x[seg] : 0;
   const int x_end = p.ptr_x ? (int)p.ptr_x[seg + 1] : p.n;
@@ -365,8 +370,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   auto row_of = [&](int v) { return 8 * (v >> 2) + 4 * half + (v & 3); };
 
   // One pass over the example's tiles; body(t, buf, rows) with the tile in
-  // LDS, every() after each kSmallQueue tiles and after the last one (true:
-  // the pass ends there).  (One
+  // LDS, every(group, last) after each DEPTH tiles (true: the pass ends
+  // there).  (One
   // barrier per tile: a buffer is overwritten a whole tile after its last
   // reader passed the barrier before.)  Slot t % DEPTH of the registers
   // holds tile t + 1 until it is stored, then tile t + 1 + DEPTH.
@@ -394,9 +399,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
           __syncthreads();
         }
       });
-      if (((t0 + DEPTH) & (kSmallQueue - 1)) == 0 || t0 + DEPTH >= count)
-        if (every())
-          break; // (uniform)
+      if (every(t0 / DEPTH, t0 + DEPTH >= count))
+        break; // (uniform)
     }
   };
 
@@ -456,10 +460,10 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
     const int sampled = min(num_tiles, kSmallSampleSteps);
     if (vec4)
       for_tiles(sampled, std::true_type(), std::true_type(), sample_step,
-                [] { return false; });
+                [](int, bool) { return false; });
     else
       for_tiles(sampled, std::true_type(), std::false_type(), sample_step,
-                [] { return false; });
+                [](int, bool) { return false; });
     // the ceil(k / 2)-th smallest sample of this lane and of its partner
     const int mine = (k + 1) / 2 - 1;
     float own = __builtin_inff();
@@ -575,9 +579,9 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   };
   // Parked steps: a lane with rows under its cut parks (step, mask); the
   // rows are evaluated exactly -- from global memory: by then their tile has
-  // left LDS -- by all lanes together, in rounds, every kSmallQueue steps and
-  // at the end (the bound from the sampled rows is tight from the start, so
-  // nothing is lost by looking late).
+  // left LDS -- by all lanes together, in rounds, when a queue is about to
+  // fill up and at the end (the bound from the sampled rows is tight from the
+  // start, so nothing is lost by looking late).
   int qn = 0;
   // (with -DPCA_FEAT_STATS: rounds of the waves, lanes that had a row in a
   // round, lanes whose row was kept -> FeatGlobals::stats[0..2])
@@ -712,18 +716,35 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
         ++qn;
       }
     }
-  }, [&] {
-    drain();
+  }, [&](int group, bool last) {
+    // All waves turn to their parked rows together (a wave on its own would
+    // keep the others waiting at the tiles' barriers), and only when it is
+    // time: at the end, and when some lane's queue could fill up before the
+    // next but one look -- a lane parks at most one word per tile, and what
+    // the waves say here is read at the next look, DEPTH tiles and as many
+    // barriers later.  Long scans with a tight cut park little: their drains
+    // are few and their rounds well filled.
+    bool go = last;
+#pragma unroll
+    for (int w = 0; w < kBlock / kWave; ++w)
+      go = go || wave_says[(group & 1) ^ 1][w] != 0;
+    if (go)
+      drain();
+    const int want = __any(qn > kSmallQueue - 2 * DEPTH) ? 1 : 0;
+    if (lane == 0)
+      wave_says[group & 1][wave] = want;
     if constexpr (RADIUS) {
-      // a workgroup whose queries all have their k hits leaves the scan
-      const int all_full = __any(!full) ? 0 : 1;
-      if (lane == 0)
-        wave_full[wave] = all_full;
-      __syncthreads();
-      const bool stop = (wave_full[0] & wave_full[1] & wave_full[2] &
-                         wave_full[3]) != 0;
-      __syncthreads();
-      return stop;
+      if (go) { // (uniform; hits only come in with a drain)
+        // a workgroup whose queries all have their k hits leaves the scan
+        const int all_full = __any(!full) ? 0 : 1;
+        if (lane == 0)
+          wave_full[wave] = all_full;
+        __syncthreads();
+        const bool stop = (wave_full[0] & wave_full[1] & wave_full[2] &
+                           wave_full[3]) != 0;
+        __syncthreads();
+        return stop;
+      }
     }
     return false;
   });
