@@ -318,7 +318,7 @@ class Cases:
 
     # the shape of a dynamic-graph layer of a point-cloud network: many small
     # clouds searched in themselves in feature space (one kernel that needs
-    # no second stage: examples of up to 8,192 rows, d <= 128, k <= 48)
+    # no second stage: examples of moderate length, d <= 128, k <= 48)
     def case_clouds64(self, reps):
         t, pca = self.torch, self.pca
         clouds, points, d, k = 32, 1024, 64, 20

@@ -543,7 +543,7 @@ int knn_call(const void *x, const void *y, const int64_t *ptr_x,
       r16 != 0 && pca::knn_feat16_supported((int)n, (int)d, (int)num_segments,
                                             (int)k, cosine != 0, r16 == 2);
   // (so does the one-kernel feature-space search)
-  if (feat16 || (feat && pca::knn_feat_one_kernel((int)n, (int)d,
+  if (feat16 || (feat && pca::knn_feat_one_kernel((int)n, (int)m, (int)d,
                                                    (int)num_segments, (int)k,
                                                    cosine != 0)))
     pca::compact_hints(dense, (int)m, compact_ws,

@@ -68,18 +68,28 @@ namespace {
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 // The one-kernel search (knn_feat_small_impl.hpp): Euclidean, up to 128
-// components, k <= 48, and examples of at most 8,192 rows on average.  Measured
-// on clouds searched in themselves, k = 20, against the better of the two
-// staged searches: 32 x 1,024 x 64 0.25 / 0.51 ms, 16 x 2,048 x 128
-// 0.47 / 0.77, 4 x 8,192 x 64 0.54 / 0.81, 2 x 16,384 x 64 0.80 / 0.93,
-// 4 x 16,384 x 128 2.33 / 1.67, 1 x 32,768 x 64 1.25 / 1.14, 1 x 65,536 x 64
-// 3.9 / 2.3: a workgroup of this kernel goes over its whole example, twice,
-// with one wave per SIMD, and longer scans are worth the staged searches'
-// sharing of an example among workgroups.  PCA_KNN_FEAT_SMALL: 0 never, 1
-// whenever the shape fits.
+// components, k <= 48, examples of moderate length.  A workgroup of that
+// kernel (128 queries) goes over its whole example, twice, with a compute unit
+// to itself and one wave per SIMD; the staged searches share an example among
+// workgroups and keep the matrix cores busier, but a call of theirs is a
+// dozen launches and every piece of a scan starts its lists cold.  Measured on
+// clouds searched in themselves, k = 20, one kernel / the better staged
+// search, whole calls in ms:
+//   32 x 1,024 x 64   0.22 / 0.51     256 x 1,024 x 64   1.29 / 2.00
+//   64 x 2,048 x 64   0.93 / 1.20     128 x 2,048 x 64   1.79 / 2.23
+//   8 x 4,096 x 64    0.39 / 0.62     64 x 4,096 x 64    2.57 / 2.51
+//   32 x 4,096 x 128  2.07 / 1.83     4 x 8,192 x 64     0.52 / 0.77
+//   8 x 8,192 x 128   1.73 / 1.62     16 x 8,192 x 32    1.33 / 1.01
+//   2 x 16,384 x 64   0.77 / 0.91     4 x 16,384 x 128   2.17 / 1.62
+//   1 x 32,768 x 64   1.19 / 1.12     1 x 65,536 x 64    3.81 / 2.25
+// Hence: examples of up to 2,048 rows on average always; up to 4,096 rows
+// while the workgroups fit the device at once (256) or the rows have at most
+// 64 components; up to 8,192 rows while the workgroups fit at once.
+// PCA_KNN_FEAT_SMALL: 0 never, 1 whenever the shape fits.
 constexpr int kFeatSmallMaxK = 48; // widest list of the one-kernel search
 
-bool feat_small_applies(int n, int d, int num_segments, int k, bool cosine) {
+bool feat_small_applies(int n, int m, int d, int num_segments, int k,
+                        bool cosine) {
   const bool fits = !cosine && d <= 128 && k <= kFeatSmallMaxK;
   if (const char *env = std::getenv("PCA_KNN_FEAT_SMALL")) {
     if (env[0] == '0')
@@ -87,7 +97,11 @@ bool feat_small_applies(int n, int d, int num_segments, int k, bool cosine) {
     if (env[0] == '1')
       return fits;
   }
-  return fits && (long long)n <= 8192LL * num_segments;
+  const long long rows = n, segments = num_segments > 0 ? num_segments : 1;
+  const bool at_once = (m + kFeatQueries - 1) / kFeatQueries <= 256;
+  return fits && (rows <= 2048 * segments ||
+                  (rows <= 4096 * segments && (at_once || d <= 64)) ||
+                  (rows <= 8192 * segments && at_once));
 }
 
 // list width for k neighbours: k + 16 real entries
@@ -647,9 +661,10 @@ void launch_widen16(const void *src, size_t count, bool bf16, float *dst,
 
 } // namespace
 
-bool knn_feat_one_kernel(int n, int d, int num_segments, int k, bool cosine) {
+bool knn_feat_one_kernel(int n, int m, int d, int num_segments, int k,
+                         bool cosine) {
   return knn_feat_supported(d, k, cosine) &&
-         feat_small_applies(n, d, num_segments, k, cosine);
+         feat_small_applies(n, m, d, num_segments, k, cosine);
 }
 
 bool radius_feat_supported(int n, int m, int d, int num_segments, int slots,
@@ -748,7 +763,8 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
   const int nb = feat_blocks(in.d);
 
   const bool small = r16 != 0 || radius != nullptr ||
-                     feat_small_applies(in.n, in.d, in.num_segments, k, cosine);
+                     feat_small_applies(in.n, in.m, in.d, in.num_segments, k,
+                                        cosine);
   hipLaunchKernelGGL(feat_init_kernel, dim3((in.m + kBlock - 1) / kBlock),
                      dim3(kBlock), 0, stream, globals, tau, in.m, hit_count,
                      redo_cap, overflow, small ? out.edge_sums : nullptr,

@@ -204,7 +204,8 @@ bool radius_feat_supported(int n, int m, int d, int num_segments, int slots,
                            int r16 = 0);
 // Whether launch_knn_feat serves such a call (fp32 rows) with its one-kernel
 // search, which counts the edges itself (compact_hints applies).
-bool knn_feat_one_kernel(int n, int d, int num_segments, int k, bool cosine);
+bool knn_feat_one_kernel(int n, int m, int d, int num_segments, int k,
+                         bool cosine);
 // fp16 / bf16 rows through the matrix-core filter (knn_feat_small_impl.hpp):
 // Euclidean, 8 < d <= 128 (bf16: 64), k <= 48; PCA_KNN_FEAT_16BIT=0: never.
 bool knn_feat16_supported(int n, int d, int num_segments, int k, bool cosine,
