@@ -46,6 +46,9 @@ PCA_DECLARE_FEAT_SMALL_BLOCKS(9, 1)
 PCA_DECLARE_FEAT_SMALL_BLOCKS(3, 2)
 PCA_DECLARE_FEAT_SMALL_BLOCKS(5, 2)
 PCA_DECLARE_FEAT_SMALL_BLOCKS(9, 2)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(3, 3)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(5, 3)
+PCA_DECLARE_FEAT_SMALL_BLOCKS(9, 3)
 #undef PCA_DECLARE_FEAT_SMALL_BLOCKS
 
 #define PCA_DECLARE_RADIUS_FEAT_BLOCKS(NB, R16)                                \
@@ -67,8 +70,8 @@ namespace {
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
-// The one-kernel search (knn_feat_small_impl.hpp): Euclidean, up to 128
-// components, k <= 48, examples of moderate length.  A workgroup of that
+// The one-kernel search (knn_feat_small_impl.hpp): up to 128 components,
+// k <= 48, examples of moderate length.  A workgroup of that
 // kernel (128 queries) goes over its whole example, twice, with a compute unit
 // to itself and one wave per SIMD; the staged searches share an example among
 // workgroups and keep the matrix cores busier, but a call of theirs is a
@@ -90,7 +93,7 @@ constexpr int kFeatSmallMaxK = 48; // widest list of the one-kernel search
 
 bool feat_small_applies(int n, int m, int d, int num_segments, int k,
                         bool cosine) {
-  const bool fits = !cosine && d <= 128 && k <= kFeatSmallMaxK;
+  const bool fits = d <= 128 && k <= kFeatSmallMaxK;
   if (const char *env = std::getenv("PCA_KNN_FEAT_SMALL")) {
     if (env[0] == '0')
       return false;
@@ -250,7 +253,7 @@ __global__ __launch_bounds__(kBlock) void feat_rows_kernel(
   // (with a histogram the scale is made from it, feat_scale_kernel: the
   // first couple of thousand workgroups of a launch all find this word at
   // zero, and their maxima on one word took 20 us)
-  if (threadIdx.x == 0 && hist == nullptr) {
+  if (threadIdx.x == 0 && hist == nullptr && g != nullptr) {
     for (int w = 1; w < kBlock / kWave; ++w)
       big = part[w] > big ? part[w] : big;
     // (one word for the whole call: only workgroups that raise it go there)
@@ -780,10 +783,12 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
     // exact distances
     (void)launch_row_norms(xf, in.n, in.d, x_norm, stream);
     (void)launch_row_norms(yf, in.m, in.d, y_norm, stream);
+    // (no scale to make: the rows are normalised one by one)
     hipLaunchKernelGGL(feat_rows_kernel,
                        dim3((in.n + rows_per_block - 1) / rows_per_block),
                        dim3(kBlock), 0, stream, xf, in.n, in.d, x_class,
-                       globals, static_cast<unsigned *>(nullptr),
+                       static_cast<FeatGlobals *>(nullptr),
+                       static_cast<unsigned *>(nullptr),
                        static_cast<unsigned *>(nullptr));
   } else {
     // (the classification buffer is free here: it holds every row's largest
@@ -895,6 +900,8 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
                                 p, kbucket, tiles_bound, stream)               \
                           : launch_radius_feat_blocks<NB, 2>(                  \
                                 p, kbucket, tiles_bound, stream))              \
+        : cosine   ? launch_knn_feat_small_blocks<NB, 3>(p, kbucket,           \
+                                                         tiles_bound, stream)  \
         : r16 == 0 ? launch_knn_feat_small_blocks<NB, 0>(p, kbucket,           \
                                                          tiles_bound, stream)  \
         : r16 == 1 ? launch_knn_feat_small_blocks<NB, 1>(p, kbucket,           \

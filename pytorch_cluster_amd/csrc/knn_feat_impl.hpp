@@ -206,7 +206,17 @@ __device__ __forceinline__ FeatQuery feat_query(const float *yrow, int d,
                                                 float norm_in) {
   FeatQuery fq;
   if (COSINE) {
-    fq.dead = !(norm_in > 0.0f);
+    // A query of zeros has no neighbours (0 / 0).  A norm of zero over
+    // components that are not all zero -- their squares underflowed -- still
+    // divides a dot product that need not be zero: the reference returns the
+    // rows with a positive one at distance -inf.  That query is left to the
+    // exact evaluation of every row, like the other norms the filter cannot
+    // take.
+    bool nonzero = false;
+    if (norm_in == 0.0f)
+      for (int c = 0; c < d; ++c)
+        nonzero = nonzero || yrow[c] != 0.0f;
+    fq.dead = !(norm_in > 0.0f) && !nonzero;
     // (below kFeatCosTiny the reference's own products underflow too much
     // for the margin Ec)
     fq.odd = !fq.dead &&
@@ -347,9 +357,16 @@ __global__ __launch_bounds__(kBlock) void feat_pack_kernel(
         }
       }
     }
+    // (cosine: also a row whose norm underflowed to zero over components
+    // that are not all zero -- its dot products need not be zero, and the
+    // reference divides them by that zero)
+    bool lost_norm = false;
+    if (COSINE && unit == 0 && nv == 0.0f)
+      for (int c = 0; c < d; ++c)
+        lost_norm = lost_norm || x[(size_t)row * d + c] != 0.0f;
     if (unit == 0 &&
         (cv == __builtin_inff() || (cv == cv && nv == __builtin_inff()) ||
-         (COSINE && nv > 0.0f && nv < kFeatCosTiny)))
+         (COSINE && nv > 0.0f && nv < kFeatCosTiny) || lost_norm))
       atomicAdd(&g->odd_rows, 1);
     if (unit < S::UNITS - 2) {
       if (usable) {

@@ -1,0 +1,7 @@
+// Feature-space kNN of moderate examples in one exact kernel: 5 blocks of 16 components (up to 64 features),
+// cosine distance of fp32 rows.
+#include "knn_feat_small_impl.hpp"
+
+namespace pca {
+PCA_KNN_FEAT_SMALL_DEFINE(5, 3)
+} // namespace pca

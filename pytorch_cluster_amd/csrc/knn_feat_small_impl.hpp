@@ -1,5 +1,5 @@
 // Feature-space kNN for examples of up to some ten thousand rows (8 < d <= 128,
-// k <= 48, Euclidean): ONE kernel, exact in itself.  It computes what
+// k <= 48, Euclidean or cosine): ONE kernel, exact in itself.  It computes what
 // knn_kernel of the reference computes (csrc/cuda/knn_cuda.cu:30-84), bit for
 // bit, with the fp16 lower bound of knn_feat_impl.hpp as its filter.
 //
@@ -57,7 +57,7 @@
 // kernel on the rows widened to fp32, with the reference's 16-bit arithmetic
 // in the exact distances (SmallChain) and a cut widened by what that
 // arithmetic can lose against the distance in real numbers -- 3 % at 64
-// components of fp16, 6 % at 128; 23 % at 64 components of bf16.
+// components of fp16, 7 % at 128; 30 % at 64 components of bf16.
 #pragma once
 
 #include <type_traits>
@@ -90,7 +90,9 @@ __device__ __forceinline__ void static_for(F &&f) {
 
 // The arithmetic of the exact distances.  R16 = 0: fp32 rows, one fused
 // multiply-add per component (csrc/cuda/knn_cuda.cu:61-64 as a GPU compiler
-// builds it).  R16 = 1 / 2: the rows were fp16 / bf16 (widened to fp32 for
+// builds it); R16 = 3: the cosine distance of fp32 rows, 1 - x.y / (|x| |y|)
+// with the dot product as such a chain (csrc/cuda/knn_cuda.cu:9-28).
+// R16 = 1 / 2: the rows were fp16 / bf16 (widened to fp32 for
 // this kernel, which is exact) and the reference computes in c10::Half /
 // c10::BFloat16: every difference, square and sum is formed in fp32 and
 // rounded to 16 bits (torch/headeronly/util/Half.h:501-560); the sentinel
@@ -105,12 +107,15 @@ template <int R16> struct SmallChain {
       const float dc = x - y;
       return __builtin_fmaf(dc, dc, acc);
     }
+    if (R16 == 3) // (the cosine distance: the dot product, fp32 rows)
+      return __builtin_fmaf(x, y, acc);
     const float dc = round_to_16<R16 == 2>(x - y);
     const float sq = round_to_16<R16 == 2>(dc * dc);
     return round_to_16<R16 == 2>(acc + sq);
   }
   static __device__ __forceinline__ float sentinel() {
-    return R16 == 0 ? kKnnSentinel : round_to_16<R16 == 2>(1e10f);
+    return (R16 == 0 || R16 == 3) ? kKnnSentinel
+                                  : round_to_16<R16 == 2>(1e10f);
   }
   // A 16-bit chain value H and the distance D in real numbers: with
   // u = 2^-11 (2^-8) + 2^-23 per rounded operation (the fp32 operation, then
@@ -121,7 +126,7 @@ template <int R16> struct SmallChain {
   // D < (h + slack()) * widen(d); the factor also carries (1 + (d + 2) 2^-24)
   // for the fp32 chain the filter's bound was proven against.
   static __device__ __forceinline__ double widen(int d) {
-    if (R16 == 0)
+    if (R16 == 0 || R16 == 3)
       return 1.0;
     const double u = (R16 == 2 ? 1.0 / 256.0 : 1.0 / 2048.0) + 1.0 / 8388608.0;
     double keep = 1.0;
@@ -130,13 +135,21 @@ template <int R16> struct SmallChain {
     return (1.0 + (double)(d + 2) * (1.0 / 16777216.0)) / keep * (1.0 + 1e-9);
   }
   static __device__ __forceinline__ double slack(int d) {
-    if (R16 == 0)
+    if (R16 == 0 || R16 == 3)
       return 0.0;
     // fp16: squares below 2^-14 round to multiples of 2^-24; bf16: squares
     // below 2^-126 may be flushed altogether
     return (double)d * (R16 == 2 ? 1.1754943508222875e-38 : 1.0 / 16777216.0);
   }
 };
+
+// The next float above v (any sign; v finite).
+__device__ __forceinline__ float small_next_up(float v) {
+  if (v == 0.0f)
+    return 1.401298464324817e-45f;
+  const uint32_t u = __float_as_uint(v);
+  return __uint_as_float(v > 0.0f ? u + 1u : u - 1u);
+}
 
 template <int NB, int K, int R16 = 0, bool RADIUS = false>
 __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
@@ -219,8 +232,12 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   __syncthreads();
   const float *const my_y = &ys[(wave * 32 + col) * ROW_F];
 
-  const float inv_sigma = feat_inv_sigma(p.globals->max_bits);
-  const FeatQuery fq = feat_query<false>(my_y, d, inv_sigma, 1.0f);
+  constexpr bool COSINE = R16 == 3;
+  static_assert(!(COSINE && RADIUS), "no radius search by cosine distance");
+  const float ynorm = COSINE && valid ? p.y_norm[q] : 1.0f;
+  const float inv_sigma =
+      COSINE ? 1.0f : feat_inv_sigma(p.globals->max_bits);
+  const FeatQuery fq = feat_query<COSINE>(my_y, d, inv_sigma, ynorm);
   // active: the query searches (a NaN component: no neighbours).  filtered:
   // it does so with the fp16 lower bound; if the filter cannot take the query
   // (a component beyond the range the scale was made for) or some row of x
@@ -228,8 +245,18 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   const bool active = valid && !fq.dead;
   const bool filtered = active && !fq.odd && p.globals->odd_rows == 0;
   const float sentinel = Chain::sentinel();
-  const double scale2 = (double)inv_sigma * (double)inv_sigma;
-  const float y_scale = -2.0f * inv_sigma;
+  const double scale2 =
+      COSINE ? kFeatCosScale : (double)inv_sigma * (double)inv_sigma;
+  const float y_scale = COSINE ? -1024.0f / ynorm : -2.0f * inv_sigma;
+  // what the reference makes of a chain's value and row g (the cosine
+  // distance divides the dot product by the norms)
+  auto finish = [&](float acc, int g) {
+    if (COSINE) {
+      acc = acc / (p.x_norm[g] * ynorm);
+      acc = 1.0f - acc;
+    }
+    return acc;
+  };
   const int seg_len = x_end - x_begin;
   const int num_tiles = (seg_len + TILE - 1) / TILE;
 
@@ -423,7 +450,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
 #pragma unroll
     for (int j = 0; j < SEEDS; ++j)
       seed[j] = __builtin_inff();
-    auto sample_step = [&](int, int buf, int rows) {
+    auto sample_step = [&](int t, int buf, int rows) {
       const feat_acc_t acc = products(buf);
       // the smallest of the lane's 16 values, its accumulator number in the
       // four lowest bits (which of two nearly equal rows is taken does not
@@ -446,7 +473,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       const float least = __builtin_fminf(m0, m3);
       const int v = (int)(__float_as_uint(least) & 15u);
       const int j = row_of(v);
-      const float e = exact(buf, j);
+      const float e =
+          finish(exact(buf, j), min(x_begin + t * TILE + j, p.n - 1));
       // (a padding row, a NaN or a distance beyond the limit is no sample)
       const float sample =
           (active && j < rows && least < __builtin_inff() && e < sentinel)
@@ -478,7 +506,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
     const float partner = __uint_as_float(half ? both[0] : both[1]);
     const float bound = __builtin_fmaxf(own, partner);
     if (active && bound < sentinel) {
-      shared = next_up_positive(bound);
+      shared = small_next_up(bound);
       thresh = __builtin_fminf(thresh, shared);
     }
   }
@@ -514,7 +542,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
     const float partner_mid = __uint_as_float(half ? mids[0] : mids[1]);
     partner = __builtin_fminf(partner, __builtin_fmaxf(mid, partner_mid));
     if (active && partner < sentinel) {
-      shared = __builtin_fminf(shared, next_up_positive(partner));
+      shared = __builtin_fminf(shared, small_next_up(partner));
       thresh = __builtin_fminf(thresh, shared);
     }
   };
@@ -657,7 +685,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
         gather_chunk(next, g_next, f0_next);
         acc = chain_chunk(now, f0, acc);
         if (last) {
-          take(acc, g, on);
+          take(finish(acc, g), g, on);
           acc = 0.0f;
           more = __any(on_next);
         }
@@ -675,7 +703,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       }
     } else {
       while (__any(on)) {
-        take(exact_unaligned(g), g, on);
+        take(finish(exact_unaligned(g), g), g, on);
         pop(g, on);
       }
     }
@@ -762,6 +790,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       for (int c = 0; c < d; ++c) {
         e = Chain::step(xr[c], my_y[c], e);
       }
+      e = finish(e, g);
       // (a query without a bound -- fewer sampled rows than it takes -- cuts
       // nowhere and has met the row among its parked ones already: the same
       // key in its list or in the partner's)

@@ -167,7 +167,17 @@ __global__ __launch_bounds__(kBlock) void mfma_pack_rows_kernel(
   // coordinates enter scaled by `scale` (0: not at all); `aug` is w
   float scale, aug;
   if (COSINE) {
-    if (!(nv > 0.0f)) { // a NaN distance anyway: never a candidate
+    // (a norm of zero over components that are not all zero: their squares
+    // underflowed, the dot products need not be zero, and the reference
+    // divides them by that zero)
+    bool lost_norm = false;
+    if (nv == 0.0f)
+      for (int c = 0; c < d; ++c)
+        lost_norm = lost_norm || x[(size_t)row * d + c] != 0.0f;
+    if (lost_norm) { // always looked at
+      scale = 0.0f;
+      aug = -1e38f;
+    } else if (!(nv > 0.0f)) { // a NaN distance anyway: never a candidate
       scale = 0.0f;
       aug = 1.7e38f;
     } else if (nv == __builtin_inff()) { // always looked at
@@ -326,7 +336,13 @@ __global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfm
   bool y_blind;    // true: the query can have no neighbours at all
   float y_scale;
   if (COSINE) {
-    y_blind = !(ynorm > 0.0f); // 0 or NaN: every distance is NaN
+    // 0 or NaN: every distance is NaN -- unless the norm is zero only
+    // because the squares underflowed: then the dot products still count
+    bool lost_norm = false;
+    if (ynorm == 0.0f)
+      for (int c = 0; c < d; ++c)
+        lost_norm = lost_norm || yrow[c] != 0.0f;
+    y_blind = !(ynorm > 0.0f) && !lost_norm;
     y_filtered = !y_blind && ynorm < __builtin_inff();
     y_scale = y_filtered ? -1.0f / ynorm : 0.0f;
   } else {

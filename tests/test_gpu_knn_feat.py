@@ -2,7 +2,7 @@
 each of the three searches behind it: the four-wave first stage
 (knn_feat_impl.hpp), the eight-wave first stage (knn_feat_wide_impl.hpp, up to
 128 components), and the one-kernel search for examples of moderate size
-(knn_feat_small_impl.hpp: Euclidean, up to 128 components, k <= 48; other
+(knn_feat_small_impl.hpp: up to 128 components, k <= 48; other
 calls fall through to the stages).  Parity with the CPU checker where the
 mechanisms of that path are exercised -- lists that overflow (near-duplicates:
 the flagged queries go through the second pass), rows and queries the filter
@@ -23,8 +23,8 @@ pytestmark = pytest.mark.gpu
 def first_stage(request, monkeypatch):
     """Which search serves the calls of a test: the four-wave kernel with its
     register lists, (where the shape fits: up to 128 components) the
-    eight-wave kernel with candidate buffers, or (Euclidean, up to 128
-    components, k <= 48) the one kernel that needs no second stage.  Left to
+    eight-wave kernel with candidate buffers, or (up to 128 components,
+    k <= 48) the one kernel that needs no second stage.  Left to
     itself the library takes the last one for examples of up to 2,048 rows on
     average (up to 8,192 while its workgroups fit the device at once), else the eight-wave stage from 4,096 queries on."""
     if request.param == "one_kernel":
@@ -45,7 +45,7 @@ def _only_once_beyond_128(first_stage, d):
 def _one_kernel(first_stage, d, k, cosine=False):
     """Whether the one-kernel search serves such a call: it keeps no
     candidate lists, so nothing is ever handed to a second pass."""
-    return first_stage == "one_kernel" and not cosine and d <= 128 and k <= 48
+    return first_stage == "one_kernel" and d <= 128 and k <= 48
 
 
 def _seed(*parts):
@@ -219,6 +219,30 @@ def test_rows_and_queries_the_filter_cannot_represent(oracle, first_stage):
     odd, flagged = _flagged_queries(x, yb, 12)
     assert odd == 0 and flagged == (1 if lists else 0)
     _run(oracle, x, yb, None, None, 12)
+
+
+@pytest.mark.parametrize("case", ["rows", "queries", "both", "one_of_each"])
+def test_cosine_norms_that_underflow_to_zero(oracle, case):
+    # components below 1e-23: every square underflows, the norm is exactly
+    # zero, yet the dot product with an ordinary vector is not -- the
+    # reference divides it by that zero and returns the rows with a positive
+    # dot product at distance -inf.  Vectors of zeros have no neighbours.
+    rng = np.random.default_rng(_seed("lost norms", case))
+    d, n, m, k = 40, 2500, 300, 12
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    y = rng.standard_normal((m, d)).astype(np.float32)
+    if case in ("rows", "both"):
+        x *= np.float32(1e-25)
+    if case in ("queries", "both"):
+        y *= np.float32(1e-25)
+    if case == "one_of_each":
+        x[17] *= np.float32(1e-25)
+        y[5] *= np.float32(1e-25)
+    x[3] = 0.0
+    y[8] = 0.0
+    ptr_x = np.array([0, 1200, n])
+    ptr_y = np.array([0, 100, m])
+    _run(oracle, x, y, ptr_x, ptr_y, k, cosine=True)
 
 
 @pytest.mark.parametrize("case", ["tiny", "huge", "mixed", "outlier",
