@@ -23,6 +23,13 @@ template <bool BF16> __device__ __forceinline__ float round_to_16(float v) {
   return (float)(_Float16)v;
 }
 
+// Smallest norm of a row or query the cosine filters take: below it the
+// squares and products of the reference's own chains reach the denormal range
+// (a few bits each), the distance it computes strays from the cosine by
+// whole per cents, and no margin of a filter holds; such vectors are always
+// evaluated exactly.
+constexpr float kCosTinyNorm = 1e-18f;
+
 // Distance every kNN slot starts from; a candidate must be strictly below it
 // to be returned (csrc/cuda/knn_cuda.cu:48,68 in the reference).
 constexpr float kKnnSentinel = 1e10f;

@@ -174,7 +174,7 @@ __global__ __launch_bounds__(kBlock) void mfma_pack_rows_kernel(
     if (nv == 0.0f)
       for (int c = 0; c < d; ++c)
         lost_norm = lost_norm || x[(size_t)row * d + c] != 0.0f;
-    if (lost_norm) { // always looked at
+    if (lost_norm || (nv > 0.0f && nv < kCosTinyNorm)) { // always looked at
       scale = 0.0f;
       aug = -1e38f;
     } else if (!(nv > 0.0f)) { // a NaN distance anyway: never a candidate
@@ -343,7 +343,7 @@ __global__ __launch_bounds__(kBlock, K > 48 ? 2 : 1) void knn_mfma_kernel(KnnMfm
       for (int c = 0; c < d; ++c)
         lost_norm = lost_norm || yrow[c] != 0.0f;
     y_blind = !(ynorm > 0.0f) && !lost_norm;
-    y_filtered = !y_blind && ynorm < __builtin_inff();
+    y_filtered = !y_blind && ynorm < __builtin_inff() && ynorm >= kCosTinyNorm;
     y_scale = y_filtered ? -1.0f / ynorm : 0.0f;
   } else {
     y_blind = false;

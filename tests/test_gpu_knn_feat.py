@@ -245,6 +245,24 @@ def test_cosine_norms_that_underflow_to_zero(oracle, case):
     _run(oracle, x, y, ptr_x, ptr_y, k, cosine=True)
 
 
+@pytest.mark.parametrize("d,k", [(9, 1), (12, 8), (40, 20)])
+def test_cosine_norms_in_the_denormal_range_of_their_squares(oracle, d, k):
+    # components around 1e-21: squares and products are denormal numbers of a
+    # few bits, the reference's distance strays from the cosine by per cents,
+    # and only an evaluation in its own arithmetic finds its neighbours (a
+    # filter with any margin made for normal numbers does not)
+    rng = np.random.default_rng(_seed("denormal squares", d, k))
+    n, m = 6000, 500
+    centres = rng.standard_normal((60, d))
+    x = centres[rng.integers(0, 60, n)] + 0.05 * rng.standard_normal((n, d))
+    y = centres[rng.integers(0, 60, m)] + 0.05 * rng.standard_normal((m, d))
+    x = (x * 1e-21).astype(np.float32)
+    y = (y * 1e-21).astype(np.float32)
+    _run(oracle, x, y, None, None, k, cosine=True)
+    _run(oracle, x, y, np.array([0, 2500, n]), np.array([0, 200, m]), k,
+         cosine=True)
+
+
 @pytest.mark.parametrize("case", ["tiny", "huge", "mixed", "outlier",
                                   "zeros", "sparse"])
 def test_scales_at_both_ends(oracle, case):
