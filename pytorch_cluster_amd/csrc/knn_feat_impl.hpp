@@ -125,7 +125,8 @@ constexpr double kFeatCosScale = 1048576.0; // 2^20
 __host__ __device__ __forceinline__ double feat_cos_err(int d) {
   return feat_rho(d) * kFeatCosScale;
 }
-constexpr float kFeatCosTiny = kCosTinyNorm; // smallest norm the cosine filter takes
+// smallest norm the cosine filter takes
+constexpr float kFeatCosTiny = kCosTinyNorm;
 
 __host__ __device__ __forceinline__ double feat_c0(int d) {
   return (double)d * (1.0 / 4096.0);

@@ -28,10 +28,10 @@
 //      (knn_feat_impl.hpp), so every row with e below a bound has s <= bound /
 //      sigma^2 - shift =: cut.  A lane parks the rows under its cut (one word
 //      per step: step and 16-bit mask); when a queue is about to fill up,
-//      and at the end, all waves turn to their parked rows: in rounds of one row per lane the rows are fetched
-//      from global memory (four lanes per 64-byte line, handed to the owner
-//      through LDS), evaluated exactly, and enter the lane's sorted list of
-//      (distance, row) keys; the list's k-th distance and the partner's
+//      and at the end, all waves turn to their parked rows: in rounds of one
+//      row per lane the rows are fetched from global memory (four lanes per
+//      64-byte line, handed to the owner through LDS), evaluated exactly, and
+//      enter the lane's sorted list of (distance, row) keys; the list's k-th distance and the partner's
 //      tighten the bound as in the low-dimensional kernel.  About 1.5 k rows
 //      per query get that far.  Nothing is approximate in what is KEPT, and
 //      every row that could be kept is looked at: no candidate list, no second
@@ -179,7 +179,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   __shared__ uint32_t queue[kSmallQueue][kBlock];
   // per wave: 16 components of 64 gathered rows (five 16-byte units from row
   // to row: neighbouring rows fall on distinct banks)
-  __shared__ __attribute__((aligned(16))) small_v4f gathered[kBlock / kWave][kWave][5];
+  __shared__ __attribute__((aligned(16)))
+  small_v4f gathered[kBlock / kWave][kWave][5];
   __shared__ int wave_full[kBlock / kWave];
   // what the waves said at the last two looks at their queues (see the search)
   __shared__ int wave_says[2][kBlock / kWave];
@@ -511,7 +512,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
     }
   }
 
-  // ---- 2. the search ----------------------------------------------------------
+  // ---- 2. the search -------------------------------------------------------
   // s below cut: the row's distance may lie below thresh (a strict test
   // against feat_float_above(c) admits everything up to c = thresh / sigma^2
   // - shift)

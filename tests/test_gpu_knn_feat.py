@@ -26,7 +26,8 @@ def first_stage(request, monkeypatch):
     eight-wave kernel with candidate buffers, or (up to 128 components,
     k <= 48) the one kernel that needs no second stage.  Left to
     itself the library takes the last one for examples of up to 2,048 rows on
-    average (up to 8,192 while its workgroups fit the device at once), else the eight-wave stage from 4,096 queries on."""
+    average (up to 8,192 while its workgroups fit the device at once), else
+    the eight-wave stage from 4,096 queries on."""
     if request.param == "one_kernel":
         monkeypatch.setenv("PCA_KNN_FEAT_SMALL", "1")
         monkeypatch.delenv("PCA_KNN_FEAT_WIDE", raising=False)
