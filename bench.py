@@ -329,16 +329,39 @@ class Cases:
         ms, out = _median_ms(t, fn, reps or 10)
         kms = _search_ms(t, self.capi, self.events, fn)
         blocks = _feat_shape(d, k)[0]
-        return {"knn_graph 32x1024 points x 64 features k=20": {
+        flop = 2 * d * clouds * points * points
+        detail = ("algorithmic 2*D flop per pair against the dense fp16 "
+                  "matrix peak; one workgroup per 128 queries goes over its "
+                  "cloud (twice for kNN: bound, then search) with one wave "
+                  "per SIMD: a latency case, 4 GFLOP per call")
+        report = {"knn_graph 32x1024 points x 64 features k=20": {
             "ms": ms, "queries_per_s": x.shape[0] / ms * 1e3,
             "edges": int(out.shape[1]),
             "roofline": _roofline(
-                "knn_feat_small_kernel<%d,24>" % blocks, kms,
-                2 * d * clouds * points * points, PEAK_BF16_TFLOPS, "mfma",
-                "algorithmic 2*D flop per pair against the dense fp16 matrix "
-                "peak; one workgroup per 128 queries goes over its cloud "
-                "twice with one wave per SIMD: a latency case, 4 GFLOP per "
-                "call")}}
+                "knn_feat_small_kernel<%d,24>" % blocks, kms, flop,
+                PEAK_BF16_TFLOPS, "mfma", detail)}}
+        # the same clouds: rows in fp16 (the reference's 16-bit arithmetic
+        # behind the same filter), cosine distance, radius search
+        variants = (
+            ("knn_graph 32x1024 points x 64 features k=20, fp16 rows",
+             "knn_feat_small_kernel<%d,24,1>" % blocks,
+             lambda h=x.half(): pca.knn_graph(h, k, b, batch_size=clouds)),
+            ("knn_graph 32x1024 points x 64 features k=20, cosine",
+             "knn_feat_small_kernel<%d,24,3>" % blocks,
+             lambda: pca.knn_graph(x, k, b, batch_size=clouds, cosine=True)),
+            ("radius_graph 32x1024 points x 64 features r=9 max 32",
+             "knn_feat_small_kernel<%d,32,0,true>" % blocks,
+             lambda: pca.radius_graph(x, 9.0, b, max_num_neighbors=32,
+                                      batch_size=clouds)))
+        for label, kernel, call in variants:
+            ms, out = _median_ms(t, call, reps or 10)
+            kms = _search_ms(t, self.capi, self.events, call)
+            report[label] = {
+                "ms": ms, "queries_per_s": x.shape[0] / ms * 1e3,
+                "edges": int(out.shape[1]),
+                "roofline": _roofline(kernel, kms, flop, PEAK_BF16_TFLOPS,
+                                      "mfma", detail)}
+        return report
 
     # nearest: every point of the LiDAR-like scans looks for the nearest of
     # its scan's every-8th point (the operator that follows the neighbour
