@@ -7,8 +7,9 @@
 Outputs (next to this file, git-ignored):
   libpca_neighbors.so   HIP kernels + the C ABI of include/pca_neighbors.h
   _torch_ops.so         TorchScript operator binding (links the above)
-  libpca_probe.so       csrc/probes/: measurement aids (`bench.py --probe`),
-                        no part of the searches
+  libpca_probe.so       csrc/probes/: measurement and checking aids
+                        (`bench.py --probe`, the bf16 rounding check of
+                        tests/test_gpu_dtypes.py), no part of the searches
 """
 import argparse
 import concurrent.futures

@@ -114,16 +114,17 @@ template <bool BF16> struct R16Traits {
       return __uint_as_float((uint32_t)v << 16);
     return __half2float(__ushort_as_half(v));
   }
+  // (the sums below end in comparisons only: round_in_chain)
   static __device__ __forceinline__ calc_t sq_step(calc_t x, calc_t y,
                                                    calc_t acc) {
-    const float d = round16(x - y);
-    const float p = round16(d * d);
-    return round16(acc + p);
+    const float d = round_in_chain<BF16>(x - y);
+    const float p = round_in_chain<BF16>(d * d);
+    return round_in_chain<BF16>(acc + p);
   }
   static __device__ __forceinline__ calc_t dot_step(calc_t x, calc_t y,
                                                     calc_t acc) {
-    const float p = round16(x * y);
-    return round16(acc + p);
+    const float p = round_in_chain<BF16>(x * y);
+    return round_in_chain<BF16>(acc + p);
   }
   static __device__ __forceinline__ calc_t norm(calc_t sq) {
     return round16(__builtin_sqrtf(sq));

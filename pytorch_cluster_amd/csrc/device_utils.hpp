@@ -14,13 +14,37 @@ constexpr int kBlock = 256; // 4 waves: one per SIMD of a CU
 // (torch/headeronly/util/Half.h:501-560, BFloat16.h).
 template <bool BF16> __device__ __forceinline__ float round_to_16(float v) {
   if (BF16) {
-    uint32_t x = __float_as_uint(v);
-    if ((x & 0x7fffffffu) > 0x7f800000u)
+    // the device's own conversion (v_cvt_pk_bf16_f32) and a shift: for every
+    // float that is not a NaN it returns the bits of c10's integer formula
+    // (x + 0x7fff + ((x >> 16) & 1), upper half), denormal numbers and the
+    // overflow to infinity included -- all 2^32 inputs are compared by
+    // pca_probe_bf16_rounding (csrc/probes/rounding_probe.hip); it keeps a
+    // NaN's sign and payload where c10 returns 0x7fc0, hence the first line
+    if (v != v)
       return __uint_as_float(0x7fc00000u);
-    x += 0x7fffu + ((x >> 16) & 1u);
-    return __uint_as_float(x & 0xffff0000u);
+    return (float)(__bf16)v;
   }
   return (float)(_Float16)v;
+}
+
+// The same inside a chain of operations whose end is only ever compared
+// (a NaN stays a NaN, whatever its sign and payload): two instructions fewer
+// per rounding for bfloat16.
+template <bool BF16> __device__ __forceinline__ float round_in_chain(float v) {
+  if (BF16)
+    return (float)(__bf16)v;
+  return (float)(_Float16)v;
+}
+
+// c10::BFloat16's rounding as the integer formula it is written as
+// (torch/headeronly/util/BFloat16.h round_to_nearest_even): the yardstick of
+// the comparison named above.
+__device__ __forceinline__ float round_to_bf16_by_integers(float v) {
+  uint32_t x = __float_as_uint(v);
+  if ((x & 0x7fffffffu) > 0x7f800000u)
+    return __uint_as_float(0x7fc00000u);
+  x += 0x7fffu + ((x >> 16) & 1u);
+  return __uint_as_float(x & 0xffff0000u);
 }
 
 // Smallest norm of a row or query the cosine filters take: below it the

@@ -109,9 +109,9 @@ template <int R16> struct SmallChain {
     }
     if (R16 == 3) // (the cosine distance: the dot product, fp32 rows)
       return __builtin_fmaf(x, y, acc);
-    const float dc = round_to_16<R16 == 2>(x - y);
-    const float sq = round_to_16<R16 == 2>(dc * dc);
-    return round_to_16<R16 == 2>(acc + sq);
+    const float dc = round_in_chain<R16 == 2>(x - y);
+    const float sq = round_in_chain<R16 == 2>(dc * dc);
+    return round_in_chain<R16 == 2>(acc + sq);
   }
   static __device__ __forceinline__ float sentinel() {
     return (R16 == 0 || R16 == 3) ? kKnnSentinel

@@ -255,3 +255,17 @@ def test_distances_only_for_fp32():
     x = torch.rand(10, 3, dtype=torch.float64, device=DEV)
     with pytest.raises(capi.PcaError, match="fp32 points only"):
         capi.knn_edges(x, x, None, None, 2, want_dist=True)
+
+
+def test_bf16_rounding_of_every_float():
+    """The 16-bit searches round to bfloat16 with the device's conversion
+    instruction; c10::BFloat16 (torch/headeronly/util/BFloat16.h,
+    round_to_nearest_even) is an integer formula.  The probe library compares
+    the two on all 2^32 bit patterns, NaNs included."""
+    import ctypes
+    import os
+    lib = ctypes.CDLL(os.path.join(os.path.dirname(pca.__file__),
+                                   "libpca_probe.so"))
+    out = (ctypes.c_ulonglong * 2)()
+    assert lib.pca_probe_bf16_rounding(out) == 0
+    assert out[0] == 0, "differs on %d floats, first 0x%08x" % (out[0], out[1])
