@@ -36,6 +36,58 @@ template <bool BF16> __device__ __forceinline__ float round_in_chain(float v) {
   return (float)(_Float16)v;
 }
 
+// What is left of a term of a sum in 16-bit arithmetic, at worst.  The
+// reference adds d squares (x_j - y_j)^2 one after the other and rounds the
+// difference, the square and every sum to 16 bits: a term has been rounded
+// 3 + e times when e sums lie behind it, so the value H the chain ends on is
+// at least  sum_j (1 - u)^(3 + d - j) (x_j - y_j)^2  minus what underflow takes
+// (u = 2^-11 for fp16, 2^-8 for bf16, plus 2^-23: the fp32 operation under
+// every rounding).  kChainKeep.s[bf16][e] is the square root of
+// (1 - u)^(3 + e), rounded DOWN to 13 (bf16: 16) significant bits: a number
+// of 11 (8) significant bits times such a factor is exact in fp32, so rows
+// and queries scaled by it component
+// by component have exactly  sum_j s_j^2 (x_j - y_j)^2 <= H + underflow  as
+// their squared distance -- the lower bound of the 16-bit searches' filter.
+constexpr int kChainKeepSums = 128; // sums behind a term: up to this many
+struct ChainKeep {
+  float s[2][kChainKeepSums + 1];
+};
+constexpr double chain_keep_root(double v) { // sqrt of v in (1/4, 1]
+  double r = v;
+  for (int i = 0; i < 64; ++i)
+    r = 0.5 * (r + v / r);
+  return r;
+}
+constexpr ChainKeep make_chain_keep() {
+  ChainKeep t{};
+  for (int b = 0; b < 2; ++b) {
+    const double u = (b ? 1.0 / 256.0 : 1.0 / 2048.0) + 1.0 / 8388608.0;
+    double keep = (1.0 - u) * (1.0 - u) * (1.0 - u);
+    for (int e = 0; e <= kChainKeepSums; ++e) {
+      // (1 - 2^-30: the root above is a double's, not the real number's)
+      const double root = chain_keep_root(keep) * (1.0 - 1.0 / 1073741824.0);
+      // root in [1/2, 1): 13 (16) bits behind the binary point, the first of
+      // them 1
+      const double unit = b ? 65536.0 : 8192.0;
+      const long long cut = (long long)(root * unit);
+      t.s[b][e] = (float)((double)cut / unit);
+      keep *= 1.0 - u;
+    }
+  }
+  return t;
+}
+__device__ constexpr ChainKeep kChainKeep = make_chain_keep();
+static_assert(make_chain_keep().s[1][kChainKeepSums] >= 0.5f &&
+                  make_chain_keep().s[0][0] < 1.0f,
+              "bits behind the point are significant bits");
+// the factor of component j of d (fp32 rows: 1)
+template <int R16>
+__device__ __forceinline__ float chain_keep(int d, int j) {
+  if (R16 == 1 || R16 == 2)
+    return kChainKeep.s[R16 - 1][d - j];
+  return 1.0f;
+}
+
 // c10::BFloat16's rounding as the integer formula it is written as
 // (torch/headeronly/util/BFloat16.h round_to_nearest_even): the yardstick of
 // the comparison named above.

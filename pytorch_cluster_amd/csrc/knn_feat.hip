@@ -639,27 +639,34 @@ size_t knn_feat_scratch_bytes(int n, int m, int d, int num_segments, int k) {
 
 namespace {
 
-// fp16 / bf16 rows as fp32 (exact)
+// fp16 / bf16 rows of d components as fp32 (exact) and, for the filter (kept
+// or null), with every component times chain_keep (exact as well)
 template <bool BF16>
 __global__ __launch_bounds__(kBlock) void widen16_kernel(
-    const uint16_t *__restrict__ src, size_t count, float *__restrict__ dst) {
+    const uint16_t *__restrict__ src, size_t count, int d,
+    float *__restrict__ dst, float *__restrict__ kept) {
   const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= count)
     return;
   const uint16_t v = src[i];
-  dst[i] = BF16 ? __uint_as_float((uint32_t)v << 16)
-                : (float)__builtin_bit_cast(_Float16, v);
+  const float wide = BF16 ? __uint_as_float((uint32_t)v << 16)
+                          : (float)__builtin_bit_cast(_Float16, v);
+  dst[i] = wide;
+  if (kept != nullptr)
+    kept[i] = wide * chain_keep<BF16 ? 2 : 1>(d, (int)(i % (size_t)d));
 }
 
-void launch_widen16(const void *src, size_t count, bool bf16, float *dst,
-                    hipStream_t stream) {
+void launch_widen16(const void *src, size_t count, int d, bool bf16,
+                    float *dst, float *kept, hipStream_t stream) {
   const unsigned grid = (unsigned)((count + kBlock - 1) / kBlock);
   if (bf16)
     hipLaunchKernelGGL(widen16_kernel<true>, dim3(grid), dim3(kBlock), 0,
-                       stream, static_cast<const uint16_t *>(src), count, dst);
+                       stream, static_cast<const uint16_t *>(src), count, d,
+                       dst, kept);
   else
     hipLaunchKernelGGL(widen16_kernel<false>, dim3(grid), dim3(kBlock), 0,
-                       stream, static_cast<const uint16_t *>(src), count, dst);
+                       stream, static_cast<const uint16_t *>(src), count, d,
+                       dst, kept);
 }
 
 } // namespace
@@ -701,7 +708,8 @@ bool knn_feat16_supported(int n, int d, int num_segments, int k, bool cosine,
 
 size_t knn_feat16_scratch_bytes(int n, int m, int d, int num_segments,
                                 int k) {
-  return align256(sizeof(float) * (size_t)n * d) +
+  // (x twice: as it is, and as the filter takes it)
+  return 2 * align256(sizeof(float) * (size_t)n * d) +
          align256(sizeof(float) * (size_t)m * d) +
          knn_feat_scratch_bytes(n, m, d, num_segments, k);
 }
@@ -714,6 +722,9 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
   SearchInput in = in_given;
   if (radius != nullptr && cosine)
     return hipErrorInvalidValue;
+  // the rows of x the filter is made from (16-bit rows: scaled, see
+  // chain_keep; else the rows themselves)
+  const float *x_for_filter = nullptr;
   if (r16 != 0) {
     // 16-bit rows: searched as fp32 rows (the widening is exact) by the one
     // kernel that can compute the exact distances in the 16-bit arithmetic
@@ -722,15 +733,21 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
     char *at = static_cast<char *>(scratch);
     float *x32 = reinterpret_cast<float *>(at);
     at += align256(sizeof(float) * (size_t)in.n * in.d);
+    float *x_kept = reinterpret_cast<float *>(at);
+    at += align256(sizeof(float) * (size_t)in.n * in.d);
     float *y32 = reinterpret_cast<float *>(at);
     at += align256(sizeof(float) * (size_t)in.m * in.d);
     scratch = at;
     const bool y_is_x = in.y == in.x && in.m == in.n;
-    launch_widen16(in.x, (size_t)in.n * in.d, r16 == 2, x32, stream);
+    launch_widen16(in.x, (size_t)in.n * in.d, in.d, r16 == 2, x32, x_kept,
+                   stream);
+    // (the search kernel scales the queries itself)
     if (!y_is_x)
-      launch_widen16(in.y, (size_t)in.m * in.d, r16 == 2, y32, stream);
+      launch_widen16(in.y, (size_t)in.m * in.d, in.d, r16 == 2, y32, nullptr,
+                     stream);
     in.x = x32;
     in.y = y_is_x ? x32 : y32;
+    x_for_filter = x_kept;
   }
   const FeatLayout lay =
       feat_layout(in.n, in.m, in.d, in.num_segments, k);
@@ -762,6 +779,7 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
   double *cand = reinterpret_cast<double *>(take(lay.cand));
 
   const float *xf = static_cast<const float *>(in.x);
+  const float *xp = x_for_filter != nullptr ? x_for_filter : xf;
   const float *yf = static_cast<const float *>(in.y);
   const int nb = feat_blocks(in.d);
 
@@ -796,7 +814,7 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
     x_big = reinterpret_cast<unsigned *>(x_class_buf);
     hipLaunchKernelGGL(feat_rows_kernel,
                        dim3((in.n + rows_per_block - 1) / rows_per_block),
-                       dim3(kBlock), 0, stream, xf, in.n, in.d, x_norm,
+                       dim3(kBlock), 0, stream, xp, in.n, in.d, x_norm,
                        globals, x_big, globals->hist_x);
     // (a cloud searched in itself: one pass over the rows serves both)
     const bool y_is_x = yf == xf && in.m == in.n;
@@ -813,23 +831,23 @@ hipError_t launch_knn_feat(const SearchInput &in_given, int k, bool cosine,
     hipError_t perr;
     switch (nb) {
     case 3:
-      perr = launch_feat_pack<3>(xf, x_norm, x_class, x_big, in.n, in.d,
+      perr = launch_feat_pack<3>(xp, x_norm, x_class, x_big, in.n, in.d,
                                  cosine, globals, x_pack, stream);
       break;
     case 5:
-      perr = launch_feat_pack<5>(xf, x_norm, x_class, x_big, in.n, in.d,
+      perr = launch_feat_pack<5>(xp, x_norm, x_class, x_big, in.n, in.d,
                                  cosine, globals, x_pack, stream);
       break;
     case 9:
-      perr = launch_feat_pack<9>(xf, x_norm, x_class, x_big, in.n, in.d,
+      perr = launch_feat_pack<9>(xp, x_norm, x_class, x_big, in.n, in.d,
                                  cosine, globals, x_pack, stream);
       break;
     case 17:
-      perr = launch_feat_pack<17>(xf, x_norm, x_class, x_big, in.n, in.d,
+      perr = launch_feat_pack<17>(xp, x_norm, x_class, x_big, in.n, in.d,
                                   cosine, globals, x_pack, stream);
       break;
     default:
-      perr = launch_feat_pack<33>(xf, x_norm, x_class, x_big, in.n, in.d,
+      perr = launch_feat_pack<33>(xp, x_norm, x_class, x_big, in.n, in.d,
                                   cosine, globals, x_pack, stream);
       break;
     }

@@ -201,7 +201,9 @@ struct FeatQuery {
 
 // Classification and bound constants of query row `yrow`.
 //   Euclid: `norm_in` unused.  cosine: the row's norm.
-template <bool COSINE>
+//   R16 = 1 / 2: the row takes part in the filter with every component times
+//   chain_keep<R16> (device_utils.hpp), as the rows of x were packed.
+template <bool COSINE, int R16 = 0>
 __device__ __forceinline__ FeatQuery feat_query(const float *yrow, int d,
                                                 float inv_sigma,
                                                 float norm_in) {
@@ -231,7 +233,7 @@ __device__ __forceinline__ FeatQuery feat_query(const float *yrow, int d,
   double ysq = 0.0;
   float top = 0.0f;
   for (int c = 0; c < d; ++c) {
-    const float v = yrow[c];
+    const float v = yrow[c] * chain_keep<R16>(d, c);
     chain = __builtin_fmaf(v, v, chain);
     const float scaled = v * inv_sigma;
     top = __builtin_fmaxf(top, __builtin_fabsf(scaled));

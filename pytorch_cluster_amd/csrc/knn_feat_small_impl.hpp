@@ -55,9 +55,10 @@
 //
 // fp16 and bf16 rows (knn_kernel<c10::Half>, <c10::BFloat16>): the same
 // kernel on the rows widened to fp32, with the reference's 16-bit arithmetic
-// in the exact distances (SmallChain) and a cut widened by what that
-// arithmetic can lose against the distance in real numbers -- 3 % at 64
-// components of fp16, 7 % at 128; 30 % at 64 components of bf16.
+// in the exact distances (SmallChain), and in the filter every component of
+// rows and queries times what that arithmetic leaves of its term at worst
+// (chain_keep: the first terms of the sum are rounded most often) -- the
+// filter's distance is then a lower bound of the reference's value.
 #pragma once
 
 #include <type_traits>
@@ -117,22 +118,21 @@ template <int R16> struct SmallChain {
     return (R16 == 0 || R16 == 3) ? kKnnSentinel
                                   : round_to_16<R16 == 2>(1e10f);
   }
-  // A 16-bit chain value H and the distance D in real numbers: with
-  // u = 2^-11 (2^-8) + 2^-23 per rounded operation (the fp32 operation, then
-  // the rounding to 16 bits), three operations on a term and at most d sums
-  // behind it, H >= D (1 - u)^(d + 3) - d t, t what a square can lose below
-  // the normal range (differences and sums there are exact: multiples of the
-  // smallest number of the format).  Hence H < h only if
-  // D < (h + slack()) * widen(d); the factor also carries (1 + (d + 2) 2^-24)
-  // for the fp32 chain the filter's bound was proven against.
+  // A 16-bit chain value H and the filter's distance D' -- the squared
+  // distance, in real numbers, of row and query with every component times
+  // chain_keep<R16> (device_utils.hpp: what the rounding of three operations
+  // on a term and of the sums behind it leaves of that term, at worst):
+  // H >= D' - d t, t what a square can lose below the normal range
+  // (differences and sums there are exact: multiples of the smallest number
+  // of the format).  Hence H < h only if D' < (h + slack()) * widen(d); the
+  // factor carries (1 + (d + 2) 2^-24) for the fp32 chain the filter's bound
+  // was proven against and 2 x 2^-24 more for the one case in which a scaled
+  // component is not exact (a bf16 component below 2^-125, next to one that
+  // is not).
   static __device__ __forceinline__ double widen(int d) {
     if (R16 == 0 || R16 == 3)
       return 1.0;
-    const double u = (R16 == 2 ? 1.0 / 256.0 : 1.0 / 2048.0) + 1.0 / 8388608.0;
-    double keep = 1.0;
-    for (int i = 0; i < d + 3; ++i)
-      keep *= 1.0 - u;
-    return (1.0 + (double)(d + 2) * (1.0 / 16777216.0)) / keep * (1.0 + 1e-9);
+    return (1.0 + (double)(d + 4) * (1.0 / 16777216.0)) * (1.0 + 1e-9);
   }
   static __device__ __forceinline__ double slack(int d) {
     if (R16 == 0 || R16 == 3)
@@ -238,7 +238,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
   const float ynorm = COSINE && valid ? p.y_norm[q] : 1.0f;
   const float inv_sigma =
       COSINE ? 1.0f : feat_inv_sigma(p.globals->max_bits);
-  const FeatQuery fq = feat_query<COSINE>(my_y, d, inv_sigma, ynorm);
+  const FeatQuery fq = feat_query<COSINE, R16>(my_y, d, inv_sigma, ynorm);
   // active: the query searches (a NaN component: no neighbours).  filtered:
   // it does so with the fp16 lower bound; if the filter cannot take the query
   // (a component beyond the range the scale was made for) or some row of x
@@ -272,7 +272,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         hb[e] = (filtered && cb + e < d)
-                    ? feat_h(my_y[min(cb + e, d - 1)] * y_scale)
+                    ? feat_h(my_y[min(cb + e, d - 1)] *
+                             chain_keep<R16>(d, min(cb + e, d - 1)) * y_scale)
                     : 0u;
     } else if (half == 0 && filtered) {
       hb[0] = 0x7800u; // 2^15

@@ -13,6 +13,8 @@ roundings alone leave the share of the budget that the header of
 knn_feat_impl.hpp reserves for accumulation (2^-22 x 2.01 of |X|^2 + |Y|^2 per
 term of the chain: 0.13 x 2^-10 at 256 components, 0.26 x 2^-10 at 512) unused.
 """
+import math
+
 import numpy as np
 import pytest
 
@@ -387,22 +389,57 @@ def _chain16(x, y, bf16):
     return acc
 
 
+def _chain_keep(bf16, sums):
+    """kChainKeep.s[bf16][sums] of csrc/device_utils.hpp, restated: the square
+    root of (1 - u)^(3 + sums), rounded down to 13 (bf16: 16) bits behind the
+    point."""
+    u = (2.0 ** -8 if bf16 else 2.0 ** -11) + 2.0 ** -23
+    root = math.sqrt((1.0 - u) ** (3 + sums)) * (1.0 - 2.0 ** -30)
+    unit = 65536.0 if bf16 else 8192.0
+    return math.floor(root * unit) / unit
+
+
 @pytest.mark.parametrize("bf16", [False, True])
-@pytest.mark.parametrize("kind", ["normal", "first_term_large", "tiny",
+def test_chain_keep_factors(bf16):
+    # below what the roundings leave of a term (in exact arithmetic), and
+    # short enough for a 16-bit number times the factor to be exact in fp32
+    from fractions import Fraction
+    u = (Fraction(1, 256) if bf16 else Fraction(1, 2048)) + Fraction(1, 2 ** 23)
+    rng = np.random.default_rng(stable_seed("keep", bf16))
+    v16 = _round16(rng.standard_normal(2000) *
+                   10.0 ** rng.integers(-6, 4, 2000), bf16)
+    for sums in range(0, 129):
+        s = _chain_keep(bf16, sums)
+        unit = 65536.0 if bf16 else 8192.0
+        assert 0.5 <= s < 1.0 and s * unit == int(s * unit)
+        assert Fraction(s) ** 2 <= (1 - u) ** (3 + sums)
+        # (not more than one part in 1,000 below it: the bound stays tight)
+        assert Fraction(s) ** 2 >= (1 - u) ** (3 + sums) * Fraction(999, 1000)
+        prod32 = (v16.astype(np.float32) * np.float32(s)).astype(np.float64)
+        assert (prod32 == v16.astype(np.float64) * s).all()
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("kind", ["normal", "first_term_large",
+                                  "last_term_large", "tiny",
                                   "mixed_scales", "grid", "decreasing"])
 def test_16bit_chain_against_the_real_distance(bf16, kind):
-    # the cut of the one-kernel search admits a row whenever its distance in
-    # real numbers D satisfies D < (h + d t) (1 - u)^-(d + 3): every row whose
-    # chain value H is below h must do so, i.e. H >= D (1 - u)^(d + 3) - d t
+    # the filter of the one-kernel search sees rows and queries with component
+    # j (of d) times chain_keep(d - j) and admits a row whenever that scaled
+    # distance D' satisfies D' < h + d t: every row whose chain value H is
+    # below h must do so, i.e. H >= D' - d t
     rng = np.random.default_rng(stable_seed("chain16", bf16, kind))
     u = (2.0 ** -8 if bf16 else 2.0 ** -11) + 2.0 ** -23
     t = 2.0 ** -126 if bf16 else 2.0 ** -24
-    for d in (9, 33, 64) + (() if bf16 else (128,)):
+    for d in (9, 33, 64, 128):
         x = rng.standard_normal((4000, d))
         y = rng.standard_normal(d)
         if kind == "first_term_large":
             x[:, 0] *= 40.0
             y[0] *= -40.0
+        elif kind == "last_term_large":
+            x[:, -1] *= 40.0
+            y[-1] *= -40.0
         elif kind == "tiny":
             x *= 3e-4
             y *= 3e-4
@@ -418,11 +455,16 @@ def test_16bit_chain_against_the_real_distance(bf16, kind):
         x16 = _round16(x, bf16)
         y16 = _round16(y, bf16)
         H = _chain16(x16, y16, bf16).astype(np.float64)
-        D = ((x16.astype(np.float64) - y16.astype(np.float64)) ** 2).sum(1)
+        keep = np.array([_chain_keep(bf16, d - j) for j in range(d)])
+        diff = x16.astype(np.float64) - y16.astype(np.float64)
+        D = (diff ** 2).sum(1)
+        scaled = ((keep * diff) ** 2).sum(1)
         finite = np.isfinite(H)
         assert finite.any()
-        lower = D * (1.0 - u) ** (d + 3) - d * t
-        assert (H[finite] >= lower[finite]).all(), (d, kind)
+        assert (H[finite] >= scaled[finite] - d * t).all(), (d, kind)
+        # the scaled distance is the tighter of the two bounds (but for the
+        # bits the factors were cut to)
+        assert (scaled >= D * (1.0 - u) ** (d + 3) * (1.0 - 2.0 ** -11)).all()
         # and the bound is not vacuous: the chain does lose something
         if kind in ("normal", "decreasing"):
             assert (H[finite] < D[finite]).any()
