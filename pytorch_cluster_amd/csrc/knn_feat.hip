@@ -680,7 +680,7 @@ bool knn_feat_one_kernel(int n, int m, int d, int num_segments, int k,
 bool radius_feat_supported(int n, int m, int d, int num_segments, int slots,
                            int r16) {
   const bool fits =
-      d > 8 && d <= (r16 == 2 ? 64 : 128) && slots >= 1 && slots <= 32;
+      d > 8 && d <= 128 && slots >= 1 && slots <= 32;
   if (const char *env = std::getenv("PCA_RADIUS_FEAT")) {
     if (env[0] == '0')
       return false;
@@ -699,9 +699,8 @@ bool knn_feat16_supported(int n, int d, int num_segments, int k, bool cosine,
   if (const char *env = std::getenv("PCA_KNN_FEAT_16BIT"))
     if (env[0] == '0')
       return false;
-  // (what 16-bit sums can lose grows with their length: at 128 components of
-  // bf16 the cut would pass rows at twice the bound)
-  return !cosine && d > 8 && d <= (bf16 ? 64 : 128) && k <= kFeatSmallMaxK &&
+  (void)bf16; // (both types up to 128 components)
+  return !cosine && d > 8 && d <= 128 && k <= kFeatSmallMaxK &&
          n >= 1 &&
          num_segments >= 1;
 }

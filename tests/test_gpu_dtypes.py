@@ -144,11 +144,11 @@ def _knn16_case(rng, kind, n, m, d, dtype):
                                   "large_rows_and_queries", "not_finite",
                                   "grid"])
 def test_knn_16bit_feature_space_parity(oracle, dtype, kind16, kind):
-    # 16-bit rows of 9 to 128 components (bf16: 64): the matrix-core filter in
+    # 16-bit rows of 9 to 128 components: the matrix-core filter in
     # front of the exact 16-bit chain (knn_feat_small_impl.hpp), against the
     # checker's chain; the 16-bit sums produce many equal distances
     rng = np.random.default_rng(len(kind) * 7 + kind16)
-    dims = (9, 20, 64, 100, 128) if kind16 == 0 else (9, 20, 33, 64)
+    dims = (9, 20, 64, 100, 128) if kind16 == 0 else (9, 33, 64, 100, 128)
     for d in dims:
         n, m = 2600, 420
         x, y = _knn16_case(rng, kind, n, m, d, dtype)
@@ -225,13 +225,13 @@ def test_radius_other_dtypes_parity(oracle, dtype, d, cap, ignore):
                                   "grid"])
 def test_radius_16bit_feature_space_parity(oracle, monkeypatch, dtype, kind16,
                                            kind):
-    # the radius search on 16-bit rows of 9 to 128 components (bf16: 64)
+    # the radius search on 16-bit rows of 9 to 128 components
     # through the matrix-core filter, against the checker's 16-bit chain:
     # radii around the typical distance, so that both "fewer than the limit"
     # and "the first 32 in row order" occur
     monkeypatch.setenv("PCA_RADIUS_FEAT", "1")
     rng = np.random.default_rng(len(kind) * 5 + kind16)
-    dims = (9, 20, 64, 100, 128) if kind16 == 0 else (9, 20, 33, 64)
+    dims = (9, 20, 64, 100, 128) if kind16 == 0 else (9, 33, 64, 100, 128)
     for d in dims:
         n, m = 2600, 420
         x, y = _knn16_case(rng, kind, n, m, d, dtype)
