@@ -114,6 +114,36 @@ template <int R16> struct SmallChain {
     const float sq = round_in_chain<R16 == 2>(dc * dc);
     return round_in_chain<R16 == 2>(acc + sq);
   }
+  // Four components.  fp16 rows: two differences and two squares per
+  // instruction (every half of a packed 16-bit operation rounds by itself,
+  // like the single one); the sums stay one after the other.
+  static __device__ __forceinline__ float step4(float x0, float x1, float x2,
+                                                float x3, float y0, float y1,
+                                                float y2, float y3,
+                                                float acc) {
+    if constexpr (R16 == 1) {
+#pragma clang fp contract(off)
+      typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+      // (exact: the numbers are fp16 numbers)
+      const half2_t xa = {(_Float16)x0, (_Float16)x1};
+      const half2_t xb = {(_Float16)x2, (_Float16)x3};
+      const half2_t ya = {(_Float16)y0, (_Float16)y1};
+      const half2_t yb = {(_Float16)y2, (_Float16)y3};
+      const half2_t da = xa - ya, db = xb - yb;
+      const half2_t sa = da * da, sb = db * db;
+      _Float16 sum = (_Float16)acc;
+      sum = sum + sa.x;
+      sum = sum + sa.y;
+      sum = sum + sb.x;
+      sum = sum + sb.y;
+      return (float)sum;
+    } else {
+      acc = step(x0, y0, acc);
+      acc = step(x1, y1, acc);
+      acc = step(x2, y2, acc);
+      return step(x3, y3, acc);
+    }
+  }
   static __device__ __forceinline__ float sentinel() {
     return (R16 == 0 || R16 == 3) ? kKnnSentinel
                                   : round_to_16<R16 == 2>(1e10f);
@@ -383,10 +413,7 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
       for (int c = 0; c < (d >> 2); ++c) {
         const float4 a = x4[c];
         const float4 b = y4[c];
-        acc = Chain::step(a.x, b.x, acc);
-        acc = Chain::step(a.y, b.y, acc);
-        acc = Chain::step(a.z, b.z, acc);
-        acc = Chain::step(a.w, b.w, acc);
+        acc = Chain::step4(a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w, acc);
       }
     } else {
       for (int c = 0; c < d; ++c) {
@@ -588,10 +615,8 @@ __global__ __launch_bounds__(kBlock, 1) void knn_feat_small_kernel(
           if (f0 + 4 * c + e < quads) {
             const small_v4f xv = gathered[wave][lane][e];
             const small_v4f b = y4[f0 + 4 * c + e];
-            acc = Chain::step(xv.x, b.x, acc);
-            acc = Chain::step(xv.y, b.y, acc);
-            acc = Chain::step(xv.z, b.z, acc);
-            acc = Chain::step(xv.w, b.w, acc);
+            acc = Chain::step4(xv.x, xv.y, xv.z, xv.w, b.x, b.y, b.z, b.w,
+                               acc);
           }
         }
       }
