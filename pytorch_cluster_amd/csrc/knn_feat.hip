@@ -679,8 +679,10 @@ bool knn_feat_one_kernel(int n, int m, int d, int num_segments, int k,
 
 bool radius_feat_supported(int n, int m, int d, int num_segments, int slots,
                            int r16) {
+  // (fp32 points of up to eight dimensions have kernels of their own; 16-bit
+  // ones have none but the exhaustive scan)
   const bool fits =
-      d > 8 && d <= 128 && slots >= 1 && slots <= 32;
+      (r16 != 0 ? d >= 1 : d > 8) && d <= 128 && slots >= 1 && slots <= 32;
   if (const char *env = std::getenv("PCA_RADIUS_FEAT")) {
     if (env[0] == '0')
       return false;
@@ -700,7 +702,7 @@ bool knn_feat16_supported(int n, int d, int num_segments, int k, bool cosine,
     if (env[0] == '0')
       return false;
   (void)bf16; // (both types up to 128 components)
-  return !cosine && d > 8 && d <= 128 && k <= kFeatSmallMaxK &&
+  return !cosine && d >= 1 && d <= 128 && k <= kFeatSmallMaxK &&
          n >= 1 &&
          num_segments >= 1;
 }

@@ -196,8 +196,8 @@ hipError_t launch_knn_feat(const SearchInput &in, int k, bool cosine,
                            hipEvent_t time_stop, hipStream_t stream,
                            int r16 = 0, const FeatRadius *radius = nullptr);
 // Feature-space radius search through the matrix-core filter
-// (knn_feat_small_impl.hpp): fp32, fp16 and bf16 rows of 8 < d <= 128
-// components, at most 32 neighbours per query, and enough pairs to
+// (knn_feat_small_impl.hpp): fp32 rows of 8 < d <= 128 components, fp16 and
+// bf16 rows of up to 128, at most 32 neighbours per query, and enough pairs to
 // pay for the preparation; PCA_RADIUS_FEAT=0: never, 1: whenever the shape
 // fits.  r16: 0 fp32, 1 fp16, 2 bf16.
 bool radius_feat_supported(int n, int m, int d, int num_segments, int slots,
@@ -207,7 +207,7 @@ bool radius_feat_supported(int n, int m, int d, int num_segments, int slots,
 bool knn_feat_one_kernel(int n, int m, int d, int num_segments, int k,
                          bool cosine);
 // fp16 / bf16 rows through the matrix-core filter (knn_feat_small_impl.hpp):
-// Euclidean, 8 < d <= 128, k <= 48; PCA_KNN_FEAT_16BIT=0: never.
+// Euclidean, d <= 128, k <= 48; PCA_KNN_FEAT_16BIT=0: never.
 bool knn_feat16_supported(int n, int d, int num_segments, int k, bool cosine,
                           bool bf16);
 size_t knn_feat16_scratch_bytes(int n, int m, int d, int num_segments, int k);
