@@ -58,7 +58,10 @@
 // in the exact distances (SmallChain), and in the filter every component of
 // rows and queries times what that arithmetic leaves of its term at worst
 // (chain_keep: the first terms of the sum are rounded most often) -- the
-// filter's distance is then a lower bound of the reference's value.
+// filter's distance is then a lower bound of the reference's value.  Such
+// rows come here with any number of components up to 128, and in any number:
+// 16-bit points of two or three dimensions have no other kernel but the
+// exhaustive scan.
 #pragma once
 
 #include <type_traits>
